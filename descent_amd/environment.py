@@ -1,0 +1,240 @@
+"""Environment: parameters, upload/download and graph execution.
+
+Host-side mirror of src/environment.rs.  The device work is delegated to a
+backend object:
+
+    alloc(nbytes) -> handle        free(handle)
+    write(handle, offset, bytes)   fill_zero(handle, offset, nbytes)
+    read(handle, offset, nbytes) -> bytes
+    launch(kernel_descriptor, [handles], rand_seed)
+    sync()
+    make_schedule(graph, fused) -> object with .run(param_handles, seed)   (optional)
+
+`descent_amd.hip_backend.HipBackend` implements it over the C ABI of
+libdescent_hip.so and is the default.  A backend that lacks `make_schedule`
+is driven kernel by kernel with the reference's own buffer-lifetime algorithm
+(`Environment._run_cluster_by_cluster`).
+"""
+from __future__ import annotations
+
+from typing import Callable, Dict, List, Optional
+
+import numpy as np
+
+from .array import Parameter, Scope
+from .graph import Graph
+from .kernel import FillKernel
+from .module import Initializer
+from .shape import Shape
+
+
+class ParameterWriter:
+    """Sequential byte writer into a parameter's fresh buffer; whatever is left
+    unwritten when it is closed is zero-filled (src/environment.rs:42-59,
+    src/device/staging.rs:181-187)."""
+
+    def __init__(self, backend, handle, nbytes: int):
+        self._backend, self._handle, self._nbytes = backend, handle, nbytes
+        self._pos = 0
+        self._closed = False
+
+    def write(self, data) -> int:
+        buf = np.ascontiguousarray(data).view(np.uint8).reshape(-1) if isinstance(data, np.ndarray) else np.frombuffer(
+            bytes(data), dtype=np.uint8
+        )
+        n = min(len(buf), self._nbytes - self._pos)
+        if n:
+            self._backend.write(self._handle, self._pos, buf[:n])
+            self._pos += n
+        return n
+
+    def zero_fill(self) -> None:
+        self.close()
+
+    def close(self) -> None:
+        if not self._closed:
+            self._closed = True
+            if self._pos < self._nbytes:
+                self._backend.fill_zero(self._handle, self._pos, self._nbytes - self._pos)
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Environment:
+    def __init__(self, backend=None, use_schedule: bool = True, fused: bool = True):
+        if backend is None:
+            from .hip_backend import HipBackend
+
+            backend = HipBackend()
+        self.backend = backend
+        self.use_schedule = use_schedule and hasattr(backend, "make_schedule")
+        self.fused = fused
+        self.parameters: List[Parameter] = []
+
+    # -- parameters (src/environment.rs:126-229) --------------------------------
+    def static_parameter(self, shape, name: str) -> Parameter:
+        p = Parameter(self, shape, name, None)
+        self.parameters.append(p)
+        return p
+
+    def trainable_parameter(self, shape, name: str, reset_to: Initializer) -> Parameter:
+        p = Parameter(self, shape, name, reset_to)
+        self.parameters.append(p)
+        return p
+
+    def writer(self, parameter: Parameter) -> ParameterWriter:
+        """Frees the old buffer and allocates a new one (src/environment.rs:160-175)."""
+        parameter.checked(self)
+        if parameter.buffer is not None:
+            self.backend.free(parameter.buffer)
+            parameter.buffer = None
+        parameter.buffer = self.backend.alloc(parameter.shape.buffer_size())
+        return ParameterWriter(self.backend, parameter.buffer, parameter.shape.buffer_size())
+
+    def write_parameter(self, parameter: Parameter, data) -> None:
+        data = np.ascontiguousarray(data)
+        if data.dtype not in (np.float32, np.uint32, np.int32):
+            data = data.astype(np.float32)
+        with self.writer(parameter) as w:
+            w.write(data)
+
+    def static_parameter_with_data(self, shape, name: str, data) -> Parameter:
+        p = self.static_parameter(shape, name)
+        self.write_parameter(p, np.asarray(data, dtype=np.float32))
+        return p
+
+    def reader(self, parameter: Parameter) -> bytes:
+        parameter.checked(self)
+        if parameter.buffer is None:
+            raise ValueError(f"parameter {parameter.name!r} has no value")
+        return self.backend.read(parameter.buffer, 0, parameter.shape.buffer_size())
+
+    def read_parameter_to_vec(self, parameter: Parameter) -> np.ndarray:
+        return np.frombuffer(self.reader(parameter), dtype=np.float32).copy()
+
+    def read_parameter(self, parameter: Parameter) -> np.ndarray:
+        return self.read_parameter_to_vec(parameter).reshape(tuple(parameter.shape))
+
+    def read_parameter_scalar(self, parameter: Parameter) -> float:
+        return float(self.read_parameter_to_vec(parameter)[0])
+
+    def reset_parameter(self, parameter: Parameter, rng: np.random.Generator) -> None:
+        """src/environment.rs:190-202. The reference draws from ChaCha20 via the
+        `rand` crate (Open01 + Box-Muller); that stream is not reproduced here,
+        only the distributions: N(0, scale^2) and U(-scale, scale)."""
+        init = parameter.reset_to
+        n = parameter.shape.element_count()
+        if init is None:
+            raise ValueError("parameter has no initializer")
+        if init.kind == "zero":
+            self.writer(parameter).zero_fill()
+        elif init.kind == "normal":
+            self.write_parameter(parameter, (rng.standard_normal(n) * init.scale).astype(np.float32))
+        else:
+            self.write_parameter(parameter, ((rng.random(n) * 2.0 - 1.0) * init.scale).astype(np.float32))
+
+    # -- graphs -------------------------------------------------------------------
+    def scope(self) -> Scope:
+        return Scope(self)
+
+    def build_graph(self, f: Callable[[Scope], None]) -> Graph:
+        scope = self.scope()
+        f(scope)
+        return scope.build_graph()
+
+    def run(self, graph: Graph, rand_seed: int) -> None:
+        """src/environment.rs:326-516"""
+        rand_seed &= 0xFFFFFFFF
+        if self.use_schedule:
+            key = (id(self.backend), self.fused)
+            cache = graph.__dict__.setdefault("_schedules", {})
+            sched = cache.get(key)
+            if sched is None:
+                sched = cache[key] = self.backend.make_schedule(graph, self.fused)
+            handles = [p.checked(self).buffer for p in sched.params]
+            handles = sched.run(handles, rand_seed)
+            for p, h in zip(sched.params, handles):
+                p.buffer = h
+        else:
+            self._run_cluster_by_cluster(graph, rand_seed)
+
+    def _run_cluster_by_cluster(self, graph: Graph, rand_seed: int) -> None:
+        be = self.backend
+        ops = graph.ops
+        inputs = [n for n in sorted(ops.nodes) if ops.nodes[n].op.kind == "Input"]
+        outputs = [n for n in sorted(ops.nodes) if ops.nodes[n].op.kind == "Output"]
+        input_params = {ops.nodes[n].op.a for n in inputs}
+        output_params = {ops.nodes[n].op.a for n in outputs}
+
+        usage: Dict[int, int] = {}
+        buffer: Dict[int, object] = {}
+        for cl in graph.clusters.values():
+            for n in cl.inputs:
+                usage[n] = usage.get(n, 0) + 1
+
+        # inputs share the parameter's buffer, or take it when the parameter is rewritten
+        for n in inputs:
+            p = ops.nodes[n].op.a.checked(self)
+            if p.buffer is None:
+                raise ValueError(f"parameter {p.name!r} has no value")
+            if p not in output_params:
+                buffer[n] = p.buffer
+                usage[n] = usage.get(n, 0) + 1
+            else:
+                buffer[n], p.buffer = p.buffer, None
+        # parameters that are only written lose their old buffer
+        for n in outputs:
+            p = ops.nodes[n].op.a.checked(self)
+            if p not in input_params and p.buffer is not None:
+                be.free(p.buffer)
+                p.buffer = None
+
+        for cid in graph.clusters_sorted:
+            cl = graph.clusters[cid]
+            for n in cl.inputs:
+                usage[n] -= 1
+            for out in cl.outputs:
+                shape = ops.nodes[out.node_id].shape
+                if out.copy_from is None:
+                    h = be.alloc(shape.buffer_size())
+                else:
+                    src = out.copy_from
+                    if usage.get(src, 0) != 0:
+                        raise NotImplementedError("deep copy of a still-used accumulator")  # environment.rs:441
+                    if buffer.get(src) is not None:
+                        h = buffer.pop(src)
+                    elif ops.nodes[src].op.kind == "Literal":
+                        h = be.alloc(shape.buffer_size())
+                        be.launch(FillKernel(ops.nodes[src].op.a, shape.element_count()), [h], rand_seed)
+                    else:
+                        raise RuntimeError("cannot copy-on-write node")
+                assert buffer.get(out.node_id) is None
+                buffer[out.node_id] = h
+            handles = [buffer[n] for n in cl.inputs] + [buffer[o.node_id] for o in cl.outputs]
+            be.launch(cl.kernel, handles, rand_seed)
+            for n in cl.inputs:
+                if usage[n] == 0 and buffer.get(n) is not None:
+                    be.free(buffer.pop(n))
+
+        for n in outputs:
+            p = ops.nodes[n].op.a
+            (src,) = ops.predecessors(n)
+            p.buffer = buffer.pop(src)
+
+    def sync(self) -> None:
+        self.backend.sync()
+
+    def print_timings(self, label: str, top_n: int = 5) -> None:
+        """src/environment.rs:518-520"""
+        if hasattr(self.backend, "timing_report"):
+            print(f"{label}:\n{self.backend.timing_report(top_n)}")
