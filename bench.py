@@ -1,0 +1,186 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X backend on the reference's headline workloads.
+
+Default workload (N=1): the standalone fp32 matmul through the array API, M=N=K=8192, with the fused
+per-element epilogue bias + leaky_relu(0.01); one step = one run of that graph with A, B and bias already
+resident in HBM.  Prints ONE JSON line; `--all` adds the other matmul shapes and the ConvNet (batch 1000)
+train-step rate under "extra".
+
+No torch: device memory, the stream and event timing all go through libdescent_hip.so.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MFMA_FP32_PEAK_TFLOPS = 157.3
+HBM_PEAK_GBS = 8000.0
+
+
+def time_graph(env, graph, steps: int, warmup: int, seed0: int = 1):
+    """W untimed runs, then K timed runs bracketed by stream syncs.  Returns (wall seconds, profiler report)."""
+    be = env.backend
+    for i in range(warmup):
+        env.run(graph, seed0 + i)
+    be.sync()
+    be.profile_reset()
+    be.profile(True)
+    t0 = time.perf_counter()
+    for i in range(steps):
+        env.run(graph, seed0 + warmup + i)
+    be.sync()
+    wall = time.perf_counter() - t0
+    be.profile(False)
+    return wall
+
+
+def bench_matmul(env, m, n, k, steps, warmup):
+    from descent_amd import workloads
+
+    w = workloads.matmul_epilogue(env, m, n, k, seed=2)
+    wall = time_graph(env, w.graph, steps, warmup)
+    avg_us, launches = env.backend.timing_query("MatMul")
+    report = env.backend.timing_report(0)
+    env.backend.profile_reset()
+    sched = next(iter(w.graph.__dict__["_schedules"].values()))
+    for p in (w.a, w.b, w.bias, w.c):
+        if p.buffer is not None:
+            env.backend.free(p.buffer)
+            p.buffer = None
+    return {
+        "shape": [m, n, k],
+        "flops": w.flops,
+        "wall_s": wall,
+        "ms_per_step": 1e3 * wall / steps,
+        "tflops_wall": w.flops * steps / wall / 1e12,
+        "kernel_avg_us": avg_us,
+        "kernel_launches": launches,
+        "tflops_kernel": (w.flops / (avg_us * 1e-6) / 1e12) if avg_us else None,
+        "launches_per_step": sched.launch_count()[0],
+        "report": report,
+    }
+
+
+def bench_convnet(env, steps, warmup, batch=1000):
+    from descent_amd import workloads
+
+    w = workloads.convnet(env, batch=batch, seed=3)
+    wall = time_graph(env, w.graph, steps, warmup)
+    report = env.backend.timing_report(12)
+    env.backend.profile_reset()
+    sched = next(iter(w.graph.__dict__["_schedules"].values()))
+    return {
+        "steps_per_s": steps / wall,
+        "ms_per_step": 1e3 * wall / steps,
+        "launches_per_step": sched.launch_count()[0],
+        "clusters": sched.launch_count()[1],
+        "report": report,
+    }
+
+
+def cpu_baseline_matmul(n: int, rows: int):
+    """The CPU oracle (restatement of the reference's algorithm; the reference itself needs Rust + Vulkan) on
+    a slab of `rows` rows of the same n^3 product, epilogue included, all host cores through OpenMP."""
+    from descent_amd import Environment, workloads
+    from oracle.cpu_backend import CpuBackend
+
+    env = Environment(CpuBackend())
+    w = workloads.matmul_epilogue(env, rows, n, n, seed=2)
+    env.run(w.graph, 1)  # warm
+    t0 = time.perf_counter()
+    env.run(w.graph, 1)
+    dt = time.perf_counter() - t0
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    threads = int(os.environ.get("OMP_NUM_THREADS", cores))
+    return {
+        "value": 2.0 * rows * n * n / dt / 1e12,
+        "unit": "TFLOP/s",
+        "cores": min(cores, threads),
+        "kind": "port",
+        "sample": f"{rows} rows of the {n}^3 product (A slab {rows}x{n}, full B), bias+leaky_relu included, {dt:.2f} s",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--size", type=int, default=8192, help="M=N=K of the headline matmul")
+    ap.add_argument("--all", action="store_true", help="also time the other matmul shapes and the ConvNet step")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-rows", type=int, default=256)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; run with --gpus 1 (nothing here uses a second device)", file=sys.stderr)
+        sys.exit(2)
+
+    from descent_amd import Environment
+    from descent_amd.hip_backend import HipBackend
+
+    env = Environment(HipBackend())
+    n = args.size
+    head = bench_matmul(env, n, n, n, args.steps, args.warmup)
+    sys.stderr.write(head["report"])
+
+    extra = {}
+    if args.all:
+        shapes = [(1024, 1024, 1024), (4096, 4096, 4096), (1000, 128, 784), (262144, 256, 256)]
+        extra["matmul"] = []
+        for (m, nn, k) in shapes:
+            r = bench_matmul(env, m, nn, k, max(args.steps, 20), args.warmup)
+            r.pop("report")
+            extra["matmul"].append(r)
+        conv = bench_convnet(env, max(args.steps, 20), args.warmup)
+        sys.stderr.write(conv.pop("report"))
+        extra["convnet_bs1000"] = conv
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline_matmul(n, args.cpu_rows)
+
+    achieved = head["tflops_kernel"] or head["tflops_wall"]
+    line = {
+        "metric": "fp32 matmul TFLOP/s (M=N=K=%d through the array API, fused bias + leaky_relu epilogue)" % n,
+        "value": head["tflops_wall"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "cfg2 standalone fp32 matmul %dx%dx%d + bias + leaky_relu(0.01), N(0,1) entries" % (n, n, n),
+                   "launches_per_step": head["launches_per_step"]},
+        "roofline": {
+            "bound": "mfma",
+            "achieved": achieved,
+            "peak": MFMA_FP32_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved / MFMA_FP32_PEAK_TFLOPS,
+            "traffic": None,
+            "kernel_avg_us": head["kernel_avg_us"],
+            "algorithmic_flops_per_launch": head["flops"],
+        },
+        "cpu_baseline": cpu,
+    }
+    if extra:
+        line["extra"] = extra
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,425 @@
+// extern "C" entry points declared in include/descent_hip.h.
+#include "schedule.hpp"
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <sstream>
+
+using namespace dsc;
+
+struct dsc_ctx {
+    Context c;
+};
+struct dsc_kernel {
+    Kernel k;
+};
+struct dsc_schedule {
+    Schedule s;
+};
+
+namespace {
+
+char* dup_string(const std::string& s) {
+    char* out = static_cast<char*>(std::malloc(s.size() + 1));
+    if (out) std::memcpy(out, s.c_str(), s.size() + 1);
+    return out;
+}
+
+#define HIP_TRY(expr)                                                                                     \
+    do {                                                                                                  \
+        hipError_t e_ = (expr);                                                                           \
+        if (e_ != hipSuccess) return fail(DSC_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(e_)); \
+    } while (0)
+
+// Waits until staging region `r` is free again.
+int staging_acquire(Context* c, int r) {
+    if (c->staging_busy[r]) {
+        HIP_TRY(hipEventSynchronize(c->staging_done[r]));
+        c->staging_busy[r] = false;
+    }
+    return DSC_OK;
+}
+
+int resolve(Context* c, dsc_buf buf, size_t offset, size_t bytes, char** ptr) {
+    void* p = nullptr;
+    size_t size = 0;
+    if (!c->heap.info(buf, &p, &size)) return fail(DSC_ERR_INVALID, "unknown buffer handle");
+    if (offset > size || bytes > size - offset) return fail(DSC_ERR_INVALID, "range outside the buffer");
+    *ptr = static_cast<char*>(p) + offset;
+    return DSC_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* dsc_last_error(void) { return last_error().c_str(); }
+
+int dsc_ctx_create(int device_ordinal, dsc_ctx** out) {
+    if (!out) return fail(DSC_ERR_INVALID, "null out pointer");
+    *out = nullptr;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        return fail(DSC_ERR_NO_DEVICE, "no HIP device available");
+    }
+    if (device_ordinal < 0 || device_ordinal >= count) return fail(DSC_ERR_INVALID, "device ordinal out of range");
+    HIP_TRY(hipSetDevice(device_ordinal));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device_ordinal));
+    auto ctx = new dsc_ctx();
+    Context& c = ctx->c;
+    c.device = device_ordinal;
+    c.arch = prop.gcnArchName;
+    const size_t colon = c.arch.find(':');
+    if (colon != std::string::npos) c.arch = c.arch.substr(0, colon);
+    c.caps.has_float_atomic_add = 1;
+    c.caps.compute_units = prop.multiProcessorCount;
+    c.caps.wavefront_size = prop.warpSize;
+    c.caps.device_memory_bytes = (int64_t)prop.totalGlobalMem;
+    std::snprintf(c.caps.arch, sizeof c.caps.arch, "%s", c.arch.c_str());
+    if (c.arch != "gfx950") {
+        delete ctx;
+        return fail(DSC_ERR_NO_DEVICE, "device is " + std::string(prop.gcnArchName) + "; this backend is written for gfx950 only");
+    }
+    hipError_t e = hipStreamCreate(&c.stream);
+    if (e != hipSuccess) {
+        delete ctx;
+        return fail(DSC_ERR_HIP, std::string("hipStreamCreate: ") + hipGetErrorString(e));
+    }
+    for (int i = 0; i < Context::kStagingRegions; ++i) {
+        void* p = nullptr;
+        e = hipHostMalloc(&p, Context::kStagingBytes, hipHostMallocDefault);
+        if (e == hipSuccess) e = hipEventCreateWithFlags(&c.staging_done[i], hipEventDisableTiming);
+        if (e != hipSuccess) {
+            delete ctx;
+            return fail(DSC_ERR_HIP, std::string("staging setup: ") + hipGetErrorString(e));
+        }
+        c.staging[i] = static_cast<char*>(p);
+    }
+    *out = ctx;
+    return DSC_OK;
+}
+
+int dsc_ctx_destroy(dsc_ctx* ctx) {
+    if (!ctx) return DSC_OK;
+    (void)hipSetDevice(ctx->c.device);
+    delete ctx;
+    return DSC_OK;
+}
+
+int dsc_ctx_caps(dsc_ctx* ctx, dsc_caps* out) {
+    if (!ctx || !out) return fail(DSC_ERR_INVALID, "null argument");
+    *out = ctx->c.caps;
+    return DSC_OK;
+}
+
+int dsc_ctx_sync(dsc_ctx* ctx) {
+    if (!ctx) return fail(DSC_ERR_INVALID, "null context");
+    HIP_TRY(hipStreamSynchronize(ctx->c.stream));
+    return DSC_OK;
+}
+
+int dsc_ctx_stream(dsc_ctx* ctx, void** out_stream) {
+    if (!ctx || !out_stream) return fail(DSC_ERR_INVALID, "null argument");
+    *out_stream = ctx->c.stream;
+    return DSC_OK;
+}
+
+int dsc_buf_alloc(dsc_ctx* ctx, size_t bytes, dsc_buf* out) {
+    if (!ctx || !out) return fail(DSC_ERR_INVALID, "null argument");
+    *out = ctx->c.heap.alloc(bytes);
+    if (!*out) return fail(DSC_ERR_OOM, "device memory exhausted allocating " + std::to_string(bytes) + " bytes");
+    return DSC_OK;
+}
+
+int dsc_buf_free(dsc_ctx* ctx, dsc_buf buf) {
+    if (!ctx) return fail(DSC_ERR_INVALID, "null context");
+    if (!ctx->c.heap.free(buf)) return fail(DSC_ERR_INVALID, "free of an unknown or already freed buffer");
+    return DSC_OK;
+}
+
+int dsc_buf_info(dsc_ctx* ctx, dsc_buf buf, void** out_device_ptr, size_t* out_bytes) {
+    if (!ctx) return fail(DSC_ERR_INVALID, "null context");
+    if (!ctx->c.heap.info(buf, out_device_ptr, out_bytes)) return fail(DSC_ERR_INVALID, "unknown buffer handle");
+    return DSC_OK;
+}
+
+int dsc_heap_stats(dsc_ctx* ctx, int64_t* out_live_buffers, int64_t* out_live_bytes, int64_t* out_arena_bytes) {
+    if (!ctx) return fail(DSC_ERR_INVALID, "null context");
+    ctx->c.heap.stats(out_live_buffers, out_live_bytes, out_arena_bytes);
+    return DSC_OK;
+}
+
+int dsc_buf_write(dsc_ctx* ctx, dsc_buf buf, size_t offset, const void* src, size_t bytes) {
+    if (!ctx || (!src && bytes)) return fail(DSC_ERR_INVALID, "null argument");
+    Context* c = &ctx->c;
+    char* dst = nullptr;
+    int rc = resolve(c, buf, offset, bytes, &dst);
+    if (rc != DSC_OK) return rc;
+    const char* s = static_cast<const char*>(src);
+    while (bytes) {
+        const int r = c->staging_next;
+        c->staging_next = (r + 1) % Context::kStagingRegions;
+        rc = staging_acquire(c, r);
+        if (rc != DSC_OK) return rc;
+        const size_t n = std::min(bytes, Context::kStagingBytes);
+        std::memcpy(c->staging[r], s, n);
+        HIP_TRY(hipMemcpyAsync(dst, c->staging[r], n, hipMemcpyHostToDevice, c->stream));
+        HIP_TRY(hipEventRecord(c->staging_done[r], c->stream));
+        c->staging_busy[r] = true;
+        s += n;
+        dst += n;
+        bytes -= n;
+    }
+    return DSC_OK;
+}
+
+int dsc_buf_fill_zero(dsc_ctx* ctx, dsc_buf buf, size_t offset, size_t bytes) {
+    if (!ctx) return fail(DSC_ERR_INVALID, "null context");
+    char* dst = nullptr;
+    int rc = resolve(&ctx->c, buf, offset, bytes, &dst);
+    if (rc != DSC_OK) return rc;
+    if (bytes) HIP_TRY(hipMemsetAsync(dst, 0, bytes, ctx->c.stream));
+    return DSC_OK;
+}
+
+int dsc_buf_read(dsc_ctx* ctx, dsc_buf buf, size_t offset, void* dst, size_t bytes) {
+    if (!ctx || (!dst && bytes)) return fail(DSC_ERR_INVALID, "null argument");
+    Context* c = &ctx->c;
+    char* src = nullptr;
+    int rc = resolve(c, buf, offset, bytes, &src);
+    if (rc != DSC_OK) return rc;
+    char* d = static_cast<char*>(dst);
+    // two regions in flight: the copy into region r+1 overlaps the host memcpy out of region r
+    size_t pending_n[Context::kStagingRegions] = {0, 0};
+    char* pending_dst[Context::kStagingRegions] = {nullptr, nullptr};
+    auto drain = [&](int r) -> int {
+        if (!pending_n[r]) return DSC_OK;
+        HIP_TRY(hipEventSynchronize(c->staging_done[r]));
+        c->staging_busy[r] = false;
+        std::memcpy(pending_dst[r], c->staging[r], pending_n[r]);
+        pending_n[r] = 0;
+        return DSC_OK;
+    };
+    int r = 0;
+    while (bytes) {
+        rc = drain(r);
+        if (rc != DSC_OK) return rc;
+        rc = staging_acquire(c, r);
+        if (rc != DSC_OK) return rc;
+        const size_t n = std::min(bytes, Context::kStagingBytes);
+        HIP_TRY(hipMemcpyAsync(c->staging[r], src, n, hipMemcpyDeviceToHost, c->stream));
+        HIP_TRY(hipEventRecord(c->staging_done[r], c->stream));
+        c->staging_busy[r] = true;
+        pending_n[r] = n;
+        pending_dst[r] = d;
+        src += n;
+        d += n;
+        bytes -= n;
+        r = (r + 1) % Context::kStagingRegions;
+    }
+    for (int i = 0; i < Context::kStagingRegions; ++i) {
+        rc = drain((r + i) % Context::kStagingRegions);
+        if (rc != DSC_OK) return rc;
+    }
+    return DSC_OK;
+}
+
+int dsc_kernel_get(dsc_ctx* ctx, const dsc_kernel_desc* desc, dsc_kernel** out) {
+    if (!ctx || !desc || !out) return fail(DSC_ERR_INVALID, "null argument");
+    *out = nullptr;
+    std::string err = validate(*desc);
+    if (!err.empty()) return fail(DSC_ERR_INVALID, err);
+    int status = DSC_OK;
+    Kernel* k = get_kernel(&ctx->c, FusedKernel::plain(*desc), &status);
+    if (!k) return status;
+    *out = reinterpret_cast<dsc_kernel*>(k);
+    return DSC_OK;
+}
+
+int dsc_kernel_buffer_count(const dsc_kernel* k) { return k ? reinterpret_cast<const Kernel*>(k)->gen.n_buffers : 0; }
+int64_t dsc_kernel_reference_group_count(const dsc_kernel* k) { return k ? reinterpret_cast<const Kernel*>(k)->reference_groups : 0; }
+const char* dsc_kernel_label(const dsc_kernel* k) { return k ? reinterpret_cast<const Kernel*>(k)->label.c_str() : ""; }
+const char* dsc_kernel_source(const dsc_kernel* k) { return k ? reinterpret_cast<const Kernel*>(k)->gen.source.c_str() : ""; }
+
+int dsc_kernel_launch(dsc_ctx* ctx, dsc_kernel* kernel, const dsc_buf* bufs, int n, uint32_t rand_seed) {
+    if (!ctx || !kernel || (!bufs && n)) return fail(DSC_ERR_INVALID, "null argument");
+    Kernel* k = reinterpret_cast<Kernel*>(kernel);
+    if (n != k->gen.n_buffers) return fail(DSC_ERR_INVALID, "wrong number of buffers for '" + k->label + "'");
+    if (n > 64) return fail(DSC_ERR_UNSUPPORTED, "more than 64 buffers");
+    void* ptrs[64];
+    // every bound buffer must hold at least what the kernel addresses
+    const dsc_kernel_desc& d = k->fused.main.raw();
+    for (int i = 0; i < n; ++i) {
+        size_t size = 0;
+        if (!ctx->c.heap.info(bufs[i], &ptrs[i], &size)) return fail(DSC_ERR_INVALID, "unknown buffer handle in launch");
+        size_t need = 0;
+        if (i < d.n_inputs) need = (size_t)element_count(d.inputs[i].in_shape) * 4;
+        else need = (size_t)element_count(d.shape) * 4;
+        if (size < need) return fail(DSC_ERR_INVALID, "buffer " + std::to_string(i) + " of '" + k->label + "' is too small");
+    }
+    return launch_kernel(&ctx->c, k, ptrs, n, rand_seed);
+}
+
+int dsc_codegen_source(const dsc_kernel_desc* desc, char** out_source) {
+    if (!desc || !out_source) return fail(DSC_ERR_INVALID, "null argument");
+    std::string err = validate(*desc);
+    if (!err.empty()) return fail(DSC_ERR_INVALID, err);
+    Generated g;
+    err = generate(FusedKernel::plain(*desc), &g);
+    if (!err.empty()) return fail(DSC_ERR_INVALID, err);
+    *out_source = dup_string(g.source);
+    return *out_source ? DSC_OK : fail(DSC_ERR_OOM, "host allocation failed");
+}
+
+int dsc_codegen_compile(const dsc_kernel_desc* desc, const char* arch, size_t* out_code_bytes) {
+    if (!desc || !arch) return fail(DSC_ERR_INVALID, "null argument");
+    std::string err = validate(*desc);
+    if (!err.empty()) return fail(DSC_ERR_INVALID, err);
+    Generated g;
+    err = generate(FusedKernel::plain(*desc), &g);
+    if (!err.empty()) return fail(DSC_ERR_INVALID, err);
+    std::vector<char> code;
+    std::string log;
+    int rc = compile_source(g.source, arch, &code, &log);
+    if (rc != DSC_OK) return rc;
+    if (out_code_bytes) *out_code_bytes = code.size();
+    return DSC_OK;
+}
+
+int dsc_codegen_check_schedule(const dsc_schedule_desc* desc, uint32_t flags, const char* arch, char** out_text) {
+    if (!desc || !arch) return fail(DSC_ERR_INVALID, "null argument");
+    Context offline;
+    offline.offline = true;
+    offline.arch = arch;
+    Schedule s;
+    int rc = s.build(&offline, *desc, flags);
+    if (rc != DSC_OK) return rc;
+    if (out_text) {
+        *out_text = dup_string(s.describe());
+        if (!*out_text) return fail(DSC_ERR_OOM, "host allocation failed");
+    }
+    return DSC_OK;
+}
+
+void dsc_free_string(char* s) { std::free(s); }
+
+int dsc_schedule_create(dsc_ctx* ctx, const dsc_schedule_desc* desc, uint32_t flags, dsc_schedule** out) {
+    if (!ctx || !desc || !out) return fail(DSC_ERR_INVALID, "null argument");
+    *out = nullptr;
+    auto s = new dsc_schedule();
+    int rc = s->s.build(&ctx->c, *desc, flags);
+    if (rc != DSC_OK) {
+        delete s;
+        return rc;
+    }
+    *out = s;
+    return DSC_OK;
+}
+
+int dsc_schedule_destroy(dsc_ctx* ctx, dsc_schedule* s) {
+    (void)ctx;
+    delete s;
+    return DSC_OK;
+}
+
+int dsc_schedule_run(dsc_ctx* ctx, dsc_schedule* s, dsc_buf* params, uint32_t rand_seed) {
+    if (!ctx || !s || !params) return fail(DSC_ERR_INVALID, "null argument");
+    return s->s.run(&ctx->c, params, rand_seed);
+}
+
+int dsc_schedule_launch_count(const dsc_schedule* s, int32_t* out_launches, int32_t* out_clusters) {
+    if (!s) return fail(DSC_ERR_INVALID, "null schedule");
+    if (out_launches) *out_launches = (int32_t)s->s.steps.size();
+    if (out_clusters) *out_clusters = s->s.n_clusters;
+    return DSC_OK;
+}
+
+int dsc_schedule_describe(const dsc_schedule* s, char** out_text) {
+    if (!s || !out_text) return fail(DSC_ERR_INVALID, "null argument");
+    *out_text = dup_string(s->s.describe());
+    return *out_text ? DSC_OK : fail(DSC_ERR_OOM, "host allocation failed");
+}
+
+int dsc_prof_enable(dsc_ctx* ctx, int enabled) {
+    if (!ctx) return fail(DSC_ERR_INVALID, "null context");
+    ctx->c.profiling = enabled != 0;
+    return DSC_OK;
+}
+
+int dsc_prof_reset(dsc_ctx* ctx) {
+    if (!ctx) return fail(DSC_ERR_INVALID, "null context");
+    HIP_TRY(hipStreamSynchronize(ctx->c.stream));
+    for (auto& p : ctx->c.profile) {
+        ctx->c.event_pool.push_back(p.start);
+        ctx->c.event_pool.push_back(p.stop);
+    }
+    ctx->c.profile.clear();
+    return DSC_OK;
+}
+
+namespace {
+struct Acc {
+    double ms = 0;
+    int64_t n = 0;
+};
+int collect(Context* c, std::map<std::string, Acc>* by_label) {
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    for (auto& p : c->profile) {
+        float ms = 0.f;
+        HIP_TRY(hipEventElapsedTime(&ms, p.start, p.stop));
+        Acc& a = (*by_label)[p.kernel->label];
+        a.ms += ms;
+        a.n += 1;
+    }
+    return DSC_OK;
+}
+}  // namespace
+
+int dsc_prof_report(dsc_ctx* ctx, int top_n, char** out_text) {
+    if (!ctx || !out_text) return fail(DSC_ERR_INVALID, "null argument");
+    std::map<std::string, Acc> by_label;
+    int rc = collect(&ctx->c, &by_label);
+    if (rc != DSC_OK) return rc;
+    std::vector<std::pair<std::string, Acc>> rows(by_label.begin(), by_label.end());
+    std::sort(rows.begin(), rows.end(), [](auto& a, auto& b) { return a.second.ms > b.second.ms; });
+    double total = 0;
+    for (auto& r : rows) total += r.second.ms;
+    std::ostringstream o;
+    char line[256];
+    std::snprintf(line, sizeof line, "total %.3f ms over %zu launches\n", total, ctx->c.profile.size());
+    o << line;
+    int shown = 0;
+    for (auto& r : rows) {
+        if (top_n > 0 && shown++ >= top_n) break;
+        std::snprintf(line, sizeof line, "%10.3f ms %8lld x %10.2f us  %s\n", r.second.ms, (long long)r.second.n,
+                      1000.0 * r.second.ms / (double)r.second.n, r.first.c_str());
+        o << line;
+    }
+    *out_text = dup_string(o.str());
+    return *out_text ? DSC_OK : fail(DSC_ERR_OOM, "host allocation failed");
+}
+
+int dsc_prof_query(dsc_ctx* ctx, const char* prefix, double* out_avg_us, int64_t* out_launches) {
+    if (!ctx || !prefix) return fail(DSC_ERR_INVALID, "null argument");
+    std::map<std::string, Acc> by_label;
+    int rc = collect(&ctx->c, &by_label);
+    if (rc != DSC_OK) return rc;
+    Acc sum;
+    const std::string pre(prefix);
+    for (auto& kv : by_label) {
+        if (kv.first.compare(0, pre.size(), pre) == 0) {
+            sum.ms += kv.second.ms;
+            sum.n += kv.second.n;
+        }
+    }
+    if (out_avg_us) *out_avg_us = sum.n ? 1000.0 * sum.ms / (double)sum.n : 0.0;
+    if (out_launches) *out_launches = sum.n;
+    return DSC_OK;
+}
+
+}  // extern "C"

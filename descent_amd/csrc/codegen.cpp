@@ -1,0 +1,686 @@
+#include "codegen.hpp"
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <map>
+#include <sstream>
+
+namespace dsc {
+
+namespace {
+
+using std::string;
+using std::to_string;
+
+string S(int64_t v) { return to_string((long long)v); }
+
+string hex32(uint32_t bits) {
+    char buf[16];
+    std::snprintf(buf, sizeof buf, "0x%08xu", bits);
+    return buf;
+}
+
+const int64_t kMaxIndex = (int64_t)1 << 31;
+
+// Largest linear index (+1) a view may produce into its input, i.e. the input's element count.
+int64_t input_extent(const dsc_view& v) { return element_count(v.in_shape); }
+
+struct Emitter {
+    const FusedKernel& fk;
+    std::ostringstream funcs;  // device functions, emitted before the kernel
+    int tmp_counter = 0;
+
+    explicit Emitter(const FusedKernel& k) : fk(k) {}
+
+    // ---- parameters ---------------------------------------------------------------------------------
+    string params_decl() const {
+        string s;
+        for (int i = 0; i < fk.n_buffers; ++i) {
+            if (i) s += ", ";
+            s += (fk.buffer_is_output[i] ? "float* __restrict__ b" : "const float* __restrict__ b") + to_string(i);
+        }
+        s += (fk.n_buffers ? ", " : "");
+        s += "uint rand_seed";
+        return s;
+    }
+    string params_pass() const {
+        string s;
+        for (int i = 0; i < fk.n_buffers; ++i) s += "b" + to_string(i) + ", ";
+        return s + "rand_seed";
+    }
+
+    // ---- coordinates --------------------------------------------------------------------------------
+    // Emits the row-major decomposition of `gid` over `shape` as ints named <pfx>0.. and returns the names.
+    std::vector<string> emit_coords(std::ostream& o, const dsc_shape& shape, const string& gid, const string& pfx) {
+        std::vector<string> names(shape.rank);
+        if (shape.rank == 1) {
+            names[0] = pfx + "0";
+            o << "    const int " << names[0] << " = (int)(" << gid << ");\n";
+            return names;
+        }
+        const string rem = pfx + "r";
+        o << "    uint " << rem << " = (uint)(" << gid << ");\n";
+        for (int i = shape.rank - 1; i >= 1; --i) {
+            names[i] = pfx + to_string(i);
+            if (shape.dims[i] == 1) {
+                o << "    const int " << names[i] << " = 0;\n";
+            } else {
+                o << "    const int " << names[i] << " = (int)(" << rem << " % " << S(shape.dims[i]) << "u); " << rem
+                  << " /= " << S(shape.dims[i]) << "u;\n";
+            }
+        }
+        names[0] = pfx + "0";
+        o << "    const int " << names[0] << " = (int)" << rem << ";\n";
+        return names;
+    }
+
+    // Linear index into the view's input for output coordinates `coord` (kernel.rs:89-133).
+    string index_expr(const dsc_view& v, const std::vector<string>& coord) const {
+        int64_t st[DSC_MAX_DIM];
+        strides_of(v.in_shape, st);
+        int64_t constant = 0;
+        std::map<string, int64_t> affine;  // coordinate name -> coefficient (un-clamped axes folded together)
+        string clamped;
+        for (int i = 0; i < v.in_shape.rank; ++i) {
+            if (!needs_clamp(v, i)) {
+                constant += v.in_offset[i] * st[i];
+                for (int j = 0; j < v.out_shape.rank; ++j)
+                    if (v.map_axis[j] == i && v.out_shape.dims[j] > 1) affine[coord[j]] += v.map_step[j] * st[i];
+            } else {
+                string e = S(v.in_offset[i]);
+                for (int j = 0; j < v.out_shape.rank; ++j)
+                    if (v.map_axis[j] == i && v.out_shape.dims[j] > 1) e += " + (" + S(v.map_step[j]) + ")*" + coord[j];
+                clamped += " + clampi(" + e + ", 0, " + S(v.in_shape.dims[i] - 1) + ")*" + S(st[i]);
+            }
+        }
+        string e = "(" + S(constant);
+        for (auto& kv : affine)
+            if (kv.second != 0) e += " + (" + S(kv.second) + ")*" + kv.first;
+        return e + clamped + ")";
+    }
+
+    string load_expr(const Source& s, const string& idx) const {
+        if (s.buffer >= 0) return "b" + to_string(s.buffer) + "[" + idx + "]";
+        return "virt" + to_string(s.virt) + "(" + idx + ", " + params_pass() + ")";
+    }
+
+    // ---- per-element bodies ---------------------------------------------------------------------------
+    // Emits the straight-line evaluation of `pe` at linear id `gid`; op i is left in variable <pfx>t<i>.
+    // `override_load[input]` replaces the load of that input by an expression.
+    void emit_pe(std::ostream& o, const dsc_kernel_desc& pe, const std::vector<Source>& srcs, const string& gid,
+                 const string& pfx, const std::map<int, string>& override_load) {
+        std::vector<std::pair<dsc_shape, std::vector<string>>> sets;
+        auto coords_for = [&](const dsc_shape& shape) -> std::vector<string> {
+            for (auto& s : sets)
+                if (same_shape(s.first, shape)) return s.second;
+            auto names = emit_coords(o, shape, gid, pfx + "c" + to_string(sets.size()) + "_");
+            sets.emplace_back(shape, names);
+            return names;
+        };
+        auto T = [&](int i) { return pfx + "t" + to_string(i); };
+        for (int i = 0; i < pe.n_ops; ++i) {
+            const dsc_pe_op& op = pe.ops[i];
+            string rhs;
+            switch (op.kind) {
+            case DSC_PE_LOAD: {
+                auto ov = override_load.find(op.input_index);
+                if (ov != override_load.end()) { rhs = ov->second; break; }
+                const dsc_view& v = pe.inputs[op.input_index];
+                if (is_identity(v)) rhs = load_expr(srcs[op.input_index], "(int)(" + gid + ")");
+                else rhs = load_expr(srcs[op.input_index], index_expr(v, coords_for(v.out_shape)));
+                break;
+            }
+            case DSC_PE_LITERAL_F32:
+            case DSC_PE_LITERAL_U32: rhs = "U2F(" + hex32(op.bits) + ")"; break;
+            case DSC_PE_COORD: {
+                const dsc_view& v = pe.builtin_views[op.view_index];
+                rhs = "(float)" + index_expr(v, coords_for(v.out_shape));
+                break;
+            }
+            case DSC_PE_RAND: {
+                const dsc_view& v = pe.builtin_views[op.view_index];
+                string idx = is_identity(v) ? "(int)(" + gid + ")" : index_expr(v, coords_for(v.out_shape));
+                rhs = "rand_from_index(rand_seed, " + S(op.bits) + "u, " + idx + ")";
+                break;
+            }
+            case DSC_PE_UNARY: {
+                const string a = T(op.args[0]);
+                switch (op.op) {
+                case DSC_UN_MOV: rhs = a; break;
+                case DSC_UN_NEG: rhs = "-" + a; break;
+                case DSC_UN_SQRT: rhs = "sqrtf(" + a + ")"; break;
+                case DSC_UN_EXP: rhs = "expf(" + a + ")"; break;
+                case DSC_UN_LOG: rhs = "logf(" + a + ")"; break;
+                case DSC_UN_SIN: rhs = "sinf(" + a + ")"; break;
+                case DSC_UN_COS: rhs = "cosf(" + a + ")"; break;
+                case DSC_UN_FLOAT_TO_UINT: rhs = "U2F((uint)" + a + ")"; break;
+                case DSC_UN_UINT_TO_FLOAT: rhs = "(float)F2U(" + a + ")"; break;
+                }
+                break;
+            }
+            case DSC_PE_BINARY: {
+                const string a = T(op.args[0]), b = T(op.args[1]);
+                switch (op.op) {
+                case DSC_BIN_ADD: rhs = a + " + " + b; break;
+                case DSC_BIN_SUB: rhs = a + " - " + b; break;
+                case DSC_BIN_MUL: rhs = a + " * " + b; break;
+                case DSC_BIN_DIV: rhs = a + " / " + b; break;
+                case DSC_BIN_POW: rhs = "powf(" + a + ", " + b + ")"; break;
+                case DSC_BIN_UADD: rhs = "U2F(F2U(" + a + ") + F2U(" + b + "))"; break;
+                case DSC_BIN_UMUL: rhs = "U2F(F2U(" + a + ") * F2U(" + b + "))"; break;
+                case DSC_BIN_UREM: rhs = "U2F(F2U(" + a + ") % F2U(" + b + "))"; break;
+                case DSC_BIN_UBITXOR: rhs = "U2F(F2U(" + a + ") ^ F2U(" + b + "))"; break;
+                }
+                break;
+            }
+            case DSC_PE_SELECT:
+                rhs = "(" + T(op.args[0]) + (op.op == DSC_CMP_EQ ? " == " : " > ") + T(op.args[1]) + ") ? " +
+                      T(op.args[2]) + " : " + T(op.args[3]);
+                break;
+            case DSC_PE_GATHER: {
+                const dsc_view& v = pe.inputs[op.input_index];
+                auto names = coords_for(op.gather_shape);
+                names[op.axis] = "F2I(" + T(op.args[0]) + ")";
+                rhs = load_expr(srcs[op.input_index], index_expr(v, names));
+                break;
+            }
+            }
+            o << "    const float " << T(i) << " = " << rhs << ";\n";
+        }
+    }
+
+    // Device functions for the virtual inputs (highest index first: a virtual only references larger ones).
+    void emit_virtuals() {
+        for (int v = (int)fk.virtuals.size() - 1; v >= 0; --v) {
+            const Virtual& vi = fk.virtuals[v];
+            funcs << "DSC_INLINE float virt" << v << "(int gid, " << params_decl() << ") {\n";
+            emit_pe(funcs, vi.pe.raw(), vi.inputs, "gid", "v", {});
+            funcs << "    return vt" << vi.out_op << ";\n}\n\n";
+        }
+    }
+};
+
+string check_sizes(const FusedKernel& fk) {
+    auto chk = [](const dsc_kernel_desc& d) -> string {
+        if (element_count(d.shape) >= kMaxIndex) return "kernel too large for 32-bit indexing";
+        for (int i = 0; i < d.n_inputs; ++i)
+            if (input_extent(d.inputs[i]) >= kMaxIndex || element_count(d.inputs[i].out_shape) >= kMaxIndex)
+                return "input too large for 32-bit indexing";
+        return "";
+    };
+    string e = chk(fk.main.raw());
+    if (!e.empty()) return e;
+    for (auto& v : fk.virtuals) {
+        e = chk(v.pe.raw());
+        if (!e.empty()) return e;
+    }
+    if (fk.has_epilogue) return chk(fk.epilogue.raw());
+    return "";
+}
+
+unsigned blocks_for(int64_t threads, int block) { return (unsigned)((threads + block - 1) / block); }
+
+// ---------------------------------------------------------------------------------------------------------
+
+string gen_fill(Emitter& em, Generated* out) {
+    const dsc_kernel_desc& d = em.fk.main.raw();
+    const int64_t n = d.shape.dims[0];
+    std::ostringstream k;
+    const bool vec = n % 4 == 0;
+    k << "extern \"C\" __global__ __launch_bounds__(256) void dsc_kernel(" << em.params_decl() << ") {\n";
+    k << "    const uint i = blockIdx.x * 256u + threadIdx.x;\n";
+    if (vec) {
+        k << "    if (i >= " << S(n / 4) << "u) return;\n";
+        k << "    const float v = U2F(" << hex32(d.fill_bits) << ");\n";
+        k << "    ((float4*)b" << em.fk.outputs[0] << ")[i] = make_float4(v, v, v, v);\n";
+    } else {
+        k << "    if (i >= " << S(n) << "u) return;\n";
+        k << "    b" << em.fk.outputs[0] << "[i] = U2F(" << hex32(d.fill_bits) << ");\n";
+    }
+    k << "}\n";
+    out->grid = blocks_for(vec ? n / 4 : n, 256);
+    out->block = 256;
+    out->source = k.str();
+    out->note = vec ? "fill x4" : "fill";
+    return "";
+}
+
+string gen_per_element(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const int64_t n = d.shape.dims[0];
+    const int vec = (n % 4 == 0 && n >= 4096) ? 4 : 1;
+    std::ostringstream k;
+    k << "extern \"C\" __global__ __launch_bounds__(256) void dsc_kernel(" << em.params_decl() << ") {\n";
+    k << "    const uint base = (blockIdx.x * 256u + threadIdx.x) * " << vec << "u;\n";
+    k << "    if (base >= " << S(n) << "u) return;\n";
+    std::map<int, string> override_load;
+    if (vec == 4) {
+        // identity-view loads of real buffers become one 16-byte load per thread
+        for (int i = 0; i < d.n_inputs; ++i) {
+            if (fk.inputs[i].buffer >= 0 && is_identity(d.inputs[i])) {
+                k << "    const float4 q" << i << " = *(const float4*)(b" << fk.inputs[i].buffer << " + base);\n";
+                k << "    const float l" << i << "[4] = {q" << i << ".x, q" << i << ".y, q" << i << ".z, q" << i << ".w};\n";
+                override_load[i] = "l" + to_string(i) + "[e]";
+            }
+        }
+        for (int o = 0; o < d.n_outputs; ++o) k << "    float o" << o << "[4];\n";
+        k << "#pragma unroll\n    for (int e = 0; e < 4; ++e) {\n    const uint gid = base + e;\n";
+    } else {
+        k << "    const uint gid = base;\n    {\n";
+    }
+    em.emit_pe(k, d, fk.inputs, "gid", "", override_load);
+    for (int o = 0; o < d.n_outputs; ++o) {
+        if (vec == 4) k << "    o" << o << "[e] = t" << d.outputs[o] << ";\n";
+        else k << "    b" << fk.outputs[o] << "[gid] = t" << d.outputs[o] << ";\n";
+    }
+    k << "    }\n";
+    if (vec == 4)
+        for (int o = 0; o < d.n_outputs; ++o)
+            k << "    *(float4*)(b" << fk.outputs[o] << " + base) = make_float4(o" << o << "[0], o" << o << "[1], o" << o
+              << "[2], o" << o << "[3]);\n";
+    k << "}\n";
+    out->grid = blocks_for(n / vec, 256);
+    out->block = 256;
+    out->source = k.str();
+    out->note = vec == 4 ? "per-element x4" : "per-element";
+    return "";
+}
+
+int64_t pow2_ceil(int64_t v) {
+    int64_t p = 1;
+    while (p < v) p <<= 1;
+    return p;
+}
+
+string gen_reduce(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const dsc_view& v = d.inputs[0];
+    const int64_t n_out = element_count(d.shape);
+    const int64_t K = v.out_shape.dims[d.axis];
+    const bool is_max = d.reduce_op == DSC_REDUCE_MAX;
+    const string init = is_max ? "U2F(0xff800000u)" : "0.f";
+    auto combine = [&](const string& a, const string& b) { return is_max ? "glsl_max(" + a + ", " + b + ")" : a + " + " + b; };
+
+    // is the reduced axis the one that walks memory fastest?
+    bool k_fastest = false;
+    if (fk.inputs[0].buffer >= 0) {
+        int64_t base, coef[DSC_MAX_DIM];
+        if (affine_form(v, &base, coef) && coef[d.axis] == 1 && K >= 4) k_fastest = true;
+    }
+
+    std::ostringstream k;
+    k << "extern \"C\" __global__ __launch_bounds__(256) void dsc_kernel(" << em.params_decl() << ") {\n";
+    std::ostringstream body;  // loads one element: expects ints oc* (output coords) and kk
+    if (k_fastest) {
+        // lanes of a group walk k; groups of G lanes own one output; butterfly over the group
+        const int64_t G = std::min<int64_t>(64, pow2_ceil(K));
+        const int64_t per_block = 256 / G;
+        k << "    const int grp = threadIdx.x / " << G << ", lk = threadIdx.x % " << G << ";\n";
+        k << "    const uint oid = blockIdx.x * " << per_block << "u + grp;\n";
+        k << "    if (oid >= " << S(n_out) << "u) return;\n";
+        auto oc = em.emit_coords(k, d.shape, "oid", "oc");
+        k << "    float acc = " << init << ";\n";
+        k << "    for (int kk = lk; kk < " << S(K) << "; kk += " << G << ") {\n";
+        auto ic = oc;
+        ic[d.axis] = "kk";
+        k << "        const float x = " << em.load_expr(fk.inputs[0], em.index_expr(v, ic)) << ";\n";
+        k << "        acc = " << combine("acc", "x") << ";\n    }\n";
+        for (int64_t off = G / 2; off >= 1; off /= 2)
+            k << "    acc = " << combine("acc", "__shfl_xor(acc, " + S(off) + ", 64)") << ";\n";
+        k << "    if (lk == 0) b" << fk.outputs[0] << "[oid] = acc;\n}\n";
+        out->grid = blocks_for(n_out, (int)per_block);
+        out->note = "reduce: " + S(G) + " lanes along k, shuffle";
+    } else {
+        // lanes walk outputs (coalesced); optional split of k over TK thread rows, combined through LDS
+        int64_t TK = 1;
+        if (n_out < 65536 && K >= 8) {
+            while (TK < 16 && n_out * TK < 65536 && TK * 4 <= K) TK *= 2;
+        }
+        const int64_t TO = 256 / TK;
+        k << "    const int to = threadIdx.x % " << TO << ", tk = threadIdx.x / " << TO << ";\n";
+        k << "    const uint oid = blockIdx.x * " << TO << "u + to;\n";
+        if (TK > 1) k << "    __shared__ float red[256];\n";
+        k << "    float acc = " << init << ";\n";
+        k << "    if (oid < " << S(n_out) << "u) {\n";
+        auto oc = em.emit_coords(k, d.shape, "oid", "oc");
+        k << "    for (int kk = tk; kk < " << S(K) << "; kk += " << TK << ") {\n";
+        auto ic = oc;
+        ic[d.axis] = "kk";
+        k << "        const float x = " << em.load_expr(fk.inputs[0], em.index_expr(v, ic)) << ";\n";
+        k << "        acc = " << combine("acc", "x") << ";\n    }\n    }\n";
+        if (TK > 1) {
+            k << "    red[threadIdx.x] = acc;\n    __syncthreads();\n";
+            k << "    if (tk == 0 && oid < " << S(n_out) << "u) {\n";
+            k << "        for (int j = 1; j < " << TK << "; ++j) acc = " << combine("acc", "red[j * " + S(TO) + " + to]") << ";\n";
+            k << "        b" << fk.outputs[0] << "[oid] = acc;\n    }\n}\n";
+        } else {
+            k << "    if (oid < " << S(n_out) << "u) b" << fk.outputs[0] << "[oid] = acc;\n}\n";
+        }
+        out->grid = blocks_for(n_out, (int)TO);
+        out->note = "reduce: lanes along outputs, k split " + S(TK);
+    }
+    out->block = 256;
+    out->source = k.str();
+    return "";
+}
+
+string gen_unpad(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const dsc_view& v = d.inputs[0];
+    const int64_t n = element_count(d.shape);
+    std::ostringstream k;
+    k << "extern \"C\" __global__ __launch_bounds__(256) void dsc_kernel(" << em.params_decl() << ") {\n";
+    k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n";
+    auto c = em.emit_coords(k, d.shape, "gid", "c");
+    const string oc = c[d.axis];
+    k << "    const int in_c = " << oc << " + " << d.pad << ";\n";
+    k << "    const int k_min = in_c - ((" << oc << " == 0) ? " << d.pad << " : 0);\n";
+    k << "    const int k_max = in_c + ((" << oc << " == " << S(d.shape.dims[d.axis] - 1) << ") ? " << d.pad << " : 0);\n";
+    k << "    float sum = 0.f;\n    for (int kk = k_min; kk <= k_max; ++kk) {\n";
+    auto ic = c;
+    ic[d.axis] = "kk";
+    k << "        sum += " << em.load_expr(fk.inputs[0], em.index_expr(v, ic)) << ";\n    }\n";
+    k << "    b" << fk.outputs[0] << "[gid] = sum;\n}\n";
+    out->grid = blocks_for(n, 256);
+    out->block = 256;
+    out->source = k.str();
+    out->note = "unpad";
+    return "";
+}
+
+string gen_windows_to_image(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const dsc_view& v = d.inputs[0];
+    const int r = v.out_shape.rank;
+    const int64_t out_h = v.out_shape.dims[r - 6], out_w = v.out_shape.dims[r - 5];
+    const int64_t fh = v.out_shape.dims[r - 3], fw = v.out_shape.dims[r - 2], group_nc = v.out_shape.dims[r - 1];
+    const int64_t sw = d.stride_w, sh = d.stride_h;
+    const int bd = d.shape.rank - 3;
+    const int64_t n = element_count(d.shape);
+    std::ostringstream k;
+    k << "extern \"C\" __global__ __launch_bounds__(256) void dsc_kernel(" << em.params_decl() << ") {\n";
+    k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n";
+    auto c = em.emit_coords(k, d.shape, "gid", "c");
+    k << "    const int in_y = " << c[bd] << ", in_x = " << c[bd + 1] << ", in_c = " << c[bd + 2] << ";\n";
+    k << "    const int group_index = in_c / " << S(group_nc) << ", group_c = in_c % " << S(group_nc) << ";\n";
+    k << "    const int fbx = in_x % " << S(sw) << ", fby = in_y % " << S(sh) << ";\n";
+    k << "    const int oxb = in_x / " << S(sw) << ", oyb = in_y / " << S(sh) << ";\n";
+    k << "    float tmp = 0.f;\n";
+    k << "#pragma unroll\n    for (int iy = 0; iy < " << S((fh + sh - 1) / sh) << "; ++iy)\n";
+    k << "#pragma unroll\n    for (int ix = 0; ix < " << S((fw + sw - 1) / sw) << "; ++ix) {\n";
+    k << "        const int fx = fbx + " << S(sw) << " * ix, fy = fby + " << S(sh) << " * iy;\n";
+    k << "        const int ox = oxb - ix, oy = oyb - iy;\n";
+    // the window must exist: the reference omits the ox/oy test (kernel.rs:775-776); the true adjoint needs it
+    k << "        if (fx < " << S(fw) << " && fy < " << S(fh) << " && ox >= 0 && ox < " << S(out_w) << " && oy >= 0 && oy < "
+      << S(out_h) << ") {\n";
+    std::vector<string> ic(r);
+    for (int i = 0; i < bd; ++i) ic[i] = c[i];
+    ic[bd] = "oy"; ic[bd + 1] = "ox"; ic[bd + 2] = "group_index"; ic[bd + 3] = "fy"; ic[bd + 4] = "fx"; ic[bd + 5] = "group_c";
+    k << "            tmp += " << em.load_expr(fk.inputs[0], em.index_expr(v, ic)) << ";\n        }\n    }\n";
+    k << "    b" << fk.outputs[0] << "[gid] = tmp;\n}\n";
+    out->grid = blocks_for(n, 256);
+    out->block = 256;
+    out->source = k.str();
+    out->note = "windows_to_image";
+    return "";
+}
+
+string gen_scatter_add(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const dsc_view& vv = d.inputs[0];
+    const dsc_view& vi = d.inputs[1];
+    const int64_t n = element_count(vv.out_shape);
+    std::ostringstream k;
+    k << "extern \"C\" __global__ __launch_bounds__(256) void dsc_kernel(" << em.params_decl() << ") {\n";
+    k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n";
+    auto c = em.emit_coords(k, vv.out_shape, "gid", "c");
+    k << "    const float value = " << em.load_expr(fk.inputs[0], em.index_expr(vv, c)) << ";\n";
+    k << "    const int si = F2I(" << em.load_expr(fk.inputs[1], em.index_expr(vi, {c[d.axis]})) << ");\n";
+    int64_t st[DSC_MAX_DIM];
+    strides_of(d.shape, st);
+    string idx = "0";
+    for (int i = 0; i < d.shape.rank; ++i) idx += " + " + (i == d.axis ? string("si") : c[i]) + "*" + S(st[i]);
+    // bounds: an index outside the accumulator would be a wild write; the reference has no check, here it is dropped
+    k << "    if (si < 0 || si >= " << S(d.shape.dims[d.axis]) << ") return;\n";
+    k << "    unsafeAtomicAdd(&b" << fk.outputs[0] << "[" << idx << "], value);\n}\n";
+    out->grid = blocks_for(n, 256);
+    out->block = 256;
+    out->source = k.str();
+    out->note = "scatter_add: global_atomic_add_f32";
+    return "";
+}
+
+// ---- matmul -------------------------------------------------------------------------------------------
+
+struct MmConfig {
+    int bm, bn, bk, wm, wn, group_m;
+};
+
+bool config_ok(const MmConfig& c) {
+    if (c.bm <= 0 || c.bn <= 0 || c.bk <= 0 || c.wm <= 0 || c.wn <= 0 || c.group_m <= 0) return false;
+    if (c.bk % 8) return false;
+    if (c.bm % (32 * c.wm) || c.bn % (32 * c.wn)) return false;
+    const int nt = 64 * c.wm * c.wn;
+    if (nt > 1024) return false;
+    if ((c.bm * c.bk) % 4 || (c.bn * c.bk) % 4) return false;
+    const int lds = 2 * 4 * (std::max(c.bm * (c.bk + 4), c.bk * (c.bm + 8)) + std::max(c.bn * (c.bk + 4), c.bk * (c.bn + 8)));
+    if (lds > 64 * 1024) return false;  // static __shared__ limit
+    const int acc = (c.bm / c.wm / 32) * (c.bn / c.wn / 32) * 16;
+    return acc <= 256;
+}
+
+MmConfig pick_config(int64_t M, int64_t N) {
+    MmConfig c{};
+    c.bk = 16;
+    c.group_m = 8;
+    c.bm = M <= 32 ? 32 : (M <= 64 ? 64 : 128);
+    c.bn = N <= 32 ? 32 : (N <= 64 ? 64 : 128);
+    if (c.bm == 128 && c.bn == 128) { c.wm = 2; c.wn = 2; }
+    else if (c.bm == 128 && c.bn == 64) { c.wm = 2; c.wn = 2; }
+    else if (c.bm == 128 && c.bn == 32) { c.wm = 4; c.wn = 1; }
+    else if (c.bm == 64 && c.bn == 128) { c.wm = 2; c.wn = 2; }
+    else if (c.bm == 64 && c.bn == 64) { c.wm = 2; c.wn = 2; }
+    else if (c.bm == 64 && c.bn == 32) { c.wm = 2; c.wn = 1; }
+    else if (c.bm == 32 && c.bn == 128) { c.wm = 1; c.wn = 4; }
+    else if (c.bm == 32 && c.bn == 64) { c.wm = 1; c.wn = 2; }
+    else { c.wm = 1; c.wn = 1; }
+    // tuning hook: DSC_MM_TILE="BM,BN,BK,WAVES_M,WAVES_N,GROUP_M" for products at least one tile large
+    if (const char* env = std::getenv("DSC_MM_TILE")) {
+        MmConfig e{};
+        if (std::sscanf(env, "%d,%d,%d,%d,%d,%d", &e.bm, &e.bn, &e.bk, &e.wm, &e.wn, &e.group_m) == 6 && config_ok(e) &&
+            M >= e.bm && N >= e.bn)
+            c = e;
+    }
+    return c;
+}
+
+string gen_matmul(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const MatMulDims g = matmul_dims(d);
+    const dsc_view& va = d.inputs[0];
+    const dsc_view& vb = d.inputs[1];
+    const bool rows = d.output_mode == DSC_MATMUL_ROWS;
+    MmConfig c = pick_config(g.m, g.n);
+
+    // k chunking: the reference writes `chunks` partial products of chunk_tiles*16 k each (kernel.rs:436)
+    int64_t kchunks = 1, chunk_k = ((g.k + c.bk - 1) / c.bk) * c.bk;
+    if (!fk.sum_chunks && g.chunks > 1) {
+        const int64_t k_tiles = (g.k + 15) / 16;
+        const int64_t chunk_tiles = (k_tiles + g.chunks - 1) / g.chunks;
+        chunk_k = chunk_tiles * 16;
+        kchunks = g.chunks;
+        if (chunk_k % c.bk) c.bk = 16;
+    }
+    if (!config_ok(c)) return "matmul: invalid tile configuration";
+
+    // operand addressing
+    int a_mode = 0, b_mode = 0;
+    int64_t a_base = 0, a_coef[DSC_MAX_DIM] = {0}, b_base = 0, b_coef[DSC_MAX_DIM] = {0};
+    const bool a_aff = fk.inputs[0].buffer >= 0 && affine_form(va, &a_base, a_coef);
+    const bool b_aff = fk.inputs[1].buffer >= 0 && affine_form(vb, &b_base, b_coef);
+    auto mult4 = [](int64_t x) { return x % 4 == 0; };
+    if (a_aff && mult4(a_base) && (g.batch == 1 || mult4(a_coef[0]))) {
+        if (a_coef[2] == 1 && mult4(g.k) && mult4(a_coef[1]) && chunk_k % 4 == 0) a_mode = 1;
+        else if (a_coef[1] == 1 && mult4(g.m) && mult4(a_coef[2])) a_mode = 2;
+    }
+    if (b_aff && mult4(b_base) && (g.batch == 1 || mult4(b_coef[0]))) {
+        if (b_coef[2] == 1 && mult4(g.n) && mult4(b_coef[1])) b_mode = 1;
+        else if (b_coef[1] == 1 && mult4(g.k) && mult4(b_coef[2]) && chunk_k % 4 == 0) b_mode = 2;
+    }
+
+    std::ostringstream k;
+    k << "#define MM_B " << S(g.batch) << "\n#define MM_M " << S(g.m) << "\n#define MM_N " << S(g.n) << "\n#define MM_K "
+      << S(g.k) << "\n";
+    k << "#define MM_KCHUNKS " << S(kchunks) << "\n#define MM_CHUNK_K " << S(chunk_k) << "\n";
+    k << "#define BM " << c.bm << "\n#define BN " << c.bn << "\n#define BK " << c.bk << "\n#define WAVES_M " << c.wm
+      << "\n#define WAVES_N " << c.wn << "\n#define GROUP_M " << c.group_m << "\n";
+    k << "#define A_MODE " << a_mode << "\n#define B_MODE " << b_mode << "\n";
+    if (a_mode) {
+        k << "#define A_PTR b" << fk.inputs[0].buffer << "\n#define A_BASE " << S(a_base) << "\n#define A_SB "
+          << S(g.batch == 1 ? 0 : a_coef[0]) << "\n#define A_SM " << S(a_coef[1]) << "\n#define A_SK " << S(a_coef[2]) << "\n";
+    } else {
+        em.funcs << "DSC_INLINE float load_a(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return "
+                 << em.load_expr(fk.inputs[0], em.index_expr(va, {"cb", "cm", "ck"})) << ";\n}\n";
+        k << "#define LOAD_A(b, m, k) load_a(b, m, k, " << em.params_pass() << ")\n";
+    }
+    if (b_mode) {
+        k << "#define B_PTR b" << fk.inputs[1].buffer << "\n#define B_BASE " << S(b_base) << "\n#define B_SB "
+          << S(g.batch == 1 ? 0 : b_coef[0]) << "\n#define B_SK " << S(b_coef[1]) << "\n#define B_SN " << S(b_coef[2]) << "\n";
+    } else {
+        em.funcs << "DSC_INLINE float load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return "
+                 << em.load_expr(fk.inputs[1], em.index_expr(vb, {"cb", "ck", "cn"})) << ";\n}\n";
+        k << "#define LOAD_B(b, k, n) load_b(b, k, n, " << em.params_pass() << ")\n";
+    }
+    const int64_t batch_stride = rows ? g.n : g.m * g.n, row_stride = rows ? g.batch * g.n : g.n;
+    k << "#define C_CHUNK_STRIDE " << S(g.batch * g.m * g.n) << "\n#define C_BATCH_STRIDE " << S(batch_stride)
+      << "\n#define C_ROW_STRIDE " << S(row_stride) << "\n";
+    k << "#define MM_PARAMS " << em.params_decl() << "\n";
+
+    if (fk.has_epilogue) {
+        const dsc_kernel_desc& pe = fk.epilogue.raw();
+        em.funcs << "DSC_INLINE void mm_store(float product, int gid, " << em.params_decl() << ") {\n";
+        std::map<int, string> ov;
+        ov[fk.epilogue_product_input] = "product";
+        em.emit_pe(em.funcs, pe, fk.epilogue_inputs, "gid", "e", ov);
+        for (int o = 0; o < pe.n_outputs; ++o) em.funcs << "    b" << fk.outputs[o] << "[gid] = et" << pe.outputs[o] << ";\n";
+        em.funcs << "}\n";
+        k << "#define MM_STORE(v, idx) mm_store(v, idx, " << em.params_pass() << ")\n";
+    } else {
+        k << "#define MM_STORE(v, idx) b" << fk.outputs[0] << "[idx] = (v)\n";
+    }
+    k << kMatmulMfmaSource;
+
+    const int64_t tiles = ((g.m + c.bm - 1) / c.bm) * ((g.n + c.bn - 1) / c.bn);
+    const int64_t grid = tiles * g.batch * kchunks;
+    if (grid >= kMaxIndex) return "matmul: grid too large";
+    out->grid = (unsigned)grid;
+    out->block = 64 * c.wm * c.wn;
+    out->source = k.str();
+    char note[160];
+    std::snprintf(note, sizeof note, "mfma 32x32x2 tile %dx%dx%d waves %dx%d A%d B%d chunks %lld%s", c.bm, c.bn, c.bk, c.wm, c.wn,
+                  a_mode, b_mode, (long long)kchunks, fk.has_epilogue ? " +epilogue" : "");
+    out->note = note;
+    return "";
+}
+
+}  // namespace
+
+FusedKernel FusedKernel::plain(const dsc_kernel_desc& d) {
+    FusedKernel fk;
+    fk.main = KernelDesc(d);
+    const int n_in = fk.main.raw().n_inputs;
+    int n_out = 1;
+    if (d.kind == DSC_KERNEL_PER_ELEMENT) n_out = d.n_outputs;
+    for (int i = 0; i < n_in; ++i) {
+        Source s;
+        s.buffer = i;
+        fk.inputs.push_back(s);
+    }
+    for (int o = 0; o < n_out; ++o) fk.outputs.push_back(n_in + o);
+    fk.n_buffers = n_in + n_out;
+    fk.buffer_is_output.assign(fk.n_buffers, false);
+    for (int o : fk.outputs) fk.buffer_is_output[o] = true;
+    return fk;
+}
+
+std::string FusedKernel::key() const {
+    std::string s = main.key();
+    auto put_src = [&](const Source& x) {
+        s.append(reinterpret_cast<const char*>(&x.buffer), 4);
+        s.append(reinterpret_cast<const char*>(&x.virt), 4);
+    };
+    s += "|I";
+    for (auto& x : inputs) put_src(x);
+    for (auto& v : virtuals) {
+        s += "|V" + v.pe.key();
+        s.append(reinterpret_cast<const char*>(&v.out_op), 4);
+        for (auto& x : v.inputs) put_src(x);
+    }
+    if (has_epilogue) {
+        s += "|E" + epilogue.key();
+        s.append(reinterpret_cast<const char*>(&epilogue_product_input), 4);
+        for (auto& x : epilogue_inputs) put_src(x);
+    }
+    s += sum_chunks ? "|S1" : "|S0";
+    s += "|O";
+    for (int o : outputs) s.append(reinterpret_cast<const char*>(&o), 4);
+    s.append(reinterpret_cast<const char*>(&n_buffers), 4);
+    if (const char* env = std::getenv("DSC_MM_TILE"))
+        if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|T") + env;
+    return s;
+}
+
+std::string generate(const FusedKernel& fk, Generated* out) {
+    string err = validate(fk.main.raw());
+    if (!err.empty()) return err;
+    for (auto& v : fk.virtuals) {
+        err = validate(v.pe.raw());
+        if (!err.empty()) return "fused producer: " + err;
+        if (v.pe.raw().kind != DSC_KERNEL_PER_ELEMENT) return "fused producer must be a per-element kernel";
+        if ((int)v.inputs.size() != v.pe.raw().n_inputs) return "fused producer: input binding count";
+    }
+    if (fk.has_epilogue) {
+        err = validate(fk.epilogue.raw());
+        if (!err.empty()) return "epilogue: " + err;
+        if (fk.main.raw().kind != DSC_KERNEL_MATMUL) return "only MatMul takes an epilogue";
+    }
+    if ((int)fk.inputs.size() != fk.main.raw().n_inputs) return "input binding count";
+    if ((int)fk.buffer_is_output.size() != fk.n_buffers) return "buffer table size";
+    err = check_sizes(fk);
+    if (!err.empty()) return err;
+
+    Emitter em(fk);
+    em.emit_virtuals();
+    Generated g;
+    switch (fk.main.raw().kind) {
+    case DSC_KERNEL_FILL: err = gen_fill(em, &g); break;
+    case DSC_KERNEL_PER_ELEMENT: err = gen_per_element(em, &g); break;
+    case DSC_KERNEL_REDUCE: err = gen_reduce(em, &g); break;
+    case DSC_KERNEL_MATMUL: err = gen_matmul(em, &g); break;
+    case DSC_KERNEL_UNPAD: err = gen_unpad(em, &g); break;
+    case DSC_KERNEL_WINDOWS_TO_IMAGE: err = gen_windows_to_image(em, &g); break;
+    case DSC_KERNEL_SCATTER_ADD: err = gen_scatter_add(em, &g); break;
+    default: err = "unknown kernel kind";
+    }
+    if (!err.empty()) return err;
+    g.source = string(kPreludeSource) + "\n" + em.funcs.str() + "\n" + g.source;
+    g.n_buffers = fk.n_buffers;
+    *out = g;
+    return "";
+}
+
+const std::vector<std::string>& compile_options() {
+    // packed fp32 instructions are kept off for every kernel; float atomicAdd maps to the hardware instruction
+    static const std::vector<std::string> opts = {"-O3", "-munsafe-fp-atomics", "-Xclang", "-target-feature",
+                                                  "-Xclang", "-packed-fp32-ops", "-std=c++17"};
+    return opts;
+}
+
+}  // namespace dsc

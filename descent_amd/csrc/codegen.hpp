@@ -1,0 +1,70 @@
+// HIP C++ source generation for kernel descriptors.  Counterpart of the reference's `generate_source`
+// implementations (src/kernel.rs:151-857): every shape, stride and offset is baked into the text as a
+// literal, so each distinct kernel is its own translation unit compiled by hipRTC.
+//
+// Beyond the one-descriptor-one-kernel mapping of the reference, the generator accepts a `FusedKernel`:
+// a main descriptor whose inputs may be *virtual* -- a per-element cluster evaluated on demand at the
+// element the main kernel reads (this is how a materialised im2col / pooling-window copy, or any
+// single-consumer elementwise producer, disappears into its consumer) -- and, for MatMul, an epilogue
+// cluster applied to the accumulator before the store (split-K partials are then summed in registers).
+#pragma once
+
+#include "desc.hpp"
+
+#include <string>
+#include <vector>
+
+namespace dsc {
+
+// Where the elements of one kernel input come from.
+struct Source {
+    int buffer = -1;  // index of a pointer parameter of the generated kernel, or
+    int virt = -1;    // index into FusedKernel::virtuals
+};
+
+// A per-element cluster evaluated lazily: value(gid) = ops[out_op] at linear element id `gid`.
+struct Virtual {
+    KernelDesc pe;
+    int out_op = 0;
+    std::vector<Source> inputs;  // one per pe input
+};
+
+struct FusedKernel {
+    KernelDesc main;
+    std::vector<Source> inputs;     // one per main input view
+    std::vector<Virtual> virtuals;  // may reference one another (a virtual's inputs may be virtual), acyclic,
+                                    // each referencing only virtuals with a larger index
+    // MatMul only: per-element cluster applied to the product (all of K accumulated in-kernel)
+    bool has_epilogue = false;
+    KernelDesc epilogue;
+    int epilogue_product_input = -1;       // which epilogue input is the product
+    std::vector<Source> epilogue_inputs;   // one per epilogue input (the product's entry is ignored)
+    bool sum_chunks = false;               // MatMul: ignore the descriptor's chunk count, write one full sum
+    std::vector<int> outputs;              // pointer parameter index of each output of main (or of the epilogue)
+    int n_buffers = 0;                     // number of pointer parameters
+    std::vector<bool> buffer_is_output;    // per pointer parameter
+
+    // The reference binding: inputs then outputs, no fusion.
+    static FusedKernel plain(const dsc_kernel_desc& d);
+    std::string key() const;
+};
+
+struct Generated {
+    std::string source;      // complete translation unit; entry point is `dsc_kernel`
+    unsigned grid = 1;       // workgroups (1-D)
+    unsigned block = 64;     // threads per workgroup
+    int n_buffers = 0;       // pointer parameters, in order; followed by `uint rand_seed`
+    std::string note;        // strategy chosen (for schedule listings)
+};
+
+// Returns "" on success or an error message.
+std::string generate(const FusedKernel& k, Generated* out);
+
+// hipRTC options every kernel is compiled with (after --offload-arch=<arch>).
+const std::vector<std::string>& compile_options();
+
+// The prelude and matmul template texts (embedded at build time from kernels/*.inc).
+extern const char* const kPreludeSource;
+extern const char* const kMatmulMfmaSource;
+
+}  // namespace dsc

@@ -1,0 +1,449 @@
+// Whole-graph schedules: cross-cluster fusion at creation, Environment::run semantics per step.
+#include "schedule.hpp"
+
+#include <algorithm>
+#include <set>
+#include <sstream>
+
+namespace dsc {
+
+namespace {
+
+// One launch being assembled: a fused kernel plus the op node bound to each pointer parameter.
+struct Draft {
+    bool alive = true;
+    FusedKernel fk;
+    std::vector<int> params;      // node id per pointer parameter
+    std::vector<StepOutput> outs; // outputs, parallel to fk.outputs
+    std::vector<int> covers;      // reference cluster indices folded into this launch
+};
+
+int param_index(Draft& d, int node, bool is_output) {
+    for (size_t i = 0; i < d.params.size(); ++i)
+        if (d.params[i] == node && d.fk.buffer_is_output[i] == is_output) return (int)i;
+    d.params.push_back(node);
+    d.fk.buffer_is_output.push_back(is_output);
+    d.fk.n_buffers = (int)d.params.size();
+    return (int)d.params.size() - 1;
+}
+
+// Copies p's virtual producers into q; returns the index offset applied to p's virtual ids.
+int import_virtuals(Draft& q, const Draft& p) {
+    const int offset = (int)q.fk.virtuals.size();
+    for (const Virtual& v : p.fk.virtuals) {
+        Virtual nv = v;
+        for (Source& s : nv.inputs) {
+            if (s.buffer >= 0) s.buffer = param_index(q, p.params[s.buffer], false);
+            else s.virt += offset;
+        }
+        q.fk.virtuals.push_back(nv);
+    }
+    return offset;
+}
+
+Source import_source(Draft& q, const Draft& p, const Source& s, int virt_offset) {
+    Source out;
+    if (s.buffer >= 0) out.buffer = param_index(q, p.params[s.buffer], false);
+    else out.virt = s.virt + virt_offset;
+    return out;
+}
+
+template <class F>
+void for_each_source(FusedKernel& fk, F f) {
+    for (auto& s : fk.inputs) f(s);
+    for (auto& v : fk.virtuals)
+        for (auto& s : v.inputs) f(s);
+    if (fk.has_epilogue)
+        for (size_t i = 0; i < fk.epilogue_inputs.size(); ++i)
+            if ((int)i != fk.epilogue_product_input) f(fk.epilogue_inputs[i]);
+}
+
+// Drops pointer parameters nothing refers to and renumbers the rest.
+void compact(Draft& d) {
+    std::vector<bool> used(d.params.size(), false);
+    for_each_source(d.fk, [&](Source& s) { if (s.buffer >= 0) used[s.buffer] = true; });
+    for (int o : d.fk.outputs) used[o] = true;
+    std::vector<int> remap(d.params.size(), -1);
+    std::vector<int> params;
+    std::vector<bool> is_out;
+    for (size_t i = 0; i < d.params.size(); ++i) {
+        if (!used[i]) continue;
+        remap[i] = (int)params.size();
+        params.push_back(d.params[i]);
+        is_out.push_back(d.fk.buffer_is_output[i]);
+    }
+    for_each_source(d.fk, [&](Source& s) { if (s.buffer >= 0) s.buffer = remap[s.buffer]; });
+    for (int& o : d.fk.outputs) o = remap[o];
+    d.params = params;
+    d.fk.buffer_is_output = is_out;
+    d.fk.n_buffers = (int)params.size();
+}
+
+std::vector<int> input_nodes(const Draft& d) {
+    std::set<int> seen;
+    std::vector<int> out;
+    Draft& md = const_cast<Draft&>(d);
+    for_each_source(md.fk, [&](Source& s) {
+        if (s.buffer >= 0 && seen.insert(d.params[s.buffer]).second) out.push_back(d.params[s.buffer]);
+    });
+    return out;
+}
+
+bool is_cheap_producer(const dsc_kernel_desc& pe) {
+    // a producer is re-evaluated by each read of its consumer: only inline copies and light arithmetic
+    int work = 0;
+    for (int i = 0; i < pe.n_ops; ++i) {
+        const dsc_pe_op& op = pe.ops[i];
+        if (op.kind == DSC_PE_UNARY && op.op != DSC_UN_MOV && op.op != DSC_UN_NEG) return false;
+        if (op.kind == DSC_PE_BINARY && (op.op == DSC_BIN_DIV || op.op == DSC_BIN_POW || op.op == DSC_BIN_UREM)) return false;
+        if (op.kind == DSC_PE_GATHER || op.kind == DSC_PE_RAND) return false;
+        if (op.kind == DSC_PE_LOAD) work += 2;
+        else if (op.kind == DSC_PE_UNARY || op.kind == DSC_PE_BINARY || op.kind == DSC_PE_SELECT) work += 1;
+    }
+    return work <= 12;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------------------
+
+int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags) {
+    n_nodes = desc.n_nodes;
+    n_params = desc.n_params;
+    n_clusters = desc.n_clusters;
+    node_bytes.assign(n_nodes, 0);
+    for (int i = 0; i < n_nodes; ++i) node_bytes[i] = (size_t)desc.node_elements[i] * 4;
+    inputs.assign(desc.inputs, desc.inputs + desc.n_inputs);
+    outputs.assign(desc.outputs, desc.outputs + desc.n_outputs);
+    for (auto& io : inputs)
+        if (io.node < 0 || io.node >= n_nodes || io.param < 0 || io.param >= n_params) return fail(DSC_ERR_INVALID, "schedule: bad input entry");
+    for (auto& io : outputs)
+        if (io.node < 0 || io.node >= n_nodes || io.param < 0 || io.param >= n_params) return fail(DSC_ERR_INVALID, "schedule: bad output entry");
+
+    std::vector<bool> is_graph_output(n_nodes, false), is_graph_input(n_nodes, false);
+    for (auto& io : outputs) is_graph_output[io.node] = true;
+    for (auto& io : inputs) is_graph_input[io.node] = true;
+
+    // one draft per reference cluster
+    std::vector<Draft> drafts(desc.n_clusters);
+    for (int c = 0; c < desc.n_clusters; ++c) {
+        const dsc_cluster& cl = desc.clusters[c];
+        std::string err = validate(cl.kernel);
+        if (!err.empty()) return fail(DSC_ERR_INVALID, "schedule: cluster " + std::to_string(c) + ": " + err);
+        const int want_in = cl.kernel.kind == DSC_KERNEL_FILL ? 0 : cl.kernel.n_inputs;
+        const int want_out = cl.kernel.kind == DSC_KERNEL_PER_ELEMENT ? cl.kernel.n_outputs : 1;
+        if (cl.n_inputs != want_in || cl.n_outputs != want_out)
+            return fail(DSC_ERR_INVALID, "schedule: cluster " + std::to_string(c) + " binds the wrong number of nodes");
+        Draft& d = drafts[c];
+        d.fk = FusedKernel::plain(cl.kernel);
+        for (int i = 0; i < cl.n_inputs; ++i) {
+            if (cl.inputs[i] < 0 || cl.inputs[i] >= n_nodes) return fail(DSC_ERR_INVALID, "schedule: bad node id");
+            d.params.push_back(cl.inputs[i]);
+        }
+        for (int o = 0; o < cl.n_outputs; ++o) {
+            const dsc_cluster_output& co = cl.outputs[o];
+            if (co.node < 0 || co.node >= n_nodes || co.copy_from >= n_nodes) return fail(DSC_ERR_INVALID, "schedule: bad node id");
+            d.params.push_back(co.node);
+            d.outs.push_back(StepOutput{co.node, co.copy_from, co.copy_from_is_literal != 0, co.literal_bits});
+        }
+        d.covers.push_back(c);
+    }
+
+    if (!(flags & DSC_SCHEDULE_NO_FUSION)) {
+        auto consumers_of = [&](int node) {
+            std::vector<int> out;
+            for (int i = 0; i < (int)drafts.size(); ++i) {
+                if (!drafts[i].alive) continue;
+                auto ins = input_nodes(drafts[i]);
+                if (std::find(ins.begin(), ins.end(), node) != ins.end()) out.push_back(i);
+            }
+            return out;
+        };
+        // no launch between `from` and `to` may take one of `nodes` over in place (ScatterAdd accumulators)
+        auto taken_in_place_between = [&](int from, int to, const std::vector<int>& nodes) {
+            for (int i = from + 1; i < to; ++i) {
+                if (!drafts[i].alive) continue;
+                for (auto& o : drafts[i].outs)
+                    if (o.copy_from >= 0 && std::find(nodes.begin(), nodes.end(), o.copy_from) != nodes.end()) return true;
+            }
+            for (auto& o : drafts[to].outs)
+                if (o.copy_from >= 0 && std::find(nodes.begin(), nodes.end(), o.copy_from) != nodes.end()) return true;
+            return false;
+        };
+
+        // Pass 1: MatMul (+ Reduce over its split-K partials) (+ per-element consumer as epilogue).
+        for (int i = 0; i < (int)drafts.size(); ++i) {
+            Draft& mm = drafts[i];
+            if (!mm.alive || mm.fk.main.raw().kind != DSC_KERNEL_MATMUL || mm.fk.has_epilogue) continue;
+            const MatMulDims g = matmul_dims(mm.fk.main.raw());
+            int product_node = mm.outs[0].node;
+            if (is_graph_output[product_node]) continue;
+            int reduce_idx = -1;
+            if (g.chunks > 1) {
+                // summing all of K in one workgroup per tile serialises the k loop: only do it when the tile
+                // grid alone fills the machine, or the partials are few
+                const int64_t tile_groups = ((g.m + 127) / 128) * ((g.n + 127) / 128) * g.batch;
+                if (tile_groups < 64 && g.chunks > 4) continue;
+                auto cons = consumers_of(product_node);
+                if (cons.size() != 1) continue;
+                Draft& r = drafts[cons[0]];
+                const dsc_kernel_desc& rd = r.fk.main.raw();
+                if (rd.kind != DSC_KERNEL_REDUCE || rd.reduce_op != DSC_REDUCE_SUM || rd.axis != 0 || !r.fk.virtuals.empty()) continue;
+                if (!is_identity(rd.inputs[0]) || element_count(rd.inputs[0].in_shape) != g.chunks * g.batch * g.m * g.n) continue;
+                if (taken_in_place_between(i, cons[0], input_nodes(mm))) continue;
+                reduce_idx = cons[0];
+                product_node = r.outs[0].node;
+            }
+            // optional epilogue
+            int pe_idx = -1, pe_input = -1;
+            if (!is_graph_output[product_node]) {
+                auto cons = consumers_of(product_node);
+                if (cons.size() == 1) {
+                    Draft& e = drafts[cons[0]];
+                    const dsc_kernel_desc& ed = e.fk.main.raw();
+                    if (ed.kind == DSC_KERNEL_PER_ELEMENT && ed.shape.dims[0] == g.batch * g.m * g.n) {
+                        int hits = 0;
+                        for (int k = 0; k < ed.n_inputs; ++k) {
+                            if (e.fk.inputs[k].buffer >= 0 && e.params[e.fk.inputs[k].buffer] == product_node) {
+                                ++hits;
+                                pe_input = k;
+                            }
+                        }
+                        bool only_loaded = true;  // the product must be read element-for-element, not gathered
+                        for (int k = 0; k < ed.n_ops; ++k)
+                            if (ed.ops[k].kind == DSC_PE_GATHER && ed.ops[k].input_index == pe_input) only_loaded = false;
+                        // and not through one of the consumer's own fused producers
+                        bool via_virtual = false;
+                        for (auto& v : e.fk.virtuals)
+                            for (auto& s : v.inputs)
+                                if (s.buffer >= 0 && e.params[s.buffer] == product_node) via_virtual = true;
+                        if (hits == 1 && only_loaded && !via_virtual && is_contiguous(ed.inputs[pe_input]) &&
+                            !taken_in_place_between(i, cons[0], input_nodes(mm)))
+                            pe_idx = cons[0];
+                    }
+                }
+            }
+            if (reduce_idx < 0 && pe_idx < 0) continue;
+
+            Draft fused;
+            fused.fk.main = mm.fk.main;
+            fused.fk.sum_chunks = true;
+            const int voff = import_virtuals(fused, mm);
+            for (auto& s : mm.fk.inputs) fused.fk.inputs.push_back(import_source(fused, mm, s, voff));
+            fused.covers = mm.covers;
+            if (reduce_idx >= 0) fused.covers.insert(fused.covers.end(), drafts[reduce_idx].covers.begin(), drafts[reduce_idx].covers.end());
+            if (pe_idx >= 0) {
+                Draft& e = drafts[pe_idx];
+                fused.fk.has_epilogue = true;
+                fused.fk.epilogue = e.fk.main;
+                fused.fk.epilogue_product_input = pe_input;
+                const int eoff = import_virtuals(fused, e);
+                for (int k = 0; k < (int)e.fk.inputs.size(); ++k) {
+                    if (k == pe_input) fused.fk.epilogue_inputs.push_back(Source{});
+                    else fused.fk.epilogue_inputs.push_back(import_source(fused, e, e.fk.inputs[k], eoff));
+                }
+                for (auto& o : e.outs) {
+                    fused.fk.outputs.push_back(param_index(fused, o.node, true));
+                    fused.outs.push_back(o);
+                }
+                fused.covers.insert(fused.covers.end(), e.covers.begin(), e.covers.end());
+                compact(fused);
+                mm.alive = false;
+                if (reduce_idx >= 0) drafts[reduce_idx].alive = false;
+                drafts[pe_idx] = fused;  // runs where the per-element cluster ran: all of its inputs exist by then
+            } else {
+                Draft& r = drafts[reduce_idx];
+                fused.fk.outputs.push_back(param_index(fused, r.outs[0].node, true));
+                fused.outs.push_back(r.outs[0]);
+                compact(fused);
+                mm.alive = false;
+                drafts[reduce_idx] = fused;
+            }
+        }
+
+        // Pass 2: per-element producers whose result need not exist in memory are evaluated inside their
+        // consumers: pure copies (materialised im2col / pooling windows) into every consumer, light arithmetic
+        // into a single consumer.
+        auto is_pure_copy = [](const dsc_kernel_desc& pe) {
+            int loads = 0;
+            for (int i = 0; i < pe.n_ops; ++i) {
+                if (pe.ops[i].kind == DSC_PE_LOAD) ++loads;
+                else if (!(pe.ops[i].kind == DSC_PE_UNARY && pe.ops[i].op == DSC_UN_MOV)) return false;
+            }
+            return loads == 1;
+        };
+        bool changed = true;
+        while (changed) {
+            changed = false;
+            for (int i = 0; i < (int)drafts.size() && !changed; ++i) {
+                Draft& p = drafts[i];
+                if (!p.alive) continue;
+                const dsc_kernel_desc& pd = p.fk.main.raw();
+                if (pd.kind != DSC_KERNEL_PER_ELEMENT || pd.n_outputs != 1 || p.fk.has_epilogue) continue;
+                const int node = p.outs[0].node;
+                if (is_graph_output[node] || p.outs[0].copy_from >= 0) continue;
+                if (!is_cheap_producer(pd)) continue;
+                auto cons = consumers_of(node);
+                if (cons.empty() || (cons.size() > 1 && !is_pure_copy(pd))) continue;
+                bool ok = true;
+                for (int ci : cons) {
+                    Draft& q = drafts[ci];
+                    if (ci <= i) ok = false;
+                    for (auto& o : q.outs)
+                        if (o.copy_from == node) ok = false;  // updated in place by the consumer
+                    if (taken_in_place_between(i, ci, input_nodes(p))) ok = false;
+                    if ((int)q.fk.virtuals.size() + (int)p.fk.virtuals.size() + 1 > 8) ok = false;
+                    // an epilogue reads its product from the accumulator, never through a producer
+                    if (q.fk.has_epilogue && q.fk.epilogue_product_input >= 0) {
+                        const Source& ps = q.fk.epilogue_inputs[q.fk.epilogue_product_input];
+                        if (ps.buffer >= 0 && q.params[ps.buffer] == node) ok = false;
+                    }
+                }
+                if (!ok) continue;
+                for (int ci : cons) {
+                    Draft& q = drafts[ci];
+                    const int new_virt = (int)q.fk.virtuals.size();
+                    q.fk.virtuals.emplace_back();
+                    const int voff = import_virtuals(q, p);
+                    {
+                        Virtual nv;
+                        nv.pe = p.fk.main;
+                        nv.out_op = pd.outputs[0];
+                        for (auto& s : p.fk.inputs) nv.inputs.push_back(import_source(q, p, s, voff));
+                        q.fk.virtuals[new_virt] = nv;
+                    }
+                    for_each_source(q.fk, [&](Source& s) {
+                        if (s.buffer >= 0 && q.params[s.buffer] == node && !q.fk.buffer_is_output[s.buffer]) {
+                            s.buffer = -1;
+                            s.virt = new_virt;
+                        }
+                    });
+                    q.covers.insert(q.covers.end(), p.covers.begin(), p.covers.end());
+                    compact(q);
+                }
+                p.alive = false;
+                changed = true;
+            }
+        }
+    }
+
+    // materialise the steps
+    for (auto& d : drafts) {
+        if (!d.alive) continue;
+        Step st;
+        int status = DSC_OK;
+        st.kernel = get_kernel(ctx, d.fk, &status);
+        if (!st.kernel) return status;
+        st.params = d.params;
+        st.inputs = input_nodes(d);
+        st.outputs = d.outs;
+        st.covers = d.covers;
+        for (auto& o : st.outputs) {
+            if (o.copy_from >= 0 && o.from_literal) {
+                dsc_kernel_desc fd{};
+                fd.kind = DSC_KERNEL_FILL;
+                fd.shape.rank = 1;
+                fd.shape.dims[0] = (int64_t)(node_bytes[o.node] / 4);
+                fd.fill_bits = o.literal_bits;
+                o.fill = get_kernel(ctx, FusedKernel::plain(fd), &status);
+                if (!o.fill) return status;
+            }
+        }
+        steps.push_back(st);
+    }
+    return DSC_OK;
+}
+
+int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
+    // environment.rs:326-516, over the fused steps
+    std::vector<int> usage(n_nodes, 0);
+    std::vector<dsc_buf> buffer(n_nodes, 0);
+    for (auto& st : steps)
+        for (int n : st.inputs) usage[n] += 1;
+
+    std::vector<bool> param_is_output(n_params, false), param_is_input(n_params, false);
+    for (auto& io : outputs) param_is_output[io.param] = true;
+    for (auto& io : inputs) param_is_input[io.param] = true;
+
+    for (auto& io : inputs) {
+        if (params[io.param] == 0) return fail(DSC_ERR_INVALID, "schedule run: an input parameter has no buffer");
+        if (!param_is_output[io.param]) {
+            buffer[io.node] = params[io.param];
+            usage[io.node] += 1;  // pinned: the parameter keeps its buffer
+        } else {
+            buffer[io.node] = params[io.param];
+            params[io.param] = 0;
+        }
+    }
+    for (auto& io : outputs) {
+        if (!param_is_input[io.param] && params[io.param] != 0) {
+            ctx->heap.free(params[io.param]);
+            params[io.param] = 0;
+        }
+    }
+
+    void* ptrs[64];
+    for (auto& st : steps) {
+        for (int n : st.inputs) usage[n] -= 1;
+        for (auto& o : st.outputs) {
+            dsc_buf h = 0;
+            if (o.copy_from < 0) {
+                h = ctx->heap.alloc(node_bytes[o.node]);
+                if (!h) return fail(DSC_ERR_OOM, "schedule run: out of device memory");
+            } else {
+                if (usage[o.copy_from] != 0) return fail(DSC_ERR_UNSUPPORTED, "schedule run: accumulator source still in use (deep copy)");
+                if (buffer[o.copy_from] != 0) {
+                    h = buffer[o.copy_from];
+                    buffer[o.copy_from] = 0;
+                } else if (o.from_literal) {
+                    h = ctx->heap.alloc(node_bytes[o.node]);
+                    if (!h) return fail(DSC_ERR_OOM, "schedule run: out of device memory");
+                    void* p = nullptr;
+                    ctx->heap.info(h, &p, nullptr);
+                    int rc = launch_kernel(ctx, o.fill, &p, 1, rand_seed);
+                    if (rc != DSC_OK) return rc;
+                } else {
+                    return fail(DSC_ERR_INVALID, "schedule run: cannot copy-on-write node");
+                }
+            }
+            if (buffer[o.node] != 0) return fail(DSC_ERR_INVALID, "schedule run: node written twice");
+            buffer[o.node] = h;
+        }
+        const int n = (int)st.params.size();
+        for (int i = 0; i < n; ++i) {
+            void* p = nullptr;
+            if (!ctx->heap.info(buffer[st.params[i]], &p, nullptr))
+                return fail(DSC_ERR_INVALID, "schedule run: node " + std::to_string(st.params[i]) + " has no buffer at '" + st.kernel->label + "'");
+            ptrs[i] = p;
+        }
+        int rc = launch_kernel(ctx, st.kernel, ptrs, n, rand_seed);
+        if (rc != DSC_OK) return rc;
+        for (int nd : st.inputs) {
+            if (usage[nd] == 0 && buffer[nd] != 0) {
+                ctx->heap.free(buffer[nd]);
+                buffer[nd] = 0;
+            }
+        }
+    }
+    for (auto& io : outputs) {
+        if (buffer[io.node] == 0) return fail(DSC_ERR_INVALID, "schedule run: output node has no buffer");
+        params[io.param] = buffer[io.node];
+        buffer[io.node] = 0;
+    }
+    return DSC_OK;
+}
+
+std::string Schedule::describe() const {
+    std::ostringstream o;
+    o << steps.size() << " launches for " << n_clusters << " clusters\n";
+    for (size_t i = 0; i < steps.size(); ++i) {
+        const Step& st = steps[i];
+        o << i << ": " << st.kernel->label << "  [" << st.kernel->gen.note << "] grid " << st.kernel->gen.grid << "x"
+          << st.kernel->gen.block << " clusters";
+        for (int c : st.covers) o << " " << c;
+        o << "\n";
+    }
+    return o.str();
+}
+
+}  // namespace dsc

@@ -1,0 +1,36 @@
+// A whole graph's clusters, fused where profitable, executed with Environment::run's buffer discipline
+// (src/environment.rs:326-516).
+#pragma once
+
+#include "runtime.hpp"
+
+namespace dsc {
+
+struct StepOutput {
+    int node;
+    int copy_from;      // -1: fresh allocation (InitialState::Undefined)
+    bool from_literal;  // copy_from is a Literal node: Fill a fresh buffer when no buffer can be taken over
+    uint32_t literal_bits;
+    Kernel* fill = nullptr;
+};
+
+struct Step {
+    Kernel* kernel = nullptr;
+    std::vector<int> params;   // op node bound to each pointer parameter of the kernel
+    std::vector<int> inputs;   // distinct nodes read (use counting)
+    std::vector<StepOutput> outputs;
+    std::vector<int> covers;   // reference cluster indices this launch stands for
+};
+
+struct Schedule {
+    int n_nodes = 0, n_params = 0, n_clusters = 0;
+    std::vector<size_t> node_bytes;
+    std::vector<dsc_param_io> inputs, outputs;
+    std::vector<Step> steps;
+
+    int build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags);
+    int run(Context* ctx, dsc_buf* params, uint32_t rand_seed);
+    std::string describe() const;
+};
+
+}  // namespace dsc

@@ -1,0 +1,252 @@
+"""ctypes binding of libdescent_hip.so (the C ABI in include/descent_hip.h) and
+the backend object `Environment` drives.
+
+There is no CPU fallback: if the library is missing, or no gfx950 device is
+present, constructing `HipBackend` raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import List
+
+import numpy as np
+
+from . import _abi
+
+_CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+LIB_PATH = os.path.join(_CSRC, "libdescent_hip.so")
+
+_lib = None
+
+
+class DescentHipError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"descent_hip error {status} ({_abi.STATUS_NAMES[status] if 0 <= status < 7 else '?'}): {message}")
+        self.status = status
+
+
+def lib():
+    """Loads the built library; raises if it has not been built (python -m descent_amd.csrc.build)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise FileNotFoundError(
+            f"{LIB_PATH} is missing: build it with `python {os.path.join(_CSRC, 'build.py')}` "
+            "(there is no CPU fallback for the HIP backend)"
+        )
+    L = C.CDLL(LIB_PATH)
+    vp, u64, sz, i32, u32 = C.c_void_p, C.c_uint64, C.c_size_t, C.c_int32, C.c_uint32
+    sig = {
+        "dsc_last_error": (C.c_char_p, []),
+        "dsc_ctx_create": (C.c_int, [C.c_int, C.POINTER(vp)]),
+        "dsc_ctx_destroy": (C.c_int, [vp]),
+        "dsc_ctx_caps": (C.c_int, [vp, C.POINTER(_abi.CCaps)]),
+        "dsc_ctx_sync": (C.c_int, [vp]),
+        "dsc_ctx_stream": (C.c_int, [vp, C.POINTER(vp)]),
+        "dsc_buf_alloc": (C.c_int, [vp, sz, C.POINTER(u64)]),
+        "dsc_buf_free": (C.c_int, [vp, u64]),
+        "dsc_buf_info": (C.c_int, [vp, u64, C.POINTER(vp), C.POINTER(sz)]),
+        "dsc_heap_stats": (C.c_int, [vp, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
+        "dsc_buf_write": (C.c_int, [vp, u64, sz, vp, sz]),
+        "dsc_buf_fill_zero": (C.c_int, [vp, u64, sz, sz]),
+        "dsc_buf_read": (C.c_int, [vp, u64, sz, vp, sz]),
+        "dsc_kernel_get": (C.c_int, [vp, C.POINTER(_abi.CKernelDesc), C.POINTER(vp)]),
+        "dsc_kernel_buffer_count": (C.c_int, [vp]),
+        "dsc_kernel_reference_group_count": (C.c_int64, [vp]),
+        "dsc_kernel_label": (C.c_char_p, [vp]),
+        "dsc_kernel_source": (C.c_char_p, [vp]),
+        "dsc_kernel_launch": (C.c_int, [vp, vp, C.POINTER(u64), C.c_int, u32]),
+        "dsc_codegen_source": (C.c_int, [C.POINTER(_abi.CKernelDesc), C.POINTER(vp)]),
+        "dsc_codegen_compile": (C.c_int, [C.POINTER(_abi.CKernelDesc), C.c_char_p, C.POINTER(sz)]),
+        "dsc_codegen_check_schedule": (C.c_int, [C.POINTER(_abi.CScheduleDesc), u32, C.c_char_p, C.POINTER(vp)]),
+        "dsc_free_string": (None, [vp]),
+        "dsc_schedule_create": (C.c_int, [vp, C.POINTER(_abi.CScheduleDesc), u32, C.POINTER(vp)]),
+        "dsc_schedule_destroy": (C.c_int, [vp, vp]),
+        "dsc_schedule_run": (C.c_int, [vp, vp, C.POINTER(u64), u32]),
+        "dsc_schedule_launch_count": (C.c_int, [vp, C.POINTER(i32), C.POINTER(i32)]),
+        "dsc_schedule_describe": (C.c_int, [vp, C.POINTER(vp)]),
+        "dsc_prof_enable": (C.c_int, [vp, C.c_int]),
+        "dsc_prof_reset": (C.c_int, [vp]),
+        "dsc_prof_report": (C.c_int, [vp, C.c_int, C.POINTER(vp)]),
+        "dsc_prof_query": (C.c_int, [vp, C.c_char_p, C.POINTER(C.c_double), C.POINTER(C.c_int64)]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(L, name)
+        fn.restype, fn.argtypes = res, args
+    _lib = L
+    return L
+
+
+EXPORTED_SYMBOLS = [
+    "dsc_last_error", "dsc_ctx_create", "dsc_ctx_destroy", "dsc_ctx_caps", "dsc_ctx_sync", "dsc_ctx_stream",
+    "dsc_buf_alloc", "dsc_buf_free", "dsc_buf_info", "dsc_heap_stats", "dsc_buf_write", "dsc_buf_fill_zero",
+    "dsc_buf_read", "dsc_kernel_get", "dsc_kernel_buffer_count", "dsc_kernel_reference_group_count",
+    "dsc_kernel_label", "dsc_kernel_source", "dsc_kernel_launch", "dsc_codegen_source", "dsc_codegen_compile",
+    "dsc_codegen_check_schedule", "dsc_free_string", "dsc_schedule_create", "dsc_schedule_destroy",
+    "dsc_schedule_run", "dsc_schedule_launch_count", "dsc_schedule_describe", "dsc_prof_enable", "dsc_prof_reset",
+    "dsc_prof_report", "dsc_prof_query",
+]
+
+
+def check(status: int) -> None:
+    if status != 0:
+        raise DescentHipError(status, lib().dsc_last_error().decode(errors="replace"))
+
+
+def _take_string(p: C.c_void_p) -> str:
+    text = C.string_at(p).decode(errors="replace")
+    lib().dsc_free_string(p)
+    return text
+
+
+# -- device-free code generation (CPU tests) -----------------------------------------------------------
+def codegen_source(kernel) -> str:
+    mk = _abi.MarshalledKernel(kernel)
+    out = C.c_void_p()
+    check(lib().dsc_codegen_source(C.byref(mk.desc), C.byref(out)))
+    return _take_string(out)
+
+
+def codegen_compile(kernel, arch: str = "gfx950") -> int:
+    mk = _abi.MarshalledKernel(kernel)
+    n = C.c_size_t()
+    check(lib().dsc_codegen_compile(C.byref(mk.desc), arch.encode(), C.byref(n)))
+    return n.value
+
+
+def check_schedule(graph, fused: bool = True, arch: str = "gfx950") -> str:
+    """Plans and compiles every kernel of a graph's schedule without a GPU; returns the listing."""
+    ms = _abi.MarshalledSchedule(graph)
+    out = C.c_void_p()
+    flags = 0 if fused else _abi.SCHEDULE_NO_FUSION
+    check(lib().dsc_codegen_check_schedule(C.byref(ms.desc), flags, arch.encode(), C.byref(out)))
+    return _take_string(out)
+
+
+class HipSchedule:
+    def __init__(self, backend: "HipBackend", graph, fused: bool):
+        self._backend = backend
+        self._ms = _abi.MarshalledSchedule(graph)
+        self.params = self._ms.params
+        self._handle = C.c_void_p()
+        flags = 0 if fused else _abi.SCHEDULE_NO_FUSION
+        check(lib().dsc_schedule_create(backend._ctx, C.byref(self._ms.desc), flags, C.byref(self._handle)))
+        self._slots = (C.c_uint64 * max(1, len(self.params)))()
+
+    def run(self, handles: List[int], rand_seed: int) -> List[int]:
+        for i, h in enumerate(handles):
+            self._slots[i] = h or 0
+        check(lib().dsc_schedule_run(self._backend._ctx, self._handle, self._slots, rand_seed & 0xFFFFFFFF))
+        return [self._slots[i] or None for i in range(len(handles))]
+
+    def launch_count(self):
+        a, b = C.c_int32(), C.c_int32()
+        check(lib().dsc_schedule_launch_count(self._handle, C.byref(a), C.byref(b)))
+        return a.value, b.value
+
+    def describe(self) -> str:
+        out = C.c_void_p()
+        check(lib().dsc_schedule_describe(self._handle, C.byref(out)))
+        return _take_string(out)
+
+
+class HipBackend:
+    def __init__(self, device: int = 0):
+        self._ctx = C.c_void_p()
+        check(lib().dsc_ctx_create(device, C.byref(self._ctx)))
+        self._kernels = {}
+
+    def close(self):
+        if self._ctx:
+            lib().dsc_ctx_destroy(self._ctx)
+            self._ctx = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # -- memory ---------------------------------------------------------------------------------------
+    def alloc(self, nbytes: int) -> int:
+        h = C.c_uint64()
+        check(lib().dsc_buf_alloc(self._ctx, nbytes, C.byref(h)))
+        return h.value
+
+    def free(self, handle: int) -> None:
+        check(lib().dsc_buf_free(self._ctx, handle))
+
+    def write(self, handle: int, offset: int, data) -> None:
+        arr = np.ascontiguousarray(data) if isinstance(data, np.ndarray) else np.frombuffer(bytes(data), dtype=np.uint8)
+        check(lib().dsc_buf_write(self._ctx, handle, offset, arr.ctypes.data, arr.nbytes))
+
+    def fill_zero(self, handle: int, offset: int, nbytes: int) -> None:
+        check(lib().dsc_buf_fill_zero(self._ctx, handle, offset, nbytes))
+
+    def read(self, handle: int, offset: int, nbytes: int) -> bytes:
+        out = np.empty(nbytes, dtype=np.uint8)
+        check(lib().dsc_buf_read(self._ctx, handle, offset, out.ctypes.data, nbytes))
+        return out.tobytes()
+
+    def device_ptr(self, handle: int) -> int:
+        p, n = C.c_void_p(), C.c_size_t()
+        check(lib().dsc_buf_info(self._ctx, handle, C.byref(p), C.byref(n)))
+        return p.value
+
+    def heap_stats(self):
+        a, b, c = C.c_int64(), C.c_int64(), C.c_int64()
+        check(lib().dsc_heap_stats(self._ctx, C.byref(a), C.byref(b), C.byref(c)))
+        return a.value, b.value, c.value
+
+    def caps(self) -> _abi.CCaps:
+        caps = _abi.CCaps()
+        check(lib().dsc_ctx_caps(self._ctx, C.byref(caps)))
+        return caps
+
+    def stream(self) -> int:
+        p = C.c_void_p()
+        check(lib().dsc_ctx_stream(self._ctx, C.byref(p)))
+        return p.value or 0
+
+    # -- kernels ----------------------------------------------------------------------------------------
+    def kernel(self, kernel):
+        k = self._kernels.get(kernel)
+        if k is None:
+            mk = _abi.MarshalledKernel(kernel)
+            k = C.c_void_p()
+            check(lib().dsc_kernel_get(self._ctx, C.byref(mk.desc), C.byref(k)))
+            self._kernels[kernel] = k
+        return k
+
+    def kernel_source(self, kernel) -> str:
+        return lib().dsc_kernel_source(self.kernel(kernel)).decode()
+
+    def launch(self, kernel, handles, rand_seed: int) -> None:
+        k = self.kernel(kernel)
+        arr = (C.c_uint64 * len(handles))(*handles)
+        check(lib().dsc_kernel_launch(self._ctx, k, arr, len(handles), rand_seed & 0xFFFFFFFF))
+
+    def make_schedule(self, graph, fused: bool = True) -> HipSchedule:
+        return HipSchedule(self, graph, fused)
+
+    def sync(self) -> None:
+        check(lib().dsc_ctx_sync(self._ctx))
+
+    # -- timing -----------------------------------------------------------------------------------------
+    def profile(self, enabled: bool) -> None:
+        check(lib().dsc_prof_enable(self._ctx, 1 if enabled else 0))
+
+    def profile_reset(self) -> None:
+        check(lib().dsc_prof_reset(self._ctx))
+
+    def timing_report(self, top_n: int = 5) -> str:
+        out = C.c_void_p()
+        check(lib().dsc_prof_report(self._ctx, top_n, C.byref(out)))
+        return _take_string(out)
+
+    def timing_query(self, prefix: str):
+        avg, n = C.c_double(), C.c_int64()
+        check(lib().dsc_prof_query(self._ctx, prefix.encode(), C.byref(avg), C.byref(n)))
+        return avg.value, n.value

@@ -205,6 +205,8 @@ int dsc_buf_fill_zero(dsc_ctx* ctx, dsc_buf buf, size_t offset, size_t bytes);
 /* StagingReader::read_slice to completion (device/staging.rs:225-302): device -> host, blocking. */
 int dsc_buf_read(dsc_ctx* ctx, dsc_buf buf, size_t offset, void* dst, size_t bytes);
 
+struct dsc_schedule_desc;
+
 /* ---------------------------------------------------------------- kernels */
 
 /* KernelCache::module (kernel.rs:1050-1055): returns the compiled kernel for a descriptor, generating HIP
@@ -229,6 +231,9 @@ int dsc_codegen_source(const dsc_kernel_desc* desc, char** out_source);
 /* Compiles the generated source for `arch` ("gfx950") with hipRTC; no GPU needed. Returns the code object
  * size through out_code_bytes. */
 int dsc_codegen_compile(const dsc_kernel_desc* desc, const char* arch, size_t* out_code_bytes);
+/* Plans a whole schedule (fusion included) and compiles every kernel it would launch for `arch`, without a
+ * device; out_text (optional) receives the listing dsc_schedule_describe would give. */
+int dsc_codegen_check_schedule(const struct dsc_schedule_desc* desc, uint32_t flags, const char* arch, char** out_text);
 void dsc_free_string(char* s);
 
 /* -------------------------------------------------------------- schedules */
