@@ -88,6 +88,27 @@ def bench_convnet(env, steps, warmup, batch=1000):
     }
 
 
+def bench_elementwise(env, n, steps, warmup):
+    """c = a * 2 + b over n elements: 2 reads + 1 write of 4n bytes each (a plain streaming kernel of known
+    size, also used to calibrate the FETCH_SIZE / WRITE_SIZE counters)."""
+    rng = np.random.Generator(np.random.PCG64(9))
+    a = env.static_parameter([n], "a")
+    b = env.static_parameter([n], "b")
+    c = env.static_parameter([n], "c")
+    env.write_parameter(a, rng.random(n, dtype=np.float32))
+    env.write_parameter(b, rng.random(n, dtype=np.float32))
+    graph = env.build_graph(lambda s: s.write_parameter_value(c, s.parameter_value(a) * 2.0 + s.parameter_value(b)))
+    wall = time_graph(env, graph, steps, warmup)
+    avg_us, launches = env.backend.timing_query("PerElement")
+    env.backend.profile_reset()
+    for p in (a, b, c):
+        env.backend.free(p.buffer)
+        p.buffer = None
+    nbytes = 12.0 * n
+    return {"elements": n, "bytes": nbytes, "kernel_avg_us": avg_us, "gbs_kernel": nbytes / (avg_us * 1e-6) / 1e9,
+            "gbs_wall": nbytes * steps / wall / 1e9, "frac_hbm": nbytes / (avg_us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+
+
 def cpu_baseline_matmul(n: int, rows: int):
     """The CPU oracle (restatement of the reference's algorithm; the reference itself needs Rust + Vulkan) on
     a slab of `rows` rows of the same n^3 product, epilogue included, all host cores through OpenMP."""
@@ -119,6 +140,8 @@ def main():
     ap.add_argument("--size", type=int, default=8192, help="M=N=K of the headline matmul")
     ap.add_argument("--all", action="store_true", help="also time the other matmul shapes and the ConvNet step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run only the streaming c=a*2+b kernel over 2^26 elements (counter calibration)")
     ap.add_argument("--cpu-rows", type=int, default=256)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -129,6 +152,9 @@ def main():
     from descent_amd.hip_backend import HipBackend
 
     env = Environment(HipBackend())
+    if args.copy_calibration:
+        print(json.dumps(bench_elementwise(env, 1 << 26, args.steps, args.warmup)))
+        return
     n = args.size
     head = bench_matmul(env, n, n, n, args.steps, args.warmup)
     sys.stderr.write(head["report"])
@@ -141,6 +167,7 @@ def main():
             r = bench_matmul(env, m, nn, k, max(args.steps, 20), args.warmup)
             r.pop("report")
             extra["matmul"].append(r)
+        extra["elementwise_axpb_64M"] = bench_elementwise(env, 1 << 26, max(args.steps, 20), args.warmup)
         conv = bench_convnet(env, max(args.steps, 20), args.warmup)
         sys.stderr.write(conv.pop("report"))
         extra["convnet_bs1000"] = conv

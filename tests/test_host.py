@@ -1,0 +1,200 @@
+"""Host-side logic without a GPU: the C-ABI library loads and exports what include/descent_hip.h declares, the
+code generator produces gfx950-compilable HIP for every kernel kind (hipRTC needs no device), the graph passes
+reproduce the reference's cluster structure, and error paths answer with errors instead of crashes."""
+import ctypes as C
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+
+from descent_amd import Environment, Initializer, _abi, hip_backend, kernel as K, workloads
+from descent_amd.shape import BATCHES, Shape, View
+from oracle.cpu_backend import CpuBackend
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _env():
+    return Environment(CpuBackend())
+
+
+def test_library_exports_every_declared_entry_point():
+    header = open(os.path.join(ROOT, "include", "descent_hip.h")).read()
+    declared = set(re.findall(r"^(?:int|int64_t|void|const char\*)\s+(dsc_[a-z_0-9]+)\s*\(", header, re.M))
+    assert len(declared) >= 30
+    lib = C.CDLL(hip_backend.LIB_PATH)
+    for name in sorted(declared):
+        assert hasattr(lib, name), f"{name} is declared in the header but not exported"
+    assert declared == set(hip_backend.EXPORTED_SYMBOLS)
+
+
+def test_no_device_is_an_error_not_a_fallback():
+    """This container has no GPU: creating a context must fail with DSC_ERR_NO_DEVICE."""
+    lib = hip_backend.lib()
+    ctx = C.c_void_p()
+    rc = lib.dsc_ctx_create(0, C.byref(ctx))
+    if rc == 0:  # running on a GPU box
+        lib.dsc_ctx_destroy(ctx)
+        pytest.skip("a GPU is present")
+    assert rc == _abi.ERR_NO_DEVICE and not ctx.value
+    with pytest.raises(hip_backend.DescentHipError):
+        hip_backend.HipBackend()
+
+
+def _kernels_of_each_kind():
+    sh = Shape((4, 6, 8))
+    ident = sh.identity_view()
+    pe = K.PerElementKernel(
+        192,
+        (ident, View.broadcast(Shape((8,)), sh)),
+        (6,),
+        (K.PeLoad(0), K.PeLoad(1), K.PeBinary("Add", (0, 1)), K.PeLiteral(K.Literal.f32(0.0)),
+         K.PeLiteral(K.Literal.f32(0.01)), K.PeBinary("Mul", (2, 4)), K.PeSelect("Gt", (2, 3, 2, 5))),
+    )
+    pe_rand = K.PerElementKernel(
+        192, (ident,), (4,),
+        (K.PeLoad(0), K.PeRand(3, ident), K.PeCoord(View.broadcast(Shape((1, 1, 8)), sh)), K.PeBinary("Mul", (0, 1)),
+         K.PeBinary("Add", (3, 2))),
+    )
+    gather_shape = Shape((4, 10, 8))
+    pe_gather = K.PerElementKernel(
+        320, (ident, View.broadcast(Shape((1, 10, 1)), gather_shape)), (1,),
+        (K.PeLoad(1), K.PeGather(gather_shape, 1, 0, 0)),
+    )
+    win = Shape((2, 3, 3, 1, 2, 2, 4))
+    return [
+        K.FillKernel(K.Literal.f32(1.5), 1000),
+        K.FillKernel(K.Literal.u32(7), 1001),
+        pe, pe_rand, pe_gather,
+        K.ReduceKernel(sh.reduce(2), ident, "Sum", 2),
+        K.ReduceKernel(sh.reduce(0), ident, "Max", 0),
+        K.MatMulKernel(Shape((1, 4, 6, 5)), BATCHES, ident, Shape((4, 8, 5)).identity_view()),
+        K.MatMulKernel(Shape((2, 1, 300, 200)), BATCHES, Shape((1, 300, 1100)).identity_view(),
+                       Shape((1, 200, 1100)).identity_view().transposed()),
+        K.UnpadKernel(Shape((4, 2, 8)), ident, 1, 2),
+        K.WindowsToImageKernel(Shape((2, 6, 6, 4)), win.identity_view(), (2, 2)),
+        K.ScatterAddKernel(Shape((4, 9, 8)), ident, 1, Shape((6,)).identity_view()),
+    ]
+
+
+@pytest.mark.parametrize("kernel", _kernels_of_each_kind(), ids=lambda k: type(k).__name__)
+def test_generated_source_compiles_for_gfx950(kernel):
+    src = hip_backend.codegen_source(kernel)
+    assert 'extern "C" __global__' in src and "dsc_kernel" in src
+    assert hip_backend.codegen_compile(kernel, "gfx950") > 0
+    if isinstance(kernel, K.MatMulKernel):
+        assert "__builtin_amdgcn_mfma_f32_32x32x2f32" in src
+    if isinstance(kernel, K.ScatterAddKernel):
+        assert "unsafeAtomicAdd" in src
+
+
+def test_malformed_descriptors_are_rejected_with_a_message():
+    sh = Shape((4, 6))
+    bad = [
+        K.PerElementKernel(24, (sh.identity_view(),), (1,), (K.PeLoad(0), K.PeUnary("Exp", 1))),  # arg not earlier
+        K.PerElementKernel(24, (sh.identity_view(),), (5,), (K.PeLoad(0),)),                      # missing output op
+        K.PerElementKernel(25, (sh.identity_view(),), (0,), (K.PeLoad(0),)),                      # element count
+        K.ReduceKernel(Shape((4, 6)), sh.identity_view(), "Sum", 1),                              # axis not collapsed
+        K.MatMulKernel(Shape((1, 1, 4, 5)), BATCHES, Shape((1, 4, 6)).identity_view(), Shape((1, 7, 5)).identity_view()),
+        K.UnpadKernel(Shape((4, 6)), sh.identity_view(), 1, 1),
+    ]
+    for kernel in bad:
+        with pytest.raises(hip_backend.DescentHipError) as e:
+            hip_backend.codegen_source(kernel)
+        assert e.value.status == _abi.ERR_INVALID and len(str(e.value)) > 20
+
+
+def test_array_api_cluster_structure_matches_the_reference_dumps():
+    """docs/array_api_values.svg / array_api_grad.svg of the reference, reduced to JSON by
+    tests/golden/make_array_api_fixture.py."""
+    want = json.load(open(os.path.join(ROOT, "tests", "golden", "array_api_clusters.json")))
+    env = _env()
+    m = env.static_parameter([3, 3], "m")
+    x = env.static_parameter([3, 1], "x")
+    y = env.static_parameter([3, 1], "y")
+    z = env.static_parameter([3, 1], "z")
+
+    def values(s):
+        mv, xv, yv = s.parameter_value(m), s.parameter_value(x), s.parameter_value(y)
+        s.write_parameter_value(z, 2.0 * mv.matmul(xv) + yv * yv + 1.0)
+
+    xp = env.trainable_parameter([1], "x", Initializer.zero())
+
+    def grad(s):
+        xd = s.parameter(xp)
+        yd = xd.sin()
+        (yd.square() + yd * 3.0).set_loss()
+        s.write_parameter_value(xp, xd.value() - 0.1 * xd.loss_grad())
+
+    for key, build in (("values", values), ("grad", grad)):
+        g = env.build_graph(build)
+        got = []
+        for cid in g.clusters_sorted:
+            k = g.clusters[cid].kernel
+            if isinstance(k, K.MatMulKernel):
+                got.append(["MatMul"])
+            else:
+                labels = []
+                for op in k.ops:
+                    if isinstance(op, (K.PeUnary, K.PeBinary)):
+                        labels.append(op.op)
+                got.append(sorted(labels))
+        assert sorted(got) == want[key]["clusters"], key
+        # literals are inlined into the cluster as the dumps show them outside any kernel node
+        n_literals = sum(1 for lab in want[key]["outside"] if re.fullmatch(r"-?\d+E-?\d+", lab))
+        pe = [g.clusters[c].kernel for c in g.clusters_sorted if isinstance(g.clusters[c].kernel, K.PerElementKernel)][0]
+        assert sum(isinstance(op, K.PeLiteral) for op in pe.ops) == n_literals
+
+
+def test_convnet_graph_shape():
+    env = _env()
+    w = workloads.convnet(env, batch=1000)
+    labels = w.graph.kernel_labels()
+    assert len(labels) == 66
+    # the GEMMs the train step contains, with the reference's split-K factors r = ceil(K/1024)
+    for want in ["MatMul (k=9) [1, 784000, 1, 16]", "MatMul (k=784000) [766, 1, 9, 16]", "MatMul (k=72) [1, 196000, 2, 16]",
+                 "MatMul (k=196000) [192, 2, 72, 16]", "MatMul (k=16) [1, 2, 196000, 72]", "MatMul (k=1568) [2, 1, 1000, 128]",
+                 "MatMul (k=1000) [1, 1, 1568, 128]", "MatMul (k=128) [1, 1, 1000, 1568]", "MatMul (k=128) [1, 1, 1000, 10]",
+                 "MatMul (k=1000) [1, 1, 128, 10]", "MatMul (k=10) [1, 1, 1000, 128]"]:
+        assert want in labels, want
+    assert sum(p.shape.element_count() for p in w.trainable) == 204618
+    listing = hip_backend.check_schedule(w.graph, fused=True)
+    launches = int(listing.split()[0])
+    assert launches < 55, listing
+
+
+def test_fused_and_unfused_schedules_compile_for_every_config():
+    env = _env()
+    graphs = [workloads.convnet(env, batch=8).graph, workloads.linear_classifier(env, batch=16).graph,
+              workloads.matmul_epilogue(env, 300, 200, 1100, upload=False).graph]
+    for g in graphs:
+        fused = hip_backend.check_schedule(g, fused=True)
+        unfused = hip_backend.check_schedule(g, fused=False)
+        assert int(unfused.split()[0]) == len(g.clusters_sorted)
+        assert int(fused.split()[0]) <= int(unfused.split()[0])
+
+
+def test_reference_error_behaviour_on_the_host():
+    env, other = _env(), _env()
+    p = other.static_parameter([4], "p")
+    with pytest.raises(ValueError, match="same environment"):  # src/parameter.rs:51-56
+        env.build_graph(lambda s: s.parameter_value(p))
+    q = env.static_parameter([4], "q")
+    r = env.static_parameter([5], "r")
+    env.write_parameter(r, np.zeros(5, np.float32))
+    with pytest.raises(ValueError, match="shape mismatch"):  # src/array.rs:1367-1370
+        env.build_graph(lambda s: s.write_parameter_value(q, s.parameter_value(r)))
+    with pytest.raises(ValueError):  # src/shape.rs:97-98
+        Shape((1, 4, 5)).batched_matmul(Shape((1, 6, 3)), BATCHES)
+    with pytest.raises(ValueError, match="no value"):  # src/environment.rs:375 (assert on missing buffer)
+        env.run(env.build_graph(lambda s: s.write_parameter_value(q, s.parameter_value(q) + 1.0)), 0)
+
+
+def test_writer_zero_fills_the_unwritten_tail():
+    env = _env()
+    p = env.static_parameter([8], "p")
+    with env.writer(p) as w:
+        w.write(np.arange(3, dtype=np.float32))
+    assert np.array_equal(env.read_parameter_to_vec(p), np.array([0, 1, 2, 0, 0, 0, 0, 0], np.float32))
