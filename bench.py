@@ -76,7 +76,7 @@ def bench_convnet(env, steps, warmup, batch=1000):
 
     w = workloads.convnet(env, batch=batch, seed=3)
     wall = time_graph(env, w.graph, steps, warmup)
-    report = env.backend.timing_report(12)
+    report = env.backend.timing_report(int(os.environ.get("DSC_BENCH_TOPN", "12")))
     env.backend.profile_reset()
     sched = next(iter(w.graph.__dict__["_schedules"].values()))
     return {
@@ -107,6 +107,47 @@ def bench_elementwise(env, n, steps, warmup):
     nbytes = 12.0 * n
     return {"elements": n, "bytes": nbytes, "kernel_avg_us": avg_us, "gbs_kernel": nbytes / (avg_us * 1e-6) / 1e9,
             "gbs_wall": nbytes * steps / wall / 1e9, "frac_hbm": nbytes / (avg_us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+
+
+def bench_workload(env, build, steps, warmup, topn=8):
+    """Step rate of one of the image-fit configurations, with the per-kernel table."""
+    w = build(env)
+    wall = time_graph(env, w.graph, steps, warmup)
+    be = env.backend
+    out = {"steps_per_s": steps / wall, "ms_per_step": 1e3 * wall / steps}
+    for prefix in ("MatMul", "ScatterAdd", "PerElement", "Reduce"):
+        avg_us, launches = be.timing_query(prefix)
+        out[prefix.lower() + "_us_per_step"] = avg_us * launches / steps
+        out[prefix.lower() + "_launches_per_step"] = launches / steps
+    report = be.timing_report(topn)
+    be.profile_reset()
+    sched = next(iter(w.graph.__dict__["_schedules"].values()))
+    out["launches_per_step"], out["clusters"] = sched.launch_count()
+    for p in list(w.inputs.values()) + w.trainable + w.state + list(w.scalars.values()):
+        if p.buffer is not None:
+            be.free(p.buffer)
+            p.buffer = None
+    return out, report
+
+
+def bench_reduce(env, rows, cols, axis, steps, warmup):
+    """Sum of a [rows, cols] array along one axis: 4*(rows*cols + outputs) bytes."""
+    rng = np.random.Generator(np.random.PCG64(10))
+    a = env.static_parameter([rows, cols], "a")
+    out_shape = [rows, 1] if axis == 1 else [1, cols]
+    o = env.static_parameter(out_shape, "o")
+    env.write_parameter(a, rng.random(rows * cols, dtype=np.float32))
+    graph = env.build_graph(lambda s: s.write_parameter_value(o, s.parameter_value(a).reduce_sum(axis, True)))
+    wall = time_graph(env, graph, steps, warmup)
+    avg_us, launches = env.backend.timing_query("Reduce")
+    per_step_us = avg_us * launches / steps
+    env.backend.profile_reset()
+    for p in (a, o):
+        env.backend.free(p.buffer)
+        p.buffer = None
+    nbytes = 4.0 * (rows * cols + (rows if axis == 1 else cols))
+    return {"shape": [rows, cols], "axis": axis, "kernels_us_per_step": per_step_us, "launches_per_step": launches / steps,
+            "gbs": nbytes / (per_step_us * 1e-6) / 1e9, "frac_hbm": nbytes / (per_step_us * 1e-6) / 1e9 / HBM_PEAK_GBS}
 
 
 def cpu_baseline_matmul(n: int, rows: int):
@@ -168,6 +209,19 @@ def main():
             r.pop("report")
             extra["matmul"].append(r)
         extra["elementwise_axpb_64M"] = bench_elementwise(env, 1 << 26, max(args.steps, 20), args.warmup)
+        extra["reduce"] = [bench_reduce(env, 8192, 8192, 1, 20, 3), bench_reduce(env, 8192, 8192, 0, 20, 3),
+                           bench_reduce(env, 262144, 256, 0, 20, 3)]
+        from descent_amd import workloads as _w
+
+        mlp, rep = bench_workload(env, lambda e: _w.coordinate_mlp(e), 10, 2)
+        sys.stderr.write("cfg4 coordinate MLP (relu-pe):\n" + rep)
+        extra["coordinate_mlp_relu_pe_512"] = mlp
+        siren, rep = bench_workload(env, lambda e: _w.coordinate_mlp(e, variant="siren"), 10, 2)
+        extra["coordinate_mlp_siren_512"] = siren
+        hg, rep = bench_workload(env, lambda e: _w.hash_grid_fit(e), 10, 2)
+        sys.stderr.write("cfg5 hash grid:\n" + rep)
+        hg["scatter_atomics_per_s"] = 16 * 4 * 2 * (1 << 18) / (hg["scatteradd_us_per_step"] * 1e-6) if hg["scatteradd_us_per_step"] else None
+        extra["hash_grid_2p18"] = hg
         conv = bench_convnet(env, max(args.steps, 20), args.warmup)
         sys.stderr.write(conv.pop("report"))
         extra["convnet_bs1000"] = conv

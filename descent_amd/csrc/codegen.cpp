@@ -1,6 +1,7 @@
 #include "codegen.hpp"
 
 #include <algorithm>
+#include <cctype>
 #include <cstdio>
 #include <cstdlib>
 #include <map>
@@ -26,10 +27,27 @@ const int64_t kMaxIndex = (int64_t)1 << 31;
 // Largest linear index (+1) a view may produce into its input, i.e. the input's element count.
 int64_t input_extent(const dsc_view& v) { return element_count(v.in_shape); }
 
+// How a linear element id was formed from named integer coordinates: id = base + sum coef_i * name_i with
+// name_i in [0, extent_i).  Lets a consumer's coordinates be turned into a producer's coordinates digit by
+// digit (no division of the combined id) whenever the terms occupy disjoint digit ranges.
+struct IndexForm {
+    bool valid = false;
+    int64_t base = 0;
+    std::vector<string> names;
+    std::vector<int64_t> coefs, extents;
+};
+
+bool is_identifier(const string& s) {
+    if (s.empty() || !(std::isalpha((unsigned char)s[0]) || s[0] == '_')) return false;
+    for (char c : s)
+        if (!(std::isalnum((unsigned char)c) || c == '_')) return false;
+    return true;
+}
+
 struct Emitter {
     const FusedKernel& fk;
     std::ostringstream funcs;  // device functions, emitted before the kernel
-    int tmp_counter = 0;
+    std::map<string, string> instances;  // (virtual, index form signature) -> function name
 
     explicit Emitter(const FusedKernel& k) : fk(k) {}
 
@@ -75,6 +93,56 @@ struct Emitter {
         return names;
     }
 
+    // Decomposition of an id given as an IndexForm: every term must start exactly on a digit boundary of
+    // `shape` and the terms' digit ranges must not overlap (then no carries cross between them).  Returns an
+    // empty vector when the form does not separate.
+    std::vector<string> emit_coords_separable(std::ostream& o, const dsc_shape& shape, const IndexForm& form, const string& pfx) {
+        if (!form.valid || form.base != 0) return {};
+        int64_t st[DSC_MAX_DIM];
+        strides_of(shape, st);
+        std::vector<int> owner(shape.rank, -1);
+        struct Span { int hi, lo; };
+        std::vector<Span> spans(form.names.size(), Span{-1, -1});
+        for (size_t t = 0; t < form.names.size(); ++t) {
+            if (form.coefs[t] == 0 || form.extents[t] <= 1) continue;
+            if (form.coefs[t] < 0) return {};
+            int lo = -1;
+            for (int i = shape.rank - 1; i >= 0; --i)
+                if (st[i] == form.coefs[t] && shape.dims[i] > 1) { lo = i; break; }
+            if (lo < 0) return {};
+            int hi = lo;
+            int64_t cover = st[lo] * shape.dims[lo];
+            const int64_t need = form.coefs[t] * form.extents[t];
+            while (cover < need) {
+                if (--hi < 0) return {};
+                cover *= shape.dims[hi];
+            }
+            for (int i = hi; i <= lo; ++i) {
+                if (owner[i] >= 0) return {};
+                owner[i] = (int)t;
+            }
+            spans[t] = Span{hi, lo};
+        }
+        std::vector<string> names(shape.rank);
+        for (int i = 0; i < shape.rank; ++i) names[i] = "0";
+        for (size_t t = 0; t < form.names.size(); ++t) {
+            if (spans[t].lo < 0) continue;
+            const int hi = spans[t].hi, lo = spans[t].lo;
+            if (hi == lo) { names[lo] = form.names[t]; continue; }
+            const string rem = pfx + "q" + to_string(t);
+            o << "    uint " << rem << " = (uint)" << form.names[t] << ";\n";
+            for (int i = lo; i > hi; --i) {
+                names[i] = pfx + to_string(i);
+                if (shape.dims[i] == 1) { o << "    const int " << names[i] << " = 0;\n"; continue; }
+                o << "    const int " << names[i] << " = (int)(" << rem << " % " << S(shape.dims[i]) << "u); " << rem << " /= "
+                  << S(shape.dims[i]) << "u;\n";
+            }
+            names[hi] = pfx + to_string(hi);
+            o << "    const int " << names[hi] << " = (int)" << rem << ";\n";
+        }
+        return names;
+    }
+
     // Linear index into the view's input for output coordinates `coord` (kernel.rs:89-133).
     string index_expr(const dsc_view& v, const std::vector<string>& coord) const {
         int64_t st[DSC_MAX_DIM];
@@ -100,21 +168,110 @@ struct Emitter {
         return e + clamped + ")";
     }
 
-    string load_expr(const Source& s, const string& idx) const {
+    // The same index as an IndexForm, when the view needs no clamp and the coordinates are plain names.
+    IndexForm index_form(const dsc_view& v, const std::vector<string>& coord) const {
+        IndexForm f;
+        int64_t coef[DSC_MAX_DIM];
+        if (!affine_form(v, &f.base, coef)) return f;
+        for (int j = 0; j < v.out_shape.rank; ++j) {
+            if (coef[j] == 0 || v.out_shape.dims[j] <= 1) continue;
+            if (!is_identifier(coord[j])) return f;
+            // the same name on two axes would need a combined extent: give up
+            for (auto& n : f.names)
+                if (n == coord[j]) return f;
+            f.names.push_back(coord[j]);
+            f.coefs.push_back(coef[j]);
+            f.extents.push_back(v.out_shape.dims[j]);
+        }
+        f.valid = true;
+        return f;
+    }
+
+    // Expression for the element of source `s` that view `v` selects at coordinates `coord`.
+    string load_view(const Source& s, const dsc_view& v, const std::vector<string>& coord) {
+        if (s.buffer >= 0) return "b" + to_string(s.buffer) + "[" + index_expr(v, coord) + "]";
+        IndexForm form = index_form(v, coord);
+        if (!form.valid) {
+            const string fn = instantiate(s.virt, IndexForm{});
+            return fn + "(" + index_expr(v, coord) + ", " + params_pass() + ")";
+        }
+        const string fn = instantiate(s.virt, form);
+        string args;
+        for (auto& n : form.names) args += n + ", ";
+        return fn + "(" + args + params_pass() + ")";
+    }
+    // Element `idx` (a linear id expression) of source `s`.
+    string load_linear(const Source& s, const string& idx) {
         if (s.buffer >= 0) return "b" + to_string(s.buffer) + "[" + idx + "]";
-        return "virt" + to_string(s.virt) + "(" + idx + ", " + params_pass() + ")";
+        return instantiate(s.virt, IndexForm{}) + "(" + idx + ", " + params_pass() + ")";
+    }
+
+    // A device function evaluating virtual producer `virt` for ids of the given form: parameters are the
+    // form's coordinates (or the linear id when the form is invalid), then the kernel's parameters.
+    string instantiate(int virt, const IndexForm& form) {
+        string sig = to_string(virt) + "|";
+        if (form.valid) {
+            sig += S(form.base);
+            for (size_t t = 0; t < form.names.size(); ++t) sig += "," + S(form.coefs[t]) + "x" + S(form.extents[t]);
+        } else {
+            sig += "lin";
+        }
+        auto it = instances.find(sig);
+        if (it != instances.end()) return it->second;
+        const string name = "virt" + to_string(virt) + "_" + to_string(instances.size());
+        instances[sig] = name;
+        const Virtual& vi = fk.virtuals[virt];
+        std::ostringstream body;
+        IndexForm local;  // the form re-expressed over this function's own parameter names
+        string decl;
+        if (form.valid) {
+            local = form;
+            string gid = S(form.base);
+            for (size_t t = 0; t < form.names.size(); ++t) {
+                local.names[t] = "a" + to_string(t);
+                decl += "int a" + to_string(t) + ", ";
+                gid += " + (" + S(form.coefs[t]) + ")*a" + to_string(t);
+            }
+            body << "    const int gid = " << gid << ";\n";
+        } else {
+            decl = "int gid, ";
+        }
+        const dsc_kernel_desc& pd = vi.pe.raw();
+        if (pd.kind == DSC_KERNEL_PER_ELEMENT) {
+            emit_pe(body, pd, vi.inputs, "gid", "v", {}, form.valid ? &local : nullptr);
+            body << "    return vt" << vi.out_op << ";\n";
+        } else {  // DSC_KERNEL_REDUCE evaluated on demand: one output element = a loop over the reduced axis
+            const dsc_view& v = pd.inputs[0];
+            std::vector<string> oc;
+            if (form.valid) oc = emit_coords_separable(body, pd.shape, local, "vo");
+            if (oc.empty()) oc = emit_coords(body, pd.shape, "gid", "vo");
+            const bool is_max = pd.reduce_op == DSC_REDUCE_MAX;
+            body << "    float acc = " << (is_max ? "U2F(0xff800000u)" : "0.f") << ";\n";
+            body << "    for (int kk = 0; kk < " << S(v.out_shape.dims[pd.axis]) << "; ++kk) {\n";
+            auto ic = oc;
+            ic[pd.axis] = "kk";
+            body << "        const float x = " << load_view(vi.inputs[0], v, ic) << ";\n";
+            body << "        acc = " << (is_max ? "glsl_max(acc, x)" : "acc + x") << ";\n    }\n";
+            body << "    return acc;\n";
+        }
+        funcs << "DSC_INLINE float " << name << "(" << decl << params_decl() << ") {\n" << body.str() << "}\n\n";
+        return name;
     }
 
     // ---- per-element bodies ---------------------------------------------------------------------------
     // Emits the straight-line evaluation of `pe` at linear id `gid`; op i is left in variable <pfx>t<i>.
-    // `override_load[input]` replaces the load of that input by an expression.
+    // `override_load[input]` replaces the load of that input by an expression.  `form` (optional) says how
+    // gid was composed, which lets coordinate sets be derived without dividing gid.
     void emit_pe(std::ostream& o, const dsc_kernel_desc& pe, const std::vector<Source>& srcs, const string& gid,
-                 const string& pfx, const std::map<int, string>& override_load) {
+                 const string& pfx, const std::map<int, string>& override_load, const IndexForm* form = nullptr) {
         std::vector<std::pair<dsc_shape, std::vector<string>>> sets;
         auto coords_for = [&](const dsc_shape& shape) -> std::vector<string> {
             for (auto& s : sets)
                 if (same_shape(s.first, shape)) return s.second;
-            auto names = emit_coords(o, shape, gid, pfx + "c" + to_string(sets.size()) + "_");
+            const string cp = pfx + "c" + to_string(sets.size()) + "_";
+            std::vector<string> names;
+            if (form) names = emit_coords_separable(o, shape, *form, cp);
+            if (names.empty()) names = emit_coords(o, shape, gid, cp);
             sets.emplace_back(shape, names);
             return names;
         };
@@ -127,8 +284,8 @@ struct Emitter {
                 auto ov = override_load.find(op.input_index);
                 if (ov != override_load.end()) { rhs = ov->second; break; }
                 const dsc_view& v = pe.inputs[op.input_index];
-                if (is_identity(v)) rhs = load_expr(srcs[op.input_index], "(int)(" + gid + ")");
-                else rhs = load_expr(srcs[op.input_index], index_expr(v, coords_for(v.out_shape)));
+                if (is_identity(v)) rhs = load_linear(srcs[op.input_index], "(int)(" + gid + ")");
+                else rhs = load_view(srcs[op.input_index], v, coords_for(v.out_shape));
                 break;
             }
             case DSC_PE_LITERAL_F32:
@@ -182,21 +339,11 @@ struct Emitter {
                 const dsc_view& v = pe.inputs[op.input_index];
                 auto names = coords_for(op.gather_shape);
                 names[op.axis] = "F2I(" + T(op.args[0]) + ")";
-                rhs = load_expr(srcs[op.input_index], index_expr(v, names));
+                rhs = load_view(srcs[op.input_index], v, names);
                 break;
             }
             }
             o << "    const float " << T(i) << " = " << rhs << ";\n";
-        }
-    }
-
-    // Device functions for the virtual inputs (highest index first: a virtual only references larger ones).
-    void emit_virtuals() {
-        for (int v = (int)fk.virtuals.size() - 1; v >= 0; --v) {
-            const Virtual& vi = fk.virtuals[v];
-            funcs << "DSC_INLINE float virt" << v << "(int gid, " << params_decl() << ") {\n";
-            emit_pe(funcs, vi.pe.raw(), vi.inputs, "gid", "v", {});
-            funcs << "    return vt" << vi.out_op << ";\n}\n\n";
         }
     }
 };
@@ -311,9 +458,39 @@ string gen_reduce(Emitter& em, Generated* out) {
         if (affine_form(v, &base, coef) && coef[d.axis] == 1 && K >= 4) k_fastest = true;
     }
 
+    // can four adjacent outputs be fetched with one 16-byte load?  (input is a real buffer, the view is affine,
+    // the innermost output axis that is not reduced walks memory with stride 1 and everything is 4-aligned)
+    bool vec_outputs = false;
+    if (!k_fastest && fk.inputs[0].buffer >= 0 && n_out % 4 == 0) {
+        int64_t base, coef[DSC_MAX_DIM];
+        int inner = d.shape.rank - 1;
+        while (inner >= 0 && d.shape.dims[inner] == 1) --inner;
+        if (inner >= 0 && inner != d.axis && affine_form(v, &base, coef) && coef[inner] == 1 && d.shape.dims[inner] % 4 == 0 && base % 4 == 0) {
+            vec_outputs = true;
+            for (int j = 0; j < d.shape.rank; ++j)
+                if (j != inner && v.out_shape.dims[j] > 1 && coef[j] % 4 != 0) vec_outputs = false;
+        }
+    }
+
     std::ostringstream k;
     k << "extern \"C\" __global__ __launch_bounds__(256) void dsc_kernel(" << em.params_decl() << ") {\n";
-    std::ostringstream body;  // loads one element: expects ints oc* (output coords) and kk
+    // The k loop is unrolled four times over independent accumulators so that four loads are in flight per
+    // thread; `first`/`step` give the thread's k sequence.
+    auto emit_k_loop = [&](const std::vector<string>& oc, const string& first, int64_t step) {
+        k << "    float acc0 = " << init << ", acc1 = " << init << ", acc2 = " << init << ", acc3 = " << init << ";\n";
+        k << "    for (int kb = " << first << "; kb < " << S(K) << "; kb += " << S(4 * step) << ") {\n";
+        for (int u = 0; u < 4; ++u) {
+            const string kk = "kk" + to_string(u);
+            k << "        const int " << kk << " = kb + " << S(u * step) << ";\n";
+            auto ic = oc;
+            ic[d.axis] = kk;
+            const string ld = em.load_view(fk.inputs[0], v, ic);
+            k << "        if (" << kk << " < " << S(K) << ") { const float x = " << ld << "; acc" << u << " = "
+              << combine("acc" + to_string(u), "x") << "; }\n";
+        }
+        k << "    }\n";
+        k << "    float acc = " << combine(combine("acc0", "acc1"), combine("acc2", "acc3")) << ";\n";
+    };
     if (k_fastest) {
         // lanes of a group walk k; groups of G lanes own one output; butterfly over the group
         const int64_t G = std::min<int64_t>(64, pow2_ceil(K));
@@ -322,42 +499,79 @@ string gen_reduce(Emitter& em, Generated* out) {
         k << "    const uint oid = blockIdx.x * " << per_block << "u + grp;\n";
         k << "    if (oid >= " << S(n_out) << "u) return;\n";
         auto oc = em.emit_coords(k, d.shape, "oid", "oc");
-        k << "    float acc = " << init << ";\n";
-        k << "    for (int kk = lk; kk < " << S(K) << "; kk += " << G << ") {\n";
-        auto ic = oc;
-        ic[d.axis] = "kk";
-        k << "        const float x = " << em.load_expr(fk.inputs[0], em.index_expr(v, ic)) << ";\n";
-        k << "        acc = " << combine("acc", "x") << ";\n    }\n";
+        emit_k_loop(oc, "lk", G);
         for (int64_t off = G / 2; off >= 1; off /= 2)
             k << "    acc = " << combine("acc", "__shfl_xor(acc, " + S(off) + ", 64)") << ";\n";
         k << "    if (lk == 0) b" << fk.outputs[0] << "[oid] = acc;\n}\n";
         out->grid = blocks_for(n_out, (int)per_block);
         out->note = "reduce: " + S(G) + " lanes along k, shuffle";
+    } else if (vec_outputs) {
+        // each thread owns 4 adjacent outputs that are adjacent in memory: 16-byte loads, lanes walk outputs;
+        // k optionally split over TK thread rows combined through LDS
+        const int64_t n_vec = n_out / 4;
+        int64_t TK = 1;
+        if (n_vec < 32768 && K >= 8) {
+            while (TK < 64 && n_vec * TK < 32768 && TK * 4 <= K) TK *= 2;
+        }
+        const int64_t TO = 256 / TK;
+        k << "    const int to = threadIdx.x % " << TO << ", tk = threadIdx.x / " << TO << ";\n";
+        k << "    const uint vid = blockIdx.x * " << TO << "u + to;\n";
+        if (TK > 1) k << "    __shared__ float4 red[256];\n";
+        k << "    float4 result = make_float4(" << init << ", " << init << ", " << init << ", " << init << ");\n";
+        k << "    if (vid < " << S(n_vec) << "u) {\n";
+        k << "    const uint oid = vid * 4u;\n";
+        auto oc = em.emit_coords(k, d.shape, "oid", "oc");
+        k << "    float4 a0 = result, a1 = result, a2 = result, a3 = result;\n";
+        k << "    for (int kb = tk; kb < " << S(K) << "; kb += " << S(4 * TK) << ") {\n";
+        for (int u = 0; u < 4; ++u) {
+            const string kk = "kk" + to_string(u);
+            k << "        const int " << kk << " = kb + " << S(u * TK) << ";\n";
+            auto ic = oc;
+            ic[d.axis] = kk;
+            k << "        if (" << kk << " < " << S(K) << ") { const float4 x = *(const float4*)(b" << fk.inputs[0].buffer << " + "
+              << em.index_expr(v, ic) << ");";
+            const string a = "a" + to_string(u);
+            for (const char* c : {"x", "y", "z", "w"}) k << " " << a << "." << c << " = " << combine(a + "." + c, string("x.") + c) << ";";
+            k << " }\n";
+        }
+        k << "    }\n";
+        for (const char* c : {"x", "y", "z", "w"})
+            k << "    result." << c << " = " << combine(combine(string("a0.") + c, string("a1.") + c), combine(string("a2.") + c, string("a3.") + c)) << ";\n";
+        k << "    }\n";
+        if (TK > 1) {
+            k << "    red[threadIdx.x] = result;\n    __syncthreads();\n";
+            k << "    if (tk == 0 && vid < " << S(n_vec) << "u) {\n";
+            k << "        for (int j = 1; j < " << TK << "; ++j) { const float4 o = red[j * " << TO << " + to];";
+            for (const char* c : {"x", "y", "z", "w"}) k << " result." << c << " = " << combine(string("result.") + c, string("o.") + c) << ";";
+            k << " }\n";
+            k << "        *(float4*)(b" << fk.outputs[0] << " + vid * 4u) = result;\n    }\n}\n";
+        } else {
+            k << "    if (vid < " << S(n_vec) << "u) *(float4*)(b" << fk.outputs[0] << " + vid * 4u) = result;\n}\n";
+        }
+        out->grid = blocks_for(n_vec, (int)TO);
+        out->note = "reduce: lanes along outputs x4, k split " + S(TK);
     } else {
         // lanes walk outputs (coalesced); optional split of k over TK thread rows, combined through LDS
         int64_t TK = 1;
         if (n_out < 65536 && K >= 8) {
-            while (TK < 16 && n_out * TK < 65536 && TK * 4 <= K) TK *= 2;
+            while (TK < 64 && n_out * TK < 65536 && TK * 4 <= K) TK *= 2;
         }
         const int64_t TO = 256 / TK;
         k << "    const int to = threadIdx.x % " << TO << ", tk = threadIdx.x / " << TO << ";\n";
         k << "    const uint oid = blockIdx.x * " << TO << "u + to;\n";
         if (TK > 1) k << "    __shared__ float red[256];\n";
-        k << "    float acc = " << init << ";\n";
+        k << "    float result = " << init << ";\n";
         k << "    if (oid < " << S(n_out) << "u) {\n";
         auto oc = em.emit_coords(k, d.shape, "oid", "oc");
-        k << "    for (int kk = tk; kk < " << S(K) << "; kk += " << TK << ") {\n";
-        auto ic = oc;
-        ic[d.axis] = "kk";
-        k << "        const float x = " << em.load_expr(fk.inputs[0], em.index_expr(v, ic)) << ";\n";
-        k << "        acc = " << combine("acc", "x") << ";\n    }\n    }\n";
+        emit_k_loop(oc, "tk", TK);
+        k << "    result = acc;\n    }\n";
         if (TK > 1) {
-            k << "    red[threadIdx.x] = acc;\n    __syncthreads();\n";
+            k << "    red[threadIdx.x] = result;\n    __syncthreads();\n";
             k << "    if (tk == 0 && oid < " << S(n_out) << "u) {\n";
-            k << "        for (int j = 1; j < " << TK << "; ++j) acc = " << combine("acc", "red[j * " + S(TO) + " + to]") << ";\n";
-            k << "        b" << fk.outputs[0] << "[oid] = acc;\n    }\n}\n";
+            k << "        for (int j = 1; j < " << TK << "; ++j) result = " << combine("result", "red[j * " + S(TO) + " + to]") << ";\n";
+            k << "        b" << fk.outputs[0] << "[oid] = result;\n    }\n}\n";
         } else {
-            k << "    if (oid < " << S(n_out) << "u) b" << fk.outputs[0] << "[oid] = acc;\n}\n";
+            k << "    if (oid < " << S(n_out) << "u) b" << fk.outputs[0] << "[oid] = result;\n}\n";
         }
         out->grid = blocks_for(n_out, (int)TO);
         out->note = "reduce: lanes along outputs, k split " + S(TK);
@@ -383,7 +597,7 @@ string gen_unpad(Emitter& em, Generated* out) {
     k << "    float sum = 0.f;\n    for (int kk = k_min; kk <= k_max; ++kk) {\n";
     auto ic = c;
     ic[d.axis] = "kk";
-    k << "        sum += " << em.load_expr(fk.inputs[0], em.index_expr(v, ic)) << ";\n    }\n";
+    k << "        sum += " << em.load_view(fk.inputs[0], v, ic) << ";\n    }\n";
     k << "    b" << fk.outputs[0] << "[gid] = sum;\n}\n";
     out->grid = blocks_for(n, 256);
     out->block = 256;
@@ -421,7 +635,7 @@ string gen_windows_to_image(Emitter& em, Generated* out) {
     std::vector<string> ic(r);
     for (int i = 0; i < bd; ++i) ic[i] = c[i];
     ic[bd] = "oy"; ic[bd + 1] = "ox"; ic[bd + 2] = "group_index"; ic[bd + 3] = "fy"; ic[bd + 4] = "fx"; ic[bd + 5] = "group_c";
-    k << "            tmp += " << em.load_expr(fk.inputs[0], em.index_expr(v, ic)) << ";\n        }\n    }\n";
+    k << "            tmp += " << em.load_view(fk.inputs[0], v, ic) << ";\n        }\n    }\n";
     k << "    b" << fk.outputs[0] << "[gid] = tmp;\n}\n";
     out->grid = blocks_for(n, 256);
     out->block = 256;
@@ -440,8 +654,8 @@ string gen_scatter_add(Emitter& em, Generated* out) {
     k << "extern \"C\" __global__ __launch_bounds__(256) void dsc_kernel(" << em.params_decl() << ") {\n";
     k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n";
     auto c = em.emit_coords(k, vv.out_shape, "gid", "c");
-    k << "    const float value = " << em.load_expr(fk.inputs[0], em.index_expr(vv, c)) << ";\n";
-    k << "    const int si = F2I(" << em.load_expr(fk.inputs[1], em.index_expr(vi, {c[d.axis]})) << ");\n";
+    k << "    const float value = " << em.load_view(fk.inputs[0], vv, c) << ";\n";
+    k << "    const int si = F2I(" << em.load_view(fk.inputs[1], vi, {c[d.axis]}) << ");\n";
     int64_t st[DSC_MAX_DIM];
     strides_of(d.shape, st);
     string idx = "0";
@@ -553,16 +767,16 @@ string gen_matmul(Emitter& em, Generated* out) {
         k << "#define A_PTR b" << fk.inputs[0].buffer << "\n#define A_BASE " << S(a_base) << "\n#define A_SB "
           << S(g.batch == 1 ? 0 : a_coef[0]) << "\n#define A_SM " << S(a_coef[1]) << "\n#define A_SK " << S(a_coef[2]) << "\n";
     } else {
-        em.funcs << "DSC_INLINE float load_a(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return "
-                 << em.load_expr(fk.inputs[0], em.index_expr(va, {"cb", "cm", "ck"})) << ";\n}\n";
+        const string la = em.load_view(fk.inputs[0], va, {"cb", "cm", "ck"});
+        em.funcs << "DSC_INLINE float load_a(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return " << la << ";\n}\n";
         k << "#define LOAD_A(b, m, k) load_a(b, m, k, " << em.params_pass() << ")\n";
     }
     if (b_mode) {
         k << "#define B_PTR b" << fk.inputs[1].buffer << "\n#define B_BASE " << S(b_base) << "\n#define B_SB "
           << S(g.batch == 1 ? 0 : b_coef[0]) << "\n#define B_SK " << S(b_coef[1]) << "\n#define B_SN " << S(b_coef[2]) << "\n";
     } else {
-        em.funcs << "DSC_INLINE float load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return "
-                 << em.load_expr(fk.inputs[1], em.index_expr(vb, {"cb", "ck", "cn"})) << ";\n}\n";
+        const string lb = em.load_view(fk.inputs[1], vb, {"cb", "ck", "cn"});
+        em.funcs << "DSC_INLINE float load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb << ";\n}\n";
         k << "#define LOAD_B(b, k, n) load_b(b, k, n, " << em.params_pass() << ")\n";
     }
     const int64_t batch_stride = rows ? g.n : g.m * g.n, row_stride = rows ? g.batch * g.n : g.n;
@@ -572,12 +786,12 @@ string gen_matmul(Emitter& em, Generated* out) {
 
     if (fk.has_epilogue) {
         const dsc_kernel_desc& pe = fk.epilogue.raw();
-        em.funcs << "DSC_INLINE void mm_store(float product, int gid, " << em.params_decl() << ") {\n";
+        std::ostringstream body;
         std::map<int, string> ov;
         ov[fk.epilogue_product_input] = "product";
-        em.emit_pe(em.funcs, pe, fk.epilogue_inputs, "gid", "e", ov);
-        for (int o = 0; o < pe.n_outputs; ++o) em.funcs << "    b" << fk.outputs[o] << "[gid] = et" << pe.outputs[o] << ";\n";
-        em.funcs << "}\n";
+        em.emit_pe(body, pe, fk.epilogue_inputs, "gid", "e", ov);
+        for (int o = 0; o < pe.n_outputs; ++o) body << "    b" << fk.outputs[o] << "[gid] = et" << pe.outputs[o] << ";\n";
+        em.funcs << "DSC_INLINE void mm_store(float product, int gid, " << em.params_decl() << ") {\n" << body.str() << "}\n";
         k << "#define MM_STORE(v, idx) mm_store(v, idx, " << em.params_pass() << ")\n";
     } else {
         k << "#define MM_STORE(v, idx) b" << fk.outputs[0] << "[idx] = (v)\n";
@@ -650,7 +864,8 @@ std::string generate(const FusedKernel& fk, Generated* out) {
     for (auto& v : fk.virtuals) {
         err = validate(v.pe.raw());
         if (!err.empty()) return "fused producer: " + err;
-        if (v.pe.raw().kind != DSC_KERNEL_PER_ELEMENT) return "fused producer must be a per-element kernel";
+        if (v.pe.raw().kind != DSC_KERNEL_PER_ELEMENT && v.pe.raw().kind != DSC_KERNEL_REDUCE)
+            return "fused producer must be a per-element or reduce kernel";
         if ((int)v.inputs.size() != v.pe.raw().n_inputs) return "fused producer: input binding count";
     }
     if (fk.has_epilogue) {
@@ -664,7 +879,6 @@ std::string generate(const FusedKernel& fk, Generated* out) {
     if (!err.empty()) return err;
 
     Emitter em(fk);
-    em.emit_virtuals();
     Generated g;
     switch (fk.main.raw().kind) {
     case DSC_KERNEL_FILL: err = gen_fill(em, &g); break;
@@ -684,8 +898,9 @@ std::string generate(const FusedKernel& fk, Generated* out) {
 }
 
 const std::vector<std::string>& compile_options() {
-    // packed fp32 instructions are kept off for every kernel; float atomicAdd maps to the hardware instruction
-    static const std::vector<std::string> opts = {"-O3", "-munsafe-fp-atomics", "-Xclang", "-target-feature",
+    // packed fp32 instructions are kept off for every kernel; float atomicAdd maps to the hardware instruction;
+    // a*b+c stays two rounded operations as written (the per-element semantics are "tmp = a * b; tmp2 = tmp + c")
+    static const std::vector<std::string> opts = {"-O3", "-munsafe-fp-atomics", "-ffp-contract=off", "-Xclang", "-target-feature",
                                                   "-Xclang", "-packed-fp32-ops", "-std=c++17"};
     return opts;
 }

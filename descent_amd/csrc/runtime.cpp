@@ -263,6 +263,10 @@ Kernel* get_kernel(Context* ctx, const FusedKernel& fk, int* status) {
     if (fk.has_epilogue) k->label += " + " + label_name(fk.epilogue.raw());
     if (!fk.virtuals.empty()) k->label += " <" + std::to_string(fk.virtuals.size()) + " fused producers>";
     k->reference_groups = reference_group_count(fk.main.raw());
+    if (const char* dump = std::getenv("DSC_DUMP_DIR")) {  // debugging aid: one source file per generated kernel
+        std::ofstream f(std::string(dump) + "/kernel_" + std::to_string(ctx->kernels.size()) + ".hip");
+        if (f) f << "// " << k->label << "\n// " << k->gen.note << "\n" << k->gen.source;
+    }
     std::vector<char> code;
     std::string log;
     int rc = compile_source(k->gen.source, ctx->arch, &code, &log);

@@ -2,6 +2,7 @@
 #include "schedule.hpp"
 
 #include <algorithm>
+#include <cstdlib>
 #include <set>
 #include <sstream>
 
@@ -16,6 +17,8 @@ struct Draft {
     std::vector<int> params;      // node id per pointer parameter
     std::vector<StepOutput> outs; // outputs, parallel to fk.outputs
     std::vector<int> covers;      // reference cluster indices folded into this launch
+    bool keep_split = false;      // MatMul re-split over k on purpose: do not sum its chunks in one workgroup
+    bool keep_output = false;     // first stage of a split reduction: its result must exist in memory
 };
 
 int param_index(Draft& d, int node, bool is_output) {
@@ -103,6 +106,57 @@ bool is_cheap_producer(const dsc_kernel_desc& pe) {
     return work <= 12;
 }
 
+// Loads issued per evaluated element, following fused producers (a Reduce producer multiplies by its k).
+double source_cost(const FusedKernel& fk, const Source& s);
+double virtual_cost(const FusedKernel& fk, const Virtual& v) {
+    const dsc_kernel_desc& d = v.pe.raw();
+    double c = 0;
+    for (auto& s : v.inputs) c += source_cost(fk, s);
+    if (d.kind == DSC_KERNEL_REDUCE) return c * (double)d.inputs[0].out_shape.dims[d.axis];
+    return c + d.n_ops / 4.0;
+}
+double source_cost(const FusedKernel& fk, const Source& s) { return s.buffer >= 0 ? 1.0 : virtual_cost(fk, fk.virtuals[s.virt]); }
+double draft_unit_cost(const Draft& d) {
+    double c = 0;
+    for (auto& s : d.fk.inputs) c += source_cost(d.fk, s);
+    return c;
+}
+// How many times one evaluation of the main kernel's element reads `node`: the product of the loop lengths of
+// the fused Reduce producers the read sits inside (1 when the main kernel reads the node directly).
+double node_multiplicity(const Draft& d, int node) {
+    const int nv = (int)d.fk.virtuals.size();
+    std::vector<double> mult(nv, 0.0);
+    auto visit = [&](const Source& s, double m, auto&& self) -> double {
+        if (s.buffer >= 0) return d.params[s.buffer] == node ? m : 0.0;
+        const Virtual& v = d.fk.virtuals[s.virt];
+        const dsc_kernel_desc& vd = v.pe.raw();
+        const double inner = m * (vd.kind == DSC_KERNEL_REDUCE ? (double)vd.inputs[0].out_shape.dims[vd.axis] : 1.0);
+        double best = 0.0;
+        for (auto& in : v.inputs) best = std::max(best, self(in, inner, self));
+        return best;
+    };
+    double best = 0.0;
+    for (auto& s : d.fk.inputs) best = std::max(best, visit(s, 1.0, visit));
+    if (d.fk.has_epilogue)
+        for (size_t i = 0; i < d.fk.epilogue_inputs.size(); ++i)
+            if ((int)i != d.fk.epilogue_product_input) best = std::max(best, visit(d.fk.epilogue_inputs[i], 1.0, visit));
+    return std::max(best, 1.0);
+}
+
+int64_t draft_reads(const Draft& d) {  // how many elements the main kernel evaluates per input
+    const dsc_kernel_desc& m = d.fk.main.raw();
+    switch (m.kind) {
+    case DSC_KERNEL_REDUCE: return element_count(m.inputs[0].out_shape);
+    case DSC_KERNEL_MATMUL: {
+        MatMulDims g = matmul_dims(m);
+        return g.batch * std::max(g.m * g.k, g.k * g.n);
+    }
+    case DSC_KERNEL_WINDOWS_TO_IMAGE: return element_count(m.inputs[0].out_shape);
+    case DSC_KERNEL_SCATTER_ADD: return element_count(m.inputs[0].out_shape);
+    default: return element_count(m.shape);
+    }
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------------------------------------
@@ -150,6 +204,142 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
     }
 
     if (!(flags & DSC_SCHEDULE_NO_FUSION)) {
+        // Pass 0: a MatMul whose output is small but whose k is long gets its k range split over many more
+        // workgroups than the reference's ceil(K/1024) chunks; the partial products go to an internal buffer and
+        // are summed by a Reduce (which pass 2 then inlines into the consumer when the split is small).
+        for (size_t i = 0; i < drafts.size(); ++i) {
+            if (drafts[i].fk.main.raw().kind != DSC_KERNEL_MATMUL) continue;
+            const MatMulDims g = matmul_dims(drafts[i].fk.main.raw());
+            if (g.k < 512) continue;
+            if (((g.m + 63) / 64) * ((g.n + 63) / 64) * g.batch >= 128) continue;  // the tile grid is already wide
+            const int64_t t64 = ((g.m + 63) / 64) * ((g.n + 63) / 64) * g.batch;
+            static const int64_t split_target = std::getenv("DSC_SPLIT_TARGET") ? std::atoll(std::getenv("DSC_SPLIT_TARGET")) : 4096;
+            int64_t S = std::min<int64_t>(split_target / t64, g.k / 64);
+            if (S < 2) continue;
+            const int64_t ktiles = (g.k + 15) / 16;
+            const int64_t chunk_tiles = (ktiles + S - 1) / S;
+            S = (ktiles + chunk_tiles - 1) / chunk_tiles;
+            if (S < 2 || (g.chunks > 1 && S <= g.chunks)) continue;
+            const int product = drafts[i].outs[0].node;
+            const int64_t out_elems = g.batch * g.m * g.n;
+            if (S * out_elems >= ((int64_t)1 << 28)) continue;
+            if (g.chunks > 1) {
+                // the reference already sums partials: retarget that Reduce
+                if (is_graph_output[product]) continue;
+                int ri = -1, uses = 0;
+                for (size_t j = i + 1; j < drafts.size(); ++j)
+                    for (int nd : input_nodes(drafts[j]))
+                        if (nd == product) { ++uses; ri = (int)j; }
+                if (uses != 1) continue;
+                const dsc_kernel_desc& rd = drafts[ri].fk.main.raw();
+                if (rd.kind != DSC_KERNEL_REDUCE || rd.reduce_op != DSC_REDUCE_SUM || rd.axis != 0 || !is_identity(rd.inputs[0]) ||
+                    element_count(rd.inputs[0].in_shape) != g.chunks * out_elems)
+                    continue;
+                drafts[ri].fk.main.inputs[0].in_shape.dims[0] = S;
+                drafts[ri].fk.main.inputs[0].out_shape.dims[0] = S;
+            } else {
+                // new internal node for the partials, and a Reduce writing the original node
+                const int partials = n_nodes++;
+                node_bytes.push_back(0);
+                is_graph_output.push_back(false);
+                is_graph_input.push_back(false);
+                Draft r;
+                dsc_kernel_desc rd{};
+                rd.kind = DSC_KERNEL_REDUCE;
+                rd.shape = drafts[i].fk.main.raw().shape;
+                dsc_view v{};
+                v.in_shape = rd.shape;
+                v.in_shape.dims[0] = S;
+                v.out_shape = v.in_shape;
+                for (int a = 0; a < v.in_shape.rank; ++a) {
+                    v.map_axis[a] = v.in_shape.dims[a] > 1 ? a : -1;
+                    v.map_step[a] = v.in_shape.dims[a] > 1 ? 1 : 0;
+                }
+                rd.n_inputs = 1;
+                rd.inputs = &v;
+                rd.reduce_op = DSC_REDUCE_SUM;
+                rd.axis = 0;
+                r.fk = FusedKernel::plain(rd);
+                r.params = {partials, product};
+                r.outs.push_back(drafts[i].outs[0]);
+                r.covers = drafts[i].covers;
+                drafts[i].params[drafts[i].fk.outputs[0]] = partials;
+                drafts[i].outs[0] = StepOutput{partials, -1, false, 0};
+                drafts.insert(drafts.begin() + i + 1, r);
+            }
+            drafts[i].fk.main.d.shape.dims[0] = S;
+            node_bytes[drafts[i].outs[0].node] = (size_t)(S * out_elems) * 4;
+            drafts[i].keep_split = true;
+        }
+
+        // Pass 0b: a Reduce with few outputs and a long axis cannot fill the machine with one thread (or one
+        // thread row) per output.  Split the axis k = s * (k/s): a first Reduce over k/s produces s partial rows
+        // per output into an internal buffer, a second one combines the s partials (pass 2 inlines it into the
+        // consumer when s is small).
+        for (size_t i = 0; i < drafts.size(); ++i) {
+            const dsc_kernel_desc rd = drafts[i].fk.main.raw();
+            if (rd.kind != DSC_KERNEL_REDUCE || !drafts[i].fk.virtuals.empty() || rd.shape.rank >= DSC_MAX_DIM) continue;
+            const dsc_view v = rd.inputs[0];
+            const int axis = rd.axis;
+            const int64_t k = v.out_shape.dims[axis], n_out = element_count(rd.shape);
+            if (k < 512 || n_out > 16384 || (k * n_out < (1 << 20) && k < 8192) || v.map_axis[axis] < 0 || needs_clamp(v, v.map_axis[axis])) continue;
+            const int64_t want = std::min<int64_t>(2048, std::max<int64_t>(2, (524288 + n_out - 1) / n_out));
+            int64_t split = 0;
+            for (int64_t c = want; c <= k / 8; ++c)
+                if (k % c == 0) { split = c; break; }
+            if (split == 0)
+                for (int64_t c = std::min(want, k / 8); c >= 2; --c)
+                    if (k % c == 0) { split = c; break; }
+            if (split < 2) continue;
+            // stage 1: view with the axis split in two; output [.., split, 1, ..]
+            dsc_view v1 = v;
+            v1.out_shape.rank = v.out_shape.rank + 1;
+            for (int j = v.out_shape.rank; j > axis; --j) {
+                v1.out_shape.dims[j] = v.out_shape.dims[j - 1];
+                v1.map_axis[j] = v.map_axis[j - 1];
+                v1.map_step[j] = v.map_step[j - 1];
+            }
+            v1.out_shape.dims[axis] = split;
+            v1.map_step[axis] = v.map_step[axis] * (k / split);
+            v1.out_shape.dims[axis + 1] = k / split;
+            dsc_kernel_desc d1 = rd;
+            d1.shape = v1.out_shape;
+            d1.shape.dims[axis + 1] = 1;
+            d1.inputs = &v1;
+            d1.axis = axis + 1;
+            // stage 2: reads the partials [.., split, 1, ..] as [.., split, ..] and reduces that axis
+            dsc_view v2{};
+            v2.in_shape = d1.shape;
+            v2.out_shape = rd.shape;
+            v2.out_shape.dims[axis] = split;
+            for (int j = 0; j < v2.out_shape.rank; ++j) {
+                const int in_axis = j <= axis ? j : j + 1;
+                v2.map_axis[j] = v2.out_shape.dims[j] > 1 ? in_axis : -1;
+                v2.map_step[j] = v2.out_shape.dims[j] > 1 ? 1 : 0;
+            }
+            dsc_kernel_desc d2 = rd;
+            d2.inputs = &v2;
+            if (!validate(d1).empty() || !validate(d2).empty()) continue;
+            const int partials = n_nodes++;
+            node_bytes.push_back((size_t)(split * n_out) * 4);
+            is_graph_output.push_back(false);
+            is_graph_input.push_back(false);
+            Draft second;
+            second.fk = FusedKernel::plain(d2);
+            second.params = {partials, drafts[i].outs[0].node};
+            second.outs.push_back(drafts[i].outs[0]);
+            second.covers = drafts[i].covers;
+            Draft first;
+            first.fk = FusedKernel::plain(d1);
+            first.params = {drafts[i].params[0], partials};
+            first.outs.push_back(StepOutput{partials, -1, false, 0});
+            first.covers = drafts[i].covers;
+            first.keep_output = true;
+            drafts[i] = first;
+            drafts.insert(drafts.begin() + i + 1, second);
+            ++i;
+        }
+
         auto consumers_of = [&](int node) {
             std::vector<int> out;
             for (int i = 0; i < (int)drafts.size(); ++i) {
@@ -174,7 +364,7 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
         // Pass 1: MatMul (+ Reduce over its split-K partials) (+ per-element consumer as epilogue).
         for (int i = 0; i < (int)drafts.size(); ++i) {
             Draft& mm = drafts[i];
-            if (!mm.alive || mm.fk.main.raw().kind != DSC_KERNEL_MATMUL || mm.fk.has_epilogue) continue;
+            if (!mm.alive || mm.fk.main.raw().kind != DSC_KERNEL_MATMUL || mm.fk.has_epilogue || mm.keep_split) continue;
             const MatMulDims g = matmul_dims(mm.fk.main.raw());
             int product_node = mm.outs[0].node;
             if (is_graph_output[product_node]) continue;
@@ -272,6 +462,9 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             }
             return loads == 1;
         };
+        // tuning hook: DSC_FUSE_INTO_MATMUL=0 keeps producers of MatMul operands materialised
+        const char* fim = std::getenv("DSC_FUSE_INTO_MATMUL");
+        const bool fuse_into_matmul = !(fim && fim[0] == '0');
         bool changed = true;
         while (changed) {
             changed = false;
@@ -279,13 +472,36 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                 Draft& p = drafts[i];
                 if (!p.alive) continue;
                 const dsc_kernel_desc& pd = p.fk.main.raw();
-                if (pd.kind != DSC_KERNEL_PER_ELEMENT || pd.n_outputs != 1 || p.fk.has_epilogue) continue;
+                const bool is_pe = pd.kind == DSC_KERNEL_PER_ELEMENT && pd.n_outputs == 1 && !p.fk.has_epilogue;
+                const bool is_red = pd.kind == DSC_KERNEL_REDUCE;
+                if ((!is_pe && !is_red) || p.keep_output) continue;
                 const int node = p.outs[0].node;
                 if (is_graph_output[node] || p.outs[0].copy_from >= 0) continue;
-                if (!is_cheap_producer(pd)) continue;
+                if (is_pe && !is_cheap_producer(pd)) continue;
                 auto cons = consumers_of(node);
-                if (cons.empty() || (cons.size() > 1 && !is_pure_copy(pd))) continue;
+                if (cons.empty()) continue;
+                if (is_pe && cons.size() > 1 && !is_pure_copy(pd)) continue;
                 bool ok = true;
+                if (is_pe && !fuse_into_matmul)
+                    for (int ci : cons)
+                        if (drafts[ci].fk.main.raw().kind == DSC_KERNEL_MATMUL) ok = false;
+                if (is_red) {
+                    // a reduction is re-run by every element that reads it: only short ones, and only where the
+                    // consumers stay small
+                    const int64_t k = pd.inputs[0].out_shape.dims[pd.axis];
+                    const double unit = (double)k * draft_unit_cost(p);
+                    if (k > 64 || unit > 512.0) ok = false;
+                    for (int ci : cons) {
+                        const dsc_kernel_desc& cd = drafts[ci].fk.main.raw();
+                        const double per_read = unit * node_multiplicity(drafts[ci], node);  // loads per main-kernel read
+                        if ((double)draft_reads(drafts[ci]) * per_read > (double)(1 << 22) || cd.kind == DSC_KERNEL_MATMUL) ok = false;
+                        if (per_read > 512.0) ok = false;
+                        // a reduction consumer with few outputs would run the inlined loops serially per output
+                        if (cd.kind == DSC_KERNEL_REDUCE && element_count(cd.shape) < 4096 &&
+                            (double)cd.inputs[0].out_shape.dims[cd.axis] * per_read > 512.0)
+                            ok = false;
+                    }
+                }
                 for (int ci : cons) {
                     Draft& q = drafts[ci];
                     if (ci <= i) ok = false;
@@ -308,7 +524,7 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                     {
                         Virtual nv;
                         nv.pe = p.fk.main;
-                        nv.out_op = pd.outputs[0];
+                        nv.out_op = is_pe ? pd.outputs[0] : 0;
                         for (auto& s : p.fk.inputs) nv.inputs.push_back(import_source(q, p, s, voff));
                         q.fk.virtuals[new_virt] = nv;
                     }
@@ -360,6 +576,9 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
     std::vector<dsc_buf> buffer(n_nodes, 0);
     for (auto& st : steps)
         for (int n : st.inputs) usage[n] += 1;
+    // A node that becomes a parameter's new value stays alive even when later clusters also read it (the
+    // reference frees it after its last cluster use and then panics on the hand-off, environment.rs:491-515).
+    for (auto& io : outputs) usage[io.node] += 1;
 
     std::vector<bool> param_is_output(n_params, false), param_is_input(n_params, false);
     for (auto& io : outputs) param_is_output[io.param] = true;

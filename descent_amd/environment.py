@@ -182,6 +182,11 @@ class Environment:
             for n in cl.inputs:
                 usage[n] = usage.get(n, 0) + 1
 
+        # a node that becomes a parameter's new value must survive its other uses
+        for n in outputs:
+            (src,) = ops.predecessors(n)
+            usage[src] = usage.get(src, 0) + 1
+
         # inputs share the parameter's buffer, or take it when the parameter is rewritten
         for n in inputs:
             p = ops.nodes[n].op.a.checked(self)

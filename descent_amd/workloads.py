@@ -164,3 +164,188 @@ def matmul_epilogue(env: Environment, m: int, n: int, k: int, seed: int = 2, upl
         env.write_parameter(b, rng.standard_normal(k * n, dtype=np.float32))
         env.write_parameter(bias, rng.standard_normal(n, dtype=np.float32))
     return MatmulWorkload(env, graph, a, b, bias, c, m, n, k)
+
+
+# ---- image fit (examples/image_fit/main.rs) ----------------------------------------------------------------------
+def positional_encoding(x, freq_count: int):
+    """sin(x * 2^i * pi + {0, pi/2}) for i < freq_count: 2*freq_count features per input coordinate
+    (examples/image_fit/main.rs:259-275)."""
+    scope = x.scope
+    pi32 = float(np.float32(np.pi))
+    freq = scope.literal(2.0).pow(scope.coord(freq_count)) * pi32
+    phase = scope.coord(2).reshape([2, 1]) * 0.5 * pi32
+    shape = x.shape
+    calc_shape = tuple(shape) + (1, 1)
+    out_shape = tuple(shape[:-1]) + (shape[-1] * 2 * freq_count,)
+    return (x.reshape(calc_shape) * freq + phase).sin().reshape(out_shape)
+
+
+class ReluMlp(Module):
+    """examples/image_fit/main.rs:52-87 (`Relu`; its activation is leaky_relu(0.01))."""
+
+    def __init__(self, env, freq_count: int, hidden_units, n_in: int = 2):
+        self.freq_count = freq_count
+        prev = n_in if freq_count == 0 else 2 * n_in * freq_count
+        self.hidden = []
+        for h in hidden_units:
+            self.hidden.append(Dense(env, prev, h))
+            prev = h
+        self.final = Dense(env, prev, 3)
+
+    def eval(self, x, ctx):
+        if self.freq_count:
+            x = positional_encoding(x, self.freq_count)
+        for layer in self.hidden:
+            x = x.apply(layer, ctx).leaky_relu(0.01)
+        return x.apply(self.final, ctx)
+
+
+class Siren(Module):
+    """examples/image_fit/main.rs:89-128: sin activations; omega_0 = 30 enters through the first layer's
+    initialiser scale (src/parameter.rs:22-25)."""
+
+    def __init__(self, env, hidden_units, n_in: int = 2):
+        from .module import Initializer
+
+        prev = n_in
+        self.hidden = []
+        for i, h in enumerate(hidden_units):
+            self.hidden.append(Dense(env, prev, h, Initializer.for_siren(prev, i == 0), Initializer.rand_uniform(1.0)))
+            prev = h
+        self.final = Dense(env, prev, 3)
+
+    def eval(self, x, ctx):
+        for layer in self.hidden:
+            x = x.apply(layer, ctx).sin()
+        return x.apply(self.final, ctx)
+
+
+HASH_PRIME = 1526263  # examples/image_fit/main.rs:139
+
+# floor(16 * b^i), b = exp((ln 2048 - ln 16) / 15): the reference evaluates this in f32 and its top level can
+# land on 2047 or 2048 depending on rounding (examples/image_fit/main.rs:222-228); the table is fixed here.
+HASH_LEVEL_SIZES = (16, 22, 30, 42, 58, 80, 111, 153, 212, 294, 406, 561, 776, 1072, 1482, 2048)
+
+
+class HashGrid(Module):
+    """One level: bilinear interpolation of 4 gathered table entries; backward scatters into the table
+    (examples/image_fit/main.rs:120-203)."""
+
+    def __init__(self, env, grid_size: int, entry_count: int, values_per_entry: int):
+        from .module import Initializer
+
+        points = grid_size + 1
+        full = points * points
+        entry_count = min(entry_count, full)
+        self.grid_size = grid_size
+        self.stride = points if entry_count == full else HASH_PRIME
+        self.t = env.trainable_parameter([entry_count, values_per_entry], "t", Initializer.rand_uniform(1.0e-4))
+
+    def eval(self, x, ctx):
+        from .array import DualArray
+
+        scope = x.scope
+        xv, _ = x.next_colour().into_inner()
+        t, dt = scope.parameter(self.t).into_inner()
+        entry_count = t.shape[0]
+        stride = self.stride
+
+        cf = (xv * 0.5 + 0.5) * float(self.grid_size)
+        c = cf.into_u32()
+        f = cf - c.into_f32()
+        c0, c1 = c.lock_axis(-1, 0, False), c.lock_axis(-1, 1, False)
+        f0, f1 = f.lock_axis(-1, 0, True), f.lock_axis(-1, 1, True)
+
+        ia = ((c0 + 0) ^ (c1 * stride + 0)) % entry_count
+        ib = ((c0 + 1) ^ (c1 * stride + 0)) % entry_count
+        ic = ((c0 + 0) ^ (c1 * stride + stride)) % entry_count
+        id_ = ((c0 + 1) ^ (c1 * stride + stride)) % entry_count
+
+        ta, tb, tc, td = (t.gather(-2, i) for i in (ia, ib, ic, id_))
+        g0, g1 = 1.0 - f0, 1.0 - f1
+        wa, wb, wc, wd = g0 * g1, f0 * g1, g0 * f1, f0 * f1
+        y, dy = (ta * wa + tb * wb + tc * wc + td * wd).with_empty_grad()
+        dt.accumulate(
+            scope.literal(0.0).value().broadcast(dt.shape)
+            .scatter_add(dy * wa, -2, ia).scatter_add(dy * wb, -2, ib)
+            .scatter_add(dy * wc, -2, ic).scatter_add(dy * wd, -2, id_)
+        )
+        return DualArray(y, dy)
+
+
+class MultiHashGrid(Module):
+    """examples/image_fit/main.rs:205-257: levels concatenated pairwise, then an MLP decoder."""
+
+    def __init__(self, env, level_sizes, entry_count: int, hidden_units, values_per_entry: int = 2):
+        self.grids = [HashGrid(env, g, entry_count, values_per_entry) for g in level_sizes]
+        prev = len(self.grids) * values_per_entry
+        self.hidden = []
+        for h in hidden_units:
+            self.hidden.append(Dense(env, prev, h))
+            prev = h
+        self.final = Dense(env, prev, 3)
+
+    def eval(self, x, ctx):
+        out = None
+        for grid in self.grids:
+            y = grid.eval(x, ctx)
+            out = y if out is None else out.concat(y, -1)
+        for layer in self.hidden:
+            out = layer.eval(out, ctx).leaky_relu(0.01)
+        return self.final.eval(out, ctx)
+
+
+def sinusoid_image(points: np.ndarray, seed: int = 4) -> np.ndarray:
+    """Target RGB in [0,1]: a seeded sum of 32 random 2-D sinusoids, clamped.  `points` is [m, 2] in [0,1]^2."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    freq = rng.uniform(-12.0, 12.0, (32, 2))
+    phase = rng.uniform(0.0, 2 * np.pi, (32, 3))
+    amp = rng.uniform(0.0, 0.25, (32, 3))
+    arg = points.astype(np.float64) @ freq.T * (2 * np.pi)  # [m, 32]
+    rgb = 0.5 + (np.sin(arg[:, :, None] + phase[None]) * amp[None]).sum(axis=1)
+    return np.clip(rgb, 0.0, 1.0).astype(np.float32)
+
+
+def _image_fit_workload(env: Environment, module: Module, points01: np.ndarray, rng, lr: float, betas, signed_inputs: bool) -> Workload:
+    """Train-graph assembly of examples/image_fit/main.rs:303-332: L2 loss, Adam."""
+    m = points01.shape[0]
+    x_param = env.static_parameter([m, 2], "x")
+    y_param = env.static_parameter([m, 3], "y")
+    loss_sum = env.static_parameter([1], "loss")
+    scope = env.scope()
+    out = module.train(scope.parameter(x_param))
+    loss = (out - y_param).square().reduce_sum(-1, True).set_loss()
+    scope.update_parameter_value(loss_sum, lambda s: s + loss.reduce_sum(0, False))
+    parameters = scope.trainable_parameters()
+    opt = Adam(env, scope, parameters, lr, betas[0], betas[1], 1e-8)
+    graph = scope.build_graph()
+    for p in parameters:
+        env.reset_parameter(p, rng)
+    env.writer(loss_sum).zero_fill()
+    x = (points01 * 2.0 - 1.0) if signed_inputs else points01
+    env.write_parameter(x_param, x.astype(np.float32))
+    env.write_parameter(y_param, sinusoid_image(points01))
+    return Workload(env, graph, {"x": x_param, "y": y_param}, parameters, opt.state, {"loss": loss_sum})
+
+
+def coordinate_mlp(env: Environment, side: int = 512, variant: str = "relu-pe", hidden=(256, 256, 256, 256),
+                   freq_count: int = 16, seed: int = 5) -> Workload:
+    """Coordinate MLP image fit: every point of a side x side grid in [0,1]^2; "relu-pe" = positional encoding
+    (freq_count sin/cos pairs per axis) + leaky_relu(0.01) hidden layers, "siren" = sin activations; Adam lr 1e-3."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    axis = (np.arange(side, dtype=np.float64) + 0.5) / side
+    pts = np.stack(np.meshgrid(axis, axis, indexing="xy"), axis=-1).reshape(-1, 2)
+    module = Siren(env, hidden) if variant == "siren" else ReluMlp(env, freq_count, hidden)
+    # the SIREN consumes coordinates in [-1, 1] as the reference feeds them (examples/image_fit/main.rs:372-375)
+    return _image_fit_workload(env, module, pts, rng, 1e-3, (0.9, 0.999), signed_inputs=variant == "siren")
+
+
+def hash_grid_fit(env: Environment, batch: int = 1 << 18, levels=HASH_LEVEL_SIZES, entry_count: int = 1 << 19,
+                  hidden=(64, 64), seed: int = 6) -> Workload:
+    """Multi-level hash encoding image fit: `batch` uniform points of [0,1]^2 (fed as 2u-1, the domain the
+    reference's HashGrid maps back with x*0.5+0.5), 2 features per entry, tables U(+-1e-4), decoder MLP with
+    leaky_relu(0.01), L2 loss, Adam lr 1e-3."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    pts = rng.random((batch, 2)) * (1.0 - 1e-6)
+    module = MultiHashGrid(env, levels, entry_count, hidden)
+    return _image_fit_workload(env, module, pts, rng, 1e-3, (0.9, 0.999), signed_inputs=True)

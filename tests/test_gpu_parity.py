@@ -157,3 +157,68 @@ def test_heap_reuse_and_errors(hip_backend_session):
     got = np.frombuffer(be.read(h, 0, 64), np.float32)
     assert np.array_equal(got, np.concatenate([np.arange(8, dtype=np.float32), np.zeros(8, np.float32)]))
     be.free(h)
+
+
+@pytest.mark.parametrize("variant", ["relu-pe", "siren"])
+def test_coordinate_mlp_steps_vs_oracle(hip_backend_session, variant):
+    """Config 4 at reduced size (64x64 grid, two hidden layers of 64): three Adam steps."""
+    from descent_amd import workloads
+
+    genv, cenv = _envs(hip_backend_session)
+    gw = workloads.coordinate_mlp(genv, side=64, variant=variant, hidden=(64, 64), freq_count=8, seed=21)
+    cw = workloads.coordinate_mlp(cenv, side=64, variant=variant, hidden=(64, 64), freq_count=8, seed=21)
+    for step in range(3):
+        genv.run(gw.graph, step)
+        cenv.run(cw.graph, step)
+    got, want = gw.snapshot(), cw.snapshot()
+    for key in want:
+        err = rel_l2(got[key], want[key])
+        assert err <= TOL, f"{variant} {key}: rel L2 {err}"
+
+
+def test_hash_grid_steps_vs_oracle(hip_backend_session):
+    """Config 5 at reduced size: dense and hashed levels, bilinear gathers, float-atomic scatter-add.
+    The atomic adds reorder fp32 sums, so the bound is the looser 1e-3 (relative L2) for every tensor here:
+    the tables directly, everything else through them after the first step."""
+    from descent_amd import workloads
+
+    genv, cenv = _envs(hip_backend_session)
+    kw = dict(batch=8192, levels=(4, 16, 40, 100), entry_count=2048, hidden=(32,), seed=22)
+    gw = workloads.hash_grid_fit(genv, **kw)
+    cw = workloads.hash_grid_fit(cenv, **kw)
+    for step in range(3):
+        genv.run(gw.graph, step)
+        cenv.run(cw.graph, step)
+    got, want = gw.snapshot(), cw.snapshot()
+    for key in want:
+        err = rel_l2(got[key], want[key])
+        assert err <= 1e-3, f"{key}: rel L2 {err}"
+
+
+def test_gather_indices_are_bit_exact(hip_backend_session):
+    """The hash index arithmetic (u32 xor / mul / rem on bit-cast floats) and the gathered values must match
+    the oracle bit for bit."""
+    genv, cenv = _envs(hip_backend_session)
+
+    def run(env):
+        rng = np.random.default_rng(3)
+        pts = env.static_parameter_with_data([4096, 2], "x", rng.random((4096, 2), dtype=np.float32) * 2 - 1)
+        table = env.static_parameter_with_data([2048, 2], "t", rng.standard_normal((2048, 2), dtype=np.float32))
+        idx_out = env.static_parameter([4096], "i")
+        val_out = env.static_parameter([4096, 2], "v")
+
+        def build(s):
+            cf = (s.parameter_value(pts) * 0.5 + 0.5) * 100.0
+            c = cf.into_u32()
+            c0, c1 = c.lock_axis(-1, 0, False), c.lock_axis(-1, 1, False)
+            i = ((c0 + 1) ^ (c1 * 1526263 + 1526263)) % 2048
+            s.write_parameter_value(idx_out, i.to_f32_bits())
+            s.write_parameter_value(val_out, s.parameter_value(table).gather(-2, i))
+
+        env.run(env.build_graph(build), 0)
+        return env.read_parameter(idx_out).view(np.uint32), env.read_parameter(val_out)
+
+    gi, gv = run(genv)
+    ci, cv = run(cenv)
+    assert np.array_equal(gi, ci) and gi.max() < 2048
+    assert np.array_equal(gv.view(np.uint32), cv.view(np.uint32))

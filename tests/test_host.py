@@ -198,3 +198,19 @@ def test_writer_zero_fills_the_unwritten_tail():
     with env.writer(p) as w:
         w.write(np.arange(3, dtype=np.float32))
     assert np.array_equal(env.read_parameter_to_vec(p), np.array([0, 1, 2, 0, 0, 0, 0, 0], np.float32))
+
+
+def test_image_fit_parameter_counts_match_the_reference_readme():
+    """examples/image_fit/README.md:31-34: ReLU 44099, ReLU-PE 51779, SIREN 44099, MULTI-HASH 43977 trainable
+    parameters for hidden units [256,128,64,32], 8 frequencies, and 10 levels from 2 to 512 with 4096 entries."""
+    env = _env()
+    hidden = (256, 128, 64, 32)
+    count = lambda m: sum(p.shape.element_count() for p in [q for layer in m.hidden + [m.final] for q in (layer.w, layer.b)])
+    assert count(workloads.ReluMlp(env, 0, hidden)) == 44099
+    assert count(workloads.ReluMlp(env, 8, hidden)) == 51779
+    assert count(workloads.Siren(env, hidden)) == 44099
+    b = np.exp((np.log(np.float32(512)) - np.log(np.float32(2))) / np.float32(9)).astype(np.float32)
+    sizes = [int(np.float32(2) * b ** np.float32(i)) for i in range(10)]
+    mh = workloads.MultiHashGrid(env, sizes, 4096, (64, 64))
+    total = count(mh) + sum(g.t.shape.element_count() for g in mh.grids)
+    assert total == 43977, (total, sizes)
