@@ -27,20 +27,29 @@ MFMA_FP32_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBS = 8000.0
 
 
-def time_graph(env, graph, steps: int, warmup: int, seed0: int = 1):
-    """W untimed runs, then K timed runs bracketed by stream syncs.  Returns (wall seconds, profiler report)."""
+def time_graph(env, graph, steps: int, warmup: int, seed0: int = 1, profile: bool = True):
+    """W untimed runs, then K timed runs bracketed by stream syncs; returns the wall seconds of the K runs.
+    With `profile` every launch of the timed region is bracketed by HIP events on the context's stream (per-kernel
+    durations for dsc_prof_query / the report).  The events cost a few microseconds per launch, so schedules
+    made of many small kernels are timed with profile=False and profiled in a second, untimed pass."""
     be = env.backend
     for i in range(warmup):
         env.run(graph, seed0 + i)
     be.sync()
     be.profile_reset()
-    be.profile(True)
+    be.profile(profile)
     t0 = time.perf_counter()
     for i in range(steps):
         env.run(graph, seed0 + warmup + i)
     be.sync()
     wall = time.perf_counter() - t0
     be.profile(False)
+    return wall
+
+
+def time_then_profile(env, graph, steps: int, warmup: int):
+    wall = time_graph(env, graph, steps, warmup, profile=False)
+    time_graph(env, graph, steps, 0, seed0=1000, profile=True)
     return wall
 
 
@@ -75,7 +84,7 @@ def bench_convnet(env, steps, warmup, batch=1000):
     from descent_amd import workloads
 
     w = workloads.convnet(env, batch=batch, seed=3)
-    wall = time_graph(env, w.graph, steps, warmup)
+    wall = time_then_profile(env, w.graph, steps, warmup)
     report = env.backend.timing_report(int(os.environ.get("DSC_BENCH_TOPN", "12")))
     env.backend.profile_reset()
     sched = next(iter(w.graph.__dict__["_schedules"].values()))
@@ -112,7 +121,7 @@ def bench_elementwise(env, n, steps, warmup):
 def bench_workload(env, build, steps, warmup, topn=8):
     """Step rate of one of the image-fit configurations, with the per-kernel table."""
     w = build(env)
-    wall = time_graph(env, w.graph, steps, warmup)
+    wall = time_then_profile(env, w.graph, steps, warmup)
     be = env.backend
     out = {"steps_per_s": steps / wall, "ms_per_step": 1e3 * wall / steps}
     for prefix in ("MatMul", "ScatterAdd", "PerElement", "Reduce"):

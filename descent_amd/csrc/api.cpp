@@ -90,6 +90,15 @@ int dsc_ctx_create(int device_ordinal, dsc_ctx** out) {
         delete ctx;
         return fail(DSC_ERR_HIP, std::string("hipStreamCreate: ") + hipGetErrorString(e));
     }
+    {
+        void* cell = nullptr;
+        e = hipMalloc(&cell, 256);
+        if (e != hipSuccess) {
+            delete ctx;
+            return fail(DSC_ERR_HIP, std::string("seed cell: ") + hipGetErrorString(e));
+        }
+        c.seed_cell = static_cast<uint32_t*>(cell);
+    }
     for (int i = 0; i < Context::kStagingRegions; ++i) {
         void* p = nullptr;
         e = hipHostMalloc(&p, Context::kStagingBytes, hipHostMallocDefault);

@@ -62,6 +62,14 @@ struct Emitter {
         s += "uint rand_seed";
         return s;
     }
+    // The __global__ signature: the seed arrives through a one-word device cell so that a captured launch
+    // sequence can be replayed with a new seed without touching its kernel arguments.
+    string kernel_params_decl() const {
+        string s;
+        for (int i = 0; i < fk.n_buffers; ++i)
+            s += (fk.buffer_is_output[i] ? "float* __restrict__ b" : "const float* __restrict__ b") + to_string(i) + ", ";
+        return s + "const uint* __restrict__ seed_cell";
+    }
     string params_pass() const {
         string s;
         for (int i = 0; i < fk.n_buffers; ++i) s += "b" + to_string(i) + ", ";
@@ -348,6 +356,19 @@ struct Emitter {
     }
 };
 
+string entry_name(const FusedKernel& fk) {
+    switch (fk.main.raw().kind) {
+    case DSC_KERNEL_FILL: return "dsc_fill";
+    case DSC_KERNEL_PER_ELEMENT: return "dsc_per_element";
+    case DSC_KERNEL_REDUCE: return "dsc_reduce";
+    case DSC_KERNEL_MATMUL: return fk.has_epilogue ? "dsc_matmul_mfma_epilogue" : "dsc_matmul_mfma";
+    case DSC_KERNEL_UNPAD: return "dsc_unpad";
+    case DSC_KERNEL_WINDOWS_TO_IMAGE: return "dsc_windows_to_image";
+    case DSC_KERNEL_SCATTER_ADD: return "dsc_scatter_add";
+    default: return "dsc_kernel";
+    }
+}
+
 string check_sizes(const FusedKernel& fk) {
     auto chk = [](const dsc_kernel_desc& d) -> string {
         if (element_count(d.shape) >= kMaxIndex) return "kernel too large for 32-bit indexing";
@@ -375,7 +396,7 @@ string gen_fill(Emitter& em, Generated* out) {
     const int64_t n = d.shape.dims[0];
     std::ostringstream k;
     const bool vec = n % 4 == 0;
-    k << "extern \"C\" __global__ __launch_bounds__(256) void dsc_kernel(" << em.params_decl() << ") {\n";
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = *seed_cell;\n";
     k << "    const uint i = blockIdx.x * 256u + threadIdx.x;\n";
     if (vec) {
         k << "    if (i >= " << S(n / 4) << "u) return;\n";
@@ -399,7 +420,7 @@ string gen_per_element(Emitter& em, Generated* out) {
     const int64_t n = d.shape.dims[0];
     const int vec = (n % 4 == 0 && n >= 4096) ? 4 : 1;
     std::ostringstream k;
-    k << "extern \"C\" __global__ __launch_bounds__(256) void dsc_kernel(" << em.params_decl() << ") {\n";
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = *seed_cell;\n";
     k << "    const uint base = (blockIdx.x * 256u + threadIdx.x) * " << vec << "u;\n";
     k << "    if (base >= " << S(n) << "u) return;\n";
     std::map<int, string> override_load;
@@ -473,7 +494,7 @@ string gen_reduce(Emitter& em, Generated* out) {
     }
 
     std::ostringstream k;
-    k << "extern \"C\" __global__ __launch_bounds__(256) void dsc_kernel(" << em.params_decl() << ") {\n";
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = *seed_cell;\n";
     // The k loop is unrolled four times over independent accumulators so that four loads are in flight per
     // thread; `first`/`step` give the thread's k sequence.
     auto emit_k_loop = [&](const std::vector<string>& oc, const string& first, int64_t step) {
@@ -587,7 +608,7 @@ string gen_unpad(Emitter& em, Generated* out) {
     const dsc_view& v = d.inputs[0];
     const int64_t n = element_count(d.shape);
     std::ostringstream k;
-    k << "extern \"C\" __global__ __launch_bounds__(256) void dsc_kernel(" << em.params_decl() << ") {\n";
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = *seed_cell;\n";
     k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n";
     auto c = em.emit_coords(k, d.shape, "gid", "c");
     const string oc = c[d.axis];
@@ -617,7 +638,7 @@ string gen_windows_to_image(Emitter& em, Generated* out) {
     const int bd = d.shape.rank - 3;
     const int64_t n = element_count(d.shape);
     std::ostringstream k;
-    k << "extern \"C\" __global__ __launch_bounds__(256) void dsc_kernel(" << em.params_decl() << ") {\n";
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = *seed_cell;\n";
     k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n";
     auto c = em.emit_coords(k, d.shape, "gid", "c");
     k << "    const int in_y = " << c[bd] << ", in_x = " << c[bd + 1] << ", in_c = " << c[bd + 2] << ";\n";
@@ -651,7 +672,7 @@ string gen_scatter_add(Emitter& em, Generated* out) {
     const dsc_view& vi = d.inputs[1];
     const int64_t n = element_count(vv.out_shape);
     std::ostringstream k;
-    k << "extern \"C\" __global__ __launch_bounds__(256) void dsc_kernel(" << em.params_decl() << ") {\n";
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = *seed_cell;\n";
     k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n";
     auto c = em.emit_coords(k, vv.out_shape, "gid", "c");
     k << "    const float value = " << em.load_view(fk.inputs[0], vv, c) << ";\n";
@@ -782,7 +803,7 @@ string gen_matmul(Emitter& em, Generated* out) {
     const int64_t batch_stride = rows ? g.n : g.m * g.n, row_stride = rows ? g.batch * g.n : g.n;
     k << "#define C_CHUNK_STRIDE " << S(g.batch * g.m * g.n) << "\n#define C_BATCH_STRIDE " << S(batch_stride)
       << "\n#define C_ROW_STRIDE " << S(row_stride) << "\n";
-    k << "#define MM_PARAMS " << em.params_decl() << "\n";
+    k << "#define MM_PARAMS " << em.kernel_params_decl() << "\n#define MM_ENTRY " << entry_name(fk) << "\n";
 
     if (fk.has_epilogue) {
         const dsc_kernel_desc& pe = fk.epilogue.raw();
@@ -893,6 +914,7 @@ std::string generate(const FusedKernel& fk, Generated* out) {
     if (!err.empty()) return err;
     g.source = string(kPreludeSource) + "\n" + em.funcs.str() + "\n" + g.source;
     g.n_buffers = fk.n_buffers;
+    g.entry = entry_name(fk);
     *out = g;
     return "";
 }

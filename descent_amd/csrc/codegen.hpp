@@ -50,10 +50,11 @@ struct FusedKernel {
 };
 
 struct Generated {
-    std::string source;      // complete translation unit; entry point is `dsc_kernel`
+    std::string source;      // complete translation unit
+    std::string entry;       // name of the __global__ function (dsc_<kind>)
     unsigned grid = 1;       // workgroups (1-D)
     unsigned block = 64;     // threads per workgroup
-    int n_buffers = 0;       // pointer parameters, in order; followed by `uint rand_seed`
+    int n_buffers = 0;       // pointer parameters, in order; followed by `const uint* seed_cell`
     std::string note;        // strategy chosen (for schedule listings)
 };
 

@@ -152,6 +152,7 @@ Context::~Context() {
         if (staging_done[i]) (void)hipEventDestroy(staging_done[i]);
         if (staging[i]) (void)hipHostFree(staging[i]);
     }
+    if (seed_cell) (void)hipFree(seed_cell);
     if (stream) (void)hipStreamDestroy(stream);
 }
 
@@ -285,7 +286,7 @@ Kernel* get_kernel(Context* ctx, const FusedKernel& fk, int* status) {
         *status = fail(DSC_ERR_HIP, std::string("hipModuleLoadData: ") + hipGetErrorString(e));
         return nullptr;
     }
-    e = hipModuleGetFunction(&k->function, k->module, "dsc_kernel");
+    e = hipModuleGetFunction(&k->function, k->module, k->gen.entry.c_str());
     if (e != hipSuccess) {
         *status = fail(DSC_ERR_HIP, std::string("hipModuleGetFunction: ") + hipGetErrorString(e));
         return nullptr;
@@ -296,8 +297,20 @@ Kernel* get_kernel(Context* ctx, const FusedKernel& fk, int* status) {
     return raw;
 }
 
+int set_seed(Context* ctx, uint32_t rand_seed) {
+    if (ctx->seed_known && ctx->seed_value == rand_seed) return DSC_OK;
+    HIP_TRY(hipMemsetD32Async(reinterpret_cast<hipDeviceptr_t>(ctx->seed_cell), (int)rand_seed, 1, ctx->stream));
+    ctx->seed_value = rand_seed;
+    ctx->seed_known = true;
+    return DSC_OK;
+}
+
 int launch_kernel(Context* ctx, Kernel* k, void* const* device_ptrs, int n, uint32_t rand_seed) {
     if (ctx->offline || !k->function) return fail(DSC_ERR_NO_DEVICE, "kernel launch without a device");
+    {
+        int rc = set_seed(ctx, rand_seed);
+        if (rc != DSC_OK) return rc;
+    }
     if (n != k->gen.n_buffers)
         return fail(DSC_ERR_INVALID, "kernel '" + k->label + "' takes " + std::to_string(k->gen.n_buffers) + " buffers, got " +
                                          std::to_string(n));
@@ -308,7 +321,8 @@ int launch_kernel(Context* ctx, Kernel* k, void* const* device_ptrs, int n, uint
         ptr_values[i] = device_ptrs[i];
         args[i] = &ptr_values[i];
     }
-    args[n] = &rand_seed;
+    void* seed_ptr = ctx->seed_cell;
+    args[n] = &seed_ptr;
     hipEvent_t start = nullptr, stop = nullptr;
     if (ctx->profiling) {
         auto take = [&](hipEvent_t* ev) -> hipError_t {

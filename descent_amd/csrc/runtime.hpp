@@ -89,6 +89,11 @@ struct Context {
     bool staging_busy[kStagingRegions] = {false, false};
     int staging_next = 0;
 
+    // one device word holding the rand seed of the launches that follow (kernels read it at entry)
+    uint32_t* seed_cell = nullptr;
+    uint32_t seed_value = 0;
+    bool seed_known = false;
+
     std::unordered_map<std::string, std::unique_ptr<Kernel>> kernels;  // by FusedKernel::key()
 
     bool profiling = false;
@@ -101,6 +106,8 @@ struct Context {
 // Compiles (or fetches) the kernel for a fused descriptor.  Returns nullptr and sets the error on failure.
 Kernel* get_kernel(Context* ctx, const FusedKernel& fk, int* status);
 int launch_kernel(Context* ctx, Kernel* k, void* const* device_ptrs, int n, uint32_t rand_seed);
+// Makes `rand_seed` the seed seen by launches enqueued after this call.
+int set_seed(Context* ctx, uint32_t rand_seed);
 // hipRTC compile without a device.
 int compile_source(const std::string& source, const std::string& arch, std::vector<char>* code, std::string* log);
 

@@ -283,6 +283,12 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             const int axis = rd.axis;
             const int64_t k = v.out_shape.dims[axis], n_out = element_count(rd.shape);
             if (k < 512 || n_out > 16384 || (k * n_out < (1 << 20) && k < 8192) || v.map_axis[axis] < 0 || needs_clamp(v, v.map_axis[axis])) continue;
+            {
+                // rows that are contiguous along k are already read by whole wavefronts (one group of lanes per
+                // output): with enough outputs that form is bandwidth bound on its own
+                int64_t base, coef[DSC_MAX_DIM];
+                if (n_out >= 1024 && affine_form(v, &base, coef) && coef[axis] == 1) continue;
+            }
             const int64_t want = std::min<int64_t>(2048, std::max<int64_t>(2, (524288 + n_out - 1) / n_out));
             int64_t split = 0;
             for (int64_t c = want; c <= k / 8; ++c)
@@ -601,7 +607,16 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
         }
     }
 
-    void* ptrs[64];
+    // Pass 1: buffer bookkeeping only -- resolve every launch's pointers (allocation and release are host-side
+    // and stream-ordered, so a buffer freed here may be handed to a later launch of the same step).
+    struct Launch {
+        Kernel* kernel;
+        size_t first;  // index into `pointers`
+        int n;
+    };
+    std::vector<Launch> launches;
+    std::vector<void*> pointers;
+    launches.reserve(steps.size() + 4);
     for (auto& st : steps) {
         for (int n : st.inputs) usage[n] -= 1;
         for (auto& o : st.outputs) {
@@ -619,8 +634,8 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
                     if (!h) return fail(DSC_ERR_OOM, "schedule run: out of device memory");
                     void* p = nullptr;
                     ctx->heap.info(h, &p, nullptr);
-                    int rc = launch_kernel(ctx, o.fill, &p, 1, rand_seed);
-                    if (rc != DSC_OK) return rc;
+                    launches.push_back(Launch{o.fill, pointers.size(), 1});
+                    pointers.push_back(p);
                 } else {
                     return fail(DSC_ERR_INVALID, "schedule run: cannot copy-on-write node");
                 }
@@ -629,14 +644,13 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
             buffer[o.node] = h;
         }
         const int n = (int)st.params.size();
+        launches.push_back(Launch{st.kernel, pointers.size(), n});
         for (int i = 0; i < n; ++i) {
             void* p = nullptr;
             if (!ctx->heap.info(buffer[st.params[i]], &p, nullptr))
                 return fail(DSC_ERR_INVALID, "schedule run: node " + std::to_string(st.params[i]) + " has no buffer at '" + st.kernel->label + "'");
-            ptrs[i] = p;
+            pointers.push_back(p);
         }
-        int rc = launch_kernel(ctx, st.kernel, ptrs, n, rand_seed);
-        if (rc != DSC_OK) return rc;
         for (int nd : st.inputs) {
             if (usage[nd] == 0 && buffer[nd] != 0) {
                 ctx->heap.free(buffer[nd]);
@@ -649,12 +663,71 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
         params[io.param] = buffer[io.node];
         buffer[io.node] = 0;
     }
+
+    // Pass 2: enqueue.  With per-launch timing on, or graphs off, launch one by one; otherwise replay the graph
+    // captured for this exact pointer table, capturing it first if it is new.
+    auto enqueue_all = [&]() -> int {
+        for (auto& l : launches) {
+            int rc = launch_kernel(ctx, l.kernel, pointers.data() + l.first, l.n, rand_seed);
+            if (rc != DSC_OK) return rc;
+        }
+        return DSC_OK;
+    };
+    static const bool graphs_enabled = [] {
+        // opt-in: replay needs a step's buffers to land on the same addresses again, which the shared best-fit
+        // heap does not guarantee (parameter buffers move every step), so by default launches are enqueued directly
+        const char* e = std::getenv("DSC_GRAPHS");
+        return e && e[0] == '1';
+    }();
+    if (ctx->profiling || !graphs_enabled || launches.size() < 4) {
+        ++direct_runs;
+        return enqueue_all();
+    }
+    int rc = set_seed(ctx, rand_seed);
+    if (rc != DSC_OK) return rc;
+    for (auto& c : captured) {
+        if (c.pointers == pointers) {
+            ++replays;
+            hipError_t e = hipGraphLaunch(c.exec, ctx->stream);
+            if (e != hipSuccess) return fail(DSC_ERR_HIP, std::string("hipGraphLaunch: ") + hipGetErrorString(e));
+            return DSC_OK;
+        }
+    }
+    if (captured.size() >= kMaxCaptured) {
+        ++direct_runs;
+        return enqueue_all();
+    }
+    hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
+    if (e != hipSuccess) return fail(DSC_ERR_HIP, std::string("hipStreamBeginCapture: ") + hipGetErrorString(e));
+    rc = enqueue_all();
+    hipGraph_t graph = nullptr;
+    e = hipStreamEndCapture(ctx->stream, &graph);
+    if (rc != DSC_OK) {
+        if (graph) (void)hipGraphDestroy(graph);
+        return rc;
+    }
+    if (e != hipSuccess) return fail(DSC_ERR_HIP, std::string("hipStreamEndCapture: ") + hipGetErrorString(e));
+    CapturedStep c;
+    c.pointers = pointers;
+    e = hipGraphInstantiate(&c.exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return fail(DSC_ERR_HIP, std::string("hipGraphInstantiate: ") + hipGetErrorString(e));
+    captured.push_back(c);
+    e = hipGraphLaunch(c.exec, ctx->stream);
+    if (e != hipSuccess) return fail(DSC_ERR_HIP, std::string("hipGraphLaunch: ") + hipGetErrorString(e));
     return DSC_OK;
+}
+
+Schedule::~Schedule() {
+    for (auto& c : captured)
+        if (c.exec) (void)hipGraphExecDestroy(c.exec);
 }
 
 std::string Schedule::describe() const {
     std::ostringstream o;
     o << steps.size() << " launches for " << n_clusters << " clusters\n";
+    if (replays + direct_runs + (int64_t)captured.size() > 0)
+        o << "# graph replays " << replays << ", captured " << captured.size() << ", direct runs " << direct_runs << "\n";
     for (size_t i = 0; i < steps.size(); ++i) {
         const Step& st = steps[i];
         o << i << ": " << st.kernel->label << "  [" << st.kernel->gen.note << "] grid " << st.kernel->gen.grid << "x"

@@ -22,7 +22,19 @@ struct Step {
     std::vector<int> covers;   // reference cluster indices this launch stands for
 };
 
+// One step's launches with their resolved device pointers, captured once as a HIP graph and replayed whenever a
+// later step resolves to the same pointers (parameter buffers alternate between a few addresses).
+struct CapturedStep {
+    std::vector<void*> pointers;  // every pointer argument of every launch, in order
+    hipGraphExec_t exec = nullptr;
+};
+
 struct Schedule {
+    static constexpr size_t kMaxCaptured = 8;
+    std::vector<CapturedStep> captured;
+    int64_t replays = 0, direct_runs = 0;
+    ~Schedule();
+
     int n_nodes = 0, n_params = 0, n_clusters = 0;
     std::vector<size_t> node_bytes;
     std::vector<dsc_param_io> inputs, outputs;
