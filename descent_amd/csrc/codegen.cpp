@@ -356,12 +356,16 @@ struct Emitter {
     }
 };
 
+bool rows_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
+
 string entry_name(const FusedKernel& fk) {
     switch (fk.main.raw().kind) {
     case DSC_KERNEL_FILL: return "dsc_fill";
     case DSC_KERNEL_PER_ELEMENT: return "dsc_per_element";
     case DSC_KERNEL_REDUCE: return "dsc_reduce";
-    case DSC_KERNEL_MATMUL: return fk.has_epilogue ? "dsc_matmul_mfma_epilogue" : "dsc_matmul_mfma";
+    case DSC_KERNEL_MATMUL:
+        if (rows_kernel_applies(fk, matmul_dims(fk.main.raw()))) return fk.has_epilogue ? "dsc_matmul_rows_epilogue" : "dsc_matmul_rows";
+        return fk.has_epilogue ? "dsc_matmul_mfma_epilogue" : "dsc_matmul_mfma";
     case DSC_KERNEL_UNPAD: return "dsc_unpad";
     case DSC_KERNEL_WINDOWS_TO_IMAGE: return "dsc_windows_to_image";
     case DSC_KERNEL_SCATTER_ADD: return "dsc_scatter_add";
@@ -742,6 +746,115 @@ MmConfig pick_config(int64_t M, int64_t N, int64_t groups /* batch * k-chunks */
     return c;
 }
 
+// Row-per-thread matmul for tall products with a narrow output (N <= 32, K <= 256): the HBM-bound GEMMs of the
+// convolutions (N = 16, K = 9 / 72) and of the narrow output layers.  Every thread owns one row of C in
+// registers.  B's address is the same for every lane of a wave, so the compiler fetches it with scalar loads
+// and the FMAs take it as an SGPR operand: no LDS traffic, no barrier.  The k loop is unrolled, so everything
+// in an operand's address that depends only on k (the filter tap of an im2col view) is a constant and only
+// the row part (image, y, x) is computed per lane, once.  No MFMA: these products have 3-7 flop per byte.
+bool rows_kernel_applies(const FusedKernel& fk, const MatMulDims& g) {
+    if (const char* e = std::getenv("DSC_MM_ROWS"))
+        if (e[0] == '0') return false;
+    if (g.chunks != 1 && !fk.sum_chunks) return false;
+    return g.n <= 32 && g.k <= 256 && g.k * g.n <= 8192 && g.m * g.batch >= 16384;
+}
+
+string gen_matmul_rows(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const MatMulDims g = matmul_dims(d);
+    const dsc_view& va = d.inputs[0];
+    const dsc_view& vb = d.inputs[1];
+    const bool rows = d.output_mode == DSC_MATMUL_ROWS;
+    const int64_t batch_stride = rows ? g.n : g.m * g.n, row_stride = rows ? g.batch * g.n : g.n;
+    // Tuning hooks.  Measured on MI355X on the ConvNet's k=72 product (196000 x 2 x 16): one row per thread,
+    // k unrolled by 8 and B through the scalar unit 35 us; B in LDS 40 us; two / four rows per thread 41 / 46 us.
+    int R = 1;  // rows per thread
+    if (const char* e = std::getenv("DSC_ROWS_R")) R = std::max(1, std::min(8, std::atoi(e)));
+    int unroll = g.k <= 16 ? (int)g.k : 8;
+    if (const char* e = std::getenv("DSC_ROWS_UNROLL")) unroll = std::max(1, std::atoi(e));
+    const int64_t blocks_per_batch = (g.m + 256 * R - 1) / (256 * R);
+    bool b_in_lds = false;
+    if (const char* e = std::getenv("DSC_ROWS_B")) b_in_lds = e[0] == 'l';
+    const int n_out = fk.has_epilogue ? fk.epilogue.raw().n_outputs : 1;
+
+    const string la = em.load_view(fk.inputs[0], va, {"cb", "cm", "ck"});
+    em.funcs << "DSC_INLINE float load_a(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return " << la << ";\n}\n";
+    const string lb = em.load_view(fk.inputs[1], vb, {"cb", "ck", "cn"});
+    em.funcs << "DSC_INLINE float load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb << ";\n}\n";
+    if (fk.has_epilogue) {
+        const dsc_kernel_desc& pe = fk.epilogue.raw();
+        std::ostringstream body;
+        std::map<int, string> ov;
+        ov[fk.epilogue_product_input] = "product";
+        em.emit_pe(body, pe, fk.epilogue_inputs, "gid", "e", ov);
+        for (int o = 0; o < pe.n_outputs; ++o) body << "    result[" << o << "] = et" << pe.outputs[o] << ";\n";
+        em.funcs << "DSC_INLINE void mm_epilogue(float product, int gid, float* result, " << em.params_decl() << ") {\n"
+                 << body.str() << "}\n";
+    }
+
+    // 16-byte stores when four consecutive columns are four consecutive, aligned words
+    const bool vec_store = g.n % 4 == 0 && batch_stride % 4 == 0 && row_stride % 4 == 0;
+    std::ostringstream k;
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
+    k << "    const uint rand_seed = *seed_cell;\n";
+    k << "    const int cb = blockIdx.x / " << S(blocks_per_batch) << ";\n";
+    k << "    const int row0 = (blockIdx.x % " << S(blocks_per_batch) << ") * " << S(256 * R) << " + threadIdx.x;\n";
+    if (b_in_lds) {
+        k << "    __shared__ __attribute__((aligned(16))) float sB[" << S(g.k * g.n) << "];\n";
+        k << "    for (int i = threadIdx.x; i < " << S(g.k * g.n) << "; i += 256) sB[i] = load_b(cb, i / " << S(g.n) << ", i % " << S(g.n)
+          << ", " << em.params_pass() << ");\n";
+        k << "    __syncthreads();\n";
+    }
+    // rows past the end repeat the last row's loads (no divergent loads) and skip the store
+    k << "    int cml[" << R << "];\n";
+    k << "#pragma unroll\n    for (int r = 0; r < " << R << "; ++r) cml[r] = min(row0 + r * 256, " << S(g.m - 1) << ");\n";
+    // R rows per thread (256 apart, so lanes stay on consecutive rows): each B word feeds R FMAs
+    k << "    float acc[" << R << "][" << S(g.n) << "];\n";
+    k << "#pragma unroll\n    for (int r = 0; r < " << R << "; ++r)\n#pragma unroll\n        for (int n = 0; n < " << S(g.n) << "; ++n) acc[r][n] = 0.f;\n";
+    k << "#pragma unroll " << unroll << "\n    for (int ck = 0; ck < " << S(g.k) << "; ++ck) {\n";
+    k << "        float a[" << R << "];\n";
+    k << "#pragma unroll\n        for (int r = 0; r < " << R << "; ++r) a[r] = load_a(cb, cml[r], ck, " << em.params_pass() << ");\n";
+    k << "#pragma unroll\n        for (int n = 0; n < " << S(g.n) << "; ++n) {\n";
+    if (b_in_lds)
+        k << "            const float bv = sB[ck * " << S(g.n) << " + n];\n";
+    else  // the address is the same for every lane: the compiler reads B through the scalar unit into SGPRs
+        k << "            const float bv = load_b(cb, ck, n, " << em.params_pass() << ");\n";
+    k << "#pragma unroll\n            for (int r = 0; r < " << R << "; ++r) acc[r][n] = fmaf(a[r], bv, acc[r][n]);\n        }\n";
+    k << "    }\n";
+    k << "#pragma unroll\n    for (int r = 0; r < " << R << "; ++r) {\n";
+    k << "    const int cm = row0 + r * 256;\n    if (cm < " << S(g.m) << ") {\n";
+    k << "    const int c_row = cb * " << S(batch_stride) << " + cm * " << S(row_stride) << ";\n";
+    if (vec_store) {
+        k << "#pragma unroll\n    for (int n = 0; n < " << S(g.n) << "; n += 4) {\n";
+        if (fk.has_epilogue) {
+            k << "        float res[4][" << n_out << "];\n";
+            k << "#pragma unroll\n        for (int j = 0; j < 4; ++j) mm_epilogue(acc[r][n + j], c_row + n + j, res[j], " << em.params_pass() << ");\n";
+            for (int o = 0; o < n_out; ++o)
+                k << "        *(float4*)(b" << fk.outputs[o] << " + c_row + n) = make_float4(res[0][" << o << "], res[1][" << o << "], res[2][" << o
+                  << "], res[3][" << o << "]);\n";
+        } else {
+            k << "        *(float4*)(b" << fk.outputs[0] << " + c_row + n) = make_float4(acc[r][n], acc[r][n + 1], acc[r][n + 2], acc[r][n + 3]);\n";
+        }
+        k << "    }\n";
+    } else {
+        k << "#pragma unroll\n    for (int n = 0; n < " << S(g.n) << "; ++n) {\n";
+        if (fk.has_epilogue) {
+            k << "        float res[" << n_out << "];\n        mm_epilogue(acc[r][n], c_row + n, res, " << em.params_pass() << ");\n";
+            for (int o = 0; o < n_out; ++o) k << "        b" << fk.outputs[o] << "[c_row + n] = res[" << o << "];\n";
+        } else {
+            k << "        b" << fk.outputs[0] << "[c_row + n] = acc[r][n];\n";
+        }
+        k << "    }\n";
+    }
+    k << "    }\n    }\n}\n";
+    out->grid = (unsigned)(blocks_per_batch * g.batch);
+    out->block = 256;
+    out->source = k.str();
+    out->note = string("row-per-thread fma, B ") + (b_in_lds ? "in LDS" : "in SGPRs") + (fk.has_epilogue ? " +epilogue" : "");
+    return "";
+}
+
 string gen_matmul(Emitter& em, Generated* out) {
     const FusedKernel& fk = em.fk;
     const dsc_kernel_desc& d = fk.main.raw();
@@ -749,6 +862,7 @@ string gen_matmul(Emitter& em, Generated* out) {
     const dsc_view& va = d.inputs[0];
     const dsc_view& vb = d.inputs[1];
     const bool rows = d.output_mode == DSC_MATMUL_ROWS;
+    if (rows_kernel_applies(fk, g)) return gen_matmul_rows(em, out);
     MmConfig c = pick_config(g.m, g.n, g.batch * ((!fk.sum_chunks && g.chunks > 1) ? g.chunks : 1));
 
     // k chunking: the reference writes `chunks` partial products of chunk_tiles*16 k each (kernel.rs:436)
@@ -876,6 +990,9 @@ std::string FusedKernel::key() const {
     s.append(reinterpret_cast<const char*>(&n_buffers), 4);
     if (const char* env = std::getenv("DSC_MM_TILE"))
         if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|T") + env;
+    for (const char* name : {"DSC_MM_ROWS", "DSC_ROWS_R", "DSC_ROWS_UNROLL"})
+        if (const char* env = std::getenv(name))
+            if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|") + name + env;
     return s;
 }
 
