@@ -47,9 +47,13 @@ def time_graph(env, graph, steps: int, warmup: int, seed0: int = 1, profile: boo
     return wall
 
 
+EVENT_PASS = True  # --no-events: skip the second, per-launch-event pass (for runs under an external profiler)
+
+
 def time_then_profile(env, graph, steps: int, warmup: int):
     wall = time_graph(env, graph, steps, warmup, profile=False)
-    time_graph(env, graph, steps, 0, seed0=1000, profile=True)
+    if EVENT_PASS:
+        time_graph(env, graph, steps, 0, seed0=1000, profile=True)
     return wall
 
 
@@ -193,7 +197,14 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only the streaming c=a*2+b kernel over 2^26 elements (counter calibration)")
     ap.add_argument("--cpu-rows", type=int, default=256)
+    ap.add_argument("--workload", default="headline",
+                    choices=["headline", "convnet", "relu-pe", "siren", "hash-grid"],
+                    help="headline: the 8192^3 matmul line with the ConvNet step rate beside it (default); "
+                         "the others run one workload alone, e.g. under rocprofv3")
+    ap.add_argument("--no-events", action="store_true", help="no per-launch HIP events (wall time only)")
     args = ap.parse_args()
+    global EVENT_PASS
+    EVENT_PASS = not args.no_events
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; run with --gpus 1 (nothing here uses a second device)", file=sys.stderr)
         sys.exit(2)
@@ -204,6 +215,20 @@ def main():
     env = Environment(HipBackend())
     if args.copy_calibration:
         print(json.dumps(bench_elementwise(env, 1 << 26, args.steps, args.warmup)))
+        return
+    if args.workload != "headline":
+        from descent_amd import workloads as _w
+
+        if args.workload == "convnet":
+            out = bench_convnet(env, args.steps, args.warmup)
+            sys.stderr.write(out.pop("report"))
+        else:
+            build = {"relu-pe": lambda e: _w.coordinate_mlp(e), "siren": lambda e: _w.coordinate_mlp(e, variant="siren"),
+                     "hash-grid": lambda e: _w.hash_grid_fit(e)}[args.workload]
+            out, rep = bench_workload(env, build, args.steps, args.warmup, topn=int(os.environ.get("DSC_BENCH_TOPN", "12")))
+            sys.stderr.write(rep)
+        out["workload"] = args.workload
+        print(json.dumps(out))
         return
     n = args.size
     head = bench_matmul(env, n, n, n, args.steps, args.warmup)
@@ -231,9 +256,10 @@ def main():
         sys.stderr.write("cfg5 hash grid:\n" + rep)
         hg["scatter_atomics_per_s"] = 16 * 4 * 2 * (1 << 18) / (hg["scatteradd_us_per_step"] * 1e-6) if hg["scatteradd_us_per_step"] else None
         extra["hash_grid_2p18"] = hg
-        conv = bench_convnet(env, max(args.steps, 20), args.warmup)
-        sys.stderr.write(conv.pop("report"))
-        extra["convnet_bs1000"] = conv
+    # the other half of the headline metric: ConvNet (batch 1000) train steps per second
+    conv = bench_convnet(env, max(args.steps, 20), args.warmup)
+    sys.stderr.write(conv.pop("report"))
+    extra["convnet_bs1000"] = conv
 
     cpu = None
     if not args.no_cpu_baseline:

@@ -357,18 +357,28 @@ struct Emitter {
 };
 
 bool rows_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
+bool tallk_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
 
+// Entry points carry the kernel kind and its size, so that a profiler's per-name statistics tell the kernels of
+// a schedule apart: dsc_matmul_mfma_epilogue_b1_m8192_n8192_k8192, dsc_reduce_k4084_n144, dsc_per_element_n12544000.
 string entry_name(const FusedKernel& fk) {
-    switch (fk.main.raw().kind) {
-    case DSC_KERNEL_FILL: return "dsc_fill";
-    case DSC_KERNEL_PER_ELEMENT: return "dsc_per_element";
-    case DSC_KERNEL_REDUCE: return "dsc_reduce";
-    case DSC_KERNEL_MATMUL:
-        if (rows_kernel_applies(fk, matmul_dims(fk.main.raw()))) return fk.has_epilogue ? "dsc_matmul_rows_epilogue" : "dsc_matmul_rows";
-        return fk.has_epilogue ? "dsc_matmul_mfma_epilogue" : "dsc_matmul_mfma";
-    case DSC_KERNEL_UNPAD: return "dsc_unpad";
-    case DSC_KERNEL_WINDOWS_TO_IMAGE: return "dsc_windows_to_image";
-    case DSC_KERNEL_SCATTER_ADD: return "dsc_scatter_add";
+    const dsc_kernel_desc& d = fk.main.raw();
+    auto count = [](int64_t v) { return to_string((long long)v); };
+    switch (d.kind) {
+    case DSC_KERNEL_FILL: return "dsc_fill_n" + count(d.shape.dims[0]);
+    case DSC_KERNEL_PER_ELEMENT: return "dsc_per_element_n" + count(d.shape.dims[0]);
+    case DSC_KERNEL_REDUCE: {
+        return "dsc_reduce_k" + count(d.inputs[0].out_shape.dims[d.axis]) + "_n" + count(element_count(d.shape));
+    }
+    case DSC_KERNEL_MATMUL: {
+        const MatMulDims g = matmul_dims(d);
+        string base = rows_kernel_applies(fk, g) ? "dsc_matmul_rows" : (tallk_kernel_applies(fk, g) ? "dsc_matmul_tallk" : "dsc_matmul_mfma");
+        if (fk.has_epilogue) base += "_epilogue";
+        return base + "_b" + count(g.batch) + "_m" + count(g.m) + "_n" + count(g.n) + "_k" + count(g.k);
+    }
+    case DSC_KERNEL_UNPAD: return "dsc_unpad_n" + count(element_count(d.shape));
+    case DSC_KERNEL_WINDOWS_TO_IMAGE: return "dsc_windows_to_image_n" + count(element_count(d.shape));
+    case DSC_KERNEL_SCATTER_ADD: return "dsc_scatter_add_n" + count(element_count(d.inputs[0].out_shape));
     default: return "dsc_kernel";
     }
 }
@@ -619,10 +629,14 @@ string gen_unpad(Emitter& em, Generated* out) {
     k << "    const int in_c = " << oc << " + " << d.pad << ";\n";
     k << "    const int k_min = in_c - ((" << oc << " == 0) ? " << d.pad << " : 0);\n";
     k << "    const int k_max = in_c + ((" << oc << " == " << S(d.shape.dims[d.axis] - 1) << ") ? " << d.pad << " : 0);\n";
-    k << "    float sum = 0.f;\n    for (int kk = k_min; kk <= k_max; ++kk) {\n";
+    // the candidates in_c - pad .. in_c + pad are all loaded (clamped into [k_min, k_max]) and the ones outside
+    // that range add zero: no loop with a data-dependent trip count, every load in flight at once
+    k << "    float sum = 0.f;\n#pragma unroll\n    for (int j = " << -d.pad << "; j <= " << d.pad << "; ++j) {\n";
+    k << "        const int kk = in_c + j;\n        const int kc = clampi(kk, k_min, k_max);\n";
     auto ic = c;
-    ic[d.axis] = "kk";
-    k << "        sum += " << em.load_view(fk.inputs[0], v, ic) << ";\n    }\n";
+    ic[d.axis] = "kc";
+    k << "        const float w = " << em.load_view(fk.inputs[0], v, ic) << ";\n";
+    k << "        sum += (kk >= k_min && kk <= k_max) ? w : 0.f;\n    }\n";
     k << "    b" << fk.outputs[0] << "[gid] = sum;\n}\n";
     out->grid = blocks_for(n, 256);
     out->block = 256;
@@ -654,13 +668,18 @@ string gen_windows_to_image(Emitter& em, Generated* out) {
     k << "#pragma unroll\n    for (int ix = 0; ix < " << S((fw + sw - 1) / sw) << "; ++ix) {\n";
     k << "        const int fx = fbx + " << S(sw) << " * ix, fy = fby + " << S(sh) << " * iy;\n";
     k << "        const int ox = oxb - ix, oy = oyb - iy;\n";
-    // the window must exist: the reference omits the ox/oy test (kernel.rs:775-776); the true adjoint needs it
-    k << "        if (fx < " << S(fw) << " && fy < " << S(fh) << " && ox >= 0 && ox < " << S(out_w) << " && oy >= 0 && oy < "
-      << S(out_h) << ") {\n";
+    // the window must exist: the reference omits the ox/oy test (kernel.rs:775-776); the true adjoint needs it.
+    // Taps without a window load a valid element instead and add zero, so that the loads of all taps are
+    // independent of the tests and in flight together.
+    k << "        const bool ok = fx < " << S(fw) << " && fy < " << S(fh) << " && ox >= 0 && ox < " << S(out_w) << " && oy >= 0 && oy < "
+      << S(out_h) << ";\n";
+    k << "        const int fxc = min(fx, " << S(fw - 1) << "), fyc = min(fy, " << S(fh - 1) << "), oxc = clampi(ox, 0, " << S(out_w - 1)
+      << "), oyc = clampi(oy, 0, " << S(out_h - 1) << ");\n";
     std::vector<string> ic(r);
     for (int i = 0; i < bd; ++i) ic[i] = c[i];
-    ic[bd] = "oy"; ic[bd + 1] = "ox"; ic[bd + 2] = "group_index"; ic[bd + 3] = "fy"; ic[bd + 4] = "fx"; ic[bd + 5] = "group_c";
-    k << "            tmp += " << em.load_view(fk.inputs[0], v, ic) << ";\n        }\n    }\n";
+    ic[bd] = "oyc"; ic[bd + 1] = "oxc"; ic[bd + 2] = "group_index"; ic[bd + 3] = "fyc"; ic[bd + 4] = "fxc"; ic[bd + 5] = "group_c";
+    k << "        const float w = " << em.load_view(fk.inputs[0], v, ic) << ";\n";
+    k << "        tmp += ok ? w : 0.f;\n    }\n";
     k << "    b" << fk.outputs[0] << "[gid] = tmp;\n}\n";
     out->grid = blocks_for(n, 256);
     out->block = 256;
@@ -855,6 +874,106 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
     return "";
 }
 
+// k range of one chunk of a MatMul descriptor: the reference writes `chunks` partial products of
+// chunk_tiles * 16 k each (src/kernel.rs:436)
+int64_t chunk_k_of(const MatMulDims& g) {
+    const int64_t k_tiles = (g.k + 15) / 16;
+    return ((k_tiles + g.chunks - 1) / g.chunks) * 16;
+}
+
+// Tall-k matmul: a small output (at most 16 tiles of 16x16) summed over a very long k that is already split
+// into many chunks -- the weight gradients of the convolutions (72x16 and 9x16 outputs, k = batch * pixels)
+// and of narrow dense layers.  There is nothing to reuse between workgroups, so the operands skip LDS: every
+// wave takes its own k steps, loads the 16x4 / 4x16 MFMA fragments straight from memory (several steps in
+// flight) and keeps the whole output in accumulators; the four waves of a workgroup are summed through LDS at
+// the end.  One workgroup per (chunk, batch).
+bool tallk_shape_impl(const MatMulDims& g) {
+    if (const char* e = std::getenv("DSC_MM_TALLK"))
+        if (e[0] == '0') return false;
+    const int64_t tiles = ((g.m + 15) / 16) * ((g.n + 15) / 16);
+    return tiles <= 16 && g.chunks > 1 && chunk_k_of(g) >= 128 && g.batch * g.chunks >= 128;
+}
+
+bool tallk_kernel_applies(const FusedKernel& fk, const MatMulDims& g) {
+    return !fk.has_epilogue && !fk.sum_chunks && tallk_shape_impl(g);
+}
+
+string gen_matmul_tallk(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const MatMulDims g = matmul_dims(d);
+    const bool rows = d.output_mode == DSC_MATMUL_ROWS;
+    const int64_t batch_stride = rows ? g.n : g.m * g.n, row_stride = rows ? g.batch * g.n : g.n;
+    const int64_t chunk_k = chunk_k_of(g);
+    const int MT = (int)((g.m + 15) / 16), NT = (int)((g.n + 15) / 16);
+    int U = std::max(1, std::min(8, 24 / (MT + NT)));  // k steps of 4 in flight per wave
+    if (const char* e = std::getenv("DSC_TALLK_UNROLL")) U = std::max(1, std::min(16, std::atoi(e)));
+
+    const string la = em.load_view(fk.inputs[0], d.inputs[0], {"cb", "cm", "ck"});
+    em.funcs << "DSC_INLINE float load_a(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return " << la << ";\n}\n";
+    const string lb = em.load_view(fk.inputs[1], d.inputs[1], {"cb", "ck", "cn"});
+    em.funcs << "DSC_INLINE float load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb << ";\n}\n";
+
+    std::ostringstream k;
+    k << "typedef float tk_float4 __attribute__((ext_vector_type(4)));\n";
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
+    k << "    const uint rand_seed = *seed_cell;\n";
+    k << "    __shared__ float red[4][" << MT * NT * 256 << "];\n";
+    k << "    const int chunk = blockIdx.x % " << S(g.chunks) << ", cb = blockIdx.x / " << S(g.chunks) << ";\n";
+    k << "    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;\n";
+    k << "    const int li = lane & 15, lk = lane >> 4;\n";
+    k << "    const int k_begin = chunk * " << S(chunk_k) << ", k_end = min(k_begin + " << S(chunk_k) << ", " << S(g.k) << ");\n";
+    k << "    tk_float4 acc[" << MT << "][" << NT << "];\n";
+    k << "#pragma unroll\n    for (int mt = 0; mt < " << MT << "; ++mt)\n#pragma unroll\n        for (int nt = 0; nt < " << NT
+      << "; ++nt) acc[mt][nt] = (tk_float4){0.f, 0.f, 0.f, 0.f};\n";
+    // A fragment of v_mfma_f32_16x16x4f32: lane l holds A[l % 16][l / 16]; B fragment: B[l / 16][l % 16]
+    k << "    for (int k0 = k_begin + wave * " << 4 * U << "; k0 < k_end; k0 += " << 16 * U << ") {\n";
+    k << "        float fa[" << U << "][" << MT << "], fb[" << U << "][" << NT << "];\n";
+    // out-of-range rows, columns and k repeat a valid element's load (no divergent loads) and are zeroed after
+    // the fence below.  Nothing before the fence consumes a loaded value, so every load of the iteration is in
+    // flight before the first wait (left alone, the compiler's schedule waits right after each load).
+    k << "#pragma unroll\n        for (int u = 0; u < " << U << "; ++u) {\n";
+    k << "            const int ckc = min(k0 + 4 * u + lk, " << S(g.k - 1) << ");\n";
+    k << "#pragma unroll\n            for (int mt = 0; mt < " << MT << "; ++mt) fa[u][mt] = load_a(cb, min(mt * 16 + li, " << S(g.m - 1)
+      << "), ckc, " << em.params_pass() << ");\n";
+    k << "#pragma unroll\n            for (int nt = 0; nt < " << NT << "; ++nt) fb[u][nt] = load_b(cb, ckc, min(nt * 16 + li, " << S(g.n - 1)
+      << "), " << em.params_pass() << ");\n";
+    k << "        }\n";
+    k << "        __builtin_amdgcn_sched_barrier(0);\n";
+    k << "#pragma unroll\n        for (int u = 0; u < " << U << "; ++u) {\n";
+    k << "            const bool k_ok = k0 + 4 * u + lk < k_end;\n";
+    k << "#pragma unroll\n            for (int mt = 0; mt < " << MT << "; ++mt) fa[u][mt] = (k_ok && mt * 16 + li < " << S(g.m)
+      << ") ? fa[u][mt] : 0.f;\n";
+    k << "#pragma unroll\n            for (int nt = 0; nt < " << NT << "; ++nt) fb[u][nt] = (k_ok && nt * 16 + li < " << S(g.n)
+      << ") ? fb[u][nt] : 0.f;\n";
+    k << "        }\n";
+    k << "#pragma unroll\n        for (int u = 0; u < " << U << "; ++u)\n#pragma unroll\n            for (int mt = 0; mt < " << MT
+      << "; ++mt)\n#pragma unroll\n                for (int nt = 0; nt < " << NT << "; ++nt)\n"
+      << "                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[u][mt], fb[u][nt], acc[mt][nt], 0, 0, 0);\n";
+    k << "    }\n";
+    k << "#pragma unroll\n    for (int mt = 0; mt < " << MT << "; ++mt)\n#pragma unroll\n        for (int nt = 0; nt < " << NT
+      << "; ++nt)\n#pragma unroll\n            for (int r = 0; r < 4; ++r) red[wave][(mt * " << NT << " + nt) * 256 + r * 64 + lane] = acc[mt][nt][r];\n";
+    k << "    __syncthreads();\n";
+    // accumulator register r of lane l is D[4 * (l / 16) + r][l % 16]
+    k << "    for (int i = threadIdx.x; i < " << MT * NT * 256 << "; i += 256) {\n";
+    k << "        const float sum = (red[0][i] + red[1][i]) + (red[2][i] + red[3][i]);\n";
+    k << "        const int tile = i >> 8, r = (i >> 6) & 3, l = i & 63;\n";
+    k << "        const int cm = (tile / " << NT << ") * 16 + 4 * (l >> 4) + r, cn = (tile % " << NT << ") * 16 + (l & 15);\n";
+    k << "        if (cm < " << S(g.m) << " && cn < " << S(g.n) << ") b" << fk.outputs[0] << "[chunk * " << S(g.batch * g.m * g.n) << " + cb * "
+      << S(batch_stride) << " + cm * " << S(row_stride) << " + cn] = sum;\n";
+    k << "    }\n}\n";
+    const int64_t grid = g.batch * g.chunks;
+    if (grid >= kMaxIndex) return "matmul: grid too large";
+    out->grid = (unsigned)grid;
+    out->block = 256;
+    out->source = k.str();
+    char note[160];
+    std::snprintf(note, sizeof note, "tall-k mfma 16x16x4, %dx%d tiles, operands from memory, %d steps in flight, chunks %lld", MT, NT, U,
+                  (long long)g.chunks);
+    out->note = note;
+    return "";
+}
+
 string gen_matmul(Emitter& em, Generated* out) {
     const FusedKernel& fk = em.fk;
     const dsc_kernel_desc& d = fk.main.raw();
@@ -863,6 +982,7 @@ string gen_matmul(Emitter& em, Generated* out) {
     const dsc_view& vb = d.inputs[1];
     const bool rows = d.output_mode == DSC_MATMUL_ROWS;
     if (rows_kernel_applies(fk, g)) return gen_matmul_rows(em, out);
+    if (tallk_kernel_applies(fk, g)) return gen_matmul_tallk(em, out);
     MmConfig c = pick_config(g.m, g.n, g.batch * ((!fk.sum_chunks && g.chunks > 1) ? g.chunks : 1));
 
     // k chunking: the reference writes `chunks` partial products of chunk_tiles*16 k each (kernel.rs:436)
@@ -948,6 +1068,8 @@ string gen_matmul(Emitter& em, Generated* out) {
 
 }  // namespace
 
+bool tallk_shape(const MatMulDims& g) { return tallk_shape_impl(g); }
+
 FusedKernel FusedKernel::plain(const dsc_kernel_desc& d) {
     FusedKernel fk;
     fk.main = KernelDesc(d);
@@ -990,7 +1112,7 @@ std::string FusedKernel::key() const {
     s.append(reinterpret_cast<const char*>(&n_buffers), 4);
     if (const char* env = std::getenv("DSC_MM_TILE"))
         if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|T") + env;
-    for (const char* name : {"DSC_MM_ROWS", "DSC_ROWS_R", "DSC_ROWS_UNROLL"})
+    for (const char* name : {"DSC_MM_ROWS", "DSC_ROWS_R", "DSC_ROWS_UNROLL", "DSC_ROWS_B", "DSC_MM_TALLK", "DSC_TALLK_UNROLL"})
         if (const char* env = std::getenv(name))
             if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|") + name + env;
     return s;

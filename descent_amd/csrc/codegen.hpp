@@ -61,6 +61,10 @@ struct Generated {
 // Returns "" on success or an error message.
 std::string generate(const FusedKernel& k, Generated* out);
 
+// Whether a MatMul of these dimensions (already split into its chunks) runs on the tall-k kernel: a small output
+// summed over a long k, one workgroup per (chunk, batch).  The schedule sizes its k re-split for that kernel.
+bool tallk_shape(const MatMulDims& g);
+
 // hipRTC options every kernel is compiled with (after --offload-arch=<arch>).
 const std::vector<std::string>& compile_options();
 

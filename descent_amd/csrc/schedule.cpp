@@ -215,6 +215,13 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             const int64_t t64 = ((g.m + 63) / 64) * ((g.n + 63) / 64) * g.batch;
             static const int64_t split_target = std::getenv("DSC_SPLIT_TARGET") ? std::atoll(std::getenv("DSC_SPLIT_TARGET")) : 4096;
             int64_t S = std::min<int64_t>(split_target / t64, g.k / 64);
+            {
+                // a small output over a long k runs on the tall-k kernel, one workgroup of four waves per
+                // (chunk, batch): a thousand workgroups with at least 256 k each
+                MatMulDims t = g;
+                t.chunks = std::min<int64_t>(std::max<int64_t>(1024 / g.batch, 1), g.k / 256);
+                if (t.chunks >= 2 && tallk_shape(t)) S = t.chunks;
+            }
             if (S < 2) continue;
             const int64_t ktiles = (g.k + 15) / 16;
             const int64_t chunk_tiles = (ktiles + S - 1) / S;

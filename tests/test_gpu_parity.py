@@ -33,6 +33,8 @@ def test_reference_known_answers(hip_backend_session, mode):
 MATMUL_SHAPES = [
     (1, 1, 1), (16, 16, 16), (33, 17, 9), (128, 128, 128), (100, 10, 784), (1000, 128, 784), (257, 130, 1030),
     (64, 300, 2100), (9, 16, 5000),
+    # small outputs over a long k: the tall-k kernel (ragged tiles, one tile, many tiles)
+    (9, 16, 50000), (72, 16, 70000), (33, 50, 140000), (250, 3, 66000),
 ]
 
 
@@ -64,7 +66,7 @@ def _transposed_case(env, rng, m, n, k, ta, tb):
 
 
 @pytest.mark.parametrize("ta,tb", [(False, True), (True, False), (True, True)])
-@pytest.mark.parametrize("m,n,k", [(128, 64, 256), (100, 36, 77), (72, 16, 3000)])
+@pytest.mark.parametrize("m,n,k", [(128, 64, 256), (100, 36, 77), (72, 16, 3000), (72, 16, 40000)])
 def test_matmul_transposed_operands(hip_backend_session, ta, tb, m, n, k):
     genv, cenv = _envs(hip_backend_session)
     got = _transposed_case(genv, np.random.default_rng(5), m, n, k, ta, tb)
