@@ -82,7 +82,7 @@ def _kernels_of_each_kind():
 @pytest.mark.parametrize("kernel", _kernels_of_each_kind(), ids=lambda k: type(k).__name__)
 def test_generated_source_compiles_for_gfx950(kernel):
     src = hip_backend.codegen_source(kernel)
-    assert 'extern "C" __global__' in src and re.search(r"void (dsc_[a-z_]+|MM_ENTRY)\(", src)
+    assert 'extern "C" __global__' in src and re.search(r"void (dsc_[a-z_0-9]+|MM_ENTRY)\(", src)
     assert hip_backend.codegen_compile(kernel, "gfx950") > 0
     if isinstance(kernel, K.MatMulKernel):
         assert "__builtin_amdgcn_mfma_f32_32x32x2f32" in src
