@@ -509,22 +509,39 @@ string gen_reduce(Emitter& em, Generated* out) {
 
     std::ostringstream k;
     k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = *seed_cell;\n";
-    // The k loop is unrolled four times over independent accumulators so that four loads are in flight per
-    // thread; `first`/`step` give the thread's k sequence.
+    // The k loop runs over groups of U independent accumulators: the U loads of a group are issued before any of
+    // them is used, with no bounds test in between (a test per load would be a branch per load, and the loads
+    // would be issued one at a time).  What is left over is handled by groups of U/2, U/4, .. 1.
+    // `first`/`step` give the thread's k sequence.
+    auto pick_unroll = [&](int64_t step, int64_t max_u) {
+        int64_t u = max_u;
+        while (u > 1 && u * step > K) u /= 2;
+        return (int)u;
+    };
     auto emit_k_loop = [&](const std::vector<string>& oc, const string& first, int64_t step) {
-        k << "    float acc0 = " << init << ", acc1 = " << init << ", acc2 = " << init << ", acc3 = " << init << ";\n";
-        k << "    for (int kb = " << first << "; kb < " << S(K) << "; kb += " << S(4 * step) << ") {\n";
-        for (int u = 0; u < 4; ++u) {
-            const string kk = "kk" + to_string(u);
-            k << "        const int " << kk << " = kb + " << S(u * step) << ";\n";
-            auto ic = oc;
-            ic[d.axis] = kk;
-            const string ld = em.load_view(fk.inputs[0], v, ic);
-            k << "        if (" << kk << " < " << S(K) << ") { const float x = " << ld << "; acc" << u << " = "
-              << combine("acc" + to_string(u), "x") << "; }\n";
+        const int U = pick_unroll(step, 8);
+        for (int u = 0; u < U; ++u) k << (u ? ", acc" : "    float acc") << u << " = " << init;
+        k << ";\n    int kb = " << first << ";\n";
+        for (int lvl = U; lvl >= 1; lvl /= 2) {
+            const string cond = "kb + " + S((lvl - 1) * step) + " < " + S(K);
+            k << (lvl == U ? "    for (; " + cond + "; kb += " + S(lvl * step) + ") {\n" : "    if (" + cond + ") {\n");
+            for (int u = 0; u < lvl; ++u) {
+                auto ic = oc;
+                ic[d.axis] = "(kb + " + S(u * step) + ")";
+                k << "        const float x" << u << " = " << em.load_view(fk.inputs[0], v, ic) << ";\n";
+            }
+            for (int u = 0; u < lvl; ++u) k << "        acc" << u << " = " << combine("acc" + to_string(u), "x" + to_string(u)) << ";\n";
+            if (lvl != U) k << "        kb += " << S(lvl * step) << ";\n";
+            k << "    }\n";
         }
-        k << "    }\n";
-        k << "    float acc = " << combine(combine("acc0", "acc1"), combine("acc2", "acc3")) << ";\n";
+        std::vector<string> terms;
+        for (int u = 0; u < U; ++u) terms.push_back("acc" + to_string(u));
+        while (terms.size() > 1) {
+            std::vector<string> next;
+            for (size_t i = 0; i + 1 < terms.size(); i += 2) next.push_back("(" + combine(terms[i], terms[i + 1]) + ")");
+            terms = next;
+        }
+        k << "    float acc = " << terms[0] << ";\n";
     };
     if (k_fastest) {
         // lanes of a group walk k; groups of G lanes own one output; butterfly over the group
@@ -556,22 +573,37 @@ string gen_reduce(Emitter& em, Generated* out) {
         k << "    if (vid < " << S(n_vec) << "u) {\n";
         k << "    const uint oid = vid * 4u;\n";
         auto oc = em.emit_coords(k, d.shape, "oid", "oc");
-        k << "    float4 a0 = result, a1 = result, a2 = result, a3 = result;\n";
-        k << "    for (int kb = tk; kb < " << S(K) << "; kb += " << S(4 * TK) << ") {\n";
-        for (int u = 0; u < 4; ++u) {
-            const string kk = "kk" + to_string(u);
-            k << "        const int " << kk << " = kb + " << S(u * TK) << ";\n";
-            auto ic = oc;
-            ic[d.axis] = kk;
-            k << "        if (" << kk << " < " << S(K) << ") { const float4 x = *(const float4*)(b" << fk.inputs[0].buffer << " + "
-              << em.index_expr(v, ic) << ");";
-            const string a = "a" + to_string(u);
-            for (const char* c : {"x", "y", "z", "w"}) k << " " << a << "." << c << " = " << combine(a + "." + c, string("x.") + c) << ";";
-            k << " }\n";
+        const int U = pick_unroll(TK, 4);
+        const char* comps[4] = {"x", "y", "z", "w"};
+        for (int u = 0; u < U; ++u) k << (u ? ", a" : "    float4 a") << u << " = result";
+        k << ";\n    int kb = " << (TK > 1 ? "tk" : "0") << ";\n";
+        for (int lvl = U; lvl >= 1; lvl /= 2) {
+            const string cond = "kb + " + S((lvl - 1) * TK) + " < " + S(K);
+            k << (lvl == U ? "    for (; " + cond + "; kb += " + S(lvl * TK) + ") {\n" : "    if (" + cond + ") {\n");
+            for (int u = 0; u < lvl; ++u) {
+                auto ic = oc;
+                ic[d.axis] = "(kb + " + S(u * TK) + ")";
+                k << "        const float4 x" << u << " = *(const float4*)(b" << fk.inputs[0].buffer << " + " << em.index_expr(v, ic) << ");\n";
+            }
+            for (int u = 0; u < lvl; ++u) {
+                const string a = "a" + to_string(u), x = "x" + to_string(u);
+                k << "       ";
+                for (const char* c : comps) k << " " << a << "." << c << " = " << combine(a + "." + c, x + "." + c) << ";";
+                k << "\n";
+            }
+            if (lvl != U) k << "        kb += " << S(lvl * TK) << ";\n";
+            k << "    }\n";
         }
-        k << "    }\n";
-        for (const char* c : {"x", "y", "z", "w"})
-            k << "    result." << c << " = " << combine(combine(string("a0.") + c, string("a1.") + c), combine(string("a2.") + c, string("a3.") + c)) << ";\n";
+        for (const char* c : comps) {
+            std::vector<string> terms;
+            for (int u = 0; u < U; ++u) terms.push_back("a" + to_string(u) + "." + c);
+            while (terms.size() > 1) {
+                std::vector<string> next;
+                for (size_t i = 0; i + 1 < terms.size(); i += 2) next.push_back("(" + combine(terms[i], terms[i + 1]) + ")");
+                terms = next;
+            }
+            k << "    result." << c << " = " << terms[0] << ";\n";
+        }
         k << "    }\n";
         if (TK > 1) {
             k << "    red[threadIdx.x] = result;\n    __syncthreads();\n";
@@ -598,7 +630,7 @@ string gen_reduce(Emitter& em, Generated* out) {
         k << "    float result = " << init << ";\n";
         k << "    if (oid < " << S(n_out) << "u) {\n";
         auto oc = em.emit_coords(k, d.shape, "oid", "oc");
-        emit_k_loop(oc, "tk", TK);
+        emit_k_loop(oc, TK > 1 ? "tk" : "0", TK);
         k << "    result = acc;\n    }\n";
         if (TK > 1) {
             k << "    red[threadIdx.x] = result;\n    __syncthreads();\n";
