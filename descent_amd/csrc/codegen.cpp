@@ -519,19 +519,22 @@ string gen_reduce(Emitter& em, Generated* out) {
         return (int)u;
     };
     auto emit_k_loop = [&](const std::vector<string>& oc, const string& first, int64_t step) {
-        const int U = pick_unroll(step, 8);
+        // a fused producer is code, not a load: fewer copies of it (groups of 4, then single steps)
+        const bool heavy = fk.inputs[0].virt >= 0;
+        const int U = pick_unroll(step, heavy ? 4 : 8);
         for (int u = 0; u < U; ++u) k << (u ? ", acc" : "    float acc") << u << " = " << init;
         k << ";\n    int kb = " << first << ";\n";
-        for (int lvl = U; lvl >= 1; lvl /= 2) {
+        for (int lvl = U; lvl >= 1; lvl = (heavy && lvl > 1) ? 1 : lvl / 2) {
             const string cond = "kb + " + S((lvl - 1) * step) + " < " + S(K);
-            k << (lvl == U ? "    for (; " + cond + "; kb += " + S(lvl * step) + ") {\n" : "    if (" + cond + ") {\n");
+            const bool loop = lvl == U || heavy;
+            k << (loop ? "    for (; " + cond + "; kb += " + S(lvl * step) + ") {\n" : "    if (" + cond + ") {\n");
             for (int u = 0; u < lvl; ++u) {
                 auto ic = oc;
                 ic[d.axis] = "(kb + " + S(u * step) + ")";
                 k << "        const float x" << u << " = " << em.load_view(fk.inputs[0], v, ic) << ";\n";
             }
             for (int u = 0; u < lvl; ++u) k << "        acc" << u << " = " << combine("acc" + to_string(u), "x" + to_string(u)) << ";\n";
-            if (lvl != U) k << "        kb += " << S(lvl * step) << ";\n";
+            if (!loop) k << "        kb += " << S(lvl * step) << ";\n";
             k << "    }\n";
         }
         std::vector<string> terms;
@@ -873,6 +876,39 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
         k << "            const float bv = load_b(cb, ck, n, " << em.params_pass() << ");\n";
     k << "#pragma unroll\n            for (int r = 0; r < " << R << "; ++r) acc[r][n] = fmaf(a[r], bv, acc[r][n]);\n        }\n";
     k << "    }\n";
+    const int Q = (int)(g.n / 4);  // 16-byte pieces per row
+    const bool transposed_store = vec_store && (Q == 1 || Q == 2 || Q == 4 || Q == 8) && !std::getenv("DSC_ROWS_DIRECT_STORE");
+    if (transposed_store) {
+        // A thread holds one whole row, so storing it directly makes every lane of a store instruction write 16
+        // bytes of a different row (N*4 bytes apart).  Instead each wave passes its 64 rows through LDS and reads
+        // them back so that Q consecutive lanes hold one row: a store instruction then writes 1 KiB of
+        // consecutive memory, and the epilogue's own loads are consecutive too.
+        const int pitch = (int)g.n + 4;
+        k << "    __shared__ __attribute__((aligned(16))) float tr[4][" << 64 * pitch << "];\n";
+        k << "    float* my = tr[threadIdx.x >> 6];\n    const int lane = threadIdx.x & 63;\n";
+        k << "    const int wave_row0 = row0 - lane;\n";
+        k << "#pragma unroll\n    for (int r = 0; r < " << R << "; ++r) {\n";
+        if (R > 1) k << "        __syncthreads();\n";
+        k << "#pragma unroll\n        for (int n = 0; n < " << S(g.n) << "; n += 4) *(float4*)&my[lane * " << pitch
+          << " + n] = make_float4(acc[r][n], acc[r][n + 1], acc[r][n + 2], acc[r][n + 3]);\n";
+        k << "        __syncthreads();\n";
+        k << "#pragma unroll\n        for (int s = 0; s < " << Q << "; ++s) {\n";
+        k << "            const int rl = s * " << 64 / Q << " + lane / " << Q << ", q = lane % " << Q << ";\n";
+        k << "            const int cm = wave_row0 + r * 256 + rl;\n";
+        k << "            const float4 p = *(const float4*)&my[rl * " << pitch << " + q * 4];\n";
+        k << "            if (cm < " << S(g.m) << ") {\n";
+        k << "                const int c_at = cb * " << S(batch_stride) << " + cm * " << S(row_stride) << " + q * 4;\n";
+        if (fk.has_epilogue) {
+            k << "                const float pv[4] = {p.x, p.y, p.z, p.w};\n                float res[4][" << n_out << "];\n";
+            k << "#pragma unroll\n                for (int j = 0; j < 4; ++j) mm_epilogue(pv[j], c_at + j, res[j], " << em.params_pass() << ");\n";
+            for (int o = 0; o < n_out; ++o)
+                k << "                *(float4*)(b" << fk.outputs[o] << " + c_at) = make_float4(res[0][" << o << "], res[1][" << o << "], res[2][" << o
+                  << "], res[3][" << o << "]);\n";
+        } else {
+            k << "                *(float4*)(b" << fk.outputs[0] << " + c_at) = p;\n";
+        }
+        k << "            }\n        }\n    }\n}\n";
+    } else {
     k << "#pragma unroll\n    for (int r = 0; r < " << R << "; ++r) {\n";
     k << "    const int cm = row0 + r * 256;\n    if (cm < " << S(g.m) << ") {\n";
     k << "    const int c_row = cb * " << S(batch_stride) << " + cm * " << S(row_stride) << ";\n";
@@ -899,6 +935,7 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
         k << "    }\n";
     }
     k << "    }\n    }\n}\n";
+    }
     out->grid = (unsigned)(blocks_per_batch * g.batch);
     out->block = 256;
     out->source = k.str();
@@ -1144,7 +1181,7 @@ std::string FusedKernel::key() const {
     s.append(reinterpret_cast<const char*>(&n_buffers), 4);
     if (const char* env = std::getenv("DSC_MM_TILE"))
         if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|T") + env;
-    for (const char* name : {"DSC_MM_ROWS", "DSC_ROWS_R", "DSC_ROWS_UNROLL", "DSC_ROWS_B", "DSC_MM_TALLK", "DSC_TALLK_UNROLL"})
+    for (const char* name : {"DSC_MM_ROWS", "DSC_ROWS_R", "DSC_ROWS_UNROLL", "DSC_ROWS_B", "DSC_ROWS_DIRECT_STORE", "DSC_MM_TALLK", "DSC_TALLK_UNROLL"})
         if (const char* env = std::getenv(name))
             if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|") + name + env;
     return s;
