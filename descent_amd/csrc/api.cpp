@@ -375,58 +375,94 @@ namespace {
 struct Acc {
     double ms = 0;
     int64_t n = 0;
+    const Kernel* kernel = nullptr;
 };
-int collect(Context* c, std::map<std::string, Acc>* by_label) {
+// Per compiled kernel: labels repeat (every hash-grid level scatters the same shape), kernels do not.
+int collect(Context* c, std::map<const Kernel*, Acc>* by_kernel) {
     HIP_TRY(hipStreamSynchronize(c->stream));
     for (auto& p : c->profile) {
         float ms = 0.f;
         HIP_TRY(hipEventElapsedTime(&ms, p.start, p.stop));
-        Acc& a = (*by_label)[p.kernel->label];
+        Acc& a = (*by_kernel)[p.kernel];
         a.ms += ms;
         a.n += 1;
+        a.kernel = p.kernel;
     }
     return DSC_OK;
 }
+const double kHbmPeakGBs = 8000.0, kMfmaFp32PeakTflops = 157.3;
 }  // namespace
 
 int dsc_prof_report(dsc_ctx* ctx, int top_n, char** out_text) {
     if (!ctx || !out_text) return fail(DSC_ERR_INVALID, "null argument");
-    std::map<std::string, Acc> by_label;
-    int rc = collect(&ctx->c, &by_label);
+    std::map<const Kernel*, Acc> by_kernel;
+    int rc = collect(&ctx->c, &by_kernel);
     if (rc != DSC_OK) return rc;
-    std::vector<std::pair<std::string, Acc>> rows(by_label.begin(), by_label.end());
-    std::sort(rows.begin(), rows.end(), [](auto& a, auto& b) { return a.second.ms > b.second.ms; });
+    std::vector<Acc> rows;
+    for (auto& kv : by_kernel) rows.push_back(kv.second);
+    std::sort(rows.begin(), rows.end(), [](const Acc& a, const Acc& b) { return a.ms > b.ms; });
     double total = 0;
-    for (auto& r : rows) total += r.second.ms;
+    for (auto& r : rows) total += r.ms;
     std::ostringstream o;
-    char line[256];
+    char line[512];
     std::snprintf(line, sizeof line, "total %.3f ms over %zu launches\n", total, ctx->c.profile.size());
     o << line;
     int shown = 0;
     for (auto& r : rows) {
         if (top_n > 0 && shown++ >= top_n) break;
-        std::snprintf(line, sizeof line, "%10.3f ms %8lld x %10.2f us  %s\n", r.second.ms, (long long)r.second.n,
-                      1000.0 * r.second.ms / (double)r.second.n, r.first.c_str());
+        const double us = 1000.0 * r.ms / (double)r.n;
+        const double gbs = r.kernel->gen.algo_bytes / (us * 1e-6) / 1e9;
+        const double tf = r.kernel->gen.algo_flops / (us * 1e-6) / 1e12;
+        // which roof bounds the kernel: the matrix units when it has at least their 20 flop per byte
+        const bool mfma_bound = r.kernel->gen.algo_flops >= 20.0 * r.kernel->gen.algo_bytes;
+        char roof[96];
+        if (mfma_bound) std::snprintf(roof, sizeof roof, "%7.1f TFLOP/s %4.1f%% mfma", tf, 100.0 * tf / kMfmaFp32PeakTflops);
+        else std::snprintf(roof, sizeof roof, "%7.0f GB/s    %4.1f%% hbm ", gbs, 100.0 * gbs / kHbmPeakGBs);
+        std::snprintf(line, sizeof line, "%10.3f ms %8lld x %10.2f us  %s  %s  (%s)\n", r.ms, (long long)r.n, us, roof,
+                      r.kernel->label.c_str(), r.kernel->gen.entry.c_str());
         o << line;
     }
     *out_text = dup_string(o.str());
     return *out_text ? DSC_OK : fail(DSC_ERR_OOM, "host allocation failed");
 }
 
+namespace {
+int sum_prefix(Context* c, const char* prefix, Acc* sum, double* bytes, double* flops) {
+    std::map<const Kernel*, Acc> by_kernel;
+    int rc = collect(c, &by_kernel);
+    if (rc != DSC_OK) return rc;
+    const std::string pre(prefix);
+    for (auto& kv : by_kernel) {
+        if (kv.first->label.compare(0, pre.size(), pre) != 0) continue;
+        sum->ms += kv.second.ms;
+        sum->n += kv.second.n;
+        if (bytes) *bytes += kv.first->gen.algo_bytes * (double)kv.second.n;
+        if (flops) *flops += kv.first->gen.algo_flops * (double)kv.second.n;
+    }
+    return DSC_OK;
+}
+}  // namespace
+
 int dsc_prof_query(dsc_ctx* ctx, const char* prefix, double* out_avg_us, int64_t* out_launches) {
     if (!ctx || !prefix) return fail(DSC_ERR_INVALID, "null argument");
-    std::map<std::string, Acc> by_label;
-    int rc = collect(&ctx->c, &by_label);
-    if (rc != DSC_OK) return rc;
     Acc sum;
-    const std::string pre(prefix);
-    for (auto& kv : by_label) {
-        if (kv.first.compare(0, pre.size(), pre) == 0) {
-            sum.ms += kv.second.ms;
-            sum.n += kv.second.n;
-        }
-    }
+    int rc = sum_prefix(&ctx->c, prefix, &sum, nullptr, nullptr);
+    if (rc != DSC_OK) return rc;
     if (out_avg_us) *out_avg_us = sum.n ? 1000.0 * sum.ms / (double)sum.n : 0.0;
+    if (out_launches) *out_launches = sum.n;
+    return DSC_OK;
+}
+
+int dsc_prof_work(dsc_ctx* ctx, const char* prefix, double* out_total_us, double* out_algo_bytes, double* out_algo_flops,
+                  int64_t* out_launches) {
+    if (!ctx || !prefix) return fail(DSC_ERR_INVALID, "null argument");
+    Acc sum;
+    double bytes = 0, flops = 0;
+    int rc = sum_prefix(&ctx->c, prefix, &sum, &bytes, &flops);
+    if (rc != DSC_OK) return rc;
+    if (out_total_us) *out_total_us = 1000.0 * sum.ms;
+    if (out_algo_bytes) *out_algo_bytes = bytes;
+    if (out_algo_flops) *out_algo_flops = flops;
     if (out_launches) *out_launches = sum.n;
     return DSC_OK;
 }

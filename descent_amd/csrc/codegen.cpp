@@ -364,11 +364,13 @@ bool tallk_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
 string entry_name(const FusedKernel& fk) {
     const dsc_kernel_desc& d = fk.main.raw();
     auto count = [](int64_t v) { return to_string((long long)v); };
+    if (!fk.row_stages.empty()) return "dsc_row_fused_m" + count(fk.row_m) + "_n" + count(fk.row_n) + "_s" + count((int64_t)fk.row_stages.size());
     switch (d.kind) {
     case DSC_KERNEL_FILL: return "dsc_fill_n" + count(d.shape.dims[0]);
     case DSC_KERNEL_PER_ELEMENT: return "dsc_per_element_n" + count(d.shape.dims[0]);
     case DSC_KERNEL_REDUCE: {
-        return "dsc_reduce_k" + count(d.inputs[0].out_shape.dims[d.axis]) + "_n" + count(element_count(d.shape));
+        return string(fk.has_epilogue ? "dsc_reduce_epilogue_k" : "dsc_reduce_k") + count(d.inputs[0].out_shape.dims[d.axis]) + "_n" +
+               count(element_count(d.shape));
     }
     case DSC_KERNEL_MATMUL: {
         const MatMulDims g = matmul_dims(d);
@@ -395,6 +397,10 @@ string check_sizes(const FusedKernel& fk) {
     if (!e.empty()) return e;
     for (auto& v : fk.virtuals) {
         e = chk(v.pe.raw());
+        if (!e.empty()) return e;
+    }
+    for (auto& st : fk.row_stages) {
+        e = chk(st.k.raw());
         if (!e.empty()) return e;
     }
     if (fk.has_epilogue) return chk(fk.epilogue.raw());
@@ -486,6 +492,35 @@ string gen_reduce(Emitter& em, Generated* out) {
     const string init = is_max ? "U2F(0xff800000u)" : "0.f";
     auto combine = [&](const string& a, const string& b) { return is_max ? "glsl_max(" + a + ", " + b + ")" : a + " + " + b; };
 
+    // the store of one result: plain, or through the fused per-element consumer
+    const int n_res = fk.has_epilogue ? fk.epilogue.raw().n_outputs : 1;
+    if (fk.has_epilogue) {
+        const dsc_kernel_desc& pe = fk.epilogue.raw();
+        std::ostringstream body;
+        std::map<int, string> ov;
+        ov[fk.epilogue_product_input] = "product";
+        em.emit_pe(body, pe, fk.epilogue_inputs, "gid", "e", ov);
+        for (int o = 0; o < pe.n_outputs; ++o) body << "    result[" << o << "] = et" << pe.outputs[o] << ";\n";
+        em.funcs << "DSC_INLINE void red_epilogue(float product, int gid, float* result, " << em.params_decl() << ") {\n"
+                 << body.str() << "}\n";
+    }
+    auto store_one = [&](const string& value, const string& oid) {
+        if (!fk.has_epilogue) return "b" + to_string(fk.outputs[0]) + "[" + oid + "] = " + value + ";";
+        string t = "{ float res[" + to_string(n_res) + "]; red_epilogue(" + value + ", (int)(" + oid + "), res, " + em.params_pass() + ");";
+        for (int o = 0; o < n_res; ++o) t += " b" + to_string(fk.outputs[o]) + "[" + oid + "] = res[" + to_string(o) + "];";
+        return t + " }";
+    };
+    auto store_four = [&](const string& value4, const string& oid) {
+        if (!fk.has_epilogue) return "*(float4*)(b" + to_string(fk.outputs[0]) + " + " + oid + ") = " + value4 + ";";
+        string t = "{ const float pv[4] = {" + value4 + ".x, " + value4 + ".y, " + value4 + ".z, " + value4 + ".w}; float res[4][" +
+                   to_string(n_res) + "];\n#pragma unroll\n        for (int j = 0; j < 4; ++j) red_epilogue(pv[j], (int)(" + oid +
+                   ") + j, res[j], " + em.params_pass() + ");";
+        for (int o = 0; o < n_res; ++o)
+            t += " *(float4*)(b" + to_string(fk.outputs[o]) + " + " + oid + ") = make_float4(res[0][" + to_string(o) + "], res[1][" +
+                 to_string(o) + "], res[2][" + to_string(o) + "], res[3][" + to_string(o) + "]);";
+        return t + " }";
+    };
+
     // is the reduced axis the one that walks memory fastest?
     bool k_fastest = false;
     if (fk.inputs[0].buffer >= 0) {
@@ -557,7 +592,7 @@ string gen_reduce(Emitter& em, Generated* out) {
         emit_k_loop(oc, "lk", G);
         for (int64_t off = G / 2; off >= 1; off /= 2)
             k << "    acc = " << combine("acc", "__shfl_xor(acc, " + S(off) + ", 64)") << ";\n";
-        k << "    if (lk == 0) b" << fk.outputs[0] << "[oid] = acc;\n}\n";
+        k << "    if (lk == 0) " << store_one("acc", "oid") << "\n}\n";
         out->grid = blocks_for(n_out, (int)per_block);
         out->note = "reduce: " + S(G) + " lanes along k, shuffle";
     } else if (vec_outputs) {
@@ -614,9 +649,9 @@ string gen_reduce(Emitter& em, Generated* out) {
             k << "        for (int j = 1; j < " << TK << "; ++j) { const float4 o = red[j * " << TO << " + to];";
             for (const char* c : {"x", "y", "z", "w"}) k << " result." << c << " = " << combine(string("result.") + c, string("o.") + c) << ";";
             k << " }\n";
-            k << "        *(float4*)(b" << fk.outputs[0] << " + vid * 4u) = result;\n    }\n}\n";
+            k << "        " << store_four("result", "vid * 4u") << "\n    }\n}\n";
         } else {
-            k << "    if (vid < " << S(n_vec) << "u) *(float4*)(b" << fk.outputs[0] << " + vid * 4u) = result;\n}\n";
+            k << "    if (vid < " << S(n_vec) << "u) " << store_four("result", "vid * 4u") << "\n}\n";
         }
         out->grid = blocks_for(n_vec, (int)TO);
         out->note = "reduce: lanes along outputs x4, k split " + S(TK);
@@ -639,9 +674,9 @@ string gen_reduce(Emitter& em, Generated* out) {
             k << "    red[threadIdx.x] = result;\n    __syncthreads();\n";
             k << "    if (tk == 0 && oid < " << S(n_out) << "u) {\n";
             k << "        for (int j = 1; j < " << TK << "; ++j) result = " << combine("result", "red[j * " + S(TO) + " + to]") << ";\n";
-            k << "        b" << fk.outputs[0] << "[oid] = result;\n    }\n}\n";
+            k << "        " << store_one("result", "oid") << "\n    }\n}\n";
         } else {
-            k << "    if (oid < " << S(n_out) << "u) b" << fk.outputs[0] << "[oid] = result;\n}\n";
+            k << "    if (oid < " << S(n_out) << "u) " << store_one("result", "oid") << "\n}\n";
         }
         out->grid = blocks_for(n_out, (int)TO);
         out->note = "reduce: lanes along outputs, k split " + S(TK);
@@ -746,6 +781,83 @@ string gen_scatter_add(Emitter& em, Generated* out) {
     out->block = 256;
     out->source = k.str();
     out->note = "scatter_add: global_atomic_add_f32";
+    return "";
+}
+
+// ---- row-fused kernel ---------------------------------------------------------------------------------
+
+string gen_row_fused(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const int64_t m = fk.row_m, n = fk.row_n;
+    if (m < 1 || n < 2 || n > 64) return "row-fused: bad row shape";
+    const int64_t G = pow2_ceil(n), per_block = 256 / G;
+    std::ostringstream k;
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
+    k << "    const uint rand_seed = *seed_cell;\n";
+    k << "    const int col = threadIdx.x % " << G << ";\n";
+    k << "    const int row = blockIdx.x * " << per_block << " + threadIdx.x / " << G << ";\n";
+    // lanes past the last row or column repeat a valid element's work (every lane takes part in the shuffles)
+    // and store nothing
+    k << "    const bool row_ok = row < " << S(m) << ", col_ok = col < " << S(n) << ";\n";
+    k << "    const int rowc = min(row, " << S(m - 1) << "), colc = min(col, " << S(n - 1) << ");\n";
+    k << "    const int wide_gid = rowc * " << S(n) << " + colc;\n";
+    IndexForm wide, narrow;
+    wide.valid = narrow.valid = true;
+    wide.names = {"rowc", "colc"};
+    wide.coefs = {n, 1};
+    wide.extents = {m, n};
+    narrow.names = {"rowc"};
+    narrow.coefs = {1};
+    narrow.extents = {m};
+    // variable holding output `o` of stage `s`
+    auto stage_var = [&](int s_idx, int o) {
+        const dsc_kernel_desc& sd = fk.row_stages[s_idx].k.raw();
+        if (sd.kind == DSC_KERNEL_REDUCE) return "s" + to_string(s_idx) + "_r";
+        return "s" + to_string(s_idx) + "_t" + to_string(sd.outputs[o]);
+    };
+    auto stage_is_wide = [&](int s_idx) {
+        const dsc_kernel_desc& sd = fk.row_stages[s_idx].k.raw();
+        return sd.kind == DSC_KERNEL_PER_ELEMENT && sd.shape.dims[0] == m * n;
+    };
+    for (int si = 0; si < (int)fk.row_stages.size(); ++si) {
+        const RowStage& st = fk.row_stages[si];
+        const dsc_kernel_desc& sd = st.k.raw();
+        const string pfx = "s" + to_string(si) + "_";
+        k << "    // stage " << si << ": " << label_name(sd) << "\n";
+        if (sd.kind == DSC_KERNEL_PER_ELEMENT) {
+            const bool is_wide = stage_is_wide(si);
+            if (!is_wide && sd.shape.dims[0] != m) return "row-fused: per-element stage of the wrong size";
+            std::map<int, string> ov;
+            for (int i = 0; i < sd.n_inputs; ++i)
+                if (st.inputs[i].stage >= 0) ov[i] = stage_var(st.inputs[i].stage, st.inputs[i].stage_out);
+            em.emit_pe(k, sd, st.inputs, is_wide ? "wide_gid" : "rowc", pfx, ov, is_wide ? &wide : &narrow);
+            for (int o = 0; o < sd.n_outputs; ++o) {
+                if (st.outputs[o] < 0) continue;
+                const string ptr = "b" + to_string(fk.outputs[st.outputs[o]]);
+                if (is_wide) k << "    if (row_ok && col_ok) " << ptr << "[row * " << S(n) << " + col] = " << stage_var(si, o) << ";\n";
+                else k << "    if (row_ok && col == 0) " << ptr << "[row] = " << stage_var(si, o) << ";\n";
+            }
+        } else if (sd.kind == DSC_KERNEL_REDUCE) {
+            const bool is_max = sd.reduce_op == DSC_REDUCE_MAX;
+            const string init = is_max ? "U2F(0xff800000u)" : "0.f";
+            string x;
+            if (st.inputs[0].stage >= 0) x = stage_var(st.inputs[0].stage, st.inputs[0].stage_out);
+            else x = em.load_view(st.inputs[0], sd.inputs[0], {"rowc", "colc"});
+            k << "    float " << pfx << "r = col_ok ? " << x << " : " << init << ";\n";
+            for (int64_t off = G / 2; off >= 1; off /= 2) {
+                const string other = "__shfl_xor(" + pfx + "r, " + S(off) + ", 64)";
+                k << "    " << pfx << "r = " << (is_max ? "glsl_max(" + pfx + "r, " + other + ")" : pfx + "r + " + other) << ";\n";
+            }
+            if (st.outputs[0] >= 0) k << "    if (row_ok && col == 0) b" << fk.outputs[st.outputs[0]] << "[row] = " << pfx << "r;\n";
+        } else {
+            return "row-fused: stage must be a per-element or reduce kernel";
+        }
+    }
+    k << "}\n";
+    out->grid = blocks_for(m, (int)per_block);
+    out->block = 256;
+    out->source = k.str();
+    out->note = "row-fused: " + S(G) + " lanes per row, " + to_string(fk.row_stages.size()) + " stages";
     return "";
 }
 
@@ -1135,6 +1247,47 @@ string gen_matmul(Emitter& em, Generated* out) {
     return "";
 }
 
+// Algorithmic bytes and flops of one launch (see Generated).
+void count_work(const FusedKernel& fk, Generated* g) {
+    const dsc_kernel_desc& d = fk.main.raw();
+    std::vector<double> touched(fk.n_buffers, 0.0), extent(fk.n_buffers, 0.0);
+    auto read = [&](const Source& s, const dsc_view& v, double elements) {
+        if (s.buffer < 0) return;
+        touched[s.buffer] += elements;
+        extent[s.buffer] = std::max(extent[s.buffer], (double)element_count(v.in_shape));
+    };
+    auto read_desc = [&](const dsc_kernel_desc& k, const std::vector<Source>& srcs, int skip) {
+        for (int i = 0; i < k.n_inputs && i < (int)srcs.size(); ++i) {
+            if (i == skip) continue;
+            double elements = (double)element_count(k.inputs[i].out_shape);
+            if (k.kind == DSC_KERNEL_PER_ELEMENT)
+                for (int o = 0; o < k.n_ops; ++o)
+                    if (k.ops[o].kind == DSC_PE_GATHER && k.ops[o].input_index == i) elements = (double)element_count(k.ops[o].gather_shape);
+            read(srcs[i], k.inputs[i], elements);
+        }
+    };
+    if (fk.row_stages.empty()) read_desc(d, fk.inputs, -1);
+    for (auto& st : fk.row_stages) read_desc(st.k.raw(), st.inputs, -1);
+    for (auto& v : fk.virtuals) read_desc(v.pe.raw(), v.inputs, -1);
+    if (fk.has_epilogue) read_desc(fk.epilogue.raw(), fk.epilogue_inputs, fk.epilogue_product_input);
+    double elements = 0;
+    for (int i = 0; i < fk.n_buffers; ++i)
+        if (!fk.buffer_is_output[i]) elements += std::min(touched[i], extent[i]);
+    double out_each = (double)element_count(d.shape);
+    if (d.kind == DSC_KERNEL_MATMUL) {
+        const MatMulDims m = matmul_dims(d);
+        out_each = (double)(m.batch * m.m * m.n) * (double)(fk.sum_chunks ? 1 : m.chunks);
+        g->algo_flops = 2.0 * (double)m.batch * (double)m.m * (double)m.n * (double)m.k;
+    }
+    if (d.kind == DSC_KERNEL_SCATTER_ADD)  // read-modify-write of the entries that receive a value
+        out_each = 2.0 * std::min((double)element_count(d.shape), (double)element_count(d.inputs[0].out_shape));
+    if (fk.row_stages.empty()) elements += out_each * (double)fk.outputs.size();
+    for (auto& st : fk.row_stages)
+        for (int o : st.outputs)
+            if (o >= 0) elements += (double)element_count(st.k.raw().shape);
+    g->algo_bytes = 4.0 * elements;
+}
+
 }  // namespace
 
 bool tallk_shape(const MatMulDims& g) { return tallk_shape_impl(g); }
@@ -1175,6 +1328,19 @@ std::string FusedKernel::key() const {
         s.append(reinterpret_cast<const char*>(&epilogue_product_input), 4);
         for (auto& x : epilogue_inputs) put_src(x);
     }
+    for (auto& st : row_stages) {
+        s += "|R" + st.k.key();
+        for (auto& x : st.inputs) {
+            put_src(x);
+            s.append(reinterpret_cast<const char*>(&x.stage), 4);
+            s.append(reinterpret_cast<const char*>(&x.stage_out), 4);
+        }
+        for (int o : st.outputs) s.append(reinterpret_cast<const char*>(&o), 4);
+    }
+    if (!row_stages.empty()) {
+        s.append(reinterpret_cast<const char*>(&row_m), 8);
+        s.append(reinterpret_cast<const char*>(&row_n), 8);
+    }
     s += sum_chunks ? "|S1" : "|S0";
     s += "|O";
     for (int o : outputs) s.append(reinterpret_cast<const char*>(&o), 4);
@@ -1200,15 +1366,25 @@ std::string generate(const FusedKernel& fk, Generated* out) {
     if (fk.has_epilogue) {
         err = validate(fk.epilogue.raw());
         if (!err.empty()) return "epilogue: " + err;
-        if (fk.main.raw().kind != DSC_KERNEL_MATMUL) return "only MatMul takes an epilogue";
+        if (fk.main.raw().kind != DSC_KERNEL_MATMUL && fk.main.raw().kind != DSC_KERNEL_REDUCE) return "only MatMul and Reduce take an epilogue";
     }
-    if ((int)fk.inputs.size() != fk.main.raw().n_inputs) return "input binding count";
+    for (auto& st : fk.row_stages) {
+        err = validate(st.k.raw());
+        if (!err.empty()) return "row stage: " + err;
+        if ((int)st.inputs.size() != st.k.raw().n_inputs) return "row stage: input binding count";
+        const int n_out = st.k.raw().kind == DSC_KERNEL_PER_ELEMENT ? st.k.raw().n_outputs : 1;
+        if ((int)st.outputs.size() != n_out) return "row stage: output binding count";
+    }
+    if (fk.row_stages.empty() && (int)fk.inputs.size() != fk.main.raw().n_inputs) return "input binding count";
     if ((int)fk.buffer_is_output.size() != fk.n_buffers) return "buffer table size";
     err = check_sizes(fk);
     if (!err.empty()) return err;
 
     Emitter em(fk);
     Generated g;
+    if (!fk.row_stages.empty()) {
+        err = gen_row_fused(em, &g);
+    } else
     switch (fk.main.raw().kind) {
     case DSC_KERNEL_FILL: err = gen_fill(em, &g); break;
     case DSC_KERNEL_PER_ELEMENT: err = gen_per_element(em, &g); break;
@@ -1223,6 +1399,7 @@ std::string generate(const FusedKernel& fk, Generated* out) {
     g.source = string(kPreludeSource) + "\n" + em.funcs.str() + "\n" + g.source;
     g.n_buffers = fk.n_buffers;
     g.entry = entry_name(fk);
+    count_work(fk, &g);
     *out = g;
     return "";
 }

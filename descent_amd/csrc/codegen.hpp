@@ -18,8 +18,10 @@ namespace dsc {
 
 // Where the elements of one kernel input come from.
 struct Source {
-    int buffer = -1;  // index of a pointer parameter of the generated kernel, or
-    int virt = -1;    // index into FusedKernel::virtuals
+    int buffer = -1;     // index of a pointer parameter of the generated kernel, or
+    int virt = -1;       // index into FusedKernel::virtuals, or
+    int stage = -1;      // (row-fused kernels) index of an earlier stage whose result stays in registers,
+    int stage_out = 0;   // and which of that stage's outputs
 };
 
 // A per-element cluster evaluated lazily: value(gid) = ops[out_op] at linear element id `gid`.
@@ -27,6 +29,13 @@ struct Virtual {
     KernelDesc pe;
     int out_op = 0;
     std::vector<Source> inputs;  // one per pe input
+};
+
+// One cluster of a row-fused kernel (see FusedKernel::row_stages).
+struct RowStage {
+    KernelDesc k;                // PerElement over [m, n] or [m] elements, or Reduce of [m, n] along n
+    std::vector<Source> inputs;  // one per input view of k
+    std::vector<int> outputs;    // per output of k: index into FusedKernel::outputs when stored, else -1
 };
 
 struct FusedKernel {
@@ -39,6 +48,13 @@ struct FusedKernel {
     KernelDesc epilogue;
     int epilogue_product_input = -1;       // which epilogue input is the product
     std::vector<Source> epilogue_inputs;   // one per epilogue input (the product's entry is ignored)
+    // Row-fused kernel: clusters that all work on the rows of one [m, n] array with n <= 64 (a softmax
+    // cross-entropy with its accuracy count: row max, exp, row sum, log, gradient, per-row loss) run as one
+    // kernel.  A group of lanes owns a row, lane j holds column j of every [m, n] value, an [m]-shaped value is
+    // the same in every lane of the group, a Reduce along n is a butterfly of shuffles.  Stages run in order;
+    // `main` is the first stage's descriptor (for the label), only the outputs someone else needs are stored.
+    std::vector<RowStage> row_stages;
+    int64_t row_m = 0, row_n = 0;
     bool sum_chunks = false;               // MatMul: ignore the descriptor's chunk count, write one full sum
     std::vector<int> outputs;              // pointer parameter index of each output of main (or of the epilogue)
     int n_buffers = 0;                     // number of pointer parameters
@@ -56,6 +72,10 @@ struct Generated {
     unsigned block = 64;     // threads per workgroup
     int n_buffers = 0;       // pointer parameters, in order; followed by `const uint* seed_cell`
     std::string note;        // strategy chosen (for schedule listings)
+    // Work one launch stands for, counted the way a roofline wants it: bytes = 4 * (distinct elements of every
+    // buffer read, a broadcast or windowed operand at its own size, + elements written; a scatter accumulator is
+    // read and written where values land), flops = 2*b*M*N*K of a MatMul (0 otherwise).
+    double algo_bytes = 0, algo_flops = 0;
 };
 
 // Returns "" on success or an error message.

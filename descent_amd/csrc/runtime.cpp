@@ -261,6 +261,9 @@ Kernel* get_kernel(Context* ctx, const FusedKernel& fk, int* status) {
         return nullptr;
     }
     k->label = label_name(fk.main.raw());
+    if (!fk.row_stages.empty())
+        k->label = "RowFused [" + std::to_string((long long)fk.row_m) + ", " + std::to_string((long long)fk.row_n) + "] (" +
+                   std::to_string(fk.row_stages.size()) + " clusters)";
     if (fk.has_epilogue) k->label += " + " + label_name(fk.epilogue.raw());
     if (!fk.virtuals.empty()) k->label += " <" + std::to_string(fk.virtuals.size()) + " fused producers>";
     k->reference_groups = reference_group_count(fk.main.raw());

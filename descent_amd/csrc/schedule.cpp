@@ -2,6 +2,7 @@
 #include "schedule.hpp"
 
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
 #include <set>
 #include <sstream>
@@ -54,6 +55,9 @@ Source import_source(Draft& q, const Draft& p, const Source& s, int virt_offset)
 template <class F>
 void for_each_source(FusedKernel& fk, F f) {
     for (auto& s : fk.inputs) f(s);
+    for (auto& st : fk.row_stages)
+        for (auto& s : st.inputs)
+            if (s.stage < 0) f(s);
     for (auto& v : fk.virtuals)
         for (auto& s : v.inputs) f(s);
     if (fk.has_epilogue)
@@ -374,6 +378,37 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             return false;
         };
 
+        // A per-element cluster that can run as the epilogue of the launch producing `product_node` (`elements`
+        // values): it is the node's only consumer, has one invocation per product element and reads the product
+        // element-for-element through a plain load.
+        auto find_epilogue = [&](int producer_idx, int product_node, int64_t elements, int* pe_idx, int* pe_input) {
+            *pe_idx = *pe_input = -1;
+            if (is_graph_output[product_node]) return;
+            auto cons = consumers_of(product_node);
+            if (cons.size() != 1 || cons[0] <= producer_idx) return;
+            Draft& e = drafts[cons[0]];
+            const dsc_kernel_desc& ed = e.fk.main.raw();
+            if (ed.kind != DSC_KERNEL_PER_ELEMENT || e.fk.has_epilogue || ed.shape.dims[0] != elements) return;
+            int hits = 0, input = -1;
+            for (int k = 0; k < ed.n_inputs; ++k) {
+                if (e.fk.inputs[k].buffer >= 0 && e.params[e.fk.inputs[k].buffer] == product_node) {
+                    ++hits;
+                    input = k;
+                }
+            }
+            if (hits != 1) return;
+            for (int k = 0; k < ed.n_ops; ++k)  // the product must be read element-for-element, not gathered
+                if (ed.ops[k].kind == DSC_PE_GATHER && ed.ops[k].input_index == input) return;
+            for (auto& v : e.fk.virtuals)  // and not through one of the consumer's own fused producers
+                for (auto& src : v.inputs)
+                    if (src.buffer >= 0 && e.params[src.buffer] == product_node) return;
+            for (auto& o : e.outs)
+                if (o.copy_from >= 0) return;
+            if (!is_contiguous(ed.inputs[input]) || taken_in_place_between(producer_idx, cons[0], input_nodes(drafts[producer_idx]))) return;
+            *pe_idx = cons[0];
+            *pe_input = input;
+        };
+
         // Pass 1: MatMul (+ Reduce over its split-K partials) (+ per-element consumer as epilogue).
         for (int i = 0; i < (int)drafts.size(); ++i) {
             Draft& mm = drafts[i];
@@ -399,33 +434,7 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             }
             // optional epilogue
             int pe_idx = -1, pe_input = -1;
-            if (!is_graph_output[product_node]) {
-                auto cons = consumers_of(product_node);
-                if (cons.size() == 1) {
-                    Draft& e = drafts[cons[0]];
-                    const dsc_kernel_desc& ed = e.fk.main.raw();
-                    if (ed.kind == DSC_KERNEL_PER_ELEMENT && ed.shape.dims[0] == g.batch * g.m * g.n) {
-                        int hits = 0;
-                        for (int k = 0; k < ed.n_inputs; ++k) {
-                            if (e.fk.inputs[k].buffer >= 0 && e.params[e.fk.inputs[k].buffer] == product_node) {
-                                ++hits;
-                                pe_input = k;
-                            }
-                        }
-                        bool only_loaded = true;  // the product must be read element-for-element, not gathered
-                        for (int k = 0; k < ed.n_ops; ++k)
-                            if (ed.ops[k].kind == DSC_PE_GATHER && ed.ops[k].input_index == pe_input) only_loaded = false;
-                        // and not through one of the consumer's own fused producers
-                        bool via_virtual = false;
-                        for (auto& v : e.fk.virtuals)
-                            for (auto& s : v.inputs)
-                                if (s.buffer >= 0 && e.params[s.buffer] == product_node) via_virtual = true;
-                        if (hits == 1 && only_loaded && !via_virtual && is_contiguous(ed.inputs[pe_input]) &&
-                            !taken_in_place_between(i, cons[0], input_nodes(mm)))
-                            pe_idx = cons[0];
-                    }
-                }
-            }
+            find_epilogue(i, product_node, g.batch * g.m * g.n, &pe_idx, &pe_input);
             if (reduce_idx < 0 && pe_idx < 0) continue;
 
             Draft fused;
@@ -464,6 +473,132 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             }
         }
 
+        // Pass 1b: clusters that all work on the rows of one [m, n] array with a short n -- Reduces along n and the
+        // per-element clusters around them (softmax cross-entropy: row max, exp, row sum, log-probability, gradient,
+        // per-row loss; the accuracy count: arg-max and comparison with the label) -- become one row-fused launch.
+        // The launch runs where the first of them ran, so a member may only read what exists by then or what
+        // another member computes.
+        {
+            std::vector<int> producer_of(n_nodes, -1);  // draft index writing each node
+            auto refresh_producers = [&]() {
+                std::fill(producer_of.begin(), producer_of.end(), -1);
+                for (int i = 0; i < (int)drafts.size(); ++i)
+                    if (drafts[i].alive)
+                        for (auto& o : drafts[i].outs) producer_of[o.node] = i;
+            };
+            auto is_plain = [&](const Draft& d) {
+                if (!d.alive || !d.fk.virtuals.empty() || d.fk.has_epilogue || !d.fk.row_stages.empty() || d.keep_output || d.keep_split) return false;
+                for (auto& o : d.outs)
+                    if (o.copy_from >= 0) return false;
+                return true;
+            };
+            auto shape_is = [](const dsc_shape& sh, int64_t a, int64_t b) { return sh.rank == 2 && sh.dims[0] == a && sh.dims[1] == b; };
+            for (int seed = 0; seed < (int)drafts.size(); ++seed) {
+                if (!is_plain(drafts[seed])) continue;
+                const dsc_kernel_desc& sd = drafts[seed].fk.main.raw();
+                if (sd.kind != DSC_KERNEL_REDUCE || sd.inputs[0].out_shape.rank != 2 || sd.axis != 1) continue;
+                const int64_t m = sd.inputs[0].out_shape.dims[0], n = sd.inputs[0].out_shape.dims[1];
+                if (n < 2 || n > 64 || m < 2 || !shape_is(sd.shape, m, 1)) continue;
+                refresh_producers();
+                std::vector<int> members;      // draft indices, in order
+                std::vector<int> member_of(drafts.size(), -1);
+                auto try_add = [&](int j) {
+                    const Draft& d = drafts[j];
+                    if (!is_plain(d)) return false;
+                    const dsc_kernel_desc& k = d.fk.main.raw();
+                    bool wide = false;
+                    if (k.kind == DSC_KERNEL_REDUCE) {
+                        if (k.axis != 1 || !shape_is(k.inputs[0].out_shape, m, n) || !shape_is(k.shape, m, 1)) return false;
+                    } else if (k.kind == DSC_KERNEL_PER_ELEMENT) {
+                        wide = k.shape.dims[0] == m * n;
+                        if (!wide && k.shape.dims[0] != m) return false;
+                        auto shape_ok = [&](const dsc_shape& sh) {
+                            return wide ? shape_is(sh, m, n) : (shape_is(sh, m, 1) || (sh.rank == 1 && sh.dims[0] == m));
+                        };
+                        for (int i = 0; i < k.n_inputs; ++i)
+                            if (!shape_ok(k.inputs[i].out_shape)) return false;
+                        for (int i = 0; i < k.n_builtin_views; ++i)
+                            if (!shape_ok(k.builtin_views[i].out_shape)) return false;
+                        for (int i = 0; i < k.n_ops; ++i)
+                            if (k.ops[i].kind == DSC_PE_GATHER) return false;
+                    } else {
+                        return false;
+                    }
+                    for (int i = 0; i < k.n_inputs; ++i) {
+                        const int node = d.params[d.fk.inputs[i].buffer];
+                        const int p = producer_of[node];
+                        if (p >= 0 && member_of[p] >= 0) {
+                            // computed by a member: must be read element for element (or one value per row)
+                            const dsc_kernel_desc& pk = drafts[p].fk.main.raw();
+                            const bool p_wide = pk.kind == DSC_KERNEL_PER_ELEMENT && pk.shape.dims[0] == m * n;
+                            const dsc_view& v = k.inputs[i];
+                            if (element_count(v.in_shape) != (p_wide ? m * n : m)) return false;
+                            int64_t base, coef[DSC_MAX_DIM];
+                            if (!affine_form(v, &base, coef) || base != 0) return false;
+                            if (p_wide) {
+                                if (!(k.kind == DSC_KERNEL_REDUCE || wide) || coef[0] != n || coef[1] != 1) return false;
+                            } else {
+                                if (k.kind == DSC_KERNEL_REDUCE || coef[0] != 1) return false;
+                                if (v.out_shape.rank == 2 && v.out_shape.dims[1] > 1 && coef[1] != 0) return false;
+                            }
+                        } else if (p >= seed) {
+                            return false;  // does not exist yet where the fused launch runs
+                        }
+                    }
+                    return true;
+                };
+                for (int j = seed; j < (int)drafts.size(); ++j) {
+                    if (!try_add(j)) {
+                        if (j == seed) break;
+                        continue;
+                    }
+                    member_of[j] = (int)members.size();
+                    members.push_back(j);
+                }
+                if (members.size() < 2 || members.size() > 24) continue;
+                Draft fused;
+                fused.fk.main = drafts[seed].fk.main;
+                fused.fk.row_m = m;
+                fused.fk.row_n = n;
+                for (int j : members) {
+                    const Draft& d = drafts[j];
+                    const dsc_kernel_desc& k = d.fk.main.raw();
+                    RowStage st;
+                    st.k = d.fk.main;
+                    for (int i = 0; i < k.n_inputs; ++i) {
+                        const int node = d.params[d.fk.inputs[i].buffer];
+                        const int p = producer_of[node];
+                        Source src;
+                        if (p >= 0 && member_of[p] >= 0) {
+                            src.stage = member_of[p];
+                            for (size_t o = 0; o < drafts[p].outs.size(); ++o)
+                                if (drafts[p].outs[o].node == node) src.stage_out = (int)o;
+                        } else {
+                            src.buffer = param_index(fused, node, false);
+                        }
+                        st.inputs.push_back(src);
+                    }
+                    for (auto& o : d.outs) {
+                        bool needed = is_graph_output[o.node];
+                        for (int c : consumers_of(o.node))
+                            if (member_of[c] < 0) needed = true;
+                        if (needed) {
+                            st.outputs.push_back((int)fused.fk.outputs.size());
+                            fused.fk.outputs.push_back(param_index(fused, o.node, true));
+                            fused.outs.push_back(o);
+                        } else {
+                            st.outputs.push_back(-1);
+                        }
+                    }
+                    fused.fk.row_stages.push_back(st);
+                    fused.covers.insert(fused.covers.end(), d.covers.begin(), d.covers.end());
+                }
+                if (fused.fk.outputs.empty()) continue;
+                for (int j : members) drafts[j].alive = false;
+                drafts[seed] = fused;
+            }
+        }
+
         // Pass 2: per-element producers whose result need not exist in memory are evaluated inside their
         // consumers: pure copies (materialised im2col / pooling windows) into every consumer, light arithmetic
         // into a single consumer.
@@ -485,6 +620,7 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                 Draft& p = drafts[i];
                 if (!p.alive) continue;
                 const dsc_kernel_desc& pd = p.fk.main.raw();
+                if (!p.fk.row_stages.empty()) continue;
                 const bool is_pe = pd.kind == DSC_KERNEL_PER_ELEMENT && pd.n_outputs == 1 && !p.fk.has_epilogue;
                 const bool is_red = pd.kind == DSC_KERNEL_REDUCE;
                 if ((!is_pe && !is_red) || p.keep_output) continue;
@@ -522,6 +658,7 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                         if (o.copy_from == node) ok = false;  // updated in place by the consumer
                     if (taken_in_place_between(i, ci, input_nodes(p))) ok = false;
                     if ((int)q.fk.virtuals.size() + (int)p.fk.virtuals.size() + 1 > 8) ok = false;
+                    if (!q.fk.row_stages.empty()) ok = false;
                     // an epilogue reads its product from the accumulator, never through a producer
                     if (q.fk.has_epilogue && q.fk.epilogue_product_input >= 0) {
                         const Source& ps = q.fk.epilogue_inputs[q.fk.epilogue_product_input];
@@ -553,6 +690,40 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                 p.alive = false;
                 changed = true;
             }
+        }
+
+        // Pass 3: a Reduce whose only consumer is a per-element cluster over its outputs (a scalar accumulated into
+        // a running sum, the optimiser update of a bias gradient) applies that cluster to each result before the
+        // store.
+        for (int i = 0; i < (int)drafts.size(); ++i) {
+            Draft& r = drafts[i];
+            if (!r.alive || r.fk.main.raw().kind != DSC_KERNEL_REDUCE || r.fk.has_epilogue || r.keep_output || !r.fk.row_stages.empty()) continue;
+            int pe_idx = -1, pe_input = -1;
+            find_epilogue(i, r.outs[0].node, element_count(r.fk.main.raw().shape), &pe_idx, &pe_input);
+            if (pe_idx < 0) continue;
+            Draft& e = drafts[pe_idx];
+            if ((int)r.fk.virtuals.size() + (int)e.fk.virtuals.size() > 8) continue;
+            Draft fused;
+            fused.fk.main = r.fk.main;
+            const int voff = import_virtuals(fused, r);
+            for (auto& src : r.fk.inputs) fused.fk.inputs.push_back(import_source(fused, r, src, voff));
+            fused.covers = r.covers;
+            fused.fk.has_epilogue = true;
+            fused.fk.epilogue = e.fk.main;
+            fused.fk.epilogue_product_input = pe_input;
+            const int eoff = import_virtuals(fused, e);
+            for (int k = 0; k < (int)e.fk.inputs.size(); ++k) {
+                if (k == pe_input) fused.fk.epilogue_inputs.push_back(Source{});
+                else fused.fk.epilogue_inputs.push_back(import_source(fused, e, e.fk.inputs[k], eoff));
+            }
+            for (auto& o : e.outs) {
+                fused.fk.outputs.push_back(param_index(fused, o.node, true));
+                fused.outs.push_back(o);
+            }
+            fused.covers.insert(fused.covers.end(), e.covers.begin(), e.covers.end());
+            compact(fused);
+            r.alive = false;
+            drafts[pe_idx] = fused;  // runs where the per-element cluster ran: all of its inputs exist by then
         }
     }
 
@@ -735,13 +906,21 @@ std::string Schedule::describe() const {
     o << steps.size() << " launches for " << n_clusters << " clusters\n";
     if (replays + direct_runs + (int64_t)captured.size() > 0)
         o << "# graph replays " << replays << ", captured " << captured.size() << ", direct runs " << direct_runs << "\n";
+    double bytes = 0, flops = 0;
     for (size_t i = 0; i < steps.size(); ++i) {
         const Step& st = steps[i];
+        char work[64];
+        std::snprintf(work, sizeof work, " %.3f MB", st.kernel->gen.algo_bytes / 1e6);
         o << i << ": " << st.kernel->label << "  [" << st.kernel->gen.note << "] grid " << st.kernel->gen.grid << "x"
-          << st.kernel->gen.block << " clusters";
+          << st.kernel->gen.block << work << " clusters";
         for (int c : st.covers) o << " " << c;
         o << "\n";
+        bytes += st.kernel->gen.algo_bytes;
+        flops += st.kernel->gen.algo_flops;
     }
+    char total[160];
+    std::snprintf(total, sizeof total, "# algorithmic work per run: %.3f MB moved, %.3f GFLOP in MatMuls\n", bytes / 1e6, flops / 1e9);
+    o << total;
     return o.str();
 }
 

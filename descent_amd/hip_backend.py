@@ -71,6 +71,8 @@ def lib():
         "dsc_prof_reset": (C.c_int, [vp]),
         "dsc_prof_report": (C.c_int, [vp, C.c_int, C.POINTER(vp)]),
         "dsc_prof_query": (C.c_int, [vp, C.c_char_p, C.POINTER(C.c_double), C.POINTER(C.c_int64)]),
+        "dsc_prof_work": (C.c_int, [vp, C.c_char_p, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_double),
+                                    C.POINTER(C.c_int64)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -86,7 +88,7 @@ EXPORTED_SYMBOLS = [
     "dsc_kernel_label", "dsc_kernel_source", "dsc_kernel_launch", "dsc_codegen_source", "dsc_codegen_compile",
     "dsc_codegen_check_schedule", "dsc_free_string", "dsc_schedule_create", "dsc_schedule_destroy",
     "dsc_schedule_run", "dsc_schedule_launch_count", "dsc_schedule_describe", "dsc_prof_enable", "dsc_prof_reset",
-    "dsc_prof_report", "dsc_prof_query",
+    "dsc_prof_report", "dsc_prof_query", "dsc_prof_work",
 ]
 
 
@@ -250,3 +252,9 @@ class HipBackend:
         avg, n = C.c_double(), C.c_int64()
         check(lib().dsc_prof_query(self._ctx, prefix.encode(), C.byref(avg), C.byref(n)))
         return avg.value, n.value
+
+    def timing_work(self, prefix: str):
+        """(total us, algorithmic bytes, algorithmic flops, launches) of the launches whose label starts with prefix."""
+        us, nbytes, flops, n = C.c_double(), C.c_double(), C.c_double(), C.c_int64()
+        check(lib().dsc_prof_work(self._ctx, prefix.encode(), C.byref(us), C.byref(nbytes), C.byref(flops), C.byref(n)))
+        return us.value, nbytes.value, flops.value, n.value

@@ -305,10 +305,17 @@ int dsc_schedule_describe(const dsc_schedule* s, char** out_text);
 int dsc_prof_enable(dsc_ctx* ctx, int enabled);
 int dsc_prof_reset(dsc_ctx* ctx);
 /* Writes a report into a malloc'd string (caller: dsc_free_string): one line per label with launches,
- * total ms and average us, sorted by total time, at most top_n lines (0 = all). */
+ * total ms, average us and the achieved GB/s or TFLOP/s against the HBM or fp32 MFMA peak, sorted by total
+ * time, at most top_n lines (0 = all). */
 int dsc_prof_report(dsc_ctx* ctx, int top_n, char** out_text);
 /* Average duration in microseconds and launch count of all launches whose label starts with `prefix`. */
 int dsc_prof_query(dsc_ctx* ctx, const char* prefix, double* out_avg_us, int64_t* out_launches);
+/* Sums over the same launches: total microseconds, and the algorithmic bytes and flops those launches stand for
+ * (bytes: 4 x distinct elements read, an operand read through a broadcast or window view at its own size, plus
+ * elements written; flops: 2*b*M*N*K per MatMul).  The reference prints times only (device/timestamp.rs:155-179);
+ * the work figures are what turns them into a fraction of the HBM or MFMA roof. */
+int dsc_prof_work(dsc_ctx* ctx, const char* prefix, double* out_total_us, double* out_algo_bytes, double* out_algo_flops,
+                  int64_t* out_launches);
 
 #ifdef __cplusplus
 }
