@@ -1341,6 +1341,10 @@ std::string FusedKernel::key() const {
         s.append(reinterpret_cast<const char*>(&row_m), 8);
         s.append(reinterpret_cast<const char*>(&row_n), 8);
     }
+    for (size_t i = 0; i < parts.size(); ++i) {
+        s += "|P{" + parts[i].key() + "}";
+        for (int j : part_params[i]) s.append(reinterpret_cast<const char*>(&j), 4);
+    }
     s += sum_chunks ? "|S1" : "|S0";
     s += "|O";
     for (int o : outputs) s.append(reinterpret_cast<const char*>(&o), 4);
@@ -1353,7 +1357,23 @@ std::string FusedKernel::key() const {
     return s;
 }
 
+namespace {
+string generate_multi(const FusedKernel& fk, Generated* out);
+}
+
+bool can_be_part(const FusedKernel& fk) {
+    if (!fk.parts.empty()) return false;
+    return fk.main.raw().kind != DSC_KERNEL_MATMUL;  // the MatMul kernels size their workgroups per shape
+}
+
+static std::string generate_one(const FusedKernel& fk, Generated* out, bool with_prelude);
+
 std::string generate(const FusedKernel& fk, Generated* out) {
+    if (!fk.parts.empty()) return generate_multi(fk, out);
+    return generate_one(fk, out, true);
+}
+
+static std::string generate_one(const FusedKernel& fk, Generated* out, bool with_prelude) {
     string err = validate(fk.main.raw());
     if (!err.empty()) return err;
     for (auto& v : fk.virtuals) {
@@ -1396,13 +1416,58 @@ std::string generate(const FusedKernel& fk, Generated* out) {
     default: err = "unknown kernel kind";
     }
     if (!err.empty()) return err;
-    g.source = string(kPreludeSource) + "\n" + em.funcs.str() + "\n" + g.source;
+    g.source = (with_prelude ? string(kPreludeSource) + "\n" : string()) + em.funcs.str() + "\n" + g.source;
     g.n_buffers = fk.n_buffers;
     g.entry = entry_name(fk);
     count_work(fk, &g);
     *out = g;
     return "";
 }
+
+namespace {
+// One launch running several independent kernels: each part is generated as usual, its entry point turned into a
+// device function taking the workgroup id, inside a namespace of its own (helper names repeat between parts).
+string generate_multi(const FusedKernel& fk, Generated* out) {
+    if (fk.parts.size() != fk.part_params.size() || fk.parts.empty()) return "multi: part tables differ";
+    Generated g;
+    std::ostringstream src, body;
+    src << kPreludeSource << "\n";
+    unsigned first = 0;
+    for (size_t i = 0; i < fk.parts.size(); ++i) {
+        const FusedKernel& part = fk.parts[i];
+        if (!can_be_part(part)) return "multi: kernel cannot be a part";
+        Generated pg;
+        string err = generate_one(part, &pg, false);
+        if (!err.empty()) return err;
+        if (pg.block != 256) return "multi: parts must use 256 threads";
+        if ((int)fk.part_params[i].size() != part.n_buffers) return "multi: part parameter count";
+        const string head = "extern \"C\" __global__ __launch_bounds__(256) void " + pg.entry + "(";
+        const size_t at = pg.source.find(head);
+        if (at == string::npos) return "multi: unexpected entry point form";
+        string text = pg.source;
+        text.replace(at, head.size(), "DSC_INLINE void part_entry(const uint dsc_block, ");
+        for (size_t pos = text.find("blockIdx.x"); pos != string::npos; pos = text.find("blockIdx.x", pos)) text.replace(pos, 10, "dsc_block");
+        if (text.find("gridDim") != string::npos) return "multi: part depends on the grid size";
+        src << "namespace part" << i << " {\n" << text << "}  // namespace part" << i << "\n\n";
+        body << "    if (blockIdx.x < " << first + pg.grid << "u) { part" << i << "::part_entry(blockIdx.x - " << first << "u";
+        for (int j : fk.part_params[i]) body << ", b" << j;
+        body << ", seed_cell); return; }\n";
+        first += pg.grid;
+        g.algo_bytes += pg.algo_bytes;
+        g.algo_flops += pg.algo_flops;
+        g.note += (i ? " | " : "multi: ") + pg.note;
+    }
+    Emitter em(fk);
+    g.entry = "dsc_multi_p" + to_string(fk.parts.size()) + "_g" + to_string(first);
+    src << "extern \"C\" __global__ __launch_bounds__(256) void " << g.entry << "(" << em.kernel_params_decl() << ") {\n" << body.str() << "}\n";
+    g.source = src.str();
+    g.grid = first;
+    g.block = 256;
+    g.n_buffers = fk.n_buffers;
+    *out = g;
+    return "";
+}
+}  // namespace
 
 const std::vector<std::string>& compile_options() {
     // packed fp32 instructions are kept off for every kernel; float atomicAdd maps to the hardware instruction;

@@ -55,6 +55,11 @@ struct FusedKernel {
     // `main` is the first stage's descriptor (for the label), only the outputs someone else needs are stored.
     std::vector<RowStage> row_stages;
     int64_t row_m = 0, row_n = 0;
+    // Several independent small kernels in one launch: workgroup ids [0, g0) run parts[0], [g0, g0 + g1) run
+    // parts[1], ...  part_params[i][j] is the pointer parameter of this kernel that part i's parameter j binds.
+    // `main` is parts[0].main (for the label); inputs/outputs of the launch are those of the parts.
+    std::vector<FusedKernel> parts;
+    std::vector<std::vector<int>> part_params;
     bool sum_chunks = false;               // MatMul: ignore the descriptor's chunk count, write one full sum
     std::vector<int> outputs;              // pointer parameter index of each output of main (or of the epilogue)
     int n_buffers = 0;                     // number of pointer parameters
@@ -80,6 +85,9 @@ struct Generated {
 
 // Returns "" on success or an error message.
 std::string generate(const FusedKernel& k, Generated* out);
+
+// Whether a kernel can be one part of a multi-part launch (256 threads per workgroup, addressed by blockIdx.x only).
+bool can_be_part(const FusedKernel& k);
 
 // Whether a MatMul of these dimensions (already split into its chunks) runs on the tall-k kernel: a small output
 // summed over a long k, one workgroup per (chunk, batch).  The schedule sizes its k re-split for that kernel.

@@ -266,6 +266,11 @@ Kernel* get_kernel(Context* ctx, const FusedKernel& fk, int* status) {
                    std::to_string(fk.row_stages.size()) + " clusters)";
     if (fk.has_epilogue) k->label += " + " + label_name(fk.epilogue.raw());
     if (!fk.virtuals.empty()) k->label += " <" + std::to_string(fk.virtuals.size()) + " fused producers>";
+    if (!fk.parts.empty()) {
+        k->label = "Multi (" + std::to_string(fk.parts.size()) + " kernels:";
+        for (auto& part : fk.parts) k->label += " " + std::string(part.row_stages.empty() ? label_name(part.main.raw()) : "RowFused") + ";";
+        k->label += ")";
+    }
     k->reference_groups = reference_group_count(fk.main.raw());
     if (const char* dump = std::getenv("DSC_DUMP_DIR")) {  // debugging aid: one source file per generated kernel
         std::ofstream f(std::string(dump) + "/kernel_" + std::to_string(ctx->kernels.size()) + ".hip");

@@ -20,6 +20,7 @@ struct Draft {
     std::vector<int> covers;      // reference cluster indices folded into this launch
     bool keep_split = false;      // MatMul re-split over k on purpose: do not sum its chunks in one workgroup
     bool keep_output = false;     // first stage of a split reduction: its result must exist in memory
+    std::vector<int> part_inputs; // multi-part launch: the distinct nodes its parts read
 };
 
 int param_index(Draft& d, int node, bool is_output) {
@@ -87,6 +88,7 @@ void compact(Draft& d) {
 }
 
 std::vector<int> input_nodes(const Draft& d) {
+    if (!d.fk.parts.empty()) return d.part_inputs;
     std::set<int> seen;
     std::vector<int> out;
     Draft& md = const_cast<Draft&>(d);
@@ -724,6 +726,72 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             compact(fused);
             r.alive = false;
             drafts[pe_idx] = fused;  // runs where the per-element cluster ran: all of its inputs exist by then
+        }
+
+        // Pass 4: launches of a few workgroups each (optimiser updates of small tensors, short reductions, scalar
+        // bookkeeping) cost a launch apiece while using a fraction of the machine.  Runs of them that do not
+        // depend on one another become one multi-part launch; a later small launch is hoisted into the run when
+        // nothing it reads is produced in between.
+        {
+            static const int64_t small_grid = std::getenv("DSC_MULTI_GRID") ? std::atoll(std::getenv("DSC_MULTI_GRID")) : 1024;
+            std::vector<int> grid_of(drafts.size(), -1);
+            auto small = [&](int i) {
+                const Draft& d = drafts[i];
+                if (!d.alive || !can_be_part(d.fk)) return false;
+                for (auto& o : d.outs)
+                    if (o.copy_from >= 0) return false;
+                if (grid_of[i] < 0) {
+                    Generated g;
+                    if (!generate(d.fk, &g).empty() || g.block != 256) { grid_of[i] = 1 << 30; return false; }
+                    grid_of[i] = (int)std::min<unsigned>(g.grid, 1u << 30);
+                }
+                return grid_of[i] <= small_grid;
+            };
+            std::vector<bool> taken(drafts.size(), false);
+            for (int i = 0; i < (int)drafts.size() && small_grid > 0; ++i) {
+                if (taken[i] || !small(i)) continue;
+                std::vector<int> batch{i};
+                std::set<int> blocked, bound;
+                for (auto& o : drafts[i].outs) blocked.insert(o.node);
+                for (int nd : drafts[i].params) bound.insert(nd);
+                for (int j = i + 1; j < (int)drafts.size(); ++j) {
+                    if (!drafts[j].alive || taken[j]) continue;
+                    bool depends = false;
+                    for (int nd : input_nodes(drafts[j]))
+                        if (blocked.count(nd)) depends = true;
+                    std::set<int> would = bound;
+                    for (int nd : drafts[j].params) would.insert(nd);
+                    if (!depends && batch.size() < 16 && would.size() <= 48 && small(j)) {
+                        batch.push_back(j);
+                        bound = would;
+                    }
+                    for (auto& o : drafts[j].outs) blocked.insert(o.node);
+                }
+                if (batch.size() < 2) continue;
+                Draft multi;
+                multi.fk.main = drafts[i].fk.main;
+                std::set<int> seen;
+                for (int j : batch) {
+                    const Draft& d = drafts[j];
+                    std::vector<int> map;
+                    for (size_t p = 0; p < d.params.size(); ++p) map.push_back(param_index(multi, d.params[p], d.fk.buffer_is_output[p]));
+                    multi.fk.parts.push_back(d.fk);
+                    multi.fk.part_params.push_back(map);
+                    for (int nd : input_nodes(d))
+                        if (seen.insert(nd).second) multi.part_inputs.push_back(nd);
+                    for (size_t o = 0; o < d.outs.size(); ++o) {
+                        multi.outs.push_back(d.outs[o]);
+                        multi.fk.outputs.push_back(param_index(multi, d.outs[o].node, true));
+                    }
+                    multi.covers.insert(multi.covers.end(), d.covers.begin(), d.covers.end());
+                }
+                for (int j : batch) {
+                    taken[j] = true;
+                    drafts[j].alive = false;
+                }
+                drafts[i] = multi;
+                taken[i] = true;
+            }
         }
     }
 
