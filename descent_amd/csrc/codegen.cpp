@@ -378,8 +378,9 @@ string entry_name(const FusedKernel& fk) {
         if (fk.has_epilogue) base += "_epilogue";
         return base + "_b" + count(g.batch) + "_m" + count(g.m) + "_n" + count(g.n) + "_k" + count(g.k);
     }
-    case DSC_KERNEL_UNPAD: return "dsc_unpad_n" + count(element_count(d.shape));
-    case DSC_KERNEL_WINDOWS_TO_IMAGE: return "dsc_windows_to_image_n" + count(element_count(d.shape));
+    case DSC_KERNEL_UNPAD: return string(fk.has_epilogue ? "dsc_unpad_epilogue_n" : "dsc_unpad_n") + count(element_count(d.shape));
+    case DSC_KERNEL_WINDOWS_TO_IMAGE:
+        return string(fk.has_epilogue ? "dsc_windows_to_image_epilogue_n" : "dsc_windows_to_image_n") + count(element_count(d.shape));
     case DSC_KERNEL_SCATTER_ADD: return "dsc_scatter_add_n" + count(element_count(d.inputs[0].out_shape));
     default: return "dsc_kernel";
     }
@@ -406,6 +407,44 @@ string check_sizes(const FusedKernel& fk) {
     if (fk.has_epilogue) return chk(fk.epilogue.raw());
     return "";
 }
+
+// The store of one result of a kernel that takes a fused per-element consumer (Reduce, WindowsToImage, Unpad):
+// plain, or through the consumer cluster (emitted once as a device function).
+struct ResultStore {
+    Emitter& em;
+    int n_res = 1;
+    explicit ResultStore(Emitter& e) : em(e) {
+        const FusedKernel& fk = em.fk;
+        if (!fk.has_epilogue) return;
+        const dsc_kernel_desc& pe = fk.epilogue.raw();
+        n_res = pe.n_outputs;
+        std::ostringstream body;
+        std::map<int, string> ov;
+        ov[fk.epilogue_product_input] = "product";
+        em.emit_pe(body, pe, fk.epilogue_inputs, "gid", "e", ov);
+        for (int o = 0; o < pe.n_outputs; ++o) body << "    result[" << o << "] = et" << pe.outputs[o] << ";\n";
+        em.funcs << "DSC_INLINE void result_epilogue(float product, int gid, float* result, " << em.params_decl() << ") {\n"
+                 << body.str() << "}\n";
+    }
+    string one(const string& value, const string& oid) const {
+        const FusedKernel& fk = em.fk;
+        if (!fk.has_epilogue) return "b" + to_string(fk.outputs[0]) + "[" + oid + "] = " + value + ";";
+        string t = "{ float res[" + to_string(n_res) + "]; result_epilogue(" + value + ", (int)(" + oid + "), res, " + em.params_pass() + ");";
+        for (int o = 0; o < n_res; ++o) t += " b" + to_string(fk.outputs[o]) + "[" + oid + "] = res[" + to_string(o) + "];";
+        return t + " }";
+    }
+    string four(const string& value4, const string& oid) const {
+        const FusedKernel& fk = em.fk;
+        if (!fk.has_epilogue) return "*(float4*)(b" + to_string(fk.outputs[0]) + " + " + oid + ") = " + value4 + ";";
+        string t = "{ const float pv[4] = {" + value4 + ".x, " + value4 + ".y, " + value4 + ".z, " + value4 + ".w}; float res[4][" +
+                   to_string(n_res) + "];\n#pragma unroll\n        for (int j = 0; j < 4; ++j) result_epilogue(pv[j], (int)(" + oid +
+                   ") + j, res[j], " + em.params_pass() + ");";
+        for (int o = 0; o < n_res; ++o)
+            t += " *(float4*)(b" + to_string(fk.outputs[o]) + " + " + oid + ") = make_float4(res[0][" + to_string(o) + "], res[1][" +
+                 to_string(o) + "], res[2][" + to_string(o) + "], res[3][" + to_string(o) + "]);";
+        return t + " }";
+    }
+};
 
 unsigned blocks_for(int64_t threads, int block) { return (unsigned)((threads + block - 1) / block); }
 
@@ -492,34 +531,9 @@ string gen_reduce(Emitter& em, Generated* out) {
     const string init = is_max ? "U2F(0xff800000u)" : "0.f";
     auto combine = [&](const string& a, const string& b) { return is_max ? "glsl_max(" + a + ", " + b + ")" : a + " + " + b; };
 
-    // the store of one result: plain, or through the fused per-element consumer
-    const int n_res = fk.has_epilogue ? fk.epilogue.raw().n_outputs : 1;
-    if (fk.has_epilogue) {
-        const dsc_kernel_desc& pe = fk.epilogue.raw();
-        std::ostringstream body;
-        std::map<int, string> ov;
-        ov[fk.epilogue_product_input] = "product";
-        em.emit_pe(body, pe, fk.epilogue_inputs, "gid", "e", ov);
-        for (int o = 0; o < pe.n_outputs; ++o) body << "    result[" << o << "] = et" << pe.outputs[o] << ";\n";
-        em.funcs << "DSC_INLINE void red_epilogue(float product, int gid, float* result, " << em.params_decl() << ") {\n"
-                 << body.str() << "}\n";
-    }
-    auto store_one = [&](const string& value, const string& oid) {
-        if (!fk.has_epilogue) return "b" + to_string(fk.outputs[0]) + "[" + oid + "] = " + value + ";";
-        string t = "{ float res[" + to_string(n_res) + "]; red_epilogue(" + value + ", (int)(" + oid + "), res, " + em.params_pass() + ");";
-        for (int o = 0; o < n_res; ++o) t += " b" + to_string(fk.outputs[o]) + "[" + oid + "] = res[" + to_string(o) + "];";
-        return t + " }";
-    };
-    auto store_four = [&](const string& value4, const string& oid) {
-        if (!fk.has_epilogue) return "*(float4*)(b" + to_string(fk.outputs[0]) + " + " + oid + ") = " + value4 + ";";
-        string t = "{ const float pv[4] = {" + value4 + ".x, " + value4 + ".y, " + value4 + ".z, " + value4 + ".w}; float res[4][" +
-                   to_string(n_res) + "];\n#pragma unroll\n        for (int j = 0; j < 4; ++j) red_epilogue(pv[j], (int)(" + oid +
-                   ") + j, res[j], " + em.params_pass() + ");";
-        for (int o = 0; o < n_res; ++o)
-            t += " *(float4*)(b" + to_string(fk.outputs[o]) + " + " + oid + ") = make_float4(res[0][" + to_string(o) + "], res[1][" +
-                 to_string(o) + "], res[2][" + to_string(o) + "], res[3][" + to_string(o) + "]);";
-        return t + " }";
-    };
+    const ResultStore store(em);
+    auto store_one = [&](const string& value, const string& oid) { return store.one(value, oid); };
+    auto store_four = [&](const string& value4, const string& oid) { return store.four(value4, oid); };
 
     // is the reduced axis the one that walks memory fastest?
     bool k_fastest = false;
@@ -707,11 +721,11 @@ string gen_unpad(Emitter& em, Generated* out) {
     ic[d.axis] = "kc";
     k << "        const float w = " << em.load_view(fk.inputs[0], v, ic) << ";\n";
     k << "        sum += (kk >= k_min && kk <= k_max) ? w : 0.f;\n    }\n";
-    k << "    b" << fk.outputs[0] << "[gid] = sum;\n}\n";
+    k << "    " << ResultStore(em).one("sum", "gid") << "\n}\n";
     out->grid = blocks_for(n, 256);
     out->block = 256;
     out->source = k.str();
-    out->note = "unpad";
+    out->note = fk.has_epilogue ? "unpad +epilogue" : "unpad";
     return "";
 }
 
@@ -750,11 +764,11 @@ string gen_windows_to_image(Emitter& em, Generated* out) {
     ic[bd] = "oyc"; ic[bd + 1] = "oxc"; ic[bd + 2] = "group_index"; ic[bd + 3] = "fyc"; ic[bd + 4] = "fxc"; ic[bd + 5] = "group_c";
     k << "        const float w = " << em.load_view(fk.inputs[0], v, ic) << ";\n";
     k << "        tmp += ok ? w : 0.f;\n    }\n";
-    k << "    b" << fk.outputs[0] << "[gid] = tmp;\n}\n";
+    k << "    " << ResultStore(em).one("tmp", "gid") << "\n}\n";
     out->grid = blocks_for(n, 256);
     out->block = 256;
     out->source = k.str();
-    out->note = "windows_to_image";
+    out->note = fk.has_epilogue ? "windows_to_image +epilogue" : "windows_to_image";
     return "";
 }
 
@@ -1386,7 +1400,9 @@ static std::string generate_one(const FusedKernel& fk, Generated* out, bool with
     if (fk.has_epilogue) {
         err = validate(fk.epilogue.raw());
         if (!err.empty()) return "epilogue: " + err;
-        if (fk.main.raw().kind != DSC_KERNEL_MATMUL && fk.main.raw().kind != DSC_KERNEL_REDUCE) return "only MatMul and Reduce take an epilogue";
+        const int mk = fk.main.raw().kind;
+        if (mk != DSC_KERNEL_MATMUL && mk != DSC_KERNEL_REDUCE && mk != DSC_KERNEL_WINDOWS_TO_IMAGE && mk != DSC_KERNEL_UNPAD)
+            return "this kernel kind takes no epilogue";
     }
     for (auto& st : fk.row_stages) {
         err = validate(st.k.raw());

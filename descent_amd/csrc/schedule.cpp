@@ -4,6 +4,7 @@
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <set>
 #include <sstream>
 
@@ -161,6 +162,43 @@ int64_t draft_reads(const Draft& d) {  // how many elements the main kernel eval
     case DSC_KERNEL_SCATTER_ADD: return element_count(m.inputs[0].out_shape);
     default: return element_count(m.shape);
     }
+}
+
+// Linear index into a view's input for integer output coordinates; the view must need no clamp.
+int64_t view_index(const dsc_view& v, const int64_t* coord) {
+    int64_t st[DSC_MAX_DIM], in[DSC_MAX_DIM];
+    strides_of(v.in_shape, st);
+    for (int i = 0; i < v.in_shape.rank; ++i) in[i] = v.in_offset[i];
+    for (int j = 0; j < v.out_shape.rank; ++j)
+        if (v.map_axis[j] >= 0) in[v.map_axis[j]] += v.map_step[j] * coord[j];
+    int64_t idx = 0;
+    for (int i = 0; i < v.in_shape.rank; ++i) idx += in[i] * st[i];
+    return idx;
+}
+
+dsc_pe_op pe_op(int kind, int op = 0, int a0 = 0, int a1 = 0, int a2 = 0, int a3 = 0) {
+    dsc_pe_op o{};
+    o.kind = kind;
+    o.op = op;
+    o.args[0] = a0; o.args[1] = a1; o.args[2] = a2; o.args[3] = a3;
+    return o;
+}
+dsc_pe_op pe_literal(float value) {
+    dsc_pe_op o = pe_op(DSC_PE_LITERAL_F32);
+    std::memcpy(&o.bits, &value, 4);
+    return o;
+}
+dsc_view identity_view(std::initializer_list<int64_t> dims) {
+    dsc_view v{};
+    v.in_shape.rank = v.out_shape.rank = (int)dims.size();
+    int i = 0;
+    for (int64_t d : dims) {
+        v.in_shape.dims[i] = v.out_shape.dims[i] = d;
+        v.map_axis[i] = d > 1 ? i : -1;
+        v.map_step[i] = d > 1 ? 1 : 0;
+        ++i;
+    }
+    return v;
 }
 
 }  // namespace
@@ -475,6 +513,183 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             }
         }
 
+        // Pass 1c: the data gradient of a stride-1 convolution arrives as MatMul (dC x filter^T, one row of
+        // fh*fw*c window elements per output pixel) -> reshape copy -> WindowsToImage (sum of the windows that
+        // cover each pixel of the padded image).  With few channels that is the product written out nine times
+        // over and read back.  Run it as one MatMul over the padded image instead: row = padded pixel,
+        // k = (fy, fx, oc), A'[pixel, k] = dC[pixel - tap, oc] where that output pixel exists (else 0),
+        // B'[k, c] = filter[oc, fy, fx, c]; both operands are fused producers of the MatMul, nothing in between
+        // is written.
+        for (int i = 0; i < (int)drafts.size(); ++i) {
+            static const bool enabled = !(std::getenv("DSC_FUSE_DGRAD") && std::getenv("DSC_FUSE_DGRAD")[0] == '0');
+            if (!enabled) break;
+            Draft& mm = drafts[i];
+            const dsc_kernel_desc& md = mm.fk.main.raw();
+            if (!mm.alive || md.kind != DSC_KERNEL_MATMUL || !mm.fk.virtuals.empty() || mm.fk.has_epilogue || mm.keep_split ||
+                md.output_mode != DSC_MATMUL_BATCHES)
+                continue;
+            const MatMulDims g = matmul_dims(md);
+            if (g.chunks != 1 || is_graph_output[mm.outs[0].node] || mm.outs[0].copy_from >= 0) continue;
+            auto cons = consumers_of(mm.outs[0].node);
+            if (cons.size() != 1 || cons[0] <= i) continue;
+            int copy_idx = -1, w_idx = cons[0];
+            {
+                const Draft& c = drafts[w_idx];
+                const dsc_kernel_desc& cd = c.fk.main.raw();
+                if (cd.kind == DSC_KERNEL_PER_ELEMENT) {
+                    if (!c.fk.virtuals.empty() || c.fk.has_epilogue || cd.n_outputs != 1 || cd.n_inputs != 1 || cd.n_ops > 2 ||
+                        cd.ops[0].kind != DSC_PE_LOAD || (cd.n_ops == 2 && !(cd.ops[1].kind == DSC_PE_UNARY && cd.ops[1].op == DSC_UN_MOV)) ||
+                        any_clamp(cd.inputs[0]) || is_graph_output[c.outs[0].node] || c.outs[0].copy_from >= 0)
+                        continue;
+                    auto cons2 = consumers_of(c.outs[0].node);
+                    if (cons2.size() != 1 || cons2[0] <= w_idx) continue;
+                    copy_idx = w_idx;
+                    w_idx = cons2[0];
+                }
+            }
+            Draft& w = drafts[w_idx];
+            const dsc_kernel_desc& wd = w.fk.main.raw();
+            if (wd.kind != DSC_KERNEL_WINDOWS_TO_IMAGE || !w.fk.virtuals.empty() || w.fk.has_epilogue || wd.stride_w != 1 || wd.stride_h != 1 ||
+                wd.shape.rank != 4 || w.outs[0].copy_from >= 0 || any_clamp(wd.inputs[0]))
+                continue;
+            const dsc_view& wv = wd.inputs[0];
+            const int64_t IMG = wv.out_shape.dims[0], OH = wv.out_shape.dims[1], OW = wv.out_shape.dims[2], G = wv.out_shape.dims[3];
+            const int64_t FH = wv.out_shape.dims[4], FW = wv.out_shape.dims[5], C = wv.out_shape.dims[6];
+            const int64_t PH = OH + FH - 1, PW = OW + FW - 1, K = g.k;
+            if (g.batch != G || g.m != IMG * OH * OW || g.n != FH * FW * C) continue;
+            // worth it where the row-per-thread kernel runs: few channels on both sides
+            if (C > 32 || FH * FW * K > 256 || FH * FW * K * C > 8192 || FH * FW < 2) continue;
+            if (IMG * PH * PW * G * FH * FW * K >= ((int64_t)1 << 31)) continue;
+            // the chain must hand element (img, oy, ox, g, fy, fx, c) of the windows exactly product element
+            // [g][(img, oy, ox)][(fy, fx, c)]: checked on every window element of the first, middle and last image
+            bool chain_ok = true;
+            for (int64_t img : {(int64_t)0, IMG / 2, IMG - 1}) {
+                for (int64_t rest = 0; rest < OH * OW * G * FH * FW * C && chain_ok; ++rest) {
+                    int64_t c7[7], r = rest;
+                    c7[6] = r % C; r /= C;
+                    c7[5] = r % FW; r /= FW;
+                    c7[4] = r % FH; r /= FH;
+                    c7[3] = r % G; r /= G;
+                    c7[2] = r % OW; r /= OW;
+                    c7[1] = r;
+                    c7[0] = img;
+                    int64_t idx = view_index(wv, c7);
+                    if (copy_idx >= 0) {
+                        const dsc_view& cv = drafts[copy_idx].fk.main.raw().inputs[0];
+                        int64_t cc[DSC_MAX_DIM], q = idx;
+                        for (int a = cv.out_shape.rank - 1; a >= 0; --a) {
+                            cc[a] = q % cv.out_shape.dims[a];
+                            q /= cv.out_shape.dims[a];
+                        }
+                        idx = view_index(cv, cc);
+                    }
+                    const int64_t want = c7[3] * g.m * g.n + ((img * OH + c7[1]) * OW + c7[2]) * g.n + (c7[4] * FW + c7[5]) * C + c7[6];
+                    if (idx != want) chain_ok = false;
+                }
+            }
+            if (!chain_ok) continue;
+            if (taken_in_place_between(i, w_idx, input_nodes(mm))) continue;
+
+            const dsc_view va = md.inputs[0], vb = md.inputs[1];
+            const int64_t Mp = IMG * PH * PW, Kp = FH * FW * K;
+            // A': out [G, IMG, PH, PW, FH, FW, K] onto dC
+            dsc_view wa = va;
+            wa.out_shape.rank = 7;
+            const int64_t a_dims[7] = {G, IMG, PH, PW, FH, FW, K};
+            const int a_from[7] = {0, 1, 1, 1, 1, 1, 2};
+            const int64_t a_scale[7] = {1, OH * OW, OW, 1, -OW, -1, 1};
+            for (int j = 0; j < 7; ++j) {
+                wa.out_shape.dims[j] = a_dims[j];
+                wa.map_axis[j] = va.map_axis[a_from[j]];
+                wa.map_step[j] = va.map_axis[a_from[j]] >= 0 ? va.map_step[a_from[j]] * a_scale[j] : 0;
+            }
+            auto coord_view = [&](int pos_axis, int tap_axis, int64_t extent, int64_t taps) {
+                dsc_view v{};
+                v.in_shape.rank = 1;
+                v.in_shape.dims[0] = extent + 2 * taps - 2;
+                v.in_offset[0] = taps - 1;
+                v.out_shape = wa.out_shape;
+                for (int j = 0; j < 7; ++j) { v.map_axis[j] = -1; v.map_step[j] = 0; }
+                v.map_axis[pos_axis] = 0; v.map_step[pos_axis] = 1;
+                v.map_axis[tap_axis] = 0; v.map_step[tap_axis] = -1;
+                return v;
+            };
+            const dsc_view builtin[2] = {coord_view(2, 4, OH, FH), coord_view(3, 5, OW, FW)};
+            const dsc_pe_op a_ops[12] = {
+                pe_op(DSC_PE_LOAD), pe_op(DSC_PE_COORD), pe_op(DSC_PE_COORD),
+                pe_literal((float)(FH - 2)), pe_literal((float)(OH + FH - 1)), pe_literal((float)(FW - 2)), pe_literal((float)(OW + FW - 1)),
+                pe_literal(0.f),
+                pe_op(DSC_PE_SELECT, DSC_CMP_GT, 1, 3, 0, 7), pe_op(DSC_PE_SELECT, DSC_CMP_GT, 4, 1, 8, 7),
+                pe_op(DSC_PE_SELECT, DSC_CMP_GT, 2, 5, 9, 7), pe_op(DSC_PE_SELECT, DSC_CMP_GT, 6, 2, 10, 7)};
+            dsc_pe_op a_ops_m[12];
+            std::memcpy(a_ops_m, a_ops, sizeof a_ops);
+            a_ops_m[2].view_index = 1;
+            const int32_t a_out = 11;
+            dsc_kernel_desc ad{};
+            ad.kind = DSC_KERNEL_PER_ELEMENT;
+            ad.shape.rank = 1;
+            ad.shape.dims[0] = G * Mp * Kp;
+            ad.n_inputs = 1; ad.inputs = &wa;
+            ad.n_ops = 12; ad.ops = a_ops_m;
+            ad.n_outputs = 1; ad.outputs = &a_out;
+            ad.n_builtin_views = 2; ad.builtin_views = builtin;
+            // B': out [G, FH, FW, K, C] onto the filter operand
+            dsc_view wb = vb;
+            wb.out_shape.rank = 5;
+            const int64_t b_dims[5] = {G, FH, FW, K, C};
+            const int b_from[5] = {0, 2, 2, 1, 2};
+            const int64_t b_scale[5] = {1, FW * C, C, 1, 1};
+            for (int j = 0; j < 5; ++j) {
+                wb.out_shape.dims[j] = b_dims[j];
+                wb.map_axis[j] = vb.map_axis[b_from[j]];
+                wb.map_step[j] = vb.map_axis[b_from[j]] >= 0 ? vb.map_step[b_from[j]] * b_scale[j] : 0;
+            }
+            for (int j = 5; j < DSC_MAX_DIM; ++j) { wb.out_shape.dims[j] = 0; wb.map_axis[j] = -1; wb.map_step[j] = 0; }
+            const dsc_pe_op b_ops[1] = {pe_op(DSC_PE_LOAD)};
+            const int32_t b_out = 0;
+            dsc_kernel_desc bd{};
+            bd.kind = DSC_KERNEL_PER_ELEMENT;
+            bd.shape.rank = 1;
+            bd.shape.dims[0] = G * Kp * C;
+            bd.n_inputs = 1; bd.inputs = &wb;
+            bd.n_ops = 1; bd.ops = b_ops;
+            bd.n_outputs = 1; bd.outputs = &b_out;
+            // the MatMul over the padded image, Rows mode: C[(img, py, px)][g][c]
+            const dsc_view m_in[2] = {identity_view({G, Mp, Kp}), identity_view({G, Kp, C})};
+            dsc_kernel_desc nd{};
+            nd.kind = DSC_KERNEL_MATMUL;
+            nd.shape.rank = 4;
+            nd.shape.dims[0] = 1; nd.shape.dims[1] = Mp; nd.shape.dims[2] = G; nd.shape.dims[3] = C;
+            nd.output_mode = DSC_MATMUL_ROWS;
+            nd.n_inputs = 2; nd.inputs = m_in;
+            if (!validate(ad).empty() || !validate(bd).empty() || !validate(nd).empty()) continue;
+
+            Draft fused;
+            fused.fk.main = KernelDesc(nd);
+            Virtual va_v, vb_v;
+            va_v.pe = KernelDesc(ad);
+            va_v.out_op = a_out;
+            va_v.inputs.push_back(Source{param_index(fused, mm.params[mm.fk.inputs[0].buffer], false), -1});
+            vb_v.pe = KernelDesc(bd);
+            vb_v.out_op = b_out;
+            vb_v.inputs.push_back(Source{param_index(fused, mm.params[mm.fk.inputs[1].buffer], false), -1});
+            fused.fk.virtuals.push_back(va_v);
+            fused.fk.virtuals.push_back(vb_v);
+            Source sa, sb;
+            sa.virt = 0;
+            sb.virt = 1;
+            fused.fk.inputs = {sa, sb};
+            fused.fk.outputs.push_back(param_index(fused, w.outs[0].node, true));
+            fused.outs.push_back(w.outs[0]);
+            fused.covers = mm.covers;
+            if (copy_idx >= 0) fused.covers.insert(fused.covers.end(), drafts[copy_idx].covers.begin(), drafts[copy_idx].covers.end());
+            fused.covers.insert(fused.covers.end(), w.covers.begin(), w.covers.end());
+            compact(fused);
+            mm.alive = false;
+            if (copy_idx >= 0) drafts[copy_idx].alive = false;
+            drafts[w_idx] = fused;
+        }
+
         // Pass 1b: clusters that all work on the rows of one [m, n] array with a short n -- Reduces along n and the
         // per-element clusters around them (softmax cross-entropy: row max, exp, row sum, log-probability, gradient,
         // per-row loss; the accuracy count: arg-max and comparison with the label) -- become one row-fused launch.
@@ -694,12 +909,15 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             }
         }
 
-        // Pass 3: a Reduce whose only consumer is a per-element cluster over its outputs (a scalar accumulated into
-        // a running sum, the optimiser update of a bias gradient) applies that cluster to each result before the
-        // store.
+        // Pass 3: a Reduce, WindowsToImage or Unpad whose only consumer is a per-element cluster over its outputs (a
+        // scalar accumulated into a running sum, the optimiser update of a bias gradient, the activation derivative
+        // applied to a pooling gradient) applies that cluster to each result before the store.
         for (int i = 0; i < (int)drafts.size(); ++i) {
             Draft& r = drafts[i];
-            if (!r.alive || r.fk.main.raw().kind != DSC_KERNEL_REDUCE || r.fk.has_epilogue || r.keep_output || !r.fk.row_stages.empty()) continue;
+            const int rk = r.fk.main.raw().kind;
+            if (!r.alive || (rk != DSC_KERNEL_REDUCE && rk != DSC_KERNEL_WINDOWS_TO_IMAGE && rk != DSC_KERNEL_UNPAD) || r.fk.has_epilogue ||
+                r.keep_output || !r.fk.row_stages.empty())
+                continue;
             int pe_idx = -1, pe_input = -1;
             find_epilogue(i, r.outs[0].node, element_count(r.fk.main.raw().shape), &pe_idx, &pe_input);
             if (pe_idx < 0) continue;

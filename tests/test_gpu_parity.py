@@ -224,3 +224,65 @@ def test_gather_indices_are_bit_exact(hip_backend_session):
     ci, cv = run(cenv)
     assert np.array_equal(gi, ci) and gi.max() < 2048
     assert np.array_equal(gv.view(np.uint32), cv.view(np.uint32))
+
+
+def _softmax_case(env, m, n, seed, quantised):
+    """Logits as a trainable parameter: per-row loss, d loss / d logits and the per-row accuracy flag."""
+    from descent_amd import Initializer
+    from descent_amd.loss import softmax_cross_entropy_accuracy, softmax_cross_entropy_loss
+
+    rng = np.random.default_rng(seed)
+    z = rng.standard_normal((m, n), dtype=np.float32) * 3
+    if quantised:  # repeated maxima in a row: the arg-max tie rule decides the accuracy flag
+        z = np.round(z)
+    zp = env.trainable_parameter([m, n], "z", Initializer.zero())
+    yp = env.static_parameter_with_data([m, 1], "y", rng.integers(0, n, (m, 1)).astype(np.float32))
+    env.write_parameter(zp, z)
+    loss_rows, acc_rows, dz = env.static_parameter([m, 1], "l"), env.static_parameter([m, 1], "a"), env.static_parameter([m, n], "dz")
+
+    def build(s):
+        zd = s.parameter(zp)
+        loss = softmax_cross_entropy_loss(zd, yp).set_loss()
+        s.write_parameter_value(loss_rows, loss)
+        s.write_parameter_value(acc_rows, softmax_cross_entropy_accuracy(zd, yp))
+        s.write_parameter_value(dz, zd.loss_grad())
+
+    g = env.build_graph(build)
+    env.run(g, 0)
+    return g, env.read_parameter(loss_rows), env.read_parameter(acc_rows), env.read_parameter(dz)
+
+
+@pytest.mark.parametrize("m,n", [(1000, 10), (37, 3), (64, 64), (5, 33), (4097, 2), (300, 17)])
+@pytest.mark.parametrize("quantised", [False, True])
+def test_softmax_cross_entropy_runs_as_one_row_fused_launch(hip_backend_session, m, n, quantised):
+    genv, cenv = _envs(hip_backend_session)
+    g, gl, ga, gdz = _softmax_case(genv, m, n, 31 + m + n, quantised)
+    _, cl, ca, cdz = _softmax_case(cenv, m, n, 31 + m + n, quantised)
+    listing = next(iter(g.__dict__["_schedules"].values())).describe()
+    assert "RowFused [%d, %d]" % (m, n) in listing and int(listing.split()[0]) <= 2, listing
+    assert rel_l2(gl, cl) <= TOL and rel_l2(gdz, cdz) <= TOL
+    assert np.array_equal(ga, ca)  # arg-max derived: exact, ties included
+
+
+def test_convnet_step_at_batch_64_vs_oracle(hip_backend_session):
+    """At this batch the convolution GEMMs are large enough for the row-per-thread kernels, among them the fused
+    data gradient of the second convolution (MatMul + reshape copy + WindowsToImage as one product over the
+    padded image): two Adam steps, every parameter and optimiser state."""
+    from descent_amd import workloads
+
+    genv, cenv = _envs(hip_backend_session)
+    gw = workloads.convnet(genv, batch=64, seed=13)
+    cw = workloads.convnet(cenv, batch=64, seed=13)
+    listing = None
+    for step in range(2):
+        genv.run(gw.graph, 500 + step)
+        cenv.run(cw.graph, 500 + step)
+    listing = next(iter(gw.graph.__dict__["_schedules"].values())).describe()
+    assert "MatMul (k=144) [1, 16384, 2, 8] <2 fused producers>  [row-per-thread" in listing, listing
+    got, want = gw.snapshot(), cw.snapshot()
+    for key in want:
+        if key == "accuracy":
+            assert np.array_equal(got[key], want[key]), key
+        else:
+            err = rel_l2(got[key], want[key])
+            assert err <= TOL, f"{key}: rel L2 {err}"

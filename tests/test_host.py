@@ -162,7 +162,28 @@ def test_convnet_graph_shape():
     assert sum(p.shape.element_count() for p in w.trainable) == 204618
     listing = hip_backend.check_schedule(w.graph, fused=True)
     launches = int(listing.split()[0])
-    assert launches < 55, listing
+    assert launches < 40, listing
+    # softmax cross-entropy and the accuracy count: one row-fused launch over the [1000, 10] logits
+    assert "RowFused [1000, 10] (8 clusters)" in listing
+    # small independent launches (optimiser updates of small tensors, short reductions) share launches
+    assert listing.count("Multi (") >= 3
+    # every reference cluster is covered exactly once, except producers inlined into several consumers
+    covered = [int(c) for line in listing.splitlines() if " clusters " in line for c in line.split(" clusters ")[1].split()]
+    assert set(covered) == set(range(66))
+    # the data gradient of the second convolution: MatMul + reshape copy + WindowsToImage as one product over
+    # the padded image, both operands fused producers
+    assert "MatMul (k=144) [1, 256000, 2, 8] <2 fused producers>" in listing
+    # the work figures of the listing: the eleven GEMMs of the step as the reference runs them
+    assert "4.373 GFLOP in MatMuls" in hip_backend.check_schedule(w.graph, fused=False)
+
+
+def test_work_figures_of_the_headline_matmul():
+    env = _env()
+    w = workloads.matmul_epilogue(env, 8192, 8192, 8192, upload=False)
+    listing = hip_backend.check_schedule(w.graph, fused=True)
+    assert int(listing.split()[0]) == 1
+    # 4 * (M*K + K*N + N + M*N) bytes and 2*M*N*K flops
+    assert "805.339 MB moved, 1099.512 GFLOP" in listing, listing
 
 
 def test_fused_and_unfused_schedules_compile_for_every_config():
