@@ -18,6 +18,7 @@ KIND_FILL, KIND_PER_ELEMENT, KIND_REDUCE, KIND_MATMUL, KIND_UNPAD, KIND_W2I, KIN
 (PE_LOAD, PE_LITERAL_F32, PE_LITERAL_U32, PE_COORD, PE_RAND, PE_UNARY, PE_BINARY, PE_SELECT, PE_GATHER) = range(9)
 
 SCHEDULE_NO_FUSION = 1
+SCHEDULE_NO_CONV_KERNELS = 2
 
 
 class CShape(C.Structure):

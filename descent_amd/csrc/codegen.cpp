@@ -62,13 +62,14 @@ struct Emitter {
         s += "uint rand_seed";
         return s;
     }
-    // The __global__ signature: the seed arrives through a one-word device cell so that a captured launch
-    // sequence can be replayed with a new seed without touching its kernel arguments.
+    // The __global__ signature: the seed arrives by value, or -- when seed_cell is not null -- through a one-word
+    // device cell, so that a captured launch sequence can be replayed with a new seed without touching its
+    // kernel arguments.
     string kernel_params_decl() const {
         string s;
         for (int i = 0; i < fk.n_buffers; ++i)
             s += (fk.buffer_is_output[i] ? "float* __restrict__ b" : "const float* __restrict__ b") + to_string(i) + ", ";
-        return s + "const uint* __restrict__ seed_cell";
+        return s + "const uint* __restrict__ seed_cell, const uint seed_value";
     }
     string params_pass() const {
         string s;
@@ -364,6 +365,11 @@ bool tallk_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
 string entry_name(const FusedKernel& fk) {
     const dsc_kernel_desc& d = fk.main.raw();
     auto count = [](int64_t v) { return to_string((long long)v); };
+    if (fk.dgrad.on) {
+        const MatMulDims g = matmul_dims(d);
+        return "dsc_conv_dgrad_img" + count(fk.dgrad.img) + "_" + count(fk.dgrad.oh) + "x" + count(fk.dgrad.ow) + "_g" + count(fk.dgrad.g) + "_k" +
+               count(g.k) + "_c" + count(fk.dgrad.c);
+    }
     if (!fk.row_stages.empty()) return "dsc_row_fused_m" + count(fk.row_m) + "_n" + count(fk.row_n) + "_s" + count((int64_t)fk.row_stages.size());
     switch (d.kind) {
     case DSC_KERNEL_FILL: return "dsc_fill_n" + count(d.shape.dims[0]);
@@ -455,7 +461,7 @@ string gen_fill(Emitter& em, Generated* out) {
     const int64_t n = d.shape.dims[0];
     std::ostringstream k;
     const bool vec = n % 4 == 0;
-    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = *seed_cell;\n";
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
     k << "    const uint i = blockIdx.x * 256u + threadIdx.x;\n";
     if (vec) {
         k << "    if (i >= " << S(n / 4) << "u) return;\n";
@@ -479,7 +485,7 @@ string gen_per_element(Emitter& em, Generated* out) {
     const int64_t n = d.shape.dims[0];
     const int vec = (n % 4 == 0 && n >= 4096) ? 4 : 1;
     std::ostringstream k;
-    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = *seed_cell;\n";
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
     k << "    const uint base = (blockIdx.x * 256u + threadIdx.x) * " << vec << "u;\n";
     k << "    if (base >= " << S(n) << "u) return;\n";
     std::map<int, string> override_load;
@@ -557,7 +563,7 @@ string gen_reduce(Emitter& em, Generated* out) {
     }
 
     std::ostringstream k;
-    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = *seed_cell;\n";
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
     // The k loop runs over groups of U independent accumulators: the U loads of a group are issued before any of
     // them is used, with no bounds test in between (a test per load would be a branch per load, and the loads
     // would be issued one at a time).  What is left over is handled by groups of U/2, U/4, .. 1.
@@ -706,7 +712,7 @@ string gen_unpad(Emitter& em, Generated* out) {
     const dsc_view& v = d.inputs[0];
     const int64_t n = element_count(d.shape);
     std::ostringstream k;
-    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = *seed_cell;\n";
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
     k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n";
     auto c = em.emit_coords(k, d.shape, "gid", "c");
     const string oc = c[d.axis];
@@ -740,7 +746,7 @@ string gen_windows_to_image(Emitter& em, Generated* out) {
     const int bd = d.shape.rank - 3;
     const int64_t n = element_count(d.shape);
     std::ostringstream k;
-    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = *seed_cell;\n";
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
     k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n";
     auto c = em.emit_coords(k, d.shape, "gid", "c");
     k << "    const int in_y = " << c[bd] << ", in_x = " << c[bd + 1] << ", in_c = " << c[bd + 2] << ";\n";
@@ -779,7 +785,7 @@ string gen_scatter_add(Emitter& em, Generated* out) {
     const dsc_view& vi = d.inputs[1];
     const int64_t n = element_count(vv.out_shape);
     std::ostringstream k;
-    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = *seed_cell;\n";
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
     k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n";
     auto c = em.emit_coords(k, vv.out_shape, "gid", "c");
     k << "    const float value = " << em.load_view(fk.inputs[0], vv, c) << ";\n";
@@ -807,7 +813,7 @@ string gen_row_fused(Emitter& em, Generated* out) {
     const int64_t G = pow2_ceil(n), per_block = 256 / G;
     std::ostringstream k;
     k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
-    k << "    const uint rand_seed = *seed_cell;\n";
+    k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
     k << "    const int col = threadIdx.x % " << G << ";\n";
     k << "    const int row = blockIdx.x * " << per_block << " + threadIdx.x / " << G << ";\n";
     // lanes past the last row or column repeat a valid element's work (every lane takes part in the shuffles)
@@ -875,6 +881,126 @@ string gen_row_fused(Emitter& em, Generated* out) {
     return "";
 }
 
+// ---- convolution data gradient ---------------------------------------------------------------------------
+
+int64_t dgrad_pitch(int64_t k) { return k % 8 == 0 ? k + 4 : k; }  // keeps 16-byte reads of neighbouring pixels off one bank
+
+int64_t dgrad_lds_floats(const FusedKernel::ConvDgrad& c, int64_t k) {
+    const int64_t th = c.oh + 2 * (c.fh - 1), tw = c.ow + 2 * (c.fw - 1), ph = c.oh + c.fh - 1, pw = c.ow + c.fw - 1;
+    return std::max(th * tw * dgrad_pitch(k), (c.pad_h || c.pad_w) ? ph * pw * c.c : 0);
+}
+
+string gen_conv_dgrad(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const FusedKernel::ConvDgrad& cv = fk.dgrad;
+    const MatMulDims g = matmul_dims(d);
+    const int64_t K = g.k, G = cv.g, C = cv.c, FH = cv.fh, FW = cv.fw, OH = cv.oh, OW = cv.ow;
+    if (g.batch != G || g.m != cv.img * OH * OW || g.n != FH * FW * C || g.chunks != 1) return "conv dgrad: geometry mismatch";
+    const int64_t TH = OH + 2 * (FH - 1), TW = OW + 2 * (FW - 1), PH = OH + FH - 1, PW = OW + FW - 1;
+    const int64_t GC = G * C, PITCH = dgrad_pitch(K);
+    const int64_t H = PH - 2 * cv.pad_h, W = PW - 2 * cv.pad_w;
+    const bool unpad = cv.pad_h > 0 || cv.pad_w > 0;
+    if (H < 1 || W < 1 || K % 4 != 0) return "conv dgrad: unsupported geometry";
+    const int64_t lds = dgrad_lds_floats(cv, K);
+    if (lds * 4 > 64 * 1024) return "conv dgrad: image tile does not fit LDS";
+
+    const string la = em.load_view(fk.inputs[0], d.inputs[0], {"cb", "cm", "ck"});
+    em.funcs << "DSC_INLINE float load_a(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return " << la << ";\n}\n";
+    const string lb = em.load_view(fk.inputs[1], d.inputs[1], {"cb", "ck", "cn"});
+    em.funcs << "DSC_INLINE float load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb << ";\n}\n";
+
+    std::ostringstream k;
+    const string out_ptr = "b" + to_string(fk.outputs[0]);
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
+    k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
+    k << "    __shared__ __attribute__((aligned(16))) float lds[" << S(lds) << "];\n";
+    k << "    const int cb = blockIdx.x % " << S(G) << ", img = blockIdx.x / " << S(G) << ";\n";
+    // 1. dC of this image and group inside a halo of fh-1 / fw-1 zeros: tile[ty][tx][oc].  Groups of 8 loads are
+    // issued before any of them is stored: one memory round trip per group, not per element.
+    const int64_t fill_n = TH * TW * K;
+    k << "    for (int i0 = threadIdx.x; i0 < " << S(fill_n) << "; i0 += 2048) {\n        float v[8];\n";
+    k << "#pragma unroll\n        for (int u = 0; u < 8; ++u) {\n";
+    k << "            const int i = min(i0 + u * 256, " << S(fill_n - 1) << ");\n";
+    k << "            const int oc = i % " << S(K) << ", tx = (i / " << S(K) << ") % " << S(TW) << ", ty = i / " << S(K * TW) << ";\n";
+    k << "            const int oy = ty - " << S(FH - 1) << ", ox = tx - " << S(FW - 1) << ";\n";
+    k << "            v[u] = load_a(cb, (img * " << S(OH) << " + clampi(oy, 0, " << S(OH - 1) << ")) * " << S(OW) << " + clampi(ox, 0, "
+      << S(OW - 1) << "), oc, " << em.params_pass() << ");\n        }\n";
+    k << "        __builtin_amdgcn_sched_barrier(0);\n";
+    k << "#pragma unroll\n        for (int u = 0; u < 8; ++u) {\n";
+    k << "            const int i = i0 + u * 256;\n";
+    k << "            const int oc = i % " << S(K) << ", tx = (i / " << S(K) << ") % " << S(TW) << ", ty = i / " << S(K * TW) << ";\n";
+    k << "            const int oy = ty - " << S(FH - 1) << ", ox = tx - " << S(FW - 1) << ";\n";
+    k << "            const bool inside = oy >= 0 && oy < " << S(OH) << " && ox >= 0 && ox < " << S(OW) << ";\n";
+    k << "            if (i < " << S(fill_n) << ") lds[(ty * " << S(TW) << " + tx) * " << S(PITCH) << " + oc] = inside ? v[u] : 0.f;\n        }\n    }\n";
+    k << "    __syncthreads();\n";
+    // 2. one padded-image pixel per thread and pass: acc[c] over taps and output channels; the filter element is
+    // the same for every lane, so it comes through the scalar unit.  The tap loop stays a loop and each block of
+    // 8 channels is fenced: unrolled whole, the scheduler would hoist all the filter loads to the top and spill
+    // the scalar registers holding them.
+    const int64_t passes = (PH * PW + 255) / 256;
+    const int64_t OCB = K % 8 == 0 ? 8 : 4;
+    k << "    float acc[" << passes << "][" << S(C) << "];\n";
+    k << "#pragma unroll\n    for (int ps = 0; ps < " << passes << "; ++ps) {\n";
+    k << "        const int p = min(ps * 256 + (int)threadIdx.x, " << S(PH * PW - 1) << ");\n";
+    k << "        const int py = p / " << S(PW) << ", px = p % " << S(PW) << ";\n";
+    k << "#pragma unroll\n        for (int c = 0; c < " << S(C) << "; ++c) acc[ps][c] = 0.f;\n";
+    k << "#pragma unroll 1\n        for (int tap = 0; tap < " << S(FH * FW) << "; ++tap) {\n";
+    k << "            const int fy = tap / " << S(FW) << ", fx = tap % " << S(FW) << ";\n";
+    k << "            const float* src = &lds[((py + " << S(FH - 1) << " - fy) * " << S(TW) << " + (px + " << S(FW - 1) << " - fx)) * "
+      << S(PITCH) << "];\n";
+    k << "#pragma unroll\n            for (int oc = 0; oc < " << S(K) << "; oc += " << OCB << ") {\n";
+    k << "                float a[" << OCB << "];\n";
+    k << "#pragma unroll\n                for (int q = 0; q < " << OCB << "; q += 4) {\n";
+    k << "                    const float4 a4 = *(const float4*)(src + oc + q);\n";
+    k << "                    a[q] = a4.x; a[q + 1] = a4.y; a[q + 2] = a4.z; a[q + 3] = a4.w;\n                }\n";
+    k << "#pragma unroll\n                for (int j = 0; j < " << OCB << "; ++j)\n";
+    k << "#pragma unroll\n                    for (int c = 0; c < " << S(C) << "; ++c)\n";
+    k << "                        acc[ps][c] = fmaf(a[j], load_b(cb, oc + j, tap * " << S(C) << " + c, " << em.params_pass() << "), acc[ps][c]);\n";
+    k << "                __builtin_amdgcn_sched_barrier(0);\n";
+    k << "            }\n        }\n    }\n";
+    if (!unpad) {
+        k << "#pragma unroll\n    for (int ps = 0; ps < " << passes << "; ++ps) {\n";
+        k << "        const int p = ps * 256 + (int)threadIdx.x;\n        if (p < " << S(PH * PW) << ") {\n";
+        k << "#pragma unroll\n            for (int c = 0; c < " << S(C) << "; ++c) " << out_ptr << "[(img * " << S(PH * PW) << " + p) * " << S(GC)
+          << " + cb * " << S(C) << " + c] = acc[ps][c];\n        }\n    }\n}\n";
+    } else {
+        // 3. the padded-image gradient goes through LDS (the tile is dead by now); each pixel of the image then sums
+        // the padded pixels that replicate it: itself, plus the border rows / columns for pixels on the edge
+        k << "    __syncthreads();\n";
+        k << "#pragma unroll\n    for (int ps = 0; ps < " << passes << "; ++ps) {\n";
+        k << "        const int p = ps * 256 + (int)threadIdx.x;\n        if (p < " << S(PH * PW) << ") {\n";
+        k << "#pragma unroll\n            for (int c = 0; c < " << S(C) << "; ++c) lds[p * " << S(C) << " + c] = acc[ps][c];\n        }\n    }\n";
+        k << "    __syncthreads();\n";
+        k << "    for (int i = threadIdx.x; i < " << S(H * W * C) << "; i += 256) {\n";
+        k << "        const int c = i % " << S(C) << ", x = (i / " << S(C) << ") % " << S(W) << ", y = i / " << S(C * W) << ";\n";
+        k << "        float sum = 0.f;\n";
+        // candidate rows / columns: the pixel's own, and the border ones when it lies on the edge (as the Unpad
+        // kernel: k_min = in - (coord == 0 ? pad : 0), k_max = in + (coord == last ? pad : 0))
+        const string outer = cv.rows_first ? "jx" : "jy", inner = cv.rows_first ? "jy" : "jx";
+        auto range = [&](const string& j) {
+            const bool is_y = j == "jy";
+            return "for (int " + j + " = " + S(-(is_y ? cv.pad_h : cv.pad_w)) + "; " + j + " <= " + S(is_y ? cv.pad_h : cv.pad_w) + "; ++" + j + ")";
+        };
+        k << "#pragma unroll\n        " << range(outer) << " {\n            float part = 0.f;\n";
+        k << "#pragma unroll\n            " << range(inner) << " {\n";
+        k << "                const bool ok_y = jy == 0 || (jy < 0 && y == 0) || (jy > 0 && y == " << S(H - 1) << ");\n";
+        k << "                const bool ok_x = jx == 0 || (jx < 0 && x == 0) || (jx > 0 && x == " << S(W - 1) << ");\n";
+        k << "                const int ky = clampi(y + " << S(cv.pad_h) << " + jy, 0, " << S(PH - 1) << "), kx = clampi(x + " << S(cv.pad_w)
+          << " + jx, 0, " << S(PW - 1) << ");\n";
+        k << "                const float w = lds[(ky * " << S(PW) << " + kx) * " << S(C) << " + c];\n";
+        k << "                part += (ok_y && ok_x) ? w : 0.f;\n            }\n            sum += part;\n        }\n";
+        k << "        " << out_ptr << "[((img * " << S(H) << " + y) * " << S(W) << " + x) * " << S(GC) << " + cb * " << S(C) << " + c] = sum;\n    }\n}\n";
+    }
+    if (cv.img * G >= kMaxIndex) return "conv dgrad: grid too large";
+    out->grid = (unsigned)(cv.img * G);
+    out->block = 256;
+    out->source = k.str();
+    out->note = "conv data gradient: workgroup per image and group, tile in LDS, " + S(FH) + "x" + S(FW) + " taps x " + S(K) + " channels" +
+                (unpad ? ", border folds fused" : "");
+    return "";
+}
+
 // ---- matmul -------------------------------------------------------------------------------------------
 
 struct MmConfig {
@@ -897,7 +1023,7 @@ bool config_ok(const MmConfig& c) {
 // Largest tile whose grid still fills the 256 CUs; small products fall back to small tiles so that more
 // workgroups exist (they are latency bound, not MFMA bound).  Measured on MI355X at 8192^3: 256x256x16 with
 // 16 waves 137 TFLOP/s, 256x128x16 with 8 waves 134, 128x128x16 with 4 waves 127.
-MmConfig pick_config(int64_t M, int64_t N, int64_t groups /* batch * k-chunks */) {
+MmConfig pick_config(int64_t M, int64_t N, int64_t K /* per chunk */, int64_t groups /* batch * k-chunks */) {
     static const MmConfig candidates[] = {
         {256, 256, 16, 4, 4, 4}, {256, 128, 16, 4, 2, 4}, {128, 128, 16, 2, 2, 8}, {128, 64, 16, 2, 2, 8},
         {64, 64, 16, 2, 2, 8},   {64, 32, 16, 2, 1, 8},   {32, 32, 16, 1, 1, 8},
@@ -916,6 +1042,14 @@ MmConfig pick_config(int64_t M, int64_t N, int64_t groups /* batch * k-chunks */
     MmConfig c = best;
     // narrow outputs: keep all four waves along m
     if (c.bn == 32 && c.bm == 64) { c.wm = 2; c.wn = 1; }
+    // Small tiles mean a small, latency-bound product: every k-tile costs one round trip to memory, so take k in
+    // fewer, deeper steps (more bytes in flight per step; LDS has room to spare at these tile sizes).
+    if (const char* e = std::getenv("DSC_MM_DEEP_K")) {
+        if (e[0] != '0') {
+            const int deep = c.bm * c.bn <= 64 * 64 ? 64 : (c.bm * c.bn <= 128 * 64 ? 32 : 16);
+            if (K >= 2 * deep) c.bk = deep;
+        }
+    }
     // tuning hook: DSC_MM_TILE="BM,BN,BK,WAVES_M,WAVES_N,GROUP_M" for products at least one tile large
     if (const char* env = std::getenv("DSC_MM_TILE")) {
         MmConfig e{};
@@ -977,7 +1111,7 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
     const bool vec_store = g.n % 4 == 0 && batch_stride % 4 == 0 && row_stride % 4 == 0;
     std::ostringstream k;
     k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
-    k << "    const uint rand_seed = *seed_cell;\n";
+    k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
     k << "    const int cb = blockIdx.x / " << S(blocks_per_batch) << ";\n";
     k << "    const int row0 = (blockIdx.x % " << S(blocks_per_batch) << ") * " << S(256 * R) << " + threadIdx.x;\n";
     if (b_in_lds) {
@@ -1112,7 +1246,7 @@ string gen_matmul_tallk(Emitter& em, Generated* out) {
     std::ostringstream k;
     k << "typedef float tk_float4 __attribute__((ext_vector_type(4)));\n";
     k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
-    k << "    const uint rand_seed = *seed_cell;\n";
+    k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
     k << "    __shared__ float red[4][" << MT * NT * 256 << "];\n";
     k << "    const int chunk = blockIdx.x % " << S(g.chunks) << ", cb = blockIdx.x / " << S(g.chunks) << ";\n";
     k << "    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;\n";
@@ -1178,7 +1312,8 @@ string gen_matmul(Emitter& em, Generated* out) {
     const bool rows = d.output_mode == DSC_MATMUL_ROWS;
     if (rows_kernel_applies(fk, g)) return gen_matmul_rows(em, out);
     if (tallk_kernel_applies(fk, g)) return gen_matmul_tallk(em, out);
-    MmConfig c = pick_config(g.m, g.n, g.batch * ((!fk.sum_chunks && g.chunks > 1) ? g.chunks : 1));
+    const bool split = !fk.sum_chunks && g.chunks > 1;
+    MmConfig c = pick_config(g.m, g.n, split ? chunk_k_of(g) : g.k, g.batch * (split ? g.chunks : 1));
 
     // k chunking: the reference writes `chunks` partial products of chunk_tiles*16 k each (kernel.rs:436)
     int64_t kchunks = 1, chunk_k = ((g.k + c.bk - 1) / c.bk) * c.bk;
@@ -1187,7 +1322,7 @@ string gen_matmul(Emitter& em, Generated* out) {
         const int64_t chunk_tiles = (k_tiles + g.chunks - 1) / g.chunks;
         chunk_k = chunk_tiles * 16;
         kchunks = g.chunks;
-        if (chunk_k % c.bk) c.bk = 16;
+        while (chunk_k % c.bk) c.bk /= 2;
     }
     if (!config_ok(c)) return "matmul: invalid tile configuration";
 
@@ -1293,6 +1428,13 @@ void count_work(const FusedKernel& fk, Generated* g) {
         out_each = (double)(m.batch * m.m * m.n) * (double)(fk.sum_chunks ? 1 : m.chunks);
         g->algo_flops = 2.0 * (double)m.batch * (double)m.m * (double)m.n * (double)m.k;
     }
+    if (fk.dgrad.on) {
+        const FusedKernel::ConvDgrad& c = fk.dgrad;
+        const MatMulDims m = matmul_dims(d);
+        const double ph = (double)(c.oh + c.fh - 1), pw = (double)(c.ow + c.fw - 1);
+        out_each = (double)c.img * (ph - 2.0 * c.pad_h) * (pw - 2.0 * c.pad_w) * (double)(c.g * c.c);
+        g->algo_flops = 2.0 * (double)c.g * (double)c.img * ph * pw * (double)(c.fh * c.fw * m.k) * (double)c.c;
+    }
     if (d.kind == DSC_KERNEL_SCATTER_ADD)  // read-modify-write of the entries that receive a value
         out_each = 2.0 * std::min((double)element_count(d.shape), (double)element_count(d.inputs[0].out_shape));
     if (fk.row_stages.empty()) elements += out_each * (double)fk.outputs.size();
@@ -1355,6 +1497,11 @@ std::string FusedKernel::key() const {
         s.append(reinterpret_cast<const char*>(&row_m), 8);
         s.append(reinterpret_cast<const char*>(&row_n), 8);
     }
+    if (dgrad.on) {
+        s += "|D";
+        for (int64_t v : {dgrad.img, dgrad.oh, dgrad.ow, dgrad.g, dgrad.fh, dgrad.fw, dgrad.c, dgrad.pad_h, dgrad.pad_w, (int64_t)dgrad.rows_first})
+            s.append(reinterpret_cast<const char*>(&v), 8);
+    }
     for (size_t i = 0; i < parts.size(); ++i) {
         s += "|P{" + parts[i].key() + "}";
         for (int j : part_params[i]) s.append(reinterpret_cast<const char*>(&j), 4);
@@ -1365,7 +1512,7 @@ std::string FusedKernel::key() const {
     s.append(reinterpret_cast<const char*>(&n_buffers), 4);
     if (const char* env = std::getenv("DSC_MM_TILE"))
         if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|T") + env;
-    for (const char* name : {"DSC_MM_ROWS", "DSC_ROWS_R", "DSC_ROWS_UNROLL", "DSC_ROWS_B", "DSC_ROWS_DIRECT_STORE", "DSC_MM_TALLK", "DSC_TALLK_UNROLL"})
+    for (const char* name : {"DSC_MM_DEEP_K", "DSC_MM_ROWS", "DSC_ROWS_R", "DSC_ROWS_UNROLL", "DSC_ROWS_B", "DSC_ROWS_DIRECT_STORE", "DSC_MM_TALLK", "DSC_TALLK_UNROLL"})
         if (const char* env = std::getenv(name))
             if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|") + name + env;
     return s;
@@ -1375,8 +1522,13 @@ namespace {
 string generate_multi(const FusedKernel& fk, Generated* out);
 }
 
+bool conv_dgrad_fits(const FusedKernel::ConvDgrad& c, int64_t k) {
+    if (k % 4 != 0 || c.g * c.c > 64 || c.fh * c.fw * k * c.g * c.c > 8192) return false;
+    return dgrad_lds_floats(c, k) * 4 <= 64 * 1024 && c.oh + c.fh - 1 > 2 * c.pad_h && c.ow + c.fw - 1 > 2 * c.pad_w;
+}
+
 bool can_be_part(const FusedKernel& fk) {
-    if (!fk.parts.empty()) return false;
+    if (!fk.parts.empty() || fk.dgrad.on) return false;
     return fk.main.raw().kind != DSC_KERNEL_MATMUL;  // the MatMul kernels size their workgroups per shape
 }
 
@@ -1420,6 +1572,9 @@ static std::string generate_one(const FusedKernel& fk, Generated* out, bool with
     Generated g;
     if (!fk.row_stages.empty()) {
         err = gen_row_fused(em, &g);
+    } else if (fk.dgrad.on) {
+        if (fk.main.raw().kind != DSC_KERNEL_MATMUL || fk.has_epilogue) return "conv dgrad: needs a plain MatMul";
+        err = gen_conv_dgrad(em, &g);
     } else
     switch (fk.main.raw().kind) {
     case DSC_KERNEL_FILL: err = gen_fill(em, &g); break;
@@ -1467,7 +1622,7 @@ string generate_multi(const FusedKernel& fk, Generated* out) {
         src << "namespace part" << i << " {\n" << text << "}  // namespace part" << i << "\n\n";
         body << "    if (blockIdx.x < " << first + pg.grid << "u) { part" << i << "::part_entry(blockIdx.x - " << first << "u";
         for (int j : fk.part_params[i]) body << ", b" << j;
-        body << ", seed_cell); return; }\n";
+        body << ", seed_cell, seed_value); return; }\n";
         first += pg.grid;
         g.algo_bytes += pg.algo_bytes;
         g.algo_flops += pg.algo_flops;

@@ -60,6 +60,17 @@ struct FusedKernel {
     // `main` is parts[0].main (for the label); inputs/outputs of the launch are those of the parts.
     std::vector<FusedKernel> parts;
     std::vector<std::vector<int>> part_params;
+    // Data gradient of a stride-1 convolution with few channels, as one kernel: `main` is the MatMul dC x filter^T
+    // ([g][(img, oy, ox)][oc] x [g][oc][(fy, fx, c)]); the kernel also does what the reference's WindowsToImage
+    // (sum of the windows covering each pixel of the padded image) and the two Unpads after it (fold the
+    // replicate-padding border back onto the edge pixels) would do.  One workgroup per image: dC of the image
+    // sits in LDS inside a halo of zeros, the padded-image gradient goes back through LDS for the border folds.
+    struct ConvDgrad {
+        bool on = false;
+        int64_t img = 0, oh = 0, ow = 0, g = 0, fh = 0, fw = 0, c = 0;  // windows [img, oh, ow, g, fh, fw, c]
+        int64_t pad_h = 0, pad_w = 0;  // Unpads folded in (0: the output is the padded image)
+        int32_t rows_first = 1;        // the Unpad along the image rows came first
+    } dgrad;
     bool sum_chunks = false;               // MatMul: ignore the descriptor's chunk count, write one full sum
     std::vector<int> outputs;              // pointer parameter index of each output of main (or of the epilogue)
     int n_buffers = 0;                     // number of pointer parameters
@@ -75,7 +86,7 @@ struct Generated {
     std::string entry;       // name of the __global__ function (dsc_<kind>)
     unsigned grid = 1;       // workgroups (1-D)
     unsigned block = 64;     // threads per workgroup
-    int n_buffers = 0;       // pointer parameters, in order; followed by `const uint* seed_cell`
+    int n_buffers = 0;       // pointer parameters, in order; followed by `const uint* seed_cell, uint seed_value`
     std::string note;        // strategy chosen (for schedule listings)
     // Work one launch stands for, counted the way a roofline wants it: bytes = 4 * (distinct elements of every
     // buffer read, a broadcast or windowed operand at its own size, + elements written; a scatter accumulator is
@@ -85,6 +96,10 @@ struct Generated {
 
 // Returns "" on success or an error message.
 std::string generate(const FusedKernel& k, Generated* out);
+
+// Whether the convolution data-gradient kernel can take this geometry (k = output channels per group): the image
+// tile must fit the workgroup's LDS.
+bool conv_dgrad_fits(const FusedKernel::ConvDgrad& c, int64_t k);
 
 // Whether a kernel can be one part of a multi-part launch (256 threads per workgroup, addressed by blockIdx.x only).
 bool can_be_part(const FusedKernel& k);

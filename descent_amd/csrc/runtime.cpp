@@ -264,6 +264,14 @@ Kernel* get_kernel(Context* ctx, const FusedKernel& fk, int* status) {
     if (!fk.row_stages.empty())
         k->label = "RowFused [" + std::to_string((long long)fk.row_m) + ", " + std::to_string((long long)fk.row_n) + "] (" +
                    std::to_string(fk.row_stages.size()) + " clusters)";
+    if (fk.dgrad.on) {
+        const auto& c = fk.dgrad;
+        char text[160];
+        std::snprintf(text, sizeof text, "ConvDataGrad [%lld, %lld, %lld, %lld] %lldx%lld taps, %lld groups", (long long)c.img,
+                      (long long)(c.oh + c.fh - 1 - 2 * c.pad_h), (long long)(c.ow + c.fw - 1 - 2 * c.pad_w), (long long)(c.g * c.c),
+                      (long long)c.fh, (long long)c.fw, (long long)c.g);
+        k->label = text;
+    }
     if (fk.has_epilogue) k->label += " + " + label_name(fk.epilogue.raw());
     if (!fk.virtuals.empty()) k->label += " <" + std::to_string(fk.virtuals.size()) + " fused producers>";
     if (!fk.parts.empty()) {
@@ -315,22 +323,20 @@ int set_seed(Context* ctx, uint32_t rand_seed) {
 
 int launch_kernel(Context* ctx, Kernel* k, void* const* device_ptrs, int n, uint32_t rand_seed) {
     if (ctx->offline || !k->function) return fail(DSC_ERR_NO_DEVICE, "kernel launch without a device");
-    {
-        int rc = set_seed(ctx, rand_seed);
-        if (rc != DSC_OK) return rc;
-    }
     if (n != k->gen.n_buffers)
         return fail(DSC_ERR_INVALID, "kernel '" + k->label + "' takes " + std::to_string(k->gen.n_buffers) + " buffers, got " +
                                          std::to_string(n));
     void* ptr_values[64];
-    void* args[65];
+    void* args[66];
     if (n > 64) return fail(DSC_ERR_UNSUPPORTED, "more than 64 buffers bound to one kernel");
     for (int i = 0; i < n; ++i) {
         ptr_values[i] = device_ptrs[i];
         args[i] = &ptr_values[i];
     }
-    void* seed_ptr = ctx->seed_cell;
+    void* seed_ptr = ctx->seed_through_cell ? ctx->seed_cell : nullptr;
+    uint32_t seed_value = rand_seed;
     args[n] = &seed_ptr;
+    args[n + 1] = &seed_value;
     hipEvent_t start = nullptr, stop = nullptr;
     if (ctx->profiling) {
         auto take = [&](hipEvent_t* ev) -> hipError_t {

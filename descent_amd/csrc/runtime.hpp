@@ -89,7 +89,9 @@ struct Context {
     bool staging_busy[kStagingRegions] = {false, false};
     int staging_next = 0;
 
-    // one device word holding the rand seed of the launches that follow (kernels read it at entry)
+    // Launches take the rand seed by value.  While `seed_through_cell` is set (a schedule capturing or replaying a
+    // HIP graph) they are given this one device word instead, which set_seed fills before the graph runs.
+    bool seed_through_cell = false;
     uint32_t* seed_cell = nullptr;
     uint32_t seed_value = 0;
     bool seed_known = false;

@@ -590,6 +590,57 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             if (!chain_ok) continue;
             if (taken_in_place_between(i, w_idx, input_nodes(mm))) continue;
 
+            // First choice: the dedicated kernel (image tile in LDS), which also takes the Unpads that fold the
+            // padding border back (one along the image rows, one along the columns, in either order).
+            {
+                FusedKernel::ConvDgrad cv;
+                cv.on = true;
+                cv.img = IMG; cv.oh = OH; cv.ow = OW; cv.g = G; cv.fh = FH; cv.fw = FW; cv.c = C;
+                std::vector<int> unpads;
+                int last = w_idx;
+                for (int step = 0; step < 2; ++step) {
+                    if (is_graph_output[drafts[last].outs[0].node]) break;
+                    auto uc = consumers_of(drafts[last].outs[0].node);
+                    if (uc.size() != 1 || uc[0] <= last) break;
+                    const Draft& u = drafts[uc[0]];
+                    const dsc_kernel_desc& ud = u.fk.main.raw();
+                    if (ud.kind != DSC_KERNEL_UNPAD || !u.fk.virtuals.empty() || u.fk.has_epilogue || u.outs[0].copy_from >= 0 ||
+                        ud.shape.rank != 4 || !is_identity(ud.inputs[0]) || ud.pad < 1)
+                        break;
+                    if (ud.axis == 1 && cv.pad_h == 0) {
+                        cv.pad_h = ud.pad;
+                        if (step == 0) cv.rows_first = 1;
+                    } else if (ud.axis == 2 && cv.pad_w == 0) {
+                        cv.pad_w = ud.pad;
+                        if (step == 0) cv.rows_first = 0;
+                    } else {
+                        break;
+                    }
+                    unpads.push_back(uc[0]);
+                    last = uc[0];
+                }
+                const bool direct = !(flags & DSC_SCHEDULE_NO_CONV_KERNELS);
+                if (direct && conv_dgrad_fits(cv, K) && !taken_in_place_between(i, last, input_nodes(mm))) {
+                    Draft fused;
+                    fused.fk.main = mm.fk.main;
+                    fused.fk.dgrad = cv;
+                    for (auto& src : mm.fk.inputs) fused.fk.inputs.push_back(import_source(fused, mm, src, 0));
+                    fused.fk.outputs.push_back(param_index(fused, drafts[last].outs[0].node, true));
+                    fused.outs.push_back(drafts[last].outs[0]);
+                    fused.covers = mm.covers;
+                    for (int j : std::vector<int>{copy_idx, w_idx})
+                        if (j >= 0) fused.covers.insert(fused.covers.end(), drafts[j].covers.begin(), drafts[j].covers.end());
+                    for (int j : unpads) fused.covers.insert(fused.covers.end(), drafts[j].covers.begin(), drafts[j].covers.end());
+                    compact(fused);
+                    mm.alive = false;
+                    if (copy_idx >= 0) drafts[copy_idx].alive = false;
+                    drafts[w_idx].alive = false;
+                    for (int j : unpads) drafts[j].alive = false;
+                    drafts[last] = fused;
+                    continue;
+                }
+            }
+
             const dsc_view va = md.inputs[0], vb = md.inputs[1];
             const int64_t Mp = IMG * PH * PW, Kp = FH * FW * K;
             // A': out [G, IMG, PH, PW, FH, FW, K] onto dC
@@ -1147,6 +1198,7 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
         ++direct_runs;
         return enqueue_all();
     }
+    // captured launches read the seed from the context's device cell
     int rc = set_seed(ctx, rand_seed);
     if (rc != DSC_OK) return rc;
     for (auto& c : captured) {
@@ -1163,7 +1215,9 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
     }
     hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
     if (e != hipSuccess) return fail(DSC_ERR_HIP, std::string("hipStreamBeginCapture: ") + hipGetErrorString(e));
+    ctx->seed_through_cell = true;
     rc = enqueue_all();
+    ctx->seed_through_cell = false;
     hipGraph_t graph = nullptr;
     e = hipStreamEndCapture(ctx->stream, &graph);
     if (rc != DSC_OK) {

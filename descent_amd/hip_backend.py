@@ -118,22 +118,30 @@ def codegen_compile(kernel, arch: str = "gfx950") -> int:
     return n.value
 
 
-def check_schedule(graph, fused: bool = True, arch: str = "gfx950") -> str:
+def schedule_flags(fused) -> int:
+    """`fused`: True (all fusion), False (one launch per reference cluster), or "generic-conv" (all fusion, but
+    convolution gradients stay on the generic MatMul path instead of the dedicated kernels)."""
+    if fused == "generic-conv":
+        return _abi.SCHEDULE_NO_CONV_KERNELS
+    return 0 if fused else _abi.SCHEDULE_NO_FUSION
+
+
+def check_schedule(graph, fused=True, arch: str = "gfx950") -> str:
     """Plans and compiles every kernel of a graph's schedule without a GPU; returns the listing."""
     ms = _abi.MarshalledSchedule(graph)
     out = C.c_void_p()
-    flags = 0 if fused else _abi.SCHEDULE_NO_FUSION
+    flags = schedule_flags(fused)
     check(lib().dsc_codegen_check_schedule(C.byref(ms.desc), flags, arch.encode(), C.byref(out)))
     return _take_string(out)
 
 
 class HipSchedule:
-    def __init__(self, backend: "HipBackend", graph, fused: bool):
+    def __init__(self, backend: "HipBackend", graph, fused):
         self._backend = backend
         self._ms = _abi.MarshalledSchedule(graph)
         self.params = self._ms.params
         self._handle = C.c_void_p()
-        flags = 0 if fused else _abi.SCHEDULE_NO_FUSION
+        flags = schedule_flags(fused)
         check(lib().dsc_schedule_create(backend._ctx, C.byref(self._ms.desc), flags, C.byref(self._handle)))
         self._slots = (C.c_uint64 * max(1, len(self.params)))()
 
@@ -230,7 +238,7 @@ class HipBackend:
         arr = (C.c_uint64 * len(handles))(*handles)
         check(lib().dsc_kernel_launch(self._ctx, k, arr, len(handles), rand_seed & 0xFFFFFFFF))
 
-    def make_schedule(self, graph, fused: bool = True) -> HipSchedule:
+    def make_schedule(self, graph, fused=True) -> HipSchedule:
         return HipSchedule(self, graph, fused)
 
     def sync(self) -> None:

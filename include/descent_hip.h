@@ -285,6 +285,8 @@ typedef struct dsc_schedule dsc_schedule;
 
 /* flags for dsc_schedule_create */
 #define DSC_SCHEDULE_NO_FUSION 1u /* launch exactly one kernel per reference cluster (for parity tests) */
+#define DSC_SCHEDULE_NO_CONV_KERNELS 2u /* keep convolution gradients on the generic MatMul path (fused producers)
+                                           instead of the dedicated LDS-tiled kernels (for parity tests) */
 
 int dsc_schedule_create(dsc_ctx* ctx, const dsc_schedule_desc* desc, uint32_t flags, dsc_schedule** out);
 int dsc_schedule_destroy(dsc_ctx* ctx, dsc_schedule* s);

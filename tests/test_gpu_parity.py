@@ -264,21 +264,25 @@ def test_softmax_cross_entropy_runs_as_one_row_fused_launch(hip_backend_session,
     assert np.array_equal(ga, ca)  # arg-max derived: exact, ties included
 
 
-def test_convnet_step_at_batch_64_vs_oracle(hip_backend_session):
-    """At this batch the convolution GEMMs are large enough for the row-per-thread kernels, among them the fused
-    data gradient of the second convolution (MatMul + reshape copy + WindowsToImage as one product over the
-    padded image): two Adam steps, every parameter and optimiser state."""
+@pytest.mark.parametrize("fused", [True, "generic-conv"])
+def test_convnet_step_at_batch_64_vs_oracle(hip_backend_session, fused):
+    """At this batch the convolution GEMMs are large enough for the row-per-thread kernels.  The data gradient of
+    the second convolution runs either as the dedicated kernel (MatMul + reshape copy + WindowsToImage + both
+    Unpads, image tile in LDS) or, with "generic-conv", as one MatMul over the padded image whose operands are
+    fused producers.  Two Adam steps, every parameter and optimiser state."""
     from descent_amd import workloads
 
-    genv, cenv = _envs(hip_backend_session)
+    genv, cenv = _envs(hip_backend_session, fused=fused)
     gw = workloads.convnet(genv, batch=64, seed=13)
     cw = workloads.convnet(cenv, batch=64, seed=13)
-    listing = None
     for step in range(2):
         genv.run(gw.graph, 500 + step)
         cenv.run(cw.graph, 500 + step)
     listing = next(iter(gw.graph.__dict__["_schedules"].values())).describe()
-    assert "MatMul (k=144) [1, 16384, 2, 8] <2 fused producers>  [row-per-thread" in listing, listing
+    if fused is True:
+        assert "ConvDataGrad [64, 14, 14, 16] 3x3 taps, 2 groups" in listing, listing
+    else:
+        assert "MatMul (k=144) [1, 16384, 2, 8] <2 fused producers>  [row-per-thread" in listing, listing
     got, want = gw.snapshot(), cw.snapshot()
     for key in want:
         if key == "accuracy":

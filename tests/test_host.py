@@ -172,7 +172,8 @@ def test_convnet_graph_shape():
     assert set(covered) == set(range(66))
     # the data gradient of the second convolution: MatMul + reshape copy + WindowsToImage as one product over
     # the padded image, both operands fused producers
-    assert "MatMul (k=144) [1, 256000, 2, 8] <2 fused producers>" in listing
+    assert "ConvDataGrad [1000, 14, 14, 16] 3x3 taps, 2 groups" in listing
+    assert "MatMul (k=144) [1, 256000, 2, 8] <2 fused producers>" in hip_backend.check_schedule(w.graph, fused="generic-conv")
     # the work figures of the listing: the eleven GEMMs of the step as the reference runs them
     assert "4.373 GFLOP in MatMuls" in hip_backend.check_schedule(w.graph, fused=False)
 
