@@ -778,15 +778,34 @@ string gen_windows_to_image(Emitter& em, Generated* out) {
     return "";
 }
 
+// Accumulators small enough for LDS that receive many values per entry (the coarse levels of a hash grid: half a
+// million adds into a few hundred entries) are summed per workgroup in LDS first; the workgroup then adds its
+// non-zero totals to memory.  Contention on the memory atomics drops by the number of values a workgroup folds.
+bool scatter_privatised(const dsc_kernel_desc& d, int64_t* workgroups) {
+    const int64_t table = element_count(d.shape), n = element_count(d.inputs[0].out_shape);
+    if (table > 8192 || n < 16 * table || n < 65536) return false;
+    *workgroups = std::max<int64_t>(16, std::min<int64_t>(256, n / (4 * table)));
+    return true;
+}
+
 string gen_scatter_add(Emitter& em, Generated* out) {
     const FusedKernel& fk = em.fk;
     const dsc_kernel_desc& d = fk.main.raw();
     const dsc_view& vv = d.inputs[0];
     const dsc_view& vi = d.inputs[1];
     const int64_t n = element_count(vv.out_shape);
+    int64_t wgs = 0;
+    const bool priv = scatter_privatised(d, &wgs);
+    const int64_t table = element_count(d.shape);
     std::ostringstream k;
     k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
-    k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n";
+    if (priv) {
+        k << "    __shared__ float acc[" << S(table) << "];\n";
+        k << "    for (int i = threadIdx.x; i < " << S(table) << "; i += 256) acc[i] = 0.f;\n    __syncthreads();\n";
+        k << "    for (uint gid = blockIdx.x * 256u + threadIdx.x; gid < " << S(n) << "u; gid += " << S(wgs * 256) << "u) {\n";
+    } else {
+        k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n    {\n";
+    }
     auto c = em.emit_coords(k, vv.out_shape, "gid", "c");
     k << "    const float value = " << em.load_view(fk.inputs[0], vv, c) << ";\n";
     k << "    const int si = F2I(" << em.load_view(fk.inputs[1], vi, {c[d.axis]}) << ");\n";
@@ -795,12 +814,18 @@ string gen_scatter_add(Emitter& em, Generated* out) {
     string idx = "0";
     for (int i = 0; i < d.shape.rank; ++i) idx += " + " + (i == d.axis ? string("si") : c[i]) + "*" + S(st[i]);
     // bounds: an index outside the accumulator would be a wild write; the reference has no check, here it is dropped
-    k << "    if (si < 0 || si >= " << S(d.shape.dims[d.axis]) << ") return;\n";
-    k << "    unsafeAtomicAdd(&b" << fk.outputs[0] << "[" << idx << "], value);\n}\n";
-    out->grid = blocks_for(n, 256);
+    k << "    if (si >= 0 && si < " << S(d.shape.dims[d.axis]) << ") ";
+    if (priv) {
+        k << "atomicAdd(&acc[" << idx << "], value);\n    }\n    __syncthreads();\n";
+        k << "    for (int i = threadIdx.x; i < " << S(table) << "; i += 256) {\n        const float total = acc[i];\n";
+        k << "        if (total != 0.f) unsafeAtomicAdd(&b" << fk.outputs[0] << "[i], total);\n    }\n}\n";
+    } else {
+        k << "unsafeAtomicAdd(&b" << fk.outputs[0] << "[" << idx << "], value);\n    }\n}\n";
+    }
+    out->grid = priv ? (unsigned)wgs : blocks_for(n, 256);
     out->block = 256;
     out->source = k.str();
-    out->note = "scatter_add: global_atomic_add_f32";
+    out->note = priv ? "scatter_add: per-workgroup sums in LDS (ds_add_f32), then global_atomic_add_f32" : "scatter_add: global_atomic_add_f32";
     return "";
 }
 

@@ -997,6 +997,65 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             drafts[pe_idx] = fused;  // runs where the per-element cluster ran: all of its inputs exist by then
         }
 
+        // Pass 3b: ScatterAdds chained through one accumulator (each takes the previous one's result in place:
+        // the four corner updates of one hash-grid level) commute, so the chain runs as one multi-part launch
+        // whose parts all add into the same buffer.  It runs where the last one ran.
+        for (int i = 0; i < (int)drafts.size(); ++i) {
+            if (!drafts[i].alive || drafts[i].fk.main.raw().kind != DSC_KERNEL_SCATTER_ADD || !drafts[i].fk.parts.empty()) continue;
+            std::vector<int> chain{i};
+            for (;;) {
+                const int node = drafts[chain.back()].outs[0].node;
+                if (is_graph_output[node]) break;
+                int next = -1, readers = 0;
+                for (int j = chain.back() + 1; j < (int)drafts.size() && next < 0; ++j) {
+                    if (!drafts[j].alive) continue;
+                    for (auto& o : drafts[j].outs)
+                        if (o.copy_from == node) next = j;
+                }
+                if (next < 0) break;
+                const Draft& nx = drafts[next];
+                if (nx.fk.main.raw().kind != DSC_KERNEL_SCATTER_ADD || !nx.fk.parts.empty() ||
+                    !same_shape(nx.fk.main.raw().shape, drafts[i].fk.main.raw().shape))
+                    break;
+                for (int c : consumers_of(node)) (void)c, ++readers;  // nobody may read the intermediate sum
+                if (readers != 0) break;
+                chain.push_back(next);
+                if (chain.size() >= 8) break;
+            }
+            if (chain.size() < 2) continue;
+            const int last = chain.back();
+            // every part's inputs must still be what they were when the merged launch runs
+            bool ok = true;
+            for (int j : chain)
+                if (j != last && taken_in_place_between(j, last, input_nodes(drafts[j]))) ok = false;
+            size_t bound = 0;
+            for (int j : chain) bound += drafts[j].params.size();
+            if (!ok || bound > 48) continue;
+            const int final_node = drafts[last].outs[0].node;
+            Draft multi;
+            multi.fk.main = drafts[i].fk.main;
+            std::set<int> seen;
+            for (int j : chain) {
+                const Draft& d = drafts[j];
+                std::vector<int> map;
+                for (size_t p = 0; p < d.params.size(); ++p) {
+                    const bool is_out = d.fk.buffer_is_output[p];
+                    map.push_back(param_index(multi, is_out ? final_node : d.params[p], is_out));
+                }
+                multi.fk.parts.push_back(d.fk);
+                multi.fk.part_params.push_back(map);
+                for (int nd : input_nodes(d))
+                    if (seen.insert(nd).second) multi.part_inputs.push_back(nd);
+                multi.covers.insert(multi.covers.end(), d.covers.begin(), d.covers.end());
+            }
+            StepOutput out = drafts[i].outs[0];  // the first link says where the accumulator comes from
+            out.node = final_node;
+            multi.outs.push_back(out);
+            multi.fk.outputs.push_back(param_index(multi, final_node, true));
+            for (int j : chain) drafts[j].alive = false;
+            drafts[last] = multi;
+        }
+
         // Pass 4: launches of a few workgroups each (optimiser updates of small tensors, short reductions, scalar
         // bookkeeping) cost a launch apiece while using a fraction of the machine.  Runs of them that do not
         // depend on one another become one multi-part launch; a later small launch is hoisted into the run when

@@ -290,3 +290,42 @@ def test_convnet_step_at_batch_64_vs_oracle(hip_backend_session, fused):
         else:
             err = rel_l2(got[key], want[key])
             assert err <= TOL, f"{key}: rel L2 {err}"
+
+
+def _scatter_chain_case(env, n, entries, links, seed):
+    """`links` scatter-adds chained through one [entries, 2] accumulator, as the corner updates of one hash-grid
+    level are: values [n, 2] ~ N(0,1), indices uniform."""
+    rng = np.random.default_rng(seed)
+    vals = [env.static_parameter_with_data([n, 2], f"v{i}", rng.standard_normal((n, 2), dtype=np.float32)) for i in range(links)]
+    idxs = [env.static_parameter_with_data([n], f"i{i}", rng.integers(0, entries, n).astype(np.float32)) for i in range(links)]
+    out = env.static_parameter([entries, 2], "acc")
+
+    def build(s):
+        acc = s.literal(0.0).value().broadcast([entries, 2])
+        for v, i in zip(vals, idxs):
+            acc = acc.scatter_add(s.parameter_value(v), 0, s.parameter_value(i).into_u32())
+        s.write_parameter_value(out, acc)
+
+    g = env.build_graph(build)
+    env.run(g, 0)
+    want = np.zeros((entries, 2), np.float64)
+    for v, i in zip(vals, idxs):
+        np.add.at(want, env.read_parameter(i).astype(np.int64), env.read_parameter(v).astype(np.float64))
+    return g, env.read_parameter(out), want
+
+
+@pytest.mark.parametrize("n,entries,links", [(131072, 289, 4), (65536, 3481, 2), (131072, 100000, 4), (70000, 3, 3)])
+def test_scatter_add_chains_vs_float64(hip_backend_session, n, entries, links):
+    """Float atomics reorder the sums, so the bound is the looser one stated for scatter-add: 1e-4 relative L2
+    against a float64 accumulation, for the GPU (small accumulators go through per-workgroup LDS sums first) and
+    for the oracle's serial fp32 sums alike."""
+    genv, cenv = _envs(hip_backend_session)
+    g, got, want = _scatter_chain_case(genv, n, entries, links, 40 + entries)
+    _, oracle, _ = _scatter_chain_case(cenv, n, entries, links, 40 + entries)
+    listing = next(iter(g.__dict__["_schedules"].values())).describe()
+    # the index conversions share one launch, the whole chain of scatter-adds another
+    assert int(listing.split()[0]) == 2 and "Multi (%d kernels: ScatterAdd" % links in listing, listing
+    if entries * 2 <= 8192 and n * 2 >= 32 * entries:
+        assert "per-workgroup sums in LDS" in listing, listing
+    assert rel_l2(got, want) <= TOL
+    assert rel_l2(oracle, want) <= TOL
