@@ -25,6 +25,10 @@ if ROOT not in sys.path:
 
 MFMA_FP32_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBS = 8000.0
+# HBM bytes one launch of the headline kernel moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same
+# command, each counter scaled by what it reads for the streaming kernel of known size (--copy-calibration); the
+# summary is profiles/matmul_mfma_8192.txt.  Only the 8192^3 workload has been counted.
+MEASURED_TRAFFIC_BYTES = {8192: 3.491e9}
 
 
 def time_graph(env, graph, steps: int, warmup: int, seed0: int = 1, profile: bool = True):
@@ -84,19 +88,46 @@ def bench_matmul(env, m, n, k, steps, warmup):
     }
 
 
+KERNEL_CLASSES = ("MatMul", "ConvDataGrad", "PerElement", "Reduce", "RowFused", "WindowsToImage", "Unpad", "ScatterAdd",
+                  "Multi (4 kernels: ScatterAdd", "Multi", "Fill")
+
+
+def class_rooflines(be, steps):
+    """Per kernel class (label prefix) of the launches profiled since the last reset: time per step, and the
+    algorithmic bytes / flops those launches stand for as GB/s against the HBM peak and TFLOP/s against the fp32
+    MFMA peak.  A "Multi" launch is several small kernels sharing one launch."""
+    out = {}
+    for prefix in KERNEL_CLASSES:
+        us, nbytes, flops, n = be.timing_work(prefix)
+        if not n:
+            continue
+        row = {"us_per_step": us / steps, "launches_per_step": n / steps, "gbs": nbytes / (us * 1e-6) / 1e9,
+               "frac_hbm": nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+        if flops:
+            row["tflops"] = flops / (us * 1e-6) / 1e12
+            row["frac_mfma"] = row["tflops"] / MFMA_FP32_PEAK_TFLOPS
+        out[prefix] = row
+    return out
+
+
 def bench_convnet(env, steps, warmup, batch=1000):
     from descent_amd import workloads
 
     w = workloads.convnet(env, batch=batch, seed=3)
     wall = time_then_profile(env, w.graph, steps, warmup)
     report = env.backend.timing_report(int(os.environ.get("DSC_BENCH_TOPN", "12")))
+    classes = class_rooflines(env.backend, steps) if EVENT_PASS else {}
     env.backend.profile_reset()
     sched = next(iter(w.graph.__dict__["_schedules"].values()))
+    listing = sched.describe()
+    work = listing.strip().splitlines()[-1]
     return {
         "steps_per_s": steps / wall,
         "ms_per_step": 1e3 * wall / steps,
         "launches_per_step": sched.launch_count()[0],
         "clusters": sched.launch_count()[1],
+        "algorithmic_work_per_step": work.lstrip("# "),
+        "kernel_classes": classes,
         "report": report,
     }
 
@@ -128,10 +159,7 @@ def bench_workload(env, build, steps, warmup, topn=8):
     wall = time_then_profile(env, w.graph, steps, warmup)
     be = env.backend
     out = {"steps_per_s": steps / wall, "ms_per_step": 1e3 * wall / steps}
-    for prefix in ("MatMul", "ScatterAdd", "PerElement", "Reduce"):
-        avg_us, launches = be.timing_query(prefix)
-        out[prefix.lower() + "_us_per_step"] = avg_us * launches / steps
-        out[prefix.lower() + "_launches_per_step"] = launches / steps
+    out["kernel_classes"] = class_rooflines(be, steps) if EVENT_PASS else {}
     report = be.timing_report(topn)
     be.profile_reset()
     sched = next(iter(w.graph.__dict__["_schedules"].values()))
@@ -254,7 +282,8 @@ def main():
         extra["coordinate_mlp_siren_512"] = siren
         hg, rep = bench_workload(env, lambda e: _w.hash_grid_fit(e), 10, 2)
         sys.stderr.write("cfg5 hash grid:\n" + rep)
-        hg["scatter_atomics_per_s"] = 16 * 4 * 2 * (1 << 18) / (hg["scatteradd_us_per_step"] * 1e-6) if hg["scatteradd_us_per_step"] else None
+        sc = hg["kernel_classes"].get("Multi (4 kernels: ScatterAdd") or hg["kernel_classes"].get("ScatterAdd")
+        hg["scatter_atomics_per_s"] = 16 * 4 * 2 * (1 << 18) / (sc["us_per_step"] * 1e-6) if sc else None
         extra["hash_grid_2p18"] = hg
     if args.workload == "headline":
         # the other half of the headline metric: ConvNet (batch 1000) train steps per second
@@ -288,7 +317,7 @@ def main():
             "peak": MFMA_FP32_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved / MFMA_FP32_PEAK_TFLOPS,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(n),
             "kernel_avg_us": head["kernel_avg_us"],
             "algorithmic_flops_per_launch": head["flops"],
         },

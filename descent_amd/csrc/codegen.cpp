@@ -1399,12 +1399,19 @@ string gen_matmul(Emitter& em, Generated* out) {
         std::ostringstream body;
         std::map<int, string> ov;
         ov[fk.epilogue_product_input] = "product";
-        em.emit_pe(body, pe, fk.epilogue_inputs, "gid", "e", ov);
+        // the element id as (batch, row, column): what the epilogue reads per column only (a bias) or per row
+        // only is then addressed without dividing the id, and is loop-invariant along the other coordinate
+        IndexForm form;
+        form.valid = true;
+        form.names = {"cb", "cm", "cn"};
+        form.coefs = {batch_stride, row_stride, 1};
+        form.extents = {g.batch, g.m, g.n};
+        em.emit_pe(body, pe, fk.epilogue_inputs, "gid", "e", ov, &form);
         for (int o = 0; o < pe.n_outputs; ++o) body << "    b" << fk.outputs[o] << "[gid] = et" << pe.outputs[o] << ";\n";
-        em.funcs << "DSC_INLINE void mm_store(float product, int gid, " << em.params_decl() << ") {\n" << body.str() << "}\n";
-        k << "#define MM_STORE(v, idx) mm_store(v, idx, " << em.params_pass() << ")\n";
+        em.funcs << "DSC_INLINE void mm_store(float product, int gid, int cb, int cm, int cn, " << em.params_decl() << ") {\n" << body.str() << "}\n";
+        k << "#define MM_STORE(v, idx, b, m, n) mm_store(v, idx, b, m, n, " << em.params_pass() << ")\n";
     } else {
-        k << "#define MM_STORE(v, idx) b" << fk.outputs[0] << "[idx] = (v)\n";
+        k << "#define MM_STORE(v, idx, b, m, n) b" << fk.outputs[0] << "[idx] = (v)\n";
     }
     k << kMatmulMfmaSource;
 
