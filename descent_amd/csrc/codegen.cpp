@@ -1421,9 +1421,13 @@ string gen_matmul(Emitter& em, Generated* out) {
     out->grid = (unsigned)grid;
     out->block = 64 * c.wm * c.wn;
     out->source = k.str();
+    {
+        const char* e = std::getenv("DSC_MM_PERSISTENT");
+        out->persistent_ok = !(e && e[0] == '0') && grid > 256 && chunk_k / c.bk <= 128;
+    }
     char note[160];
-    std::snprintf(note, sizeof note, "mfma 32x32x2 tile %dx%dx%d waves %dx%d A%d B%d chunks %lld%s", c.bm, c.bn, c.bk, c.wm, c.wn,
-                  a_mode, b_mode, (long long)kchunks, fk.has_epilogue ? " +epilogue" : "");
+    std::snprintf(note, sizeof note, "mfma 32x32x2 tile %dx%dx%d waves %dx%d A%d B%d chunks %lld%s%s", c.bm, c.bn, c.bk, c.wm, c.wn,
+                  a_mode, b_mode, (long long)kchunks, fk.has_epilogue ? " +epilogue" : "", out->persistent_ok ? " persistent" : "");
     out->note = note;
     return "";
 }
@@ -1544,7 +1548,7 @@ std::string FusedKernel::key() const {
     s.append(reinterpret_cast<const char*>(&n_buffers), 4);
     if (const char* env = std::getenv("DSC_MM_TILE"))
         if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|T") + env;
-    for (const char* name : {"DSC_MM_DEEP_K", "DSC_MM_ROWS", "DSC_ROWS_R", "DSC_ROWS_UNROLL", "DSC_ROWS_B", "DSC_ROWS_DIRECT_STORE", "DSC_MM_TALLK", "DSC_TALLK_UNROLL"})
+    for (const char* name : {"DSC_MM_PERSISTENT", "DSC_MM_DEEP_K", "DSC_MM_ROWS", "DSC_ROWS_R", "DSC_ROWS_UNROLL", "DSC_ROWS_B", "DSC_ROWS_DIRECT_STORE", "DSC_MM_TALLK", "DSC_TALLK_UNROLL"})
         if (const char* env = std::getenv(name))
             if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|") + name + env;
     return s;

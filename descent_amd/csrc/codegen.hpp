@@ -92,6 +92,10 @@ struct Generated {
     // buffer read, a broadcast or windowed operand at its own size, + elements written; a scatter accumulator is
     // read and written where values land), flops = 2*b*M*N*K of a MatMul (0 otherwise).
     double algo_bytes = 0, algo_flops = 0;
+    // MFMA MatMul with a short k: `grid` counts the (chunk, batch, tile) units, and the kernel accepts any smaller
+    // grid (its workgroups then walk several units each, overlapping one unit's stores with the next one's first
+    // loads).  The runtime shrinks the grid to what the device holds at once.
+    bool persistent_ok = false;
 };
 
 // Returns "" on success or an error message.

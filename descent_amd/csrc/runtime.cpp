@@ -307,6 +307,17 @@ Kernel* get_kernel(Context* ctx, const FusedKernel& fk, int* status) {
         *status = fail(DSC_ERR_HIP, std::string("hipModuleGetFunction: ") + hipGetErrorString(e));
         return nullptr;
     }
+    if (k->gen.persistent_ok) {
+        // as many workgroups as the device holds at once (a multiple of the 8 XCDs), never more than the units
+        int per_cu = 0;
+        e = hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k->function, (int)k->gen.block, 0);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            per_cu = 0;
+        }
+        const int64_t resident = (int64_t)per_cu * ctx->caps.compute_units / 8 * 8;
+        if (resident >= 8 && resident < (int64_t)k->gen.grid) k->gen.grid = (unsigned)resident;
+    }
     Kernel* raw = k.get();
     ctx->kernels[key] = std::move(k);
     *status = DSC_OK;
