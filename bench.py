@@ -193,7 +193,8 @@ def bench_reduce(env, rows, cols, axis, steps, warmup):
 
 def cpu_baseline_matmul(n: int, rows: int):
     """The CPU oracle (restatement of the reference's algorithm; the reference itself needs Rust + Vulkan) on
-    a slab of `rows` rows of the same n^3 product, epilogue included, all host cores through OpenMP."""
+    a slab of `rows` rows of the same n^3 product, epilogue included, and on a few ConvNet train steps, all host
+    cores through OpenMP."""
     from descent_amd import Environment, workloads
     from oracle.cpu_backend import CpuBackend
 
@@ -205,12 +206,22 @@ def cpu_baseline_matmul(n: int, rows: int):
     dt = time.perf_counter() - t0
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
     threads = int(os.environ.get("OMP_NUM_THREADS", cores))
+    # the other half of the headline metric on the same cores: ConvNet (batch 1000) train steps
+    cw = workloads.convnet(env, batch=1000, seed=3)
+    env.run(cw.graph, 1)  # warm
+    conv_steps = 6
+    t0 = time.perf_counter()
+    for i in range(conv_steps):
+        env.run(cw.graph, 2 + i)
+    conv_dt = time.perf_counter() - t0
     return {
         "value": 2.0 * rows * n * n / dt / 1e12,
         "unit": "TFLOP/s",
         "cores": min(cores, threads),
         "kind": "port",
-        "sample": f"{rows} rows of the {n}^3 product (A slab {rows}x{n}, full B), bias+leaky_relu included, {dt:.2f} s",
+        "sample": f"{rows} rows of the {n}^3 product (A slab {rows}x{n}, full B), bias+leaky_relu included, {dt:.2f} s; "
+                  f"plus {conv_steps} ConvNet bs1000 train steps, {conv_dt:.2f} s",
+        "convnet_bs1000_steps_per_s": conv_steps / conv_dt,
     }
 
 
@@ -224,7 +235,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only the streaming c=a*2+b kernel over 2^26 elements (counter calibration)")
-    ap.add_argument("--cpu-rows", type=int, default=256)
+    ap.add_argument("--cpu-rows", type=int, default=4096,
+                    help="rows of the headline product the CPU baseline computes (a bounded sample of the same workload)")
     ap.add_argument("--workload", default="headline",
                     choices=["headline", "matmul", "convnet", "relu-pe", "siren", "hash-grid"],
                     help="headline: the 8192^3 matmul line with the ConvNet step rate beside it (default); matmul: "
