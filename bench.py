@@ -191,6 +191,37 @@ def bench_reduce(env, rows, cols, axis, steps, warmup):
             "gbs": nbytes / (per_step_us * 1e-6) / 1e9, "frac_hbm": nbytes / (per_step_us * 1e-6) / 1e9 / HBM_PEAK_GBS}
 
 
+def bench_upload(env, n):
+    """Host -> device through the library's pinned staging ring (dsc_buf_write), and the headline product with the
+    upload of A and B inside the timed region (the rate a caller sees when its operands start in host memory)."""
+    from descent_amd import workloads
+
+    be = env.backend
+    w = workloads.matmul_epilogue(env, n, n, n, seed=2)
+    env.run(w.graph, 0)
+    be.sync()
+    rng = np.random.Generator(np.random.PCG64(4))
+    a = rng.standard_normal(n * n, dtype=np.float32)
+    b = rng.standard_normal(n * n, dtype=np.float32)
+    reps = 3
+    t0 = time.perf_counter()
+    for i in range(reps):
+        be.write(w.a.buffer, 0, a)
+        be.write(w.b.buffer, 0, b)
+        env.run(w.graph, i)
+    be.sync()
+    dt = (time.perf_counter() - t0) / reps
+    t0 = time.perf_counter()
+    be.write(w.a.buffer, 0, a)
+    be.sync()
+    up = time.perf_counter() - t0
+    for p in (w.a, w.b, w.bias, w.c):
+        if p.buffer is not None:
+            be.free(p.buffer)
+            p.buffer = None
+    return {"upload_gbs": a.nbytes / up / 1e9, "matmul_with_upload_tflops": w.flops / dt / 1e12, "ms_per_step_with_upload": dt * 1e3}
+
+
 def cpu_baseline_matmul(n: int, rows: int):
     """The CPU oracle (restatement of the reference's algorithm; the reference itself needs Rust + Vulkan) on
     a slab of `rows` rows of the same n^3 product, epilogue included, and on a few ConvNet train steps, all host
@@ -283,6 +314,7 @@ def main():
             r.pop("report")
             extra["matmul"].append(r)
         extra["elementwise_axpb_64M"] = bench_elementwise(env, 1 << 26, max(args.steps, 20), args.warmup)
+        extra["host_operands"] = bench_upload(env, n)
         extra["reduce"] = [bench_reduce(env, 8192, 8192, 1, 20, 3), bench_reduce(env, 8192, 8192, 0, 20, 3),
                            bench_reduce(env, 262144, 256, 0, 20, 3)]
         from descent_amd import workloads as _w

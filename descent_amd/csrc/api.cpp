@@ -132,6 +132,71 @@ int dsc_ctx_sync(dsc_ctx* ctx) {
     return DSC_OK;
 }
 
+int dsc_fence_record(dsc_ctx* ctx, uint64_t* out_fence) {
+    if (!ctx || !out_fence) return fail(DSC_ERR_INVALID, "null argument");
+    Context* c = &ctx->c;
+    hipEvent_t ev = nullptr;
+    if (!c->fence_pool.empty()) {
+        ev = c->fence_pool.back();
+        c->fence_pool.pop_back();
+    } else {
+        HIP_TRY(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+    }
+    hipError_t e = hipEventRecord(ev, c->stream);
+    if (e != hipSuccess) {
+        c->fence_pool.push_back(ev);
+        return fail(DSC_ERR_HIP, std::string("hipEventRecord: ") + hipGetErrorString(e));
+    }
+    *out_fence = c->fence_next++;
+    c->fences[*out_fence] = ev;
+    return DSC_OK;
+}
+
+namespace {
+// everything recorded at or before `fence` has finished: recycle those events
+void retire_fences(Context* c, uint64_t fence) {
+    while (!c->fences.empty() && c->fences.begin()->first <= fence) {
+        c->fence_pool.push_back(c->fences.begin()->second);
+        c->fences.erase(c->fences.begin());
+    }
+    if (fence > c->fence_retired) c->fence_retired = fence;
+}
+}  // namespace
+
+int dsc_fence_wait(dsc_ctx* ctx, uint64_t fence) {
+    if (!ctx) return fail(DSC_ERR_INVALID, "null context");
+    Context* c = &ctx->c;
+    if (fence == 0 || fence >= c->fence_next) return fail(DSC_ERR_INVALID, "unknown fence id");
+    if (fence <= c->fence_retired) return DSC_OK;
+    auto it = c->fences.find(fence);
+    if (it == c->fences.end()) return fail(DSC_ERR_INVALID, "unknown fence id");
+    HIP_TRY(hipEventSynchronize(it->second));
+    retire_fences(c, fence);  // the stream is in order: older fences have finished too
+    return DSC_OK;
+}
+
+int dsc_fence_query(dsc_ctx* ctx, uint64_t fence, int* out_finished) {
+    if (!ctx || !out_finished) return fail(DSC_ERR_INVALID, "null argument");
+    Context* c = &ctx->c;
+    if (fence == 0 || fence >= c->fence_next) return fail(DSC_ERR_INVALID, "unknown fence id");
+    if (fence <= c->fence_retired) {
+        *out_finished = 1;
+        return DSC_OK;
+    }
+    auto it = c->fences.find(fence);
+    if (it == c->fences.end()) return fail(DSC_ERR_INVALID, "unknown fence id");
+    const hipError_t e = hipEventQuery(it->second);
+    if (e == hipSuccess) {
+        *out_finished = 1;
+        retire_fences(c, fence);
+        return DSC_OK;
+    }
+    if (e != hipErrorNotReady) return fail(DSC_ERR_HIP, std::string("hipEventQuery: ") + hipGetErrorString(e));
+    (void)hipGetLastError();
+    *out_finished = 0;
+    return DSC_OK;
+}
+
 int dsc_ctx_stream(dsc_ctx* ctx, void** out_stream) {
     if (!ctx || !out_stream) return fail(DSC_ERR_INVALID, "null argument");
     *out_stream = ctx->c.stream;

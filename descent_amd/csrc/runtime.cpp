@@ -148,6 +148,8 @@ Context::~Context() {
         (void)hipEventDestroy(p.stop);
     }
     for (auto e : event_pool) (void)hipEventDestroy(e);
+    for (auto& kv : fences) (void)hipEventDestroy(kv.second);
+    for (auto e : fence_pool) (void)hipEventDestroy(e);
     for (int i = 0; i < kStagingRegions; ++i) {
         if (staging_done[i]) (void)hipEventDestroy(staging_done[i]);
         if (staging[i]) (void)hipHostFree(staging[i]);

@@ -98,6 +98,11 @@ struct Context {
 
     std::unordered_map<std::string, std::unique_ptr<Kernel>> kernels;  // by FusedKernel::key()
 
+    // fences: id -> event recorded on the stream; ids at or below `fence_retired` are known to have finished
+    std::map<uint64_t, hipEvent_t> fences;
+    std::vector<hipEvent_t> fence_pool;
+    uint64_t fence_next = 1, fence_retired = 0;
+
     bool profiling = false;
     std::vector<ProfileEntry> profile;
     std::vector<hipEvent_t> event_pool;

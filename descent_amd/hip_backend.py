@@ -45,6 +45,9 @@ def lib():
         "dsc_ctx_caps": (C.c_int, [vp, C.POINTER(_abi.CCaps)]),
         "dsc_ctx_sync": (C.c_int, [vp]),
         "dsc_ctx_stream": (C.c_int, [vp, C.POINTER(vp)]),
+        "dsc_fence_record": (C.c_int, [vp, C.POINTER(u64)]),
+        "dsc_fence_wait": (C.c_int, [vp, u64]),
+        "dsc_fence_query": (C.c_int, [vp, u64, C.POINTER(C.c_int)]),
         "dsc_buf_alloc": (C.c_int, [vp, sz, C.POINTER(u64)]),
         "dsc_buf_free": (C.c_int, [vp, u64]),
         "dsc_buf_info": (C.c_int, [vp, u64, C.POINTER(vp), C.POINTER(sz)]),
@@ -83,6 +86,7 @@ def lib():
 
 EXPORTED_SYMBOLS = [
     "dsc_last_error", "dsc_ctx_create", "dsc_ctx_destroy", "dsc_ctx_caps", "dsc_ctx_sync", "dsc_ctx_stream",
+    "dsc_fence_record", "dsc_fence_wait", "dsc_fence_query",
     "dsc_buf_alloc", "dsc_buf_free", "dsc_buf_info", "dsc_heap_stats", "dsc_buf_write", "dsc_buf_fill_zero",
     "dsc_buf_read", "dsc_kernel_get", "dsc_kernel_buffer_count", "dsc_kernel_reference_group_count",
     "dsc_kernel_label", "dsc_kernel_source", "dsc_kernel_launch", "dsc_codegen_source", "dsc_codegen_compile",
@@ -243,6 +247,20 @@ class HipBackend:
 
     def sync(self) -> None:
         check(lib().dsc_ctx_sync(self._ctx))
+
+    # -- fences (device/fence.rs) -------------------------------------------------------------------------
+    def fence_record(self) -> int:
+        f = C.c_uint64()
+        check(lib().dsc_fence_record(self._ctx, C.byref(f)))
+        return f.value
+
+    def fence_wait(self, fence: int) -> None:
+        check(lib().dsc_fence_wait(self._ctx, fence))
+
+    def fence_finished(self, fence: int) -> bool:
+        out = C.c_int()
+        check(lib().dsc_fence_query(self._ctx, fence, C.byref(out)))
+        return bool(out.value)
 
     # -- timing -----------------------------------------------------------------------------------------
     def profile(self, enabled: bool) -> None:

@@ -183,6 +183,15 @@ int dsc_ctx_destroy(dsc_ctx* ctx);
 int dsc_ctx_caps(dsc_ctx* ctx, dsc_caps* out);
 /* Replaces FenceSet::wait_for_signal on the latest fence (device/fence.rs:73-86). */
 int dsc_ctx_sync(dsc_ctx* ctx);
+/* FenceSet (device/fence.rs:21-86) as the reference uses it around command-buffer submission
+ * (device/command_buffer.rs:64-123): dsc_fence_record marks everything enqueued on the context so far and returns
+ * an id (next_unsignaled + the submit's signal); dsc_fence_wait blocks until that work has finished
+ * (wait_for_signal); dsc_fence_query answers without blocking (1 = finished).  Ids grow by one per record; waiting
+ * on an id also retires every older one.  A caller keeping two steps in flight, as the reference does, records a
+ * fence after each dsc_schedule_run and waits on the one from two steps ago. */
+int dsc_fence_record(dsc_ctx* ctx, uint64_t* out_fence);
+int dsc_fence_wait(dsc_ctx* ctx, uint64_t fence);
+int dsc_fence_query(dsc_ctx* ctx, uint64_t fence, int* out_finished);
 /* The HIP stream of the context as a hipStream_t (for event timing by a harness). */
 int dsc_ctx_stream(dsc_ctx* ctx, void** out_stream);
 

@@ -329,3 +329,27 @@ def test_scatter_add_chains_vs_float64(hip_backend_session, n, entries, links):
         assert "per-workgroup sums in LDS" in listing, listing
     assert rel_l2(got, want) <= TOL
     assert rel_l2(oracle, want) <= TOL
+
+
+def test_fences_order_work_like_the_reference_fence_set(hip_backend_session):
+    """device/fence.rs:21-86: ids grow by one, waiting on one retires the older ones, unknown ids are errors."""
+    from descent_amd import Environment, workloads
+    from descent_amd.hip_backend import DescentHipError
+
+    be = hip_backend_session
+    env = Environment(be)
+    w = workloads.matmul_epilogue(env, 1024, 1024, 1024, seed=3)
+    fences = []
+    for step in range(4):  # two steps in flight, as the reference keeps them (device/command_buffer.rs:64-123)
+        env.run(w.graph, step)
+        fences.append(be.fence_record())
+        if len(fences) > 2:
+            be.fence_wait(fences[-3])
+            assert be.fence_finished(fences[-3])
+    assert fences == list(range(fences[0], fences[0] + 4))
+    be.fence_wait(fences[-1])
+    assert all(be.fence_finished(f) for f in fences)
+    with pytest.raises(DescentHipError):
+        be.fence_wait(fences[-1] + 100)
+    with pytest.raises(DescentHipError):
+        be.fence_wait(0)
