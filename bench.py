@@ -262,6 +262,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--size", type=int, default=8192, help="M=N=K of the headline matmul")
+    ap.add_argument("--shape", default=None, help="M,N,K: with --workload matmul, time this matmul + bias + leaky_relu "
+                                                  "alone and print its line (e.g. under rocprofv3 --pmc)")
     ap.add_argument("--all", action="store_true", help="also time the other matmul shapes and the ConvNet step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -302,6 +304,12 @@ def main():
         print(json.dumps(out))
         return
     n = args.size
+    if args.shape:
+        m_, n_, k_ = (int(v) for v in args.shape.split(","))
+        r = bench_matmul(env, m_, n_, k_, args.steps, args.warmup)
+        sys.stderr.write(r.pop("report"))
+        print(json.dumps(r))
+        return
     head = bench_matmul(env, n, n, n, args.steps, args.warmup)
     sys.stderr.write(head["report"])
 
