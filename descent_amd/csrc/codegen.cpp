@@ -784,7 +784,9 @@ string gen_windows_to_image(Emitter& em, Generated* out) {
 bool scatter_privatised(const dsc_kernel_desc& d, int64_t* workgroups) {
     const int64_t table = element_count(d.shape), n = element_count(d.inputs[0].out_shape);
     if (table > 8192 || n < 16 * table || n < 65536) return false;
-    *workgroups = std::max<int64_t>(16, std::min<int64_t>(256, n / (4 * table)));
+    // every workgroup ends with one memory atomic per non-zero entry: enough workgroups to fill the machine, few
+    // enough that those closing atomics stay well below the values folded
+    *workgroups = std::max<int64_t>(64, std::min<int64_t>(512, n / (2 * table)));
     return true;
 }
 
@@ -797,30 +799,40 @@ string gen_scatter_add(Emitter& em, Generated* out) {
     int64_t wgs = 0;
     const bool priv = scatter_privatised(d, &wgs);
     const int64_t table = element_count(d.shape);
-    std::ostringstream k;
-    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
-    if (priv) {
-        k << "    __shared__ float acc[" << S(table) << "];\n";
-        k << "    for (int i = threadIdx.x; i < " << S(table) << "; i += 256) acc[i] = 0.f;\n    __syncthreads();\n";
-        k << "    for (uint gid = blockIdx.x * 256u + threadIdx.x; gid < " << S(n) << "u; gid += " << S(wgs * 256) << "u) {\n";
-    } else {
-        k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n    {\n";
-    }
-    auto c = em.emit_coords(k, vv.out_shape, "gid", "c");
-    k << "    const float value = " << em.load_view(fk.inputs[0], vv, c) << ";\n";
-    k << "    const int si = F2I(" << em.load_view(fk.inputs[1], vi, {c[d.axis]}) << ");\n";
     int64_t st[DSC_MAX_DIM];
     strides_of(d.shape, st);
-    string idx = "0";
-    for (int i = 0; i < d.shape.rank; ++i) idx += " + " + (i == d.axis ? string("si") : c[i]) + "*" + S(st[i]);
-    // bounds: an index outside the accumulator would be a wild write; the reference has no check, here it is dropped
-    k << "    if (si >= 0 && si < " << S(d.shape.dims[d.axis]) << ") ";
+    std::ostringstream k;
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
+    // value, index and target of element `gid` (names suffixed by `sfx`)
+    auto emit_element = [&](const string& gid, const string& sfx) {
+        auto c = em.emit_coords(k, vv.out_shape, gid, "c" + sfx + "_");
+        k << "    const float value" << sfx << " = " << em.load_view(fk.inputs[0], vv, c) << ";\n";
+        k << "    const int si" << sfx << " = F2I(" << em.load_view(fk.inputs[1], vi, {c[d.axis]}) << ");\n";
+        string idx = "0";
+        for (int i = 0; i < d.shape.rank; ++i) idx += " + " + (i == d.axis ? "si" + sfx : c[i]) + "*" + S(st[i]);
+        k << "    const int at" << sfx << " = " << idx << ";\n";
+        // bounds: an index outside the accumulator would be a wild write; the reference has no check, here it is dropped
+        k << "    const bool ok" << sfx << " = si" << sfx << " >= 0 && si" << sfx << " < " << S(d.shape.dims[d.axis]) << ";\n";
+    };
     if (priv) {
-        k << "atomicAdd(&acc[" << idx << "], value);\n    }\n    __syncthreads();\n";
+        const int U = 4;  // elements per thread and trip: their loads are all issued before the first LDS atomic
+        k << "    __shared__ float acc[" << S(table) << "];\n";
+        k << "    for (int i = threadIdx.x; i < " << S(table) << "; i += 256) acc[i] = 0.f;\n    __syncthreads();\n";
+        k << "    for (uint g0 = blockIdx.x * 256u + threadIdx.x; g0 < " << S(n) << "u; g0 += " << S(wgs * 256 * U) << "u) {\n";
+        for (int u = 0; u < U; ++u) {
+            k << "    const uint gid" << u << " = min(g0 + " << S(u * wgs * 256) << "u, " << S(n - 1) << "u);\n";
+            emit_element("gid" + to_string(u), to_string(u));
+        }
+        k << "    __builtin_amdgcn_sched_barrier(0);\n";
+        for (int u = 0; u < U; ++u)
+            k << "    if (ok" << u << " && g0 + " << S(u * wgs * 256) << "u < " << S(n) << "u) atomicAdd(&acc[at" << u << "], value" << u << ");\n";
+        k << "    }\n    __syncthreads();\n";
         k << "    for (int i = threadIdx.x; i < " << S(table) << "; i += 256) {\n        const float total = acc[i];\n";
         k << "        if (total != 0.f) unsafeAtomicAdd(&b" << fk.outputs[0] << "[i], total);\n    }\n}\n";
     } else {
-        k << "unsafeAtomicAdd(&b" << fk.outputs[0] << "[" << idx << "], value);\n    }\n}\n";
+        k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n";
+        emit_element("gid", "");
+        k << "    if (ok) unsafeAtomicAdd(&b" << fk.outputs[0] << "[at], value);\n}\n";
     }
     out->grid = priv ? (unsigned)wgs : blocks_for(n, 256);
     out->block = 256;
