@@ -1406,6 +1406,17 @@ string gen_matmul(Emitter& em, Generated* out) {
       << "\n#define C_ROW_STRIDE " << S(row_stride) << "\n";
     k << "#define MM_PARAMS " << em.kernel_params_decl() << "\n#define MM_ENTRY " << entry_name(fk) << "\n";
 
+    // results leave through LDS as 16-byte row pieces when the output allows it
+    bool vec_store = g.n % 4 == 0 && batch_stride % 4 == 0 && row_stride % 4 == 0 && (g.batch * g.m * g.n) % 4 == 0;
+    {
+        const int64_t sa = a_mode == 1 ? c.bm * (c.bk + 4) : c.bk * (c.bm + 8), sb = b_mode == 2 ? c.bn * (c.bk + 4) : c.bk * (c.bn + 8);
+        const int64_t per_wave = 32 * 36, waves = (int64_t)c.wm * c.wn;
+        const int64_t in_a = std::min(waves, 2 * sa / per_wave);
+        if ((waves - in_a) * per_wave > 2 * sb) vec_store = false;
+        if (const char* e = std::getenv("DSC_MM_VEC_STORE"))
+            if (e[0] == '0') vec_store = false;
+    }
+    k << "#define MM_VEC_STORE " << (vec_store ? 1 : 0) << "\n";
     if (fk.has_epilogue) {
         const dsc_kernel_desc& pe = fk.epilogue.raw();
         std::ostringstream body;
@@ -1419,11 +1430,27 @@ string gen_matmul(Emitter& em, Generated* out) {
         form.coefs = {batch_stride, row_stride, 1};
         form.extents = {g.batch, g.m, g.n};
         em.emit_pe(body, pe, fk.epilogue_inputs, "gid", "e", ov, &form);
-        for (int o = 0; o < pe.n_outputs; ++o) body << "    b" << fk.outputs[o] << "[gid] = et" << pe.outputs[o] << ";\n";
-        em.funcs << "DSC_INLINE void mm_store(float product, int gid, int cb, int cm, int cn, " << em.params_decl() << ") {\n" << body.str() << "}\n";
+        for (int o = 0; o < pe.n_outputs; ++o) body << "    result[" << o << "] = et" << pe.outputs[o] << ";\n";
+        em.funcs << "DSC_INLINE void mm_epilogue(float product, int gid, int cb, int cm, int cn, float* result, " << em.params_decl() << ") {\n"
+                 << body.str() << "}\n";
+        std::ostringstream one, four;
+        one << "DSC_INLINE void mm_store(float product, int gid, int cb, int cm, int cn, " << em.params_decl() << ") {\n";
+        one << "    float res[" << pe.n_outputs << "];\n    mm_epilogue(product, gid, cb, cm, cn, res, " << em.params_pass() << ");\n";
+        for (int o = 0; o < pe.n_outputs; ++o) one << "    b" << fk.outputs[o] << "[gid] = res[" << o << "];\n";
+        one << "}\n";
+        four << "DSC_INLINE void mm_store4(float4 p, int gid, int cb, int cm, int cn, " << em.params_decl() << ") {\n";
+        four << "    const float pv[4] = {p.x, p.y, p.z, p.w};\n    float res[4][" << pe.n_outputs << "];\n";
+        four << "#pragma unroll\n    for (int j = 0; j < 4; ++j) mm_epilogue(pv[j], gid + j, cb, cm, cn + j, res[j], " << em.params_pass() << ");\n";
+        for (int o = 0; o < pe.n_outputs; ++o)
+            four << "    *(float4*)(b" << fk.outputs[o] << " + gid) = make_float4(res[0][" << o << "], res[1][" << o << "], res[2][" << o
+                 << "], res[3][" << o << "]);\n";
+        four << "}\n";
+        em.funcs << one.str() << four.str();
         k << "#define MM_STORE(v, idx, b, m, n) mm_store(v, idx, b, m, n, " << em.params_pass() << ")\n";
+        k << "#define MM_STORE4(v, idx, b, m, n) mm_store4(v, idx, b, m, n, " << em.params_pass() << ")\n";
     } else {
         k << "#define MM_STORE(v, idx, b, m, n) b" << fk.outputs[0] << "[idx] = (v)\n";
+        k << "#define MM_STORE4(v, idx, b, m, n) *(float4*)(b" << fk.outputs[0] << " + (idx)) = (v)\n";
     }
     k << kMatmulMfmaSource;
 
@@ -1560,7 +1587,7 @@ std::string FusedKernel::key() const {
     s.append(reinterpret_cast<const char*>(&n_buffers), 4);
     if (const char* env = std::getenv("DSC_MM_TILE"))
         if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|T") + env;
-    for (const char* name : {"DSC_MM_PERSISTENT", "DSC_MM_DEEP_K", "DSC_MM_ROWS", "DSC_ROWS_R", "DSC_ROWS_UNROLL", "DSC_ROWS_B", "DSC_ROWS_DIRECT_STORE", "DSC_MM_TALLK", "DSC_TALLK_UNROLL"})
+    for (const char* name : {"DSC_MM_VEC_STORE", "DSC_MM_PERSISTENT", "DSC_MM_DEEP_K", "DSC_MM_ROWS", "DSC_ROWS_R", "DSC_ROWS_UNROLL", "DSC_ROWS_B", "DSC_ROWS_DIRECT_STORE", "DSC_MM_TALLK", "DSC_TALLK_UNROLL"})
         if (const char* env = std::getenv(name))
             if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|") + name + env;
     return s;
