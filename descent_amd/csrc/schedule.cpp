@@ -206,6 +206,7 @@ dsc_view identity_view(std::initializer_list<int64_t> dims) {
 // ---------------------------------------------------------------------------------------------------------
 
 int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags) {
+    graph_replay = (flags & DSC_SCHEDULE_GRAPH_REPLAY) != 0;
     n_nodes = desc.n_nodes;
     n_params = desc.n_params;
     n_clusters = desc.n_clusters;
@@ -1247,13 +1248,14 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
         }
         return DSC_OK;
     };
-    static const bool graphs_enabled = [] {
-        // opt-in: replay needs a step's buffers to land on the same addresses again, which the shared best-fit
-        // heap does not guarantee (parameter buffers move every step), so by default launches are enqueued directly
+    // opt-in (DSC_SCHEDULE_GRAPH_REPLAY, or DSC_GRAPHS=1 for every schedule): replay needs a step's buffers to land
+    // on the same addresses again, which the shared best-fit heap does not guarantee (parameter buffers move every
+    // step), so by default launches are enqueued directly
+    static const bool graphs_by_env = [] {
         const char* e = std::getenv("DSC_GRAPHS");
         return e && e[0] == '1';
     }();
-    if (ctx->profiling || !graphs_enabled || launches.size() < 4) {
+    if (ctx->profiling || !(graph_replay || graphs_by_env) || launches.size() < 4) {
         ++direct_runs;
         return enqueue_all();
     }

@@ -33,6 +33,7 @@ struct Schedule {
     static constexpr size_t kMaxCaptured = 8;
     std::vector<CapturedStep> captured;
     int64_t replays = 0, direct_runs = 0;
+    bool graph_replay = false;  // DSC_SCHEDULE_GRAPH_REPLAY
     ~Schedule();
 
     int n_nodes = 0, n_params = 0, n_clusters = 0;

@@ -294,6 +294,9 @@ typedef struct dsc_schedule dsc_schedule;
 
 /* flags for dsc_schedule_create */
 #define DSC_SCHEDULE_NO_FUSION 1u /* launch exactly one kernel per reference cluster (for parity tests) */
+#define DSC_SCHEDULE_GRAPH_REPLAY 4u /* capture each run's launches as a HIP graph and replay it whenever a later run's
+                                        buffers land on the same addresses (the Submit half of the reference's
+                                        command buffer, device/command_buffer.rs:64-123, recorded once) */
 #define DSC_SCHEDULE_NO_CONV_KERNELS 2u /* keep convolution gradients on the generic MatMul path (fused producers)
                                            instead of the dedicated LDS-tiled kernels (for parity tests) */
 

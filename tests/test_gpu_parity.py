@@ -353,3 +353,28 @@ def test_fences_order_work_like_the_reference_fence_set(hip_backend_session):
         be.fence_wait(fences[-1] + 100)
     with pytest.raises(DescentHipError):
         be.fence_wait(0)
+
+
+def test_graph_replay_matches_direct_launches_on_every_replay(hip_backend_session):
+    """Ten ConvNet steps (batch 16, a new dropout seed each step) with HIP-graph replay against the same steps on
+    the oracle, parameters compared after every step: replays after the first must see the new seed (it travels
+    through a device cell) and the same buffers, with eager uploads and reads between them."""
+    from descent_amd import workloads
+
+    genv, cenv = _envs(hip_backend_session, fused="graph-replay")
+    gw = workloads.convnet(genv, batch=16, seed=17)
+    cw = workloads.convnet(cenv, batch=16, seed=17)
+    for step in range(10):
+        genv.run(gw.graph, 300 + step)
+        cenv.run(cw.graph, 300 + step)
+        got, want = gw.snapshot(), cw.snapshot()  # eager device-to-host reads between the replays
+        for key in want:
+            if key == "accuracy":
+                assert np.array_equal(got[key], want[key]), (step, key)
+            else:
+                assert rel_l2(got[key], want[key]) <= TOL, (step, key, rel_l2(got[key], want[key]))
+    listing = next(iter(gw.graph.__dict__["_schedules"].values())).describe()
+    import re
+    m = re.search(r"graph replays (\d+), captured (\d+), direct runs (\d+)", listing)
+    assert m and int(m.group(1)) + int(m.group(2)) + int(m.group(3)) >= 10, listing
+    assert int(m.group(2)) >= 1, listing  # at least one capture happened
