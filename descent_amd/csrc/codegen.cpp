@@ -358,6 +358,7 @@ struct Emitter {
 };
 
 bool rows_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
+bool smallk_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
 bool tallk_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
 
 // Entry points carry the kernel kind and its size, so that a profiler's per-name statistics tell the kernels of
@@ -380,7 +381,10 @@ string entry_name(const FusedKernel& fk) {
     }
     case DSC_KERNEL_MATMUL: {
         const MatMulDims g = matmul_dims(d);
-        string base = rows_kernel_applies(fk, g) ? "dsc_matmul_rows" : (tallk_kernel_applies(fk, g) ? "dsc_matmul_tallk" : "dsc_matmul_mfma");
+        string base = rows_kernel_applies(fk, g)     ? "dsc_matmul_rows"
+                      : smallk_kernel_applies(fk, g) ? "dsc_matmul_shortk"
+                      : tallk_kernel_applies(fk, g)  ? "dsc_matmul_tallk"
+                                                     : "dsc_matmul_mfma";
         if (fk.has_epilogue) base += "_epilogue";
         return base + "_b" + count(g.batch) + "_m" + count(g.m) + "_n" + count(g.n) + "_k" + count(g.k);
     }
@@ -1110,6 +1114,74 @@ bool rows_kernel_applies(const FusedKernel& fk, const MatMulDims& g) {
     return g.n <= 32 && g.k <= 256 && g.k * g.n <= 8192 && g.m * g.batch >= 16384;
 }
 
+// Products with a very short k (the three input coordinates or output channels of a coordinate network: k <= 8) are
+// outer-product sums, bound by streaming C: one thread computes four adjacent columns of one row, A's k values
+// and B's 16-byte pieces come from L1, and the fused consumer runs on the four results before one 16-byte store
+// per output.  No LDS, no MFMA.
+bool smallk_kernel_applies(const FusedKernel& fk, const MatMulDims& g) {
+    if (const char* e = std::getenv("DSC_MM_SMALLK"))
+        if (e[0] == '0') return false;
+    if (g.chunks != 1 && !fk.sum_chunks) return false;
+    const bool rows = fk.main.raw().output_mode == DSC_MATMUL_ROWS;
+    const int64_t batch_stride = rows ? g.n : g.m * g.n, row_stride = rows ? g.batch * g.n : g.n;
+    return g.k <= 8 && g.n >= 16 && g.n % 4 == 0 && batch_stride % 4 == 0 && row_stride % 4 == 0 && g.m * g.n * g.batch >= 65536;
+}
+
+string gen_matmul_smallk(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const MatMulDims g = matmul_dims(d);
+    const bool rows = d.output_mode == DSC_MATMUL_ROWS;
+    const int64_t batch_stride = rows ? g.n : g.m * g.n, row_stride = rows ? g.batch * g.n : g.n;
+    const int n_out = fk.has_epilogue ? fk.epilogue.raw().n_outputs : 1;
+    const string la = em.load_view(fk.inputs[0], d.inputs[0], {"cb", "cm", "ck"});
+    em.funcs << "DSC_INLINE float load_a(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return " << la << ";\n}\n";
+    const string lb = em.load_view(fk.inputs[1], d.inputs[1], {"cb", "ck", "cn"});
+    em.funcs << "DSC_INLINE float load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb << ";\n}\n";
+    if (fk.has_epilogue) {
+        const dsc_kernel_desc& pe = fk.epilogue.raw();
+        std::ostringstream body;
+        std::map<int, string> ov;
+        ov[fk.epilogue_product_input] = "product";
+        IndexForm form;
+        form.valid = true;
+        form.names = {"cb", "cm", "cn"};
+        form.coefs = {batch_stride, row_stride, 1};
+        form.extents = {g.batch, g.m, g.n};
+        em.emit_pe(body, pe, fk.epilogue_inputs, "gid", "e", ov, &form);
+        for (int o = 0; o < pe.n_outputs; ++o) body << "    result[" << o << "] = et" << pe.outputs[o] << ";\n";
+        em.funcs << "DSC_INLINE void mm_epilogue(float product, int gid, int cb, int cm, int cn, float* result, " << em.params_decl() << ") {\n"
+                 << body.str() << "}\n";
+    }
+    const int64_t nq = g.n / 4, total = g.batch * g.m * nq;
+    if (total >= kMaxIndex) return "matmul: too large";
+    std::ostringstream k;
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
+    k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
+    k << "    const uint t = blockIdx.x * 256u + threadIdx.x;\n    if (t >= " << S(total) << "u) return;\n";
+    k << "    const int cn = (int)(t % " << S(nq) << "u) * 4, cm = (int)((t / " << S(nq) << "u) % " << S(g.m) << "u), cb = (int)(t / " << S(nq * g.m) << "u);\n";
+    k << "    float acc[4] = {0.f, 0.f, 0.f, 0.f};\n";
+    k << "#pragma unroll\n    for (int ck = 0; ck < " << S(g.k) << "; ++ck) {\n";
+    k << "        const float a = load_a(cb, cm, ck, " << em.params_pass() << ");\n";
+    k << "#pragma unroll\n        for (int j = 0; j < 4; ++j) acc[j] = fmaf(a, load_b(cb, ck, cn + j, " << em.params_pass() << "), acc[j]);\n    }\n";
+    k << "    const int c_at = cb * " << S(batch_stride) << " + cm * " << S(row_stride) << " + cn;\n";
+    if (fk.has_epilogue) {
+        k << "    float res[4][" << n_out << "];\n";
+        k << "#pragma unroll\n    for (int j = 0; j < 4; ++j) mm_epilogue(acc[j], c_at + j, cb, cm, cn + j, res[j], " << em.params_pass() << ");\n";
+        for (int o = 0; o < n_out; ++o)
+            k << "    *(float4*)(b" << fk.outputs[o] << " + c_at) = make_float4(res[0][" << o << "], res[1][" << o << "], res[2][" << o << "], res[3]["
+              << o << "]);\n";
+    } else {
+        k << "    *(float4*)(b" << fk.outputs[0] << " + c_at) = make_float4(acc[0], acc[1], acc[2], acc[3]);\n";
+    }
+    k << "}\n";
+    out->grid = blocks_for(total, 256);
+    out->block = 256;
+    out->source = k.str();
+    out->note = string("short-k fma, four columns per thread") + (fk.has_epilogue ? " +epilogue" : "");
+    return "";
+}
+
 string gen_matmul_rows(Emitter& em, Generated* out) {
     const FusedKernel& fk = em.fk;
     const dsc_kernel_desc& d = fk.main.raw();
@@ -1348,6 +1420,7 @@ string gen_matmul(Emitter& em, Generated* out) {
     const dsc_view& vb = d.inputs[1];
     const bool rows = d.output_mode == DSC_MATMUL_ROWS;
     if (rows_kernel_applies(fk, g)) return gen_matmul_rows(em, out);
+    if (smallk_kernel_applies(fk, g)) return gen_matmul_smallk(em, out);
     if (tallk_kernel_applies(fk, g)) return gen_matmul_tallk(em, out);
     const bool split = !fk.sum_chunks && g.chunks > 1;
     MmConfig c = pick_config(g.m, g.n, split ? chunk_k_of(g) : g.k, g.batch * (split ? g.chunks : 1));
@@ -1587,7 +1660,7 @@ std::string FusedKernel::key() const {
     s.append(reinterpret_cast<const char*>(&n_buffers), 4);
     if (const char* env = std::getenv("DSC_MM_TILE"))
         if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|T") + env;
-    for (const char* name : {"DSC_MM_VEC_STORE", "DSC_MM_PERSISTENT", "DSC_MM_DEEP_K", "DSC_MM_ROWS", "DSC_ROWS_R", "DSC_ROWS_UNROLL", "DSC_ROWS_B", "DSC_ROWS_DIRECT_STORE", "DSC_MM_TALLK", "DSC_TALLK_UNROLL"})
+    for (const char* name : {"DSC_MM_SMALLK", "DSC_MM_VEC_STORE", "DSC_MM_PERSISTENT", "DSC_MM_DEEP_K", "DSC_MM_ROWS", "DSC_ROWS_R", "DSC_ROWS_UNROLL", "DSC_ROWS_B", "DSC_ROWS_DIRECT_STORE", "DSC_MM_TALLK", "DSC_TALLK_UNROLL"})
         if (const char* env = std::getenv(name))
             if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|") + name + env;
     return s;

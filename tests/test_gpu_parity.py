@@ -33,6 +33,8 @@ def test_reference_known_answers(hip_backend_session, mode):
 MATMUL_SHAPES = [
     (1, 1, 1), (16, 16, 16), (33, 17, 9), (128, 128, 128), (100, 10, 784), (1000, 128, 784), (257, 130, 1030),
     (64, 300, 2100), (9, 16, 5000),
+    # very short k with a wide output: the short-k kernel
+    (20000, 64, 3), (5000, 256, 8), (70000, 16, 1),
     # small outputs over a long k: the tall-k kernel (ragged tiles, one tile, many tiles)
     (9, 16, 50000), (72, 16, 70000), (33, 50, 140000), (250, 3, 66000),
 ]
