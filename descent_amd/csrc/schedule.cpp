@@ -1021,7 +1021,10 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                 for (int c : consumers_of(node)) (void)c, ++readers;  // nobody may read the intermediate sum
                 if (readers != 0) break;
                 chain.push_back(next);
-                if (chain.size() >= 8) break;
+                // every link may keep a copy of the accumulator in LDS (small tables): stay well inside the 160 KiB
+                const int64_t table = element_count(drafts[i].fk.main.raw().shape);
+                const int64_t max_links = table <= 8192 ? std::max<int64_t>(2, std::min<int64_t>(8, 32768 / table)) : 8;
+                if ((int64_t)chain.size() >= max_links) break;
             }
             if (chain.size() < 2) continue;
             const int last = chain.back();

@@ -380,3 +380,56 @@ def test_graph_replay_matches_direct_launches_on_every_replay(hip_backend_sessio
     m = re.search(r"graph replays (\d+), captured (\d+), direct runs (\d+)", listing)
     assert m and int(m.group(1)) + int(m.group(2)) + int(m.group(3)) >= 10, listing
     assert int(m.group(2)) >= 1, listing  # at least one capture happened
+
+
+def _conv_grad_case(env, m, h, w, c_in, c_out, fh, fw, pad, groups, seed):
+    """x -> conv2d -> 0.5 * sum(y^2): the gradients with respect to the image and the filter."""
+    from descent_amd import Initializer
+
+    rng = np.random.default_rng(seed)
+    xp = env.trainable_parameter([m, h, w, c_in], "x", Initializer.zero())
+    fp = env.trainable_parameter([groups, c_out // groups, fh, fw, c_in // groups], "f", Initializer.zero())
+    env.write_parameter(xp, rng.standard_normal((m, h, w, c_in), dtype=np.float32))
+    env.write_parameter(fp, rng.standard_normal((groups, c_out // groups, fh, fw, c_in // groups), dtype=np.float32) * 0.2)
+    dx, df = env.static_parameter([m, h, w, c_in], "dx"), env.static_parameter(list(fp.shape), "df")
+    y_out = env.static_parameter([m, h + 2 * pad - fh + 1, w + 2 * pad - fw + 1, c_out], "y")
+
+    def build(s):
+        x, f = s.parameter(xp), s.parameter(fp)
+        y = x.conv2d(f, pad)
+        s.write_parameter_value(y_out, y.value() * 1.0)
+        (y.square() * 0.5).set_loss()
+        s.write_parameter_value(dx, x.loss_grad())
+        s.write_parameter_value(df, f.loss_grad())
+
+    g = env.build_graph(build)
+    env.run(g, 0)
+    return g, env.read_parameter(y_out), env.read_parameter(dx), env.read_parameter(df)
+
+
+CONV_GEOMETRIES = [
+    # m, h, w, c_in, c_out, fh, fw, pad, groups
+    (64, 14, 14, 16, 32, 3, 3, 1, 2),   # the ConvNet's second convolution
+    (50, 12, 10, 4, 8, 3, 3, 1, 1),     # not square
+    (40, 9, 9, 8, 8, 5, 5, 2, 2),       # 5x5 taps, pad 2
+    (30, 20, 20, 4, 4, 3, 3, 1, 1),     # padded image larger than one pass of 256 pixels
+    (60, 8, 8, 4, 8, 3, 3, 0, 1),       # no padding: no Unpads to fold
+    (25, 7, 5, 16, 16, 3, 1, 0, 1),     # 3x1 taps
+    (3, 6, 6, 64, 64, 3, 3, 1, 1),      # many channels: stays on the generic path
+]
+
+
+@pytest.mark.parametrize("geom", CONV_GEOMETRIES, ids=lambda g: "x".join(map(str, g)))
+@pytest.mark.parametrize("fused", [True, "generic-conv", False])
+def test_conv2d_gradients_over_geometries(hip_backend_session, geom, fused):
+    genv, cenv = _envs(hip_backend_session, fused=fused)
+    g, gy, gdx, gdf = _conv_grad_case(genv, *geom, seed=90)
+    _, cy, cdx, cdf = _conv_grad_case(cenv, *geom, seed=90)
+    listing = next(iter(g.__dict__["_schedules"].values())).describe()
+    if fused is True:  # all but the many-channel case run the dedicated data-gradient kernel
+        assert ("ConvDataGrad" in listing) == (geom is not CONV_GEOMETRIES[-1]), listing
+    if fused == "generic-conv" and geom is not CONV_GEOMETRIES[-1]:
+        assert "<2 fused producers>" in listing, listing
+    assert rel_l2(gy, cy) <= TOL, listing
+    assert rel_l2(gdx, cdx) <= TOL, (rel_l2(gdx, cdx), listing)
+    assert rel_l2(gdf, cdf) <= TOL, (rel_l2(gdf, cdf), listing)
