@@ -1676,8 +1676,13 @@ bool conv_dgrad_fits(const FusedKernel::ConvDgrad& c, int64_t k) {
 }
 
 bool can_be_part(const FusedKernel& fk) {
-    if (!fk.parts.empty() || fk.dgrad.on) return false;
-    return fk.main.raw().kind != DSC_KERNEL_MATMUL;  // the MatMul kernels size their workgroups per shape
+    if (!fk.parts.empty()) return false;
+    if (fk.dgrad.on || !fk.row_stages.empty()) return true;
+    if (fk.main.raw().kind != DSC_KERNEL_MATMUL) return true;
+    // of the MatMul kernels, the row-per-thread, short-k and tall-k ones run 256 threads addressed by blockIdx.x; the
+    // MFMA template sizes its workgroups per shape and reads the grid size
+    const MatMulDims g = matmul_dims(fk.main.raw());
+    return rows_kernel_applies(fk, g) || smallk_kernel_applies(fk, g) || tallk_kernel_applies(fk, g);
 }
 
 static std::string generate_one(const FusedKernel& fk, Generated* out, bool with_prelude);

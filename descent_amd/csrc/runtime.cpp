@@ -278,7 +278,8 @@ Kernel* get_kernel(Context* ctx, const FusedKernel& fk, int* status) {
     if (!fk.virtuals.empty()) k->label += " <" + std::to_string(fk.virtuals.size()) + " fused producers>";
     if (!fk.parts.empty()) {
         k->label = "Multi (" + std::to_string(fk.parts.size()) + " kernels:";
-        for (auto& part : fk.parts) k->label += " " + std::string(part.row_stages.empty() ? label_name(part.main.raw()) : "RowFused") + ";";
+        for (auto& part : fk.parts)
+            k->label += " " + std::string(part.dgrad.on ? "ConvDataGrad" : part.row_stages.empty() ? label_name(part.main.raw()) : "RowFused") + ";";
         k->label += ")";
     }
     k->reference_groups = reference_group_count(fk.main.raw());

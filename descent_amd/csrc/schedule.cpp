@@ -1062,27 +1062,30 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
 
         // Pass 4: launches of a few workgroups each (optimiser updates of small tensors, short reductions, scalar
         // bookkeeping) cost a launch apiece while using a fraction of the machine.  Runs of them that do not
-        // depend on one another become one multi-part launch; a later small launch is hoisted into the run when
-        // nothing it reads is produced in between.
+        // depend on one another become one multi-part launch; a later launch is hoisted into the run when nothing
+        // it reads is produced in between.  One large kernel may ride along (its workgroups come last, so the
+        // small parts start at once and finish in its shadow).
         {
             static const int64_t small_grid = std::getenv("DSC_MULTI_GRID") ? std::atoll(std::getenv("DSC_MULTI_GRID")) : 1024;
-            std::vector<int> grid_of(drafts.size(), -1);
-            auto small = [&](int i) {
+            std::vector<int64_t> grid_of(drafts.size(), -1);
+            auto partable = [&](int i) {
                 const Draft& d = drafts[i];
                 if (!d.alive || !can_be_part(d.fk)) return false;
                 for (auto& o : d.outs)
                     if (o.copy_from >= 0) return false;
                 if (grid_of[i] < 0) {
                     Generated g;
-                    if (!generate(d.fk, &g).empty() || g.block != 256) { grid_of[i] = 1 << 30; return false; }
-                    grid_of[i] = (int)std::min<unsigned>(g.grid, 1u << 30);
+                    if (!generate(d.fk, &g).empty() || g.block != 256) { grid_of[i] = (int64_t)1 << 40; return false; }
+                    grid_of[i] = g.grid;
                 }
-                return grid_of[i] <= small_grid;
+                return grid_of[i] < ((int64_t)1 << 30);
             };
             std::vector<bool> taken(drafts.size(), false);
             for (int i = 0; i < (int)drafts.size() && small_grid > 0; ++i) {
-                if (taken[i] || !small(i)) continue;
+                if (taken[i] || !partable(i)) continue;
                 std::vector<int> batch{i};
+                int large = grid_of[i] > small_grid ? 1 : 0;
+                int64_t total_grid = grid_of[i];
                 std::set<int> blocked, bound;
                 for (auto& o : drafts[i].outs) blocked.insert(o.node);
                 for (int nd : drafts[i].params) bound.insert(nd);
@@ -1093,12 +1096,18 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                         if (blocked.count(nd)) depends = true;
                     std::set<int> would = bound;
                     for (int nd : drafts[j].params) would.insert(nd);
-                    if (!depends && batch.size() < 16 && would.size() <= 48 && small(j)) {
+                    if (!depends && batch.size() < 16 && would.size() <= 48 && partable(j) && (grid_of[j] <= small_grid || large == 0) &&
+                        total_grid + grid_of[j] < ((int64_t)1 << 30)) {
                         batch.push_back(j);
                         bound = would;
+                        large += grid_of[j] > small_grid ? 1 : 0;
+                        total_grid += grid_of[j];
                     }
                     for (auto& o : drafts[j].outs) blocked.insert(o.node);
                 }
+                // a lone large kernel with nothing small to carry stays as it is
+                if (batch.size() < 2) continue;
+                std::stable_sort(batch.begin(), batch.end(), [&](int a, int b) { return grid_of[a] < grid_of[b]; });
                 if (batch.size() < 2) continue;
                 Draft multi;
                 multi.fk.main = drafts[i].fk.main;

@@ -162,7 +162,7 @@ def test_convnet_graph_shape():
     assert sum(p.shape.element_count() for p in w.trainable) == 204618
     listing = hip_backend.check_schedule(w.graph, fused=True)
     launches = int(listing.split()[0])
-    assert launches < 40, listing
+    assert launches < 30, listing
     # softmax cross-entropy and the accuracy count: one row-fused launch over the [1000, 10] logits
     assert "RowFused [1000, 10] (8 clusters)" in listing
     # small independent launches (optimiser updates of small tensors, short reductions) share launches
@@ -172,8 +172,8 @@ def test_convnet_graph_shape():
     assert set(covered) == set(range(66))
     # the data gradient of the second convolution: MatMul + reshape copy + WindowsToImage as one product over
     # the padded image, both operands fused producers
-    assert "ConvDataGrad [1000, 14, 14, 16] 3x3 taps, 2 groups" in listing
-    assert "MatMul (k=144) [1, 256000, 2, 8] <2 fused producers>" in hip_backend.check_schedule(w.graph, fused="generic-conv")
+    assert "ConvDataGrad" in listing and "conv data gradient: workgroup per image and group, tile in LDS, 3x3 taps x 16 channels, border folds fused" in listing
+    assert "MatMul (k=144) [1, 256000, 2, 8]" in hip_backend.check_schedule(w.graph, fused="generic-conv")
     # the work figures of the listing: the eleven GEMMs of the step as the reference runs them
     assert "4.373 GFLOP in MatMuls" in hip_backend.check_schedule(w.graph, fused=False)
 
