@@ -635,7 +635,7 @@ string gen_reduce(Emitter& em, Generated* out) {
         k << "    if (vid < " << S(n_vec) << "u) {\n";
         k << "    const uint oid = vid * 4u;\n";
         auto oc = em.emit_coords(k, d.shape, "oid", "oc");
-        const int U = pick_unroll(TK, 4);
+        const int U = pick_unroll(TK, std::getenv("DSC_REDUCE_VEC_UNROLL") ? std::atoi(std::getenv("DSC_REDUCE_VEC_UNROLL")) : 16);
         const char* comps[4] = {"x", "y", "z", "w"};
         for (int u = 0; u < U; ++u) k << (u ? ", a" : "    float4 a") << u << " = result";
         k << ";\n    int kb = " << (TK > 1 ? "tk" : "0") << ";\n";
