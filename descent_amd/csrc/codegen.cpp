@@ -1114,7 +1114,7 @@ bool rows_kernel_applies(const FusedKernel& fk, const MatMulDims& g) {
     return g.n <= 32 && g.k <= 256 && g.k * g.n <= 8192 && g.m * g.batch >= 16384;
 }
 
-// Products with a very short k (the three input coordinates or output channels of a coordinate network: k <= 8) are
+// Products with a very short k (the three input coordinates or output channels of a coordinate network: k <= 16) are
 // outer-product sums, bound by streaming C: one thread computes four adjacent columns of one row, A's k values
 // and B's 16-byte pieces come from L1, and the fused consumer runs on the four results before one 16-byte store
 // per output.  No LDS, no MFMA.
@@ -1124,7 +1124,7 @@ bool smallk_kernel_applies(const FusedKernel& fk, const MatMulDims& g) {
     if (g.chunks != 1 && !fk.sum_chunks) return false;
     const bool rows = fk.main.raw().output_mode == DSC_MATMUL_ROWS;
     const int64_t batch_stride = rows ? g.n : g.m * g.n, row_stride = rows ? g.batch * g.n : g.n;
-    return g.k <= 8 && g.n >= 16 && g.n % 4 == 0 && batch_stride % 4 == 0 && row_stride % 4 == 0 && g.m * g.n * g.batch >= 65536;
+    return g.k <= 16 && g.n >= 16 && g.n % 4 == 0 && batch_stride % 4 == 0 && row_stride % 4 == 0 && g.m * g.n * g.batch >= 65536;
 }
 
 string gen_matmul_smallk(Emitter& em, Generated* out) {
