@@ -271,7 +271,7 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=4096,
                     help="rows of the headline product the CPU baseline computes (a bounded sample of the same workload)")
     ap.add_argument("--workload", default="headline",
-                    choices=["headline", "matmul", "convnet", "relu-pe", "siren", "hash-grid"],
+                    choices=["headline", "matmul", "convnet", "linear", "relu-pe", "siren", "hash-grid"],
                     help="headline: the 8192^3 matmul line with the ConvNet step rate beside it (default); matmul: "
                          "that line without the ConvNet; the others run one workload alone, e.g. under rocprofv3")
     ap.add_argument("--no-events", action="store_true", help="no per-launch HIP events (wall time only)")
@@ -296,7 +296,7 @@ def main():
             out = bench_convnet(env, args.steps, args.warmup)
             sys.stderr.write(out.pop("report"))
         else:
-            build = {"relu-pe": lambda e: _w.coordinate_mlp(e), "siren": lambda e: _w.coordinate_mlp(e, variant="siren"),
+            build = {"linear": lambda e: _w.linear_classifier(e), "relu-pe": lambda e: _w.coordinate_mlp(e), "siren": lambda e: _w.coordinate_mlp(e, variant="siren"),
                      "hash-grid": lambda e: _w.hash_grid_fit(e)}[args.workload]
             out, rep = bench_workload(env, build, args.steps, args.warmup, topn=int(os.environ.get("DSC_BENCH_TOPN", "12")))
             sys.stderr.write(rep)
@@ -332,6 +332,9 @@ def main():
         extra["coordinate_mlp_relu_pe_512"] = mlp
         siren, rep = bench_workload(env, lambda e: _w.coordinate_mlp(e, variant="siren"), 10, 2)
         extra["coordinate_mlp_siren_512"] = siren
+        lin, rep = bench_workload(env, lambda e: _w.linear_classifier(e), 50, 5)
+        sys.stderr.write("cfg1 linear classifier:\n" + rep)
+        extra["linear_classifier_bs1000"] = lin
         hg, rep = bench_workload(env, lambda e: _w.hash_grid_fit(e), 10, 2)
         sys.stderr.write("cfg5 hash grid:\n" + rep)
         sc = hg["kernel_classes"].get("Multi (4 kernels: ScatterAdd") or hg["kernel_classes"].get("ScatterAdd")

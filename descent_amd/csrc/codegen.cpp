@@ -927,8 +927,8 @@ string gen_row_fused(Emitter& em, Generated* out) {
 int64_t dgrad_pitch(int64_t k) { return k % 8 == 0 ? k + 4 : k; }  // keeps 16-byte reads of neighbouring pixels off one bank
 
 int64_t dgrad_lds_floats(const FusedKernel::ConvDgrad& c, int64_t k) {
-    const int64_t th = c.oh + 2 * (c.fh - 1), tw = c.ow + 2 * (c.fw - 1), ph = c.oh + c.fh - 1, pw = c.ow + c.fw - 1;
-    return std::max(th * tw * dgrad_pitch(k), (c.pad_h || c.pad_w) ? ph * pw * c.c : 0);
+    const int64_t ph = c.oh + c.fh - 1, pw = c.ow + c.fw - 1;
+    return std::max(c.oh * c.ow * dgrad_pitch(k), (c.pad_h || c.pad_w) ? ph * pw * c.c : 0);
 }
 
 string gen_conv_dgrad(Emitter& em, Generated* out) {
@@ -938,7 +938,7 @@ string gen_conv_dgrad(Emitter& em, Generated* out) {
     const MatMulDims g = matmul_dims(d);
     const int64_t K = g.k, G = cv.g, C = cv.c, FH = cv.fh, FW = cv.fw, OH = cv.oh, OW = cv.ow;
     if (g.batch != G || g.m != cv.img * OH * OW || g.n != FH * FW * C || g.chunks != 1) return "conv dgrad: geometry mismatch";
-    const int64_t TH = OH + 2 * (FH - 1), TW = OW + 2 * (FW - 1), PH = OH + FH - 1, PW = OW + FW - 1;
+    const int64_t PH = OH + FH - 1, PW = OW + FW - 1;
     const int64_t GC = G * C, PITCH = dgrad_pitch(K);
     const int64_t H = PH - 2 * cv.pad_h, W = PW - 2 * cv.pad_w;
     const bool unpad = cv.pad_h > 0 || cv.pad_w > 0;
@@ -957,23 +957,19 @@ string gen_conv_dgrad(Emitter& em, Generated* out) {
     k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
     k << "    __shared__ __attribute__((aligned(16))) float lds[" << S(lds) << "];\n";
     k << "    const int cb = blockIdx.x % " << S(G) << ", img = blockIdx.x / " << S(G) << ";\n";
-    // 1. dC of this image and group inside a halo of fh-1 / fw-1 zeros: tile[ty][tx][oc].  Groups of 8 loads are
-    // issued before any of them is stored: one memory round trip per group, not per element.
-    const int64_t fill_n = TH * TW * K;
+    // 1. dC of this image and group: tile[oy][ox][oc].  (No halo: the taps that fall outside the output are
+    // predicated below, which keeps the tile small enough for every workgroup of a ConvNet-sized launch to be
+    // resident at once.)  Groups of 8 loads are issued before any of them is stored: one memory round trip per
+    // group, not per element.
+    const int64_t fill_n = OH * OW * K;
     k << "    for (int i0 = threadIdx.x; i0 < " << S(fill_n) << "; i0 += 2048) {\n        float v[8];\n";
     k << "#pragma unroll\n        for (int u = 0; u < 8; ++u) {\n";
     k << "            const int i = min(i0 + u * 256, " << S(fill_n - 1) << ");\n";
-    k << "            const int oc = i % " << S(K) << ", tx = (i / " << S(K) << ") % " << S(TW) << ", ty = i / " << S(K * TW) << ";\n";
-    k << "            const int oy = ty - " << S(FH - 1) << ", ox = tx - " << S(FW - 1) << ";\n";
-    k << "            v[u] = load_a(cb, (img * " << S(OH) << " + clampi(oy, 0, " << S(OH - 1) << ")) * " << S(OW) << " + clampi(ox, 0, "
-      << S(OW - 1) << "), oc, " << em.params_pass() << ");\n        }\n";
+    k << "            v[u] = load_a(cb, img * " << S(OH * OW) << " + i / " << S(K) << ", i % " << S(K) << ", " << em.params_pass() << ");\n        }\n";
     k << "        __builtin_amdgcn_sched_barrier(0);\n";
     k << "#pragma unroll\n        for (int u = 0; u < 8; ++u) {\n";
     k << "            const int i = i0 + u * 256;\n";
-    k << "            const int oc = i % " << S(K) << ", tx = (i / " << S(K) << ") % " << S(TW) << ", ty = i / " << S(K * TW) << ";\n";
-    k << "            const int oy = ty - " << S(FH - 1) << ", ox = tx - " << S(FW - 1) << ";\n";
-    k << "            const bool inside = oy >= 0 && oy < " << S(OH) << " && ox >= 0 && ox < " << S(OW) << ";\n";
-    k << "            if (i < " << S(fill_n) << ") lds[(ty * " << S(TW) << " + tx) * " << S(PITCH) << " + oc] = inside ? v[u] : 0.f;\n        }\n    }\n";
+    k << "            if (i < " << S(fill_n) << ") lds[(i / " << S(K) << ") * " << S(PITCH) << " + i % " << S(K) << "] = v[u];\n        }\n    }\n";
     k << "    __syncthreads();\n";
     // 2. one padded-image pixel per thread and pass: acc[c] over taps and output channels; the filter element is
     // the same for every lane, so it comes through the scalar unit.  The tap loop stays a loop and each block of
@@ -988,13 +984,15 @@ string gen_conv_dgrad(Emitter& em, Generated* out) {
     k << "#pragma unroll\n        for (int c = 0; c < " << S(C) << "; ++c) acc[ps][c] = 0.f;\n";
     k << "#pragma unroll 1\n        for (int tap = 0; tap < " << S(FH * FW) << "; ++tap) {\n";
     k << "            const int fy = tap / " << S(FW) << ", fx = tap % " << S(FW) << ";\n";
-    k << "            const float* src = &lds[((py + " << S(FH - 1) << " - fy) * " << S(TW) << " + (px + " << S(FW - 1) << " - fx)) * "
+    k << "            const int oy = py - fy, ox = px - fx;\n";
+    k << "            const bool inside = oy >= 0 && oy < " << S(OH) << " && ox >= 0 && ox < " << S(OW) << ";\n";
+    k << "            const float* src = &lds[(clampi(oy, 0, " << S(OH - 1) << ") * " << S(OW) << " + clampi(ox, 0, " << S(OW - 1) << ")) * "
       << S(PITCH) << "];\n";
     k << "#pragma unroll\n            for (int oc = 0; oc < " << S(K) << "; oc += " << OCB << ") {\n";
     k << "                float a[" << OCB << "];\n";
     k << "#pragma unroll\n                for (int q = 0; q < " << OCB << "; q += 4) {\n";
     k << "                    const float4 a4 = *(const float4*)(src + oc + q);\n";
-    k << "                    a[q] = a4.x; a[q + 1] = a4.y; a[q + 2] = a4.z; a[q + 3] = a4.w;\n                }\n";
+    k << "                    a[q] = inside ? a4.x : 0.f; a[q + 1] = inside ? a4.y : 0.f; a[q + 2] = inside ? a4.z : 0.f; a[q + 3] = inside ? a4.w : 0.f;\n                }\n";
     k << "#pragma unroll\n                for (int j = 0; j < " << OCB << "; ++j)\n";
     k << "#pragma unroll\n                    for (int c = 0; c < " << S(C) << "; ++c)\n";
     k << "                        acc[ps][c] = fmaf(a[j], load_b(cb, oc + j, tap * " << S(C) << " + c, " << em.params_pass() << "), acc[ps][c]);\n";
