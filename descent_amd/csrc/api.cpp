@@ -408,7 +408,7 @@ int dsc_schedule_run(dsc_ctx* ctx, dsc_schedule* s, dsc_buf* params, uint32_t ra
 
 int dsc_schedule_launch_count(const dsc_schedule* s, int32_t* out_launches, int32_t* out_clusters) {
     if (!s) return fail(DSC_ERR_INVALID, "null schedule");
-    if (out_launches) *out_launches = (int32_t)s->s.steps.size();
+    if (out_launches) *out_launches = (int32_t)s->s.launches_per_run();
     if (out_clusters) *out_clusters = s->s.n_clusters;
     return DSC_OK;
 }

@@ -1160,6 +1160,36 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
         }
         steps.push_back(st);
     }
+    if (!(flags & DSC_SCHEDULE_NO_FUSION)) {
+        std::vector<std::pair<int, uint32_t>> fills;  // (node, literal bits)
+        for (auto& st : steps)
+            for (auto& o : st.outputs)
+                if (o.copy_from >= 0 && o.from_literal) fills.emplace_back(o.node, o.literal_bits);
+        for (size_t first = 0; fills.size() >= 2 && first < fills.size(); first += 32) {
+            const size_t last = std::min(fills.size(), first + 32);
+            if (last - first < 2) break;
+            FusedKernel multi;
+            Prefill pf;
+            for (size_t i = first; i < last; ++i) {
+                dsc_kernel_desc fd{};
+                fd.kind = DSC_KERNEL_FILL;
+                fd.shape.rank = 1;
+                fd.shape.dims[0] = (int64_t)(node_bytes[fills[i].first] / 4);
+                fd.fill_bits = fills[i].second;
+                multi.parts.push_back(FusedKernel::plain(fd));
+                multi.part_params.push_back({(int)(i - first)});
+                multi.outputs.push_back((int)(i - first));
+                multi.buffer_is_output.push_back(true);
+                pf.nodes.push_back(fills[i].first);
+            }
+            multi.main = multi.parts[0].main;
+            multi.n_buffers = (int)pf.nodes.size();
+            int status = DSC_OK;
+            pf.kernel = get_kernel(ctx, multi, &status);
+            if (!pf.kernel) return status;
+            prefills.push_back(pf);
+        }
+    }
     return DSC_OK;
 }
 
@@ -1204,6 +1234,18 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
     std::vector<Launch> launches;
     std::vector<void*> pointers;
     launches.reserve(steps.size() + 4);
+    std::vector<dsc_buf> prefilled(prefills.empty() ? 0 : n_nodes, 0);
+    for (auto& pf : prefills) {
+        launches.push_back(Launch{pf.kernel, pointers.size(), (int)pf.nodes.size()});
+        for (int node : pf.nodes) {
+            const dsc_buf h = ctx->heap.alloc(node_bytes[node]);
+            if (!h) return fail(DSC_ERR_OOM, "schedule run: out of device memory");
+            void* p = nullptr;
+            ctx->heap.info(h, &p, nullptr);
+            pointers.push_back(p);
+            prefilled[node] = h;
+        }
+    }
     for (auto& st : steps) {
         for (int n : st.inputs) usage[n] -= 1;
         for (auto& o : st.outputs) {
@@ -1216,6 +1258,9 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
                 if (buffer[o.copy_from] != 0) {
                     h = buffer[o.copy_from];
                     buffer[o.copy_from] = 0;
+                } else if (o.from_literal && !prefilled.empty() && prefilled[o.node] != 0) {
+                    h = prefilled[o.node];  // allocated and filled at the start of the run
+                    prefilled[o.node] = 0;
                 } else if (o.from_literal) {
                     h = ctx->heap.alloc(node_bytes[o.node]);
                     if (!h) return fail(DSC_ERR_OOM, "schedule run: out of device memory");
@@ -1314,11 +1359,23 @@ Schedule::~Schedule() {
         if (c.exec) (void)hipGraphExecDestroy(c.exec);
 }
 
+int Schedule::launches_per_run() const {
+    int n = (int)steps.size() + (int)prefills.size();
+    if (prefills.empty())
+        for (auto& st : steps)
+            for (auto& o : st.outputs)
+                if (o.copy_from >= 0 && o.from_literal) ++n;
+    return n;
+}
+
 std::string Schedule::describe() const {
     std::ostringstream o;
-    o << steps.size() << " launches for " << n_clusters << " clusters\n";
+    o << launches_per_run() << " launches for " << n_clusters << " clusters\n";
     if (replays + direct_runs + (int64_t)captured.size() > 0)
         o << "# graph replays " << replays << ", captured " << captured.size() << ", direct runs " << direct_runs << "\n";
+    for (auto& pf : prefills)
+        o << "prefill: " << pf.kernel->label << "  grid " << pf.kernel->gen.grid << "x" << pf.kernel->gen.block << " (" << pf.nodes.size()
+          << " literal-initialised accumulators)\n";
     double bytes = 0, flops = 0;
     for (size_t i = 0; i < steps.size(); ++i) {
         const Step& st = steps[i];

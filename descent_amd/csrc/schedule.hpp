@@ -40,10 +40,20 @@ struct Schedule {
     std::vector<size_t> node_bytes;
     std::vector<dsc_param_io> inputs, outputs;
     std::vector<Step> steps;
+    // Accumulators that start as a literal (a ScatterAdd into zeros): with several of them in one graph, all are
+    // allocated and filled by one multi-part launch at the start of a run instead of one Fill launch each.
+    struct Prefill {
+        Kernel* kernel = nullptr;
+        std::vector<int> nodes;  // one per pointer parameter
+    };
+    std::vector<Prefill> prefills;
 
     int build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags);
     int run(Context* ctx, dsc_buf* params, uint32_t rand_seed);
     std::string describe() const;
+    // kernels one run enqueues: the steps, the prefill launches, and a Fill per literal-initialised accumulator
+    // that no prefill covers
+    int launches_per_run() const;
 };
 
 }  // namespace dsc

@@ -325,8 +325,9 @@ def test_scatter_add_chains_vs_float64(hip_backend_session, n, entries, links):
     g, got, want = _scatter_chain_case(genv, n, entries, links, 40 + entries)
     _, oracle, _ = _scatter_chain_case(cenv, n, entries, links, 40 + entries)
     listing = next(iter(g.__dict__["_schedules"].values())).describe()
-    # the index conversions share one launch, the whole chain of scatter-adds another
-    assert int(listing.split()[0]) == 2 and "Multi (%d kernels: ScatterAdd" % links in listing, listing
+    # the index conversions share one launch, the whole chain of scatter-adds another; the third is the Fill that
+    # zeroes the accumulator
+    assert int(listing.split()[0]) == 3 and "Multi (%d kernels: ScatterAdd" % links in listing, listing
     if entries * 2 <= 8192 and n * 2 >= 32 * entries:
         assert "per-workgroup sums in LDS" in listing, listing
     assert rel_l2(got, want) <= TOL
