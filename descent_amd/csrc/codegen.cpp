@@ -794,30 +794,34 @@ bool scatter_privatised(const dsc_kernel_desc& d, int64_t* workgroups) {
     return true;
 }
 
-string gen_scatter_add(Emitter& em, Generated* out) {
+// value, index and target of ScatterAdd element `gid` (names suffixed by `sfx`): value<sfx>, at<sfx>, ok<sfx>
+void emit_scatter_element(Emitter& em, std::ostream& k, const string& gid, const string& sfx) {
     const FusedKernel& fk = em.fk;
     const dsc_kernel_desc& d = fk.main.raw();
     const dsc_view& vv = d.inputs[0];
     const dsc_view& vi = d.inputs[1];
-    const int64_t n = element_count(vv.out_shape);
+    int64_t st[DSC_MAX_DIM];
+    strides_of(d.shape, st);
+    auto c = em.emit_coords(k, vv.out_shape, gid, "c" + sfx + "_");
+    k << "    const float value" << sfx << " = " << em.load_view(fk.inputs[0], vv, c) << ";\n";
+    k << "    const int si" << sfx << " = F2I(" << em.load_view(fk.inputs[1], vi, {c[d.axis]}) << ");\n";
+    string idx = "0";
+    for (int i = 0; i < d.shape.rank; ++i) idx += " + " + (i == d.axis ? "si" + sfx : c[i]) + "*" + S(st[i]);
+    k << "    const int at" << sfx << " = " << idx << ";\n";
+    // bounds: an index outside the accumulator would be a wild write; the reference has no check, here it is dropped
+    k << "    const bool ok" << sfx << " = si" << sfx << " >= 0 && si" << sfx << " < " << S(d.shape.dims[d.axis]) << ";\n";
+}
+
+string gen_scatter_add(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const int64_t n = element_count(d.inputs[0].out_shape);
     int64_t wgs = 0;
     const bool priv = scatter_privatised(d, &wgs);
     const int64_t table = element_count(d.shape);
-    int64_t st[DSC_MAX_DIM];
-    strides_of(d.shape, st);
     std::ostringstream k;
     k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
-    // value, index and target of element `gid` (names suffixed by `sfx`)
-    auto emit_element = [&](const string& gid, const string& sfx) {
-        auto c = em.emit_coords(k, vv.out_shape, gid, "c" + sfx + "_");
-        k << "    const float value" << sfx << " = " << em.load_view(fk.inputs[0], vv, c) << ";\n";
-        k << "    const int si" << sfx << " = F2I(" << em.load_view(fk.inputs[1], vi, {c[d.axis]}) << ");\n";
-        string idx = "0";
-        for (int i = 0; i < d.shape.rank; ++i) idx += " + " + (i == d.axis ? "si" + sfx : c[i]) + "*" + S(st[i]);
-        k << "    const int at" << sfx << " = " << idx << ";\n";
-        // bounds: an index outside the accumulator would be a wild write; the reference has no check, here it is dropped
-        k << "    const bool ok" << sfx << " = si" << sfx << " >= 0 && si" << sfx << " < " << S(d.shape.dims[d.axis]) << ";\n";
-    };
+    auto emit_element = [&](const string& gid, const string& sfx) { emit_scatter_element(em, k, gid, sfx); };
     if (priv) {
         const int U = 4;  // elements per thread and trip: their loads are all issued before the first LDS atomic
         k << "    __shared__ float acc[" << S(table) << "];\n";
@@ -1648,6 +1652,7 @@ std::string FusedKernel::key() const {
         for (int64_t v : {dgrad.img, dgrad.oh, dgrad.ow, dgrad.g, dgrad.fh, dgrad.fw, dgrad.c, dgrad.pad_h, dgrad.pad_w, (int64_t)dgrad.rows_first})
             s.append(reinterpret_cast<const char*>(&v), 8);
     }
+    if (shared_scatter) s += "|SS";
     for (size_t i = 0; i < parts.size(); ++i) {
         s += "|P{" + parts[i].key() + "}";
         for (int j : part_params[i]) s.append(reinterpret_cast<const char*>(&j), 4);
@@ -1666,6 +1671,7 @@ std::string FusedKernel::key() const {
 
 namespace {
 string generate_multi(const FusedKernel& fk, Generated* out);
+string generate_scatter_chain(const FusedKernel& fk, Generated* out);
 }
 
 bool conv_dgrad_fits(const FusedKernel::ConvDgrad& c, int64_t k) {
@@ -1686,6 +1692,7 @@ bool can_be_part(const FusedKernel& fk) {
 static std::string generate_one(const FusedKernel& fk, Generated* out, bool with_prelude);
 
 std::string generate(const FusedKernel& fk, Generated* out) {
+    if (!fk.parts.empty() && fk.shared_scatter) return generate_scatter_chain(fk, out);
     if (!fk.parts.empty()) return generate_multi(fk, out);
     return generate_one(fk, out, true);
 }
@@ -1744,6 +1751,75 @@ static std::string generate_one(const FusedKernel& fk, Generated* out, bool with
     count_work(fk, &g);
     *out = g;
     return "";
+}
+
+namespace {
+// ScatterAdds chained through one accumulator that fits LDS (see FusedKernel::shared_scatter).  1024 threads per
+// workgroup, one accumulator copy per workgroup: with tables of tens of kilobytes only one workgroup fits a CU, so
+// the waves that hide the value / index loads have to come from inside it.
+string generate_scatter_chain(const FusedKernel& fk, Generated* out) {
+    const dsc_kernel_desc& first = fk.parts[0].main.raw();
+    const int64_t table = element_count(first.shape);
+    int64_t total = 0;
+    for (auto& part : fk.parts) {
+        const dsc_kernel_desc& d = part.main.raw();
+        if (d.kind != DSC_KERNEL_SCATTER_ADD || !same_shape(d.shape, first.shape)) return "scatter chain: parts differ";
+        total += element_count(d.inputs[0].out_shape);
+    }
+    if (table * 4 > 144 * 1024) return "scatter chain: accumulator does not fit LDS";
+    const int64_t wgs = std::max<int64_t>(64, std::min<int64_t>(256, total / 16384));
+    const int U = 4;
+    Generated g;
+    std::ostringstream src, body;
+    src << kPreludeSource << "\n";
+    int out_param = -1;
+    for (size_t i = 0; i < fk.parts.size(); ++i) {
+        const FusedKernel& part = fk.parts[i];
+        if ((int)fk.part_params[i].size() != part.n_buffers) return "scatter chain: part parameter count";
+        Emitter em(part);
+        const int64_t n = element_count(part.main.raw().inputs[0].out_shape);
+        std::ostringstream fn;
+        fn << "DSC_INLINE void accumulate(float* acc, const uint first, " << em.params_decl() << ") {\n";
+        fn << "    for (uint g0 = first; g0 < " << S(n) << "u; g0 += " << S(wgs * 1024 * U) << "u) {\n";
+        for (int u = 0; u < U; ++u) {
+            fn << "    const uint gid" << u << " = min(g0 + " << S(u * wgs * 1024) << "u, " << S(n - 1) << "u);\n";
+            emit_scatter_element(em, fn, "gid" + to_string(u), to_string(u));
+        }
+        fn << "    __builtin_amdgcn_sched_barrier(0);\n";
+        for (int u = 0; u < U; ++u)
+            fn << "    if (ok" << u << " && g0 + " << S(u * wgs * 1024) << "u < " << S(n) << "u) atomicAdd(&acc[at" << u << "], value" << u << ");\n";
+        fn << "    }\n}\n";
+        src << "namespace part" << i << " {\n" << em.funcs.str() << fn.str() << "}  // namespace part" << i << "\n\n";
+        body << "    part" << i << "::accumulate(acc, blockIdx.x * 1024u + threadIdx.x";
+        for (int j : fk.part_params[i]) body << ", b" << j;
+        body << ", rand_seed);\n";
+        out_param = fk.part_params[i][part.outputs[0]];
+        Generated pg;  // for the work figures only
+        if (generate_one(part, &pg, false).empty()) g.algo_bytes += pg.algo_bytes;
+    }
+    Emitter em(fk);
+    g.entry = "dsc_scatter_chain_l" + to_string(fk.parts.size()) + "_t" + S(table) + "_n" + S(total);
+    src << "extern \"C\" __global__ __launch_bounds__(1024) void " << g.entry << "(" << em.kernel_params_decl() << ") {\n";
+    src << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
+    src << "    __shared__ float acc[" << S(table) << "];\n";
+    src << "    for (int i = threadIdx.x; i < " << S(table) << "; i += 1024) acc[i] = 0.f;\n    __syncthreads();\n";
+    src << body.str();
+    src << "    __syncthreads();\n";
+    src << "    for (int i = threadIdx.x; i < " << S(table) << "; i += 1024) {\n        const float sum = acc[i];\n";
+    src << "        if (sum != 0.f) unsafeAtomicAdd(&b" << out_param << "[i], sum);\n    }\n}\n";
+    g.source = src.str();
+    g.grid = (unsigned)wgs;
+    g.block = 1024;
+    g.n_buffers = fk.n_buffers;
+    g.note = "scatter chain: " + to_string(fk.parts.size()) + " links into one accumulator of " + S(table) +
+             " floats kept in LDS per workgroup (ds_add_f32), then global_atomic_add_f32";
+    *out = g;
+    return "";
+}
+}  // namespace
+
+bool scatter_chain_in_lds(int64_t table_elements, int64_t total_values) {
+    return table_elements * 4 <= 144 * 1024 && total_values >= 16 * table_elements && total_values >= 65536;
 }
 
 namespace {

@@ -60,6 +60,10 @@ struct FusedKernel {
     // `main` is parts[0].main (for the label); inputs/outputs of the launch are those of the parts.
     std::vector<FusedKernel> parts;
     std::vector<std::vector<int>> part_params;
+    // Multi-part launch whose parts are ScatterAdds into one accumulator small enough for LDS: every workgroup keeps
+    // ONE copy of the accumulator in LDS, folds its share of every part's values into it and adds the non-zero
+    // totals to memory once.
+    bool shared_scatter = false;
     // Data gradient of a stride-1 convolution with few channels, as one kernel: `main` is the MatMul dC x filter^T
     // ([g][(img, oy, ox)][oc] x [g][oc][(fy, fx, c)]); the kernel also does what the reference's WindowsToImage
     // (sum of the windows covering each pixel of the padded image) and the two Unpads after it (fold the
@@ -104,6 +108,10 @@ std::string generate(const FusedKernel& k, Generated* out);
 // Whether the convolution data-gradient kernel can take this geometry (k = output channels per group): the image
 // tile must fit the workgroup's LDS.
 bool conv_dgrad_fits(const FusedKernel::ConvDgrad& c, int64_t k);
+
+// Whether a chain of ScatterAdds with this accumulator size and this many values in total runs as one kernel with
+// the accumulator in LDS (shared_scatter).
+bool scatter_chain_in_lds(int64_t table_elements, int64_t total_values);
 
 // Whether a kernel can be one part of a multi-part launch (256 threads per workgroup, addressed by blockIdx.x only).
 bool can_be_part(const FusedKernel& k);

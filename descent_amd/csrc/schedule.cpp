@@ -1021,10 +1021,7 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                 for (int c : consumers_of(node)) (void)c, ++readers;  // nobody may read the intermediate sum
                 if (readers != 0) break;
                 chain.push_back(next);
-                // every link may keep a copy of the accumulator in LDS (small tables): stay well inside the 160 KiB
-                const int64_t table = element_count(drafts[i].fk.main.raw().shape);
-                const int64_t max_links = table <= 8192 ? std::max<int64_t>(2, std::min<int64_t>(8, 32768 / table)) : 8;
-                if ((int64_t)chain.size() >= max_links) break;
+                if (chain.size() >= 8) break;
             }
             if (chain.size() < 2) continue;
             const int last = chain.back();
@@ -1051,6 +1048,11 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                 for (int nd : input_nodes(d))
                     if (seen.insert(nd).second) multi.part_inputs.push_back(nd);
                 multi.covers.insert(multi.covers.end(), d.covers.begin(), d.covers.end());
+            }
+            {
+                int64_t total_values = 0;
+                for (int j : chain) total_values += element_count(drafts[j].fk.main.raw().inputs[0].out_shape);
+                multi.fk.shared_scatter = scatter_chain_in_lds(element_count(drafts[i].fk.main.raw().shape), total_values);
             }
             StepOutput out = drafts[i].outs[0];  // the first link says where the accumulator comes from
             out.node = final_node;

@@ -316,10 +316,10 @@ def _scatter_chain_case(env, n, entries, links, seed):
     return g, env.read_parameter(out), want
 
 
-@pytest.mark.parametrize("n,entries,links", [(131072, 289, 4), (65536, 3481, 2), (131072, 100000, 4), (70000, 3, 3)])
+@pytest.mark.parametrize("n,entries,links", [(131072, 289, 4), (65536, 3481, 2), (131072, 100000, 4), (70000, 3, 3), (262144, 12544, 4), (100001, 17000, 5)])
 def test_scatter_add_chains_vs_float64(hip_backend_session, n, entries, links):
     """Float atomics reorder the sums, so the bound is the looser one stated for scatter-add: 1e-4 relative L2
-    against a float64 accumulation, for the GPU (small accumulators go through per-workgroup LDS sums first) and
+    against a float64 accumulation, for the GPU (accumulators that fit LDS go through per-workgroup sums first) and
     for the oracle's serial fp32 sums alike."""
     genv, cenv = _envs(hip_backend_session)
     g, got, want = _scatter_chain_case(genv, n, entries, links, 40 + entries)
@@ -328,8 +328,11 @@ def test_scatter_add_chains_vs_float64(hip_backend_session, n, entries, links):
     # the index conversions share one launch, the whole chain of scatter-adds another; the third is the Fill that
     # zeroes the accumulator
     assert int(listing.split()[0]) == 3 and "Multi (%d kernels: ScatterAdd" % links in listing, listing
-    if entries * 2 <= 8192 and n * 2 >= 32 * entries:
-        assert "per-workgroup sums in LDS" in listing, listing
+    # accumulators of up to 144 KiB with at least 16 values per entry: one LDS copy per workgroup takes every link
+    if entries * 2 * 4 <= 144 * 1024 and links * n * 2 >= 16 * entries * 2:
+        assert "accumulator of %d floats kept in LDS" % (entries * 2) in listing, listing
+    else:
+        assert "kept in LDS" not in listing, listing
     assert rel_l2(got, want) <= TOL
     assert rel_l2(oracle, want) <= TOL
 
