@@ -132,6 +132,46 @@ def bench_convnet(env, steps, warmup, batch=1000):
     }
 
 
+def bench_convnet_minibatch_uploads(env, steps=300, batch=1000):
+    """ConvNet train steps with a new mini-batch (x: batch x 28 x 28 floats, y: batch labels) uploaded before every
+    step, as a training loop does: through the compute stream (the reference's writer contract), and through the
+    copy stream from alternating pinned arrays, where the upload of step n+1 runs beside step n."""
+    from descent_amd import workloads
+
+    be = env.backend
+    w = workloads.convnet(env, batch=batch, seed=3)
+    x, y = w.inputs["x"], w.inputs["y"]
+    px = [env.host_array(x) for _ in range(2)]
+    py = [env.host_array(y) for _ in range(2)]
+    rng = np.random.default_rng(0)
+    for a in px:
+        a[...] = rng.random(a.shape, dtype=np.float32)
+    for a in py:
+        a[...] = rng.integers(0, 10, a.shape).astype(np.float32)
+
+    def loop(n, mode):
+        for i in range(n):
+            s = i & 1
+            if mode == "serial":
+                env.write_parameter(x, px[s])
+                env.write_parameter(y, py[s])
+            elif mode == "overlapped":
+                env.write_parameter_async(x, px[s])
+                env.write_parameter_async(y, py[s])
+            env.run(w.graph, i)
+        be.sync()
+
+    out = {"upload_bytes_per_step": int(px[0].nbytes + py[0].nbytes)}
+    for mode in ("resident", "serial", "overlapped"):
+        loop(20, mode)
+        t0 = time.perf_counter()
+        loop(steps, mode)
+        out[mode + "_steps_per_s"] = steps / (time.perf_counter() - t0)
+    for a in px + py:
+        be.host_release(a)
+    return out
+
+
 def bench_elementwise(env, n, steps, warmup):
     """c = a * 2 + b over n elements: 2 reads + 1 write of 4n bytes each (a plain streaming kernel of known
     size, also used to calibrate the FETCH_SIZE / WRITE_SIZE counters)."""
@@ -323,6 +363,7 @@ def main():
             extra["matmul"].append(r)
         extra["elementwise_axpb_64M"] = bench_elementwise(env, 1 << 26, max(args.steps, 20), args.warmup)
         extra["host_operands"] = bench_upload(env, n)
+        extra["convnet_bs1000_minibatch_uploads"] = bench_convnet_minibatch_uploads(env)
         extra["reduce"] = [bench_reduce(env, 8192, 8192, 1, 20, 3), bench_reduce(env, 8192, 8192, 0, 20, 3),
                            bench_reduce(env, 262144, 256, 0, 20, 3)]
         from descent_amd import workloads as _w

@@ -128,50 +128,57 @@ int dsc_ctx_caps(dsc_ctx* ctx, dsc_caps* out) {
 
 int dsc_ctx_sync(dsc_ctx* ctx) {
     if (!ctx) return fail(DSC_ERR_INVALID, "null context");
+    if (ctx->c.copy_stream) HIP_TRY(hipStreamSynchronize(ctx->c.copy_stream));
     HIP_TRY(hipStreamSynchronize(ctx->c.stream));
     return DSC_OK;
 }
 
-int dsc_fence_record(dsc_ctx* ctx, uint64_t* out_fence) {
-    if (!ctx || !out_fence) return fail(DSC_ERR_INVALID, "null argument");
-    Context* c = &ctx->c;
-    hipEvent_t ev = nullptr;
-    if (!c->fence_pool.empty()) {
-        ev = c->fence_pool.back();
-        c->fence_pool.pop_back();
-    } else {
-        HIP_TRY(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+namespace {
+// Records a new fence on `stream` and returns its id (0 on failure, with the error set).
+uint64_t record_fence(Context* c, hipStream_t stream, bool on_copy_stream) {
+    hipEvent_t ev = take_plain_event(c);
+    if (!ev) {
+        fail(DSC_ERR_HIP, "hipEventCreate failed");
+        return 0;
     }
-    hipError_t e = hipEventRecord(ev, c->stream);
+    const hipError_t e = hipEventRecord(ev, stream);
     if (e != hipSuccess) {
         c->fence_pool.push_back(ev);
-        return fail(DSC_ERR_HIP, std::string("hipEventRecord: ") + hipGetErrorString(e));
+        fail(DSC_ERR_HIP, std::string("hipEventRecord: ") + hipGetErrorString(e));
+        return 0;
     }
-    *out_fence = c->fence_next++;
-    c->fences[*out_fence] = ev;
-    return DSC_OK;
+    const uint64_t id = c->fence_next++;
+    c->fences[id] = Context::Fence{ev, on_copy_stream};
+    return id;
 }
 
-namespace {
-// everything recorded at or before `fence` has finished: recycle those events
-void retire_fences(Context* c, uint64_t fence) {
-    while (!c->fences.empty() && c->fences.begin()->first <= fence) {
-        c->fence_pool.push_back(c->fences.begin()->second);
-        c->fences.erase(c->fences.begin());
+// `fence` has finished; each stream is in order, so the older fences of its stream have finished too
+void retire_fences(Context* c, uint64_t fence, bool on_copy_stream) {
+    for (auto it = c->fences.begin(); it != c->fences.end() && it->first <= fence;) {
+        if (it->second.on_copy_stream == on_copy_stream) {
+            c->fence_pool.push_back(it->second.event);
+            it = c->fences.erase(it);
+        } else {
+            ++it;
+        }
     }
-    if (fence > c->fence_retired) c->fence_retired = fence;
 }
 }  // namespace
+
+int dsc_fence_record(dsc_ctx* ctx, uint64_t* out_fence) {
+    if (!ctx || !out_fence) return fail(DSC_ERR_INVALID, "null argument");
+    *out_fence = record_fence(&ctx->c, ctx->c.stream, false);
+    return *out_fence ? DSC_OK : DSC_ERR_HIP;
+}
 
 int dsc_fence_wait(dsc_ctx* ctx, uint64_t fence) {
     if (!ctx) return fail(DSC_ERR_INVALID, "null context");
     Context* c = &ctx->c;
     if (fence == 0 || fence >= c->fence_next) return fail(DSC_ERR_INVALID, "unknown fence id");
-    if (fence <= c->fence_retired) return DSC_OK;
     auto it = c->fences.find(fence);
-    if (it == c->fences.end()) return fail(DSC_ERR_INVALID, "unknown fence id");
-    HIP_TRY(hipEventSynchronize(it->second));
-    retire_fences(c, fence);  // the stream is in order: older fences have finished too
+    if (it == c->fences.end()) return DSC_OK;  // retired
+    HIP_TRY(hipEventSynchronize(it->second.event));
+    retire_fences(c, fence, it->second.on_copy_stream);
     return DSC_OK;
 }
 
@@ -179,16 +186,15 @@ int dsc_fence_query(dsc_ctx* ctx, uint64_t fence, int* out_finished) {
     if (!ctx || !out_finished) return fail(DSC_ERR_INVALID, "null argument");
     Context* c = &ctx->c;
     if (fence == 0 || fence >= c->fence_next) return fail(DSC_ERR_INVALID, "unknown fence id");
-    if (fence <= c->fence_retired) {
+    auto it = c->fences.find(fence);
+    if (it == c->fences.end()) {
         *out_finished = 1;
         return DSC_OK;
     }
-    auto it = c->fences.find(fence);
-    if (it == c->fences.end()) return fail(DSC_ERR_INVALID, "unknown fence id");
-    const hipError_t e = hipEventQuery(it->second);
+    const hipError_t e = hipEventQuery(it->second.event);
     if (e == hipSuccess) {
         *out_finished = 1;
-        retire_fences(c, fence);
+        retire_fences(c, fence, it->second.on_copy_stream);
         return DSC_OK;
     }
     if (e != hipErrorNotReady) return fail(DSC_ERR_HIP, std::string("hipEventQuery: ") + hipGetErrorString(e));
@@ -206,6 +212,13 @@ int dsc_ctx_stream(dsc_ctx* ctx, void** out_stream) {
 int dsc_buf_alloc(dsc_ctx* ctx, size_t bytes, dsc_buf* out) {
     if (!ctx || !out) return fail(DSC_ERR_INVALID, "null argument");
     *out = ctx->c.heap.alloc(bytes);
+    if (!*out) return fail(DSC_ERR_OOM, "device memory exhausted allocating " + std::to_string(bytes) + " bytes");
+    return DSC_OK;
+}
+
+int dsc_buf_alloc_io(dsc_ctx* ctx, size_t bytes, dsc_buf* out) {
+    if (!ctx || !out) return fail(DSC_ERR_INVALID, "null argument");
+    *out = ctx->c.heap.alloc(bytes, true);
     if (!*out) return fail(DSC_ERR_OOM, "device memory exhausted allocating " + std::to_string(bytes) + " bytes");
     return DSC_OK;
 }
@@ -233,7 +246,9 @@ int dsc_buf_write(dsc_ctx* ctx, dsc_buf buf, size_t offset, const void* src, siz
     Context* c = &ctx->c;
     char* dst = nullptr;
     int rc = resolve(c, buf, offset, bytes, &dst);
+    if (rc == DSC_OK) rc = join_copies(c);
     if (rc != DSC_OK) return rc;
+    c->heap.touch(buf, ++c->work_seq);
     const char* s = static_cast<const char*>(src);
     while (bytes) {
         const int r = c->staging_next;
@@ -256,7 +271,9 @@ int dsc_buf_fill_zero(dsc_ctx* ctx, dsc_buf buf, size_t offset, size_t bytes) {
     if (!ctx) return fail(DSC_ERR_INVALID, "null context");
     char* dst = nullptr;
     int rc = resolve(&ctx->c, buf, offset, bytes, &dst);
+    if (rc == DSC_OK) rc = join_copies(&ctx->c);
     if (rc != DSC_OK) return rc;
+    ctx->c.heap.touch(buf, ++ctx->c.work_seq);
     if (bytes) HIP_TRY(hipMemsetAsync(dst, 0, bytes, ctx->c.stream));
     return DSC_OK;
 }
@@ -266,7 +283,9 @@ int dsc_buf_read(dsc_ctx* ctx, dsc_buf buf, size_t offset, void* dst, size_t byt
     Context* c = &ctx->c;
     char* src = nullptr;
     int rc = resolve(c, buf, offset, bytes, &src);
+    if (rc == DSC_OK) rc = join_copies(c);
     if (rc != DSC_OK) return rc;
+    c->heap.touch(buf, ++c->work_seq);
     char* d = static_cast<char*>(dst);
     // two regions in flight: the copy into region r+1 overlaps the host memcpy out of region r
     size_t pending_n[Context::kStagingRegions] = {0, 0};
@@ -303,6 +322,108 @@ int dsc_buf_read(dsc_ctx* ctx, dsc_buf buf, size_t offset, void* dst, size_t byt
     return DSC_OK;
 }
 
+int dsc_host_alloc(dsc_ctx* ctx, size_t bytes, void** out_ptr) {
+    if (!ctx || !out_ptr || !bytes) return fail(DSC_ERR_INVALID, "null argument or empty allocation");
+    void* p = nullptr;
+    if (hipHostMalloc(&p, bytes, hipHostMallocDefault) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(DSC_ERR_OOM, "pinned host memory exhausted allocating " + std::to_string(bytes) + " bytes");
+    }
+    ctx->c.pinned[static_cast<const char*>(p)] = bytes;
+    *out_ptr = p;
+    return DSC_OK;
+}
+
+int dsc_host_free(dsc_ctx* ctx, void* ptr) {
+    if (!ctx) return fail(DSC_ERR_INVALID, "null context");
+    Context* c = &ctx->c;
+    auto it = c->pinned.find(static_cast<const char*>(ptr));
+    if (it == c->pinned.end()) return fail(DSC_ERR_INVALID, "not a dsc_host_alloc pointer");
+    // a copy may still be reading or writing it
+    if (c->copy_stream) HIP_TRY(hipStreamSynchronize(c->copy_stream));
+    HIP_TRY(hipHostFree(ptr));
+    c->pinned.erase(it);
+    return DSC_OK;
+}
+
+namespace {
+// whether [p, p + bytes) lies inside one dsc_host_alloc range
+bool is_pinned(const Context* c, const void* p, size_t bytes) {
+    const char* q = static_cast<const char*>(p);
+    auto it = c->pinned.upper_bound(q);
+    if (it == c->pinned.begin()) return false;
+    --it;
+    return q >= it->first && bytes <= it->second && size_t(q - it->first) <= it->second - bytes;
+}
+
+// after a copy-stream operation: the fence the caller (or only the compute stream) will wait for
+int finish_copy(Context* c, uint64_t* out_fence) {
+    if (out_fence) {
+        *out_fence = record_fence(c, c->copy_stream, true);
+        if (!*out_fence) return DSC_ERR_HIP;
+        c->copies.push_back(Context::CopyInFlight{*out_fence, nullptr});
+        return DSC_OK;
+    }
+    hipEvent_t ev = take_plain_event(c);
+    if (!ev) return fail(DSC_ERR_HIP, "hipEventCreate failed");
+    const hipError_t e = hipEventRecord(ev, c->copy_stream);
+    if (e != hipSuccess) {
+        c->fence_pool.push_back(ev);
+        return fail(DSC_ERR_HIP, std::string("hipEventRecord: ") + hipGetErrorString(e));
+    }
+    c->copies.push_back(Context::CopyInFlight{0, ev});
+    return DSC_OK;
+}
+}  // namespace
+
+int dsc_buf_write_async(dsc_ctx* ctx, dsc_buf buf, size_t offset, const void* src, size_t bytes, uint64_t* out_fence) {
+    if (!ctx || (!src && bytes)) return fail(DSC_ERR_INVALID, "null argument");
+    Context* c = &ctx->c;
+    if (out_fence) *out_fence = 0;
+    char* dst = nullptr;
+    int rc = resolve(c, buf, offset, bytes, &dst);
+    if (rc == DSC_OK) rc = enable_async_io(c);
+    // the copy may start once the compute work that last used this memory -- as this buffer, or as whatever the
+    // range held before -- has finished; work enqueued earlier that does not touch it keeps running beside the copy
+    if (rc == DSC_OK) rc = copy_stream_wait(c, c->heap.stamp_of(buf));
+    if (rc != DSC_OK) return rc;
+    if (is_pinned(c, src, bytes)) {
+        if (bytes) HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, c->copy_stream));
+        return finish_copy(c, out_fence);
+    }
+    const char* s = static_cast<const char*>(src);
+    while (bytes) {
+        const int r = c->staging_next;
+        c->staging_next = (r + 1) % Context::kStagingRegions;
+        rc = staging_acquire(c, r);
+        if (rc != DSC_OK) return rc;
+        const size_t n = std::min(bytes, Context::kStagingBytes);
+        std::memcpy(c->staging[r], s, n);
+        HIP_TRY(hipMemcpyAsync(dst, c->staging[r], n, hipMemcpyHostToDevice, c->copy_stream));
+        HIP_TRY(hipEventRecord(c->staging_done[r], c->copy_stream));
+        c->staging_busy[r] = true;
+        s += n;
+        dst += n;
+        bytes -= n;
+    }
+    return finish_copy(c, out_fence);
+}
+
+int dsc_buf_read_async(dsc_ctx* ctx, dsc_buf buf, size_t offset, void* dst, size_t bytes, uint64_t* out_fence) {
+    if (!ctx || !out_fence || (!dst && bytes)) return fail(DSC_ERR_INVALID, "null argument");
+    Context* c = &ctx->c;
+    *out_fence = 0;
+    if (!is_pinned(c, dst, bytes)) return fail(DSC_ERR_INVALID, "dsc_buf_read_async needs a destination from dsc_host_alloc");
+    char* src = nullptr;
+    int rc = resolve(c, buf, offset, bytes, &src);
+    if (rc == DSC_OK) rc = enable_async_io(c);
+    // the value is whatever the compute work enqueued so far leaves in the buffer
+    if (rc == DSC_OK) rc = copy_stream_wait(c, c->heap.stamp_of(buf));
+    if (rc != DSC_OK) return rc;
+    if (bytes) HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, c->copy_stream));
+    return finish_copy(c, out_fence);
+}
+
 int dsc_kernel_get(dsc_ctx* ctx, const dsc_kernel_desc* desc, dsc_kernel** out) {
     if (!ctx || !desc || !out) return fail(DSC_ERR_INVALID, "null argument");
     *out = nullptr;
@@ -336,7 +457,12 @@ int dsc_kernel_launch(dsc_ctx* ctx, dsc_kernel* kernel, const dsc_buf* bufs, int
         else need = (size_t)element_count(d.shape) * 4;
         if (size < need) return fail(DSC_ERR_INVALID, "buffer " + std::to_string(i) + " of '" + k->label + "' is too small");
     }
-    return launch_kernel(&ctx->c, k, ptrs, n, rand_seed);
+    int rc = join_copies(&ctx->c);
+    if (rc != DSC_OK) return rc;
+    rc = launch_kernel(&ctx->c, k, ptrs, n, rand_seed);
+    if (rc == DSC_OK && ctx->c.async_io)
+        for (int i = 0; i < n; ++i) ctx->c.heap.touch(bufs[i], ctx->c.work_seq);
+    return rc;
 }
 
 int dsc_codegen_source(const dsc_kernel_desc* desc, char** out_source) {
@@ -403,7 +529,17 @@ int dsc_schedule_destroy(dsc_ctx* ctx, dsc_schedule* s) {
 
 int dsc_schedule_run(dsc_ctx* ctx, dsc_schedule* s, dsc_buf* params, uint32_t rand_seed) {
     if (!ctx || !s || !params) return fail(DSC_ERR_INVALID, "null argument");
-    return s->s.run(&ctx->c, params, rand_seed);
+    Context* c = &ctx->c;
+    int rc = join_copies(c);
+    if (rc != DSC_OK) return rc;
+    // memory released while the run is put together is still used by the run's launches: stamp it with a count
+    // that only a mark recorded after the run covers
+    ++c->work_seq;
+    rc = s->s.run(c, params, rand_seed);
+    if (rc != DSC_OK || !c->async_io) return rc;
+    for (int i = 0; i < s->s.n_params; ++i)
+        if (params[i]) c->heap.touch(params[i], c->work_seq);
+    return mark_stream(c);
 }
 
 int dsc_schedule_launch_count(const dsc_schedule* s, int32_t* out_launches, int32_t* out_clusters) {

@@ -36,22 +36,72 @@ DeviceHeap::~DeviceHeap() {
         if (c.base) (void)hipFree(c.base);
 }
 
-void DeviceHeap::add_free(int chunk, size_t offset, size_t size) { free_by_size_.emplace(size, std::make_pair(chunk, offset)); }
+void DeviceHeap::add_free(int chunk, size_t offset, size_t size) {
+    free_by_size_[chunks_[chunk].io].emplace(size, std::make_pair(chunk, offset));
+}
 
 void DeviceHeap::remove_free(int chunk, size_t offset, size_t size) {
-    auto range = free_by_size_.equal_range(size);
+    auto& by_size = free_by_size_[chunks_[chunk].io];
+    auto range = by_size.equal_range(size);
     for (auto it = range.first; it != range.second; ++it) {
         if (it->second.first == chunk && it->second.second == offset) {
-            free_by_size_.erase(it);
+            by_size.erase(it);
             return;
         }
     }
 }
 
-uint64_t DeviceHeap::alloc(size_t bytes) {
+uint64_t DeviceHeap::alloc_io(size_t bytes, size_t need) {
+    auto& by_size = free_by_size_[1];
+    auto range = by_size.equal_range(need);
+    auto best = by_size.end();
+    for (auto it = range.first; it != range.second; ++it)
+        if (best == by_size.end() ||
+            chunks_[it->second.first].blocks[it->second.second].stamp < chunks_[best->second.first].blocks[best->second.second].stamp)
+            best = it;
+    int ci = -1;
+    size_t off = 0;
+    uint64_t stamp = 0;
+    if (best != by_size.end()) {
+        ci = best->second.first;
+        off = best->second.second;
+        by_size.erase(best);
+        Block& b = chunks_[ci].blocks[off];
+        b.is_free = false;
+        stamp = b.stamp;
+    } else {
+        for (int i = 0; i < (int)chunks_.size() && ci < 0; ++i)
+            if (chunks_[i].io && chunks_[i].size - chunks_[i].tail >= need) ci = i;
+        if (ci < 0) {
+            Chunk c;
+            c.io = true;
+            c.size = std::max(kIoChunkBytes, need);
+            void* p = nullptr;
+            if (hipMalloc(&p, c.size) != hipSuccess) {
+                (void)hipGetLastError();
+                return 0;
+            }
+            c.base = static_cast<char*>(p);
+            chunks_.push_back(std::move(c));
+            ci = (int)chunks_.size() - 1;
+        }
+        Chunk& c = chunks_[ci];
+        off = c.tail;
+        c.tail += need;
+        c.blocks[off] = Block{need, false, 0};
+    }
+    const uint64_t h = next_handle_++;
+    live_[h] = Live{ci, off, bytes, stamp};
+    live_bytes_ += (int64_t)need;
+    return h;
+}
+
+uint64_t DeviceHeap::alloc(size_t bytes, bool io) {
     const size_t need = std::max(kAlign, (bytes + kAlign - 1) / kAlign * kAlign);
-    auto it = free_by_size_.lower_bound(need);
-    if (it == free_by_size_.end()) {
+    if (io) return alloc_io(bytes, need);
+    auto& by_size = free_by_size_[0];
+    auto it = by_size.lower_bound(need);
+    if (it == by_size.end()) {
         Chunk c;
         c.size = std::max(kChunkBytes, need);
         void* p = nullptr;
@@ -65,23 +115,24 @@ uint64_t DeviceHeap::alloc(size_t bytes) {
             }
         }
         c.base = static_cast<char*>(p);
-        c.blocks[0] = Block{c.size, true};
+        c.blocks[0] = Block{c.size, true, 0};
         chunks_.push_back(std::move(c));
         add_free((int)chunks_.size() - 1, 0, chunks_.back().size);
-        it = free_by_size_.lower_bound(need);
+        it = by_size.lower_bound(need);
     }
     const int ci = it->second.first;
     const size_t off = it->second.second;
     const size_t have = it->first;
-    free_by_size_.erase(it);
+    by_size.erase(it);
     Chunk& c = chunks_[ci];
-    c.blocks[off] = Block{need, false};
+    const uint64_t stamp = c.blocks[off].stamp;
+    c.blocks[off] = Block{need, false, stamp};
     if (have > need) {
-        c.blocks[off + need] = Block{have - need, true};
+        c.blocks[off + need] = Block{have - need, true, stamp};
         add_free(ci, off + need, have - need);
     }
     const uint64_t h = next_handle_++;
-    live_[h] = Live{ci, off, bytes};
+    live_[h] = Live{ci, off, bytes, stamp};
     live_bytes_ += (int64_t)need;
     return h;
 }
@@ -91,16 +142,23 @@ bool DeviceHeap::free(uint64_t handle) {
     if (lit == live_.end()) return false;
     const int ci = lit->second.chunk;
     size_t off = lit->second.offset;
+    uint64_t stamp = std::max(lit->second.stamp, clock ? *clock : 0);
     live_.erase(lit);
     Chunk& c = chunks_[ci];
     auto it = c.blocks.find(off);
     size_t size = it->second.size;
     live_bytes_ -= (int64_t)size;
+    if (c.io) {  // recycled whole, by size
+        it->second = Block{size, true, stamp};
+        add_free(ci, off, size);
+        return true;
+    }
     // coalesce with the next range, then with the previous one
     auto next = std::next(it);
     if (next != c.blocks.end() && next->second.is_free) {
         remove_free(ci, next->first, next->second.size);
         size += next->second.size;
+        stamp = std::max(stamp, next->second.stamp);
         c.blocks.erase(next);
     }
     if (it != c.blocks.begin()) {
@@ -108,12 +166,13 @@ bool DeviceHeap::free(uint64_t handle) {
         if (prev->second.is_free) {
             remove_free(ci, prev->first, prev->second.size);
             size += prev->second.size;
+            stamp = std::max(stamp, prev->second.stamp);
             off = prev->first;
             c.blocks.erase(it);
             it = prev;
         }
     }
-    it->second = Block{size, true};
+    it->second = Block{size, true, stamp};
     add_free(ci, off, size);
     return true;
 }
@@ -124,6 +183,16 @@ bool DeviceHeap::info(uint64_t handle, void** ptr, size_t* bytes) const {
     if (ptr) *ptr = chunks_[it->second.chunk].base + it->second.offset;
     if (bytes) *bytes = it->second.bytes;
     return true;
+}
+
+uint64_t DeviceHeap::stamp_of(uint64_t handle) const {
+    auto it = live_.find(handle);
+    return it == live_.end() ? 0 : it->second.stamp;
+}
+
+void DeviceHeap::touch(uint64_t handle, uint64_t stamp) {
+    auto it = live_.find(handle);
+    if (it != live_.end() && it->second.stamp < stamp) it->second.stamp = stamp;
 }
 
 void DeviceHeap::stats(int64_t* live, int64_t* live_bytes, int64_t* arena_bytes) const {
@@ -140,7 +209,13 @@ void DeviceHeap::stats(int64_t* live, int64_t* live_bytes, int64_t* arena_bytes)
 
 Context::~Context() {
     if (offline) return;
+    if (copy_stream) (void)hipStreamSynchronize(copy_stream);
     if (stream) (void)hipStreamSynchronize(stream);
+    for (auto& m : marks) (void)hipEventDestroy(m.second);
+    for (auto& cp : copies)
+        if (cp.own) (void)hipEventDestroy(cp.own);
+    for (auto& kv : pinned) (void)hipHostFree(const_cast<char*>(kv.first));
+    if (copy_stream) (void)hipStreamDestroy(copy_stream);
     for (auto& kv : kernels)
         if (kv.second->module) (void)hipModuleUnload(kv.second->module);
     for (auto& p : profile) {
@@ -148,7 +223,7 @@ Context::~Context() {
         (void)hipEventDestroy(p.stop);
     }
     for (auto e : event_pool) (void)hipEventDestroy(e);
-    for (auto& kv : fences) (void)hipEventDestroy(kv.second);
+    for (auto& kv : fences) (void)hipEventDestroy(kv.second.event);
     for (auto e : fence_pool) (void)hipEventDestroy(e);
     for (int i = 0; i < kStagingRegions; ++i) {
         if (staging_done[i]) (void)hipEventDestroy(staging_done[i]);
@@ -335,6 +410,105 @@ int set_seed(Context* ctx, uint32_t rand_seed) {
     return DSC_OK;
 }
 
+hipEvent_t take_plain_event(Context* ctx) {
+    hipEvent_t ev = nullptr;
+    if (!ctx->fence_pool.empty()) {
+        ev = ctx->fence_pool.back();
+        ctx->fence_pool.pop_back();
+        return ev;
+    }
+    if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    return ev;
+}
+
+int enable_async_io(Context* ctx) {
+    if (ctx->async_io) return DSC_OK;
+    if (ctx->offline) return fail(DSC_ERR_NO_DEVICE, "overlapped I/O without a device");
+    if (!ctx->copy_stream) HIP_TRY(hipStreamCreate(&ctx->copy_stream));
+    // stamps were not kept up to date until now: start from an idle stream
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    ctx->work_done = ctx->work_seq;
+    ctx->async_io = true;
+    return DSC_OK;
+}
+
+namespace {
+// marks whose event has fired are dropped; the last one dropped says how far the compute stream has come
+void prune_marks(Context* ctx) {
+    while (!ctx->marks.empty()) {
+        const hipError_t e = hipEventQuery(ctx->marks.front().second);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return;
+        }
+        ctx->work_done = std::max(ctx->work_done, ctx->marks.front().first);
+        ctx->fence_pool.push_back(ctx->marks.front().second);
+        ctx->marks.pop_front();
+    }
+}
+}  // namespace
+
+int mark_stream(Context* ctx) {
+    prune_marks(ctx);
+    if (ctx->work_done >= ctx->work_seq) return DSC_OK;
+    if (!ctx->marks.empty() && ctx->marks.back().first >= ctx->work_seq) return DSC_OK;
+    hipEvent_t ev = take_plain_event(ctx);
+    if (!ev) return fail(DSC_ERR_HIP, "hipEventCreate failed");
+    const hipError_t e = hipEventRecord(ev, ctx->stream);
+    if (e != hipSuccess) {
+        ctx->fence_pool.push_back(ev);
+        return fail(DSC_ERR_HIP, std::string("hipEventRecord: ") + hipGetErrorString(e));
+    }
+    ctx->marks.emplace_back(ctx->work_seq, ev);
+    return DSC_OK;
+}
+
+int copy_stream_wait(Context* ctx, uint64_t stamp) {
+    if (stamp <= ctx->work_done) return DSC_OK;
+    prune_marks(ctx);
+    if (stamp <= ctx->work_done) return DSC_OK;
+    if (ctx->marks.empty() || ctx->marks.back().first < stamp) {
+        const int rc = mark_stream(ctx);
+        if (rc != DSC_OK) return rc;
+        if (stamp <= ctx->work_done) return DSC_OK;
+    }
+    // The host waits, not the copy stream: memory that an upload reuses was last read two runs ago when buffers
+    // alternate, so this only holds back a host that is further ahead than that -- and a queue of copies that each
+    // wait in the copy stream for a compute event has measured slower than uploads on the compute stream itself.
+    for (auto& m : ctx->marks) {
+        if (m.first >= stamp) {
+            HIP_TRY(hipEventSynchronize(m.second));
+            prune_marks(ctx);
+            return DSC_OK;
+        }
+    }
+    return fail(DSC_ERR_INVALID, "no mark covers a buffer's last use");
+}
+
+int join_copies(Context* ctx) {
+    if (ctx->copies.empty()) return DSC_OK;
+    for (auto& cp : ctx->copies) {
+        hipEvent_t ev = cp.own;
+        if (!ev) {
+            auto it = ctx->fences.find(cp.fence);
+            if (it == ctx->fences.end()) continue;  // waited for and retired: the copy has finished
+            ev = it->second.event;
+        }
+        // a copy that has already finished needs no barrier in the compute queue
+        if (hipEventQuery(ev) != hipSuccess) {
+            (void)hipGetLastError();
+            HIP_TRY(hipStreamWaitEvent(ctx->stream, ev, 0));
+        }
+        if (cp.own) ctx->fence_pool.push_back(cp.own);
+        cp.own = nullptr;
+    }
+    ctx->copies.clear();
+    return DSC_OK;
+}
+
 int launch_kernel(Context* ctx, Kernel* k, void* const* device_ptrs, int n, uint32_t rand_seed) {
     if (ctx->offline || !k->function) return fail(DSC_ERR_NO_DEVICE, "kernel launch without a device");
     if (n != k->gen.n_buffers)
@@ -366,6 +540,7 @@ int launch_kernel(Context* ctx, Kernel* k, void* const* device_ptrs, int n, uint
         HIP_TRY(hipEventRecord(start, ctx->stream));
     }
     HIP_TRY(hipModuleLaunchKernel(k->function, k->gen.grid, 1, 1, k->gen.block, 1, 1, 0, ctx->stream, args, nullptr));
+    ++ctx->work_seq;
     if (ctx->profiling) {
         HIP_TRY(hipEventRecord(stop, ctx->stream));
         ctx->profile.push_back(ProfileEntry{start, stop, k});

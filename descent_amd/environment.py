@@ -95,11 +95,45 @@ class Environment:
     def writer(self, parameter: Parameter) -> ParameterWriter:
         """Frees the old buffer and allocates a new one (src/environment.rs:160-175)."""
         parameter.checked(self)
-        if parameter.buffer is not None:
-            self.backend.free(parameter.buffer)
-            parameter.buffer = None
-        parameter.buffer = self.backend.alloc(parameter.shape.buffer_size())
+        self._fresh_buffer(parameter)
         return ParameterWriter(self.backend, parameter.buffer, parameter.shape.buffer_size())
+
+    def _fresh_buffer(self, parameter: Parameter, io: bool = False) -> None:
+        # The new buffer is taken before the old one is given back (the reference frees first): the old one is
+        # still read by the step enqueued before this call, and an upload into other memory can run beside that step.
+        old = parameter.buffer
+        alloc = self.backend.alloc_io if io else self.backend.alloc
+        parameter.buffer = alloc(parameter.shape.buffer_size())
+        if old is not None:
+            self.backend.free(old)
+
+    def host_array(self, parameter: Parameter) -> np.ndarray:
+        """Pinned host array of the parameter's shape for write_parameter_async / read_parameter_async."""
+        parameter.checked(self)
+        return self.backend.host_array(tuple(parameter.shape), np.float32)
+
+    def write_parameter_async(self, parameter: Parameter, data: np.ndarray) -> int:
+        """Like write_parameter, on the backend's copy stream: the upload overlaps with graph runs enqueued before
+        it, later runs wait for it.  `data` from host_array() is read in place and must not be rewritten before
+        the returned fence has finished (backend.fence_wait); other arrays are copied before the call returns."""
+        parameter.checked(self)
+        data = np.ascontiguousarray(data)
+        if data.dtype not in (np.float32, np.uint32, np.int32):
+            data = data.astype(np.float32)
+        if data.nbytes != parameter.shape.buffer_size():
+            raise ValueError(f"parameter {parameter.name!r} holds {parameter.shape.buffer_size()} bytes, got {data.nbytes}")
+        self._fresh_buffer(parameter, io=True)
+        return self.backend.write_async(parameter.buffer, 0, data)
+
+    def read_parameter_async(self, parameter: Parameter, out: np.ndarray) -> int:
+        """Starts a read-back of the parameter's current value into `out` (from host_array()) without blocking;
+        `out` holds it once the returned fence has finished."""
+        parameter.checked(self)
+        if parameter.buffer is None:
+            raise ValueError(f"parameter {parameter.name!r} has no value")
+        if out.nbytes != parameter.shape.buffer_size():
+            raise ValueError(f"parameter {parameter.name!r} holds {parameter.shape.buffer_size()} bytes, got {out.nbytes}")
+        return self.backend.read_async(parameter.buffer, 0, out)
 
     def write_parameter(self, parameter: Parameter, data) -> None:
         data = np.ascontiguousarray(data)
@@ -127,6 +161,32 @@ class Environment:
 
     def read_parameter_scalar(self, parameter: Parameter) -> float:
         return float(self.read_parameter_to_vec(parameter)[0])
+
+    def save_parameters(self, path, parameters) -> int:
+        """Writes the parameters' values to `path` as raw little-endian f32, in the order given and with no header --
+        what piping each `reader()` (io::Read, src/environment.rs:63-67, 177-189) into one file gives.  Returns the
+        number of bytes written."""
+        total = 0
+        with open(path, "wb") as f:
+            for p in parameters:
+                data = self.reader(p)
+                f.write(data)
+                total += len(data)
+        return total
+
+    def load_parameters(self, path, parameters) -> None:
+        """Reads a file written by save_parameters back through `writer()` (io::Write, src/environment.rs:50-61).
+        The file must hold exactly the listed parameters' bytes."""
+        import os
+
+        want = sum(p.shape.buffer_size() for p in parameters)
+        have = os.path.getsize(path)
+        if have != want:
+            raise ValueError(f"{path}: {have} bytes, the parameters hold {want}")
+        with open(path, "rb") as f:
+            for p in parameters:
+                with self.writer(p) as w:
+                    w.write(np.frombuffer(f.read(p.shape.buffer_size()), dtype=np.float32))
 
     def reset_parameter(self, parameter: Parameter, rng: np.random.Generator) -> None:
         """src/environment.rs:190-202. The reference draws from ChaCha20 via the

@@ -55,6 +55,11 @@ def lib():
         "dsc_buf_write": (C.c_int, [vp, u64, sz, vp, sz]),
         "dsc_buf_fill_zero": (C.c_int, [vp, u64, sz, sz]),
         "dsc_buf_read": (C.c_int, [vp, u64, sz, vp, sz]),
+        "dsc_buf_alloc_io": (C.c_int, [vp, sz, C.POINTER(u64)]),
+        "dsc_host_alloc": (C.c_int, [vp, sz, C.POINTER(vp)]),
+        "dsc_host_free": (C.c_int, [vp, vp]),
+        "dsc_buf_write_async": (C.c_int, [vp, u64, sz, vp, sz, C.POINTER(u64)]),
+        "dsc_buf_read_async": (C.c_int, [vp, u64, sz, vp, sz, C.POINTER(u64)]),
         "dsc_kernel_get": (C.c_int, [vp, C.POINTER(_abi.CKernelDesc), C.POINTER(vp)]),
         "dsc_kernel_buffer_count": (C.c_int, [vp]),
         "dsc_kernel_reference_group_count": (C.c_int64, [vp]),
@@ -88,7 +93,7 @@ EXPORTED_SYMBOLS = [
     "dsc_last_error", "dsc_ctx_create", "dsc_ctx_destroy", "dsc_ctx_caps", "dsc_ctx_sync", "dsc_ctx_stream",
     "dsc_fence_record", "dsc_fence_wait", "dsc_fence_query",
     "dsc_buf_alloc", "dsc_buf_free", "dsc_buf_info", "dsc_heap_stats", "dsc_buf_write", "dsc_buf_fill_zero",
-    "dsc_buf_read", "dsc_kernel_get", "dsc_kernel_buffer_count", "dsc_kernel_reference_group_count",
+    "dsc_buf_read", "dsc_buf_alloc_io", "dsc_host_alloc", "dsc_host_free", "dsc_buf_write_async", "dsc_buf_read_async", "dsc_kernel_get", "dsc_kernel_buffer_count", "dsc_kernel_reference_group_count",
     "dsc_kernel_label", "dsc_kernel_source", "dsc_kernel_launch", "dsc_codegen_source", "dsc_codegen_compile",
     "dsc_codegen_check_schedule", "dsc_free_string", "dsc_schedule_create", "dsc_schedule_destroy",
     "dsc_schedule_run", "dsc_schedule_launch_count", "dsc_schedule_describe", "dsc_prof_enable", "dsc_prof_reset",
@@ -174,6 +179,7 @@ class HipBackend:
         self._ctx = C.c_void_p()
         check(lib().dsc_ctx_create(device, C.byref(self._ctx)))
         self._kernels = {}
+        self._pinned = {}
 
     def close(self):
         if self._ctx:
@@ -192,6 +198,12 @@ class HipBackend:
         check(lib().dsc_buf_alloc(self._ctx, nbytes, C.byref(h)))
         return h.value
 
+    def alloc_io(self, nbytes: int) -> int:
+        """A buffer from the device memory set aside for overlapped uploads."""
+        h = C.c_uint64()
+        check(lib().dsc_buf_alloc_io(self._ctx, nbytes, C.byref(h)))
+        return h.value
+
     def free(self, handle: int) -> None:
         check(lib().dsc_buf_free(self._ctx, handle))
 
@@ -206,6 +218,36 @@ class HipBackend:
         out = np.empty(nbytes, dtype=np.uint8)
         check(lib().dsc_buf_read(self._ctx, handle, offset, out.ctypes.data, nbytes))
         return out.tobytes()
+
+    # -- overlapped I/O (second stream) -----------------------------------------------------------------------
+    def host_array(self, shape, dtype=np.float32) -> np.ndarray:
+        """A numpy array over pinned host memory (dsc_host_alloc) that write_async / read_async use in place.
+        The memory lives until host_release(array) or the backend is closed."""
+        dtype = np.dtype(dtype)
+        count = int(np.prod(shape)) if np.ndim(shape) else int(shape)
+        nbytes = max(1, count * dtype.itemsize)
+        p = C.c_void_p()
+        check(lib().dsc_host_alloc(self._ctx, nbytes, C.byref(p)))
+        raw = (C.c_uint8 * nbytes).from_address(p.value)
+        arr = np.frombuffer(raw, dtype=dtype, count=count).reshape(shape)
+        self._pinned[arr.ctypes.data] = p.value
+        return arr
+
+    def host_release(self, arr: np.ndarray) -> None:
+        check(lib().dsc_host_free(self._ctx, self._pinned.pop(arr.ctypes.data)))
+
+    def write_async(self, handle: int, offset: int, data: np.ndarray) -> int:
+        """Upload on the copy stream; returns the fence after which a pinned `data` may be rewritten."""
+        arr = np.ascontiguousarray(data)
+        f = C.c_uint64()
+        check(lib().dsc_buf_write_async(self._ctx, handle, offset, arr.ctypes.data, arr.nbytes, C.byref(f)))
+        return f.value
+
+    def read_async(self, handle: int, offset: int, out: np.ndarray) -> int:
+        """Read-back into a host_array; the data is valid once the returned fence has finished."""
+        f = C.c_uint64()
+        check(lib().dsc_buf_read_async(self._ctx, handle, offset, out.ctypes.data, out.nbytes, C.byref(f)))
+        return f.value
 
     def device_ptr(self, handle: int) -> int:
         p, n = C.c_void_p(), C.c_size_t()

@@ -214,6 +214,33 @@ int dsc_buf_fill_zero(dsc_ctx* ctx, dsc_buf buf, size_t offset, size_t bytes);
 /* StagingReader::read_slice to completion (device/staging.rs:225-302): device -> host, blocking. */
 int dsc_buf_read(dsc_ctx* ctx, dsc_buf buf, size_t offset, void* dst, size_t bytes);
 
+/* Overlapped parameter I/O.  The reference pushes every upload and read-back through the one queue that also runs
+ * the kernels (StagingWriter / StagingReader submit on the shared command buffers, device/staging.rs:143-178,
+ * 262-302), so a mini-batch upload (examples/fashion_mnist/main.rs:42-60 through Environment::writer,
+ * environment.rs:160-175) serialises with the step before it.  These entry points use a second stream:
+ *   dsc_buf_alloc_io                 a buffer like dsc_buf_alloc's (same handle type, same dsc_buf_free), from device
+ *                                    memory set aside for uploads: nothing else is ever placed there, so what the
+ *                                    memory held before is an older upload buffer and not a temporary of the step
+ *                                    that is still running;
+ *   dsc_host_alloc / dsc_host_free   pinned host memory that copies can use in place (no staging copy);
+ *   dsc_buf_write_async              host -> device on the copy stream.  The copy waits only for the compute work that
+ *                                    last used the buffer's memory, so it runs beside a step enqueued earlier when the
+ *                                    buffer was not taken from memory that step used (dsc_buf_alloc_io, and allocate the
+ *                                    new buffer before freeing the old one); every later launch, run or copy on the compute stream waits
+ *                                    for it.  `src` inside a dsc_host_alloc range is read in place and must stay
+ *                                    untouched until *out_fence has finished; any other `src` is copied through the
+ *                                    staging ring before the call returns.  out_fence may be null.
+ *   dsc_buf_read_async               device -> pinned host (dst must come from dsc_host_alloc) of the value that the
+ *                                    work enqueued so far leaves in the buffer; the data is there once *out_fence has
+ *                                    finished (dsc_fence_wait / dsc_fence_query).  The host does not block.
+ * Fences of the copy stream share the id space of dsc_fence_record; waiting for one retires only older fences of the
+ * same stream. */
+int dsc_buf_alloc_io(dsc_ctx* ctx, size_t bytes, dsc_buf* out);
+int dsc_host_alloc(dsc_ctx* ctx, size_t bytes, void** out_ptr);
+int dsc_host_free(dsc_ctx* ctx, void* ptr);
+int dsc_buf_write_async(dsc_ctx* ctx, dsc_buf buf, size_t offset, const void* src, size_t bytes, uint64_t* out_fence);
+int dsc_buf_read_async(dsc_ctx* ctx, dsc_buf buf, size_t offset, void* dst, size_t bytes, uint64_t* out_fence);
+
 struct dsc_schedule_desc;
 
 /* ---------------------------------------------------------------- kernels */

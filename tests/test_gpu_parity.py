@@ -437,3 +437,83 @@ def test_conv2d_gradients_over_geometries(hip_backend_session, geom, fused):
     assert rel_l2(gy, cy) <= TOL, listing
     assert rel_l2(gdx, cdx) <= TOL, (rel_l2(gdx, cdx), listing)
     assert rel_l2(gdf, cdf) <= TOL, (rel_l2(gdf, cdf), listing)
+
+
+@pytest.mark.parametrize("batch", [64, 1000])
+def test_overlapped_uploads_and_readbacks_match_the_serial_path(hip_backend_session, batch):
+    """Fourteen ConvNet steps (batch 64: steps shorter than an upload's latency; batch 1000: 3 MB uploads beside
+    270 us steps), a new mini-batch uploaded before each: once through Environment.writer on
+    the compute stream, once through the copy stream from alternating pinned arrays (uploads overlap the step before,
+    the host never waits for a step), with a non-blocking read-back of the running loss after every step.  Same
+    kernels, same data, no float atomics in this graph: every parameter and every loss must be bit-equal."""
+    from descent_amd import Environment, workloads
+
+    be = hip_backend_session
+    steps = 14
+    rng = np.random.default_rng(5)
+    xs = [rng.random((batch, 28, 28, 1), dtype=np.float32) for _ in range(steps)]
+    ys = [rng.integers(0, 10, (batch, 1)).astype(np.float32) for _ in range(steps)]
+
+    env_a, env_b = Environment(be), Environment(be)
+    wa = workloads.convnet(env_a, batch=batch, seed=23)
+    wb = workloads.convnet(env_b, batch=batch, seed=23)
+    losses_a = []
+    for i in range(steps):
+        env_a.write_parameter(wa.inputs["x"], xs[i])
+        env_a.write_parameter(wa.inputs["y"], ys[i])
+        env_a.run(wa.graph, 900 + i)
+        losses_a.append(env_a.read_parameter_scalar(wa.scalars["loss"]))
+
+    px = [env_b.host_array(wb.inputs["x"]) for _ in range(2)]
+    py = [env_b.host_array(wb.inputs["y"]) for _ in range(2)]
+    loss_out = [be.host_array((1,), np.float32) for _ in range(steps)]
+    upload_fence, read_fence = [0, 0], []
+    for i in range(steps):
+        s = i & 1
+        if upload_fence[s]:
+            be.fence_wait(upload_fence[s])  # the pinned pair is free again once its last upload has finished
+        px[s][...] = xs[i]
+        py[s][...] = ys[i]
+        env_b.write_parameter_async(wb.inputs["x"], px[s])
+        upload_fence[s] = env_b.write_parameter_async(wb.inputs["y"], py[s])
+        env_b.run(wb.graph, 900 + i)
+        read_fence.append(env_b.read_parameter_async(wb.scalars["loss"], loss_out[i]))
+    for f in read_fence:
+        be.fence_wait(f)
+    losses_b = [float(v[0]) for v in loss_out]
+    assert losses_a == losses_b
+    got, want = wb.snapshot(), wa.snapshot()
+    for key in want:
+        assert np.array_equal(got[key], want[key]), key
+    for arr in px + py + loss_out:
+        be.host_release(arr)
+
+
+def test_overlapped_io_argument_checks(hip_backend_session):
+    from descent_amd.hip_backend import DescentHipError
+
+    be = hip_backend_session
+    buf = be.alloc_io(4096)
+    pinned = be.host_array((1024,), np.float32)
+    pinned[:] = np.arange(1024, dtype=np.float32)
+    compute_fence = be.fence_record()
+    copy_fence = be.write_async(buf, 0, pinned)
+    be.fence_wait(copy_fence)
+    # ids are shared between the streams, order is per stream: the older compute fence is still known and waitable
+    be.fence_wait(compute_fence)
+    assert be.fence_finished(copy_fence) and be.fence_finished(compute_fence)
+    back = be.host_array((1024,), np.float32)
+    be.fence_wait(be.read_async(buf, 0, back))
+    assert np.array_equal(back, pinned)
+    # pageable sources are staged (the array may be reused at once); pageable destinations are refused
+    data = np.full(1024, 3.0, np.float32)
+    be.write_async(buf, 0, data)
+    data[:] = 0.0
+    assert np.array_equal(np.frombuffer(be.read(buf, 0, 4096), np.float32), np.full(1024, 3.0, np.float32))
+    with pytest.raises(DescentHipError):
+        be.read_async(buf, 0, np.empty(1024, np.float32))
+    with pytest.raises(DescentHipError):
+        be.write_async(buf, 8, pinned)  # range outside the buffer
+    be.host_release(pinned)
+    be.host_release(back)
+    be.free(buf)

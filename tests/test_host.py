@@ -222,6 +222,24 @@ def test_writer_zero_fills_the_unwritten_tail():
     assert np.array_equal(env.read_parameter_to_vec(p), np.array([0, 1, 2, 0, 0, 0, 0, 0], np.float32))
 
 
+def test_parameters_round_trip_through_a_raw_f32_file(tmp_path):
+    env = _env()
+    rng = np.random.default_rng(1)
+    shapes = ([3, 5], [7], [2, 2, 2])
+    params = [env.static_parameter_with_data(sh, f"p{i}", rng.standard_normal(sh, dtype=np.float32)) for i, sh in enumerate(shapes)]
+    before = [env.read_parameter(p) for p in params]
+    path = tmp_path / "params.f32"
+    assert env.save_parameters(path, params) == 4 * (15 + 7 + 8)
+    assert np.array_equal(np.fromfile(path, dtype="<f4"), np.concatenate([b.ravel() for b in before]))
+    for p in params:
+        env.writer(p).zero_fill()
+    env.load_parameters(path, params)
+    for p, b in zip(params, before):
+        assert np.array_equal(env.read_parameter(p), b)
+    with pytest.raises(ValueError, match="bytes"):
+        env.load_parameters(path, params[:2])
+
+
 def test_image_fit_parameter_counts_match_the_reference_readme():
     """examples/image_fit/README.md:31-34: ReLU 44099, ReLU-PE 51779, SIREN 44099, MULTI-HASH 43977 trainable
     parameters for hidden units [256,128,64,32], 8 frequencies, and 10 levels from 2 to 512 with 4096 entries."""
