@@ -315,6 +315,8 @@ def main():
                     help="headline: the 8192^3 matmul line with the ConvNet step rate beside it (default); matmul: "
                          "that line without the ConvNet; the others run one workload alone, e.g. under rocprofv3")
     ap.add_argument("--no-events", action="store_true", help="no per-launch HIP events (wall time only)")
+    ap.add_argument("--markers", action="store_true",
+                    help="wrap every launch in a ROCTx range named by the kernel's label (rocprofv3 --marker-trace)")
     args = ap.parse_args()
     global EVENT_PASS
     EVENT_PASS = not args.no_events
@@ -326,6 +328,8 @@ def main():
     from descent_amd.hip_backend import HipBackend
 
     env = Environment(HipBackend())
+    if args.markers:
+        env.backend.markers(True)
     if args.copy_calibration:
         print(json.dumps(bench_elementwise(env, 1 << 26, args.steps, args.warmup)))
         return

@@ -555,6 +555,22 @@ int dsc_schedule_describe(const dsc_schedule* s, char** out_text) {
     return *out_text ? DSC_OK : fail(DSC_ERR_OOM, "host allocation failed");
 }
 
+int dsc_schedule_dot(const dsc_schedule* s, char** out_text) {
+    if (!s || !out_text) return fail(DSC_ERR_INVALID, "null argument");
+    *out_text = dup_string(s->s.dot());
+    return *out_text ? DSC_OK : fail(DSC_ERR_OOM, "host allocation failed");
+}
+
+int dsc_prof_markers(dsc_ctx* ctx, int enabled) {
+    if (!ctx) return fail(DSC_ERR_INVALID, "null context");
+    if (!enabled) {
+        ctx->c.range_push = nullptr;
+        ctx->c.range_pop = nullptr;
+        return DSC_OK;
+    }
+    return load_markers(&ctx->c);
+}
+
 int dsc_prof_enable(dsc_ctx* ctx, int enabled) {
     if (!ctx) return fail(DSC_ERR_INVALID, "null context");
     ctx->c.profiling = enabled != 0;

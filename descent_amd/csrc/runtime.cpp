@@ -1,5 +1,7 @@
 #include "runtime.hpp"
 
+#include <dlfcn.h>
+
 #include <hip/hiprtc.h>
 
 #include <algorithm>
@@ -424,6 +426,25 @@ hipEvent_t take_plain_event(Context* ctx) {
     return ev;
 }
 
+int load_markers(Context* ctx) {
+    if (ctx->range_push && ctx->range_pop) return DSC_OK;
+    static void* roctx = [] {
+        void* h = dlopen("librocprofiler-sdk-roctx.so.1", RTLD_NOW | RTLD_GLOBAL);
+        if (!h) h = dlopen("librocprofiler-sdk-roctx.so", RTLD_NOW | RTLD_GLOBAL);
+        if (!h) h = dlopen("libroctx64.so.4", RTLD_NOW | RTLD_GLOBAL);
+        return h;
+    }();
+    if (!roctx) return fail(DSC_ERR_UNSUPPORTED, "no ROCTx library (librocprofiler-sdk-roctx.so, libroctx64.so) could be loaded");
+    ctx->range_push = reinterpret_cast<int (*)(const char*)>(dlsym(roctx, "roctxRangePushA"));
+    ctx->range_pop = reinterpret_cast<int (*)()>(dlsym(roctx, "roctxRangePop"));
+    if (!ctx->range_push || !ctx->range_pop) {
+        ctx->range_push = nullptr;
+        ctx->range_pop = nullptr;
+        return fail(DSC_ERR_UNSUPPORTED, "the ROCTx library lacks roctxRangePushA / roctxRangePop");
+    }
+    return DSC_OK;
+}
+
 int enable_async_io(Context* ctx) {
     if (ctx->async_io) return DSC_OK;
     if (ctx->offline) return fail(DSC_ERR_NO_DEVICE, "overlapped I/O without a device");
@@ -539,7 +560,10 @@ int launch_kernel(Context* ctx, Kernel* k, void* const* device_ptrs, int n, uint
         HIP_TRY(take(&stop));
         HIP_TRY(hipEventRecord(start, ctx->stream));
     }
-    HIP_TRY(hipModuleLaunchKernel(k->function, k->gen.grid, 1, 1, k->gen.block, 1, 1, 0, ctx->stream, args, nullptr));
+    if (ctx->range_push) (void)ctx->range_push(k->label.c_str());
+    const hipError_t launched = hipModuleLaunchKernel(k->function, k->gen.grid, 1, 1, k->gen.block, 1, 1, 0, ctx->stream, args, nullptr);
+    if (ctx->range_pop) (void)ctx->range_pop();
+    if (launched != hipSuccess) return fail(DSC_ERR_HIP, "hipModuleLaunchKernel '" + k->label + "': " + hipGetErrorString(launched));
     ++ctx->work_seq;
     if (ctx->profiling) {
         HIP_TRY(hipEventRecord(stop, ctx->stream));

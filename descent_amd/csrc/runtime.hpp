@@ -141,6 +141,11 @@ struct Context {
     std::vector<CopyInFlight> copies;
     std::map<const char*, size_t> pinned;  // dsc_host_alloc ranges: base -> bytes
 
+    // ROCTx ranges named by the kernel label around every launch (reference: debug-utils labels per cluster,
+    // src/environment.rs:452-463); resolved from the ROCTx library at run time, null when off
+    int (*range_push)(const char*) = nullptr;
+    int (*range_pop)() = nullptr;
+
     bool profiling = false;
     std::vector<ProfileEntry> profile;
     std::vector<hipEvent_t> event_pool;
@@ -156,7 +161,8 @@ int enable_async_io(Context* ctx);                  // creates the copy stream; 
 int mark_stream(Context* ctx);                      // an event on `stream` that covers work_seq
 int copy_stream_wait(Context* ctx, uint64_t stamp); // copy stream waits for compute work up to `stamp`
 int join_copies(Context* ctx);                      // `stream` waits for the copies enqueued so far
-hipEvent_t take_plain_event(Context* ctx);          // from fence_pool, or new; nullptr on failure
+hipEvent_t take_plain_event(Context* ctx);
+int load_markers(Context* ctx);                     // resolves roctxRangePushA / roctxRangePop          // from fence_pool, or new; nullptr on failure
 
 
 // Compiles (or fetches) the kernel for a fused descriptor.  Returns nullptr and sets the error on failure.

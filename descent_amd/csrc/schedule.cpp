@@ -1396,4 +1396,56 @@ std::string Schedule::describe() const {
     return o.str();
 }
 
+std::string Schedule::dot() const {
+    auto escaped = [](const std::string& t) {
+        std::string r;
+        for (char ch : t) {
+            if (ch == '"' || ch == '\\') r += '\\';
+            r += ch;
+        }
+        return r;
+    };
+    std::ostringstream o;
+    o << "digraph schedule {\n  rankdir=TB;\n  node [fontname=\"monospace\",fontsize=10];\n";
+    std::vector<int> producer(n_nodes, -1);    // step that writes the node
+    std::vector<int> from_param(n_nodes, -1);  // parameter slot the node's buffer comes from
+    for (auto& io : inputs) {
+        from_param[io.node] = io.param;
+        o << "  pin" << io.param << " [shape=ellipse,label=\"parameter " << io.param << "\\n" << node_bytes[io.node] << " B\"];\n";
+    }
+    for (size_t pi = 0; pi < prefills.size(); ++pi) {
+        o << "  f" << pi << " [shape=box,style=dashed,label=\"prefill: " << escaped(prefills[pi].kernel->label) << "\"];\n";
+    }
+    for (size_t i = 0; i < steps.size(); ++i) {
+        const Step& st = steps[i];
+        char work[64];
+        std::snprintf(work, sizeof work, "%.3f MB", st.kernel->gen.algo_bytes / 1e6);
+        o << "  s" << i << " [shape=box,style=filled,fillcolor=\"" << (st.covers.size() > 1 ? "#cfe8ff" : "#eeeeee") << "\",label=\"" << i
+          << ": " << escaped(st.kernel->label) << "\\n" << escaped(st.kernel->gen.note) << "\\ngrid " << st.kernel->gen.grid << "x"
+          << st.kernel->gen.block << ", " << work << ", clusters";
+        for (int c : st.covers) o << " " << c;
+        o << "\"];\n";
+        for (int nd : st.inputs) {
+            if (producer[nd] >= 0)
+                o << "  s" << producer[nd] << " -> s" << i << " [label=\"n" << nd << ": " << node_bytes[nd] << " B\"];\n";
+            else if (from_param[nd] >= 0)
+                o << "  pin" << from_param[nd] << " -> s" << i << ";\n";
+        }
+        for (auto& out : st.outputs) {
+            // an accumulator taken over from another node (or from a literal) continues that node's buffer
+            if (out.copy_from >= 0 && producer[out.copy_from] >= 0)
+                o << "  s" << producer[out.copy_from] << " -> s" << i << " [style=dashed,label=\"n" << out.copy_from << " in place\"];\n";
+            else if (out.copy_from >= 0 && from_param[out.copy_from] >= 0)
+                o << "  pin" << from_param[out.copy_from] << " -> s" << i << " [style=dashed,label=\"in place\"];\n";
+            producer[out.node] = (int)i;
+        }
+    }
+    for (auto& io : outputs) {
+        o << "  pout" << io.param << " [shape=ellipse,peripheries=2,label=\"parameter " << io.param << "\\n" << node_bytes[io.node] << " B\"];\n";
+        if (producer[io.node] >= 0) o << "  s" << producer[io.node] << " -> pout" << io.param << ";\n";
+    }
+    o << "}\n";
+    return o.str();
+}
+
 }  // namespace dsc

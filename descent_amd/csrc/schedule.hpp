@@ -51,6 +51,9 @@ struct Schedule {
     int build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags);
     int run(Context* ctx, dsc_buf* params, uint32_t rand_seed);
     std::string describe() const;
+    // The schedule after fusion as a graphviz digraph (the reference exports its graph before scheduling,
+    // src/graph.rs:656-760): one box per launch, one ellipse per parameter slot, one edge per buffer.
+    std::string dot() const;
     // kernels one run enqueues: the steps, the prefill launches, and a Fill per literal-initialised accumulator
     // that no prefill covers
     int launches_per_run() const;

@@ -75,6 +75,8 @@ def lib():
         "dsc_schedule_run": (C.c_int, [vp, vp, C.POINTER(u64), u32]),
         "dsc_schedule_launch_count": (C.c_int, [vp, C.POINTER(i32), C.POINTER(i32)]),
         "dsc_schedule_describe": (C.c_int, [vp, C.POINTER(vp)]),
+        "dsc_schedule_dot": (C.c_int, [vp, C.POINTER(vp)]),
+        "dsc_prof_markers": (C.c_int, [vp, C.c_int]),
         "dsc_prof_enable": (C.c_int, [vp, C.c_int]),
         "dsc_prof_reset": (C.c_int, [vp]),
         "dsc_prof_report": (C.c_int, [vp, C.c_int, C.POINTER(vp)]),
@@ -96,7 +98,7 @@ EXPORTED_SYMBOLS = [
     "dsc_buf_read", "dsc_buf_alloc_io", "dsc_host_alloc", "dsc_host_free", "dsc_buf_write_async", "dsc_buf_read_async", "dsc_kernel_get", "dsc_kernel_buffer_count", "dsc_kernel_reference_group_count",
     "dsc_kernel_label", "dsc_kernel_source", "dsc_kernel_launch", "dsc_codegen_source", "dsc_codegen_compile",
     "dsc_codegen_check_schedule", "dsc_free_string", "dsc_schedule_create", "dsc_schedule_destroy",
-    "dsc_schedule_run", "dsc_schedule_launch_count", "dsc_schedule_describe", "dsc_prof_enable", "dsc_prof_reset",
+    "dsc_schedule_run", "dsc_schedule_launch_count", "dsc_schedule_describe", "dsc_schedule_dot", "dsc_prof_markers", "dsc_prof_enable", "dsc_prof_reset",
     "dsc_prof_report", "dsc_prof_query", "dsc_prof_work",
 ]
 
@@ -171,6 +173,12 @@ class HipSchedule:
     def describe(self) -> str:
         out = C.c_void_p()
         check(lib().dsc_schedule_describe(self._handle, C.byref(out)))
+        return _take_string(out)
+
+    def dot(self) -> str:
+        """The fused schedule as a graphviz digraph."""
+        out = C.c_void_p()
+        check(lib().dsc_schedule_dot(self._handle, C.byref(out)))
         return _take_string(out)
 
 
@@ -310,6 +318,10 @@ class HipBackend:
     # -- timing -----------------------------------------------------------------------------------------
     def profile(self, enabled: bool) -> None:
         check(lib().dsc_prof_enable(self._ctx, 1 if enabled else 0))
+
+    def markers(self, enabled: bool) -> None:
+        """Wraps every launch in a ROCTx range named by the kernel's label (rocprofv3 --marker-trace)."""
+        check(lib().dsc_prof_markers(self._ctx, 1 if enabled else 0))
 
     def profile_reset(self) -> None:
         check(lib().dsc_prof_reset(self._ctx))

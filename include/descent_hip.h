@@ -337,6 +337,10 @@ int dsc_schedule_launch_count(const dsc_schedule* s, int32_t* out_launches, int3
 /* Text listing of the post-fusion schedule (reference: Graph::write_dot, graph.rs:661-763). Caller releases
  * with dsc_free_string. */
 int dsc_schedule_describe(const dsc_schedule* s, char** out_text);
+/* Graph::write_dot_file (graph.rs:656-760), for the schedule after fusion: a graphviz digraph with one box per
+ * launch (label, kernel choice, grid, algorithmic bytes, reference clusters covered), one ellipse per parameter slot
+ * and one edge per buffer handed from launch to launch.  Free the text with dsc_free_string. */
+int dsc_schedule_dot(const dsc_schedule* s, char** out_text);
 
 /* ----------------------------------------------------------------- timing */
 
@@ -344,6 +348,10 @@ int dsc_schedule_describe(const dsc_schedule* s, char** out_text);
  * elapsed time is accumulated per kernel label; dsc_prof_report prints total and top-N like
  * print_timings (device/timestamp.rs:155-179, environment.rs:518-520). */
 int dsc_prof_enable(dsc_ctx* ctx, int enabled);
+/* Debug labels per cluster (environment.rs:452-463 wraps each dispatch in a debug-utils label named
+ * Kernel::label_name): with `enabled`, every launch is wrapped in a ROCTx range named by the kernel's label, which
+ * rocprofv3 --marker-trace records.  DSC_ERR_UNSUPPORTED when no ROCTx library can be loaded. */
+int dsc_prof_markers(dsc_ctx* ctx, int enabled);
 int dsc_prof_reset(dsc_ctx* ctx);
 /* Writes a report into a malloc'd string (caller: dsc_free_string): one line per label with launches,
  * total ms, average us and the achieved GB/s or TFLOP/s against the HBM or fp32 MFMA peak, sorted by total

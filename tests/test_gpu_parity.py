@@ -517,3 +517,35 @@ def test_overlapped_io_argument_checks(hip_backend_session):
     be.host_release(pinned)
     be.host_release(back)
     be.free(buf)
+
+
+def test_schedule_dot_export_and_launch_labels(hip_backend_session):
+    """The fused schedule as graphviz text: every launch is a box, every buffer between launches an edge, and the
+    parameter slots the graph writes appear as sinks; ROCTx ranges around launches switch on and off without
+    changing results."""
+    from descent_amd import Environment, workloads
+
+    be = hip_backend_session
+    env = Environment(be)
+    w = workloads.convnet(env, batch=16, seed=2)
+    env.run(w.graph, 1)
+    sched = next(iter(w.graph.__dict__["_schedules"].values()))
+    dot = sched.dot()
+    launches, _ = sched.launch_count()
+    assert dot.startswith("digraph schedule {") and dot.rstrip().endswith("}")
+    assert dot.count("[shape=box,style=filled") == launches
+    assert "ConvDataGrad" in dot and "RowFused" in dot
+    assert dot.count("peripheries=2") == len(w.trainable) + len(w.state) + len(w.scalars)
+    assert dot.count("{") == dot.count("}") and dot.count('"') % 2 == 0
+    before = w.snapshot()
+    be.markers(True)
+    env.run(w.graph, 2)
+    be.markers(False)
+    env2 = Environment(be)
+    w2 = workloads.convnet(env2, batch=16, seed=2)
+    env2.run(w2.graph, 1)
+    env2.run(w2.graph, 2)
+    after, want = w.snapshot(), w2.snapshot()
+    for key in want:
+        assert np.array_equal(after[key], want[key]), key
+    assert any(not np.array_equal(before[k], after[k]) for k in want)
