@@ -318,8 +318,8 @@ struct Emitter {
                 case DSC_UN_SQRT: rhs = "sqrtf(" + a + ")"; break;
                 case DSC_UN_EXP: rhs = "expf(" + a + ")"; break;
                 case DSC_UN_LOG: rhs = "logf(" + a + ")"; break;
-                case DSC_UN_SIN: rhs = "sinf(" + a + ")"; break;
-                case DSC_UN_COS: rhs = "cosf(" + a + ")"; break;
+                case DSC_UN_SIN: rhs = "dsc_sin(" + a + ")"; break;
+                case DSC_UN_COS: rhs = "dsc_cos(" + a + ")"; break;
                 case DSC_UN_FLOAT_TO_UINT: rhs = "U2F((uint)" + a + ")"; break;
                 case DSC_UN_UINT_TO_FLOAT: rhs = "(float)F2U(" + a + ")"; break;
                 }
