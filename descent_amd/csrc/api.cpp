@@ -471,7 +471,7 @@ int dsc_codegen_source(const dsc_kernel_desc* desc, char** out_source) {
     if (!err.empty()) return fail(DSC_ERR_INVALID, err);
     Generated g;
     err = generate(FusedKernel::plain(*desc), &g);
-    if (!err.empty()) return fail(DSC_ERR_INVALID, err);
+    if (!err.empty()) return fail(err.find("too large") != std::string::npos ? DSC_ERR_UNSUPPORTED : DSC_ERR_INVALID, err);
     *out_source = dup_string(g.source);
     return *out_source ? DSC_OK : fail(DSC_ERR_OOM, "host allocation failed");
 }
@@ -482,7 +482,7 @@ int dsc_codegen_compile(const dsc_kernel_desc* desc, const char* arch, size_t* o
     if (!err.empty()) return fail(DSC_ERR_INVALID, err);
     Generated g;
     err = generate(FusedKernel::plain(*desc), &g);
-    if (!err.empty()) return fail(DSC_ERR_INVALID, err);
+    if (!err.empty()) return fail(err.find("too large") != std::string::npos ? DSC_ERR_UNSUPPORTED : DSC_ERR_INVALID, err);
     std::vector<char> code;
     std::string log;
     int rc = compile_source(g.source, arch, &code, &log);

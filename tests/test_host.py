@@ -106,6 +106,25 @@ def test_malformed_descriptors_are_rejected_with_a_message():
         assert e.value.status == _abi.ERR_INVALID and len(str(e.value)) > 20
 
 
+def test_tensors_beyond_32_bit_indexing_are_refused_not_wrapped():
+    """Kernels index with 32-bit integers: a descriptor whose output or any input reaches 2^31 elements is refused
+    with DSC_ERR_UNSUPPORTED; the largest size below the limit still generates."""
+    big = Shape((32768, 65536))
+    edge = Shape((32768, 65535))
+    over = [
+        K.PerElementKernel(big.element_count(), (big.identity_view(),), (1,), (K.PeLoad(0), K.PeUnary("Exp", 0))),
+        K.ReduceKernel(Shape((1, 65536)), big.identity_view(), "Sum", 0),
+        K.MatMulKernel(Shape((1, 1, 8, 8)), BATCHES, Shape((1, 8, 1 << 28)).identity_view(), Shape((1, 1 << 28, 8)).identity_view()),
+        K.FillKernel(K.Literal.f32(0.0), 1 << 31),
+    ]
+    for kernel in over:
+        with pytest.raises(hip_backend.DescentHipError) as e:
+            hip_backend.codegen_source(kernel)
+        assert e.value.status == _abi.ERR_UNSUPPORTED and "32-bit" in str(e.value), str(e.value)
+    ok = K.PerElementKernel(edge.element_count(), (edge.identity_view(),), (1,), (K.PeLoad(0), K.PeUnary("Exp", 0)))
+    assert "dsc_per_element_n2147450880" in hip_backend.codegen_source(ok)
+
+
 def test_array_api_cluster_structure_matches_the_reference_dumps():
     """docs/array_api_values.svg / array_api_grad.svg of the reference, reduced to JSON by
     tests/golden/make_array_api_fixture.py."""
