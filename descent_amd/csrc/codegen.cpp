@@ -1767,10 +1767,16 @@ string generate_scatter_chain(const FusedKernel& fk, Generated* out) {
         total += element_count(d.inputs[0].out_shape);
     }
     if (table * 4 > 144 * 1024) return "scatter chain: accumulator does not fit LDS";
-    const int64_t wgs = std::max<int64_t>(64, std::min<int64_t>(256, total / 16384));
-    const int U = 4;
+    // One workgroup per CU when there is work for that many: measured on hash-grid levels (2.1 M values), the LDS adds
+    // take about 1 ns each per CU, so halving the workgroups costs more than the smaller flush (every workgroup
+    // flushes the whole accumulator) gives back, up to the largest accumulator that fits.  A thread fetches U values
+    // of every link before it adds any (one memory round trip per trip, not one per link).
+    int64_t nmax = 0;
+    for (auto& part : fk.parts) nmax = std::max(nmax, element_count(part.main.raw().inputs[0].out_shape));
+    const int U = 2;
+    const int64_t wgs = std::max<int64_t>(64, std::min<int64_t>(256, (nmax + 1024 * U - 1) / (1024 * U)));
     Generated g;
-    std::ostringstream src, body;
+    std::ostringstream src, fetches, adds;
     src << kPreludeSource << "\n";
     int out_param = -1;
     for (size_t i = 0; i < fk.parts.size(); ++i) {
@@ -1779,24 +1785,26 @@ string generate_scatter_chain(const FusedKernel& fk, Generated* out) {
         Emitter em(part);
         const int64_t n = element_count(part.main.raw().inputs[0].out_shape);
         std::ostringstream fn;
-        fn << "DSC_INLINE void accumulate(float* acc, const uint first, " << em.params_decl() << ") {\n";
-        fn << "    for (uint g0 = first; g0 < " << S(n) << "u; g0 += " << S(wgs * 1024 * U) << "u) {\n";
-        for (int u = 0; u < U; ++u) {
-            fn << "    const uint gid" << u << " = min(g0 + " << S(u * wgs * 1024) << "u, " << S(n - 1) << "u);\n";
-            emit_scatter_element(em, fn, "gid" + to_string(u), to_string(u));
-        }
-        fn << "    __builtin_amdgcn_sched_barrier(0);\n";
-        for (int u = 0; u < U; ++u)
-            fn << "    if (ok" << u << " && g0 + " << S(u * wgs * 1024) << "u < " << S(n) << "u) atomicAdd(&acc[at" << u << "], value" << u << ");\n";
-        fn << "    }\n}\n";
+        fn << "DSC_INLINE void fetch(const uint gid, float* out_value, int* out_at, bool* out_ok, " << em.params_decl() << ") {\n";
+        emit_scatter_element(em, fn, "gid", "");
+        fn << "    *out_value = value;\n    *out_at = at;\n    *out_ok = ok;\n}\n";
         src << "namespace part" << i << " {\n" << em.funcs.str() << fn.str() << "}  // namespace part" << i << "\n\n";
-        body << "    part" << i << "::accumulate(acc, blockIdx.x * 1024u + threadIdx.x";
-        for (int j : fk.part_params[i]) body << ", b" << j;
-        body << ", rand_seed);\n";
+        for (int u = 0; u < U; ++u) {
+            const string id = "p" + to_string(i) + "u" + to_string(u);
+            const string gid = "g0 + " + S(u * wgs * 1024) + "u";
+            fetches << "        float v" << id << "; int a" << id << "; bool k" << id << ";\n";
+            fetches << "        part" << i << "::fetch(min(" << gid << ", " << S(n - 1) << "u), &v" << id << ", &a" << id << ", &k" << id;
+            for (int j : fk.part_params[i]) fetches << ", b" << j;
+            fetches << ", rand_seed);\n";
+            adds << "        if (k" << id << " && " << gid << " < " << S(n) << "u) atomicAdd(&acc[a" << id << "], v" << id << ");\n";
+        }
         out_param = fk.part_params[i][part.outputs[0]];
         Generated pg;  // for the work figures only
         if (generate_one(part, &pg, false).empty()) g.algo_bytes += pg.algo_bytes;
     }
+    std::ostringstream body;
+    body << "    for (uint g0 = blockIdx.x * 1024u + threadIdx.x; g0 < " << S(nmax) << "u; g0 += " << S(wgs * 1024 * U) << "u) {\n"
+         << fetches.str() << "        __builtin_amdgcn_sched_barrier(0);\n" << adds.str() << "    }\n";
     Emitter em(fk);
     g.entry = "dsc_scatter_chain_l" + to_string(fk.parts.size()) + "_t" + S(table) + "_n" + S(total);
     src << "extern \"C\" __global__ __launch_bounds__(1024) void " << g.entry << "(" << em.kernel_params_decl() << ") {\n";
