@@ -311,7 +311,7 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=4096,
                     help="rows of the headline product the CPU baseline computes (a bounded sample of the same workload)")
     ap.add_argument("--workload", default="headline",
-                    choices=["headline", "matmul", "convnet", "linear", "relu-pe", "siren", "hash-grid"],
+                    choices=["headline", "matmul", "convnet", "convnet-uploads", "linear", "relu-pe", "siren", "hash-grid"],
                     help="headline: the 8192^3 matmul line with the ConvNet step rate beside it (default); matmul: "
                          "that line without the ConvNet; the others run one workload alone, e.g. under rocprofv3")
     ap.add_argument("--no-events", action="store_true", help="no per-launch HIP events (wall time only)")
@@ -339,6 +339,8 @@ def main():
         if args.workload == "convnet":
             out = bench_convnet(env, args.steps, args.warmup)
             sys.stderr.write(out.pop("report"))
+        elif args.workload == "convnet-uploads":
+            out = bench_convnet_minibatch_uploads(env, steps=max(args.steps, 20))
         else:
             build = {"linear": lambda e: _w.linear_classifier(e), "relu-pe": lambda e: _w.coordinate_mlp(e), "siren": lambda e: _w.coordinate_mlp(e, variant="siren"),
                      "hash-grid": lambda e: _w.hash_grid_fit(e)}[args.workload]
