@@ -439,8 +439,8 @@ def test_conv2d_gradients_over_geometries(hip_backend_session, geom, fused):
     assert rel_l2(gdf, cdf) <= TOL, (rel_l2(gdf, cdf), listing)
 
 
-@pytest.mark.parametrize("batch", [64, 1000])
-def test_overlapped_uploads_and_readbacks_match_the_serial_path(hip_backend_session, batch):
+@pytest.mark.parametrize("batch,fused", [(64, True), (1000, True), (64, "graph-replay")])
+def test_overlapped_uploads_and_readbacks_match_the_serial_path(hip_backend_session, batch, fused):
     """Fourteen ConvNet steps (batch 64: steps shorter than an upload's latency; batch 1000: 3 MB uploads beside
     270 us steps), a new mini-batch uploaded before each: once through Environment.writer on
     the compute stream, once through the copy stream from alternating pinned arrays (uploads overlap the step before,
@@ -454,7 +454,7 @@ def test_overlapped_uploads_and_readbacks_match_the_serial_path(hip_backend_sess
     xs = [rng.random((batch, 28, 28, 1), dtype=np.float32) for _ in range(steps)]
     ys = [rng.integers(0, 10, (batch, 1)).astype(np.float32) for _ in range(steps)]
 
-    env_a, env_b = Environment(be), Environment(be)
+    env_a, env_b = Environment(be), Environment(be, fused=fused)  # with graph replay: copies join before the capture
     wa = workloads.convnet(env_a, batch=batch, seed=23)
     wb = workloads.convnet(env_b, batch=batch, seed=23)
     losses_a = []
