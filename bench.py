@@ -280,7 +280,7 @@ def cpu_baseline_matmul(n: int, rows: int):
     # the other half of the headline metric on the same cores: ConvNet (batch 1000) train steps
     cw = workloads.convnet(env, batch=1000, seed=3)
     env.run(cw.graph, 1)  # warm
-    conv_steps = 6
+    conv_steps = 24
     t0 = time.perf_counter()
     for i in range(conv_steps):
         env.run(cw.graph, 2 + i)
@@ -290,7 +290,7 @@ def cpu_baseline_matmul(n: int, rows: int):
         "unit": "TFLOP/s",
         "cores": min(cores, threads),
         "kind": "port",
-        "sample": f"{rows} rows of the {n}^3 product (A slab {rows}x{n}, full B), bias+leaky_relu included, {dt:.2f} s; "
+        "sample": f"{rows} of {n} rows of the {n}^3 product (A slab {rows}x{n}, full B), bias+leaky_relu included, {dt:.2f} s; "
                   f"plus {conv_steps} ConvNet bs1000 train steps, {conv_dt:.2f} s",
         "convnet_bs1000_steps_per_s": conv_steps / conv_dt,
     }
@@ -308,7 +308,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only the streaming c=a*2+b kernel over 2^26 elements (counter calibration)")
-    ap.add_argument("--cpu-rows", type=int, default=4096,
+    ap.add_argument("--cpu-rows", type=int, default=8192,
                     help="rows of the headline product the CPU baseline computes (a bounded sample of the same workload)")
     ap.add_argument("--workload", default="headline",
                     choices=["headline", "matmul", "convnet", "convnet-uploads", "linear", "relu-pe", "siren", "hash-grid"],
