@@ -1414,6 +1414,35 @@ string gen_matmul_tallk(Emitter& em, Generated* out) {
     return "";
 }
 
+// Tile configuration, k chunking and grid of the MFMA template for one product.
+struct MmPlan {
+    MmConfig c;
+    int64_t kchunks = 1, chunk_k = 0, grid = 0;
+};
+
+bool plan_mfma(const FusedKernel& fk, const MatMulDims& g, MmPlan* plan, bool as_part) {
+    const bool split = !fk.sum_chunks && g.chunks > 1;
+    MmConfig c = pick_config(g.m, g.n, split ? chunk_k_of(g) : g.k, g.batch * (split ? g.chunks : 1));
+    // inside a multi-part launch every part runs four waves: the one- and two-wave choices become 128x32 (narrow
+    // outputs) or 64x64 tiles
+    if (as_part && c.wm * c.wn < 4) c = g.n <= 32 ? MmConfig{128, 32, 16, 4, 1, 8} : MmConfig{64, 64, 16, 2, 2, 8};
+    // k chunking: the reference writes `chunks` partial products of chunk_tiles*16 k each (kernel.rs:436)
+    int64_t kchunks = 1, chunk_k = ((g.k + c.bk - 1) / c.bk) * c.bk;
+    if (split) {
+        const int64_t k_tiles = (g.k + 15) / 16;
+        const int64_t chunk_tiles = (k_tiles + g.chunks - 1) / g.chunks;
+        chunk_k = chunk_tiles * 16;
+        kchunks = g.chunks;
+        while (chunk_k % c.bk) c.bk /= 2;
+    }
+    if (!config_ok(c)) return false;
+    plan->c = c;
+    plan->kchunks = kchunks;
+    plan->chunk_k = chunk_k;
+    plan->grid = ((g.m + c.bm - 1) / c.bm) * ((g.n + c.bn - 1) / c.bn) * g.batch * kchunks;
+    return true;
+}
+
 string gen_matmul(Emitter& em, Generated* out) {
     const FusedKernel& fk = em.fk;
     const dsc_kernel_desc& d = fk.main.raw();
@@ -1424,19 +1453,11 @@ string gen_matmul(Emitter& em, Generated* out) {
     if (rows_kernel_applies(fk, g)) return gen_matmul_rows(em, out);
     if (smallk_kernel_applies(fk, g)) return gen_matmul_smallk(em, out);
     if (tallk_kernel_applies(fk, g)) return gen_matmul_tallk(em, out);
-    const bool split = !fk.sum_chunks && g.chunks > 1;
-    MmConfig c = pick_config(g.m, g.n, split ? chunk_k_of(g) : g.k, g.batch * (split ? g.chunks : 1));
-
-    // k chunking: the reference writes `chunks` partial products of chunk_tiles*16 k each (kernel.rs:436)
-    int64_t kchunks = 1, chunk_k = ((g.k + c.bk - 1) / c.bk) * c.bk;
-    if (!fk.sum_chunks && g.chunks > 1) {
-        const int64_t k_tiles = (g.k + 15) / 16;
-        const int64_t chunk_tiles = (k_tiles + g.chunks - 1) / g.chunks;
-        chunk_k = chunk_tiles * 16;
-        kchunks = g.chunks;
-        while (chunk_k % c.bk) c.bk /= 2;
-    }
-    if (!config_ok(c)) return "matmul: invalid tile configuration";
+    MmPlan plan;
+    if (!plan_mfma(fk, g, &plan, fk.as_part)) return "matmul: invalid tile configuration";
+    const MmConfig c = plan.c;
+    const int64_t kchunks = plan.kchunks, chunk_k = plan.chunk_k;
+    if (fk.as_part && 64 * c.wm * c.wn != 256) return "matmul: a part of a multi-part launch runs 256 threads";
 
     // operand addressing
     int a_mode = 0, b_mode = 0;
@@ -1480,6 +1501,7 @@ string gen_matmul(Emitter& em, Generated* out) {
     k << "#define C_CHUNK_STRIDE " << S(g.batch * g.m * g.n) << "\n#define C_BATCH_STRIDE " << S(batch_stride)
       << "\n#define C_ROW_STRIDE " << S(row_stride) << "\n";
     k << "#define MM_PARAMS " << em.kernel_params_decl() << "\n#define MM_ENTRY " << entry_name(fk) << "\n";
+    k << "#define MM_AS_PART " << (fk.as_part ? 1 : 0) << "\n#define MM_GRID " << S(plan.grid) << "\n";
 
     // results leave through LDS as 16-byte row pieces when the output allows it
     bool vec_store = g.n % 4 == 0 && batch_stride % 4 == 0 && row_stride % 4 == 0 && (g.batch * g.m * g.n) % 4 == 0;
@@ -1529,15 +1551,14 @@ string gen_matmul(Emitter& em, Generated* out) {
     }
     k << kMatmulMfmaSource;
 
-    const int64_t tiles = ((g.m + c.bm - 1) / c.bm) * ((g.n + c.bn - 1) / c.bn);
-    const int64_t grid = tiles * g.batch * kchunks;
+    const int64_t grid = plan.grid;
     if (grid >= kMaxIndex) return "matmul: grid too large";
     out->grid = (unsigned)grid;
     out->block = 64 * c.wm * c.wn;
     out->source = k.str();
     {
         const char* e = std::getenv("DSC_MM_PERSISTENT");
-        out->persistent_ok = !(e && e[0] == '0') && grid > 256 && chunk_k / c.bk <= 128;
+        out->persistent_ok = !(e && e[0] == '0') && !fk.as_part && grid > 256 && chunk_k / c.bk <= 128;
     }
     char note[160];
     std::snprintf(note, sizeof note, "mfma 32x32x2 tile %dx%dx%d waves %dx%d A%d B%d chunks %lld%s%s", c.bm, c.bn, c.bk, c.wm, c.wn,
@@ -1658,12 +1679,13 @@ std::string FusedKernel::key() const {
         for (int j : part_params[i]) s.append(reinterpret_cast<const char*>(&j), 4);
     }
     s += sum_chunks ? "|S1" : "|S0";
+    if (as_part) s += "|AP";
     s += "|O";
     for (int o : outputs) s.append(reinterpret_cast<const char*>(&o), 4);
     s.append(reinterpret_cast<const char*>(&n_buffers), 4);
     if (const char* env = std::getenv("DSC_MM_TILE"))
         if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|T") + env;
-    for (const char* name : {"DSC_MM_SMALLK", "DSC_MM_VEC_STORE", "DSC_MM_PERSISTENT", "DSC_MM_DEEP_K", "DSC_MM_ROWS", "DSC_ROWS_R", "DSC_ROWS_UNROLL", "DSC_ROWS_B", "DSC_ROWS_DIRECT_STORE", "DSC_MM_TALLK", "DSC_TALLK_UNROLL"})
+    for (const char* name : {"DSC_MM_SMALLK", "DSC_MM_VEC_STORE", "DSC_MM_PERSISTENT", "DSC_MM_DEEP_K", "DSC_MM_PART", "DSC_MM_ROWS", "DSC_ROWS_R", "DSC_ROWS_UNROLL", "DSC_ROWS_B", "DSC_ROWS_DIRECT_STORE", "DSC_MM_TALLK", "DSC_TALLK_UNROLL"})
         if (const char* env = std::getenv(name))
             if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|") + name + env;
     return s;
@@ -1683,10 +1705,15 @@ bool can_be_part(const FusedKernel& fk) {
     if (!fk.parts.empty()) return false;
     if (fk.dgrad.on || !fk.row_stages.empty()) return true;
     if (fk.main.raw().kind != DSC_KERNEL_MATMUL) return true;
-    // of the MatMul kernels, the row-per-thread, short-k and tall-k ones run 256 threads addressed by blockIdx.x; the
-    // MFMA template sizes its workgroups per shape and reads the grid size
+    // of the MatMul kernels, the row-per-thread, short-k and tall-k ones run 256 threads addressed by blockIdx.x
     const MatMulDims g = matmul_dims(fk.main.raw());
-    return rows_kernel_applies(fk, g) || smallk_kernel_applies(fk, g) || tallk_kernel_applies(fk, g);
+    if (rows_kernel_applies(fk, g) || smallk_kernel_applies(fk, g) || tallk_kernel_applies(fk, g)) return true;
+    // the MFMA template, when its tile choice runs four waves: small products only (large ones want their
+    // workgroups persistent and the CU's whole LDS, which a shared launch cannot give them)
+    if (const char* e = std::getenv("DSC_MM_PART"))
+        if (e[0] == '0') return false;
+    MmPlan plan;
+    return plan_mfma(fk, g, &plan, true) && 64 * plan.c.wm * plan.c.wn == 256 && plan.grid <= 1024;
 }
 
 static std::string generate_one(const FusedKernel& fk, Generated* out, bool with_prelude);
@@ -1843,17 +1870,21 @@ string generate_multi(const FusedKernel& fk, Generated* out) {
         const FusedKernel& part = fk.parts[i];
         if (!can_be_part(part)) return "multi: kernel cannot be a part";
         Generated pg;
-        string err = generate_one(part, &pg, false);
+        FusedKernel as_part = part;
+        as_part.as_part = true;
+        string err = generate_one(as_part, &pg, false);
         if (!err.empty()) return err;
         if (pg.block != 256) return "multi: parts must use 256 threads";
         if ((int)fk.part_params[i].size() != part.n_buffers) return "multi: part parameter count";
-        const string head = "extern \"C\" __global__ __launch_bounds__(256) void " + pg.entry + "(";
-        const size_t at = pg.source.find(head);
-        if (at == string::npos) return "multi: unexpected entry point form";
         string text = pg.source;
-        text.replace(at, head.size(), "DSC_INLINE void part_entry(const uint dsc_block, ");
-        for (size_t pos = text.find("blockIdx.x"); pos != string::npos; pos = text.find("blockIdx.x", pos)) text.replace(pos, 10, "dsc_block");
-        if (text.find("gridDim") != string::npos) return "multi: part depends on the grid size";
+        if (text.find("#define MM_AS_PART 1") == string::npos) {  // the MFMA template emits its part form itself
+            const string head = "extern \"C\" __global__ __launch_bounds__(256) void " + pg.entry + "(";
+            const size_t at = text.find(head);
+            if (at == string::npos) return "multi: unexpected entry point form";
+            text.replace(at, head.size(), "DSC_INLINE void part_entry(const uint dsc_block, ");
+            for (size_t pos = text.find("blockIdx.x"); pos != string::npos; pos = text.find("blockIdx.x", pos)) text.replace(pos, 10, "dsc_block");
+            if (text.find("gridDim") != string::npos) return "multi: part depends on the grid size";
+        }
         src << "namespace part" << i << " {\n" << text << "}  // namespace part" << i << "\n\n";
         body << "    if (blockIdx.x < " << first + pg.grid << "u) { part" << i << "::part_entry(blockIdx.x - " << first << "u";
         for (int j : fk.part_params[i]) body << ", b" << j;

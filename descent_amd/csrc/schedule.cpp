@@ -1077,7 +1077,9 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                     if (o.copy_from >= 0) return false;
                 if (grid_of[i] < 0) {
                     Generated g;
-                    if (!generate(d.fk, &g).empty() || g.block != 256) { grid_of[i] = (int64_t)1 << 40; return false; }
+                    FusedKernel probe = d.fk;
+                    probe.as_part = true;  // a kernel may pick another workgroup shape inside a shared launch
+                    if (!generate(probe, &g).empty() || g.block != 256) { grid_of[i] = (int64_t)1 << 40; return false; }
                     grid_of[i] = g.grid;
                 }
                 return grid_of[i] < ((int64_t)1 << 30);
