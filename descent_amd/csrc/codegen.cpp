@@ -1450,6 +1450,8 @@ string gen_matmul(Emitter& em, Generated* out) {
     const dsc_view& va = d.inputs[0];
     const dsc_view& vb = d.inputs[1];
     const bool rows = d.output_mode == DSC_MATMUL_ROWS;
+    if (fk.colsum_out >= 0 && (rows_kernel_applies(fk, g) || smallk_kernel_applies(fk, g) || tallk_kernel_applies(fk, g)))
+        return "matmul: column sums need the MFMA template";
     if (rows_kernel_applies(fk, g)) return gen_matmul_rows(em, out);
     if (smallk_kernel_applies(fk, g)) return gen_matmul_smallk(em, out);
     if (tallk_kernel_applies(fk, g)) return gen_matmul_tallk(em, out);
@@ -1502,6 +1504,13 @@ string gen_matmul(Emitter& em, Generated* out) {
       << "\n#define C_ROW_STRIDE " << S(row_stride) << "\n";
     k << "#define MM_PARAMS " << em.kernel_params_decl() << "\n#define MM_ENTRY " << entry_name(fk) << "\n";
     k << "#define MM_AS_PART " << (fk.as_part ? 1 : 0) << "\n#define MM_GRID " << S(plan.grid) << "\n";
+    if (fk.colsum_out >= 0) {
+        // the column sums are written as float4: n and the row of partials must be 16-byte aligned
+        if (b_mode != 1 || g.n % 4 != 0 || (64 * c.wm * c.wn) % (c.bn / 4) != 0) return "matmul: column sums need B contiguous along n";
+        k << "#define MM_COLSUM 1\n#define CS_PTR b" << fk.colsum_out << "\n";
+    } else {
+        k << "#define MM_COLSUM 0\n";
+    }
 
     // results leave through LDS as 16-byte row pieces when the output allows it
     bool vec_store = g.n % 4 == 0 && batch_stride % 4 == 0 && row_stride % 4 == 0 && (g.batch * g.m * g.n) % 4 == 0;
@@ -1561,8 +1570,9 @@ string gen_matmul(Emitter& em, Generated* out) {
         out->persistent_ok = !(e && e[0] == '0') && !fk.as_part && grid > 256 && chunk_k / c.bk <= 128;
     }
     char note[160];
-    std::snprintf(note, sizeof note, "mfma 32x32x2 tile %dx%dx%d waves %dx%d A%d B%d chunks %lld%s%s", c.bm, c.bn, c.bk, c.wm, c.wn,
-                  a_mode, b_mode, (long long)kchunks, fk.has_epilogue ? " +epilogue" : "", out->persistent_ok ? " persistent" : "");
+    std::snprintf(note, sizeof note, "mfma 32x32x2 tile %dx%dx%d waves %dx%d A%d B%d chunks %lld%s%s%s", c.bm, c.bn, c.bk, c.wm, c.wn,
+                  a_mode, b_mode, (long long)kchunks, fk.has_epilogue ? " +epilogue" : "", fk.colsum_out >= 0 ? " +column sums of B" : "",
+                  out->persistent_ok ? " persistent" : "");
     out->note = note;
     return "";
 }
@@ -1680,6 +1690,7 @@ std::string FusedKernel::key() const {
     }
     s += sum_chunks ? "|S1" : "|S0";
     if (as_part) s += "|AP";
+    if (colsum_out >= 0) s += "|CS" + to_string(colsum_out);
     s += "|O";
     for (int o : outputs) s.append(reinterpret_cast<const char*>(&o), 4);
     s.append(reinterpret_cast<const char*>(&n_buffers), 4);
@@ -1708,6 +1719,7 @@ bool can_be_part(const FusedKernel& fk) {
     // of the MatMul kernels, the row-per-thread, short-k and tall-k ones run 256 threads addressed by blockIdx.x
     const MatMulDims g = matmul_dims(fk.main.raw());
     if (rows_kernel_applies(fk, g) || smallk_kernel_applies(fk, g) || tallk_kernel_applies(fk, g)) return true;
+    if (fk.colsum_out >= 0) return false;
     // the MFMA template, when its tile choice runs four waves: small products only (large ones want their
     // workgroups persistent and the CU's whole LDS, which a shared launch cannot give them)
     if (const char* e = std::getenv("DSC_MM_PART"))

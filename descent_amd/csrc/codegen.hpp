@@ -76,6 +76,7 @@ struct FusedKernel {
         int32_t rows_first = 1;        // the Unpad along the image rows came first
     } dgrad;
     bool sum_chunks = false;               // MatMul: ignore the descriptor's chunk count, write one full sum
+    int colsum_out = -1;                   // MatMul (MFMA template): buffer that takes the column sums of B per k chunk
     bool as_part = false;                  // generated as one part of a multi-part launch (set while the launch is generated)
     std::vector<int> outputs;              // pointer parameter index of each output of main (or of the epilogue)
     int n_buffers = 0;                     // number of pointer parameters

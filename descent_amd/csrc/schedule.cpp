@@ -335,6 +335,118 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             drafts[i].keep_split = true;
         }
 
+        // Pass 0c: a bias gradient is the sum of dZ [K, N] over its rows, and the weight gradient A^T dZ of the same
+        // layer reads dZ as its B operand, k chunk by k chunk.  The MFMA kernel then also writes the column sums of
+        // the B tiles it loads, one row of partials per chunk, and the Reduce shrinks from K rows to `chunks` rows: one
+        // pass over dZ instead of two.  Only large dZ (the Reduce is a launch of its own there).
+        for (size_t ri = 0; ri < drafts.size(); ++ri) {
+            const dsc_kernel_desc rd = drafts[ri].fk.main.raw();
+            if (rd.kind != DSC_KERNEL_REDUCE || rd.reduce_op != DSC_REDUCE_SUM || !drafts[ri].fk.virtuals.empty()) continue;
+            const dsc_view rv = rd.inputs[0];
+            if (!reads_in_order(rv)) continue;
+            // [K, N] with the reduced axis first (size-1 axes aside)
+            std::vector<int> big;
+            for (int q = 0; q < rv.out_shape.rank; ++q)
+                if (rv.out_shape.dims[q] > 1) big.push_back(q);
+            if (big.size() != 2 || big[0] != rd.axis) continue;
+            const int64_t K = rv.out_shape.dims[big[0]], N = rv.out_shape.dims[big[1]];
+            if (K * N < (1 << 22) || N % 4 != 0) continue;
+            const int x = drafts[ri].params[0];
+            const int r_out = drafts[ri].outs[0].node;
+            if (drafts[ri].outs[0].copy_from >= 0) continue;
+            // the MatMul that reads x as B = [1, K, N] in order, after the Reduce in the list
+            int mi = -1;
+            for (size_t q = ri + 1; q < drafts.size() && mi < 0; ++q) {
+                const Draft& md = drafts[q];
+                const dsc_kernel_desc& m = md.fk.main.raw();
+                if (m.kind != DSC_KERNEL_MATMUL || !md.fk.virtuals.empty() || md.fk.has_epilogue || md.fk.colsum_out >= 0) continue;
+                if (md.fk.inputs[1].buffer < 0 || md.params[md.fk.inputs[1].buffer] != x) continue;
+                const MatMulDims g = matmul_dims(m);
+                if (g.batch != 1 || g.k != K || g.n != N || !reads_in_order(m.inputs[1])) continue;
+                mi = (int)q;
+            }
+            if (mi < 0) continue;
+            // everything between the two that hangs on the Reduce moves behind the MatMul with it
+            std::set<int> produced{r_out};
+            std::vector<int> moving{(int)ri};
+            bool ok = true;
+            for (int q = (int)ri + 1; q < mi; ++q) {
+                bool dep = false;
+                for (int nd : input_nodes(drafts[q]))
+                    if (produced.count(nd)) dep = true;
+                for (auto& o : drafts[q].outs)
+                    if (o.copy_from >= 0 && produced.count(o.copy_from)) dep = true;
+                if (!dep) continue;
+                for (auto& o : drafts[q].outs) {
+                    produced.insert(o.node);
+                    if (o.copy_from >= 0) ok = false;
+                }
+                moving.push_back(q);
+            }
+            for (int nd : input_nodes(drafts[mi]))
+                if (produced.count(nd)) ok = false;
+            if (!ok) continue;
+            // nothing that stays may write what a moving launch reads later than it does now... the moving launches
+            // only read nodes produced before `ri` or by each other, and nodes are written once: safe to delay them
+            const MatMulDims g = matmul_dims(drafts[mi].fk.main.raw());
+            const int64_t chunks = drafts[mi].fk.sum_chunks ? 1 : g.chunks;
+            Draft trial = drafts[mi];
+            const int partials = n_nodes;
+            trial.fk.colsum_out = param_index(trial, partials, true);
+            trial.fk.outputs.push_back(trial.fk.colsum_out);
+            trial.outs.push_back(StepOutput{partials, -1, false, 0});
+            {
+                Generated probe;
+                if (!generate(trial.fk, &probe).empty()) continue;
+            }
+            // the Reduce over the partials [chunks, N]
+            dsc_view pv{};
+            pv.in_shape.rank = 2;
+            pv.in_shape.dims[0] = chunks;
+            pv.in_shape.dims[1] = N;
+            pv.out_shape = rd.shape;
+            int placed = 0;
+            bool shaped = true;
+            // the Reduce keeps its output shape; its input gets the same rank with `chunks` on the reduced axis
+            if (rd.shape.rank != rv.out_shape.rank) shaped = false;
+            for (int q = 0; q < pv.out_shape.rank && shaped; ++q) {
+                if (q == rd.axis) {
+                    pv.out_shape.dims[q] = chunks;
+                    pv.map_axis[q] = chunks > 1 ? 0 : -1;
+                    pv.map_step[q] = chunks > 1 ? 1 : 0;
+                } else if (pv.out_shape.dims[q] > 1) {
+                    if (pv.out_shape.dims[q] != N || placed++) shaped = false;
+                    pv.map_axis[q] = 1;
+                    pv.map_step[q] = 1;
+                } else {
+                    pv.map_axis[q] = -1;
+                    pv.map_step[q] = 0;
+                }
+            }
+            if (!shaped || placed != 1) continue;
+            dsc_kernel_desc nd = rd;
+            nd.inputs = &pv;
+            if (!validate(nd).empty()) continue;
+            n_nodes++;
+            node_bytes.push_back((size_t)(chunks * N) * 4);
+            is_graph_output.push_back(false);
+            is_graph_input.push_back(false);
+            drafts[mi] = trial;
+            Draft nr;
+            nr.fk = FusedKernel::plain(nd);
+            nr.params = {partials, r_out};
+            nr.outs = drafts[ri].outs;
+            nr.covers = drafts[ri].covers;
+            drafts[ri] = nr;
+            // move: stable order, right behind the MatMul
+            std::vector<Draft> moved;
+            for (int q : moving) moved.push_back(drafts[q]);
+            for (int q = (int)moving.size() - 1; q >= 0; --q) drafts.erase(drafts.begin() + moving[q]);
+            const int at = mi - (int)moving.size() + 1;
+            drafts.insert(drafts.begin() + at, moved.begin(), moved.end());
+            --ri;  // the slot now holds another draft
+        }
+
         // Pass 0a: chains of Reduces over neighbouring axes (the reference sums a bias gradient back to the bias' shape
         // one axis at a time: [m, h, w, c] -> [1, h, w, c] -> [1, w, c] -> [c], three clusters) become one Reduce over
         // the merged axis: fewer launches.  Only small inputs are merged (the tail of such a chain): a large first

@@ -163,6 +163,27 @@ def test_heap_reuse_and_errors(hip_backend_session):
     be.free(h)
 
 
+def test_bias_gradient_rides_on_the_weight_gradient_matmul(hip_backend_session):
+    """A 128x128 grid through two hidden layers of 256: dZ is [16384, 256], large enough for the schedule to take the
+    bias gradients (column sums of dZ) out of the weight-gradient MatMuls that read dZ as their B operand, instead of
+    a Reduce pass of its own.  Three Adam steps against the oracle."""
+    from descent_amd import workloads
+
+    genv, cenv = _envs(hip_backend_session)
+    kw = dict(side=128, variant="relu-pe", hidden=(256, 256), freq_count=4, seed=31)
+    gw = workloads.coordinate_mlp(genv, **kw)
+    cw = workloads.coordinate_mlp(cenv, **kw)
+    for step in range(3):
+        genv.run(gw.graph, step)
+        cenv.run(cw.graph, step)
+    listing = next(iter(gw.graph.__dict__["_schedules"].values())).describe()
+    assert listing.count("+column sums of B") >= 2, listing
+    got, want = gw.snapshot(), cw.snapshot()
+    for key in want:
+        err = rel_l2(got[key], want[key])
+        assert err <= TOL, f"{key}: rel L2 {err}"
+
+
 @pytest.mark.parametrize("variant", ["relu-pe", "siren"])
 def test_coordinate_mlp_steps_vs_oracle(hip_backend_session, variant):
     """Config 4 at reduced size (64x64 grid, two hidden layers of 64): three Adam steps."""
