@@ -948,7 +948,7 @@ string gen_conv_dgrad(Emitter& em, Generated* out) {
     const bool unpad = cv.pad_h > 0 || cv.pad_w > 0;
     if (H < 1 || W < 1 || K % 4 != 0) return "conv dgrad: unsupported geometry";
     const int64_t lds = dgrad_lds_floats(cv, K);
-    if (lds * 4 > 64 * 1024) return "conv dgrad: image tile does not fit LDS";
+    if ((lds + PITCH + 4) * 4 > 64 * 1024) return "conv dgrad: image tile does not fit LDS";
 
     const string la = em.load_view(fk.inputs[0], d.inputs[0], {"cb", "cm", "ck"});
     em.funcs << "DSC_INLINE float load_a(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return " << la << ";\n}\n";
@@ -959,7 +959,10 @@ string gen_conv_dgrad(Emitter& em, Generated* out) {
     const string out_ptr = "b" + to_string(fk.outputs[0]);
     k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
     k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
-    k << "    __shared__ __attribute__((aligned(16))) float lds[" << S(lds) << "];\n";
+    // the last PITCH floats stay zero: a tap outside the output reads them instead of masking every value it loads
+    const int64_t zero_at = (lds + 3) / 4 * 4;
+    k << "    __shared__ __attribute__((aligned(16))) float lds[" << S(zero_at + PITCH) << "];\n";
+    k << "    if (threadIdx.x < " << S(PITCH) << ") lds[" << S(zero_at) << " + threadIdx.x] = 0.f;\n";
     k << "    const int cb = blockIdx.x % " << S(G) << ", img = blockIdx.x / " << S(G) << ";\n";
     // 1. dC of this image and group: tile[oy][ox][oc].  (No halo: the taps that fall outside the output are
     // predicated below, which keeps the tile small enough for every workgroup of a ConvNet-sized launch to be
@@ -990,13 +993,12 @@ string gen_conv_dgrad(Emitter& em, Generated* out) {
     k << "            const int fy = tap / " << S(FW) << ", fx = tap % " << S(FW) << ";\n";
     k << "            const int oy = py - fy, ox = px - fx;\n";
     k << "            const bool inside = oy >= 0 && oy < " << S(OH) << " && ox >= 0 && ox < " << S(OW) << ";\n";
-    k << "            const float* src = &lds[(clampi(oy, 0, " << S(OH - 1) << ") * " << S(OW) << " + clampi(ox, 0, " << S(OW - 1) << ")) * "
-      << S(PITCH) << "];\n";
+    k << "            const float* src = &lds[inside ? (oy * " << S(OW) << " + ox) * " << S(PITCH) << " : " << S(zero_at) << "];\n";
     k << "#pragma unroll\n            for (int oc = 0; oc < " << S(K) << "; oc += " << OCB << ") {\n";
     k << "                float a[" << OCB << "];\n";
     k << "#pragma unroll\n                for (int q = 0; q < " << OCB << "; q += 4) {\n";
     k << "                    const float4 a4 = *(const float4*)(src + oc + q);\n";
-    k << "                    a[q] = inside ? a4.x : 0.f; a[q + 1] = inside ? a4.y : 0.f; a[q + 2] = inside ? a4.z : 0.f; a[q + 3] = inside ? a4.w : 0.f;\n                }\n";
+    k << "                    a[q] = a4.x; a[q + 1] = a4.y; a[q + 2] = a4.z; a[q + 3] = a4.w;\n                }\n";
     k << "#pragma unroll\n                for (int j = 0; j < " << OCB << "; ++j)\n";
     k << "#pragma unroll\n                    for (int c = 0; c < " << S(C) << "; ++c)\n";
     k << "                        acc[ps][c] = fmaf(a[j], load_b(cb, oc + j, tap * " << S(C) << " + c, " << em.params_pass() << "), acc[ps][c]);\n";
@@ -1709,7 +1711,7 @@ string generate_scatter_chain(const FusedKernel& fk, Generated* out);
 
 bool conv_dgrad_fits(const FusedKernel::ConvDgrad& c, int64_t k) {
     if (k % 4 != 0 || c.g * c.c > 64 || c.fh * c.fw * k * c.g * c.c > 8192) return false;
-    return dgrad_lds_floats(c, k) * 4 <= 64 * 1024 && c.oh + c.fh - 1 > 2 * c.pad_h && c.ow + c.fw - 1 > 2 * c.pad_w;
+    return (dgrad_lds_floats(c, k) + dgrad_pitch(k) + 4) * 4 <= 64 * 1024 && c.oh + c.fh - 1 > 2 * c.pad_h && c.ow + c.fw - 1 > 2 * c.pad_w;
 }
 
 bool can_be_part(const FusedKernel& fk) {
