@@ -385,6 +385,17 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             }
             for (int nd : input_nodes(drafts[mi]))
                 if (produced.count(nd)) ok = false;
+            {
+                // a launch that stays put must not take over, in place, a buffer that a delayed launch still reads
+                std::set<int> read_by_moving;
+                for (int q : moving)
+                    for (int nd : input_nodes(drafts[q])) read_by_moving.insert(nd);
+                for (int q = (int)ri + 1; q <= mi; ++q) {
+                    if (std::find(moving.begin(), moving.end(), q) != moving.end()) continue;
+                    for (auto& o : drafts[q].outs)
+                        if (o.copy_from >= 0 && read_by_moving.count(o.copy_from)) ok = false;
+                }
+            }
             if (!ok) continue;
             // nothing that stays may write what a moving launch reads later than it does now... the moving launches
             // only read nodes produced before `ri` or by each other, and nodes are written once: safe to delay them
