@@ -1361,6 +1361,11 @@ string gen_matmul_tallk(Emitter& em, Generated* out) {
     k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
     k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
     k << "    __shared__ float red[4][" << MT * NT * 256 << "];\n";
+    const bool colsum = fk.colsum_out >= 0;
+    if (colsum) {
+        k << "    __shared__ float cs_red[4][" << NT * 16 << "];\n";
+        k << "    float cs[" << NT << "];\n#pragma unroll\n    for (int nt = 0; nt < " << NT << "; ++nt) cs[nt] = 0.f;\n";
+    }
     k << "    const int chunk = blockIdx.x % " << S(g.chunks) << ", cb = blockIdx.x / " << S(g.chunks) << ";\n";
     k << "    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;\n";
     k << "    const int li = lane & 15, lk = lane >> 4;\n";
@@ -1389,13 +1394,27 @@ string gen_matmul_tallk(Emitter& em, Generated* out) {
     k << "#pragma unroll\n            for (int nt = 0; nt < " << NT << "; ++nt) fb[u][nt] = (k_ok && nt * 16 + li < " << S(g.n)
       << ") ? fb[u][nt] : 0.f;\n";
     k << "        }\n";
+    // column sums of B (a bias gradient riding on the weight gradient): the B fragments are summed per lane here,
+    // over the lane groups and waves after the loop
+    if (colsum)
+        k << "#pragma unroll\n        for (int u = 0; u < " << U << "; ++u)\n#pragma unroll\n            for (int nt = 0; nt < " << NT
+          << "; ++nt) cs[nt] += fb[u][nt];\n";
     k << "#pragma unroll\n        for (int u = 0; u < " << U << "; ++u)\n#pragma unroll\n            for (int mt = 0; mt < " << MT
       << "; ++mt)\n#pragma unroll\n                for (int nt = 0; nt < " << NT << "; ++nt)\n"
       << "                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[u][mt], fb[u][nt], acc[mt][nt], 0, 0, 0);\n";
     k << "    }\n";
     k << "#pragma unroll\n    for (int mt = 0; mt < " << MT << "; ++mt)\n#pragma unroll\n        for (int nt = 0; nt < " << NT
       << "; ++nt)\n#pragma unroll\n            for (int r = 0; r < 4; ++r) red[wave][(mt * " << NT << " + nt) * 256 + r * 64 + lane] = acc[mt][nt][r];\n";
+    if (colsum) {
+        k << "#pragma unroll\n    for (int nt = 0; nt < " << NT << "; ++nt) {\n";
+        k << "        float t = cs[nt];\n        t += __shfl_xor(t, 16, 64);\n        t += __shfl_xor(t, 32, 64);\n";
+        k << "        if (lk == 0) cs_red[wave][nt * 16 + li] = t;\n    }\n";
+    }
     k << "    __syncthreads();\n";
+    if (colsum) {
+        k << "    if (threadIdx.x < " << NT * 16 << " && threadIdx.x < " << S(g.n) << ")\n";
+        k << "        b" << fk.colsum_out << "[(chunk * " << S(g.batch) << " + cb) * " << S(g.n) << " + threadIdx.x] = (cs_red[0][threadIdx.x] + cs_red[1][threadIdx.x]) + (cs_red[2][threadIdx.x] + cs_red[3][threadIdx.x]);\n";
+    }
     // accumulator register r of lane l is D[4 * (l / 16) + r][l % 16]
     k << "    for (int i = threadIdx.x; i < " << MT * NT * 256 << "; i += 256) {\n";
     k << "        const float sum = (red[0][i] + red[1][i]) + (red[2][i] + red[3][i]);\n";
@@ -1410,8 +1429,8 @@ string gen_matmul_tallk(Emitter& em, Generated* out) {
     out->block = 256;
     out->source = k.str();
     char note[160];
-    std::snprintf(note, sizeof note, "tall-k mfma 16x16x4, %dx%d tiles, operands from memory, %d steps in flight, chunks %lld", MT, NT, U,
-                  (long long)g.chunks);
+    std::snprintf(note, sizeof note, "tall-k mfma 16x16x4, %dx%d tiles, operands from memory, %d steps in flight, chunks %lld%s", MT, NT, U,
+                  (long long)g.chunks, colsum ? " +column sums of B" : "");
     out->note = note;
     return "";
 }
@@ -1452,8 +1471,8 @@ string gen_matmul(Emitter& em, Generated* out) {
     const dsc_view& va = d.inputs[0];
     const dsc_view& vb = d.inputs[1];
     const bool rows = d.output_mode == DSC_MATMUL_ROWS;
-    if (fk.colsum_out >= 0 && (rows_kernel_applies(fk, g) || smallk_kernel_applies(fk, g) || tallk_kernel_applies(fk, g)))
-        return "matmul: column sums need the MFMA template";
+    if (fk.colsum_out >= 0 && (rows_kernel_applies(fk, g) || smallk_kernel_applies(fk, g)))
+        return "matmul: column sums need the MFMA template or the tall-k kernel";
     if (rows_kernel_applies(fk, g)) return gen_matmul_rows(em, out);
     if (smallk_kernel_applies(fk, g)) return gen_matmul_smallk(em, out);
     if (tallk_kernel_applies(fk, g)) return gen_matmul_tallk(em, out);

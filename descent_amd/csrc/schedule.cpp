@@ -94,6 +94,7 @@ void compact(Draft& d) {
     }
     for_each_source(d.fk, [&](Source& s) { if (s.buffer >= 0) s.buffer = remap[s.buffer]; });
     for (int& o : d.fk.outputs) o = remap[o];
+    if (d.fk.colsum_out >= 0) d.fk.colsum_out = remap[d.fk.colsum_out];
     d.params = params;
     d.fk.buffer_is_output = is_out;
     d.fk.n_buffers = (int)params.size();
@@ -335,13 +336,119 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             drafts[i].keep_split = true;
         }
 
+        // One step of merging a chain of Reduces over neighbouring axes (pass 0a below says when): the Reduce in draft
+        // `i` and the Reduce that alone consumes it become one Reduce over the merged axis, in draft `i`.
+        auto merge_reduce_step = [&](size_t i, bool small_only) -> bool {
+            const dsc_kernel_desc r1 = drafts[i].fk.main.raw();
+            if (r1.kind != DSC_KERNEL_REDUCE || !drafts[i].fk.virtuals.empty() || drafts[i].fk.has_epilogue) return false;
+            if (small_only && element_count(r1.inputs[0].out_shape) > (1 << 18)) return false;
+            {
+                // a short Reduce along the rows of a matrix is left to the row fusion (pass 1b)
+                const dsc_shape& os = r1.inputs[0].out_shape;
+                bool innermost = true;
+                for (int q = r1.axis + 1; q < os.rank; ++q)
+                    if (os.dims[q] > 1) innermost = false;
+                if (innermost && os.dims[r1.axis] <= 64) return false;
+            }
+            const int mid = drafts[i].outs[0].node;
+            if (is_graph_output[mid] || drafts[i].outs[0].copy_from >= 0) return false;
+            int j = -1, uses = 0;
+            for (size_t q = 0; q < drafts.size(); ++q) {
+                if (q == i) continue;
+                for (int nd : input_nodes(drafts[q]))
+                    if (nd == mid) { ++uses; j = (int)q; }
+                for (auto& o : drafts[q].outs)
+                    if (o.copy_from == mid) uses += 2;
+            }
+            if (uses != 1 || j < (int)i) return false;
+            const dsc_kernel_desc r2 = drafts[j].fk.main.raw();
+            if (r2.kind != DSC_KERNEL_REDUCE || r2.reduce_op != r1.reduce_op || !drafts[j].fk.virtuals.empty() ||
+                drafts[j].fk.has_epilogue || !reads_in_order(r2.inputs[0]))
+                return false;
+            const dsc_view v = r1.inputs[0];
+            const int a = r1.axis;
+            // the second Reduce's axis, as an axis of the first one's output
+            std::vector<int> kept1, kept2;
+            for (int q = 0; q < v.out_shape.rank; ++q)
+                if (q != a && v.out_shape.dims[q] > 1) kept1.push_back(q);
+            for (int q = 0; q < r2.inputs[0].out_shape.rank; ++q)
+                if (r2.inputs[0].out_shape.dims[q] > 1) kept2.push_back(q);
+            if (kept1.size() != kept2.size()) return false;
+            int b = -1;
+            bool same = true;
+            for (size_t q = 0; q < kept1.size(); ++q) {
+                if (v.out_shape.dims[kept1[q]] != r2.inputs[0].out_shape.dims[kept2[q]]) same = false;
+                if (kept2[q] == r2.axis) b = kept1[q];
+            }
+            if (!same || b < 0) return false;
+            bool neighbours = true;
+            for (int q = std::min(a, b) + 1; q < std::max(a, b); ++q)
+                if (v.out_shape.dims[q] > 1) neighbours = false;
+            const int ia = v.map_axis[a], ib = v.map_axis[b];
+            if (!neighbours || ia < 0 || ib < 0 || ia == ib || (a < b) != (ia < ib)) return false;
+            auto whole = [&](int out_axis, int in_axis) {
+                return v.map_step[out_axis] == 1 && v.in_offset[in_axis] == 0 && v.out_shape.dims[out_axis] == v.in_shape.dims[in_axis];
+            };
+            if (!whole(a, ia) || !whole(b, ib)) return false;
+            for (int q = std::min(ia, ib) + 1; q < std::max(ia, ib); ++q)
+                if (v.in_shape.dims[q] > 1) neighbours = false;
+            // no other output axis may walk the two input axes
+            for (int q = 0; q < v.out_shape.rank; ++q)
+                if (q != a && q != b && (v.map_axis[q] == ia || v.map_axis[q] == ib)) neighbours = false;
+            if (!neighbours) return false;
+            const int64_t merged = v.out_shape.dims[a] * v.out_shape.dims[b];
+            const int lo_in = std::min(ia, ib), hi_in = std::max(ia, ib);
+            const int lo_out = ia < ib ? a : b, hi_out = ia < ib ? b : a;
+            dsc_view m = v;
+            m.in_shape.dims[lo_in] = merged;
+            m.in_shape.dims[hi_in] = 1;
+            m.out_shape.dims[lo_out] = merged;
+            m.out_shape.dims[hi_out] = 1;
+            m.map_axis[hi_out] = -1;
+            m.map_step[hi_out] = 0;
+            dsc_kernel_desc d = r1;
+            d.inputs = &m;
+            d.axis = lo_out;
+            d.shape = m.out_shape;
+            d.shape.dims[lo_out] = 1;
+            if (!validate(d).empty() || element_count(d.shape) != element_count(r2.shape)) return false;
+            Draft mergedDraft;
+            mergedDraft.fk = FusedKernel::plain(d);
+            mergedDraft.params = {drafts[i].params[0], drafts[j].outs[0].node};
+            mergedDraft.outs.push_back(drafts[j].outs[0]);
+            mergedDraft.covers = drafts[i].covers;
+            mergedDraft.covers.insert(mergedDraft.covers.end(), drafts[j].covers.begin(), drafts[j].covers.end());
+            drafts[i] = mergedDraft;
+            drafts.erase(drafts.begin() + j);
+            return true;
+        };
+
         // Pass 0c: a bias gradient is the sum of dZ [K, N] over its rows, and the weight gradient A^T dZ of the same
         // layer reads dZ as its B operand, k chunk by k chunk.  The MFMA kernel then also writes the column sums of
         // the B tiles it loads, one row of partials per chunk, and the Reduce shrinks from K rows to `chunks` rows: one
         // pass over dZ instead of two.  Only large dZ (the Reduce is a launch of its own there).
         for (size_t ri = 0; ri < drafts.size(); ++ri) {
+            if (drafts[ri].fk.main.raw().kind != DSC_KERNEL_REDUCE || drafts[ri].fk.main.raw().reduce_op != DSC_REDUCE_SUM ||
+                !drafts[ri].fk.virtuals.empty())
+                continue;
+            // a sum taken axis by axis ([m, h, w, c] -> [h, w, c] -> [w, c] -> [c]) is looked at as one Reduce; the
+            // chain stays as it was when no MatMul takes it
+            const std::vector<Draft> before = drafts;
+            const int nodes_before = n_nodes;
+            bool merged_chain = false;
+            while (merge_reduce_step(ri, false)) merged_chain = true;
+            bool taken = false;
+            struct Restore {
+                std::vector<Draft>& drafts;
+                const std::vector<Draft>& before;
+                const bool& taken;
+                const bool& merged;
+                ~Restore() {
+                    if (!taken && merged) drafts = before;
+                }
+            } restore{drafts, before, taken, merged_chain};
+            (void)nodes_before;
             const dsc_kernel_desc rd = drafts[ri].fk.main.raw();
-            if (rd.kind != DSC_KERNEL_REDUCE || rd.reduce_op != DSC_REDUCE_SUM || !drafts[ri].fk.virtuals.empty()) continue;
             const dsc_view rv = rd.inputs[0];
             if (!reads_in_order(rv)) continue;
             // [K, N] with the reduced axis first (size-1 axes aside)
@@ -362,7 +469,13 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                 if (m.kind != DSC_KERNEL_MATMUL || !md.fk.virtuals.empty() || md.fk.has_epilogue || md.fk.colsum_out >= 0) continue;
                 if (md.fk.inputs[1].buffer < 0 || md.params[md.fk.inputs[1].buffer] != x) continue;
                 const MatMulDims g = matmul_dims(m);
-                if (g.batch != 1 || g.k != K || g.n != N || !reads_in_order(m.inputs[1])) continue;
+                // B[b][k][n] = x[k][b * n_per_batch + n]: with one batch x read in order, with several (the groups of
+                // a convolution) each batch takes its own run of columns
+                int64_t base = 0, coef[DSC_MAX_DIM];
+                if (g.k != K || g.batch * g.n != N || g.n % 4 != 0 || !affine_form(m.inputs[1], &base, coef) || base != 0 ||
+                    element_count(m.inputs[1].in_shape) != K * N || m.inputs[1].out_shape.rank != 3)
+                    continue;
+                if ((g.batch > 1 && coef[0] != g.n) || coef[1] != N || coef[2] != 1) continue;
                 mi = (int)q;
             }
             if (mi < 0) continue;
@@ -438,6 +551,7 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             dsc_kernel_desc nd = rd;
             nd.inputs = &pv;
             if (!validate(nd).empty()) continue;
+            taken = true;
             n_nodes++;
             node_bytes.push_back((size_t)(chunks * N) * 4);
             is_graph_output.push_back(false);
@@ -464,91 +578,9 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
         // Reduce streams its input with every lane on consecutive outputs, which a merged axis over short rows would
         // give up (measured on the ConvNet's conv bias gradients: merged 3666 steps/s, tail only 3950+).  Sums are
         // re-associated (as in every split reduction); max is order-free.
-        for (size_t i = 0; i < drafts.size(); ++i) {
-            for (;;) {
-                const dsc_kernel_desc r1 = drafts[i].fk.main.raw();
-                if (r1.kind != DSC_KERNEL_REDUCE || !drafts[i].fk.virtuals.empty() || drafts[i].fk.has_epilogue) break;
-                if (element_count(r1.inputs[0].out_shape) > (1 << 18)) break;
-                {
-                    // a short Reduce along the rows of a matrix is left to the row fusion (pass 1b)
-                    const dsc_shape& os = r1.inputs[0].out_shape;
-                    bool innermost = true;
-                    for (int q = r1.axis + 1; q < os.rank; ++q)
-                        if (os.dims[q] > 1) innermost = false;
-                    if (innermost && os.dims[r1.axis] <= 64) break;
-                }
-                const int mid = drafts[i].outs[0].node;
-                if (is_graph_output[mid] || drafts[i].outs[0].copy_from >= 0) break;
-                int j = -1, uses = 0;
-                for (size_t q = 0; q < drafts.size(); ++q) {
-                    if (q == i) continue;
-                    for (int nd : input_nodes(drafts[q]))
-                        if (nd == mid) { ++uses; j = (int)q; }
-                    for (auto& o : drafts[q].outs)
-                        if (o.copy_from == mid) uses += 2;
-                }
-                if (uses != 1 || j < (int)i) break;
-                const dsc_kernel_desc r2 = drafts[j].fk.main.raw();
-                if (r2.kind != DSC_KERNEL_REDUCE || r2.reduce_op != r1.reduce_op || !drafts[j].fk.virtuals.empty() ||
-                    drafts[j].fk.has_epilogue || !reads_in_order(r2.inputs[0]))
-                    break;
-                const dsc_view v = r1.inputs[0];
-                const int a = r1.axis;
-                // the second Reduce's axis, as an axis of the first one's output
-                std::vector<int> kept1, kept2;
-                for (int q = 0; q < v.out_shape.rank; ++q)
-                    if (q != a && v.out_shape.dims[q] > 1) kept1.push_back(q);
-                for (int q = 0; q < r2.inputs[0].out_shape.rank; ++q)
-                    if (r2.inputs[0].out_shape.dims[q] > 1) kept2.push_back(q);
-                if (kept1.size() != kept2.size()) break;
-                int b = -1;
-                bool same = true;
-                for (size_t q = 0; q < kept1.size(); ++q) {
-                    if (v.out_shape.dims[kept1[q]] != r2.inputs[0].out_shape.dims[kept2[q]]) same = false;
-                    if (kept2[q] == r2.axis) b = kept1[q];
-                }
-                if (!same || b < 0) break;
-                bool neighbours = true;
-                for (int q = std::min(a, b) + 1; q < std::max(a, b); ++q)
-                    if (v.out_shape.dims[q] > 1) neighbours = false;
-                const int ia = v.map_axis[a], ib = v.map_axis[b];
-                if (!neighbours || ia < 0 || ib < 0 || ia == ib || (a < b) != (ia < ib)) break;
-                auto whole = [&](int out_axis, int in_axis) {
-                    return v.map_step[out_axis] == 1 && v.in_offset[in_axis] == 0 && v.out_shape.dims[out_axis] == v.in_shape.dims[in_axis];
-                };
-                if (!whole(a, ia) || !whole(b, ib)) break;
-                for (int q = std::min(ia, ib) + 1; q < std::max(ia, ib); ++q)
-                    if (v.in_shape.dims[q] > 1) neighbours = false;
-                // no other output axis may walk the two input axes
-                for (int q = 0; q < v.out_shape.rank; ++q)
-                    if (q != a && q != b && (v.map_axis[q] == ia || v.map_axis[q] == ib)) neighbours = false;
-                if (!neighbours) break;
-                const int64_t merged = v.out_shape.dims[a] * v.out_shape.dims[b];
-                const int lo_in = std::min(ia, ib), hi_in = std::max(ia, ib);
-                const int lo_out = ia < ib ? a : b, hi_out = ia < ib ? b : a;
-                dsc_view m = v;
-                m.in_shape.dims[lo_in] = merged;
-                m.in_shape.dims[hi_in] = 1;
-                m.out_shape.dims[lo_out] = merged;
-                m.out_shape.dims[hi_out] = 1;
-                m.map_axis[hi_out] = -1;
-                m.map_step[hi_out] = 0;
-                dsc_kernel_desc d = r1;
-                d.inputs = &m;
-                d.axis = lo_out;
-                d.shape = m.out_shape;
-                d.shape.dims[lo_out] = 1;
-                if (!validate(d).empty() || element_count(d.shape) != element_count(r2.shape)) break;
-                Draft mergedDraft;
-                mergedDraft.fk = FusedKernel::plain(d);
-                mergedDraft.params = {drafts[i].params[0], drafts[j].outs[0].node};
-                mergedDraft.outs.push_back(drafts[j].outs[0]);
-                mergedDraft.covers = drafts[i].covers;
-                mergedDraft.covers.insert(mergedDraft.covers.end(), drafts[j].covers.begin(), drafts[j].covers.end());
-                drafts[i] = mergedDraft;
-                drafts.erase(drafts.begin() + j);
+        for (size_t i = 0; i < drafts.size(); ++i)
+            while (merge_reduce_step(i, true)) {
             }
-        }
 
         // Pass 0b: a Reduce with few outputs and a long axis cannot fill the machine with one thread (or one
         // thread row) per output.  Split the axis k = s * (k/s): a first Reduce over k/s produces s partial rows
@@ -1154,6 +1186,9 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                     if (taken_in_place_between(i, ci, input_nodes(p))) ok = false;
                     if ((int)q.fk.virtuals.size() + (int)p.fk.virtuals.size() + 1 > 8) ok = false;
                     if (!q.fk.row_stages.empty()) ok = false;
+                    // a MatMul that sums its B operand's columns on the side took over the operand's other reader: the
+                    // operand stays a buffer, as it was when two launches read it
+                    if (q.fk.colsum_out >= 0 && q.fk.inputs[1].buffer >= 0 && q.params[q.fk.inputs[1].buffer] == node) ok = false;
                     // an epilogue reads its product from the accumulator, never through a producer
                     if (q.fk.has_epilogue && q.fk.epilogue_product_input >= 0) {
                         const Source& ps = q.fk.epilogue_inputs[q.fk.epilogue_product_input];
