@@ -30,6 +30,35 @@ def test_library_exports_every_declared_entry_point():
     assert declared == set(hip_backend.EXPORTED_SYMBOLS)
 
 
+def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):
+    """The boundary is a C ABI: the header compiles as C99 with no C++ in it, and a C program that includes it links
+    against the library and gets DSC_ERR_NO_DEVICE (here) or a context (on a GPU box) from dsc_ctx_create."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if not gcc:
+        pytest.skip("no gcc")
+    header_dir = os.path.join(ROOT, "include")
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-x", "c",
+                    os.path.join(header_dir, "descent_hip.h")], check=True)
+    src = tmp_path / "probe.c"
+    src.write_text(
+        '#include "descent_hip.h"\n#include <stdio.h>\n'
+        "int main(void) {\n"
+        "    dsc_ctx* ctx = 0;\n"
+        "    int rc = dsc_ctx_create(0, &ctx);\n"
+        '    printf("%d %s\\n", rc, rc ? dsc_last_error() : "ok");\n'
+        "    if (rc == 0) dsc_ctx_destroy(ctx);\n"
+        "    return 0;\n}\n")
+    exe = tmp_path / "probe"
+    lib_dir = os.path.dirname(hip_backend.LIB_PATH)
+    subprocess.run([gcc, "-std=c99", "-I", header_dir, str(src), "-o", str(exe), "-L", lib_dir, "-ldescent_hip",
+                    "-Wl,-rpath," + lib_dir, "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split(None, 1)
+    assert int(out[0]) in (0, _abi.ERR_NO_DEVICE), out
+
+
 def test_no_device_is_an_error_not_a_fallback():
     """This container has no GPU: creating a context must fail with DSC_ERR_NO_DEVICE."""
     lib = hip_backend.lib()
