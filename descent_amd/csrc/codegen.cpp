@@ -1233,6 +1233,51 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
           << ", " << em.params_pass() << ");\n";
         k << "    __syncthreads();\n";
     }
+    const int Q = (int)(g.n / 4);  // 16-byte pieces per row
+    const bool transposed_store = vec_store && (Q == 1 || Q == 2 || Q == 4 || Q == 8) && !std::getenv("DSC_ROWS_DIRECT_STORE");
+    // With at most 16 columns and a k of some length the products go through v_mfma_f32_16x16x4f32 instead of
+    // scalar-operand FMAs (twice the fp32 rate with packed math off): a wave takes its 64 rows as four 16-row tiles,
+    // lane l feeds A[row l % 16][k = 4 s + l / 16] straight from memory (the same generated load, so an im2col view
+    // costs what it costs the FMA path) and keeps B's K/4 fragments in registers; the results land in the LDS
+    // staging buffer of the store below in row order.
+    bool use_mfma = transposed_store && g.n <= 16 && g.k >= 16 && g.k % 4 == 0 && R == 1 && !b_in_lds;
+    if (const char* e = std::getenv("DSC_ROWS_MFMA"))
+        if (e[0] == '0') use_mfma = false;
+    if (use_mfma) {
+        // k is taken in blocks of four consecutive values (one 16-byte piece of an im2col row: four channels of one
+        // tap), block q * J + j going to lane group q = l / 16: a lane then computes one address per block, not per
+        // k, and feeds the four values to four MFMA steps.  A and B use the same order of k, so the sum is the same.
+        const int64_t blocks = g.k / 4;
+        const int64_t J = (blocks + 3) / 4;
+        k << "    typedef float rm_float4 __attribute__((ext_vector_type(4)));\n";
+        k << "    const int lane = threadIdx.x & 63, li = lane & 15, lk = lane >> 4;\n";
+        k << "    const int wave_row0 = row0 - lane;\n";
+        k << "    float fb[" << S(J) << "][4];\n";
+        k << "#pragma unroll\n    for (int j = 0; j < " << S(J) << "; ++j) {\n";
+        k << "        const int blk = lk * " << S(J) << " + j;\n";
+        k << "#pragma unroll\n        for (int i = 0; i < 4; ++i) {\n";
+        k << "            const float v = load_b(cb, min(4 * blk + i, " << S(g.k - 1) << "), min(li, " << S(g.n - 1) << "), " << em.params_pass() << ");\n";
+        k << "            fb[j][i] = (blk < " << S(blocks) << " && li < " << S(g.n) << ") ? v : 0.f;\n        }\n    }\n";
+        k << "    int cmt[4];\n#pragma unroll\n    for (int t = 0; t < 4; ++t) cmt[t] = min(wave_row0 + t * 16 + li, " << S(g.m - 1) << ");\n";
+        k << "    rm_float4 acc4[4];\n#pragma unroll\n    for (int t = 0; t < 4; ++t) acc4[t] = (rm_float4){0.f, 0.f, 0.f, 0.f};\n";
+        // the A loads of JG blocks are issued before their MFMAs.  Measured on the ConvNet's second convolution
+        // (392000 rows, k = 72): JG 1 / 2 / 3 / 5 = 24.9 / 23.6 / 23.8 / 27.4 us against 25.4 for the FMA path -- the
+        // kernel is bound by the 64 cache lines that every 16-byte load instruction of an im2col row block touches,
+        // not by either arithmetic pipe.
+        const int64_t JG = std::getenv("DSC_ROWS_MFMA_JG") ? std::max<int64_t>(1, std::atoll(std::getenv("DSC_ROWS_MFMA_JG"))) : std::min<int64_t>(2, J);
+        k << "#pragma unroll\n    for (int j0 = 0; j0 < " << S(J) << "; j0 += " << S(JG) << ") {\n";
+        k << "        float fa[" << S(JG) << "][4][4];\n";
+        k << "#pragma unroll\n        for (int jj = 0; jj < " << S(JG) << "; ++jj) {\n";
+        k << "            const int blk = min(lk * " << S(J) << " + min(j0 + jj, " << S(J - 1) << "), " << S(blocks - 1) << ");\n";
+        k << "#pragma unroll\n            for (int t = 0; t < 4; ++t)\n#pragma unroll\n                for (int i = 0; i < 4; ++i) fa[jj][t][i] = load_a(cb, cmt[t], 4 * blk + i, "
+          << em.params_pass() << ");\n        }\n";
+        k << "        __builtin_amdgcn_sched_barrier(0);\n";
+        // B is zero for the blocks past the end, so whatever A repeats there adds nothing
+        k << "#pragma unroll\n        for (int jj = 0; jj < " << S(JG) << "; ++jj)\n            if (j0 + jj < " << S(J) << ")\n";
+        k << "#pragma unroll\n                for (int i = 0; i < 4; ++i)\n#pragma unroll\n                    for (int t = 0; t < 4; ++t)\n";
+        k << "                        acc4[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[jj][t][i], fb[j0 + jj][i], acc4[t], 0, 0, 0);\n";
+        k << "    }\n";
+    } else {
     // rows past the end repeat the last row's loads (no divergent loads) and skip the store
     k << "    int cml[" << R << "];\n";
     k << "#pragma unroll\n    for (int r = 0; r < " << R << "; ++r) cml[r] = min(row0 + r * 256, " << S(g.m - 1) << ");\n";
@@ -1249,8 +1294,7 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
         k << "            const float bv = load_b(cb, ck, n, " << em.params_pass() << ");\n";
     k << "#pragma unroll\n            for (int r = 0; r < " << R << "; ++r) acc[r][n] = fmaf(a[r], bv, acc[r][n]);\n        }\n";
     k << "    }\n";
-    const int Q = (int)(g.n / 4);  // 16-byte pieces per row
-    const bool transposed_store = vec_store && (Q == 1 || Q == 2 || Q == 4 || Q == 8) && !std::getenv("DSC_ROWS_DIRECT_STORE");
+    }
     if (transposed_store) {
         // A thread holds one whole row, so storing it directly makes every lane of a store instruction write 16
         // bytes of a different row (N*4 bytes apart).  Instead each wave passes its 64 rows through LDS and reads
@@ -1258,12 +1302,18 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
         // consecutive memory, and the epilogue's own loads are consecutive too.
         const int pitch = (int)g.n + 4;
         k << "    __shared__ __attribute__((aligned(16))) float tr[4][" << 64 * pitch << "];\n";
-        k << "    float* my = tr[threadIdx.x >> 6];\n    const int lane = threadIdx.x & 63;\n";
-        k << "    const int wave_row0 = row0 - lane;\n";
+        k << "    float* my = tr[threadIdx.x >> 6];\n";
+        if (!use_mfma) k << "    const int lane = threadIdx.x & 63;\n    const int wave_row0 = row0 - lane;\n";
         k << "#pragma unroll\n    for (int r = 0; r < " << R << "; ++r) {\n";
         if (R > 1) k << "        __syncthreads();\n";
+        if (use_mfma) {
+            // accumulator register i of lane l is D[4 * (l / 16) + i][l % 16] of its tile
+            k << "#pragma unroll\n        for (int t = 0; t < 4; ++t)\n#pragma unroll\n            for (int i = 0; i < 4; ++i)\n";
+            k << "                if (li < " << S(g.n) << ") my[(t * 16 + 4 * lk + i) * " << pitch << " + li] = acc4[t][i];\n";
+        } else {
         k << "#pragma unroll\n        for (int n = 0; n < " << S(g.n) << "; n += 4) *(float4*)&my[lane * " << pitch
           << " + n] = make_float4(acc[r][n], acc[r][n + 1], acc[r][n + 2], acc[r][n + 3]);\n";
+        }
         k << "        __syncthreads();\n";
         k << "#pragma unroll\n        for (int s = 0; s < " << Q << "; ++s) {\n";
         k << "            const int rl = s * " << 64 / Q << " + lane / " << Q << ", q = lane % " << Q << ";\n";
@@ -1312,7 +1362,9 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
     out->grid = (unsigned)(blocks_per_batch * g.batch);
     out->block = 256;
     out->source = k.str();
-    out->note = string("row-per-thread fma, B ") + (b_in_lds ? "in LDS" : "in SGPRs") + (fk.has_epilogue ? " +epilogue" : "");
+    out->note = (use_mfma ? string("row-per-thread store, mfma 16x16x4 from memory, B in registers")
+                          : string("row-per-thread fma, B ") + (b_in_lds ? "in LDS" : "in SGPRs")) +
+                (fk.has_epilogue ? " +epilogue" : "");
     return "";
 }
 
@@ -1717,7 +1769,7 @@ std::string FusedKernel::key() const {
     s.append(reinterpret_cast<const char*>(&n_buffers), 4);
     if (const char* env = std::getenv("DSC_MM_TILE"))
         if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|T") + env;
-    for (const char* name : {"DSC_MM_SMALLK", "DSC_MM_VEC_STORE", "DSC_MM_PERSISTENT", "DSC_MM_DEEP_K", "DSC_MM_PART", "DSC_MM_ROWS", "DSC_ROWS_R", "DSC_ROWS_UNROLL", "DSC_ROWS_B", "DSC_ROWS_DIRECT_STORE", "DSC_MM_TALLK", "DSC_TALLK_UNROLL"})
+    for (const char* name : {"DSC_MM_SMALLK", "DSC_MM_VEC_STORE", "DSC_MM_PERSISTENT", "DSC_MM_DEEP_K", "DSC_MM_PART", "DSC_MM_ROWS", "DSC_ROWS_MFMA", "DSC_ROWS_MFMA_JG", "DSC_ROWS_R", "DSC_ROWS_UNROLL", "DSC_ROWS_B", "DSC_ROWS_DIRECT_STORE", "DSC_MM_TALLK", "DSC_TALLK_UNROLL"})
         if (const char* env = std::getenv(name))
             if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|") + name + env;
     return s;

@@ -305,7 +305,7 @@ def test_convnet_step_at_batch_64_vs_oracle(hip_backend_session, fused):
     if fused is True:
         assert "ConvDataGrad" in listing and "3x3 taps x 16 channels, border folds fused" in listing, listing
     else:
-        assert "MatMul (k=144) [1, 16384, 2, 8]" in listing and "row-per-thread fma" in listing, listing
+        assert "MatMul (k=144) [1, 16384, 2, 8]" in listing and "row-per-thread" in listing, listing
     got, want = gw.snapshot(), cw.snapshot()
     for key in want:
         if key == "accuracy":
