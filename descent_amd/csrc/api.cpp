@@ -149,6 +149,20 @@ uint64_t record_fence(Context* c, hipStream_t stream, bool on_copy_stream) {
     }
     const uint64_t id = c->fence_next++;
     c->fences[id] = Context::Fence{ev, on_copy_stream};
+    // a caller that never waits for its fences (fire-and-forget uploads) must not pile up events: past a thousand
+    // known fences the finished ones among the oldest are retired (an id that is no longer known counts as finished)
+    if (c->fences.size() > 1024) {
+        int looked = 0;
+        for (auto it = c->fences.begin(); it != c->fences.end() && looked < 64 && it->first != id; ++looked) {
+            if (hipEventQuery(it->second.event) == hipSuccess) {
+                c->fence_pool.push_back(it->second.event);
+                it = c->fences.erase(it);
+            } else {
+                (void)hipGetLastError();
+                ++it;
+            }
+        }
+    }
     return id;
 }
 

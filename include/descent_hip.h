@@ -187,8 +187,10 @@ int dsc_ctx_sync(dsc_ctx* ctx);
  * (device/command_buffer.rs:64-123): dsc_fence_record marks everything enqueued on the context so far and returns
  * an id (next_unsignaled + the submit's signal); dsc_fence_wait blocks until that work has finished
  * (wait_for_signal); dsc_fence_query answers without blocking (1 = finished).  Ids grow by one per record; waiting
- * on an id also retires every older one.  A caller keeping two steps in flight, as the reference does, records a
- * fence after each dsc_schedule_run and waits on the one from two steps ago. */
+ * on an id also retires every older one of its stream.  A caller keeping two steps in flight, as the reference does,
+ * records a fence after each dsc_schedule_run and waits on the one from two steps ago.  Fences need not be waited
+ * for: finished ones are retired in the background once more than a thousand are outstanding, and an id that was
+ * issued and is no longer tracked answers "finished". */
 int dsc_fence_record(dsc_ctx* ctx, uint64_t* out_fence);
 int dsc_fence_wait(dsc_ctx* ctx, uint64_t fence);
 int dsc_fence_query(dsc_ctx* ctx, uint64_t fence, int* out_finished);

@@ -602,3 +602,40 @@ def test_sin_cos_accuracy_over_argument_ranges(hip_backend_session):
     out = env.static_parameter([3], "out")
     env.run(env.build_graph(lambda s: s.write_parameter_value(out, s.parameter_value(bad).sin() + s.parameter_value(bad).cos())), 0)
     assert np.all(np.isnan(env.read_parameter(out)))
+
+
+def test_long_loop_keeps_device_and_host_memory_bounded(hip_backend_session):
+    """4000 ConvNet steps (batch 16) with an overlapped upload before each and a read-back started after each, none
+    of whose fences is ever waited for: the heap's live-buffer count and arena size, and the process's resident set,
+    stay where they were after the first 500 steps (buffers recycle; marks, events and fences of finished work are
+    pooled or retired, not accumulated)."""
+    import psutil
+
+    from descent_amd import Environment, workloads
+
+    be = hip_backend_session
+    env = Environment(be)
+    w = workloads.convnet(env, batch=16, seed=4)
+    px = [env.host_array(w.inputs["x"]) for _ in range(2)]
+    out = be.host_array((1,), np.float32)
+    for a in px:
+        a[...] = 0.5
+
+    def loop(n, base):
+        for i in range(n):
+            env.write_parameter_async(w.inputs["x"], px[i & 1])
+            env.run(w.graph, base + i)
+            env.read_parameter_async(w.scalars["loss"], out)
+        be.sync()
+
+    loop(500, 0)
+    live0, _, arena0 = be.heap_stats()
+    rss0 = psutil.Process().memory_info().rss
+    loop(3500, 500)
+    live1, _, arena1 = be.heap_stats()
+    rss1 = psutil.Process().memory_info().rss
+    assert (live1, arena1) == (live0, arena0)
+    assert rss1 - rss0 < 64 << 20, f"resident set grew by {(rss1 - rss0) >> 20} MiB"
+    assert np.isfinite(out[0])
+    for a in px + [out]:
+        be.host_release(a)
