@@ -371,6 +371,10 @@ string entry_name(const FusedKernel& fk) {
         return "dsc_conv_dgrad_img" + count(fk.dgrad.img) + "_" + count(fk.dgrad.oh) + "x" + count(fk.dgrad.ow) + "_g" + count(fk.dgrad.g) + "_k" +
                count(g.k) + "_c" + count(fk.dgrad.c);
     }
+    if (fk.cfwd.on)
+        return string(fk.has_epilogue ? "dsc_conv_fwd_epilogue_img" : "dsc_conv_fwd_img") + count(fk.cfwd.img) + "_" + count(fk.cfwd.h) + "x" +
+               count(fk.cfwd.w) + "_g" + count(fk.cfwd.g) + "_c" + count(fk.cfwd.c) + "_f" + count(fk.cfwd.fh) + "x" + count(fk.cfwd.fw) + "_n" +
+               count(matmul_dims(d).n);
     if (!fk.row_stages.empty()) return "dsc_row_fused_m" + count(fk.row_m) + "_n" + count(fk.row_n) + "_s" + count((int64_t)fk.row_stages.size());
     switch (d.kind) {
     case DSC_KERNEL_FILL: return "dsc_fill_n" + count(d.shape.dims[0]);
@@ -1046,6 +1050,189 @@ string gen_conv_dgrad(Emitter& em, Generated* out) {
     return "";
 }
 
+// ---- convolution forward ---------------------------------------------------------------------------------
+
+// One workgroup per (image, group).  The group's channels of the image go to LDS once with replicate padding applied
+// (a tile of (oh + fh - 1) x (ow + fw - 1) pixels), so that an im2col element is one LDS word at
+// window origin + tap offset with no clamping left in the inner loop: an im2col row read from memory is fh*fw
+// separate pieces, and a load instruction over 64 rows touches 64 cache lines.  Products run on
+// v_mfma_f32_16x16x4f32 with the operands swapped (D^T = B^T A^T): a wave takes 16 output pixels at a time, lane l
+// feeds the im2col value of pixel l % 16 at k = 4 s + l / 16 from LDS, holds B's K/4 fragments in registers for the
+// whole kernel, and ends up with four consecutive output channels of its pixel: one 16-byte store per output.
+// The kernel is bound by instruction issue, not by MFMA or memory, so everything per element is kept off the VALU:
+// tap offsets are literals when the channel count is a multiple of four, and the fused consumer gets its
+// coordinates instead of dividing an index.
+string gen_conv_fwd(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const FusedKernel::ConvFwd& cv = fk.cfwd;
+    const MatMulDims g = matmul_dims(d);
+    const bool rows = d.output_mode == DSC_MATMUL_ROWS;
+    const int64_t batch_stride = rows ? g.n : g.m * g.n, row_stride = rows ? g.batch * g.n : g.n;
+    const int64_t K = g.k, C = cv.c, GC = cv.g * cv.c, PIX = cv.oh * cv.ow;
+    if (g.batch != cv.g || g.m != cv.img * PIX || K != cv.fh * cv.fw * C || g.chunks != 1 || fk.inputs[0].buffer < 0 ||
+        !conv_fwd_fits(cv, g.n))
+        return "conv forward: geometry mismatch";
+    const int64_t PH = cv.oh + cv.fh - 1, PW = cv.ow + cv.fw - 1;
+    // words per pixel in LDS: 16 neighbouring pixels times four channels should fall into 64 different banks, which
+    // they do when the pitch is an odd multiple of four words
+    const int64_t CP = (C % 4 == 0 && (C / 4) % 2 == 0) ? C + 4 : C;
+    const int64_t steps = (K + 3) / 4, tiles = (PIX + 15) / 16;
+    const int n_out = fk.has_epilogue ? fk.epilogue.raw().n_outputs : 1;
+    const string lb = em.load_view(fk.inputs[1], d.inputs[1], {"cb", "ck", "cn"});
+    em.funcs << "DSC_INLINE float load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb << ";\n}\n";
+    if (fk.has_epilogue) {
+        const dsc_kernel_desc& pe = fk.epilogue.raw();
+        std::ostringstream body;
+        std::map<int, string> ov;
+        ov[fk.epilogue_product_input] = "product";
+        IndexForm form;
+        form.valid = true;
+        form.names = {"cb", "cm", "cn"};
+        form.coefs = {batch_stride, row_stride, 1};
+        form.extents = {g.batch, g.m, g.n};
+        em.emit_pe(body, pe, fk.epilogue_inputs, "gid", "e", ov, &form);
+        for (int o = 0; o < pe.n_outputs; ++o) body << "    result[" << o << "] = et" << pe.outputs[o] << ";\n";
+        em.funcs << "DSC_INLINE void mm_epilogue(float product, int gid, int cb, int cm, int cn, float* result, " << em.params_decl() << ") {\n"
+                 << body.str() << "}\n";
+    }
+    const string img_ptr = "b" + to_string(fk.inputs[0].buffer);
+    const bool vec_fill = C % 4 == 0;                         // 16-byte pieces of a pixel's channels
+    const bool literal_taps = C % 4 == 0;                     // then a k step's four values share one tap
+    const bool vec_store = g.n % 4 == 0 && batch_stride % 4 == 0 && row_stride % 4 == 0;
+    std::ostringstream k;
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
+    k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
+    k << "    typedef float cf_float4 __attribute__((ext_vector_type(4)));\n";
+    const int64_t unit = vec_fill ? 4 : 1, fill_n = PH * PW * C / unit, per_thread = (fill_n + 255) / 256;
+    const int64_t FU = std::min<int64_t>(per_thread, 8);
+    k << "    __shared__ __attribute__((aligned(16))) float tile[" << S(PH * PW * CP) << "];\n";
+    k << "    __shared__ float sB[" << S(steps * 64) << "];\n";
+    k << "    const int cb = blockIdx.x % " << S(cv.g) << ", img = blockIdx.x / " << S(cv.g) << ";\n";
+    k << "    const int lane = threadIdx.x & 63, li = lane & 15, lk = lane >> 4;\n";
+    // the 16-pixel tiles are dealt to the four waves in turn; which wave takes the odd ones out rotates with the
+    // workgroup, so that no SIMD of a CU collects all of them
+    k << "    const int wv = ((threadIdx.x >> 6) + blockIdx.x) & 3;\n";
+    // 1. B goes through LDS: every wave needs all of it in MFMA fragment order, and when each wave of every
+    // workgroup fetched its fragments itself (K/4 loads per lane, the same few cache lines for the whole grid) those
+    // loads alone cost a third of the kernel.  Zero beyond k and n.
+    const int64_t BU = (steps * 64 + 255) / 256;
+    k << "    float bv[" << S(BU) << "];\n";
+    k << "#pragma unroll\n    for (int u = 0; u < " << S(BU) << "; ++u) {\n";
+    k << "        const int e = threadIdx.x + u * 256, kk = e >> 4, nn = e & 15;\n";
+    k << "        const float v = load_b(cb, min(kk, " << S(K - 1) << "), min(nn, " << S(g.n - 1) << "), " << em.params_pass() << ");\n";
+    k << "        bv[u] = (kk < " << S(K) << " && nn < " << S(g.n) << ") ? v : 0.f;\n    }\n";
+    // 2. the padded tile: tile[py][px][c] = image[clamp(py - pad_h)][clamp(px - pad_w)][c]
+    const string vt = vec_fill ? "float4" : "float";
+    auto emit_fill_loads = [&](const string& ind) {
+        k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(FU) << "; ++u) {\n";
+        k << ind << "    const int e = min(i0 + u * 256, " << S(fill_n - 1) << ") * " << S(unit) << ";\n";
+        k << ind << "    const int ch = e % " << S(C) << ", px = (e / " << S(C) << ") % " << S(PW) << ", py = e / " << S(C * PW) << ";\n";
+        k << ind << "    const int sy = clampi(py - " << S(cv.pad_h) << ", 0, " << S(cv.h - 1) << "), sx = clampi(px - " << S(cv.pad_w) << ", 0, " << S(cv.w - 1) << ");\n";
+        k << ind << "    v[u] = *(const " << vt << "*)(" << img_ptr << " + ((img * " << S(cv.h) << " + sy) * " << S(cv.w) << " + sx) * " << S(GC) << " + cb * " << S(C)
+          << " + ch);\n" << ind << "}\n";
+    };
+    auto emit_fill_stores = [&](const string& ind) {
+        k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(FU) << "; ++u)\n" << ind << "    if (i0 + u * 256 < " << S(fill_n) << ") *(" << vt << "*)(tile + "
+          << (CP == C ? "(i0 + u * 256) * " + S(unit) : "((i0 + u * 256) * " + S(unit) + " / " + S(C) + ") * " + S(CP) + " + (i0 + u * 256) * " + S(unit) + " % " + S(C))
+          << ") = v[u];\n";
+    };
+    k << "    " << vt << " v[" << S(FU) << "];\n";
+    if (per_thread <= 8) {
+        k << "    const int i0 = threadIdx.x;\n";
+        emit_fill_loads("    ");
+        emit_fill_stores("    ");
+    } else {
+        k << "    for (int i0 = threadIdx.x; i0 < " << S(fill_n) << "; i0 += " << S(256 * FU) << ") {\n";
+        emit_fill_loads("        ");
+        emit_fill_stores("        ");
+        k << "    }\n";
+    }
+    k << "#pragma unroll\n    for (int u = 0; u < " << S(BU) << "; ++u)\n        if (threadIdx.x + u * 256 < " << S(steps * 64) << ") sB[threadIdx.x + u * 256] = bv[u];\n";
+    k << "    __syncthreads();\n";
+    // lane l holds B[k = 4 s + l / 16][n = l % 16]
+    k << "    float fb[" << S(steps) << "];\n";
+    k << "#pragma unroll\n    for (int s = 0; s < " << S(steps) << "; ++s) fb[s] = sB[s * 64 + lane];\n";
+    // 3. offsets of the k steps inside a pixel's window
+    if (literal_taps) {
+        k << "    constexpr int KO[" << S(steps) << "] = {";
+        for (int64_t s = 0; s < steps; ++s) {
+            const int64_t tap = 4 * s / C, ch = 4 * s % C;
+            k << (s ? ", " : "") << S(((tap / cv.fw) * PW + tap % cv.fw) * CP + ch);
+        }
+        k << "};\n";
+    }
+    auto emit_group = [&](int64_t TG, const string& q0, const string& ind) {
+        k << ind << "int pb[" << S(TG) << "];\n" << ind << "cf_float4 acc[" << S(TG) << "];\n";
+        k << "#pragma unroll\n" << ind << "for (int j = 0; j < " << S(TG) << "; ++j) {\n";
+        k << ind << "    const int p = min(((" << q0 << " + j) * 4 + wv) * 16 + li, " << S(PIX - 1) << ");\n";
+        k << ind << "    pb[j] = ((p / " << S(cv.ow) << ") * " << S(PW) << " + p % " << S(cv.ow) << ") * " << S(CP) << (literal_taps ? " + lk" : "") << ";\n";
+        k << ind << "    acc[j] = (cf_float4){0.f, 0.f, 0.f, 0.f};\n" << ind << "}\n";
+        k << "#pragma unroll\n" << ind << "for (int s = 0; s < " << S(steps) << "; ++s) {\n";
+        if (literal_taps) {
+            k << ind << "    const int ko = KO[s];\n";
+        } else {
+            // past the end of k the B fragment is zero, so the repeated value adds nothing
+            k << ind << "    const int kk = min(4 * s + lk, " << S(K - 1) << "), tap = kk / " << S(C) << ";\n";
+            k << ind << "    const int ko = ((tap / " << S(cv.fw) << ") * " << S(PW) << " + tap % " << S(cv.fw) << ") * " << S(C) << " + kk % " << S(C) << ";\n";
+        }
+        k << "#pragma unroll\n" << ind << "    for (int j = 0; j < " << S(TG) << "; ++j)\n";
+        k << ind << "        acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fb[s], tile[pb[j] + ko], acc[j], 0, 0, 0);\n" << ind << "}\n";
+        // accumulator register i of lane l is D^T[column 4 * (l / 16) + i][pixel l % 16]
+        k << "#pragma unroll\n" << ind << "for (int j = 0; j < " << S(TG) << "; ++j) {\n";
+        k << ind << "    const int pp = ((" << q0 << " + j) * 4 + wv) * 16 + li, cm = img * " << S(PIX) << " + pp, cn = 4 * lk;\n";
+        k << ind << "    const int c_at = cb * " << S(batch_stride) << " + cm * " << S(row_stride) << " + cn;\n";
+        k << ind << "    if (pp < " << S(PIX) << " && cn < " << S(g.n) << ") {\n";
+        if (fk.has_epilogue) {
+            k << ind << "        float res[4][" << n_out << "];\n";
+            k << "#pragma unroll\n" << ind << "        for (int i = 0; i < 4; ++i) mm_epilogue(acc[j][i], c_at + i, cb, cm, min(cn + i, " << S(g.n - 1) << "), res[i], "
+              << em.params_pass() << ");\n";
+        }
+        for (int o = 0; o < n_out; ++o) {
+            const string ptr = "b" + to_string(fk.outputs[o]);
+            auto val = [&](int i) { return fk.has_epilogue ? "res[" + to_string(i) + "][" + to_string(o) + "]" : "acc[j][" + to_string(i) + "]"; };
+            if (vec_store) {
+                k << ind << "        *(float4*)(" << ptr << " + c_at) = make_float4(" << val(0) << ", " << val(1) << ", " << val(2) << ", " << val(3) << ");\n";
+            } else {
+                for (int i = 0; i < 4; ++i)
+                    k << ind << "        if (cn + " << i << " < " << S(g.n) << ") " << ptr << "[c_at + " << i << "] = " << val(i) << ";\n";
+            }
+        }
+        k << ind << "    }\n" << ind << "}\n";
+    };
+    // 4. every wave has `full` whole turns, taken TGMAX tiles at a time so that their MFMA chains interleave; the
+    // waves with wv < rem have one more
+    const int64_t full = tiles / 4, rem = tiles % 4, TGMAX = 8;
+    const int64_t whole_groups = full / TGMAX, tail = full % TGMAX;
+    if (whole_groups == 1) {
+        k << "    {\n";
+        emit_group(TGMAX, "0", "        ");
+        k << "    }\n";
+    } else if (whole_groups > 1) {
+        k << "    for (int q0 = 0; q0 < " << S(whole_groups * TGMAX) << "; q0 += " << S(TGMAX) << ") {\n";
+        emit_group(TGMAX, "q0", "        ");
+        k << "    }\n";
+    }
+    if (tail) {
+        k << "    {\n";
+        emit_group(tail, S(whole_groups * TGMAX), "        ");
+        k << "    }\n";
+    }
+    if (rem) {
+        k << "    if (wv < " << S(rem) << ") {\n";
+        emit_group(1, S(full), "        ");
+        k << "    }\n";
+    }
+    k << "}\n";
+    if (cv.img * cv.g >= kMaxIndex) return "conv forward: grid too large";
+    out->grid = (unsigned)(cv.img * cv.g);
+    out->block = 256;
+    out->source = k.str();
+    out->note = "conv forward: workgroup per image and group, padded image tile in LDS, mfma 16x16x4, " + S(cv.fh) + "x" + S(cv.fw) + " taps x " + S(C) +
+                " channels" + (fk.has_epilogue ? " +epilogue" : "");
+    return "";
+}
+
 // ---- matmul -------------------------------------------------------------------------------------------
 
 struct MmConfig {
@@ -1673,6 +1860,9 @@ void count_work(const FusedKernel& fk, Generated* g) {
     for (auto& st : fk.row_stages) read_desc(st.k.raw(), st.inputs, -1);
     for (auto& v : fk.virtuals) read_desc(v.pe.raw(), v.inputs, -1);
     if (fk.has_epilogue) read_desc(fk.epilogue.raw(), fk.epilogue_inputs, fk.epilogue_product_input);
+    // the convolution kernel reads the image itself, not the window copy its MatMul descriptor speaks of
+    if (fk.cfwd.on && fk.inputs[0].buffer >= 0)
+        touched[fk.inputs[0].buffer] = extent[fk.inputs[0].buffer] = (double)(fk.cfwd.img * fk.cfwd.h * fk.cfwd.w * fk.cfwd.g * fk.cfwd.c);
     double elements = 0;
     for (int i = 0; i < fk.n_buffers; ++i)
         if (!fk.buffer_is_output[i]) elements += std::min(touched[i], extent[i]);
@@ -1756,6 +1946,11 @@ std::string FusedKernel::key() const {
         for (int64_t v : {dgrad.img, dgrad.oh, dgrad.ow, dgrad.g, dgrad.fh, dgrad.fw, dgrad.c, dgrad.pad_h, dgrad.pad_w, (int64_t)dgrad.rows_first})
             s.append(reinterpret_cast<const char*>(&v), 8);
     }
+    if (cfwd.on) {
+        s += "|CF";
+        for (int64_t v : {cfwd.img, cfwd.h, cfwd.w, cfwd.g, cfwd.c, cfwd.fh, cfwd.fw, cfwd.oh, cfwd.ow, cfwd.pad_h, cfwd.pad_w})
+            s.append(reinterpret_cast<const char*>(&v), 8);
+    }
     if (shared_scatter) s += "|SS";
     for (size_t i = 0; i < parts.size(); ++i) {
         s += "|P{" + parts[i].key() + "}";
@@ -1780,6 +1975,10 @@ string generate_multi(const FusedKernel& fk, Generated* out);
 string generate_scatter_chain(const FusedKernel& fk, Generated* out);
 }
 
+bool conv_fwd_fits(const FusedKernel::ConvFwd& c, int64_t n) {
+    return (c.oh + c.fh - 1) * (c.ow + c.fw - 1) * c.c * 4 <= 48 * 1024 && n <= 16 && c.fh * c.fw * c.c >= 4 && c.fh * c.fw * c.c <= 512 && c.oh * c.ow >= 16;
+}
+
 bool conv_dgrad_fits(const FusedKernel::ConvDgrad& c, int64_t k) {
     if (k % 4 != 0 || c.g * c.c > 64 || c.fh * c.fw * k * c.g * c.c > 8192) return false;
     return (dgrad_lds_floats(c, k) + dgrad_pitch(k) + 4) * 4 <= 64 * 1024 && c.oh + c.fh - 1 > 2 * c.pad_h && c.ow + c.fw - 1 > 2 * c.pad_w;
@@ -1787,7 +1986,7 @@ bool conv_dgrad_fits(const FusedKernel::ConvDgrad& c, int64_t k) {
 
 bool can_be_part(const FusedKernel& fk) {
     if (!fk.parts.empty()) return false;
-    if (fk.dgrad.on || !fk.row_stages.empty()) return true;
+    if (fk.dgrad.on || fk.cfwd.on || !fk.row_stages.empty()) return true;
     if (fk.main.raw().kind != DSC_KERNEL_MATMUL) return true;
     // of the MatMul kernels, the row-per-thread, short-k and tall-k ones run 256 threads addressed by blockIdx.x
     const MatMulDims g = matmul_dims(fk.main.raw());
@@ -1845,6 +2044,9 @@ static std::string generate_one(const FusedKernel& fk, Generated* out, bool with
     } else if (fk.dgrad.on) {
         if (fk.main.raw().kind != DSC_KERNEL_MATMUL || fk.has_epilogue) return "conv dgrad: needs a plain MatMul";
         err = gen_conv_dgrad(em, &g);
+    } else if (fk.cfwd.on) {
+        if (fk.main.raw().kind != DSC_KERNEL_MATMUL) return "conv forward: needs a MatMul";
+        err = gen_conv_fwd(em, &g);
     } else
     switch (fk.main.raw().kind) {
     case DSC_KERNEL_FILL: err = gen_fill(em, &g); break;

@@ -75,6 +75,14 @@ struct FusedKernel {
         int64_t pad_h = 0, pad_w = 0;  // Unpads folded in (0: the output is the padded image)
         int32_t rows_first = 1;        // the Unpad along the image rows came first
     } dgrad;
+    // MatMul whose A operand is the im2col of a stride-1 convolution's (replicate-padded) input: the kernel reads the
+    // image [img, h, w, g*c] itself, one workgroup per (image, group) with the group's channels of the image in LDS,
+    // instead of the materialised or generated window copy (main.inputs[0] is the image; the descriptor keeps the
+    // MatMul's shapes).  k = (fy * fw + fx) * c + ch, row = (img * oh + oy) * ow + ox.
+    struct ConvFwd {
+        bool on = false;
+        int64_t img = 0, h = 0, w = 0, g = 0, c = 0, fh = 0, fw = 0, oh = 0, ow = 0, pad_h = 0, pad_w = 0;
+    } cfwd;
     bool sum_chunks = false;               // MatMul: ignore the descriptor's chunk count, write one full sum
     int colsum_out = -1;                   // MatMul (MFMA template): buffer that takes the column sums of B per k chunk
     bool as_part = false;                  // generated as one part of a multi-part launch (set while the launch is generated)
@@ -110,6 +118,8 @@ std::string generate(const FusedKernel& k, Generated* out);
 // Whether the convolution data-gradient kernel can take this geometry (k = output channels per group): the image
 // tile must fit the workgroup's LDS.
 bool conv_dgrad_fits(const FusedKernel::ConvDgrad& c, int64_t k);
+// Whether the convolution-forward kernel takes this geometry with n output channels per group.
+bool conv_fwd_fits(const FusedKernel::ConvFwd& c, int64_t n);
 
 // Whether a chain of ScatterAdds with this accumulator size and this many values in total runs as one kernel with
 // the accumulator in LDS (shared_scatter).

@@ -351,12 +351,19 @@ Kernel* get_kernel(Context* ctx, const FusedKernel& fk, int* status) {
                       (long long)c.fh, (long long)c.fw, (long long)c.g);
         k->label = text;
     }
+    if (fk.cfwd.on) {
+        const auto& c = fk.cfwd;
+        char text[160];
+        std::snprintf(text, sizeof text, "ConvForward [%lld, %lld, %lld, %lld] %lldx%lld taps, %lld groups", (long long)c.img, (long long)c.oh,
+                      (long long)c.ow, (long long)(c.g * matmul_dims(fk.main.raw()).n), (long long)c.fh, (long long)c.fw, (long long)c.g);
+        k->label = text;
+    }
     if (fk.has_epilogue) k->label += " + " + label_name(fk.epilogue.raw());
     if (!fk.virtuals.empty()) k->label += " <" + std::to_string(fk.virtuals.size()) + " fused producers>";
     if (!fk.parts.empty()) {
         k->label = "Multi (" + std::to_string(fk.parts.size()) + " kernels:";
         for (auto& part : fk.parts)
-            k->label += " " + std::string(part.dgrad.on ? "ConvDataGrad" : part.row_stages.empty() ? label_name(part.main.raw()) : "RowFused") + ";";
+            k->label += " " + std::string(part.dgrad.on ? "ConvDataGrad" : part.cfwd.on ? "ConvForward" : part.row_stages.empty() ? label_name(part.main.raw()) : "RowFused") + ";";
         k->label += ")";
     }
     k->reference_groups = reference_group_count(fk.main.raw());

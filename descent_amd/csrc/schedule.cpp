@@ -188,6 +188,19 @@ int64_t view_index(const dsc_view& v, const int64_t* coord) {
     return idx;
 }
 
+// The same with every input coordinate clamped into its axis: what a load through the view reads (padding by
+// replication is a view whose coordinates leave the array and are clamped, src/shape.rs:374-379, 503-526).
+int64_t view_index_clamped(const dsc_view& v, const int64_t* coord) {
+    int64_t st[DSC_MAX_DIM], in[DSC_MAX_DIM];
+    strides_of(v.in_shape, st);
+    for (int i = 0; i < v.in_shape.rank; ++i) in[i] = v.in_offset[i];
+    for (int j = 0; j < v.out_shape.rank; ++j)
+        if (v.map_axis[j] >= 0) in[v.map_axis[j]] += v.map_step[j] * coord[j];
+    int64_t idx = 0;
+    for (int i = 0; i < v.in_shape.rank; ++i) idx += std::min(std::max<int64_t>(in[i], 0), v.in_shape.dims[i] - 1) * st[i];
+    return idx;
+}
+
 dsc_pe_op pe_op(int kind, int op = 0, int a0 = 0, int a1 = 0, int a2 = 0, int a3 = 0) {
     dsc_pe_op o{};
     o.kind = kind;
@@ -998,6 +1011,100 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             mm.alive = false;
             if (copy_idx >= 0) drafts[copy_idx].alive = false;
             drafts[w_idx] = fused;
+        }
+
+        // Pass 1d: the forward of a stride-1 convolution arrives as a copy cluster that writes the im2col of the
+        // (replicate-padded) image, and a MatMul over it.  The dedicated kernel reads the image itself.  The geometry
+        // is a hypothesis (filter height from the divisors of k / c, padding from the output size) that is then
+        // checked on every (pixel, k) of three images against the addresses the copy's view really produces.
+        for (int i = 0; i < (int)drafts.size(); ++i) {
+            static const bool enabled = !(std::getenv("DSC_FUSE_CONV_FWD") && std::getenv("DSC_FUSE_CONV_FWD")[0] == '0');
+            if (!enabled || (flags & DSC_SCHEDULE_NO_CONV_KERNELS)) break;
+            Draft& mm = drafts[i];
+            const dsc_kernel_desc& md = mm.fk.main.raw();
+            if (!mm.alive || md.kind != DSC_KERNEL_MATMUL || !mm.fk.virtuals.empty() || mm.keep_split || mm.fk.colsum_out >= 0 ||
+                mm.fk.dgrad.on || mm.fk.inputs[0].buffer < 0)
+                continue;
+            const MatMulDims g = matmul_dims(md);
+            if (g.chunks != 1 || g.n > 16) continue;
+            const int a_node = mm.params[mm.fk.inputs[0].buffer];
+            int ci = -1;
+            for (int q = 0; q < i; ++q)
+                if (drafts[q].alive && !drafts[q].outs.empty() && drafts[q].outs[0].node == a_node) ci = q;
+            if (ci < 0) continue;
+            const Draft& cp = drafts[ci];
+            const dsc_kernel_desc& cd = cp.fk.main.raw();
+            if (cd.kind != DSC_KERNEL_PER_ELEMENT || !cp.fk.virtuals.empty() || cp.fk.has_epilogue || cd.n_outputs != 1 || cd.n_inputs != 1 ||
+                cd.n_ops > 2 || cd.ops[0].kind != DSC_PE_LOAD || (cd.n_ops == 2 && !(cd.ops[1].kind == DSC_PE_UNARY && cd.ops[1].op == DSC_UN_MOV)) ||
+                is_graph_output[a_node] || cp.outs[0].copy_from >= 0 || cp.fk.inputs[0].buffer < 0)
+                continue;
+            // (the filter gradient reads the same copy: it stays for that reader, which takes it as a fused producer)
+            const bool only_reader = consumers_of(a_node).size() == 1;
+            const dsc_view& cvw = cd.inputs[0];  // element of the copy -> element of the image
+            const dsc_view& av = md.inputs[0];   // (batch, row, k) -> element of the copy
+            if (cvw.in_shape.rank != 4 || any_clamp(av)) continue;
+            const int64_t IMG = cvw.in_shape.dims[0], H = cvw.in_shape.dims[1], W = cvw.in_shape.dims[2], GC = cvw.in_shape.dims[3];
+            const int64_t G = g.batch;
+            if (GC % G != 0 || g.m % IMG != 0) continue;
+            const int64_t C = GC / G, PIX = g.m / IMG;
+            if (g.k % C != 0) continue;
+            const int64_t taps = g.k / C;
+            auto image_index = [&](int64_t cb, int64_t cm, int64_t ck) {
+                const int64_t c3[3] = {cb, cm, ck};
+                int64_t idx = view_index(av, c3);
+                int64_t cc[DSC_MAX_DIM];
+                for (int a = cvw.out_shape.rank - 1; a >= 0; --a) {
+                    cc[a] = idx % cvw.out_shape.dims[a];
+                    idx /= cvw.out_shape.dims[a];
+                }
+                return view_index_clamped(cvw, cc);
+            };
+            FusedKernel::ConvFwd found;
+            for (int64_t FH = 1; FH <= taps && !found.on; ++FH) {
+                if (taps % FH != 0) continue;
+                const int64_t FW = taps / FH;
+                for (int64_t ph = 0; ph <= FH && !found.on; ++ph) {
+                    const int64_t OH = H + 2 * ph - FH + 1;
+                    if (OH < 1 || PIX % OH != 0) continue;
+                    const int64_t OW = PIX / OH;
+                    if ((OW + FW - 1 - W) % 2 != 0) continue;
+                    const int64_t pw = (OW + FW - 1 - W) / 2;
+                    if (pw < 0 || pw > FW) continue;
+                    auto clampv = [](int64_t v, int64_t hi) { return v < 0 ? 0 : (v > hi ? hi : v); };
+                    bool ok = true;
+                    for (int64_t img : {(int64_t)0, IMG / 2, IMG - 1}) {
+                        for (int64_t p = 0; p < PIX && ok; ++p)
+                            for (int64_t cb = 0; cb < G && ok; ++cb)
+                                for (int64_t ck = 0; ck < g.k && ok; ++ck) {
+                                    const int64_t tap = ck / C, ch = ck % C;
+                                    const int64_t y = clampv(p / OW + tap / FW - ph, H - 1), x = clampv(p % OW + tap % FW - pw, W - 1);
+                                    const int64_t want = ((img * H + y) * W + x) * GC + cb * C + ch;
+                                    if (image_index(cb, img * PIX + p, ck) != want) ok = false;
+                                }
+                    }
+                    if (!ok) continue;
+                    found.on = true;
+                    found.img = IMG; found.h = H; found.w = W; found.g = G; found.c = C;
+                    found.fh = FH; found.fw = FW; found.oh = OH; found.ow = OW; found.pad_h = ph; found.pad_w = pw;
+                }
+            }
+            if (!found.on || !conv_fwd_fits(found, g.n)) continue;
+            const int image_node = cp.params[cp.fk.inputs[0].buffer];
+            if (taken_in_place_between(ci, i, {image_node})) continue;
+            Draft fused = mm;
+            fused.fk.cfwd = found;
+            fused.fk.inputs[0] = Source{};
+            fused.fk.inputs[0].buffer = param_index(fused, image_node, false);
+            {
+                Generated probe;
+                if (!generate(fused.fk, &probe).empty()) continue;
+            }
+            compact(fused);
+            if (only_reader) {
+                fused.covers.insert(fused.covers.end(), cp.covers.begin(), cp.covers.end());
+                drafts[ci].alive = false;
+            }
+            drafts[i] = fused;
         }
 
         // Pass 1b: clusters that all work on the rows of one [m, n] array with a short n -- Reduces along n and the
