@@ -1052,6 +1052,10 @@ string gen_conv_dgrad(Emitter& em, Generated* out) {
 
 // ---- convolution forward ---------------------------------------------------------------------------------
 
+// Words per pixel of the forward kernel's LDS tile: 16 neighbouring pixels times four channels should fall into 64
+// different banks, which they do when the pitch is an odd multiple of four words.
+int64_t conv_fwd_pitch(int64_t c) { return (c % 4 == 0 && (c / 4) % 2 == 0) ? c + 4 : c; }
+
 // One workgroup per (image, group).  The group's channels of the image go to LDS once with replicate padding applied
 // (a tile of (oh + fh - 1) x (ow + fw - 1) pixels), so that an im2col element is one LDS word at
 // window origin + tap offset with no clamping left in the inner loop: an im2col row read from memory is fh*fw
@@ -1074,9 +1078,7 @@ string gen_conv_fwd(Emitter& em, Generated* out) {
         !conv_fwd_fits(cv, g.n))
         return "conv forward: geometry mismatch";
     const int64_t PH = cv.oh + cv.fh - 1, PW = cv.ow + cv.fw - 1;
-    // words per pixel in LDS: 16 neighbouring pixels times four channels should fall into 64 different banks, which
-    // they do when the pitch is an odd multiple of four words
-    const int64_t CP = (C % 4 == 0 && (C / 4) % 2 == 0) ? C + 4 : C;
+    const int64_t CP = conv_fwd_pitch(C);  // words per pixel in LDS
     const int64_t steps = (K + 3) / 4, tiles = (PIX + 15) / 16;
     const int n_out = fk.has_epilogue ? fk.epilogue.raw().n_outputs : 1;
     const string lb = em.load_view(fk.inputs[1], d.inputs[1], {"cb", "ck", "cn"});
@@ -1976,7 +1978,9 @@ string generate_scatter_chain(const FusedKernel& fk, Generated* out);
 }
 
 bool conv_fwd_fits(const FusedKernel::ConvFwd& c, int64_t n) {
-    return (c.oh + c.fh - 1) * (c.ow + c.fw - 1) * c.c * 4 <= 48 * 1024 && n <= 16 && c.fh * c.fw * c.c >= 4 && c.fh * c.fw * c.c <= 512 && c.oh * c.ow >= 16;
+    const int64_t k = c.fh * c.fw * c.c;
+    const int64_t lds_bytes = (c.oh + c.fh - 1) * (c.ow + c.fw - 1) * conv_fwd_pitch(c.c) * 4 + (k + 3) / 4 * 256;  // image tile + B fragments
+    return lds_bytes <= 60 * 1024 && n <= 16 && k >= 4 && k <= 512 && c.oh * c.ow >= 16;
 }
 
 bool conv_dgrad_fits(const FusedKernel::ConvDgrad& c, int64_t k) {

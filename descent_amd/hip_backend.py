@@ -131,7 +131,7 @@ def codegen_compile(kernel, arch: str = "gfx950") -> int:
 
 def schedule_flags(fused) -> int:
     """`fused`: True (all fusion), False (one launch per reference cluster), "generic-conv" (all fusion, but
-    convolution gradients stay on the generic MatMul path instead of the dedicated kernels), or "graph-replay"
+    convolutions stay on the generic MatMul path instead of the dedicated kernels), or "graph-replay"
     (all fusion, each run captured as a HIP graph and replayed when the buffers land on the same addresses)."""
     if fused == "generic-conv":
         return _abi.SCHEDULE_NO_CONV_KERNELS

@@ -326,8 +326,9 @@ typedef struct dsc_schedule dsc_schedule;
 #define DSC_SCHEDULE_GRAPH_REPLAY 4u /* capture each run's launches as a HIP graph and replay it whenever a later run's
                                         buffers land on the same addresses (the Submit half of the reference's
                                         command buffer, device/command_buffer.rs:64-123, recorded once) */
-#define DSC_SCHEDULE_NO_CONV_KERNELS 2u /* keep convolution gradients on the generic MatMul path (fused producers)
-                                           instead of the dedicated LDS-tiled kernels (for parity tests) */
+#define DSC_SCHEDULE_NO_CONV_KERNELS 2u /* keep convolutions (forward and data gradient) on the generic MatMul path
+                                           (fused producers) instead of the dedicated LDS-tiled kernels (for
+                                           parity tests) */
 
 int dsc_schedule_create(dsc_ctx* ctx, const dsc_schedule_desc* desc, uint32_t flags, dsc_schedule** out);
 int dsc_schedule_destroy(dsc_ctx* ctx, dsc_schedule* s);

@@ -441,7 +441,11 @@ CONV_GEOMETRIES = [
     (60, 8, 8, 4, 8, 3, 3, 0, 1),       # no padding: no Unpads to fold
     (25, 7, 5, 16, 16, 3, 1, 0, 1),     # 3x1 taps
     (3, 6, 6, 64, 64, 3, 3, 1, 1),      # many channels: stays on the generic path
+    (20, 10, 10, 3, 6, 3, 3, 1, 1),     # three input channels, six outputs: no 16-byte pieces anywhere
+    (16, 8, 8, 6, 20, 3, 3, 1, 2),      # the same per group, ten outputs
 ]
+CONV_WITHOUT_DATA_GRAD_KERNEL = set(CONV_GEOMETRIES[-3:])
+CONV_WITHOUT_FORWARD_KERNEL = {CONV_GEOMETRIES[-3]}
 
 
 @pytest.mark.parametrize("geom", CONV_GEOMETRIES, ids=lambda g: "x".join(map(str, g)))
@@ -451,10 +455,11 @@ def test_conv2d_gradients_over_geometries(hip_backend_session, geom, fused):
     g, gy, gdx, gdf = _conv_grad_case(genv, *geom, seed=90)
     _, cy, cdx, cdf = _conv_grad_case(cenv, *geom, seed=90)
     listing = next(iter(g.__dict__["_schedules"].values())).describe()
-    if fused is True:  # all but the many-channel case run the dedicated data-gradient kernel
-        assert ("ConvDataGrad" in listing) == (geom is not CONV_GEOMETRIES[-1]), listing
+    if fused is True:  # the dedicated kernels: image tile in LDS
+        assert ("ConvDataGrad" in listing) == (geom not in CONV_WITHOUT_DATA_GRAD_KERNEL), listing
+        assert ("ConvForward" in listing) == (geom not in CONV_WITHOUT_FORWARD_KERNEL), listing
     if fused == "generic-conv":
-        assert "ConvDataGrad" not in listing, listing
+        assert "ConvDataGrad" not in listing and "ConvForward" not in listing, listing
     assert rel_l2(gy, cy) <= TOL, listing
     assert rel_l2(gdx, cdx) <= TOL, (rel_l2(gdx, cdx), listing)
     assert rel_l2(gdf, cdf) <= TOL, (rel_l2(gdf, cdf), listing)

@@ -221,7 +221,11 @@ def test_convnet_graph_shape():
     # the data gradient of the second convolution: MatMul + reshape copy + WindowsToImage as one product over
     # the padded image, both operands fused producers
     assert "ConvDataGrad" in listing and "conv data gradient: workgroup per image and group, tile in LDS, 3x3 taps x 16 channels, border folds fused" in listing
-    assert "MatMul (k=144) [1, 256000, 2, 8]" in hip_backend.check_schedule(w.graph, fused="generic-conv")
+    # both forward convolutions: the image tile goes to LDS, the im2col copy stays only for the filter gradient
+    assert listing.count("ConvForward") == 2
+    assert "conv forward: workgroup per image and group, padded image tile in LDS, mfma 16x16x4, 3x3 taps x 8 channels +epilogue" in listing
+    generic = hip_backend.check_schedule(w.graph, fused="generic-conv")
+    assert "MatMul (k=144) [1, 256000, 2, 8]" in generic and "ConvForward" not in generic and "ConvDataGrad" not in generic
     # the work figures of the listing: the eleven GEMMs of the step as the reference runs them
     assert "4.373 GFLOP in MatMuls" in hip_backend.check_schedule(w.graph, fused=False)
 
