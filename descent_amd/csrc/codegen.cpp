@@ -360,6 +360,7 @@ struct Emitter {
 bool rows_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
 bool smallk_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
 bool tallk_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
+bool dot_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
 
 // Entry points carry the kernel kind and its size, so that a profiler's per-name statistics tell the kernels of
 // a schedule apart: dsc_matmul_mfma_epilogue_b1_m8192_n8192_k8192, dsc_reduce_k4084_n144, dsc_per_element_n12544000.
@@ -388,6 +389,7 @@ string entry_name(const FusedKernel& fk) {
         string base = rows_kernel_applies(fk, g)     ? "dsc_matmul_rows"
                       : smallk_kernel_applies(fk, g) ? "dsc_matmul_shortk"
                       : tallk_kernel_applies(fk, g)  ? "dsc_matmul_tallk"
+                      : dot_kernel_applies(fk, g)    ? "dsc_matmul_dot"
                                                      : "dsc_matmul_mfma";
         if (fk.has_epilogue) base += "_epilogue";
         return base + "_b" + count(g.batch) + "_m" + count(g.m) + "_n" + count(g.n) + "_k" + count(g.k);
@@ -1031,6 +1033,22 @@ string gen_conv_dgrad(Emitter& em, Generated* out) {
             const bool is_y = j == "jy";
             return "for (int " + j + " = " + S(-(is_y ? cv.pad_h : cv.pad_w)) + "; " + j + " <= " + S(is_y ? cv.pad_h : cv.pad_w) + "; ++" + j + ")";
         };
+        if (H > 1 && W > 1) {
+            // a pixel lies on at most one edge per axis, so it has at most pad + 1 candidates per axis, taken in rising
+            // order: on the first edge the padded coordinates 0..pad, on the last one own..own + pad, else its own
+            auto slots = [&](const string& q, bool is_y) {
+                return "for (int " + q + " = 0; " + q + " <= " + S(is_y ? cv.pad_h : cv.pad_w) + "; ++" + q + ")";
+            };
+            const string qo = cv.rows_first ? "qx" : "qy", qi = cv.rows_first ? "qy" : "qx";
+            k << "        const bool edge_y = y == 0 || y == " << S(H - 1) << ", edge_x = x == 0 || x == " << S(W - 1) << ";\n";
+            k << "        const int base_y = y == 0 ? 0 : y + " << S(cv.pad_h) << ", base_x = x == 0 ? 0 : x + " << S(cv.pad_w) << ";\n";
+            k << "#pragma unroll\n        " << slots(qo, !cv.rows_first) << " {\n            float part = 0.f;\n";
+            k << "#pragma unroll\n            " << slots(qi, cv.rows_first) << " {\n";
+            k << "                const bool ok = (edge_y || qy == 0) && (edge_x || qx == 0);\n";
+            k << "                const int ky = base_y + (edge_y ? qy : 0), kx = base_x + (edge_x ? qx : 0);\n";
+            k << "                const float w = lds[(ky * " << S(PW) << " + kx) * " << S(C) << " + c];\n";
+            k << "                part += ok ? w : 0.f;\n            }\n            sum += part;\n        }\n";
+        } else {
         k << "#pragma unroll\n        " << range(outer) << " {\n            float part = 0.f;\n";
         k << "#pragma unroll\n            " << range(inner) << " {\n";
         k << "                const bool ok_y = jy == 0 || (jy < 0 && y == 0) || (jy > 0 && y == " << S(H - 1) << ");\n";
@@ -1039,6 +1057,7 @@ string gen_conv_dgrad(Emitter& em, Generated* out) {
           << " + jx, 0, " << S(PW - 1) << ");\n";
         k << "                const float w = lds[(ky * " << S(PW) << " + kx) * " << S(C) << " + c];\n";
         k << "                part += (ok_y && ok_x) ? w : 0.f;\n            }\n            sum += part;\n        }\n";
+        }
         k << "        " << out_ptr << "[((img * " << S(H) << " + y) * " << S(W) << " + x) * " << S(GC) << " + cb * " << S(C) << " + c] = sum;\n    }\n}\n";
     }
     if (cv.img * G >= kMaxIndex) return "conv dgrad: grid too large";
@@ -1372,6 +1391,103 @@ string gen_matmul_smallk(Emitter& em, Generated* out) {
     out->block = 256;
     out->source = k.str();
     out->note = string("short-k fma, four columns per thread") + (fk.has_epilogue ? " +epilogue" : "");
+    return "";
+}
+
+// Dot-product kernel for products with few columns and not many rows (a classifier head: 1000 x 128 -> 10): too
+// small to fill the MFMA template's tiles -- a 32x32 tile grid of such a product is a few dozen single-wave
+// workgroups, each walking k in eight sequential load -> LDS -> MFMA round trips.  Here L lanes share one row: lane l
+// takes the 16-byte blocks l, l + L, ... of the row's k range (consecutive lanes read consecutive memory), multiplies
+// them with B from LDS (the whole of B is a few KB), and the lanes' partial sums meet in a shuffle butterfly.  All
+// loads of a lane are independent, so the kernel is one memory round trip deep.
+bool dot_shape(const MatMulDims& g) {
+    // B is staged by every workgroup, for the 256 / L rows it holds: beyond a few KB that costs more than the k
+    // re-split + MFMA path (1000 x 784 -> 10: 14.6 us against 9.1 + a reduce that rides in the consumer)
+    return g.chunks == 1 && g.n <= 16 && g.k >= 32 && g.k * g.n <= 4096 && g.m * g.batch >= 64 && g.m * g.batch < 16384;
+}
+
+bool dot_kernel_applies(const FusedKernel& fk, const MatMulDims& g) {
+    if (const char* e = std::getenv("DSC_MM_DOT"))
+        if (e[0] == '0') return false;
+    MatMulDims whole = g;
+    if (fk.sum_chunks) whole.chunks = 1;  // one full sum over k is what this kernel computes anyway
+    return fk.colsum_out < 0 && dot_shape(whole);
+}
+
+string gen_matmul_dot(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const MatMulDims g = matmul_dims(d);
+    const bool rows = d.output_mode == DSC_MATMUL_ROWS;
+    const int64_t batch_stride = rows ? g.n : g.m * g.n, row_stride = rows ? g.batch * g.n : g.n;
+    const int n_out = fk.has_epilogue ? fk.epilogue.raw().n_outputs : 1;
+    const int64_t N = g.n, K = g.k, blocks = (K + 3) / 4;
+    int64_t L = 4;
+    while (L < 64 && L * 2 < blocks) L *= 2;  // about two blocks per lane
+    const int64_t J = (blocks + L - 1) / L, RPW = 256 / L, total_rows = g.m * g.batch;
+    const string la = em.load_view(fk.inputs[0], d.inputs[0], {"cb", "cm", "ck"});
+    em.funcs << "DSC_INLINE float load_a(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return " << la << ";\n}\n";
+    const string lb = em.load_view(fk.inputs[1], d.inputs[1], {"cb", "ck", "cn"});
+    em.funcs << "DSC_INLINE float load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb << ";\n}\n";
+    if (fk.has_epilogue) {
+        const dsc_kernel_desc& pe = fk.epilogue.raw();
+        std::ostringstream body;
+        std::map<int, string> ov;
+        ov[fk.epilogue_product_input] = "product";
+        IndexForm form;
+        form.valid = true;
+        form.names = {"cb", "cm", "cn"};
+        form.coefs = {batch_stride, row_stride, 1};
+        form.extents = {g.batch, g.m, g.n};
+        em.emit_pe(body, pe, fk.epilogue_inputs, "gid", "e", ov, &form);
+        for (int o = 0; o < pe.n_outputs; ++o) body << "    result[" << o << "] = et" << pe.outputs[o] << ";\n";
+        em.funcs << "DSC_INLINE void mm_epilogue(float product, int gid, int cb, int cm, int cn, float* result, " << em.params_decl() << ") {\n"
+                 << body.str() << "}\n";
+    }
+    std::ostringstream k;
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
+    k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
+    // B of this workgroup's batch: [k][n], zero beyond k (a workgroup's rows may straddle two batches only when
+    // the batch has fewer rows than a workgroup, which the row -> batch split below rules out by using one batch
+    // per workgroup)
+    const int64_t wgs_per_batch = (g.m + RPW - 1) / RPW;
+    k << "    __shared__ float sB[" << S(blocks * 4 * N) << "];\n";
+    k << "    const int cb = blockIdx.x / " << S(wgs_per_batch) << ", row0 = (blockIdx.x % " << S(wgs_per_batch) << ") * " << S(RPW) << ";\n";
+    k << "    for (int e = threadIdx.x; e < " << S(blocks * 4 * N) << "; e += 256) {\n";
+    k << "        const int kk = e / " << S(N) << ", nn = e % " << S(N) << ";\n";
+    k << "        const float v = load_b(cb, min(kk, " << S(K - 1) << "), nn, " << em.params_pass() << ");\n";
+    k << "        sB[e] = kk < " << S(K) << " ? v : 0.f;\n    }\n";
+    k << "    const int lg = threadIdx.x % " << S(L) << ", cm = row0 + threadIdx.x / " << S(L) << ", cml = min(cm, " << S(g.m - 1) << ");\n";
+    // A: every block of the lane requested before anything is used; beyond k the clamped loads repeat valid
+    // elements, which meet zeros of B
+    k << "    float a[" << S(J) << "][4];\n";
+    k << "#pragma unroll\n    for (int j = 0; j < " << S(J) << "; ++j)\n#pragma unroll\n        for (int i = 0; i < 4; ++i)\n";
+    k << "            a[j][i] = load_a(cb, cml, min(4 * (lg + j * " << S(L) << ") + i, " << S(K - 1) << "), " << em.params_pass() << ");\n";
+    k << "    __syncthreads();\n";
+    k << "    float acc[" << S(N) << "];\n#pragma unroll\n    for (int n = 0; n < " << S(N) << "; ++n) acc[n] = 0.f;\n";
+    k << "#pragma unroll\n    for (int j = 0; j < " << S(J) << "; ++j) {\n";
+    k << "        const int blk = lg + j * " << S(L) << ";\n";
+    k << "        if (blk < " << S(blocks) << ") {\n";
+    k << "#pragma unroll\n            for (int i = 0; i < 4; ++i)\n#pragma unroll\n                for (int n = 0; n < " << S(N) << "; ++n)\n";
+    k << "                    acc[n] = fmaf(a[j][i], sB[(4 * blk + i) * " << S(N) << " + n], acc[n]);\n        }\n    }\n";
+    k << "#pragma unroll\n    for (int n = 0; n < " << S(N) << "; ++n)\n#pragma unroll\n        for (int s = 1; s < " << S(L) << "; s *= 2) acc[n] += __shfl_xor(acc[n], s);\n";
+    // every lane of the group now holds the row's sums; lane lg stores columns lg, lg + L, ...
+    k << "    if (cm < " << S(g.m) << ") {\n";
+    k << "#pragma unroll\n        for (int n = 0; n < " << S(N) << "; ++n)\n            if (n % " << S(L) << " == lg) {\n";
+    k << "                const int c_at = cb * " << S(batch_stride) << " + cm * " << S(row_stride) << " + n;\n";
+    if (fk.has_epilogue) {
+        k << "                float res[" << n_out << "];\n                mm_epilogue(acc[n], c_at, cb, cm, n, res, " << em.params_pass() << ");\n";
+        for (int o = 0; o < n_out; ++o) k << "                b" << fk.outputs[o] << "[c_at] = res[" << o << "];\n";
+    } else {
+        k << "                b" << fk.outputs[0] << "[c_at] = acc[n];\n";
+    }
+    k << "            }\n    }\n}\n";
+    (void)total_rows;
+    if (wgs_per_batch * g.batch >= kMaxIndex) return "matmul: grid too large";
+    out->grid = (unsigned)(wgs_per_batch * g.batch);
+    out->block = 256;
+    out->source = k.str();
+    out->note = "dot products: " + S(L) + " lanes per row, B in LDS" + (fk.has_epilogue ? " +epilogue" : "");
     return "";
 }
 
@@ -1717,6 +1833,7 @@ string gen_matmul(Emitter& em, Generated* out) {
     if (rows_kernel_applies(fk, g)) return gen_matmul_rows(em, out);
     if (smallk_kernel_applies(fk, g)) return gen_matmul_smallk(em, out);
     if (tallk_kernel_applies(fk, g)) return gen_matmul_tallk(em, out);
+    if (dot_kernel_applies(fk, g)) return gen_matmul_dot(em, out);
     MmPlan plan;
     if (!plan_mfma(fk, g, &plan, fk.as_part)) return "matmul: invalid tile configuration";
     const MmConfig c = plan.c;
@@ -1893,6 +2010,10 @@ void count_work(const FusedKernel& fk, Generated* g) {
 }  // namespace
 
 bool tallk_shape(const MatMulDims& g) { return tallk_shape_impl(g); }
+bool dot_kernel_shape(const MatMulDims& g) {
+    const char* e = std::getenv("DSC_MM_DOT");
+    return !(e && e[0] == '0') && dot_shape(g);
+}
 
 FusedKernel FusedKernel::plain(const dsc_kernel_desc& d) {
     FusedKernel fk;
@@ -1994,7 +2115,7 @@ bool can_be_part(const FusedKernel& fk) {
     if (fk.main.raw().kind != DSC_KERNEL_MATMUL) return true;
     // of the MatMul kernels, the row-per-thread, short-k and tall-k ones run 256 threads addressed by blockIdx.x
     const MatMulDims g = matmul_dims(fk.main.raw());
-    if (rows_kernel_applies(fk, g) || smallk_kernel_applies(fk, g) || tallk_kernel_applies(fk, g)) return true;
+    if (rows_kernel_applies(fk, g) || smallk_kernel_applies(fk, g) || tallk_kernel_applies(fk, g) || dot_kernel_applies(fk, g)) return true;
     if (fk.colsum_out >= 0) return false;
     // the MFMA template, when its tile choice runs four waves: small products only (large ones want their
     // workgroups persistent and the CU's whole LDS, which a shared launch cannot give them)

@@ -131,6 +131,8 @@ bool can_be_part(const FusedKernel& k);
 // Whether a MatMul of these dimensions (already split into its chunks) runs on the tall-k kernel: a small output
 // summed over a long k, one workgroup per (chunk, batch).  The schedule sizes its k re-split for that kernel.
 bool tallk_shape(const MatMulDims& g);
+// the dot-product kernel takes this product (rows x few columns over a k of moderate length)
+bool dot_kernel_shape(const MatMulDims& g);
 
 // hipRTC options every kernel is compiled with (after --offload-arch=<arch>).
 const std::vector<std::string>& compile_options();

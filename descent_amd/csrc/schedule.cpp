@@ -282,6 +282,12 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             const MatMulDims g = matmul_dims(drafts[i].fk.main.raw());
             if (g.k < 512) continue;
             if (((g.m + 63) / 64) * ((g.n + 63) / 64) * g.batch >= 128) continue;  // the tile grid is already wide
+            {
+                // rows of k-contiguous memory times a few columns: the dot-product kernel spreads k over lanes itself
+                const dsc_view& av = drafts[i].fk.main.raw().inputs[0];
+                const int64_t c0[3] = {0, 0, 0}, c1[3] = {0, 0, 1};
+                if (g.chunks == 1 && g.m >= 256 && dot_kernel_shape(g) && av.out_shape.rank == 3 && view_index(av, c1) - view_index(av, c0) == 1) continue;
+            }
             const int64_t t64 = ((g.m + 63) / 64) * ((g.n + 63) / 64) * g.batch;
             static const int64_t split_target = std::getenv("DSC_SPLIT_TARGET") ? std::atoll(std::getenv("DSC_SPLIT_TARGET")) : 4096;
             int64_t S = std::min<int64_t>(split_target / t64, g.k / 64);

@@ -37,6 +37,8 @@ MATMUL_SHAPES = [
     (20000, 64, 3), (5000, 256, 8), (70000, 16, 1),
     # small outputs over a long k: the tall-k kernel (ragged tiles, one tile, many tiles)
     (9, 16, 50000), (72, 16, 70000), (33, 50, 140000), (250, 3, 66000),
+    # few columns, a moderate number of rows: the dot-product kernel (lanes share a row's k range)
+    (1000, 10, 128), (1000, 10, 400), (300, 16, 100), (70, 3, 37), (5000, 1, 64), (64, 13, 315), (16383, 5, 33), (200, 2, 2048),
 ]
 
 
@@ -68,7 +70,7 @@ def _transposed_case(env, rng, m, n, k, ta, tb):
 
 
 @pytest.mark.parametrize("ta,tb", [(False, True), (True, False), (True, True)])
-@pytest.mark.parametrize("m,n,k", [(128, 64, 256), (100, 36, 77), (72, 16, 3000), (72, 16, 40000)])
+@pytest.mark.parametrize("m,n,k", [(128, 64, 256), (100, 36, 77), (72, 16, 3000), (72, 16, 40000), (128, 10, 400), (100, 7, 50)])
 def test_matmul_transposed_operands(hip_backend_session, ta, tb, m, n, k):
     genv, cenv = _envs(hip_backend_session)
     got = _transposed_case(genv, np.random.default_rng(5), m, n, k, ta, tb)
