@@ -467,6 +467,33 @@ def test_conv2d_gradients_over_geometries(hip_backend_session, geom, fused):
     assert rel_l2(gdf, cdf) <= TOL, (rel_l2(gdf, cdf), listing)
 
 
+def _random_conv_geometry(rng):
+    while True:
+        groups = int(rng.choice([1, 1, 2, 3, 4]))
+        c_in = groups * int(rng.choice([1, 2, 3, 4, 5, 8, 12, 16]))
+        c_out = groups * int(rng.choice([1, 2, 4, 6, 8, 10, 16, 20]))
+        fh, fw = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        pad = int(rng.integers(0, min(fh, fw) // 2 + 2))
+        h, w = int(rng.integers(max(fh, 3), 24)), int(rng.integers(max(fw, 3), 24))
+        if h + 2 * pad - fh + 1 >= 1 and w + 2 * pad - fw + 1 >= 1:
+            return (int(rng.integers(1, 40)), h, w, c_in, c_out, fh, fw, pad, groups)
+
+
+@pytest.mark.parametrize("seed", list(range(24)))
+def test_conv2d_random_geometries(hip_backend_session, seed):
+    """Seeded random convolutions (filters 1x1..5x5 not square, padding 0..3, 1-4 groups, channel counts with and without
+    16-byte pieces, images down to the filter's size): forward, data gradient and filter gradient through whatever
+    kernels the schedule picks (the dedicated forward / data-gradient kernels where they fit, the dot-product, row and
+    MFMA kernels elsewhere) against the oracle."""
+    geom = _random_conv_geometry(np.random.default_rng(4000 + seed))
+    genv, cenv = _envs(hip_backend_session, fused=True)
+    g, gy, gdx, gdf = _conv_grad_case(genv, *geom, seed=seed)
+    _, cy, cdx, cdf = _conv_grad_case(cenv, *geom, seed=seed)
+    listing = next(iter(g.__dict__["_schedules"].values())).describe()
+    for name, got, want in (("y", gy, cy), ("dx", gdx, cdx), ("df", gdf, cdf)):
+        assert rel_l2(got, want) <= TOL, (geom, name, rel_l2(got, want), listing)
+
+
 @pytest.mark.parametrize("batch,fused", [(64, True), (1000, True), (64, "graph-replay")])
 def test_overlapped_uploads_and_readbacks_match_the_serial_path(hip_backend_session, batch, fused):
     """Fourteen ConvNet steps (batch 64: steps shorter than an upload's latency; batch 1000: 3 MB uploads beside
