@@ -61,7 +61,21 @@ def time_then_profile(env, graph, steps: int, warmup: int):
     return wall
 
 
-def bench_matmul(env, m, n, k, steps, warmup):
+def verify_matmul_rows(env, w, count=64):
+    """`count` sampled rows of the product the timed launches left in C, against a float64 product of the operands
+    read back from the device: relative L2 error over those rows (the tolerance of the benchmark definition is 1e-4)."""
+    be = env.backend
+    rows = np.sort(np.random.default_rng(0).choice(w.m, min(count, w.m), replace=False))
+    b = np.frombuffer(be.read(w.b.buffer, 0, 4 * w.k * w.n), np.float32).reshape(w.k, w.n).astype(np.float64)
+    bias = np.frombuffer(be.read(w.bias.buffer, 0, 4 * w.n), np.float32).astype(np.float64)
+    a = np.stack([np.frombuffer(be.read(w.a.buffer, 4 * w.k * int(r), 4 * w.k), np.float32) for r in rows]).astype(np.float64)
+    got = np.stack([np.frombuffer(be.read(w.c.buffer, 4 * w.n * int(r), 4 * w.n), np.float32) for r in rows]).astype(np.float64)
+    z = a @ b + bias
+    want = np.where(z > 0, z, 0.01 * z)
+    return float(np.linalg.norm(got - want) / np.linalg.norm(want))
+
+
+def bench_matmul(env, m, n, k, steps, warmup, verify=False):
     from descent_amd import workloads
 
     w = workloads.matmul_epilogue(env, m, n, k, seed=2)
@@ -69,6 +83,7 @@ def bench_matmul(env, m, n, k, steps, warmup):
     avg_us, launches = env.backend.timing_query("MatMul")
     report = env.backend.timing_report(0)
     env.backend.profile_reset()
+    rel_err = verify_matmul_rows(env, w) if verify else None
     sched = next(iter(w.graph.__dict__["_schedules"].values()))
     for p in (w.a, w.b, w.bias, w.c):
         if p.buffer is not None:
@@ -85,6 +100,7 @@ def bench_matmul(env, m, n, k, steps, warmup):
         "tflops_kernel": (w.flops / (avg_us * 1e-6) / 1e12) if avg_us else None,
         "launches_per_step": sched.launch_count()[0],
         "report": report,
+        "rel_l2_error_sampled_rows": rel_err,
     }
 
 
@@ -356,8 +372,12 @@ def main():
         sys.stderr.write(r.pop("report"))
         print(json.dumps(r))
         return
-    head = bench_matmul(env, n, n, n, args.steps, args.warmup)
+    head = bench_matmul(env, n, n, n, args.steps, args.warmup, verify=True)
     sys.stderr.write(head["report"])
+    if not head["rel_l2_error_sampled_rows"] <= 1e-4:
+        print("bench.py: the timed product is wrong: relative L2 error %r on 64 sampled rows against float64"
+              % head["rel_l2_error_sampled_rows"], file=sys.stderr)
+        sys.exit(1)
 
     extra = {}
     if args.all:
@@ -424,6 +444,9 @@ def main():
             "algorithmic_flops_per_launch": head["flops"],
         },
         "cpu_baseline": cpu,
+        # 64 sampled rows of the C the timed launches wrote, against a float64 product of the operands read back
+        "verified": True,
+        "rel_l2_error_sampled_rows": head["rel_l2_error_sampled_rows"],
     }
     if extra:
         line["extra"] = extra
