@@ -20,7 +20,33 @@ struct dsc_schedule {
     Schedule s;
 };
 
+// Device memory for the intermediates of dsc_schedule_run_static.  It is part of this library's device code, so
+// every GPU the library runs on holds its own copy from the first use of the library there until the process ends,
+// and using it needs no allocation.  In host code this name only stands for the array (it is what
+// hipGetSymbolAddress looks up); the array's device address on a GPU is what scratch_address() stores per device.
+static __device__ __align__(256) unsigned char scratch[DSC_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+char* g_scratch_ptr[kMaxDevices];  // per device: its copy's address, once resolved
+
+// Resolves (once per device) the address of `device`'s copy of the scratch array.  `device` must be current.
+hipError_t scratch_address(int device, char** out) {
+    *out = nullptr;
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    if (!g_scratch_ptr[device]) {
+        void* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return e;
+        }
+        g_scratch_ptr[device] = static_cast<char*>(p);
+    }
+    *out = g_scratch_ptr[device];
+    return hipSuccess;
+}
 
 char* dup_string(const std::string& s) {
     char* out = static_cast<char*>(std::malloc(s.size() + 1));
@@ -90,6 +116,10 @@ int dsc_ctx_create(int device_ordinal, dsc_ctx** out) {
         delete ctx;
         return fail(DSC_ERR_HIP, std::string("hipStreamCreate: ") + hipGetErrorString(e));
     }
+    // this device's copy of the static scratch array (the device is current here); a failure only disables
+    // dsc_schedule_run_static, which then reports it
+    e = scratch_address(device_ordinal, &c.static_scratch);
+    if (e != hipSuccess) c.static_scratch_error = std::string("hipGetSymbolAddress(scratch): ") + hipGetErrorString(e);
     {
         void* cell = nullptr;
         e = hipMalloc(&cell, 256);
@@ -554,6 +584,28 @@ int dsc_schedule_run(dsc_ctx* ctx, dsc_schedule* s, dsc_buf* params, uint32_t ra
     for (int i = 0; i < s->s.n_params; ++i)
         if (params[i]) c->heap.touch(params[i], c->work_seq);
     return mark_stream(c);
+}
+
+int dsc_schedule_run_static(dsc_ctx* ctx, dsc_schedule* s, dsc_buf* params, dsc_buf* spare, uint32_t rand_seed) {
+    if (!ctx || !s || !params || !spare) return fail(DSC_ERR_INVALID, "null argument");
+    Context* c = &ctx->c;
+    if (c->offline) return fail(DSC_ERR_NO_DEVICE, "static run without a device");
+    if (!c->static_scratch) return fail(DSC_ERR_HIP, "static run: the scratch array has no address on this device: " + c->static_scratch_error);
+    if (c->profiling) return fail(DSC_ERR_UNSUPPORTED, "static run: per-launch timing is on (it creates events); dsc_prof_enable(ctx, 0) first");
+    if (s->s.graph_replay) return fail(DSC_ERR_UNSUPPORTED, "static run: the schedule was created with DSC_SCHEDULE_GRAPH_REPLAY (instantiating a graph allocates)");
+    // copies on the second stream enqueued so far come first (waits on their existing events; nothing is created)
+    int rc = join_copies(c);
+    if (rc != DSC_OK) return rc;
+    ++c->work_seq;
+    rc = s->s.run_static(c, params, spare, rand_seed, c->static_scratch, DSC_STATIC_SCRATCH_BYTES);
+    if (rc != DSC_OK || !c->async_io) return rc;
+    // use stamps for later uploads on the copy stream.  dsc_schedule_run also records an event here; this call leaves
+    // that to the next upload that needs one (copy_stream_wait records a mark when none covers a buffer's stamp)
+    for (int i = 0; i < s->s.n_params; ++i) {
+        if (params[i]) c->heap.touch(params[i], c->work_seq);
+        if (spare[i]) c->heap.touch(spare[i], c->work_seq);
+    }
+    return DSC_OK;
 }
 
 int dsc_schedule_launch_count(const dsc_schedule* s, int32_t* out_launches, int32_t* out_clusters) {

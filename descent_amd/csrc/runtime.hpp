@@ -146,6 +146,11 @@ struct Context {
     int (*range_push)(const char*) = nullptr;
     int (*range_pop)() = nullptr;
 
+    // this device's copy of the library's static scratch array (dsc_schedule_run_static); null when its address
+    // could not be resolved, with the reason in static_scratch_error
+    char* static_scratch = nullptr;
+    std::string static_scratch_error;
+
     bool profiling = false;
     std::vector<ProfileEntry> profile;
     std::vector<hipEvent_t> event_pool;

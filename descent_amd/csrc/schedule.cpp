@@ -1732,6 +1732,209 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
     return DSC_OK;
 }
 
+namespace {
+
+// Offsets inside a fixed region: first fit over the free ranges in address order, 256-byte granules, neighbours merged
+// on release.  Host-side bookkeeping only.
+class RegionPlanner {
+  public:
+    explicit RegionPlanner(size_t bytes) { free_[0] = bytes; }
+    bool take(size_t bytes, size_t* offset) {
+        const size_t need = std::max<size_t>(DeviceHeap::kAlign, (bytes + DeviceHeap::kAlign - 1) / DeviceHeap::kAlign * DeviceHeap::kAlign);
+        for (auto it = free_.begin(); it != free_.end(); ++it) {
+            if (it->second < need) continue;
+            *offset = it->first;
+            const size_t rest = it->second - need;
+            free_.erase(it);
+            if (rest) free_[*offset + need] = rest;
+            in_use_ += need;
+            return true;
+        }
+        return false;
+    }
+    void give(size_t offset, size_t bytes) {
+        size_t size = std::max<size_t>(DeviceHeap::kAlign, (bytes + DeviceHeap::kAlign - 1) / DeviceHeap::kAlign * DeviceHeap::kAlign);
+        in_use_ -= size;
+        auto next = free_.lower_bound(offset);
+        if (next != free_.end() && offset + size == next->first) {
+            size += next->second;
+            next = free_.erase(next);
+        }
+        if (next != free_.begin()) {
+            auto prev = std::prev(next);
+            if (prev->first + prev->second == offset) {
+                prev->second += size;
+                return;
+            }
+        }
+        free_[offset] = size;
+    }
+    size_t in_use() const { return in_use_; }
+
+  private:
+    std::map<size_t, size_t> free_;  // offset -> size
+    size_t in_use_ = 0;
+};
+
+}  // namespace
+
+int Schedule::run_static(Context* ctx, dsc_buf* params, dsc_buf* spare, uint32_t rand_seed, char* scratch, size_t scratch_bytes) {
+    // Environment::run's bookkeeping (environment.rs:326-516) with the allocator taken out: where run() asks the heap,
+    // a node that ends up as a parameter's new value is placed in the caller's spare buffer of that slot, and every
+    // other node at an offset of `scratch`.  A buffer that one node hands to the next (ScatterAdd accumulators) is
+    // placed once, where the last node of that chain needs it.
+    enum Where { kNone = 0, kParam, kSpare, kScratch };
+    struct Place {
+        Where where = kNone;
+        void* ptr = nullptr;
+        int slot = -1;      // kParam / kSpare
+        size_t offset = 0;  // kScratch
+        size_t bytes = 0;
+    };
+    std::vector<int> usage(n_nodes, 0), out_slot(n_nodes, -1), successor(n_nodes, -1);
+    std::vector<Place> place(n_nodes);
+    for (auto& st : steps) {
+        for (int n : st.inputs) usage[n] += 1;
+        for (auto& o : st.outputs)
+            if (o.copy_from >= 0) successor[o.copy_from] = o.node;
+    }
+    for (auto& io : outputs) {
+        usage[io.node] += 1;
+        if (out_slot[io.node] >= 0) return fail(DSC_ERR_UNSUPPORTED, "static run: one node is the new value of two parameters");
+        out_slot[io.node] = io.param;
+    }
+    std::vector<bool> param_is_output(n_params, false), spare_taken(n_params, false);
+    for (auto& io : outputs) param_is_output[io.param] = true;
+    for (auto& io : inputs) {
+        void* p = nullptr;
+        size_t have = 0;
+        if (params[io.param] == 0 || !ctx->heap.info(params[io.param], &p, &have))
+            return fail(DSC_ERR_INVALID, "static run: an input parameter has no buffer");
+        if (have < node_bytes[io.node]) return fail(DSC_ERR_INVALID, "static run: an input parameter's buffer is smaller than the parameter");
+        place[io.node] = Place{kParam, p, io.param, 0, have};
+        if (!param_is_output[io.param]) usage[io.node] += 1;  // the parameter keeps its buffer
+    }
+
+    RegionPlanner region(scratch_bytes);
+    size_t peak = 0;
+    std::string error;
+    // where a node that nothing hands a buffer to gets its memory
+    auto settle_node = [&](int node) -> bool {
+        int slot = -1;
+        for (int n = node; n >= 0 && slot < 0; n = successor[n]) slot = out_slot[n];
+        Place pl;
+        pl.bytes = node_bytes[node];
+        if (slot >= 0) {
+            void* p = nullptr;
+            size_t have = 0;
+            if (spare[slot] == 0 || !ctx->heap.info(spare[slot], &p, &have)) {
+                error = "static run: parameter slot " + std::to_string(slot) + " is written and has no spare buffer";
+                return false;
+            }
+            if (spare[slot] == params[slot] || spare_taken[slot] || have < node_bytes[node]) {
+                error = "static run: the spare buffer of parameter slot " + std::to_string(slot) +
+                        (have < node_bytes[node] ? " is smaller than the parameter" : " is the parameter's own buffer or is used twice");
+                return false;
+            }
+            spare_taken[slot] = true;
+            pl.where = kSpare;
+            pl.ptr = p;
+            pl.slot = slot;
+        } else {
+            if (!region.take(pl.bytes, &pl.offset)) {
+                error = "static run: an intermediate of " + std::to_string(pl.bytes) + " bytes does not fit beside the " +
+                        std::to_string(region.in_use()) + " bytes of intermediates alive at that point; the static scratch array holds " +
+                        std::to_string(scratch_bytes) + " bytes (dsc_schedule_run has no such limit)";
+                return false;
+            }
+            peak = std::max(peak, region.in_use());
+            pl.where = kScratch;
+            pl.ptr = scratch + pl.offset;
+        }
+        place[node] = pl;
+        return true;
+    };
+    auto settle = [&](int node) -> int {
+        if (settle_node(node)) return DSC_OK;
+        return fail(error.find("does not fit") != std::string::npos ? DSC_ERR_UNSUPPORTED : DSC_ERR_INVALID, error);
+    };
+
+    struct Launch {
+        Kernel* kernel;
+        size_t first;
+        int n;
+    };
+    std::vector<Launch> launches;
+    std::vector<void*> pointers;
+    launches.reserve(steps.size() + 4);
+    std::vector<Place> prefilled(prefills.empty() ? 0 : n_nodes);
+    for (auto& pf : prefills) {
+        launches.push_back(Launch{pf.kernel, pointers.size(), (int)pf.nodes.size()});
+        for (int node : pf.nodes) {
+            if (int rc = settle(node)) return rc;
+            prefilled[node] = place[node];
+            place[node] = Place{};
+            pointers.push_back(prefilled[node].ptr);
+        }
+    }
+    for (auto& st : steps) {
+        for (int n : st.inputs) usage[n] -= 1;
+        for (auto& o : st.outputs) {
+            if (place[o.node].where != kNone) return fail(DSC_ERR_INVALID, "static run: node written twice");
+            if (o.copy_from < 0) {
+                if (int rc = settle(o.node)) return rc;
+                continue;
+            }
+            if (usage[o.copy_from] != 0) return fail(DSC_ERR_UNSUPPORTED, "static run: accumulator source still in use (deep copy)");
+            if (place[o.copy_from].where != kNone) {
+                place[o.node] = place[o.copy_from];
+                place[o.copy_from] = Place{};
+            } else if (o.from_literal && !prefilled.empty() && prefilled[o.node].where != kNone) {
+                place[o.node] = prefilled[o.node];
+                prefilled[o.node] = Place{};
+            } else if (o.from_literal) {
+                if (int rc = settle(o.node)) return rc;
+                launches.push_back(Launch{o.fill, pointers.size(), 1});
+                pointers.push_back(place[o.node].ptr);
+            } else {
+                return fail(DSC_ERR_INVALID, "static run: cannot copy-on-write node");
+            }
+        }
+        const int n = (int)st.params.size();
+        launches.push_back(Launch{st.kernel, pointers.size(), n});
+        for (int i = 0; i < n; ++i) {
+            const Place& pl = place[st.params[i]];
+            if (pl.where == kNone)
+                return fail(DSC_ERR_INVALID, "static run: node " + std::to_string(st.params[i]) + " has no buffer at '" + st.kernel->label + "'");
+            pointers.push_back(pl.ptr);
+        }
+        for (int nd : st.inputs) {
+            if (usage[nd] != 0 || place[nd].where == kNone) continue;
+            if (place[nd].where == kScratch) region.give(place[nd].offset, place[nd].bytes);
+            place[nd] = Place{};  // a parameter's old buffer stays with the caller
+        }
+    }
+    // every written parameter must have landed in its own slot's spare, or still sit in its own buffer (updated in
+    // place): anything else would hand a caller's buffer to another slot
+    for (auto& io : outputs) {
+        const Place& pl = place[io.node];
+        const bool in_spare = pl.where == kSpare && pl.slot == io.param;
+        const bool in_place = pl.where == kParam && pl.slot == io.param;
+        if (!in_spare && !in_place)
+            return fail(DSC_ERR_UNSUPPORTED, "static run: parameter slot " + std::to_string(io.param) +
+                                                 " would receive another parameter's buffer; use dsc_schedule_run for this graph");
+    }
+
+    for (auto& l : launches) {
+        int rc = launch_kernel(ctx, l.kernel, pointers.data() + l.first, l.n, rand_seed);
+        if (rc != DSC_OK) return rc;
+    }
+    for (auto& io : outputs)
+        if (place[io.node].where == kSpare) std::swap(params[io.param], spare[io.param]);
+    static_peak_bytes = std::max(static_peak_bytes, peak);
+    return DSC_OK;
+}
+
 Schedule::~Schedule() {
     for (auto& c : captured)
         if (c.exec) (void)hipGraphExecDestroy(c.exec);
@@ -1751,6 +1954,7 @@ std::string Schedule::describe() const {
     o << launches_per_run() << " launches for " << n_clusters << " clusters\n";
     if (replays + direct_runs + (int64_t)captured.size() > 0)
         o << "# graph replays " << replays << ", captured " << captured.size() << ", direct runs " << direct_runs << "\n";
+    if (static_peak_bytes) o << "# static runs: at most " << static_peak_bytes << " bytes of the scratch array in use at once\n";
     for (auto& pf : prefills)
         o << "prefill: " << pf.kernel->label << "  grid " << pf.kernel->gen.grid << "x" << pf.kernel->gen.block << " (" << pf.nodes.size()
           << " literal-initialised accumulators)\n";

@@ -33,6 +33,7 @@ struct Schedule {
     static constexpr size_t kMaxCaptured = 8;
     std::vector<CapturedStep> captured;
     int64_t replays = 0, direct_runs = 0;
+    size_t static_peak_bytes = 0;  // most scratch a run_static of this schedule has had in use at once
     bool graph_replay = false;  // DSC_SCHEDULE_GRAPH_REPLAY
     ~Schedule();
 
@@ -50,6 +51,9 @@ struct Schedule {
 
     int build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags);
     int run(Context* ctx, dsc_buf* params, uint32_t rand_seed);
+    // The same launches with every intermediate inside `scratch` (a fixed device array of `scratch_bytes`) and every
+    // written parameter in the caller's `spare` buffer of its slot: no device allocation, no heap traffic.
+    int run_static(Context* ctx, dsc_buf* params, dsc_buf* spare, uint32_t rand_seed, char* scratch, size_t scratch_bytes);
     std::string describe() const;
     // The schedule after fusion as a graphviz digraph (the reference exports its graph before scheduling,
     // src/graph.rs:656-760): one box per launch, one ellipse per parameter slot, one edge per buffer.

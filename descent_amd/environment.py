@@ -228,6 +228,32 @@ class Environment:
         else:
             self._run_cluster_by_cluster(graph, rand_seed)
 
+    def run_static(self, graph: Graph, rand_seed: int) -> None:
+        """`run` through dsc_schedule_run_static: the step's intermediates live in the library's fixed scratch array
+        and every parameter the graph writes alternates between its buffer and one spare buffer, allocated here the
+        first time the parameter is written this way -- after that a step allocates no device memory at all."""
+        rand_seed &= 0xFFFFFFFF
+        key = (id(self.backend), self.fused)
+        cache = graph.__dict__.setdefault("_schedules", {})
+        sched = cache.get(key)
+        if sched is None:
+            sched = cache[key] = self.backend.make_schedule(graph, self.fused)
+        written = set(sched.written_slots())
+        spare = []
+        for i, p in enumerate(sched.params):
+            p.checked(self)
+            if i in written:
+                if p.__dict__.get("spare") is None:
+                    p.spare = self.backend.alloc(p.shape.buffer_size())
+                spare.append(p.spare)
+            else:
+                spare.append(None)
+        handles, spare = sched.run_static([p.buffer for p in sched.params], spare, rand_seed)
+        for i, (p, h) in enumerate(zip(sched.params, handles)):
+            p.buffer = h
+            if i in written:
+                p.spare = spare[i]
+
     def _run_cluster_by_cluster(self, graph: Graph, rand_seed: int) -> None:
         be = self.backend
         ops = graph.ops

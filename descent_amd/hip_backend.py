@@ -73,6 +73,7 @@ def lib():
         "dsc_schedule_create": (C.c_int, [vp, C.POINTER(_abi.CScheduleDesc), u32, C.POINTER(vp)]),
         "dsc_schedule_destroy": (C.c_int, [vp, vp]),
         "dsc_schedule_run": (C.c_int, [vp, vp, C.POINTER(u64), u32]),
+        "dsc_schedule_run_static": (C.c_int, [vp, vp, C.POINTER(u64), C.POINTER(u64), u32]),
         "dsc_schedule_launch_count": (C.c_int, [vp, C.POINTER(i32), C.POINTER(i32)]),
         "dsc_schedule_describe": (C.c_int, [vp, C.POINTER(vp)]),
         "dsc_schedule_dot": (C.c_int, [vp, C.POINTER(vp)]),
@@ -98,7 +99,7 @@ EXPORTED_SYMBOLS = [
     "dsc_buf_read", "dsc_buf_alloc_io", "dsc_host_alloc", "dsc_host_free", "dsc_buf_write_async", "dsc_buf_read_async", "dsc_kernel_get", "dsc_kernel_buffer_count", "dsc_kernel_reference_group_count",
     "dsc_kernel_label", "dsc_kernel_source", "dsc_kernel_launch", "dsc_codegen_source", "dsc_codegen_compile",
     "dsc_codegen_check_schedule", "dsc_free_string", "dsc_schedule_create", "dsc_schedule_destroy",
-    "dsc_schedule_run", "dsc_schedule_launch_count", "dsc_schedule_describe", "dsc_schedule_dot", "dsc_prof_markers", "dsc_prof_enable", "dsc_prof_reset",
+    "dsc_schedule_run", "dsc_schedule_run_static", "dsc_schedule_launch_count", "dsc_schedule_describe", "dsc_schedule_dot", "dsc_prof_markers", "dsc_prof_enable", "dsc_prof_reset",
     "dsc_prof_report", "dsc_prof_query", "dsc_prof_work",
 ]
 
@@ -164,6 +165,21 @@ class HipSchedule:
             self._slots[i] = h or 0
         check(lib().dsc_schedule_run(self._backend._ctx, self._handle, self._slots, rand_seed & 0xFFFFFFFF))
         return [self._slots[i] or None for i in range(len(handles))]
+
+    def run_static(self, handles: List[int], spare: List[int], rand_seed: int):
+        """dsc_schedule_run_static: no device allocation; every written parameter goes into its slot's spare buffer and
+        the two swap.  Returns (handles, spare) after the call."""
+        spares = (C.c_uint64 * max(1, len(self.params)))()
+        for i, h in enumerate(handles):
+            self._slots[i] = h or 0
+            spares[i] = spare[i] or 0
+        check(lib().dsc_schedule_run_static(self._backend._ctx, self._handle, self._slots, spares, rand_seed & 0xFFFFFFFF))
+        return [self._slots[i] or None for i in range(len(handles))], [spares[i] or None for i in range(len(handles))]
+
+    def written_slots(self) -> List[int]:
+        """Parameter slots a run writes (they need a spare buffer for run_static)."""
+        d = self._ms.desc
+        return sorted({d.outputs[i].param for i in range(d.n_outputs)})
 
     def launch_count(self):
         a, b = C.c_int32(), C.c_int32()

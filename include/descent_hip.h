@@ -335,6 +335,31 @@ int dsc_schedule_destroy(dsc_ctx* ctx, dsc_schedule* s);
 /* Environment::run (environment.rs:326-516). `params[slot]` holds each parameter's current buffer (0 if
  * none) and is updated in place with the buffers the run leaves in the parameters. */
 int dsc_schedule_run(dsc_ctx* ctx, dsc_schedule* s, dsc_buf* params, uint32_t rand_seed);
+/*
+ * dsc_schedule_run for callers that cannot allocate device memory (code under HIP-graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose run allocates every
+ * cluster output from the BufferHeap as it goes (environment.rs:404-444).
+ *
+ * Same work, same kernels and same results as dsc_schedule_run, but no hipMalloc / hipFree and no call into the
+ * library's heap: every intermediate of the run is placed in a fixed array of DSC_STATIC_SCRATCH_BYTES that is part
+ * of the library's device code (each GPU the library runs on holds its own copy from first use until the process
+ * ends), and every parameter the run writes goes into a buffer the caller provides:
+ *   params[slot]  the current buffer of every parameter, as for dsc_schedule_run;
+ *   spare[slot]   for every slot the schedule writes: a caller-owned buffer, different from params[slot], of at
+ *                 least the parameter's size; slots the schedule only reads are ignored (0 is fine).
+ * On success the two are swapped for every written slot: params[slot] holds the new value and spare[slot] the
+ * buffer the old value was in, ready to be the spare of the next call (a parameter that the run updates in place,
+ * by ScatterAdd into its own buffer, keeps its buffer; its spare is left alone).  Nothing is freed.
+ *
+ * A run whose intermediates do not fit the array at once is refused with DSC_ERR_UNSUPPORTED before anything is
+ * enqueued (the message names the size that did not fit); so are a context with per-launch timing on
+ * (dsc_prof_enable creates events) and DSC_SCHEDULE_GRAPH_REPLAY schedules.  All calls on one GPU share
+ * that GPU's array and it keeps the last call's contents: the schedule's own Fill launches clear what has to start
+ * at zero, and two calls whose work overlaps on one GPU (two contexts, two streams) race -- finish one
+ * (dsc_ctx_sync / a fence) before another context starts the next.
+ */
+#define DSC_STATIC_SCRATCH_BYTES (64u << 20)
+int dsc_schedule_run_static(dsc_ctx* ctx, dsc_schedule* s, dsc_buf* params, dsc_buf* spare, uint32_t rand_seed);
 /* Number of device kernels one run launches after fusion, and the reference cluster count. */
 int dsc_schedule_launch_count(const dsc_schedule* s, int32_t* out_launches, int32_t* out_clusters);
 /* Text listing of the post-fusion schedule (reference: Graph::write_dot, graph.rs:661-763). Caller releases
