@@ -552,6 +552,14 @@ int dsc_codegen_check_schedule(const dsc_schedule_desc* desc, uint32_t flags, co
 
 void dsc_free_string(char* s) { std::free(s); }
 
+int dsc_cache_stats(int64_t* out_hits, int64_t* out_compiles, int64_t* out_rejected) {
+    const CacheStats& st = cache_stats();
+    if (out_hits) *out_hits = st.hits;
+    if (out_compiles) *out_compiles = st.compiles;
+    if (out_rejected) *out_rejected = st.rejected;
+    return DSC_OK;
+}
+
 int dsc_schedule_create(dsc_ctx* ctx, const dsc_schedule_desc* desc, uint32_t flags, dsc_schedule** out) {
     if (!ctx || !desc || !out) return fail(DSC_ERR_INVALID, "null argument");
     *out = nullptr;

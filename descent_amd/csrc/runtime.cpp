@@ -239,6 +239,8 @@ Context::~Context() {
 
 namespace {
 
+CacheStats g_cache_stats;
+
 uint64_t fnv1a(const std::string& s, uint64_t seed) {
     uint64_t h = seed;
     for (unsigned char c : s) {
@@ -268,28 +270,110 @@ std::string cache_dir() {
     return dir;
 }
 
+// What a cached object depends on besides its source: the target, the compile options, the compiler (hipRTC) and
+// runtime versions, and the layout of the cache file itself.
+std::string cache_salt(const std::string& arch) {
+    std::string salt = arch;
+    for (auto& o : compile_options()) salt += "|" + o;
+    int rtc_major = 0, rtc_minor = 0, runtime = 0;
+    (void)hiprtcVersion(&rtc_major, &rtc_minor);
+    if (hipRuntimeGetVersion(&runtime) != hipSuccess) (void)hipGetLastError();
+    salt += "|hiprtc " + std::to_string(rtc_major) + "." + std::to_string(rtc_minor) + "|hip " + std::to_string(runtime) + "|file v2";
+    return salt;
+}
+
 std::string cache_path(const std::string& source, const std::string& arch) {
     const std::string dir = cache_dir();
     if (dir.empty()) return "";
-    std::string salt = arch;
-    for (auto& o : compile_options()) salt += "|" + o;
+    const std::string salt = cache_salt(arch);
     char name[64];
     std::snprintf(name, sizeof name, "%016llx%016llx.co", (unsigned long long)fnv1a(source + salt, 1469598103934665603ull),
                   (unsigned long long)fnv1a(salt + source, 0x9e3779b97f4a7c15ull));
     return dir + "/" + name;
 }
 
+// Cache file = 24-byte header (magic, payload length, FNV-1a of the payload) + the code object.  A file is used only
+// if the header matches what follows it and the payload is an AMDGPU ELF image; anything else (a truncated write, a
+// file from another tool, bit rot) is deleted and counted as rejected.
+constexpr char kCacheMagic[8] = {'D', 'S', 'C', 'C', 'O', 'B', 'J', '2'};
+constexpr size_t kCacheHeader = 24;
+
+uint64_t fnv1a_bytes(const char* p, size_t n) {
+    uint64_t h = 1469598103934665603ull;
+    for (size_t i = 0; i < n; ++i) {
+        h ^= (unsigned char)p[i];
+        h *= 1099511628211ull;
+    }
+    return h;
+}
+
+bool plausible_code_object(const char* p, size_t n) {
+    // ELF64 little-endian, e_machine EM_AMDGPU (224), section header table inside the file
+    if (n < 64 || std::memcmp(p, "\177ELF", 4) != 0 || p[4] != 2 || p[5] != 1) return false;
+    uint16_t machine, shentsize, shnum;
+    uint64_t shoff;
+    std::memcpy(&machine, p + 18, 2);
+    std::memcpy(&shoff, p + 40, 8);
+    std::memcpy(&shentsize, p + 58, 2);
+    std::memcpy(&shnum, p + 60, 2);
+    if (machine != 224) return false;
+    return shoff <= n && (uint64_t)shentsize * shnum <= n - shoff;
+}
+
+bool read_cache_file(const std::string& path, std::vector<char>* code) {
+    std::ifstream f(path, std::ios::binary);
+    if (!f) return false;
+    std::vector<char> all((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+    uint64_t length = 0, hash = 0;
+    bool ok = all.size() > kCacheHeader && std::memcmp(all.data(), kCacheMagic, 8) == 0;
+    if (ok) {
+        std::memcpy(&length, all.data() + 8, 8);
+        std::memcpy(&hash, all.data() + 16, 8);
+        ok = length == all.size() - kCacheHeader && hash == fnv1a_bytes(all.data() + kCacheHeader, (size_t)length) &&
+             plausible_code_object(all.data() + kCacheHeader, (size_t)length);
+    }
+    if (!ok) {
+        f.close();
+        std::remove(path.c_str());
+        ++g_cache_stats.rejected;
+        return false;
+    }
+    code->assign(all.begin() + kCacheHeader, all.end());
+    return true;
+}
+
+void write_cache_file(const std::string& path, const std::vector<char>& code) {
+    const std::string tmp = path + ".tmp" + std::to_string((long long)::getpid());
+    std::ofstream f(tmp, std::ios::binary);
+    if (!f) return;
+    const uint64_t length = code.size(), hash = fnv1a_bytes(code.data(), code.size());
+    f.write(kCacheMagic, 8);
+    f.write(reinterpret_cast<const char*>(&length), 8);
+    f.write(reinterpret_cast<const char*>(&hash), 8);
+    f.write(code.data(), (std::streamsize)code.size());
+    f.close();
+    if (!f || std::rename(tmp.c_str(), path.c_str()) != 0) std::remove(tmp.c_str());
+}
+
 }  // namespace
 
-int compile_source(const std::string& source, const std::string& arch, std::vector<char>* code, std::string* log) {
+const CacheStats& cache_stats() { return g_cache_stats; }
+
+void drop_cached_object(const std::string& source, const std::string& arch) {
     const std::string path = cache_path(source, arch);
-    if (!path.empty()) {
-        std::ifstream f(path, std::ios::binary);
-        if (f) {
-            code->assign(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
-            if (!code->empty()) return DSC_OK;
-        }
+    if (path.empty()) return;
+    if (std::remove(path.c_str()) == 0) ++g_cache_stats.rejected;
+}
+
+int compile_source(const std::string& source, const std::string& arch, std::vector<char>* code, std::string* log, bool* from_cache) {
+    if (from_cache) *from_cache = false;
+    const std::string path = cache_path(source, arch);
+    if (!path.empty() && read_cache_file(path, code)) {
+        ++g_cache_stats.hits;
+        if (from_cache) *from_cache = true;
+        return DSC_OK;
     }
+    ++g_cache_stats.compiles;
     hiprtcProgram prog;
     if (hiprtcCreateProgram(&prog, source.c_str(), "dsc_kernel.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
         return fail(DSC_ERR_COMPILE, "hiprtcCreateProgram failed");
@@ -313,17 +397,27 @@ int compile_source(const std::string& source, const std::string& arch, std::vect
     code->resize(code_size);
     hiprtcGetCode(prog, code->data());
     hiprtcDestroyProgram(&prog);
-    if (!path.empty()) {
-        const std::string tmp = path + ".tmp" + std::to_string((long long)::getpid());
-        std::ofstream f(tmp, std::ios::binary);
-        if (f) {
-            f.write(code->data(), (std::streamsize)code->size());
-            f.close();
-            if (std::rename(tmp.c_str(), path.c_str()) != 0) std::remove(tmp.c_str());
-        }
-    }
+    if (!path.empty()) write_cache_file(path, *code);
     return DSC_OK;
 }
+
+namespace {
+
+// Loads a code object and looks up the entry point.
+hipError_t load_module(const std::vector<char>& code, const std::string& entry, hipModule_t* module, hipFunction_t* function, const char** what) {
+    *what = "hipModuleLoadData";
+    hipError_t e = hipModuleLoadData(module, code.data());
+    if (e != hipSuccess) return e;
+    *what = "hipModuleGetFunction";
+    e = hipModuleGetFunction(function, *module, entry.c_str());
+    if (e != hipSuccess) {
+        (void)hipModuleUnload(*module);
+        *module = nullptr;
+    }
+    return e;
+}
+
+}  // namespace
 
 Kernel* get_kernel(Context* ctx, const FusedKernel& fk, int* status) {
     const std::string key = fk.key();
@@ -373,7 +467,8 @@ Kernel* get_kernel(Context* ctx, const FusedKernel& fk, int* status) {
     }
     std::vector<char> code;
     std::string log;
-    int rc = compile_source(k->gen.source, ctx->arch, &code, &log);
+    bool from_cache = false;
+    int rc = compile_source(k->gen.source, ctx->arch, &code, &log, &from_cache);
     if (rc != DSC_OK) {
         *status = rc;
         return nullptr;
@@ -384,14 +479,21 @@ Kernel* get_kernel(Context* ctx, const FusedKernel& fk, int* status) {
         *status = DSC_OK;
         return raw_offline;
     }
-    hipError_t e = hipModuleLoadData(&k->module, code.data());
-    if (e != hipSuccess) {
-        *status = fail(DSC_ERR_HIP, std::string("hipModuleLoadData: ") + hipGetErrorString(e));
-        return nullptr;
+    const char* what = "";
+    hipError_t e = load_module(code, k->gen.entry, &k->module, &k->function, &what);
+    if (e != hipSuccess && from_cache) {
+        // the cached object passed the file checks and the runtime still refuses it: drop it and compile afresh, once
+        (void)hipGetLastError();
+        drop_cached_object(k->gen.source, ctx->arch);
+        rc = compile_source(k->gen.source, ctx->arch, &code, &log, &from_cache);
+        if (rc != DSC_OK) {
+            *status = rc;
+            return nullptr;
+        }
+        e = load_module(code, k->gen.entry, &k->module, &k->function, &what);
     }
-    e = hipModuleGetFunction(&k->function, k->module, k->gen.entry.c_str());
     if (e != hipSuccess) {
-        *status = fail(DSC_ERR_HIP, std::string("hipModuleGetFunction: ") + hipGetErrorString(e));
+        *status = fail(DSC_ERR_HIP, std::string(what) + ": " + hipGetErrorString(e));
         return nullptr;
     }
     if (k->gen.persistent_ok) {

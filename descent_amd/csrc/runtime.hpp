@@ -175,7 +175,15 @@ Kernel* get_kernel(Context* ctx, const FusedKernel& fk, int* status);
 int launch_kernel(Context* ctx, Kernel* k, void* const* device_ptrs, int n, uint32_t rand_seed);
 // Makes `rand_seed` the seed seen by launches enqueued after this call.
 int set_seed(Context* ctx, uint32_t rand_seed);
-// hipRTC compile without a device.
-int compile_source(const std::string& source, const std::string& arch, std::vector<char>* code, std::string* log);
+// Code object for `source`: from the on-disk cache when a valid file is there (then *from_cache is set), else compiled
+// with hipRTC (no device needed) and written to the cache.
+int compile_source(const std::string& source, const std::string& arch, std::vector<char>* code, std::string* log, bool* from_cache = nullptr);
+// Deletes the cache file of `source` (after the runtime refused to load what it held).
+void drop_cached_object(const std::string& source, const std::string& arch);
+// Process-wide counters of the on-disk cache: files used, hipRTC compilations, files refused and deleted.
+struct CacheStats {
+    int64_t hits = 0, compiles = 0, rejected = 0;
+};
+const CacheStats& cache_stats();
 
 }  // namespace dsc

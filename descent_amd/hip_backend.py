@@ -70,6 +70,7 @@ def lib():
         "dsc_codegen_compile": (C.c_int, [C.POINTER(_abi.CKernelDesc), C.c_char_p, C.POINTER(sz)]),
         "dsc_codegen_check_schedule": (C.c_int, [C.POINTER(_abi.CScheduleDesc), u32, C.c_char_p, C.POINTER(vp)]),
         "dsc_free_string": (None, [vp]),
+        "dsc_cache_stats": (C.c_int, [C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
         "dsc_schedule_create": (C.c_int, [vp, C.POINTER(_abi.CScheduleDesc), u32, C.POINTER(vp)]),
         "dsc_schedule_destroy": (C.c_int, [vp, vp]),
         "dsc_schedule_run": (C.c_int, [vp, vp, C.POINTER(u64), u32]),
@@ -98,7 +99,7 @@ EXPORTED_SYMBOLS = [
     "dsc_buf_alloc", "dsc_buf_free", "dsc_buf_info", "dsc_heap_stats", "dsc_buf_write", "dsc_buf_fill_zero",
     "dsc_buf_read", "dsc_buf_alloc_io", "dsc_host_alloc", "dsc_host_free", "dsc_buf_write_async", "dsc_buf_read_async", "dsc_kernel_get", "dsc_kernel_buffer_count", "dsc_kernel_reference_group_count",
     "dsc_kernel_label", "dsc_kernel_source", "dsc_kernel_launch", "dsc_codegen_source", "dsc_codegen_compile",
-    "dsc_codegen_check_schedule", "dsc_free_string", "dsc_schedule_create", "dsc_schedule_destroy",
+    "dsc_codegen_check_schedule", "dsc_free_string", "dsc_cache_stats", "dsc_schedule_create", "dsc_schedule_destroy",
     "dsc_schedule_run", "dsc_schedule_run_static", "dsc_schedule_launch_count", "dsc_schedule_describe", "dsc_schedule_dot", "dsc_prof_markers", "dsc_prof_enable", "dsc_prof_reset",
     "dsc_prof_report", "dsc_prof_query", "dsc_prof_work",
 ]
@@ -128,6 +129,13 @@ def codegen_compile(kernel, arch: str = "gfx950") -> int:
     n = C.c_size_t()
     check(lib().dsc_codegen_compile(C.byref(mk.desc), arch.encode(), C.byref(n)))
     return n.value
+
+
+def cache_stats():
+    """(files used, hipRTC compilations, files refused and deleted) of the on-disk code-object cache, process-wide."""
+    a, b, c = C.c_int64(), C.c_int64(), C.c_int64()
+    check(lib().dsc_cache_stats(C.byref(a), C.byref(b), C.byref(c)))
+    return a.value, b.value, c.value
 
 
 def schedule_flags(fused) -> int:

@@ -272,6 +272,14 @@ int dsc_codegen_compile(const dsc_kernel_desc* desc, const char* arch, size_t* o
 /* Plans a whole schedule (fusion included) and compiles every kernel it would launch for `arch`, without a
  * device; out_text (optional) receives the listing dsc_schedule_describe would give. */
 int dsc_codegen_check_schedule(const struct dsc_schedule_desc* desc, uint32_t flags, const char* arch, char** out_text);
+/* The on-disk code-object cache behind dsc_kernel_get and dsc_schedule_create (the reference keeps compiled
+ * modules per process only, keyed by descriptor, kernel.rs:1037-1056; here a code object also survives the process,
+ * as a file named by a hash of the generated source, the target, the compile options and the hipRTC / HIP runtime
+ * versions, in $DSC_CACHE_DIR or ~/.cache/descent_amd; DSC_CACHE_DIR=off disables it).  A file is used only if its
+ * header (length and checksum of the payload) matches and the payload is an AMDGPU ELF image; any other file is
+ * deleted and the kernel recompiled, and so is an object the runtime refuses to load.  Process-wide counters:
+ * files used, hipRTC compilations, files refused and deleted.  Any pointer may be null. */
+int dsc_cache_stats(int64_t* out_hits, int64_t* out_compiles, int64_t* out_rejected);
 void dsc_free_string(char* s);
 
 /* -------------------------------------------------------------- schedules */

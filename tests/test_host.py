@@ -308,3 +308,60 @@ def test_image_fit_parameter_counts_match_the_reference_readme():
     mh = workloads.MultiHashGrid(env, sizes, 4096, (64, 64))
     total = count(mh) + sum(g.t.shape.element_count() for g in mh.grids)
     assert total == 43977, (total, sizes)
+
+
+def test_code_object_cache_hit_miss_and_damaged_files(tmp_path, monkeypatch):
+    """The on-disk code-object cache through the device-free compile path: a miss compiles and writes a file, a hit
+    uses it without calling hipRTC, and a truncated, a bit-flipped and a foreign file are each deleted and the kernel
+    compiled again (the counterpart of the reference's per-process KernelCache, src/kernel.rs:1037-1056)."""
+    cache = tmp_path / "cache"
+    cache.mkdir()
+    monkeypatch.setenv("DSC_CACHE_DIR", str(cache))
+    kernel = K.FillKernel(K.Literal.f32(2.25), 4321)
+
+    def compile_once():
+        before = hip_backend.cache_stats()
+        size = hip_backend.codegen_compile(kernel)
+        after = hip_backend.cache_stats()
+        return size, tuple(a - b for a, b in zip(after, before))
+
+    size, delta = compile_once()
+    assert delta == (0, 1, 0)  # miss: one hipRTC compilation
+    files = list(cache.iterdir())
+    assert len(files) == 1 and files[0].suffix == ".co"
+    blob = files[0].read_bytes()
+    assert blob[:8] == b"DSCCOBJ2" and blob[24:28] == b"\x7fELF" and len(blob) == 24 + size
+
+    size2, delta = compile_once()
+    assert (size2, delta) == (size, (1, 0, 0))  # hit: the file, no compilation
+
+    damaged = {
+        "truncated": blob[: len(blob) // 2],
+        "one bit flipped in the payload": blob[:1000] + bytes([blob[1000] ^ 0x10]) + blob[1001:],
+        "not a cache file": b"\x7fELF" + b"\0" * 4096,
+        "header only": blob[:24],
+        "right header, payload is not a code object": None,
+    }
+    junk = b"#!/bin/sh\n" * 100
+    import struct
+
+    def fnv(data):
+        h = 1469598103934665603
+        for byte in data:
+            h = ((h ^ byte) * 1099511628211) & 0xFFFFFFFFFFFFFFFF
+        return h
+
+    damaged["right header, payload is not a code object"] = b"DSCCOBJ2" + struct.pack("<QQ", len(junk), fnv(junk)) + junk
+    for what, data in damaged.items():
+        files[0].write_bytes(data)
+        size3, delta = compile_once()
+        assert (size3, delta) == (size, (0, 1, 1)), what  # refused, deleted, compiled again
+        assert files[0].read_bytes() == blob, what         # and the cache holds a good file again
+
+    # the key covers the compile options and tool versions: another kernel is another file
+    hip_backend.codegen_compile(K.FillKernel(K.Literal.f32(2.25), 4322))
+    assert len(list(cache.iterdir())) == 2
+
+    monkeypatch.setenv("DSC_CACHE_DIR", "off")
+    _, delta = compile_once()
+    assert delta == (0, 1, 0) and len(list(cache.iterdir())) == 2
