@@ -347,7 +347,10 @@ struct Emitter {
             case DSC_PE_GATHER: {
                 const dsc_view& v = pe.inputs[op.input_index];
                 auto names = coords_for(op.gather_shape);
-                names[op.axis] = "F2I(" + T(op.args[0]) + ")";
+                // The index comes from data, so its range is unknown when the kernel is generated.  The reference
+                // (kernel.rs:336-351) loads with whatever it gets and leans on Vulkan's bounds-checked buffers; a HIP
+                // load has no such net, so the index is clamped to the gathered axis (indices inside it are untouched).
+                names[op.axis] = "clampi(F2I(" + T(op.args[0]) + "), 0, " + S(v.out_shape.dims[op.axis] - 1) + ")";
                 rhs = load_view(srcs[op.input_index], v, names);
                 break;
             }
