@@ -20,6 +20,7 @@ KIND_FILL, KIND_PER_ELEMENT, KIND_REDUCE, KIND_MATMUL, KIND_UNPAD, KIND_W2I, KIN
 SCHEDULE_NO_FUSION = 1
 SCHEDULE_NO_CONV_KERNELS = 2
 SCHEDULE_GRAPH_REPLAY = 4
+SCHEDULE_SPLIT_CONV_GRADS = 8
 
 
 class CShape(C.Structure):

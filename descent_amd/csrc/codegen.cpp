@@ -372,7 +372,7 @@ string entry_name(const FusedKernel& fk) {
     auto count = [](int64_t v) { return to_string((long long)v); };
     if (fk.dgrad.on) {
         const MatMulDims g = matmul_dims(d);
-        return "dsc_conv_dgrad_img" + count(fk.dgrad.img) + "_" + count(fk.dgrad.oh) + "x" + count(fk.dgrad.ow) + "_g" + count(fk.dgrad.g) + "_k" +
+        return string(fk.dgrad.wgrad ? "dsc_conv_bwd_img" : "dsc_conv_dgrad_img") + count(fk.dgrad.img) + "_" + count(fk.dgrad.oh) + "x" + count(fk.dgrad.ow) + "_g" + count(fk.dgrad.g) + "_k" +
                count(g.k) + "_c" + count(fk.dgrad.c);
     }
     if (fk.cfwd.on)
@@ -444,23 +444,52 @@ struct ResultStore {
         for (int o = 0; o < pe.n_outputs; ++o) body << "    result[" << o << "] = et" << pe.outputs[o] << ";\n";
         em.funcs << "DSC_INLINE void result_epilogue(float product, int gid, float* result, " << em.params_decl() << ") {\n"
                  << body.str() << "}\n";
+        if (fk.epilogue_permuted) {
+            // result r is element `r` of the product array; the epilogue element that reads it has, on every output
+            // axis j of the view, the coordinate (c_i / step_j) % extent_j of the input axis i the axis walks
+            const dsc_view& v = pe.inputs[fk.epilogue_product_input];
+            int64_t ist[DSC_MAX_DIM], ost[DSC_MAX_DIM];
+            strides_of(v.in_shape, ist);
+            strides_of(v.out_shape, ost);
+            std::ostringstream f;
+            f << "DSC_INLINE int epilogue_element_of(int r) {\n    int e = 0;\n";
+            for (int j = 0; j < v.out_shape.rank; ++j) {
+                if (v.out_shape.dims[j] <= 1 || v.map_axis[j] < 0) continue;
+                const int i = v.map_axis[j];
+                f << "    e += (((r / " << S(ist[i]) << ") % " << S(v.in_shape.dims[i]) << ") / " << S(v.map_step[j]) << ") % " << S(v.out_shape.dims[j]) << " * "
+                  << S(ost[j]) << ";\n";
+            }
+            f << "    return e;\n}\n";
+            em.funcs << f.str();
+        }
     }
     string one(const string& value, const string& oid) const {
         const FusedKernel& fk = em.fk;
         if (!fk.has_epilogue) return "b" + to_string(fk.outputs[0]) + "[" + oid + "] = " + value + ";";
+        if (fk.epilogue_permuted) {
+            string t = "{ float res[" + to_string(n_res) + "]; const int ee = epilogue_element_of((int)(" + oid + ")); result_epilogue(" + value + ", ee, res, " +
+                       em.params_pass() + ");";
+            for (int o = 0; o < n_res; ++o) t += " b" + to_string(fk.outputs[o]) + "[ee] = res[" + to_string(o) + "];";
+            return t + " }";
+        }
         string t = "{ float res[" + to_string(n_res) + "]; result_epilogue(" + value + ", (int)(" + oid + "), res, " + em.params_pass() + ");";
         for (int o = 0; o < n_res; ++o) t += " b" + to_string(fk.outputs[o]) + "[" + oid + "] = res[" + to_string(o) + "];";
+        if (fk.epilogue_keeps_product) t += " b" + to_string(fk.outputs.back()) + "[" + oid + "] = " + value + ";";
         return t + " }";
     }
     string four(const string& value4, const string& oid) const {
         const FusedKernel& fk = em.fk;
         if (!fk.has_epilogue) return "*(float4*)(b" + to_string(fk.outputs[0]) + " + " + oid + ") = " + value4 + ";";
+        if (fk.epilogue_permuted)
+            return "{ " + one(value4 + ".x", oid) + " " + one(value4 + ".y", "(" + oid + ") + 1") + " " + one(value4 + ".z", "(" + oid + ") + 2") + " " +
+                   one(value4 + ".w", "(" + oid + ") + 3") + " }";
         string t = "{ const float pv[4] = {" + value4 + ".x, " + value4 + ".y, " + value4 + ".z, " + value4 + ".w}; float res[4][" +
                    to_string(n_res) + "];\n#pragma unroll\n        for (int j = 0; j < 4; ++j) result_epilogue(pv[j], (int)(" + oid +
                    ") + j, res[j], " + em.params_pass() + ");";
         for (int o = 0; o < n_res; ++o)
             t += " *(float4*)(b" + to_string(fk.outputs[o]) + " + " + oid + ") = make_float4(res[0][" + to_string(o) + "], res[1][" +
                  to_string(o) + "], res[2][" + to_string(o) + "], res[3][" + to_string(o) + "]);";
+        if (fk.epilogue_keeps_product) t += " *(float4*)(b" + to_string(fk.outputs.back()) + " + " + oid + ") = " + value4 + ";";
         return t + " }";
     }
 };
@@ -937,6 +966,10 @@ string gen_row_fused(Emitter& em, Generated* out) {
 
 // ---- convolution data gradient ---------------------------------------------------------------------------
 
+// Words per pixel of the forward kernel's LDS tile: 16 neighbouring pixels times four channels should fall into 64
+// different banks, which they do when the pitch is an odd multiple of four words.
+int64_t conv_fwd_pitch(int64_t c) { return (c % 4 == 0 && (c / 4) % 2 == 0) ? c + 4 : c; }
+
 int64_t dgrad_pitch(int64_t k) { return k % 8 == 0 ? k + 4 : k; }  // keeps 16-byte reads of neighbouring pixels off one bank
 
 int64_t dgrad_lds_floats(const FusedKernel::ConvDgrad& c, int64_t k) {
@@ -1082,11 +1115,355 @@ string gen_conv_dgrad(Emitter& em, Generated* out) {
     return "";
 }
 
+// ---- convolution backward: data gradient and filter gradient in one kernel ---------------------------------
+
+// Workgroup = (group, set of images).  Per image: dC of the image goes to LDS in *slots* -- slot oy * PW + ox with
+// PW = ow + fw - 1 the width of the padded image, so that the slots of an output row are followed by fw - 1 slots
+// that stay zero -- and the image's padded input tile goes to LDS as in the forward kernel.  The data gradient is
+// then what the data-gradient kernel computes (one padded pixel per thread, taps x output channels, border folds
+// through LDS).  The filter gradient is im2col^T x dC over the slots: with the padded pitch, the im2col element of
+// slot q for tap (fy, fx) and channel c is one tile word at (q + fy * PW + fx) * pitch + c, so the A fragment of
+// v_mfma_f32_16x16x4f32 (lane l: row kidx = 16 * mt + l % 16, slot 4 * s + l / 16) is a per-lane constant plus a
+// per-step term, and the B fragment is dC[slot][oc].  Slots without a pixel multiply a zero, whatever the tile word
+// beside them holds.  One im2col row of ones (kidx = fh * fw * c) makes row fh*fw*c of the product the column sums
+// of dC: the bias gradient.  The accumulators live across the workgroup's images; the four waves take every fourth
+// step and are summed through LDS at the end, one partial product per workgroup.
+struct ConvBwdLayout {
+    int64_t PH, PW, KD, PITCH, CP, SLP, steps, ZERO_AT, XT_AT, XT_FLOATS, ONE_AT, ZW_AT, GB_AT, TOTAL;
+    int MT, NT;
+    // data gradient on the matrix cores (see gen_conv_bwd): pixels per group, shifted taps per filter row, B fragments
+    // per lane, groups per image row, groups, tiles of 16 groups, tiles per wave
+    bool mfma_dgrad;
+    int64_t P, TQ, GS, GPR, GROUPS, TILES, TPW;
+};
+
+ConvBwdLayout conv_bwd_layout(const FusedKernel::ConvDgrad& c, int64_t K, int64_t cp_override = 0) {
+    ConvBwdLayout L{};
+    L.PH = c.oh + c.fh - 1;
+    L.PW = c.ow + c.fw - 1;
+    L.KD = c.fh * c.fw * c.c;
+    L.CP = cp_override > 0 ? cp_override : conv_fwd_pitch(c.c);
+    L.MT = (int)((L.KD + (c.bias ? 1 : 0) + 15) / 16);
+    L.NT = (int)((K + 15) / 16);
+    L.P = (c.c == 4 || c.c == 8 || c.c == 16) ? 16 / c.c : 0;
+    L.TQ = c.fw + L.P - 1;
+    L.GS = L.P ? c.fh * L.TQ * K / 4 : 0;
+    L.GPR = L.P ? (L.PW + L.P - 1) / L.P : 1;
+    L.GROUPS = L.PH * L.GPR;
+    L.TILES = (L.GROUPS + 15) / 16;
+    L.TPW = (L.TILES + 3) / 4;
+    L.mfma_dgrad = L.P > 0 && L.GS <= 96 && L.TPW <= 8;
+    L.PITCH = dgrad_pitch(K);  // the FMA form reads 16-byte pieces of a slot
+    if (L.mfma_dgrad) {
+        // words per slot: the one (from k to k + 8) that spreads an A fragment load of the data gradient -- lane l reads
+        // word l / 16 of the slot of group l % 16 -- over the most of the 64 banks
+        int best_worst = 1 << 30;
+        for (int64_t pitch = K; pitch <= K + 8; ++pitch) {
+            int lanes_on_bank[64] = {0};
+            int worst = 0;
+            for (int l = 0; l < 64; ++l) {
+                const int64_t grp = l % 16, slot = (grp / L.GPR) * L.PW + (grp % L.GPR) * L.P;
+                worst = std::max(worst, ++lanes_on_bank[(slot * pitch + l / 16) % 64]);
+            }
+            if (worst < best_worst) {
+                best_worst = worst;
+                L.PITCH = pitch;
+            }
+        }
+    }
+    L.SLP = (c.oh * L.PW + 3) / 4 * 4;
+    L.steps = L.SLP / 4;
+    L.ZERO_AT = L.SLP * L.PITCH;
+    L.XT_AT = (L.ZERO_AT + L.PITCH + 3) / 4 * 4;
+    const int64_t pixels = std::max(L.PH * L.PW, L.SLP + (c.fh - 1) * L.PW + c.fw - 1);  // what a fragment load may address
+    L.XT_FLOATS = (pixels * L.CP + 3) / 4 * 4;
+    L.ONE_AT = L.XT_AT + L.XT_FLOATS;
+    L.ZW_AT = L.ONE_AT + 1;
+    // the data gradient's B fragments (one word per lane and step) stay in LDS: in registers they would cost the
+    // kernel a wave of occupancy
+    L.GB_AT = L.ONE_AT + 4;
+    L.TOTAL = std::max<int64_t>(L.GB_AT + (L.mfma_dgrad ? L.GS * 64 : 0), (int64_t)4 * L.MT * L.NT * 256);
+    // four workgroups per CU (160 KB of LDS) matter more than the input tile's bank spread
+    if (cp_override == 0 && L.CP != c.c && L.TOTAL * 4 * 4 > 160 * 1024) {
+        const ConvBwdLayout tight = conv_bwd_layout(c, K, c.c);
+        if (tight.TOTAL * 4 * 4 <= 160 * 1024) return tight;
+    }
+    return L;
+}
+
+bool conv_bwd_fits_impl(const FusedKernel::ConvDgrad& c, int64_t k) {
+    if (!conv_dgrad_fits(c, k)) return false;
+    const ConvBwdLayout L = conv_bwd_layout(c, k);
+    return L.TOTAL * 4 <= 64 * 1024 && L.MT * L.NT <= 8 && c.chunks >= 8 && c.chunks % 8 == 0;
+}
+
+string gen_conv_bwd(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const FusedKernel::ConvDgrad& cv = fk.dgrad;
+    const MatMulDims g = matmul_dims(d);
+    const int64_t K = g.k, G = cv.g, C = cv.c, FH = cv.fh, FW = cv.fw, OH = cv.oh, OW = cv.ow, IMG = cv.img;
+    if (g.batch != G || g.m != IMG * OH * OW || g.n != FH * FW * C || g.chunks != 1) return "conv backward: geometry mismatch";
+    if (fk.inputs.size() != 3 || fk.inputs[2].buffer < 0) return "conv backward: the image must be a buffer";
+    if ((int)fk.outputs.size() != 2 + (cv.bias ? 1 : 0)) return "conv backward: output count";
+    if (!conv_bwd_fits_impl(cv, K)) return "conv backward: geometry does not fit";
+    const ConvBwdLayout L = conv_bwd_layout(cv, K);
+    const int64_t PH = L.PH, PW = L.PW, KD = L.KD, PITCH = L.PITCH, CP = L.CP, GC = G * C;
+    const int64_t H = PH - 2 * cv.pad_h, W = PW - 2 * cv.pad_w;
+    const bool unpad = cv.pad_h > 0 || cv.pad_w > 0;
+    const int MT = L.MT, NT = L.NT;
+    if (H < 1 || W < 1 || K % 4 != 0) return "conv backward: unsupported geometry";
+
+    const string la = em.load_view(fk.inputs[0], d.inputs[0], {"cb", "cm", "ck"});
+    em.funcs << "DSC_INLINE float load_a(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return " << la << ";\n}\n";
+    const string lb = em.load_view(fk.inputs[1], d.inputs[1], {"cb", "ck", "cn"});
+    em.funcs << "DSC_INLINE float load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb << ";\n}\n";
+
+    std::ostringstream k;
+    const string out_ptr = "b" + to_string(fk.outputs[0]), part_ptr = "b" + to_string(fk.outputs[1]);
+    const string img_ptr = "b" + to_string(fk.inputs[2].buffer);
+    k << "typedef float cb_float4 __attribute__((ext_vector_type(4)));\n";
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
+    k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
+    k << "    __shared__ __attribute__((aligned(16))) float smem[" << S(L.TOTAL) << "];\n";
+    k << "    float* const lds = smem;\n    float* const xt = smem + " << S(L.XT_AT) << ";\n";
+    // the groups of a set of images sit 8 workgroups apart: same XCD, same L2 (they share the lines of dC, of the
+    // image and of the output)
+    k << "    const int cb = (blockIdx.x / 8) % " << S(G) << ", chunk = (blockIdx.x / " << S(8 * G) << ") * 8 + blockIdx.x % 8;\n";
+    k << "    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 15, lk = lane >> 4;\n";
+    // what stays zero for the whole kernel: slots without a pixel, the zero row, the tile words behind the last pixel
+    k << "    for (int i = threadIdx.x; i < " << S(L.ONE_AT) << "; i += 256) smem[i] = 0.f;\n";
+    k << "    if (threadIdx.x == 0) { smem[" << S(L.ONE_AT) << "] = 1.f; smem[" << S(L.ZW_AT) << "] = 0.f; }\n";
+    // fragment addresses of this lane: a constant, plus the step's slot term where the mask says so
+    k << "    int a_off[" << MT << "], a_msk[" << MT << "], b_off[" << NT << "], b_msk[" << NT << "];\n";
+    k << "#pragma unroll\n    for (int mt = 0; mt < " << MT << "; ++mt) {\n";
+    k << "        const int kidx = mt * 16 + li, tap = kidx / " << S(C) << ";\n";
+    k << "        const bool real = kidx < " << S(KD) << ";\n";
+    k << "        a_off[mt] = real ? " << S(L.XT_AT) << " + ((tap / " << S(FW) << ") * " << S(PW) << " + tap % " << S(FW) << ") * " << S(CP) << " + kidx % " << S(C)
+      << " : (" << (cv.bias ? "kidx == " + S(KD) : string("false")) << " ? " << S(L.ONE_AT) << " : " << S(L.ZW_AT) << ");\n";
+    k << "        a_msk[mt] = real ? -1 : 0;\n    }\n";
+    k << "#pragma unroll\n    for (int nt = 0; nt < " << NT << "; ++nt) {\n";
+    k << "        const int oc = nt * 16 + li;\n";
+    k << "        b_off[nt] = oc < " << S(K) << " ? oc : " << S(L.ZERO_AT) << ";\n        b_msk[nt] = oc < " << S(K) << " ? -1 : 0;\n    }\n";
+    k << "    cb_float4 wacc[" << MT << "][" << NT << "];\n";
+    k << "#pragma unroll\n    for (int mt = 0; mt < " << MT << "; ++mt)\n#pragma unroll\n        for (int nt = 0; nt < " << NT
+      << "; ++nt) wacc[mt][nt] = (cb_float4){0.f, 0.f, 0.f, 0.f};\n";
+    // Data gradient on the matrix cores.  With few channels a 16-wide MFMA column block would be mostly empty, so a
+    // row of the product is a *group* of P = 16 / c neighbouring pixels of the padded image and a column is (pixel of
+    // the group, channel): dX[y][x0 + par][c] = sum over (ty, tq, oc) of dC[y - ty][x0 - tq][oc] * W'[ty][tq][oc][(par, c)]
+    // with tq = tx - par running over fw + P - 1 values and W' = W[oc][ty][tq + par][c] where that tap exists, else 0.
+    // The A fragment (lane l: group l % 16, k = 4 s + l / 16) is then dC of one slot for all four k of a step, and
+    // the B fragments are the same for every group: they stay in registers for the whole kernel.
+    const int64_t P = L.P, TQ = L.TQ, GS = L.GS, GPR = L.GPR, GROUPS = L.GROUPS, TPW = L.TPW;
+    const bool mfma_dgrad = L.mfma_dgrad;
+    if (mfma_dgrad) {
+        k << "    {\n";
+        k << "        const int par = li / " << S(C) << ", gc = li % " << S(C) << ";\n";
+        for (int64_t s = 0; s < GS; ++s) {
+            const int64_t oc0 = (4 * s) % K, tt = (4 * s) / K, ty = tt / TQ, tq = tt % TQ - (P - 1);
+            k << "        { const int tx = " << S(tq) << " + par; const float w = load_b(cb, " << S(oc0) << " + lk, (" << S(ty * FW) << " + clampi(tx, 0, " << S(FW - 1)
+              << ")) * " << S(C) << " + gc, " << em.params_pass() << "); smem[" << S(L.GB_AT + s * 64) << " + lane] = (tx >= 0 && tx < " << S(FW) << ") ? w : 0.f; }\n";
+        }
+        k << "    }\n";
+    }
+    // Fills.  The loads of an image -- dC of the image and group, and the image's padded input tile,
+    // xt[py][px][c] = image[clamp(py - pad_h)][clamp(px - pad_w)][c] -- are all issued before the first of them is
+    // stored to LDS: one round trip to memory per image.  (Requesting the next image's loads before the matrix phases
+    // of the current one, to have them in flight meanwhile, measured slower: 45.8 us against 42.2 for the ConvNet's
+    // second convolution -- the registers that hold them cost a wave of occupancy.)
+    // dC in 16-byte pieces when the operand is a buffer whose k runs along memory
+    int64_t dc_base = 0, dc_coef[DSC_MAX_DIM] = {0};
+    const bool vec_dc = fk.inputs[0].buffer >= 0 && K % 4 == 0 && affine_form(d.inputs[0], &dc_base, dc_coef) && dc_coef[2] == 1 && dc_base % 4 == 0 &&
+                        dc_coef[1] % 4 == 0 && (G == 1 || dc_coef[0] % 4 == 0);
+    const int64_t dunit = vec_dc ? 4 : 1;
+    const int64_t fill_n = OH * OW * K / dunit, NC = (fill_n + 255) / 256;
+    const bool vec_fill = C % 4 == 0;
+    const int64_t unit = vec_fill ? 4 : 1, xn = PH * PW * C / unit, NX = (xn + 255) / 256;
+    const string vt = vec_fill ? "float4" : "float", dvt = vec_dc ? "float4" : "float";
+    auto emit_issue = [&](const string& img, const string& ind) {
+        k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NC) << "; ++u) {\n";
+        k << ind << "    const int i = min((int)threadIdx.x + u * 256, " << S(fill_n - 1) << ") * " << S(dunit) << ";\n";
+        if (vec_dc)
+            k << ind << "    pv[u] = *(const float4*)(b" << fk.inputs[0].buffer << " + " << S(dc_base) << " + cb * " << S(G == 1 ? 0 : dc_coef[0]) << " + (" << img << " * "
+              << S(OH * OW) << " + i / " << S(K) << ") * " << S(dc_coef[1]) << " + i % " << S(K) << ");\n" << ind << "}\n";
+        else
+            k << ind << "    pv[u] = load_a(cb, " << img << " * " << S(OH * OW) << " + i / " << S(K) << ", i % " << S(K) << ", " << em.params_pass() << ");\n" << ind << "}\n";
+        k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NX) << "; ++u) {\n";
+        k << ind << "    const int e = min((int)threadIdx.x + u * 256, " << S(xn - 1) << ") * " << S(unit) << ";\n";
+        k << ind << "    const int ch = e % " << S(C) << ", px = (e / " << S(C) << ") % " << S(PW) << ", py = e / " << S(C * PW) << ";\n";
+        k << ind << "    const int sy = clampi(py - " << S(cv.pad_h) << ", 0, " << S(H - 1) << "), sx = clampi(px - " << S(cv.pad_w) << ", 0, " << S(W - 1) << ");\n";
+        k << ind << "    xv[u] = *(const " << vt << "*)(" << img_ptr << " + ((" << img << " * " << S(H) << " + sy) * " << S(W) << " + sx) * " << S(GC) << " + cb * " << S(C)
+          << " + ch);\n" << ind << "}\n";
+        k << ind << "__builtin_amdgcn_sched_barrier(0);\n";
+    };
+    auto emit_tile_stores = [&](const string& ind) {
+        k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NC) << "; ++u) {\n";
+        k << ind << "    const int i = ((int)threadIdx.x + u * 256) * " << S(dunit) << ", pi = i / " << S(K) << ";\n";
+        k << ind << "    float* const at = lds + ((pi / " << S(OW) << ") * " << S(PW) << " + pi % " << S(OW) << ") * " << S(PITCH) << " + i % " << S(K) << ";\n";
+        if (vec_dc)
+            k << ind << "    if ((int)threadIdx.x + u * 256 < " << S(fill_n) << ") { at[0] = pv[u].x; at[1] = pv[u].y; at[2] = pv[u].z; at[3] = pv[u].w; }\n" << ind << "}\n";
+        else
+            k << ind << "    if ((int)threadIdx.x + u * 256 < " << S(fill_n) << ") at[0] = pv[u];\n" << ind << "}\n";
+        k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NX) << "; ++u) {\n";
+        k << ind << "    const int e = ((int)threadIdx.x + u * 256) * " << S(unit) << ";\n";
+        k << ind << "    if ((int)threadIdx.x + u * 256 < " << S(xn) << ") *(" << vt << "*)(xt + (e / " << S(C) << ") * " << S(CP) << " + e % " << S(C) << ") = xv[u];\n"
+          << ind << "}\n";
+    };
+    k << "    __syncthreads();\n";
+    k << "    for (int img = chunk; img < " << S(IMG) << "; img += " << S(cv.chunks) << ") {\n";
+    k << "        {\n            " << dvt << " pv[" << S(NC) << "];\n            " << vt << " xv[" << S(NX) << "];\n";
+    emit_issue("img", "            ");
+    emit_tile_stores("            ");
+    k << "        }\n";
+    k << "        __syncthreads();\n";
+    // 2a. filter gradient: this wave's steps of four slots
+    k << "#pragma unroll 2\n        for (int s = wave; s < " << S(L.steps) << "; s += 4) {\n";
+    k << "            const int q = 4 * s + lk, qa = q * " << S(CP) << ", qb = q * " << S(PITCH) << ";\n";
+    k << "            float fa[" << MT << "], fb[" << NT << "];\n";
+    k << "#pragma unroll\n            for (int mt = 0; mt < " << MT << "; ++mt) fa[mt] = smem[a_off[mt] + (qa & a_msk[mt])];\n";
+    k << "#pragma unroll\n            for (int nt = 0; nt < " << NT << "; ++nt) fb[nt] = smem[b_off[nt] + (qb & b_msk[nt])];\n";
+    k << "#pragma unroll\n            for (int mt = 0; mt < " << MT << "; ++mt)\n#pragma unroll\n                for (int nt = 0; nt < " << NT << "; ++nt)\n";
+    k << "                    wacc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[mt], fb[nt], wacc[mt][nt], 0, 0, 0);\n";
+    k << "        }\n";
+    const int64_t passes = (PH * PW + 255) / 256;
+    if (mfma_dgrad) {
+        // 2b. data gradient: every wave takes every fourth tile of 16 pixel groups
+        k << "        cb_float4 dacc[" << S(TPW) << "];\n";
+        k << "#pragma unroll\n        for (int t = 0; t < " << S(TPW) << "; ++t) {\n";
+        k << "            const int grp = (t * 4 + wave) * 16 + li, gy = grp / " << S(GPR) << ", gx0 = (grp % " << S(GPR) << ") * " << S(P) << ";\n";
+        k << "            cb_float4 d = (cb_float4){0.f, 0.f, 0.f, 0.f};\n";
+        // (the filter rows stay a loop: unrolled whole, the scheduler hoists every LDS load of a tile and the kernel
+        // loses a wave of occupancy to the registers that hold them)
+        k << "#pragma unroll 1\n            for (int ty = 0; ty < " << S(FH) << "; ++ty) {\n";
+        k << "                const int oy = gy - ty;\n                const float* const gbp = smem + " << S(L.GB_AT) << " + ty * " << S(TQ * (K / 4) * 64) << " + lane;\n";
+        for (int64_t tqi = 0; tqi < TQ; ++tqi) {
+            const int64_t tq = tqi - (P - 1);
+            k << "                {\n                    const int ox = gx0 - " << S(tq) << ";\n";
+            k << "                    const int at = (oy >= 0 && oy < " << S(OH) << " && ox >= 0 && ox < " << S(OW) << ") ? (oy * " << S(PW) << " + ox) * " << S(PITCH) << " : "
+              << S(L.ZERO_AT) << ";\n";
+            for (int64_t o4 = 0; o4 < K / 4; ++o4)
+                k << "                    d = __builtin_amdgcn_mfma_f32_16x16x4f32(lds[at + " << S(4 * o4) << " + lk], gbp[" << S((tqi * (K / 4) + o4) * 64) << "], d, 0, 0, 0);\n";
+            k << "                }\n";
+        }
+        k << "            }\n";
+        k << "            dacc[t] = d;\n        }\n";
+        // register r of lane l is D[group 4 * (l / 16) + r][(pixel of the group, channel) = l % 16]
+        auto emit_dacc_stores = [&](const string& target_of_p) {
+            k << "#pragma unroll\n        for (int t = 0; t < " << S(TPW) << "; ++t)\n#pragma unroll\n            for (int r = 0; r < 4; ++r) {\n";
+            k << "                const int grp = (t * 4 + wave) * 16 + 4 * lk + r, gy = grp / " << S(GPR) << ", gx = (grp % " << S(GPR) << ") * " << S(P) << " + li / " << S(C)
+              << ", gc = li % " << S(C) << ";\n";
+            k << "                const int p = gy * " << S(PW) << " + gx;\n";
+            k << "                if (grp < " << S(GROUPS) << " && gx < " << S(PW) << ") " << target_of_p << " = dacc[t][r];\n            }\n";
+        };
+        if (!unpad) {
+            emit_dacc_stores(out_ptr + "[(img * " + S(PH * PW) + " + p) * " + S(GC) + " + cb * " + S(C) + " + gc]");
+            k << "        __syncthreads();\n";
+        } else {
+            k << "        __syncthreads();\n";
+            emit_dacc_stores("xt[p * " + S(C) + " + gc]");
+            k << "        __syncthreads();\n";
+        }
+    } else {
+    // 2b. data gradient: one padded-image pixel per thread and pass, taps x output channels, the filter element
+    // through the scalar unit (as the data-gradient kernel)
+    const int64_t OCB = K % 8 == 0 ? 8 : 4;
+    k << "        float acc[" << passes << "][" << S(C) << "];\n";
+    k << "#pragma unroll\n        for (int ps = 0; ps < " << passes << "; ++ps) {\n";
+    k << "            const int p = min(ps * 256 + (int)threadIdx.x, " << S(PH * PW - 1) << ");\n";
+    k << "            const int py = p / " << S(PW) << ", px = p % " << S(PW) << ";\n";
+    k << "#pragma unroll\n            for (int c = 0; c < " << S(C) << "; ++c) acc[ps][c] = 0.f;\n";
+    k << "#pragma unroll 1\n            for (int tap = 0; tap < " << S(FH * FW) << "; ++tap) {\n";
+    k << "                const int fy = tap / " << S(FW) << ", fx = tap % " << S(FW) << ";\n";
+    k << "                const int oy = py - fy, ox = px - fx;\n";
+    k << "                const bool inside = oy >= 0 && oy < " << S(OH) << " && ox >= 0 && ox < " << S(OW) << ";\n";
+    k << "                const float* src = &lds[inside ? (oy * " << S(PW) << " + ox) * " << S(PITCH) << " : " << S(L.ZERO_AT) << "];\n";
+    k << "#pragma unroll\n                for (int oc = 0; oc < " << S(K) << "; oc += " << OCB << ") {\n";
+    k << "                    float a[" << OCB << "];\n";
+    k << "#pragma unroll\n                    for (int q = 0; q < " << OCB << "; q += 4) {\n";
+    k << "                        const float4 a4 = *(const float4*)(src + oc + q);\n";
+    k << "                        a[q] = a4.x; a[q + 1] = a4.y; a[q + 2] = a4.z; a[q + 3] = a4.w;\n                    }\n";
+    k << "#pragma unroll\n                    for (int j = 0; j < " << OCB << "; ++j)\n";
+    k << "#pragma unroll\n                        for (int c = 0; c < " << S(C) << "; ++c)\n";
+    k << "                            acc[ps][c] = fmaf(a[j], load_b(cb, oc + j, tap * " << S(C) << " + c, " << em.params_pass() << "), acc[ps][c]);\n";
+    k << "                    __builtin_amdgcn_sched_barrier(0);\n";
+    k << "                }\n            }\n        }\n";
+    if (!unpad) {
+        k << "#pragma unroll\n        for (int ps = 0; ps < " << passes << "; ++ps) {\n";
+        k << "            const int p = ps * 256 + (int)threadIdx.x;\n            if (p < " << S(PH * PW) << ") {\n";
+        k << "#pragma unroll\n                for (int c = 0; c < " << S(C) << "; ++c) " << out_ptr << "[(img * " << S(PH * PW) << " + p) * " << S(GC)
+          << " + cb * " << S(C) << " + c] = acc[ps][c];\n            }\n        }\n";
+        k << "        __syncthreads();\n";
+    } else {
+        // 3. the padded-image gradient goes through the input tile's memory (dead by now); each pixel of the image sums
+        // the padded pixels that replicate it
+        k << "        __syncthreads();\n";
+        k << "#pragma unroll\n        for (int ps = 0; ps < " << passes << "; ++ps) {\n";
+        k << "            const int p = ps * 256 + (int)threadIdx.x;\n            if (p < " << S(PH * PW) << ") {\n";
+        k << "#pragma unroll\n                for (int c = 0; c < " << S(C) << "; ++c) xt[p * " << S(C) << " + c] = acc[ps][c];\n            }\n        }\n";
+        k << "        __syncthreads();\n";
+    }
+    }
+    if (unpad) {
+        k << "        for (int i = threadIdx.x; i < " << S(H * W * C) << "; i += 256) {\n";
+        k << "            const int c = i % " << S(C) << ", x = (i / " << S(C) << ") % " << S(W) << ", y = i / " << S(C * W) << ";\n";
+        k << "            float sum = 0.f;\n";
+        const string outer = cv.rows_first ? "jx" : "jy", inner = cv.rows_first ? "jy" : "jx";
+        auto range = [&](const string& j) {
+            const bool is_y = j == "jy";
+            return "for (int " + j + " = " + S(-(is_y ? cv.pad_h : cv.pad_w)) + "; " + j + " <= " + S(is_y ? cv.pad_h : cv.pad_w) + "; ++" + j + ")";
+        };
+        if (H > 1 && W > 1) {
+            auto slots = [&](const string& q, bool is_y) {
+                return "for (int " + q + " = 0; " + q + " <= " + S(is_y ? cv.pad_h : cv.pad_w) + "; ++" + q + ")";
+            };
+            const string qo = cv.rows_first ? "qx" : "qy", qi = cv.rows_first ? "qy" : "qx";
+            k << "            const bool edge_y = y == 0 || y == " << S(H - 1) << ", edge_x = x == 0 || x == " << S(W - 1) << ";\n";
+            k << "            const int base_y = y == 0 ? 0 : y + " << S(cv.pad_h) << ", base_x = x == 0 ? 0 : x + " << S(cv.pad_w) << ";\n";
+            k << "#pragma unroll\n            " << slots(qo, !cv.rows_first) << " {\n                float part = 0.f;\n";
+            k << "#pragma unroll\n                " << slots(qi, cv.rows_first) << " {\n";
+            k << "                    const bool ok = (edge_y || qy == 0) && (edge_x || qx == 0);\n";
+            k << "                    const int ky = base_y + (edge_y ? qy : 0), kx = base_x + (edge_x ? qx : 0);\n";
+            k << "                    const float w = xt[(ky * " << S(PW) << " + kx) * " << S(C) << " + c];\n";
+            k << "                    part += ok ? w : 0.f;\n                }\n                sum += part;\n            }\n";
+        } else {
+            k << "#pragma unroll\n            " << range(outer) << " {\n                float part = 0.f;\n";
+            k << "#pragma unroll\n                " << range(inner) << " {\n";
+            k << "                    const bool ok_y = jy == 0 || (jy < 0 && y == 0) || (jy > 0 && y == " << S(H - 1) << ");\n";
+            k << "                    const bool ok_x = jx == 0 || (jx < 0 && x == 0) || (jx > 0 && x == " << S(W - 1) << ");\n";
+            k << "                    const int ky = clampi(y + " << S(cv.pad_h) << " + jy, 0, " << S(PH - 1) << "), kx = clampi(x + " << S(cv.pad_w)
+              << " + jx, 0, " << S(PW - 1) << ");\n";
+            k << "                    const float w = xt[(ky * " << S(PW) << " + kx) * " << S(C) << " + c];\n";
+            k << "                    part += (ok_y && ok_x) ? w : 0.f;\n                }\n                sum += part;\n            }\n";
+        }
+        k << "            " << out_ptr << "[((img * " << S(H) << " + y) * " << S(W) << " + x) * " << S(GC) << " + cb * " << S(C) << " + c] = sum;\n        }\n";
+        k << "        __syncthreads();\n";  // the next image's fills overwrite what the folds read
+    }
+    k << "    }\n";
+    // 4. the four waves' accumulators are summed through LDS; register r of lane l is D[4 * (l / 16) + r][l % 16]
+    const int64_t R = (int64_t)MT * NT * 256;
+    k << "#pragma unroll\n    for (int mt = 0; mt < " << MT << "; ++mt)\n#pragma unroll\n        for (int nt = 0; nt < " << NT
+      << "; ++nt)\n#pragma unroll\n            for (int r = 0; r < 4; ++r) smem[wave * " << S(R) << " + (mt * " << NT << " + nt) * 256 + r * 64 + lane] = wacc[mt][nt][r];\n";
+    k << "    __syncthreads();\n";
+    k << "    for (int i = threadIdx.x; i < " << S(R) << "; i += 256) {\n";
+    k << "        const float sum = (smem[i] + smem[" << S(R) << " + i]) + (smem[" << S(2 * R) << " + i] + smem[" << S(3 * R) << " + i]);\n";
+    k << "        const int tile = i >> 8, r = (i >> 6) & 3, l = i & 63;\n";
+    k << "        const int cm = (tile / " << NT << ") * 16 + 4 * (l >> 4) + r, cn = (tile % " << NT << ") * 16 + (l & 15);\n";
+    k << "        if (cm < " << S(KD) << " && cn < " << S(K) << ") " << part_ptr << "[(chunk * " << S(G) << " + cb) * " << S(KD * K) << " + cm * " << S(K) << " + cn] = sum;\n";
+    if (cv.bias)
+        k << "        if (cm == " << S(KD) << " && cn < " << S(K) << ") b" << fk.outputs[2] << "[(chunk * " << S(G) << " + cb) * " << S(K) << " + cn] = sum;\n";
+    k << "    }\n}\n";
+    if (cv.chunks * G >= kMaxIndex) return "conv backward: grid too large";
+    out->grid = (unsigned)(cv.chunks * G);
+    out->block = 256;
+    out->source = k.str();
+    out->note = "conv backward: workgroup per group and image set (" + S(cv.chunks) + " sets), dC and input tile in LDS, data gradient " + S(FH) + "x" + S(FW) +
+                " taps x " + S(K) + " channels" + (unpad ? " with border folds" : "") + ", filter gradient mfma 16x16x4 " + to_string(MT) + "x" + to_string(NT) +
+                " tiles" + (cv.bias ? " +column sums of dC" : "");
+    return "";
+}
+
 // ---- convolution forward ---------------------------------------------------------------------------------
 
-// Words per pixel of the forward kernel's LDS tile: 16 neighbouring pixels times four channels should fall into 64
-// different banks, which they do when the pitch is an odd multiple of four words.
-int64_t conv_fwd_pitch(int64_t c) { return (c % 4 == 0 && (c / 4) % 2 == 0) ? c + 4 : c; }
 
 // One workgroup per (image, group).  The group's channels of the image go to LDS once with replicate padding applied
 // (a tile of (oh + fh - 1) x (ow + fw - 1) pixels), so that an im2col element is one LDS word at
@@ -1111,8 +1488,26 @@ string gen_conv_fwd(Emitter& em, Generated* out) {
         return "conv forward: geometry mismatch";
     const int64_t PH = cv.oh + cv.fh - 1, PW = cv.ow + cv.fw - 1;
     const int64_t CP = conv_fwd_pitch(C);  // words per pixel in LDS
-    const int64_t steps = (K + 3) / 4, tiles = (PIX + 15) / 16;
+    // with pooling a tile of 16 pixels is two image rows by eight columns, so that a pooling window's four pixels sit in
+    // lanes l, l ^ 1, l ^ 8, l ^ 9 of one tile
+    const bool pooled = fk.pool.on;
+    const int64_t TPR = (cv.ow + 7) / 8, OH2 = cv.oh / 2, OW2 = cv.ow / 2;
+    const int64_t steps = (K + 3) / 4, tiles = pooled ? OH2 * TPR : (PIX + 15) / 16;
     const int n_out = fk.has_epilogue ? fk.epilogue.raw().n_outputs : 1;
+    const int n_pool_out = pooled && fk.pool.has_epilogue ? fk.pool.epilogue.raw().n_outputs : 0;
+    if (pooled) {
+        if (cv.oh % 2 || cv.ow % 2 || g.n % 4 || fk.pool.source < 0 || fk.pool.source >= n_out) return "conv forward: pooling needs even extents and whole 16-byte channel pieces";
+        if ((int)fk.outputs.size() != n_out + n_pool_out + (fk.pool.store_pooled ? 1 : 0)) return "conv forward: pooled output count";
+        if (fk.pool.has_epilogue) {
+            const dsc_kernel_desc& pe = fk.pool.epilogue.raw();
+            std::ostringstream body;
+            std::map<int, string> ov;
+            ov[fk.pool.epilogue_product_input] = "product";
+            em.emit_pe(body, pe, fk.pool.epilogue_inputs, "gid", "q", ov);
+            for (int o = 0; o < pe.n_outputs; ++o) body << "    result[" << o << "] = qt" << pe.outputs[o] << ";\n";
+            em.funcs << "DSC_INLINE void pool_epilogue(float product, int gid, float* result, " << em.params_decl() << ") {\n" << body.str() << "}\n";
+        }
+    }
     const string lb = em.load_view(fk.inputs[1], d.inputs[1], {"cb", "ck", "cn"});
     em.funcs << "DSC_INLINE float load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb << ";\n}\n";
     if (fk.has_epilogue) {
@@ -1134,6 +1529,7 @@ string gen_conv_fwd(Emitter& em, Generated* out) {
     const bool vec_fill = C % 4 == 0;                         // 16-byte pieces of a pixel's channels
     const bool literal_taps = C % 4 == 0;                     // then a k step's four values share one tap
     const bool vec_store = g.n % 4 == 0 && batch_stride % 4 == 0 && row_stride % 4 == 0;
+    if (pooled && !vec_store) return "conv forward: pooling needs 16-byte stores";
     std::ostringstream k;
     k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
     k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
@@ -1202,8 +1598,14 @@ string gen_conv_fwd(Emitter& em, Generated* out) {
     auto emit_group = [&](int64_t TG, const string& q0, const string& ind) {
         k << ind << "int pb[" << S(TG) << "];\n" << ind << "cf_float4 acc[" << S(TG) << "];\n";
         k << "#pragma unroll\n" << ind << "for (int j = 0; j < " << S(TG) << "; ++j) {\n";
-        k << ind << "    const int p = min(((" << q0 << " + j) * 4 + wv) * 16 + li, " << S(PIX - 1) << ");\n";
-        k << ind << "    pb[j] = ((p / " << S(cv.ow) << ") * " << S(PW) << " + p % " << S(cv.ow) << ") * " << S(CP) << (literal_taps ? " + lk" : "") << ";\n";
+        if (pooled) {
+            k << ind << "    const int t = (" << q0 << " + j) * 4 + wv;\n";
+            k << ind << "    pb[j] = ((2 * (t / " << S(TPR) << ") + (li >> 3)) * " << S(PW) << " + min(8 * (t % " << S(TPR) << ") + (li & 7), " << S(cv.ow - 1) << ")) * " << S(CP)
+              << (literal_taps ? " + lk" : "") << ";\n";
+        } else {
+            k << ind << "    const int p = min(((" << q0 << " + j) * 4 + wv) * 16 + li, " << S(PIX - 1) << ");\n";
+            k << ind << "    pb[j] = ((p / " << S(cv.ow) << ") * " << S(PW) << " + p % " << S(cv.ow) << ") * " << S(CP) << (literal_taps ? " + lk" : "") << ";\n";
+        }
         k << ind << "    acc[j] = (cf_float4){0.f, 0.f, 0.f, 0.f};\n" << ind << "}\n";
         k << "#pragma unroll\n" << ind << "for (int s = 0; s < " << S(steps) << "; ++s) {\n";
         if (literal_taps) {
@@ -1217,23 +1619,54 @@ string gen_conv_fwd(Emitter& em, Generated* out) {
         k << ind << "        acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fb[s], tile[pb[j] + ko], acc[j], 0, 0, 0);\n" << ind << "}\n";
         // accumulator register i of lane l is D^T[column 4 * (l / 16) + i][pixel l % 16]
         k << "#pragma unroll\n" << ind << "for (int j = 0; j < " << S(TG) << "; ++j) {\n";
-        k << ind << "    const int pp = ((" << q0 << " + j) * 4 + wv) * 16 + li, cm = img * " << S(PIX) << " + pp, cn = 4 * lk;\n";
-        k << ind << "    const int c_at = cb * " << S(batch_stride) << " + cm * " << S(row_stride) << " + cn;\n";
-        k << ind << "    if (pp < " << S(PIX) << " && cn < " << S(g.n) << ") {\n";
+        if (pooled) {
+            // every lane runs the consumer on a pixel that exists (the shuffles below need all lanes); only the lanes
+            // whose own pixel and channels exist store
+            k << ind << "    const int t = (" << q0 << " + j) * 4 + wv, yy = 2 * (t / " << S(TPR) << ") + (li >> 3), xr = 8 * (t % " << S(TPR) << ") + (li & 7);\n";
+            k << ind << "    const bool valid = xr < " << S(cv.ow) << " && 4 * lk < " << S(g.n) << ";\n";
+            k << ind << "    const int cm = img * " << S(PIX) << " + yy * " << S(cv.ow) << " + min(xr, " << S(cv.ow - 1) << "), cn = min(4 * lk, " << S(g.n - 4) << ");\n";
+            k << ind << "    const int c_at = cb * " << S(batch_stride) << " + cm * " << S(row_stride) << " + cn;\n";
+            k << ind << "    {\n";
+        } else {
+            k << ind << "    const int pp = ((" << q0 << " + j) * 4 + wv) * 16 + li, cm = img * " << S(PIX) << " + pp, cn = 4 * lk;\n";
+            k << ind << "    const int c_at = cb * " << S(batch_stride) << " + cm * " << S(row_stride) << " + cn;\n";
+            k << ind << "    if (pp < " << S(PIX) << " && cn < " << S(g.n) << ") {\n";
+        }
         if (fk.has_epilogue) {
             k << ind << "        float res[4][" << n_out << "];\n";
             k << "#pragma unroll\n" << ind << "        for (int i = 0; i < 4; ++i) mm_epilogue(acc[j][i], c_at + i, cb, cm, min(cn + i, " << S(g.n - 1) << "), res[i], "
               << em.params_pass() << ");\n";
         }
+        auto val = [&](int i, int o) { return fk.has_epilogue ? "res[" + to_string(i) + "][" + to_string(o) + "]" : "acc[j][" + to_string(i) + "]"; };
         for (int o = 0; o < n_out; ++o) {
             const string ptr = "b" + to_string(fk.outputs[o]);
-            auto val = [&](int i) { return fk.has_epilogue ? "res[" + to_string(i) + "][" + to_string(o) + "]" : "acc[j][" + to_string(i) + "]"; };
             if (vec_store) {
-                k << ind << "        *(float4*)(" << ptr << " + c_at) = make_float4(" << val(0) << ", " << val(1) << ", " << val(2) << ", " << val(3) << ");\n";
+                k << ind << "        " << (pooled ? "if (valid) " : "") << "*(float4*)(" << ptr << " + c_at) = make_float4(" << val(0, o) << ", " << val(1, o) << ", " << val(2, o) << ", "
+                  << val(3, o) << ");\n";
             } else {
                 for (int i = 0; i < 4; ++i)
-                    k << ind << "        if (cn + " << i << " < " << S(g.n) << ") " << ptr << "[c_at + " << i << "] = " << val(i) << ";\n";
+                    k << ind << "        if (cn + " << i << " < " << S(g.n) << ") " << ptr << "[c_at + " << i << "] = " << val(i, o) << ";\n";
             }
+        }
+        if (pooled) {
+            // the window's maximum: across the column pair, then across the row pair
+            k << ind << "        float pm[4];\n";
+            for (int i = 0; i < 4; ++i) {
+                k << ind << "        { float v = " << val(i, fk.pool.source) << "; v = glsl_max(v, __shfl_xor(v, 1, 64)); pm[" << i << "] = glsl_max(v, __shfl_xor(v, 8, 64)); }\n";
+            }
+            const int64_t pbs = rows ? g.n : (int64_t)cv.img * OH2 * OW2 * g.n, prs = rows ? g.batch * g.n : g.n;
+            k << ind << "        if (valid && (li & 9) == 0) {\n";
+            k << ind << "            const int p_at = cb * " << S(pbs) << " + (img * " << S(OH2 * OW2) << " + (t / " << S(TPR) << ") * " << S(OW2) << " + (xr >> 1)) * " << S(prs) << " + cn;\n";
+            if (fk.pool.has_epilogue) {
+                k << ind << "            float pres[4][" << n_pool_out << "];\n";
+                k << "#pragma unroll\n" << ind << "            for (int i = 0; i < 4; ++i) pool_epilogue(pm[i], p_at + i, pres[i], " << em.params_pass() << ");\n";
+                for (int o = 0; o < n_pool_out; ++o)
+                    k << ind << "            *(float4*)(b" << fk.outputs[n_out + o] << " + p_at) = make_float4(pres[0][" << o << "], pres[1][" << o << "], pres[2][" << o
+                      << "], pres[3][" << o << "]);\n";
+            }
+            if (fk.pool.store_pooled)
+                k << ind << "            *(float4*)(b" << fk.outputs[n_out + n_pool_out] << " + p_at) = make_float4(pm[0], pm[1], pm[2], pm[3]);\n";
+            k << ind << "        }\n";
         }
         k << ind << "    }\n" << ind << "}\n";
     };
@@ -1266,7 +1699,8 @@ string gen_conv_fwd(Emitter& em, Generated* out) {
     out->block = 256;
     out->source = k.str();
     out->note = "conv forward: workgroup per image and group, padded image tile in LDS, mfma 16x16x4, " + S(cv.fh) + "x" + S(cv.fw) + " taps x " + S(C) +
-                " channels" + (fk.has_epilogue ? " +epilogue" : "");
+                " channels" + (fk.has_epilogue ? " +epilogue" : "") +
+                (pooled ? string(" +2x2 max-pool") + (fk.pool.has_epilogue ? " with its consumer" : "") : string());
     return "";
 }
 
@@ -1997,6 +2431,7 @@ void count_work(const FusedKernel& fk, Generated* g) {
     for (auto& st : fk.row_stages) read_desc(st.k.raw(), st.inputs, -1);
     for (auto& v : fk.virtuals) read_desc(v.pe.raw(), v.inputs, -1);
     if (fk.has_epilogue) read_desc(fk.epilogue.raw(), fk.epilogue_inputs, fk.epilogue_product_input);
+    if (fk.pool.on && fk.pool.has_epilogue) read_desc(fk.pool.epilogue.raw(), fk.pool.epilogue_inputs, fk.pool.epilogue_product_input);
     // the convolution kernel reads the image itself, not the window copy its MatMul descriptor speaks of
     if (fk.cfwd.on && fk.inputs[0].buffer >= 0)
         touched[fk.inputs[0].buffer] = extent[fk.inputs[0].buffer] = (double)(fk.cfwd.img * fk.cfwd.h * fk.cfwd.w * fk.cfwd.g * fk.cfwd.c);
@@ -2015,6 +2450,19 @@ void count_work(const FusedKernel& fk, Generated* g) {
         const double ph = (double)(c.oh + c.fh - 1), pw = (double)(c.ow + c.fw - 1);
         out_each = (double)c.img * (ph - 2.0 * c.pad_h) * (pw - 2.0 * c.pad_w) * (double)(c.g * c.c);
         g->algo_flops = 2.0 * (double)c.g * (double)c.img * ph * pw * (double)(c.fh * c.fw * m.k) * (double)c.c;
+        if (c.wgrad) {
+            // the image is read as well; the filter gradient's flops are those of the MatMul it stands for
+            // (k = images x output pixels), its partials and column sums are written once per image set
+            elements += out_each;  // the image has the size of its gradient
+            g->algo_flops += 2.0 * (double)c.g * (double)(c.fh * c.fw * c.c) * (double)m.k * (double)(c.img * c.oh * c.ow);
+            elements += (double)c.chunks * (double)c.g * ((double)(c.fh * c.fw * c.c) * (double)m.k + (c.bias ? (double)m.k : 0.0));
+            elements -= out_each * (double)(fk.outputs.size() - 1);  // only the first output has the image's size
+        }
+    }
+    if (fk.pool.on) {
+        // the pooled array and what its consumer writes have a quarter of the convolution's elements
+        const double extra = (double)((fk.pool.has_epilogue ? fk.pool.epilogue.raw().n_outputs : 0) + (fk.pool.store_pooled ? 1 : 0));
+        elements -= out_each * extra * 0.75;
     }
     if (d.kind == DSC_KERNEL_SCATTER_ADD)  // read-modify-write of the entries that receive a value
         out_each = 2.0 * std::min((double)element_count(d.shape), (double)element_count(d.inputs[0].out_shape));
@@ -2065,7 +2513,9 @@ std::string FusedKernel::key() const {
         for (auto& x : v.inputs) put_src(x);
     }
     if (has_epilogue) {
-        s += "|E" + epilogue.key();
+        s += epilogue_permuted ? "|EP" : "|E";
+        if (epilogue_keeps_product) s += "K";
+        s += epilogue.key();
         s.append(reinterpret_cast<const char*>(&epilogue_product_input), 4);
         for (auto& x : epilogue_inputs) put_src(x);
     }
@@ -2084,13 +2534,24 @@ std::string FusedKernel::key() const {
     }
     if (dgrad.on) {
         s += "|D";
-        for (int64_t v : {dgrad.img, dgrad.oh, dgrad.ow, dgrad.g, dgrad.fh, dgrad.fw, dgrad.c, dgrad.pad_h, dgrad.pad_w, (int64_t)dgrad.rows_first})
+        for (int64_t v : {dgrad.img, dgrad.oh, dgrad.ow, dgrad.g, dgrad.fh, dgrad.fw, dgrad.c, dgrad.pad_h, dgrad.pad_w, (int64_t)dgrad.rows_first,
+                          (int64_t)dgrad.wgrad, (int64_t)dgrad.bias, dgrad.chunks})
             s.append(reinterpret_cast<const char*>(&v), 8);
     }
     if (cfwd.on) {
         s += "|CF";
         for (int64_t v : {cfwd.img, cfwd.h, cfwd.w, cfwd.g, cfwd.c, cfwd.fh, cfwd.fw, cfwd.oh, cfwd.ow, cfwd.pad_h, cfwd.pad_w})
             s.append(reinterpret_cast<const char*>(&v), 8);
+    }
+    if (pool.on) {
+        s += "|PL";
+        s.append(reinterpret_cast<const char*>(&pool.source), 4);
+        s += pool.store_pooled ? "S" : "-";
+        if (pool.has_epilogue) {
+            s += "E" + pool.epilogue.key();
+            s.append(reinterpret_cast<const char*>(&pool.epilogue_product_input), 4);
+            for (auto& x : pool.epilogue_inputs) put_src(x);
+        }
     }
     if (shared_scatter) s += "|SS";
     for (size_t i = 0; i < parts.size(); ++i) {
@@ -2126,6 +2587,8 @@ bool conv_dgrad_fits(const FusedKernel::ConvDgrad& c, int64_t k) {
     if (k % 4 != 0 || c.g * c.c > 64 || c.fh * c.fw * k * c.g * c.c > 8192) return false;
     return (dgrad_lds_floats(c, k) + dgrad_pitch(k) + 4) * 4 <= 64 * 1024 && c.oh + c.fh - 1 > 2 * c.pad_h && c.ow + c.fw - 1 > 2 * c.pad_w;
 }
+
+bool conv_bwd_fits(const FusedKernel::ConvDgrad& c, int64_t k) { return conv_bwd_fits_impl(c, k); }
 
 bool can_be_part(const FusedKernel& fk) {
     if (!fk.parts.empty()) return false;
@@ -2167,6 +2630,17 @@ static std::string generate_one(const FusedKernel& fk, Generated* out, bool with
         const int mk = fk.main.raw().kind;
         if (mk != DSC_KERNEL_MATMUL && mk != DSC_KERNEL_REDUCE && mk != DSC_KERNEL_WINDOWS_TO_IMAGE && mk != DSC_KERNEL_UNPAD)
             return "this kernel kind takes no epilogue";
+        if (fk.epilogue_permuted && mk != DSC_KERNEL_REDUCE) return "only a Reduce takes an epilogue through a permuting view";
+        if (fk.epilogue_keeps_product && (mk == DSC_KERNEL_MATMUL || fk.epilogue_permuted)) return "this epilogue cannot keep its product";
+        if (!fk.pool.on && (int)fk.outputs.size() != fk.epilogue.raw().n_outputs + (fk.epilogue_keeps_product ? 1 : 0)) return "epilogue output count";
+    }
+    if (fk.pool.on) {
+        if (!fk.cfwd.on) return "pooling rides on the convolution-forward kernel only";
+        if (fk.pool.has_epilogue) {
+            err = validate(fk.pool.epilogue.raw());
+            if (!err.empty()) return "pool consumer: " + err;
+            if ((int)fk.pool.epilogue_inputs.size() != fk.pool.epilogue.raw().n_inputs) return "pool consumer: input binding count";
+        }
     }
     for (auto& st : fk.row_stages) {
         err = validate(st.k.raw());
@@ -2175,7 +2649,7 @@ static std::string generate_one(const FusedKernel& fk, Generated* out, bool with
         const int n_out = st.k.raw().kind == DSC_KERNEL_PER_ELEMENT ? st.k.raw().n_outputs : 1;
         if ((int)st.outputs.size() != n_out) return "row stage: output binding count";
     }
-    if (fk.row_stages.empty() && (int)fk.inputs.size() != fk.main.raw().n_inputs) return "input binding count";
+    if (fk.row_stages.empty() && (int)fk.inputs.size() != fk.main.raw().n_inputs + (fk.dgrad.on && fk.dgrad.wgrad ? 1 : 0)) return "input binding count";
     if ((int)fk.buffer_is_output.size() != fk.n_buffers) return "buffer table size";
     err = check_sizes(fk);
     if (!err.empty()) return err;
@@ -2186,7 +2660,7 @@ static std::string generate_one(const FusedKernel& fk, Generated* out, bool with
         err = gen_row_fused(em, &g);
     } else if (fk.dgrad.on) {
         if (fk.main.raw().kind != DSC_KERNEL_MATMUL || fk.has_epilogue) return "conv dgrad: needs a plain MatMul";
-        err = gen_conv_dgrad(em, &g);
+        err = fk.dgrad.wgrad ? gen_conv_bwd(em, &g) : gen_conv_dgrad(em, &g);
     } else if (fk.cfwd.on) {
         if (fk.main.raw().kind != DSC_KERNEL_MATMUL) return "conv forward: needs a MatMul";
         err = gen_conv_fwd(em, &g);

@@ -48,6 +48,13 @@ struct FusedKernel {
     KernelDesc epilogue;
     int epilogue_product_input = -1;       // which epilogue input is the product
     std::vector<Source> epilogue_inputs;   // one per epilogue input (the product's entry is ignored)
+    // Reduce only: the epilogue reads the product through a view that is a bijection of the elements but not the
+    // identity (a weight gradient summed as [k, n] and consumed as [n, k] by its optimiser update).  The kernel then
+    // turns the index of each result into the epilogue element that reads it.
+    bool epilogue_permuted = false;
+    // Reduce, WindowsToImage, Unpad: the product has readers besides the epilogue, so the kernel stores it as well;
+    // it is the last entry of `outputs`, after the epilogue's own.
+    bool epilogue_keeps_product = false;
     // Row-fused kernel: clusters that all work on the rows of one [m, n] array with n <= 64 (a softmax
     // cross-entropy with its accuracy count: row max, exp, row sum, log, gradient, per-row loss) run as one
     // kernel.  A group of lanes owns a row, lane j holds column j of every [m, n] value, an [m]-shaped value is
@@ -74,6 +81,13 @@ struct FusedKernel {
         int64_t img = 0, oh = 0, ow = 0, g = 0, fh = 0, fw = 0, c = 0;  // windows [img, oh, ow, g, fh, fw, c]
         int64_t pad_h = 0, pad_w = 0;  // Unpads folded in (0: the output is the padded image)
         int32_t rows_first = 1;        // the Unpad along the image rows came first
+        // The filter gradient of the same convolution rides along (`wgrad`): the workgroup that holds dC of an image
+        // in LDS also takes the image's (replicate-padded) input tile and accumulates im2col^T x dC on the matrix
+        // cores, over the `chunks` (a multiple of 8) sets the images are dealt into; with `bias` the column sums of
+        // dC come out of the same products (one im2col row of ones).  Then inputs[2] is the image [img, h, w, g*c]
+        // and the outputs are {data gradient, partials [chunks, g, fh*fw*c, k], (column sums [chunks, g*k])}.
+        bool wgrad = false, bias = false;
+        int64_t chunks = 0;
     } dgrad;
     // MatMul whose A operand is the im2col of a stride-1 convolution's (replicate-padded) input: the kernel reads the
     // image [img, h, w, g*c] itself, one workgroup per (image, group) with the group's channels of the image in LDS,
@@ -83,6 +97,19 @@ struct FusedKernel {
         bool on = false;
         int64_t img = 0, h = 0, w = 0, g = 0, c = 0, fh = 0, fw = 0, oh = 0, ow = 0, pad_h = 0, pad_w = 0;
     } cfwd;
+    // Convolution-forward kernel that also max-pools what it computes (2x2 windows, stride 2): the Reduce(max) over
+    // the window copy of one of the kernel's outputs, with that Reduce's own per-element consumer where it had one
+    // (a dropout select), runs on the values while they are in registers.  The pooled array and the consumer's
+    // outputs follow the kernel's own in `outputs`: {conv outputs..., consumer outputs..., pooled (when stored)}.
+    struct ConvPool {
+        bool on = false;
+        int source = 0;                 // which of the convolution's outputs is pooled
+        bool has_epilogue = false;      // the Reduce carried a per-element consumer
+        bool store_pooled = true;       // the pooled array itself is written (no consumer, or a consumer that keeps it)
+        KernelDesc epilogue;
+        int epilogue_product_input = -1;
+        std::vector<Source> epilogue_inputs;
+    } pool;
     bool sum_chunks = false;               // MatMul: ignore the descriptor's chunk count, write one full sum
     int colsum_out = -1;                   // MatMul (MFMA template): buffer that takes the column sums of B per k chunk
     bool as_part = false;                  // generated as one part of a multi-part launch (set while the launch is generated)
@@ -118,6 +145,8 @@ std::string generate(const FusedKernel& k, Generated* out);
 // Whether the convolution data-gradient kernel can take this geometry (k = output channels per group): the image
 // tile must fit the workgroup's LDS.
 bool conv_dgrad_fits(const FusedKernel::ConvDgrad& c, int64_t k);
+// The same for the kernel that also takes the filter gradient (c.wgrad, c.bias and c.chunks set).
+bool conv_bwd_fits(const FusedKernel::ConvDgrad& c, int64_t k);
 // Whether the convolution-forward kernel takes this geometry with n output channels per group.
 bool conv_fwd_fits(const FusedKernel::ConvFwd& c, int64_t n);
 

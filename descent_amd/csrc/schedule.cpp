@@ -76,6 +76,9 @@ void for_each_source(FusedKernel& fk, F f) {
     if (fk.has_epilogue)
         for (size_t i = 0; i < fk.epilogue_inputs.size(); ++i)
             if ((int)i != fk.epilogue_product_input) f(fk.epilogue_inputs[i]);
+    if (fk.pool.on && fk.pool.has_epilogue)
+        for (size_t i = 0; i < fk.pool.epilogue_inputs.size(); ++i)
+            if ((int)i != fk.pool.epilogue_product_input) f(fk.pool.epilogue_inputs[i]);
 }
 
 // Drops pointer parameters nothing refers to and renumbers the rest.
@@ -699,11 +702,28 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
         // A per-element cluster that can run as the epilogue of the launch producing `product_node` (`elements`
         // values): it is the node's only consumer, has one invocation per product element and reads the product
         // element-for-element through a plain load.
-        auto find_epilogue = [&](int producer_idx, int product_node, int64_t elements, int* pe_idx, int* pe_input) {
+        // With `permuted` given, the view may also be any bijection of a small product's elements (a transposed or
+        // re-split reading of it); *permuted then says whether it is one.
+        // With `shared` given, the product may have further readers after the cluster (the kernel then stores the
+        // product too); *shared says whether it has.
+        auto find_epilogue = [&](int producer_idx, int product_node, int64_t elements, int* pe_idx, int* pe_input, bool* permuted = nullptr,
+                                 bool* shared = nullptr) {
             *pe_idx = *pe_input = -1;
+            if (permuted) *permuted = false;
+            if (shared) *shared = false;
             if (is_graph_output[product_node]) return;
             auto cons = consumers_of(product_node);
-            if (cons.size() != 1 || cons[0] <= producer_idx) return;
+            if (cons.empty() || cons[0] <= producer_idx) return;
+            if (cons.size() != 1) {
+                // the cluster must be the first reader, nobody may take the product over in place, and a large product
+                // only (a small one costs less as a launch part than as a second store)
+                if (!shared || elements < (1 << 16)) return;
+                for (auto& dr : drafts)
+                    if (dr.alive)
+                        for (auto& o : dr.outs)
+                            if (o.copy_from == product_node) return;
+                *shared = true;
+            }
             Draft& e = drafts[cons[0]];
             const dsc_kernel_desc& ed = e.fk.main.raw();
             if (ed.kind != DSC_KERNEL_PER_ELEMENT || e.fk.has_epilogue || ed.shape.dims[0] != elements) return;
@@ -722,7 +742,36 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                     if (src.buffer >= 0 && e.params[src.buffer] == product_node) return;
             for (auto& o : e.outs)
                 if (o.copy_from >= 0) return;
-            if (!is_contiguous(ed.inputs[input]) || taken_in_place_between(producer_idx, cons[0], input_nodes(drafts[producer_idx]))) return;
+            if (!is_contiguous(ed.inputs[input])) {
+                const dsc_view& v = ed.inputs[input];
+                if (!permuted || elements > 65536 || element_count(v.in_shape) != elements || any_clamp(v)) return;
+                // every element read exactly once, and recovered by the per-axis inverse the kernel will use
+                std::vector<char> seen((size_t)elements, 0);
+                int64_t ist[DSC_MAX_DIM], ost[DSC_MAX_DIM];
+                strides_of(v.in_shape, ist);
+                strides_of(v.out_shape, ost);
+                for (int64_t e = 0; e < elements; ++e) {
+                    int64_t cc[DSC_MAX_DIM], q = e;
+                    for (int a = v.out_shape.rank - 1; a >= 0; --a) {
+                        cc[a] = q % v.out_shape.dims[a];
+                        q /= v.out_shape.dims[a];
+                    }
+                    const int64_t r = view_index(v, cc);
+                    if (r < 0 || r >= elements || seen[(size_t)r]) return;
+                    seen[(size_t)r] = 1;
+                    int64_t back = 0;
+                    for (int j = 0; j < v.out_shape.rank; ++j) {
+                        if (v.out_shape.dims[j] <= 1 || v.map_axis[j] < 0) continue;
+                        if (v.map_step[j] <= 0) return;
+                        const int i = v.map_axis[j];
+                        back += (((r / ist[i]) % v.in_shape.dims[i]) / v.map_step[j]) % v.out_shape.dims[j] * ost[j];
+                    }
+                    if (back != e) return;
+                }
+                if (shared && *shared) return;
+                *permuted = true;
+            }
+            if (taken_in_place_between(producer_idx, cons[0], input_nodes(drafts[producer_idx]))) return;
             *pe_idx = cons[0];
             *pe_input = input;
         };
@@ -1023,6 +1072,15 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
         // (replicate-padded) image, and a MatMul over it.  The dedicated kernel reads the image itself.  The geometry
         // is a hypothesis (filter height from the divisors of k / c, padding from the output size) that is then
         // checked on every (pixel, k) of three images against the addresses the copy's view really produces.
+        // what pass 1d learns about each convolution, for pass 1e
+        struct ConvSite {
+            int copy_idx;    // draft that writes the im2col copy
+            int a_node;      // the copy
+            int image_node;  // the convolution's input [img, h, w, g*c]
+            FusedKernel::ConvFwd geo;
+            dsc_view a_view; // (group, row, k) -> element of the copy, as the forward MatMul reads it
+        };
+        std::vector<ConvSite> conv_sites;
         for (int i = 0; i < (int)drafts.size(); ++i) {
             static const bool enabled = !(std::getenv("DSC_FUSE_CONV_FWD") && std::getenv("DSC_FUSE_CONV_FWD")[0] == '0');
             if (!enabled || (flags & DSC_SCHEDULE_NO_CONV_KERNELS)) break;
@@ -1094,8 +1152,10 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                     found.fh = FH; found.fw = FW; found.oh = OH; found.ow = OW; found.pad_h = ph; found.pad_w = pw;
                 }
             }
-            if (!found.on || !conv_fwd_fits(found, g.n)) continue;
+            if (!found.on) continue;
             const int image_node = cp.params[cp.fk.inputs[0].buffer];
+            conv_sites.push_back(ConvSite{ci, a_node, image_node, found, av});
+            if (!conv_fwd_fits(found, g.n)) continue;
             if (taken_in_place_between(ci, i, {image_node})) continue;
             Draft fused = mm;
             fused.fk.cfwd = found;
@@ -1111,6 +1171,133 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                 drafts[ci].alive = false;
             }
             drafts[i] = fused;
+        }
+
+        // Pass 1e: both gradients of a convolution in one kernel.  The data-gradient kernel (pass 1c) holds dC of an
+        // image in LDS; the filter gradient im2col^T x dC of the same convolution -- by now a MatMul whose k (images x
+        // output pixels) pass 0 split into many chunks, summed by a Reduce, possibly with the bias gradient's column
+        // sums riding on it (pass 0c) -- needs the same dC and the image's input tile.  The kernel takes both: its
+        // workgroups each own a set of images, and the partial products (and column sums) come out once per set, in
+        // the layout the MatMul's chunks had, so the Reduces stay and only learn the new number of partials.
+        for (const ConvSite& site : conv_sites) {
+            static const bool enabled = !(std::getenv("DSC_FUSE_CONV_BWD") && std::getenv("DSC_FUSE_CONV_BWD")[0] == '0');
+            if (!enabled || (flags & DSC_SCHEDULE_SPLIT_CONV_GRADS)) break;
+            const FusedKernel::ConvFwd& f = site.geo;
+            int di = -1;
+            for (int q = 0; q < (int)drafts.size() && di < 0; ++q) {
+                const Draft& D = drafts[q];
+                if (!D.alive || !D.fk.dgrad.on || D.fk.dgrad.wgrad || D.fk.inputs[0].buffer < 0) continue;
+                const FusedKernel::ConvDgrad& cv = D.fk.dgrad;
+                if (cv.img == f.img && cv.oh == f.oh && cv.ow == f.ow && cv.g == f.g && cv.fh == f.fh && cv.fw == f.fw && cv.c == f.c &&
+                    cv.pad_h == f.pad_h && cv.pad_w == f.pad_w)
+                    di = q;
+            }
+            if (di < 0) continue;
+            const MatMulDims gd = matmul_dims(drafts[di].fk.main.raw());  // [g][(img, oy, ox)][oc] x [g][oc][(fy, fx, c)]
+            const int dc_node = drafts[di].params[drafts[di].fk.inputs[0].buffer];
+            int ti = -1;
+            for (int q = 0; q < (int)drafts.size() && ti < 0; ++q) {
+                const Draft& T = drafts[q];
+                const dsc_kernel_desc& td = T.fk.main.raw();
+                if (!T.alive || q == di || td.kind != DSC_KERNEL_MATMUL || !T.keep_split || !T.fk.virtuals.empty() || T.fk.has_epilogue ||
+                    td.output_mode != DSC_MATMUL_BATCHES || T.fk.dgrad.on || T.fk.cfwd.on || T.fk.inputs[0].buffer < 0 || T.fk.inputs[1].buffer < 0)
+                    continue;
+                if (T.params[T.fk.inputs[0].buffer] != site.a_node || T.params[T.fk.inputs[1].buffer] != dc_node) continue;
+                const MatMulDims gt = matmul_dims(td);
+                if (gt.batch != f.g || gt.m != f.fh * f.fw * f.c || gt.n != gd.k || gt.k != gd.m) continue;
+                // its A is the forward's A transposed, its B is the data gradient's A: same elements of the same nodes
+                int64_t bt, bf, ct[DSC_MAX_DIM], cf[DSC_MAX_DIM];
+                if (!affine_form(td.inputs[0], &bt, ct) || !affine_form(site.a_view, &bf, cf) || bt != bf || ct[1] != cf[2] || ct[2] != cf[1] ||
+                    (gt.batch > 1 && ct[0] != cf[0]))
+                    continue;
+                if (!affine_form(td.inputs[1], &bt, ct) || !affine_form(drafts[di].fk.main.raw().inputs[0], &bf, cf) || bt != bf || ct[1] != cf[1] ||
+                    ct[2] != cf[2] || (gt.batch > 1 && ct[0] != cf[0]))
+                    continue;
+                ti = q;
+            }
+            if (ti < 0) continue;
+            Draft& T = drafts[ti];
+            const MatMulDims gt = matmul_dims(T.fk.main.raw());
+            const bool bias = T.fk.colsum_out >= 0;
+            if ((int)T.outs.size() != (bias ? 2 : 1) || T.outs[0].copy_from >= 0 || is_graph_output[T.outs[0].node]) continue;
+            // the Reduces over the partials and over the column sums
+            auto only_reduce_of = [&](int node) {
+                auto cons = consumers_of(node);
+                if (cons.size() != 1 || cons[0] <= ti) return -1;
+                const Draft& r = drafts[cons[0]];
+                const dsc_kernel_desc& rd = r.fk.main.raw();
+                if (rd.kind != DSC_KERNEL_REDUCE || rd.reduce_op != DSC_REDUCE_SUM || !r.fk.virtuals.empty() || r.fk.has_epilogue) return -1;
+                return cons[0];
+            };
+            const int r1 = only_reduce_of(T.outs[0].node);
+            if (r1 < 0) continue;
+            {
+                const dsc_kernel_desc& rd = drafts[r1].fk.main.raw();
+                if (rd.axis != 0 || !is_identity(rd.inputs[0]) || rd.inputs[0].in_shape.dims[0] != gt.chunks ||
+                    element_count(rd.inputs[0].in_shape) != gt.chunks * gt.batch * gt.m * gt.n)
+                    continue;
+            }
+            int r2 = -1;
+            if (bias) {
+                if (is_graph_output[T.outs[1].node]) continue;
+                r2 = only_reduce_of(T.outs[1].node);
+                if (r2 < 0) continue;
+                const dsc_kernel_desc& rd = drafts[r2].fk.main.raw();
+                const dsc_view& pv = rd.inputs[0];
+                if (pv.in_shape.rank != 2 || pv.in_shape.dims[0] != gt.chunks || pv.in_shape.dims[1] != gt.batch * gt.n ||
+                    pv.out_shape.dims[rd.axis] != gt.chunks || (gt.chunks > 1 && pv.map_axis[rd.axis] != 0))
+                    continue;
+            }
+            const int at = std::min(di, ti), other = std::max(di, ti);
+            {
+                std::vector<int> reads = input_nodes(drafts[di]);
+                reads.push_back(site.image_node);
+                if (taken_in_place_between(at, other, reads)) continue;
+            }
+            // image sets: about a thousand workgroups, a multiple of eight sets
+            // (measured on the ConvNet's second convolution, 2000 image-groups: ~1000 workgroups 38.8 us, ~2000 43.9, ~500 43.1)
+            const int64_t per_group = std::max<int64_t>(8, 1024 / f.g);
+            const int64_t images_per_set = (f.img + per_group - 1) / per_group;
+            const int64_t sets = ((f.img + images_per_set - 1) / images_per_set + 7) / 8 * 8;
+            Draft fused = drafts[di];
+            fused.fk.dgrad.wgrad = true;
+            fused.fk.dgrad.bias = bias;
+            fused.fk.dgrad.chunks = sets;
+            {
+                Source xs;
+                xs.buffer = param_index(fused, site.image_node, false);
+                fused.fk.inputs.push_back(xs);
+            }
+            for (auto& o : T.outs) {
+                fused.fk.outputs.push_back(param_index(fused, o.node, true));
+                fused.outs.push_back(o);
+            }
+            if (!conv_bwd_fits(fused.fk.dgrad, gd.k)) continue;
+            {
+                Generated probe;
+                if (!generate(fused.fk, &probe).empty()) continue;
+            }
+            fused.covers.insert(fused.covers.end(), T.covers.begin(), T.covers.end());
+            // the Reduces sum `sets` partials now
+            node_bytes[T.outs[0].node] = (size_t)(sets * gt.batch * gt.m * gt.n) * 4;
+            drafts[r1].fk.main.inputs[0].in_shape.dims[0] = sets;
+            drafts[r1].fk.main.inputs[0].out_shape.dims[0] = sets;
+            if (bias) {
+                node_bytes[T.outs[1].node] = (size_t)(sets * gt.batch * gt.n) * 4;
+                const int axis = drafts[r2].fk.main.raw().axis;
+                dsc_view& pv = drafts[r2].fk.main.inputs[0];
+                pv.in_shape.dims[0] = sets;
+                pv.out_shape.dims[axis] = sets;
+                pv.map_axis[axis] = 0;
+                pv.map_step[axis] = 1;
+            }
+            drafts[other].alive = false;
+            drafts[at] = fused;
+            // the im2col copy has lost a reader; with the last one it goes
+            if (drafts[site.copy_idx].alive && consumers_of(site.a_node).empty()) {
+                drafts[at].covers.insert(drafts[at].covers.end(), drafts[site.copy_idx].covers.begin(), drafts[site.copy_idx].covers.end());
+                drafts[site.copy_idx].alive = false;
+            }
         }
 
         // Pass 1b: clusters that all work on the rows of one [m, n] array with a short n -- Reduces along n and the
@@ -1302,6 +1489,9 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                     // a MatMul that sums its B operand's columns on the side took over the operand's other reader: the
                     // operand stays a buffer, as it was when two launches read it
                     if (q.fk.colsum_out >= 0 && q.fk.inputs[1].buffer >= 0 && q.params[q.fk.inputs[1].buffer] == node) ok = false;
+                    // the kernel that takes both gradients of a convolution requests dC of its next image while it
+                    // works on the current one: plain loads, nothing evaluated in between
+                    if (q.fk.dgrad.on && q.fk.dgrad.wgrad && q.fk.inputs[0].buffer >= 0 && q.params[q.fk.inputs[0].buffer] == node) ok = false;
                     // an epilogue reads its product from the accumulator, never through a producer
                     if (q.fk.has_epilogue && q.fk.epilogue_product_input >= 0) {
                         const Source& ps = q.fk.epilogue_inputs[q.fk.epilogue_product_input];
@@ -1345,12 +1535,14 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                 r.keep_output || !r.fk.row_stages.empty())
                 continue;
             int pe_idx = -1, pe_input = -1;
-            find_epilogue(i, r.outs[0].node, element_count(r.fk.main.raw().shape), &pe_idx, &pe_input);
+            bool permuted = false, shared = false;
+            find_epilogue(i, r.outs[0].node, element_count(r.fk.main.raw().shape), &pe_idx, &pe_input, rk == DSC_KERNEL_REDUCE ? &permuted : nullptr, &shared);
             if (pe_idx < 0) continue;
             Draft& e = drafts[pe_idx];
             if ((int)r.fk.virtuals.size() + (int)e.fk.virtuals.size() > 8) continue;
             Draft fused;
             fused.fk.main = r.fk.main;
+            fused.fk.epilogue_permuted = permuted;
             const int voff = import_virtuals(fused, r);
             for (auto& src : r.fk.inputs) fused.fk.inputs.push_back(import_source(fused, r, src, voff));
             fused.covers = r.covers;
@@ -1366,10 +1558,150 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                 fused.fk.outputs.push_back(param_index(fused, o.node, true));
                 fused.outs.push_back(o);
             }
+            if (shared) {
+                fused.fk.epilogue_keeps_product = true;
+                fused.fk.outputs.push_back(param_index(fused, r.outs[0].node, true));
+                fused.outs.push_back(r.outs[0]);
+            }
             fused.covers.insert(fused.covers.end(), e.covers.begin(), e.covers.end());
             compact(fused);
             r.alive = false;
             drafts[pe_idx] = fused;  // runs where the per-element cluster ran: all of its inputs exist by then
+        }
+
+        // Pass 3c: max-pooling joins the convolution that feeds it.  By now the pooling is a Reduce(max) over four
+        // window elements whose input is a fused producer -- the window copy of the convolution kernel's (activated)
+        // output -- possibly with a per-element consumer of its own (pass 3: a dropout select).  The convolution
+        // kernel has those values in registers: it takes the maximum over each 2x2 window with two shuffles and runs the
+        // consumer, and the convolution's output is not read back.  The geometry is checked element by element: every
+        // pooled element of three images must read exactly the four window elements the kernel will combine.
+        for (int ri = 0; ri < (int)drafts.size(); ++ri) {
+            static const bool enabled = !(std::getenv("DSC_FUSE_CONV_POOL") && std::getenv("DSC_FUSE_CONV_POOL")[0] == '0');
+            if (!enabled || (flags & DSC_SCHEDULE_NO_CONV_KERNELS)) break;
+            Draft& R = drafts[ri];
+            const dsc_kernel_desc& rd = R.fk.main.raw();
+            if (!R.alive || rd.kind != DSC_KERNEL_REDUCE || rd.reduce_op != DSC_REDUCE_MAX || R.fk.virtuals.size() != 1 || R.fk.epilogue_permuted ||
+                !R.fk.row_stages.empty() || R.fk.inputs[0].virt != 0 || R.keep_output || rd.inputs[0].out_shape.dims[rd.axis] != 4)
+                continue;
+            const Virtual& win = R.fk.virtuals[0];
+            const dsc_kernel_desc& wd = win.pe.raw();
+            if (wd.kind != DSC_KERNEL_PER_ELEMENT || wd.n_inputs != 1 || win.inputs[0].buffer < 0) continue;
+            {
+                int loads = 0;
+                bool copy = true;
+                for (int q = 0; q < wd.n_ops; ++q) {
+                    if (wd.ops[q].kind == DSC_PE_LOAD) ++loads;
+                    else if (!(wd.ops[q].kind == DSC_PE_UNARY && wd.ops[q].op == DSC_UN_MOV)) copy = false;
+                }
+                if (!copy || loads != 1) continue;
+            }
+            const int x_node = R.params[win.inputs[0].buffer];
+            int fi = -1, source = -1;
+            for (int q = 0; q < ri && fi < 0; ++q) {
+                if (!drafts[q].alive || !drafts[q].fk.cfwd.on || drafts[q].fk.pool.on) continue;
+                for (size_t o = 0; o < drafts[q].outs.size(); ++o)
+                    if (drafts[q].outs[o].node == x_node) { fi = q; source = (int)o; }
+            }
+            if (fi < 0) continue;
+            Draft& F = drafts[fi];
+            const FusedKernel::ConvFwd& cv = F.fk.cfwd;
+            const dsc_kernel_desc& fd = F.fk.main.raw();
+            const MatMulDims g = matmul_dims(fd);
+            const bool rows = fd.output_mode == DSC_MATMUL_ROWS;
+            const int64_t batch_stride = rows ? g.n : g.m * g.n, row_stride = rows ? g.batch * g.n : g.n;
+            if (cv.oh % 2 || cv.ow % 2 || g.n % 4 || batch_stride % 4 || row_stride % 4) continue;
+            const int64_t OH2 = cv.oh / 2, OW2 = cv.ow / 2, pooled_elems = cv.img * OH2 * OW2 * g.batch * g.n;
+            if (element_count(rd.shape) != pooled_elems || element_count(wd.inputs[0].in_shape) != cv.img * cv.oh * cv.ow * g.batch * g.n) continue;
+            const int64_t pbs = rows ? g.n : cv.img * OH2 * OW2 * g.n, prs = rows ? g.batch * g.n : g.n;
+            // pooled element -> the four elements of x it reads, through the Reduce's view and the window copy's view
+            const dsc_view& rv = rd.inputs[0];
+            const dsc_view& wv = wd.inputs[0];
+            auto sources_of = [&](int64_t e, int64_t* out4) {
+                int64_t oc[DSC_MAX_DIM], q = e;
+                for (int a = rd.shape.rank - 1; a >= 0; --a) {
+                    oc[a] = q % rd.shape.dims[a];
+                    q /= rd.shape.dims[a];
+                }
+                for (int64_t w = 0; w < 4; ++w) {
+                    int64_t rc[DSC_MAX_DIM];
+                    for (int a = 0; a < rv.out_shape.rank; ++a) rc[a] = a == rd.axis ? w : oc[a];
+                    int64_t idx = view_index_clamped(rv, rc), cc[DSC_MAX_DIM];
+                    for (int a = wv.out_shape.rank - 1; a >= 0; --a) {
+                        cc[a] = idx % wv.out_shape.dims[a];
+                        idx /= wv.out_shape.dims[a];
+                    }
+                    out4[w] = view_index_clamped(wv, cc);
+                }
+                std::sort(out4, out4 + 4);
+            };
+            if (rv.out_shape.rank != rd.shape.rank || element_count(rv.in_shape) != element_count(wv.out_shape)) continue;
+            bool ok = true;
+            for (int64_t img : {(int64_t)0, cv.img / 2, cv.img - 1})
+                for (int64_t yp = 0; yp < OH2 && ok; ++yp)
+                    for (int64_t xp = 0; xp < OW2 && ok; ++xp)
+                        for (int64_t cb = 0; cb < g.batch && ok; ++cb)
+                            for (int64_t cn = 0; cn < g.n && ok; ++cn) {
+                                const int64_t e = cb * pbs + (img * OH2 * OW2 + yp * OW2 + xp) * prs + cn;
+                                int64_t got[4], want[4];
+                                sources_of(e, got);
+                                for (int64_t w = 0; w < 4; ++w)
+                                    want[w] = cb * batch_stride + (img * cv.oh * cv.ow + (2 * yp + w / 2) * cv.ow + 2 * xp + w % 2) * row_stride + cn;
+                                std::sort(want, want + 4);
+                                for (int w = 0; w < 4; ++w)
+                                    if (got[w] != want[w]) ok = false;
+                            }
+            if (!ok) continue;
+            // the Reduce's consumer (if any) moves to where the convolution runs: what it reads must exist by then
+            std::vector<int> produced_before(n_nodes, 0);
+            for (int q = 0; q < fi; ++q)
+                if (drafts[q].alive)
+                    for (auto& o : drafts[q].outs) produced_before[o.node] = 1;
+            for (int nd : input_nodes(R)) {
+                if (nd == x_node) continue;
+                if (!is_graph_input[nd] && !produced_before[nd]) ok = false;
+            }
+            for (auto& o : R.outs)
+                if (o.copy_from >= 0) ok = false;
+            if (!ok || taken_in_place_between(fi, ri, input_nodes(R)) || taken_in_place_between(fi, ri, input_nodes(F))) continue;
+            Draft fused = F;
+            fused.fk.pool.on = true;
+            fused.fk.pool.source = source;
+            fused.fk.pool.has_epilogue = R.fk.has_epilogue;
+            fused.fk.pool.store_pooled = !R.fk.has_epilogue || R.fk.epilogue_keeps_product;
+            if (R.fk.has_epilogue) {
+                fused.fk.pool.epilogue = R.fk.epilogue;
+                fused.fk.pool.epilogue_product_input = R.fk.epilogue_product_input;
+                // (R's only fused producer is the window copy, which the Reduce's main input used: the consumer's own
+                // inputs are buffers)
+                bool plain = true;
+                for (size_t q = 0; q < R.fk.epilogue_inputs.size(); ++q) {
+                    if ((int)q == R.fk.epilogue_product_input) {
+                        fused.fk.pool.epilogue_inputs.push_back(Source{});
+                        continue;
+                    }
+                    if (R.fk.epilogue_inputs[q].buffer < 0) plain = false;
+                    else fused.fk.pool.epilogue_inputs.push_back(import_source(fused, R, R.fk.epilogue_inputs[q], 0));
+                }
+                if (!plain) continue;
+            }
+            // outputs: the convolution's, then the consumer's, then the pooled array
+            const int n_epi = R.fk.has_epilogue ? R.fk.epilogue.raw().n_outputs : 0;
+            for (int o = 0; o < n_epi; ++o) {
+                fused.fk.outputs.push_back(param_index(fused, R.outs[o].node, true));
+                fused.outs.push_back(R.outs[o]);
+            }
+            if (fused.fk.pool.store_pooled) {
+                const StepOutput& po = R.outs[n_epi];
+                fused.fk.outputs.push_back(param_index(fused, po.node, true));
+                fused.outs.push_back(po);
+            }
+            {
+                Generated probe;
+                if (!generate(fused.fk, &probe).empty()) continue;
+            }
+            fused.covers.insert(fused.covers.end(), R.covers.begin(), R.covers.end());
+            R.alive = false;
+            drafts[fi] = fused;
         }
 
         // Pass 3b: ScatterAdds chained through one accumulator (each takes the previous one's result in place:

@@ -140,12 +140,15 @@ def cache_stats():
 
 def schedule_flags(fused) -> int:
     """`fused`: True (all fusion), False (one launch per reference cluster), "generic-conv" (all fusion, but
-    convolutions stay on the generic MatMul path instead of the dedicated kernels), or "graph-replay"
-    (all fusion, each run captured as a HIP graph and replayed when the buffers land on the same addresses)."""
+    convolutions stay on the generic MatMul path instead of the dedicated kernels), "graph-replay"
+    (all fusion, each run captured as a HIP graph and replayed when the buffers land on the same addresses), or
+    "split-conv-grads" (all fusion, but a convolution's data and filter gradients stay two kernels)."""
     if fused == "generic-conv":
         return _abi.SCHEDULE_NO_CONV_KERNELS
     if fused == "graph-replay":
         return _abi.SCHEDULE_GRAPH_REPLAY
+    if fused == "split-conv-grads":
+        return _abi.SCHEDULE_SPLIT_CONV_GRADS
     return 0 if fused else _abi.SCHEDULE_NO_FUSION
 
 

@@ -338,6 +338,10 @@ typedef struct dsc_schedule dsc_schedule;
                                            (fused producers) instead of the dedicated LDS-tiled kernels (for
                                            parity tests) */
 
+#define DSC_SCHEDULE_SPLIT_CONV_GRADS 8u /* a convolution's data gradient and filter gradient stay two kernels (the
+                                           dedicated data-gradient kernel and the tall-k MatMul) instead of sharing
+                                           the one that holds dC and the input tile in LDS (for parity tests) */
+
 int dsc_schedule_create(dsc_ctx* ctx, const dsc_schedule_desc* desc, uint32_t flags, dsc_schedule** out);
 int dsc_schedule_destroy(dsc_ctx* ctx, dsc_schedule* s);
 /* Environment::run (environment.rs:326-516). `params[slot]` holds each parameter's current buffer (0 if

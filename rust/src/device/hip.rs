@@ -49,6 +49,7 @@ pub const DSC_PE_GATHER: i32 = 8;
 pub const DSC_SCHEDULE_NO_FUSION: u32 = 1;
 pub const DSC_SCHEDULE_NO_CONV_KERNELS: u32 = 2;
 pub const DSC_SCHEDULE_GRAPH_REPLAY: u32 = 4;
+pub const DSC_SCHEDULE_SPLIT_CONV_GRADS: u32 = 8;
 
 #[repr(C)]
 #[derive(Clone, Copy)]

@@ -289,7 +289,7 @@ def test_softmax_cross_entropy_runs_as_one_row_fused_launch(hip_backend_session,
     assert np.array_equal(ga, ca)  # arg-max derived: exact, ties included
 
 
-@pytest.mark.parametrize("fused", [True, "generic-conv"])
+@pytest.mark.parametrize("fused", [True, "split-conv-grads", "generic-conv"])
 def test_convnet_step_at_batch_64_vs_oracle(hip_backend_session, fused):
     """At this batch the convolution GEMMs are large enough for the row-per-thread kernels.  The data gradient of
     the second convolution runs either as the dedicated kernel (MatMul + reshape copy + WindowsToImage + both
@@ -305,6 +305,8 @@ def test_convnet_step_at_batch_64_vs_oracle(hip_backend_session, fused):
         cenv.run(cw.graph, 500 + step)
     listing = next(iter(gw.graph.__dict__["_schedules"].values())).describe()
     if fused is True:
+        assert "ConvBackward" in listing and "filter gradient mfma 16x16x4 5x1 tiles" in listing, listing
+    elif fused == "split-conv-grads":
         assert "ConvDataGrad" in listing and "3x3 taps x 16 channels, border folds fused" in listing, listing
     else:
         assert "MatMul (k=144) [1, 16384, 2, 8]" in listing and "row-per-thread" in listing, listing
@@ -442,6 +444,7 @@ CONV_GEOMETRIES = [
     (30, 20, 20, 4, 4, 3, 3, 1, 1),     # padded image larger than one pass of 256 pixels
     (60, 8, 8, 4, 8, 3, 3, 0, 1),       # no padding: no Unpads to fold
     (25, 7, 5, 16, 16, 3, 1, 0, 1),     # 3x1 taps
+    (40, 10, 10, 6, 8, 3, 3, 1, 1),     # six channels: the data gradient stays on the vector units beside the filter gradient
     (3, 6, 6, 64, 64, 3, 3, 1, 1),      # many channels: stays on the generic path
     (20, 10, 10, 3, 6, 3, 3, 1, 1),     # three input channels, six outputs: no 16-byte pieces anywhere
     (16, 8, 8, 6, 20, 3, 3, 1, 2),      # the same per group, ten outputs
@@ -451,17 +454,20 @@ CONV_WITHOUT_FORWARD_KERNEL = {CONV_GEOMETRIES[-3]}
 
 
 @pytest.mark.parametrize("geom", CONV_GEOMETRIES, ids=lambda g: "x".join(map(str, g)))
-@pytest.mark.parametrize("fused", [True, "generic-conv", False])
+@pytest.mark.parametrize("fused", [True, "split-conv-grads", "generic-conv", False])
 def test_conv2d_gradients_over_geometries(hip_backend_session, geom, fused):
     genv, cenv = _envs(hip_backend_session, fused=fused)
     g, gy, gdx, gdf = _conv_grad_case(genv, *geom, seed=90)
     _, cy, cdx, cdf = _conv_grad_case(cenv, *geom, seed=90)
     listing = next(iter(g.__dict__["_schedules"].values())).describe()
-    if fused is True:  # the dedicated kernels: image tile in LDS
-        assert ("ConvDataGrad" in listing) == (geom not in CONV_WITHOUT_DATA_GRAD_KERNEL), listing
+    if fused in (True, "split-conv-grads"):  # the dedicated kernels: image tile in LDS
+        # (the data gradient alone, or together with the filter gradient where that one's k is long enough to be split)
+        assert ("ConvDataGrad" in listing or "ConvBackward" in listing) == (geom not in CONV_WITHOUT_DATA_GRAD_KERNEL), listing
         assert ("ConvForward" in listing) == (geom not in CONV_WITHOUT_FORWARD_KERNEL), listing
+    if fused == "split-conv-grads":
+        assert "ConvBackward" not in listing, listing
     if fused == "generic-conv":
-        assert "ConvDataGrad" not in listing and "ConvForward" not in listing, listing
+        assert "ConvDataGrad" not in listing and "ConvBackward" not in listing and "ConvForward" not in listing, listing
     assert rel_l2(gy, cy) <= TOL, listing
     assert rel_l2(gdx, cdx) <= TOL, (rel_l2(gdx, cdx), listing)
     assert rel_l2(gdf, cdf) <= TOL, (rel_l2(gdf, cdf), listing)
@@ -589,7 +595,7 @@ def test_schedule_dot_export_and_launch_labels(hip_backend_session):
     launches, _ = sched.launch_count()
     assert dot.startswith("digraph schedule {") and dot.rstrip().endswith("}")
     assert dot.count("[shape=box,style=filled") == launches
-    assert "ConvDataGrad" in dot and "RowFused" in dot
+    assert "ConvBackward" in dot and "RowFused" in dot
     assert dot.count("peripheries=2") == len(w.trainable) + len(w.state) + len(w.scalars)
     assert dot.count("{") == dot.count("}") and dot.count('"') % 2 == 0
     before = w.snapshot()

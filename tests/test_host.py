@@ -220,7 +220,10 @@ def test_convnet_graph_shape():
     assert set(covered) == set(range(66))
     # the data gradient of the second convolution: MatMul + reshape copy + WindowsToImage as one product over
     # the padded image, both operands fused producers
-    assert "ConvDataGrad" in listing and "conv data gradient: workgroup per image and group, tile in LDS, 3x3 taps x 16 channels, border folds fused" in listing
+    assert "ConvBackward" in listing and "data gradient 3x3 taps x 16 channels with border folds, filter gradient mfma 16x16x4 5x1 tiles +column sums of dC" in listing
+    split = hip_backend.check_schedule(w.graph, fused="split-conv-grads")
+    assert "ConvDataGrad" in split and "conv data gradient: workgroup per image and group, tile in LDS, 3x3 taps x 16 channels, border folds fused" in split
+    assert "tall-k mfma 16x16x4, 5x1 tiles" in split and "ConvBackward" not in split
     # the classifier head (1000 x 128 -> 10): lanes share a row's k range, no MFMA tile grid of 32 single-wave workgroups
     assert "MatMul (k=128) [1, 1, 1000, 10] + PerElement (3 ops) [10000]  [dot products: 16 lanes per row, B in LDS +epilogue]" in listing
     # both forward convolutions: the image tile goes to LDS, the im2col copy stays only for the filter gradient
