@@ -1904,7 +1904,9 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
 }
 
 int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
-    // environment.rs:326-516, over the fused steps
+    // environment.rs:326-516, over the fused steps.  Unlike the reference (which panics), a run that cannot be put
+    // together leaves `params` and the caller's buffers as they were: until every launch's pointers are resolved
+    // nothing the caller owns is released or handed on, and what the attempt allocated is given back.
     std::vector<int> usage(n_nodes, 0);
     std::vector<dsc_buf> buffer(n_nodes, 0);
     for (auto& st : steps)
@@ -1917,21 +1919,14 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
     for (auto& io : outputs) param_is_output[io.param] = true;
     for (auto& io : inputs) param_is_input[io.param] = true;
 
+    std::set<dsc_buf> callers;  // buffers the caller handed in: released only once the run is certain to go ahead
+    const std::vector<dsc_buf> handed_in(params, params + n_params);
+    for (int i = 0; i < n_params; ++i)
+        if (params[i]) callers.insert(params[i]);
     for (auto& io : inputs) {
         if (params[io.param] == 0) return fail(DSC_ERR_INVALID, "schedule run: an input parameter has no buffer");
-        if (!param_is_output[io.param]) {
-            buffer[io.node] = params[io.param];
-            usage[io.node] += 1;  // pinned: the parameter keeps its buffer
-        } else {
-            buffer[io.node] = params[io.param];
-            params[io.param] = 0;
-        }
-    }
-    for (auto& io : outputs) {
-        if (!param_is_input[io.param] && params[io.param] != 0) {
-            ctx->heap.free(params[io.param]);
-            params[io.param] = 0;
-        }
+        buffer[io.node] = params[io.param];
+        if (!param_is_output[io.param]) usage[io.node] += 1;  // pinned: the parameter keeps its buffer
     }
 
     // Pass 1: buffer bookkeeping only -- resolve every launch's pointers (allocation and release are host-side
@@ -1945,11 +1940,21 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
     std::vector<void*> pointers;
     launches.reserve(steps.size() + 4);
     std::vector<dsc_buf> prefilled(prefills.empty() ? 0 : n_nodes, 0);
+    auto give_up = [&](int status, const std::string& msg) {
+        for (dsc_buf h : buffer)
+            if (h && !callers.count(h)) ctx->heap.free(h);
+        for (dsc_buf h : prefilled)
+            if (h) ctx->heap.free(h);
+        return fail(status, msg);
+    };
+    auto release = [&](dsc_buf h) {
+        if (!callers.count(h)) ctx->heap.free(h);
+    };
     for (auto& pf : prefills) {
         launches.push_back(Launch{pf.kernel, pointers.size(), (int)pf.nodes.size()});
         for (int node : pf.nodes) {
             const dsc_buf h = ctx->heap.alloc(node_bytes[node]);
-            if (!h) return fail(DSC_ERR_OOM, "schedule run: out of device memory");
+            if (!h) return give_up(DSC_ERR_OOM, "schedule run: out of device memory");
             void* p = nullptr;
             ctx->heap.info(h, &p, nullptr);
             pointers.push_back(p);
@@ -1962,9 +1967,9 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
             dsc_buf h = 0;
             if (o.copy_from < 0) {
                 h = ctx->heap.alloc(node_bytes[o.node]);
-                if (!h) return fail(DSC_ERR_OOM, "schedule run: out of device memory");
+                if (!h) return give_up(DSC_ERR_OOM, "schedule run: out of device memory");
             } else {
-                if (usage[o.copy_from] != 0) return fail(DSC_ERR_UNSUPPORTED, "schedule run: accumulator source still in use (deep copy)");
+                if (usage[o.copy_from] != 0) return give_up(DSC_ERR_UNSUPPORTED, "schedule run: accumulator source still in use (deep copy)");
                 if (buffer[o.copy_from] != 0) {
                     h = buffer[o.copy_from];
                     buffer[o.copy_from] = 0;
@@ -1973,16 +1978,19 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
                     prefilled[o.node] = 0;
                 } else if (o.from_literal) {
                     h = ctx->heap.alloc(node_bytes[o.node]);
-                    if (!h) return fail(DSC_ERR_OOM, "schedule run: out of device memory");
+                    if (!h) return give_up(DSC_ERR_OOM, "schedule run: out of device memory");
                     void* p = nullptr;
                     ctx->heap.info(h, &p, nullptr);
                     launches.push_back(Launch{o.fill, pointers.size(), 1});
                     pointers.push_back(p);
                 } else {
-                    return fail(DSC_ERR_INVALID, "schedule run: cannot copy-on-write node");
+                    return give_up(DSC_ERR_INVALID, "schedule run: cannot copy-on-write node");
                 }
             }
-            if (buffer[o.node] != 0) return fail(DSC_ERR_INVALID, "schedule run: node written twice");
+            if (buffer[o.node] != 0) {
+                if (!callers.count(h)) ctx->heap.free(h);
+                return give_up(DSC_ERR_INVALID, "schedule run: node written twice");
+            }
             buffer[o.node] = h;
         }
         const int n = (int)st.params.size();
@@ -1990,20 +1998,32 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
         for (int i = 0; i < n; ++i) {
             void* p = nullptr;
             if (!ctx->heap.info(buffer[st.params[i]], &p, nullptr))
-                return fail(DSC_ERR_INVALID, "schedule run: node " + std::to_string(st.params[i]) + " has no buffer at '" + st.kernel->label + "'");
+                return give_up(DSC_ERR_INVALID, "schedule run: node " + std::to_string(st.params[i]) + " has no buffer at '" + st.kernel->label + "'");
             pointers.push_back(p);
         }
         for (int nd : st.inputs) {
             if (usage[nd] == 0 && buffer[nd] != 0) {
-                ctx->heap.free(buffer[nd]);
+                release(buffer[nd]);
                 buffer[nd] = 0;
             }
         }
     }
+    for (auto& io : outputs)
+        if (buffer[io.node] == 0) return give_up(DSC_ERR_INVALID, "schedule run: output node has no buffer");
+    // from here on the run goes ahead: parameters that are rewritten give their old buffers up, outputs move in
+    for (auto& io : inputs)
+        if (param_is_output[io.param]) params[io.param] = 0;
     for (auto& io : outputs) {
-        if (buffer[io.node] == 0) return fail(DSC_ERR_INVALID, "schedule run: output node has no buffer");
+        if (!param_is_input[io.param]) params[io.param] = 0;
         params[io.param] = buffer[io.node];
         buffer[io.node] = 0;
+    }
+    // a rewritten parameter's old buffer goes back to the heap, unless it was taken over in place and is some
+    // parameter's new value
+    {
+        const std::set<dsc_buf> kept(params, params + n_params);
+        for (int i = 0; i < n_params; ++i)
+            if (param_is_output[i] && handed_in[i] && !kept.count(handed_in[i])) ctx->heap.free(handed_in[i]);
     }
 
     // Pass 2: enqueue.  With per-launch timing on, or graphs off, launch one by one; otherwise replay the graph

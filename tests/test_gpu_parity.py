@@ -679,3 +679,37 @@ def test_long_loop_keeps_device_and_host_memory_bounded(hip_backend_session):
     assert np.isfinite(out[0])
     for a in px + [out]:
         be.host_release(a)
+
+
+def test_a_run_that_cannot_be_put_together_changes_nothing(hip_backend_session):
+    """One parameter's buffer handle is stale (freed behind the schedule's back), which the run only notices when it
+    resolves the pointers of the launch that reads it, several launches and allocations into its bookkeeping.  The
+    call must fail with every other handle untouched, every trainable value intact and no buffer leaked; the same
+    schedule then runs normally once the parameter has a buffer again."""
+    from descent_amd import Environment, workloads
+    from descent_amd.hip_backend import DescentHipError
+
+    be = hip_backend_session
+    env = Environment(be)
+    w = workloads.convnet(env, batch=16, seed=4)
+    env.run(w.graph, 1)
+    be.sync()
+    sched = next(iter(w.graph.__dict__["_schedules"].values()))
+    before = w.snapshot()
+    y = w.inputs["y"]
+    labels = env.read_parameter(y)
+    handles = [p.buffer for p in sched.params]
+    be.free(y.buffer)  # the handle in `handles` is now stale
+    live = be.heap_stats()[0]
+    with pytest.raises(DescentHipError):
+        sched.run(list(handles), 2)
+    assert be.heap_stats()[0] == live  # what the attempt allocated was given back
+    assert [sched._slots[i] for i in range(len(handles))] == handles  # the parameter table the library was given
+    y.buffer = None
+    env.write_parameter(y, labels)
+    after = w.snapshot()
+    for key in before:
+        assert np.array_equal(before[key].view(np.uint32), after[key].view(np.uint32)), key
+    env.run(w.graph, 2)
+    be.sync()
+    assert np.all(np.isfinite(w.snapshot()["loss"]))
