@@ -673,7 +673,7 @@ string gen_reduce(Emitter& em, Generated* out) {
         k << "    if (vid < " << S(n_vec) << "u) {\n";
         k << "    const uint oid = vid * 4u;\n";
         auto oc = em.emit_coords(k, d.shape, "oid", "oc");
-        const int U = pick_unroll(TK, std::getenv("DSC_REDUCE_VEC_UNROLL") ? std::atoi(std::getenv("DSC_REDUCE_VEC_UNROLL")) : 16);
+        const int U = pick_unroll(TK, 16);
         const char* comps[4] = {"x", "y", "z", "w"};
         for (int u = 0; u < U; ++u) k << (u ? ", a" : "    float4 a") << u << " = result";
         k << ";\n    int kb = " << (TK > 1 ? "tk" : "0") << ";\n";
@@ -1951,15 +1951,13 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
     const dsc_view& vb = d.inputs[1];
     const bool rows = d.output_mode == DSC_MATMUL_ROWS;
     const int64_t batch_stride = rows ? g.n : g.m * g.n, row_stride = rows ? g.batch * g.n : g.n;
-    // Tuning hooks.  Measured on MI355X on the ConvNet's k=72 product (196000 x 2 x 16): one row per thread,
-    // k unrolled by 8 and B through the scalar unit 35 us; B in LDS 40 us; two / four rows per thread 41 / 46 us.
-    int R = 1;  // rows per thread
-    if (const char* e = std::getenv("DSC_ROWS_R")) R = std::max(1, std::min(8, std::atoi(e)));
-    int unroll = g.k <= 16 ? (int)g.k : 8;
-    if (const char* e = std::getenv("DSC_ROWS_UNROLL")) unroll = std::max(1, std::atoi(e));
+    // Measured on MI355X on the ConvNet's k=72 product (196000 x 2 x 16): one row per thread, k unrolled by 8 and B
+    // through the scalar unit 35 us; B in LDS 40 us; two / four rows per thread 41 / 46 us.  The slower variants stay
+    // in the generator (R, b_in_lds) because other shapes may want them; nothing selects them today.
+    const int R = 1;  // rows per thread
+    const int unroll = g.k <= 16 ? (int)g.k : 8;
     const int64_t blocks_per_batch = (g.m + 256 * R - 1) / (256 * R);
-    bool b_in_lds = false;
-    if (const char* e = std::getenv("DSC_ROWS_B")) b_in_lds = e[0] == 'l';
+    const bool b_in_lds = false;
     const int n_out = fk.has_epilogue ? fk.epilogue.raw().n_outputs : 1;
 
     const string la = em.load_view(fk.inputs[0], va, {"cb", "cm", "ck"});
@@ -1991,7 +1989,7 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
         k << "    __syncthreads();\n";
     }
     const int Q = (int)(g.n / 4);  // 16-byte pieces per row
-    const bool transposed_store = vec_store && (Q == 1 || Q == 2 || Q == 4 || Q == 8) && !std::getenv("DSC_ROWS_DIRECT_STORE");
+    const bool transposed_store = vec_store && (Q == 1 || Q == 2 || Q == 4 || Q == 8);
     // With at most 16 columns and a k of some length the products go through v_mfma_f32_16x16x4f32 instead of
     // scalar-operand FMAs (twice the fp32 rate with packed math off): a wave takes its 64 rows as four 16-row tiles,
     // lane l feeds A[row l % 16][k = 4 s + l / 16] straight from memory (the same generated load, so an im2col view
@@ -2021,7 +2019,7 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
         // (392000 rows, k = 72): JG 1 / 2 / 3 / 5 = 24.9 / 23.6 / 23.8 / 27.4 us against 25.4 for the FMA path -- the
         // kernel is bound by the 64 cache lines that every 16-byte load instruction of an im2col row block touches,
         // not by either arithmetic pipe.
-        const int64_t JG = std::getenv("DSC_ROWS_MFMA_JG") ? std::max<int64_t>(1, std::atoll(std::getenv("DSC_ROWS_MFMA_JG"))) : std::min<int64_t>(2, J);
+        const int64_t JG = std::min<int64_t>(2, J);
         k << "#pragma unroll\n    for (int j0 = 0; j0 < " << S(J) << "; j0 += " << S(JG) << ") {\n";
         k << "        float fa[" << S(JG) << "][4][4];\n";
         k << "#pragma unroll\n        for (int jj = 0; jj < " << S(JG) << "; ++jj) {\n";
@@ -2157,8 +2155,7 @@ string gen_matmul_tallk(Emitter& em, Generated* out) {
     const int64_t batch_stride = rows ? g.n : g.m * g.n, row_stride = rows ? g.batch * g.n : g.n;
     const int64_t chunk_k = chunk_k_of(g);
     const int MT = (int)((g.m + 15) / 16), NT = (int)((g.n + 15) / 16);
-    int U = std::max(1, std::min(8, 24 / (MT + NT)));  // k steps of 4 in flight per wave
-    if (const char* e = std::getenv("DSC_TALLK_UNROLL")) U = std::max(1, std::min(16, std::atoi(e)));
+    const int U = std::max(1, std::min(8, 24 / (MT + NT)));  // k steps of 4 in flight per wave
 
     const string la = em.load_view(fk.inputs[0], d.inputs[0], {"cb", "cm", "ck"});
     em.funcs << "DSC_INLINE float load_a(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return " << la << ";\n}\n";
@@ -2566,7 +2563,7 @@ std::string FusedKernel::key() const {
     s.append(reinterpret_cast<const char*>(&n_buffers), 4);
     if (const char* env = std::getenv("DSC_MM_TILE"))
         if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|T") + env;
-    for (const char* name : {"DSC_MM_SMALLK", "DSC_MM_VEC_STORE", "DSC_MM_PERSISTENT", "DSC_MM_DEEP_K", "DSC_MM_PART", "DSC_MM_ROWS", "DSC_ROWS_MFMA", "DSC_ROWS_MFMA_JG", "DSC_ROWS_R", "DSC_ROWS_UNROLL", "DSC_ROWS_B", "DSC_ROWS_DIRECT_STORE", "DSC_MM_TALLK", "DSC_TALLK_UNROLL"})
+    for (const char* name : {"DSC_MM_SMALLK", "DSC_MM_VEC_STORE", "DSC_MM_PERSISTENT", "DSC_MM_DEEP_K", "DSC_MM_ROWS", "DSC_MM_DOT", "DSC_ROWS_MFMA", "DSC_MM_TALLK"})
         if (const char* env = std::getenv(name))
             if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|") + name + env;
     return s;
@@ -2600,8 +2597,6 @@ bool can_be_part(const FusedKernel& fk) {
     if (fk.colsum_out >= 0) return false;
     // the MFMA template, when its tile choice runs four waves: small products only (large ones want their
     // workgroups persistent and the CU's whole LDS, which a shared launch cannot give them)
-    if (const char* e = std::getenv("DSC_MM_PART"))
-        if (e[0] == '0') return false;
     MmPlan plan;
     return plan_mfma(fk, g, &plan, true) && 64 * plan.c.wm * plan.c.wn == 256 && plan.grid <= 1024;
 }

@@ -229,138 +229,30 @@ dsc_view identity_view(std::initializer_list<int64_t> dims) {
     return v;
 }
 
-}  // namespace
+// The fusion planner.  One draft per reference cluster goes in; each pass below merges, splits or re-targets
+// drafts (and may add internal nodes).  Nothing is compiled here: a pass that is unsure whether a candidate can be
+// expressed generates its source as a probe and drops the candidate when that fails.  `run` holds the order.
+struct Planner {
+    const uint32_t flags;
+    int& n_nodes;
+    std::vector<size_t>& node_bytes;
+    std::vector<Draft>& drafts;
+    std::vector<bool>& is_graph_output;
+    std::vector<bool>& is_graph_input;
 
-// ---------------------------------------------------------------------------------------------------------
+    // what pass 1d learns about each convolution, for pass 1e
+    struct ConvSite {
+        int copy_idx;    // draft that writes the im2col copy
+        int a_node;      // the copy
+        int image_node;  // the convolution's input [img, h, w, g*c]
+        FusedKernel::ConvFwd geo;
+        dsc_view a_view; // (group, row, k) -> element of the copy, as the forward MatMul reads it
+    };
+    std::vector<ConvSite> conv_sites;
 
-int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags) {
-    graph_replay = (flags & DSC_SCHEDULE_GRAPH_REPLAY) != 0;
-    n_nodes = desc.n_nodes;
-    n_params = desc.n_params;
-    n_clusters = desc.n_clusters;
-    node_bytes.assign(n_nodes, 0);
-    for (int i = 0; i < n_nodes; ++i) node_bytes[i] = (size_t)desc.node_elements[i] * 4;
-    inputs.assign(desc.inputs, desc.inputs + desc.n_inputs);
-    outputs.assign(desc.outputs, desc.outputs + desc.n_outputs);
-    for (auto& io : inputs)
-        if (io.node < 0 || io.node >= n_nodes || io.param < 0 || io.param >= n_params) return fail(DSC_ERR_INVALID, "schedule: bad input entry");
-    for (auto& io : outputs)
-        if (io.node < 0 || io.node >= n_nodes || io.param < 0 || io.param >= n_params) return fail(DSC_ERR_INVALID, "schedule: bad output entry");
-
-    std::vector<bool> is_graph_output(n_nodes, false), is_graph_input(n_nodes, false);
-    for (auto& io : outputs) is_graph_output[io.node] = true;
-    for (auto& io : inputs) is_graph_input[io.node] = true;
-
-    // one draft per reference cluster
-    std::vector<Draft> drafts(desc.n_clusters);
-    for (int c = 0; c < desc.n_clusters; ++c) {
-        const dsc_cluster& cl = desc.clusters[c];
-        std::string err = validate(cl.kernel);
-        if (!err.empty()) return fail(DSC_ERR_INVALID, "schedule: cluster " + std::to_string(c) + ": " + err);
-        const int want_in = cl.kernel.kind == DSC_KERNEL_FILL ? 0 : cl.kernel.n_inputs;
-        const int want_out = cl.kernel.kind == DSC_KERNEL_PER_ELEMENT ? cl.kernel.n_outputs : 1;
-        if (cl.n_inputs != want_in || cl.n_outputs != want_out)
-            return fail(DSC_ERR_INVALID, "schedule: cluster " + std::to_string(c) + " binds the wrong number of nodes");
-        Draft& d = drafts[c];
-        d.fk = FusedKernel::plain(cl.kernel);
-        for (int i = 0; i < cl.n_inputs; ++i) {
-            if (cl.inputs[i] < 0 || cl.inputs[i] >= n_nodes) return fail(DSC_ERR_INVALID, "schedule: bad node id");
-            d.params.push_back(cl.inputs[i]);
-        }
-        for (int o = 0; o < cl.n_outputs; ++o) {
-            const dsc_cluster_output& co = cl.outputs[o];
-            if (co.node < 0 || co.node >= n_nodes || co.copy_from >= n_nodes) return fail(DSC_ERR_INVALID, "schedule: bad node id");
-            d.params.push_back(co.node);
-            d.outs.push_back(StepOutput{co.node, co.copy_from, co.copy_from_is_literal != 0, co.literal_bits});
-        }
-        d.covers.push_back(c);
-    }
-
-    if (!(flags & DSC_SCHEDULE_NO_FUSION)) {
-        // Pass 0: a MatMul whose output is small but whose k is long gets its k range split over many more
-        // workgroups than the reference's ceil(K/1024) chunks; the partial products go to an internal buffer and
-        // are summed by a Reduce (which pass 2 then inlines into the consumer when the split is small).
-        for (size_t i = 0; i < drafts.size(); ++i) {
-            if (drafts[i].fk.main.raw().kind != DSC_KERNEL_MATMUL) continue;
-            const MatMulDims g = matmul_dims(drafts[i].fk.main.raw());
-            if (g.k < 512) continue;
-            if (((g.m + 63) / 64) * ((g.n + 63) / 64) * g.batch >= 128) continue;  // the tile grid is already wide
-            {
-                // rows of k-contiguous memory times a few columns: the dot-product kernel spreads k over lanes itself
-                const dsc_view& av = drafts[i].fk.main.raw().inputs[0];
-                const int64_t c0[3] = {0, 0, 0}, c1[3] = {0, 0, 1};
-                if (g.chunks == 1 && g.m >= 256 && dot_kernel_shape(g) && av.out_shape.rank == 3 && view_index(av, c1) - view_index(av, c0) == 1) continue;
-            }
-            const int64_t t64 = ((g.m + 63) / 64) * ((g.n + 63) / 64) * g.batch;
-            static const int64_t split_target = std::getenv("DSC_SPLIT_TARGET") ? std::atoll(std::getenv("DSC_SPLIT_TARGET")) : 4096;
-            int64_t S = std::min<int64_t>(split_target / t64, g.k / 64);
-            {
-                // a small output over a long k runs on the tall-k kernel, one workgroup of four waves per
-                // (chunk, batch): a thousand workgroups with at least 256 k each
-                MatMulDims t = g;
-                t.chunks = std::min<int64_t>(std::max<int64_t>(1024 / g.batch, 1), g.k / 256);
-                if (t.chunks >= 2 && tallk_shape(t)) S = t.chunks;
-            }
-            if (S < 2) continue;
-            const int64_t ktiles = (g.k + 15) / 16;
-            const int64_t chunk_tiles = (ktiles + S - 1) / S;
-            S = (ktiles + chunk_tiles - 1) / chunk_tiles;
-            if (S < 2 || (g.chunks > 1 && S <= g.chunks)) continue;
-            const int product = drafts[i].outs[0].node;
-            const int64_t out_elems = g.batch * g.m * g.n;
-            if (S * out_elems >= ((int64_t)1 << 28)) continue;
-            if (g.chunks > 1) {
-                // the reference already sums partials: retarget that Reduce
-                if (is_graph_output[product]) continue;
-                int ri = -1, uses = 0;
-                for (size_t j = i + 1; j < drafts.size(); ++j)
-                    for (int nd : input_nodes(drafts[j]))
-                        if (nd == product) { ++uses; ri = (int)j; }
-                if (uses != 1) continue;
-                const dsc_kernel_desc& rd = drafts[ri].fk.main.raw();
-                if (rd.kind != DSC_KERNEL_REDUCE || rd.reduce_op != DSC_REDUCE_SUM || rd.axis != 0 || !is_identity(rd.inputs[0]) ||
-                    element_count(rd.inputs[0].in_shape) != g.chunks * out_elems)
-                    continue;
-                drafts[ri].fk.main.inputs[0].in_shape.dims[0] = S;
-                drafts[ri].fk.main.inputs[0].out_shape.dims[0] = S;
-            } else {
-                // new internal node for the partials, and a Reduce writing the original node
-                const int partials = n_nodes++;
-                node_bytes.push_back(0);
-                is_graph_output.push_back(false);
-                is_graph_input.push_back(false);
-                Draft r;
-                dsc_kernel_desc rd{};
-                rd.kind = DSC_KERNEL_REDUCE;
-                rd.shape = drafts[i].fk.main.raw().shape;
-                dsc_view v{};
-                v.in_shape = rd.shape;
-                v.in_shape.dims[0] = S;
-                v.out_shape = v.in_shape;
-                for (int a = 0; a < v.in_shape.rank; ++a) {
-                    v.map_axis[a] = v.in_shape.dims[a] > 1 ? a : -1;
-                    v.map_step[a] = v.in_shape.dims[a] > 1 ? 1 : 0;
-                }
-                rd.n_inputs = 1;
-                rd.inputs = &v;
-                rd.reduce_op = DSC_REDUCE_SUM;
-                rd.axis = 0;
-                r.fk = FusedKernel::plain(rd);
-                r.params = {partials, product};
-                r.outs.push_back(drafts[i].outs[0]);
-                r.covers = drafts[i].covers;
-                drafts[i].params[drafts[i].fk.outputs[0]] = partials;
-                drafts[i].outs[0] = StepOutput{partials, -1, false, 0};
-                drafts.insert(drafts.begin() + i + 1, r);
-            }
-            drafts[i].fk.main.d.shape.dims[0] = S;
-            node_bytes[drafts[i].outs[0].node] = (size_t)(S * out_elems) * 4;
-            drafts[i].keep_split = true;
-        }
-
-        // One step of merging a chain of Reduces over neighbouring axes (pass 0a below says when): the Reduce in draft
-        // `i` and the Reduce that alone consumes it become one Reduce over the merged axis, in draft `i`.
-        auto merge_reduce_step = [&](size_t i, bool small_only) -> bool {
+    // One step of merging a chain of Reduces over neighbouring axes (pass 0a below says when): the Reduce in draft
+    // `i` and the Reduce that alone consumes it become one Reduce over the merged axis, in draft `i`.
+    bool merge_reduce_step(size_t i, bool small_only) {
             const dsc_kernel_desc r1 = drafts[i].fk.main.raw();
             if (r1.kind != DSC_KERNEL_REDUCE || !drafts[i].fk.virtuals.empty() || drafts[i].fk.has_epilogue) return false;
             if (small_only && element_count(r1.inputs[0].out_shape) > (1 << 18)) return false;
@@ -443,12 +335,205 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             drafts[i] = mergedDraft;
             drafts.erase(drafts.begin() + j);
             return true;
-        };
+    }
 
-        // Pass 0c: a bias gradient is the sum of dZ [K, N] over its rows, and the weight gradient A^T dZ of the same
-        // layer reads dZ as its B operand, k chunk by k chunk.  The MFMA kernel then also writes the column sums of
-        // the B tiles it loads, one row of partials per chunk, and the Reduce shrinks from K rows to `chunks` rows: one
-        // pass over dZ instead of two.  Only large dZ (the Reduce is a launch of its own there).
+    std::vector<int> consumers_of(int node) const {
+            std::vector<int> out;
+            for (int i = 0; i < (int)drafts.size(); ++i) {
+                if (!drafts[i].alive) continue;
+                auto ins = input_nodes(drafts[i]);
+                if (std::find(ins.begin(), ins.end(), node) != ins.end()) out.push_back(i);
+            }
+            return out;
+    }
+
+    // no launch between `from` and `to` may take one of `nodes` over in place (ScatterAdd accumulators)
+    bool taken_in_place_between(int from, int to, const std::vector<int>& nodes) const {
+            for (int i = from + 1; i < to; ++i) {
+                if (!drafts[i].alive) continue;
+                for (auto& o : drafts[i].outs)
+                    if (o.copy_from >= 0 && std::find(nodes.begin(), nodes.end(), o.copy_from) != nodes.end()) return true;
+            }
+            for (auto& o : drafts[to].outs)
+                if (o.copy_from >= 0 && std::find(nodes.begin(), nodes.end(), o.copy_from) != nodes.end()) return true;
+            return false;
+    }
+
+    // A per-element cluster that can run as the epilogue of the launch producing `product_node` (`elements`
+    // values): it is the node's only consumer, has one invocation per product element and reads the product
+    // element-for-element through a plain load.
+    // With `permuted` given, the view may also be any bijection of a small product's elements (a transposed or
+    // re-split reading of it); *permuted then says whether it is one.
+    // With `shared` given, the product may have further readers after the cluster (the kernel then stores the
+    // product too); *shared says whether it has.
+    void find_epilogue(int producer_idx, int product_node, int64_t elements, int* pe_idx, int* pe_input, bool* permuted = nullptr,
+                       bool* shared = nullptr) const {
+            *pe_idx = *pe_input = -1;
+            if (permuted) *permuted = false;
+            if (shared) *shared = false;
+            if (is_graph_output[product_node]) return;
+            auto cons = consumers_of(product_node);
+            if (cons.empty() || cons[0] <= producer_idx) return;
+            if (cons.size() != 1) {
+                // the cluster must be the first reader, nobody may take the product over in place, and a large product
+                // only (a small one costs less as a launch part than as a second store)
+                if (!shared || elements < (1 << 16)) return;
+                for (auto& dr : drafts)
+                    if (dr.alive)
+                        for (auto& o : dr.outs)
+                            if (o.copy_from == product_node) return;
+                *shared = true;
+            }
+            Draft& e = drafts[cons[0]];
+            const dsc_kernel_desc& ed = e.fk.main.raw();
+            if (ed.kind != DSC_KERNEL_PER_ELEMENT || e.fk.has_epilogue || ed.shape.dims[0] != elements) return;
+            int hits = 0, input = -1;
+            for (int k = 0; k < ed.n_inputs; ++k) {
+                if (e.fk.inputs[k].buffer >= 0 && e.params[e.fk.inputs[k].buffer] == product_node) {
+                    ++hits;
+                    input = k;
+                }
+            }
+            if (hits != 1) return;
+            for (int k = 0; k < ed.n_ops; ++k)  // the product must be read element-for-element, not gathered
+                if (ed.ops[k].kind == DSC_PE_GATHER && ed.ops[k].input_index == input) return;
+            for (auto& v : e.fk.virtuals)  // and not through one of the consumer's own fused producers
+                for (auto& src : v.inputs)
+                    if (src.buffer >= 0 && e.params[src.buffer] == product_node) return;
+            for (auto& o : e.outs)
+                if (o.copy_from >= 0) return;
+            if (!is_contiguous(ed.inputs[input])) {
+                const dsc_view& v = ed.inputs[input];
+                if (!permuted || elements > 65536 || element_count(v.in_shape) != elements || any_clamp(v)) return;
+                // every element read exactly once, and recovered by the per-axis inverse the kernel will use
+                std::vector<char> seen((size_t)elements, 0);
+                int64_t ist[DSC_MAX_DIM], ost[DSC_MAX_DIM];
+                strides_of(v.in_shape, ist);
+                strides_of(v.out_shape, ost);
+                for (int64_t e = 0; e < elements; ++e) {
+                    int64_t cc[DSC_MAX_DIM], q = e;
+                    for (int a = v.out_shape.rank - 1; a >= 0; --a) {
+                        cc[a] = q % v.out_shape.dims[a];
+                        q /= v.out_shape.dims[a];
+                    }
+                    const int64_t r = view_index(v, cc);
+                    if (r < 0 || r >= elements || seen[(size_t)r]) return;
+                    seen[(size_t)r] = 1;
+                    int64_t back = 0;
+                    for (int j = 0; j < v.out_shape.rank; ++j) {
+                        if (v.out_shape.dims[j] <= 1 || v.map_axis[j] < 0) continue;
+                        if (v.map_step[j] <= 0) return;
+                        const int i = v.map_axis[j];
+                        back += (((r / ist[i]) % v.in_shape.dims[i]) / v.map_step[j]) % v.out_shape.dims[j] * ost[j];
+                    }
+                    if (back != e) return;
+                }
+                if (shared && *shared) return;
+                *permuted = true;
+            }
+            if (taken_in_place_between(producer_idx, cons[0], input_nodes(drafts[producer_idx]))) return;
+            *pe_idx = cons[0];
+            *pe_input = input;
+    }
+
+    // one load passed on unchanged
+    static bool is_pure_copy(const dsc_kernel_desc& pe) {
+            int loads = 0;
+            for (int i = 0; i < pe.n_ops; ++i) {
+                if (pe.ops[i].kind == DSC_PE_LOAD) ++loads;
+                else if (!(pe.ops[i].kind == DSC_PE_UNARY && pe.ops[i].op == DSC_UN_MOV)) return false;
+            }
+            return loads == 1;
+    }
+
+    // Pass 0: a MatMul whose output is small but whose k is long gets its k range split over many more
+    // workgroups than the reference's ceil(K/1024) chunks; the partial products go to an internal buffer and
+    // are summed by a Reduce (which pass 2 then inlines into the consumer when the split is small).
+    void split_long_k() {
+        for (size_t i = 0; i < drafts.size(); ++i) {
+            if (drafts[i].fk.main.raw().kind != DSC_KERNEL_MATMUL) continue;
+            const MatMulDims g = matmul_dims(drafts[i].fk.main.raw());
+            if (g.k < 512) continue;
+            if (((g.m + 63) / 64) * ((g.n + 63) / 64) * g.batch >= 128) continue;  // the tile grid is already wide
+            {
+                // rows of k-contiguous memory times a few columns: the dot-product kernel spreads k over lanes itself
+                const dsc_view& av = drafts[i].fk.main.raw().inputs[0];
+                const int64_t c0[3] = {0, 0, 0}, c1[3] = {0, 0, 1};
+                if (g.chunks == 1 && g.m >= 256 && dot_kernel_shape(g) && av.out_shape.rank == 3 && view_index(av, c1) - view_index(av, c0) == 1) continue;
+            }
+            const int64_t t64 = ((g.m + 63) / 64) * ((g.n + 63) / 64) * g.batch;
+            const int64_t split_target = 4096;  // workgroup tiles a split product should reach
+            int64_t S = std::min<int64_t>(split_target / t64, g.k / 64);
+            {
+                // a small output over a long k runs on the tall-k kernel, one workgroup of four waves per
+                // (chunk, batch): a thousand workgroups with at least 256 k each
+                MatMulDims t = g;
+                t.chunks = std::min<int64_t>(std::max<int64_t>(1024 / g.batch, 1), g.k / 256);
+                if (t.chunks >= 2 && tallk_shape(t)) S = t.chunks;
+            }
+            if (S < 2) continue;
+            const int64_t ktiles = (g.k + 15) / 16;
+            const int64_t chunk_tiles = (ktiles + S - 1) / S;
+            S = (ktiles + chunk_tiles - 1) / chunk_tiles;
+            if (S < 2 || (g.chunks > 1 && S <= g.chunks)) continue;
+            const int product = drafts[i].outs[0].node;
+            const int64_t out_elems = g.batch * g.m * g.n;
+            if (S * out_elems >= ((int64_t)1 << 28)) continue;
+            if (g.chunks > 1) {
+                // the reference already sums partials: retarget that Reduce
+                if (is_graph_output[product]) continue;
+                int ri = -1, uses = 0;
+                for (size_t j = i + 1; j < drafts.size(); ++j)
+                    for (int nd : input_nodes(drafts[j]))
+                        if (nd == product) { ++uses; ri = (int)j; }
+                if (uses != 1) continue;
+                const dsc_kernel_desc& rd = drafts[ri].fk.main.raw();
+                if (rd.kind != DSC_KERNEL_REDUCE || rd.reduce_op != DSC_REDUCE_SUM || rd.axis != 0 || !is_identity(rd.inputs[0]) ||
+                    element_count(rd.inputs[0].in_shape) != g.chunks * out_elems)
+                    continue;
+                drafts[ri].fk.main.inputs[0].in_shape.dims[0] = S;
+                drafts[ri].fk.main.inputs[0].out_shape.dims[0] = S;
+            } else {
+                // new internal node for the partials, and a Reduce writing the original node
+                const int partials = n_nodes++;
+                node_bytes.push_back(0);
+                is_graph_output.push_back(false);
+                is_graph_input.push_back(false);
+                Draft r;
+                dsc_kernel_desc rd{};
+                rd.kind = DSC_KERNEL_REDUCE;
+                rd.shape = drafts[i].fk.main.raw().shape;
+                dsc_view v{};
+                v.in_shape = rd.shape;
+                v.in_shape.dims[0] = S;
+                v.out_shape = v.in_shape;
+                for (int a = 0; a < v.in_shape.rank; ++a) {
+                    v.map_axis[a] = v.in_shape.dims[a] > 1 ? a : -1;
+                    v.map_step[a] = v.in_shape.dims[a] > 1 ? 1 : 0;
+                }
+                rd.n_inputs = 1;
+                rd.inputs = &v;
+                rd.reduce_op = DSC_REDUCE_SUM;
+                rd.axis = 0;
+                r.fk = FusedKernel::plain(rd);
+                r.params = {partials, product};
+                r.outs.push_back(drafts[i].outs[0]);
+                r.covers = drafts[i].covers;
+                drafts[i].params[drafts[i].fk.outputs[0]] = partials;
+                drafts[i].outs[0] = StepOutput{partials, -1, false, 0};
+                drafts.insert(drafts.begin() + i + 1, r);
+            }
+            drafts[i].fk.main.d.shape.dims[0] = S;
+            node_bytes[drafts[i].outs[0].node] = (size_t)(S * out_elems) * 4;
+            drafts[i].keep_split = true;
+        }
+    }
+
+    // Pass 0c: a bias gradient is the sum of dZ [K, N] over its rows, and the weight gradient A^T dZ of the same
+    // layer reads dZ as its B operand, k chunk by k chunk.  The MFMA kernel then also writes the column sums of
+    // the B tiles it loads, one row of partials per chunk, and the Reduce shrinks from K rows to `chunks` rows: one
+    // pass over dZ instead of two.  Only large dZ (the Reduce is a launch of its own there).
+    void bias_sums_ride_on_weight_gradients() {
         for (size_t ri = 0; ri < drafts.size(); ++ri) {
             if (drafts[ri].fk.main.raw().kind != DSC_KERNEL_REDUCE || drafts[ri].fk.main.raw().reduce_op != DSC_REDUCE_SUM ||
                 !drafts[ri].fk.virtuals.empty())
@@ -593,21 +678,25 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             drafts.insert(drafts.begin() + at, moved.begin(), moved.end());
             --ri;  // the slot now holds another draft
         }
+    }
 
-        // Pass 0a: chains of Reduces over neighbouring axes (the reference sums a bias gradient back to the bias' shape
-        // one axis at a time: [m, h, w, c] -> [1, h, w, c] -> [1, w, c] -> [c], three clusters) become one Reduce over
-        // the merged axis: fewer launches.  Only small inputs are merged (the tail of such a chain): a large first
-        // Reduce streams its input with every lane on consecutive outputs, which a merged axis over short rows would
-        // give up (measured on the ConvNet's conv bias gradients: merged 3666 steps/s, tail only 3950+).  Sums are
-        // re-associated (as in every split reduction); max is order-free.
+    // Pass 0a: chains of Reduces over neighbouring axes (the reference sums a bias gradient back to the bias' shape
+    // one axis at a time: [m, h, w, c] -> [1, h, w, c] -> [1, w, c] -> [c], three clusters) become one Reduce over
+    // the merged axis: fewer launches.  Only small inputs are merged (the tail of such a chain): a large first
+    // Reduce streams its input with every lane on consecutive outputs, which a merged axis over short rows would
+    // give up (measured on the ConvNet's conv bias gradients: merged 3666 steps/s, tail only 3950+).  Sums are
+    // re-associated (as in every split reduction); max is order-free.
+    void merge_reduce_chains() {
         for (size_t i = 0; i < drafts.size(); ++i)
             while (merge_reduce_step(i, true)) {
             }
+    }
 
-        // Pass 0b: a Reduce with few outputs and a long axis cannot fill the machine with one thread (or one
-        // thread row) per output.  Split the axis k = s * (k/s): a first Reduce over k/s produces s partial rows
-        // per output into an internal buffer, a second one combines the s partials (pass 2 inlines it into the
-        // consumer when s is small).
+    // Pass 0b: a Reduce with few outputs and a long axis cannot fill the machine with one thread (or one
+    // thread row) per output.  Split the axis k = s * (k/s): a first Reduce over k/s produces s partial rows
+    // per output into an internal buffer, a second one combines the s partials (pass 2 inlines it into the
+    // consumer when s is small).
+    void split_long_reduces() {
         for (size_t i = 0; i < drafts.size(); ++i) {
             const dsc_kernel_desc rd = drafts[i].fk.main.raw();
             if (rd.kind != DSC_KERNEL_REDUCE || !drafts[i].fk.virtuals.empty() || rd.shape.rank >= DSC_MAX_DIM) continue;
@@ -677,106 +766,10 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             drafts.insert(drafts.begin() + i + 1, second);
             ++i;
         }
+    }
 
-        auto consumers_of = [&](int node) {
-            std::vector<int> out;
-            for (int i = 0; i < (int)drafts.size(); ++i) {
-                if (!drafts[i].alive) continue;
-                auto ins = input_nodes(drafts[i]);
-                if (std::find(ins.begin(), ins.end(), node) != ins.end()) out.push_back(i);
-            }
-            return out;
-        };
-        // no launch between `from` and `to` may take one of `nodes` over in place (ScatterAdd accumulators)
-        auto taken_in_place_between = [&](int from, int to, const std::vector<int>& nodes) {
-            for (int i = from + 1; i < to; ++i) {
-                if (!drafts[i].alive) continue;
-                for (auto& o : drafts[i].outs)
-                    if (o.copy_from >= 0 && std::find(nodes.begin(), nodes.end(), o.copy_from) != nodes.end()) return true;
-            }
-            for (auto& o : drafts[to].outs)
-                if (o.copy_from >= 0 && std::find(nodes.begin(), nodes.end(), o.copy_from) != nodes.end()) return true;
-            return false;
-        };
-
-        // A per-element cluster that can run as the epilogue of the launch producing `product_node` (`elements`
-        // values): it is the node's only consumer, has one invocation per product element and reads the product
-        // element-for-element through a plain load.
-        // With `permuted` given, the view may also be any bijection of a small product's elements (a transposed or
-        // re-split reading of it); *permuted then says whether it is one.
-        // With `shared` given, the product may have further readers after the cluster (the kernel then stores the
-        // product too); *shared says whether it has.
-        auto find_epilogue = [&](int producer_idx, int product_node, int64_t elements, int* pe_idx, int* pe_input, bool* permuted = nullptr,
-                                 bool* shared = nullptr) {
-            *pe_idx = *pe_input = -1;
-            if (permuted) *permuted = false;
-            if (shared) *shared = false;
-            if (is_graph_output[product_node]) return;
-            auto cons = consumers_of(product_node);
-            if (cons.empty() || cons[0] <= producer_idx) return;
-            if (cons.size() != 1) {
-                // the cluster must be the first reader, nobody may take the product over in place, and a large product
-                // only (a small one costs less as a launch part than as a second store)
-                if (!shared || elements < (1 << 16)) return;
-                for (auto& dr : drafts)
-                    if (dr.alive)
-                        for (auto& o : dr.outs)
-                            if (o.copy_from == product_node) return;
-                *shared = true;
-            }
-            Draft& e = drafts[cons[0]];
-            const dsc_kernel_desc& ed = e.fk.main.raw();
-            if (ed.kind != DSC_KERNEL_PER_ELEMENT || e.fk.has_epilogue || ed.shape.dims[0] != elements) return;
-            int hits = 0, input = -1;
-            for (int k = 0; k < ed.n_inputs; ++k) {
-                if (e.fk.inputs[k].buffer >= 0 && e.params[e.fk.inputs[k].buffer] == product_node) {
-                    ++hits;
-                    input = k;
-                }
-            }
-            if (hits != 1) return;
-            for (int k = 0; k < ed.n_ops; ++k)  // the product must be read element-for-element, not gathered
-                if (ed.ops[k].kind == DSC_PE_GATHER && ed.ops[k].input_index == input) return;
-            for (auto& v : e.fk.virtuals)  // and not through one of the consumer's own fused producers
-                for (auto& src : v.inputs)
-                    if (src.buffer >= 0 && e.params[src.buffer] == product_node) return;
-            for (auto& o : e.outs)
-                if (o.copy_from >= 0) return;
-            if (!is_contiguous(ed.inputs[input])) {
-                const dsc_view& v = ed.inputs[input];
-                if (!permuted || elements > 65536 || element_count(v.in_shape) != elements || any_clamp(v)) return;
-                // every element read exactly once, and recovered by the per-axis inverse the kernel will use
-                std::vector<char> seen((size_t)elements, 0);
-                int64_t ist[DSC_MAX_DIM], ost[DSC_MAX_DIM];
-                strides_of(v.in_shape, ist);
-                strides_of(v.out_shape, ost);
-                for (int64_t e = 0; e < elements; ++e) {
-                    int64_t cc[DSC_MAX_DIM], q = e;
-                    for (int a = v.out_shape.rank - 1; a >= 0; --a) {
-                        cc[a] = q % v.out_shape.dims[a];
-                        q /= v.out_shape.dims[a];
-                    }
-                    const int64_t r = view_index(v, cc);
-                    if (r < 0 || r >= elements || seen[(size_t)r]) return;
-                    seen[(size_t)r] = 1;
-                    int64_t back = 0;
-                    for (int j = 0; j < v.out_shape.rank; ++j) {
-                        if (v.out_shape.dims[j] <= 1 || v.map_axis[j] < 0) continue;
-                        if (v.map_step[j] <= 0) return;
-                        const int i = v.map_axis[j];
-                        back += (((r / ist[i]) % v.in_shape.dims[i]) / v.map_step[j]) % v.out_shape.dims[j] * ost[j];
-                    }
-                    if (back != e) return;
-                }
-                if (shared && *shared) return;
-                *permuted = true;
-            }
-            if (taken_in_place_between(producer_idx, cons[0], input_nodes(drafts[producer_idx]))) return;
-            *pe_idx = cons[0];
-            *pe_input = input;
-        };
-
-        // Pass 1: MatMul (+ Reduce over its split-K partials) (+ per-element consumer as epilogue).
+    // Pass 1: MatMul (+ Reduce over its split-K partials) (+ per-element consumer as epilogue).
+    void matmul_with_reduce_and_epilogue() {
         for (int i = 0; i < (int)drafts.size(); ++i) {
             Draft& mm = drafts[i];
             if (!mm.alive || mm.fk.main.raw().kind != DSC_KERNEL_MATMUL || mm.fk.has_epilogue || mm.keep_split) continue;
@@ -839,14 +832,16 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                 drafts[reduce_idx] = fused;
             }
         }
+    }
 
-        // Pass 1c: the data gradient of a stride-1 convolution arrives as MatMul (dC x filter^T, one row of
-        // fh*fw*c window elements per output pixel) -> reshape copy -> WindowsToImage (sum of the windows that
-        // cover each pixel of the padded image).  With few channels that is the product written out nine times
-        // over and read back.  Run it as one MatMul over the padded image instead: row = padded pixel,
-        // k = (fy, fx, oc), A'[pixel, k] = dC[pixel - tap, oc] where that output pixel exists (else 0),
-        // B'[k, c] = filter[oc, fy, fx, c]; both operands are fused producers of the MatMul, nothing in between
-        // is written.
+    // Pass 1c: the data gradient of a stride-1 convolution arrives as MatMul (dC x filter^T, one row of
+    // fh*fw*c window elements per output pixel) -> reshape copy -> WindowsToImage (sum of the windows that
+    // cover each pixel of the padded image).  With few channels that is the product written out nine times
+    // over and read back.  Run it as one MatMul over the padded image instead: row = padded pixel,
+    // k = (fy, fx, oc), A'[pixel, k] = dC[pixel - tap, oc] where that output pixel exists (else 0),
+    // B'[k, c] = filter[oc, fy, fx, c]; both operands are fused producers of the MatMul, nothing in between
+    // is written.
+    void conv_data_gradient() {
         for (int i = 0; i < (int)drafts.size(); ++i) {
             static const bool enabled = !(std::getenv("DSC_FUSE_DGRAD") && std::getenv("DSC_FUSE_DGRAD")[0] == '0');
             if (!enabled) break;
@@ -1067,20 +1062,13 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             if (copy_idx >= 0) drafts[copy_idx].alive = false;
             drafts[w_idx] = fused;
         }
+    }
 
-        // Pass 1d: the forward of a stride-1 convolution arrives as a copy cluster that writes the im2col of the
-        // (replicate-padded) image, and a MatMul over it.  The dedicated kernel reads the image itself.  The geometry
-        // is a hypothesis (filter height from the divisors of k / c, padding from the output size) that is then
-        // checked on every (pixel, k) of three images against the addresses the copy's view really produces.
-        // what pass 1d learns about each convolution, for pass 1e
-        struct ConvSite {
-            int copy_idx;    // draft that writes the im2col copy
-            int a_node;      // the copy
-            int image_node;  // the convolution's input [img, h, w, g*c]
-            FusedKernel::ConvFwd geo;
-            dsc_view a_view; // (group, row, k) -> element of the copy, as the forward MatMul reads it
-        };
-        std::vector<ConvSite> conv_sites;
+    // Pass 1d: the forward of a stride-1 convolution arrives as a copy cluster that writes the im2col of the
+    // (replicate-padded) image, and a MatMul over it.  The dedicated kernel reads the image itself.  The geometry
+    // is a hypothesis (filter height from the divisors of k / c, padding from the output size) that is then
+    // checked on every (pixel, k) of three images against the addresses the copy's view really produces.
+    void conv_forward() {
         for (int i = 0; i < (int)drafts.size(); ++i) {
             static const bool enabled = !(std::getenv("DSC_FUSE_CONV_FWD") && std::getenv("DSC_FUSE_CONV_FWD")[0] == '0');
             if (!enabled || (flags & DSC_SCHEDULE_NO_CONV_KERNELS)) break;
@@ -1172,13 +1160,15 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             }
             drafts[i] = fused;
         }
+    }
 
-        // Pass 1e: both gradients of a convolution in one kernel.  The data-gradient kernel (pass 1c) holds dC of an
-        // image in LDS; the filter gradient im2col^T x dC of the same convolution -- by now a MatMul whose k (images x
-        // output pixels) pass 0 split into many chunks, summed by a Reduce, possibly with the bias gradient's column
-        // sums riding on it (pass 0c) -- needs the same dC and the image's input tile.  The kernel takes both: its
-        // workgroups each own a set of images, and the partial products (and column sums) come out once per set, in
-        // the layout the MatMul's chunks had, so the Reduces stay and only learn the new number of partials.
+    // Pass 1e: both gradients of a convolution in one kernel.  The data-gradient kernel (pass 1c) holds dC of an
+    // image in LDS; the filter gradient im2col^T x dC of the same convolution -- by now a MatMul whose k (images x
+    // output pixels) pass 0 split into many chunks, summed by a Reduce, possibly with the bias gradient's column
+    // sums riding on it (pass 0c) -- needs the same dC and the image's input tile.  The kernel takes both: its
+    // workgroups each own a set of images, and the partial products (and column sums) come out once per set, in
+    // the layout the MatMul's chunks had, so the Reduces stay and only learn the new number of partials.
+    void conv_backward() {
         for (const ConvSite& site : conv_sites) {
             static const bool enabled = !(std::getenv("DSC_FUSE_CONV_BWD") && std::getenv("DSC_FUSE_CONV_BWD")[0] == '0');
             if (!enabled || (flags & DSC_SCHEDULE_SPLIT_CONV_GRADS)) break;
@@ -1299,144 +1289,138 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                 drafts[site.copy_idx].alive = false;
             }
         }
+    }
 
-        // Pass 1b: clusters that all work on the rows of one [m, n] array with a short n -- Reduces along n and the
-        // per-element clusters around them (softmax cross-entropy: row max, exp, row sum, log-probability, gradient,
-        // per-row loss; the accuracy count: arg-max and comparison with the label) -- become one row-fused launch.
-        // The launch runs where the first of them ran, so a member may only read what exists by then or what
-        // another member computes.
-        {
-            std::vector<int> producer_of(n_nodes, -1);  // draft index writing each node
-            auto refresh_producers = [&]() {
-                std::fill(producer_of.begin(), producer_of.end(), -1);
-                for (int i = 0; i < (int)drafts.size(); ++i)
-                    if (drafts[i].alive)
-                        for (auto& o : drafts[i].outs) producer_of[o.node] = i;
-            };
-            auto is_plain = [&](const Draft& d) {
-                if (!d.alive || !d.fk.virtuals.empty() || d.fk.has_epilogue || !d.fk.row_stages.empty() || d.keep_output || d.keep_split) return false;
-                for (auto& o : d.outs)
-                    if (o.copy_from >= 0) return false;
+    // Pass 1b: clusters that all work on the rows of one [m, n] array with a short n -- Reduces along n and the
+    // per-element clusters around them (softmax cross-entropy: row max, exp, row sum, log-probability, gradient,
+    // per-row loss; the accuracy count: arg-max and comparison with the label) -- become one row-fused launch.
+    // The launch runs where the first of them ran, so a member may only read what exists by then or what
+    // another member computes.
+    void row_kernels() {
+        std::vector<int> producer_of(n_nodes, -1);  // draft index writing each node
+        auto refresh_producers = [&]() {
+            std::fill(producer_of.begin(), producer_of.end(), -1);
+            for (int i = 0; i < (int)drafts.size(); ++i)
+                if (drafts[i].alive)
+                    for (auto& o : drafts[i].outs) producer_of[o.node] = i;
+        };
+        auto is_plain = [&](const Draft& d) {
+            if (!d.alive || !d.fk.virtuals.empty() || d.fk.has_epilogue || !d.fk.row_stages.empty() || d.keep_output || d.keep_split) return false;
+            for (auto& o : d.outs)
+                if (o.copy_from >= 0) return false;
+            return true;
+        };
+        auto shape_is = [](const dsc_shape& sh, int64_t a, int64_t b) { return sh.rank == 2 && sh.dims[0] == a && sh.dims[1] == b; };
+        for (int seed = 0; seed < (int)drafts.size(); ++seed) {
+            if (!is_plain(drafts[seed])) continue;
+            const dsc_kernel_desc& sd = drafts[seed].fk.main.raw();
+            if (sd.kind != DSC_KERNEL_REDUCE || sd.inputs[0].out_shape.rank != 2 || sd.axis != 1) continue;
+            const int64_t m = sd.inputs[0].out_shape.dims[0], n = sd.inputs[0].out_shape.dims[1];
+            if (n < 2 || n > 64 || m < 2 || !shape_is(sd.shape, m, 1)) continue;
+            refresh_producers();
+            std::vector<int> members;      // draft indices, in order
+            std::vector<int> member_of(drafts.size(), -1);
+            auto try_add = [&](int j) {
+                const Draft& d = drafts[j];
+                if (!is_plain(d)) return false;
+                const dsc_kernel_desc& k = d.fk.main.raw();
+                bool wide = false;
+                if (k.kind == DSC_KERNEL_REDUCE) {
+                    if (k.axis != 1 || !shape_is(k.inputs[0].out_shape, m, n) || !shape_is(k.shape, m, 1)) return false;
+                } else if (k.kind == DSC_KERNEL_PER_ELEMENT) {
+                    wide = k.shape.dims[0] == m * n;
+                    if (!wide && k.shape.dims[0] != m) return false;
+                    auto shape_ok = [&](const dsc_shape& sh) {
+                        return wide ? shape_is(sh, m, n) : (shape_is(sh, m, 1) || (sh.rank == 1 && sh.dims[0] == m));
+                    };
+                    for (int i = 0; i < k.n_inputs; ++i)
+                        if (!shape_ok(k.inputs[i].out_shape)) return false;
+                    for (int i = 0; i < k.n_builtin_views; ++i)
+                        if (!shape_ok(k.builtin_views[i].out_shape)) return false;
+                    for (int i = 0; i < k.n_ops; ++i)
+                        if (k.ops[i].kind == DSC_PE_GATHER) return false;
+                } else {
+                    return false;
+                }
+                for (int i = 0; i < k.n_inputs; ++i) {
+                    const int node = d.params[d.fk.inputs[i].buffer];
+                    const int p = producer_of[node];
+                    if (p >= 0 && member_of[p] >= 0) {
+                        // computed by a member: must be read element for element (or one value per row)
+                        const dsc_kernel_desc& pk = drafts[p].fk.main.raw();
+                        const bool p_wide = pk.kind == DSC_KERNEL_PER_ELEMENT && pk.shape.dims[0] == m * n;
+                        const dsc_view& v = k.inputs[i];
+                        if (element_count(v.in_shape) != (p_wide ? m * n : m)) return false;
+                        int64_t base, coef[DSC_MAX_DIM];
+                        if (!affine_form(v, &base, coef) || base != 0) return false;
+                        if (p_wide) {
+                            if (!(k.kind == DSC_KERNEL_REDUCE || wide) || coef[0] != n || coef[1] != 1) return false;
+                        } else {
+                            if (k.kind == DSC_KERNEL_REDUCE || coef[0] != 1) return false;
+                            if (v.out_shape.rank == 2 && v.out_shape.dims[1] > 1 && coef[1] != 0) return false;
+                        }
+                    } else if (p >= seed) {
+                        return false;  // does not exist yet where the fused launch runs
+                    }
+                }
                 return true;
             };
-            auto shape_is = [](const dsc_shape& sh, int64_t a, int64_t b) { return sh.rank == 2 && sh.dims[0] == a && sh.dims[1] == b; };
-            for (int seed = 0; seed < (int)drafts.size(); ++seed) {
-                if (!is_plain(drafts[seed])) continue;
-                const dsc_kernel_desc& sd = drafts[seed].fk.main.raw();
-                if (sd.kind != DSC_KERNEL_REDUCE || sd.inputs[0].out_shape.rank != 2 || sd.axis != 1) continue;
-                const int64_t m = sd.inputs[0].out_shape.dims[0], n = sd.inputs[0].out_shape.dims[1];
-                if (n < 2 || n > 64 || m < 2 || !shape_is(sd.shape, m, 1)) continue;
-                refresh_producers();
-                std::vector<int> members;      // draft indices, in order
-                std::vector<int> member_of(drafts.size(), -1);
-                auto try_add = [&](int j) {
-                    const Draft& d = drafts[j];
-                    if (!is_plain(d)) return false;
-                    const dsc_kernel_desc& k = d.fk.main.raw();
-                    bool wide = false;
-                    if (k.kind == DSC_KERNEL_REDUCE) {
-                        if (k.axis != 1 || !shape_is(k.inputs[0].out_shape, m, n) || !shape_is(k.shape, m, 1)) return false;
-                    } else if (k.kind == DSC_KERNEL_PER_ELEMENT) {
-                        wide = k.shape.dims[0] == m * n;
-                        if (!wide && k.shape.dims[0] != m) return false;
-                        auto shape_ok = [&](const dsc_shape& sh) {
-                            return wide ? shape_is(sh, m, n) : (shape_is(sh, m, 1) || (sh.rank == 1 && sh.dims[0] == m));
-                        };
-                        for (int i = 0; i < k.n_inputs; ++i)
-                            if (!shape_ok(k.inputs[i].out_shape)) return false;
-                        for (int i = 0; i < k.n_builtin_views; ++i)
-                            if (!shape_ok(k.builtin_views[i].out_shape)) return false;
-                        for (int i = 0; i < k.n_ops; ++i)
-                            if (k.ops[i].kind == DSC_PE_GATHER) return false;
+            for (int j = seed; j < (int)drafts.size(); ++j) {
+                if (!try_add(j)) {
+                    if (j == seed) break;
+                    continue;
+                }
+                member_of[j] = (int)members.size();
+                members.push_back(j);
+            }
+            if (members.size() < 2 || members.size() > 24) continue;
+            Draft fused;
+            fused.fk.main = drafts[seed].fk.main;
+            fused.fk.row_m = m;
+            fused.fk.row_n = n;
+            for (int j : members) {
+                const Draft& d = drafts[j];
+                const dsc_kernel_desc& k = d.fk.main.raw();
+                RowStage st;
+                st.k = d.fk.main;
+                for (int i = 0; i < k.n_inputs; ++i) {
+                    const int node = d.params[d.fk.inputs[i].buffer];
+                    const int p = producer_of[node];
+                    Source src;
+                    if (p >= 0 && member_of[p] >= 0) {
+                        src.stage = member_of[p];
+                        for (size_t o = 0; o < drafts[p].outs.size(); ++o)
+                            if (drafts[p].outs[o].node == node) src.stage_out = (int)o;
                     } else {
-                        return false;
+                        src.buffer = param_index(fused, node, false);
                     }
-                    for (int i = 0; i < k.n_inputs; ++i) {
-                        const int node = d.params[d.fk.inputs[i].buffer];
-                        const int p = producer_of[node];
-                        if (p >= 0 && member_of[p] >= 0) {
-                            // computed by a member: must be read element for element (or one value per row)
-                            const dsc_kernel_desc& pk = drafts[p].fk.main.raw();
-                            const bool p_wide = pk.kind == DSC_KERNEL_PER_ELEMENT && pk.shape.dims[0] == m * n;
-                            const dsc_view& v = k.inputs[i];
-                            if (element_count(v.in_shape) != (p_wide ? m * n : m)) return false;
-                            int64_t base, coef[DSC_MAX_DIM];
-                            if (!affine_form(v, &base, coef) || base != 0) return false;
-                            if (p_wide) {
-                                if (!(k.kind == DSC_KERNEL_REDUCE || wide) || coef[0] != n || coef[1] != 1) return false;
-                            } else {
-                                if (k.kind == DSC_KERNEL_REDUCE || coef[0] != 1) return false;
-                                if (v.out_shape.rank == 2 && v.out_shape.dims[1] > 1 && coef[1] != 0) return false;
-                            }
-                        } else if (p >= seed) {
-                            return false;  // does not exist yet where the fused launch runs
-                        }
-                    }
-                    return true;
-                };
-                for (int j = seed; j < (int)drafts.size(); ++j) {
-                    if (!try_add(j)) {
-                        if (j == seed) break;
-                        continue;
-                    }
-                    member_of[j] = (int)members.size();
-                    members.push_back(j);
+                    st.inputs.push_back(src);
                 }
-                if (members.size() < 2 || members.size() > 24) continue;
-                Draft fused;
-                fused.fk.main = drafts[seed].fk.main;
-                fused.fk.row_m = m;
-                fused.fk.row_n = n;
-                for (int j : members) {
-                    const Draft& d = drafts[j];
-                    const dsc_kernel_desc& k = d.fk.main.raw();
-                    RowStage st;
-                    st.k = d.fk.main;
-                    for (int i = 0; i < k.n_inputs; ++i) {
-                        const int node = d.params[d.fk.inputs[i].buffer];
-                        const int p = producer_of[node];
-                        Source src;
-                        if (p >= 0 && member_of[p] >= 0) {
-                            src.stage = member_of[p];
-                            for (size_t o = 0; o < drafts[p].outs.size(); ++o)
-                                if (drafts[p].outs[o].node == node) src.stage_out = (int)o;
-                        } else {
-                            src.buffer = param_index(fused, node, false);
-                        }
-                        st.inputs.push_back(src);
+                for (auto& o : d.outs) {
+                    bool needed = is_graph_output[o.node];
+                    for (int c : consumers_of(o.node))
+                        if (member_of[c] < 0) needed = true;
+                    if (needed) {
+                        st.outputs.push_back((int)fused.fk.outputs.size());
+                        fused.fk.outputs.push_back(param_index(fused, o.node, true));
+                        fused.outs.push_back(o);
+                    } else {
+                        st.outputs.push_back(-1);
                     }
-                    for (auto& o : d.outs) {
-                        bool needed = is_graph_output[o.node];
-                        for (int c : consumers_of(o.node))
-                            if (member_of[c] < 0) needed = true;
-                        if (needed) {
-                            st.outputs.push_back((int)fused.fk.outputs.size());
-                            fused.fk.outputs.push_back(param_index(fused, o.node, true));
-                            fused.outs.push_back(o);
-                        } else {
-                            st.outputs.push_back(-1);
-                        }
-                    }
-                    fused.fk.row_stages.push_back(st);
-                    fused.covers.insert(fused.covers.end(), d.covers.begin(), d.covers.end());
                 }
-                if (fused.fk.outputs.empty()) continue;
-                for (int j : members) drafts[j].alive = false;
-                drafts[seed] = fused;
+                fused.fk.row_stages.push_back(st);
+                fused.covers.insert(fused.covers.end(), d.covers.begin(), d.covers.end());
             }
+            if (fused.fk.outputs.empty()) continue;
+            for (int j : members) drafts[j].alive = false;
+            drafts[seed] = fused;
         }
+    }
 
-        // Pass 2: per-element producers whose result need not exist in memory are evaluated inside their
-        // consumers: pure copies (materialised im2col / pooling windows) into every consumer, light arithmetic
-        // into a single consumer.
-        auto is_pure_copy = [](const dsc_kernel_desc& pe) {
-            int loads = 0;
-            for (int i = 0; i < pe.n_ops; ++i) {
-                if (pe.ops[i].kind == DSC_PE_LOAD) ++loads;
-                else if (!(pe.ops[i].kind == DSC_PE_UNARY && pe.ops[i].op == DSC_UN_MOV)) return false;
-            }
-            return loads == 1;
-        };
+    // Pass 2: per-element producers whose result need not exist in memory are evaluated inside their
+    // consumers: pure copies (materialised im2col / pooling windows) into every consumer, light arithmetic
+    // into a single consumer.
+    void inline_producers() {
         // tuning hook: DSC_FUSE_INTO_MATMUL=0 keeps producers of MatMul operands materialised
         const char* fim = std::getenv("DSC_FUSE_INTO_MATMUL");
         const bool fuse_into_matmul = !(fim && fim[0] == '0');
@@ -1524,10 +1508,12 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
                 changed = true;
             }
         }
+    }
 
-        // Pass 3: a Reduce, WindowsToImage or Unpad whose only consumer is a per-element cluster over its outputs (a
-        // scalar accumulated into a running sum, the optimiser update of a bias gradient, the activation derivative
-        // applied to a pooling gradient) applies that cluster to each result before the store.
+    // Pass 3: a Reduce, WindowsToImage or Unpad whose only consumer is a per-element cluster over its outputs (a
+    // scalar accumulated into a running sum, the optimiser update of a bias gradient, the activation derivative
+    // applied to a pooling gradient) applies that cluster to each result before the store.
+    void attach_epilogues() {
         for (int i = 0; i < (int)drafts.size(); ++i) {
             Draft& r = drafts[i];
             const int rk = r.fk.main.raw().kind;
@@ -1568,13 +1554,15 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             r.alive = false;
             drafts[pe_idx] = fused;  // runs where the per-element cluster ran: all of its inputs exist by then
         }
+    }
 
-        // Pass 3c: max-pooling joins the convolution that feeds it.  By now the pooling is a Reduce(max) over four
-        // window elements whose input is a fused producer -- the window copy of the convolution kernel's (activated)
-        // output -- possibly with a per-element consumer of its own (pass 3: a dropout select).  The convolution
-        // kernel has those values in registers: it takes the maximum over each 2x2 window with two shuffles and runs the
-        // consumer, and the convolution's output is not read back.  The geometry is checked element by element: every
-        // pooled element of three images must read exactly the four window elements the kernel will combine.
+    // Pass 3c: max-pooling joins the convolution that feeds it.  By now the pooling is a Reduce(max) over four
+    // window elements whose input is a fused producer -- the window copy of the convolution kernel's (activated)
+    // output -- possibly with a per-element consumer of its own (pass 3: a dropout select).  The convolution
+    // kernel has those values in registers: it takes the maximum over each 2x2 window with two shuffles and runs the
+    // consumer, and the convolution's output is not read back.  The geometry is checked element by element: every
+    // pooled element of three images must read exactly the four window elements the kernel will combine.
+    void pool_joins_conv_forward() {
         for (int ri = 0; ri < (int)drafts.size(); ++ri) {
             static const bool enabled = !(std::getenv("DSC_FUSE_CONV_POOL") && std::getenv("DSC_FUSE_CONV_POOL")[0] == '0');
             if (!enabled || (flags & DSC_SCHEDULE_NO_CONV_KERNELS)) break;
@@ -1703,10 +1691,12 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             R.alive = false;
             drafts[fi] = fused;
         }
+    }
 
-        // Pass 3b: ScatterAdds chained through one accumulator (each takes the previous one's result in place:
-        // the four corner updates of one hash-grid level) commute, so the chain runs as one multi-part launch
-        // whose parts all add into the same buffer.  It runs where the last one ran.
+    // Pass 3b: ScatterAdds chained through one accumulator (each takes the previous one's result in place:
+    // the four corner updates of one hash-grid level) commute, so the chain runs as one multi-part launch
+    // whose parts all add into the same buffer.  It runs where the last one ran.
+    void chain_scatter_adds() {
         for (int i = 0; i < (int)drafts.size(); ++i) {
             if (!drafts[i].alive || drafts[i].fk.main.raw().kind != DSC_KERNEL_SCATTER_ADD || !drafts[i].fk.parts.empty()) continue;
             std::vector<int> chain{i};
@@ -1767,83 +1757,154 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
             for (int j : chain) drafts[j].alive = false;
             drafts[last] = multi;
         }
+    }
 
-        // Pass 4: launches of a few workgroups each (optimiser updates of small tensors, short reductions, scalar
-        // bookkeeping) cost a launch apiece while using a fraction of the machine.  Runs of them that do not
-        // depend on one another become one multi-part launch; a later launch is hoisted into the run when nothing
-        // it reads is produced in between.  One large kernel may ride along (its workgroups come last, so the
-        // small parts start at once and finish in its shadow).
-        {
-            static const int64_t small_grid = std::getenv("DSC_MULTI_GRID") ? std::atoll(std::getenv("DSC_MULTI_GRID")) : 1024;
-            std::vector<int64_t> grid_of(drafts.size(), -1);
-            auto partable = [&](int i) {
-                const Draft& d = drafts[i];
-                if (!d.alive || !can_be_part(d.fk)) return false;
-                for (auto& o : d.outs)
-                    if (o.copy_from >= 0) return false;
-                if (grid_of[i] < 0) {
-                    Generated g;
-                    FusedKernel probe = d.fk;
-                    probe.as_part = true;  // a kernel may pick another workgroup shape inside a shared launch
-                    if (!generate(probe, &g).empty() || g.block != 256) { grid_of[i] = (int64_t)1 << 40; return false; }
-                    grid_of[i] = g.grid;
-                }
-                return grid_of[i] < ((int64_t)1 << 30);
-            };
-            std::vector<bool> taken(drafts.size(), false);
-            for (int i = 0; i < (int)drafts.size() && small_grid > 0; ++i) {
-                if (taken[i] || !partable(i)) continue;
-                std::vector<int> batch{i};
-                int large = grid_of[i] > small_grid ? 1 : 0;
-                int64_t total_grid = grid_of[i];
-                std::set<int> blocked, bound;
-                for (auto& o : drafts[i].outs) blocked.insert(o.node);
-                for (int nd : drafts[i].params) bound.insert(nd);
-                for (int j = i + 1; j < (int)drafts.size(); ++j) {
-                    if (!drafts[j].alive || taken[j]) continue;
-                    bool depends = false;
-                    for (int nd : input_nodes(drafts[j]))
-                        if (blocked.count(nd)) depends = true;
-                    std::set<int> would = bound;
-                    for (int nd : drafts[j].params) would.insert(nd);
-                    if (!depends && batch.size() < 16 && would.size() <= 48 && partable(j) && (grid_of[j] <= small_grid || large == 0) &&
-                        total_grid + grid_of[j] < ((int64_t)1 << 30)) {
-                        batch.push_back(j);
-                        bound = would;
-                        large += grid_of[j] > small_grid ? 1 : 0;
-                        total_grid += grid_of[j];
-                    }
-                    for (auto& o : drafts[j].outs) blocked.insert(o.node);
-                }
-                // a lone large kernel with nothing small to carry stays as it is
-                if (batch.size() < 2) continue;
-                std::stable_sort(batch.begin(), batch.end(), [&](int a, int b) { return grid_of[a] < grid_of[b]; });
-                if (batch.size() < 2) continue;
-                Draft multi;
-                multi.fk.main = drafts[i].fk.main;
-                std::set<int> seen;
-                for (int j : batch) {
-                    const Draft& d = drafts[j];
-                    std::vector<int> map;
-                    for (size_t p = 0; p < d.params.size(); ++p) map.push_back(param_index(multi, d.params[p], d.fk.buffer_is_output[p]));
-                    multi.fk.parts.push_back(d.fk);
-                    multi.fk.part_params.push_back(map);
-                    for (int nd : input_nodes(d))
-                        if (seen.insert(nd).second) multi.part_inputs.push_back(nd);
-                    for (size_t o = 0; o < d.outs.size(); ++o) {
-                        multi.outs.push_back(d.outs[o]);
-                        multi.fk.outputs.push_back(param_index(multi, d.outs[o].node, true));
-                    }
-                    multi.covers.insert(multi.covers.end(), d.covers.begin(), d.covers.end());
-                }
-                for (int j : batch) {
-                    taken[j] = true;
-                    drafts[j].alive = false;
-                }
-                drafts[i] = multi;
-                taken[i] = true;
+    // Pass 4: launches of a few workgroups each (optimiser updates of small tensors, short reductions, scalar
+    // bookkeeping) cost a launch apiece while using a fraction of the machine.  Runs of them that do not
+    // depend on one another become one multi-part launch; a later launch is hoisted into the run when nothing
+    // it reads is produced in between.  One large kernel may ride along (its workgroups come last, so the
+    // small parts start at once and finish in its shadow).
+    void share_launches() {
+        static const int64_t small_grid = std::getenv("DSC_MULTI_GRID") ? std::atoll(std::getenv("DSC_MULTI_GRID")) : 1024;
+        std::vector<int64_t> grid_of(drafts.size(), -1);
+        auto partable = [&](int i) {
+            const Draft& d = drafts[i];
+            if (!d.alive || !can_be_part(d.fk)) return false;
+            for (auto& o : d.outs)
+                if (o.copy_from >= 0) return false;
+            if (grid_of[i] < 0) {
+                Generated g;
+                FusedKernel probe = d.fk;
+                probe.as_part = true;  // a kernel may pick another workgroup shape inside a shared launch
+                if (!generate(probe, &g).empty() || g.block != 256) { grid_of[i] = (int64_t)1 << 40; return false; }
+                grid_of[i] = g.grid;
             }
+            return grid_of[i] < ((int64_t)1 << 30);
+        };
+        std::vector<bool> taken(drafts.size(), false);
+        for (int i = 0; i < (int)drafts.size() && small_grid > 0; ++i) {
+            if (taken[i] || !partable(i)) continue;
+            std::vector<int> batch{i};
+            int large = grid_of[i] > small_grid ? 1 : 0;
+            int64_t total_grid = grid_of[i];
+            std::set<int> blocked, bound;
+            for (auto& o : drafts[i].outs) blocked.insert(o.node);
+            for (int nd : drafts[i].params) bound.insert(nd);
+            for (int j = i + 1; j < (int)drafts.size(); ++j) {
+                if (!drafts[j].alive || taken[j]) continue;
+                bool depends = false;
+                for (int nd : input_nodes(drafts[j]))
+                    if (blocked.count(nd)) depends = true;
+                std::set<int> would = bound;
+                for (int nd : drafts[j].params) would.insert(nd);
+                if (!depends && batch.size() < 16 && would.size() <= 48 && partable(j) && (grid_of[j] <= small_grid || large == 0) &&
+                    total_grid + grid_of[j] < ((int64_t)1 << 30)) {
+                    batch.push_back(j);
+                    bound = would;
+                    large += grid_of[j] > small_grid ? 1 : 0;
+                    total_grid += grid_of[j];
+                }
+                for (auto& o : drafts[j].outs) blocked.insert(o.node);
+            }
+            // a lone large kernel with nothing small to carry stays as it is
+            if (batch.size() < 2) continue;
+            std::stable_sort(batch.begin(), batch.end(), [&](int a, int b) { return grid_of[a] < grid_of[b]; });
+            if (batch.size() < 2) continue;
+            Draft multi;
+            multi.fk.main = drafts[i].fk.main;
+            std::set<int> seen;
+            for (int j : batch) {
+                const Draft& d = drafts[j];
+                std::vector<int> map;
+                for (size_t p = 0; p < d.params.size(); ++p) map.push_back(param_index(multi, d.params[p], d.fk.buffer_is_output[p]));
+                multi.fk.parts.push_back(d.fk);
+                multi.fk.part_params.push_back(map);
+                for (int nd : input_nodes(d))
+                    if (seen.insert(nd).second) multi.part_inputs.push_back(nd);
+                for (size_t o = 0; o < d.outs.size(); ++o) {
+                    multi.outs.push_back(d.outs[o]);
+                    multi.fk.outputs.push_back(param_index(multi, d.outs[o].node, true));
+                }
+                multi.covers.insert(multi.covers.end(), d.covers.begin(), d.covers.end());
+            }
+            for (int j : batch) {
+                taken[j] = true;
+                drafts[j].alive = false;
+            }
+            drafts[i] = multi;
+            taken[i] = true;
         }
+    }
+
+    // The order matters: each pass names the ones it relies on.
+    void run() {
+        split_long_k();                         // pass 0
+        bias_sums_ride_on_weight_gradients();   // pass 0c
+        merge_reduce_chains();                  // pass 0a
+        split_long_reduces();                   // pass 0b
+        matmul_with_reduce_and_epilogue();      // pass 1
+        conv_data_gradient();                   // pass 1c
+        conv_forward();                         // pass 1d
+        conv_backward();                        // pass 1e
+        row_kernels();                          // pass 1b
+        inline_producers();                     // pass 2
+        attach_epilogues();                     // pass 3
+        pool_joins_conv_forward();              // pass 3c
+        chain_scatter_adds();                   // pass 3b
+        share_launches();                       // pass 4
+    }
+};
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------------------
+
+int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags) {
+    graph_replay = (flags & DSC_SCHEDULE_GRAPH_REPLAY) != 0;
+    n_nodes = desc.n_nodes;
+    n_params = desc.n_params;
+    n_clusters = desc.n_clusters;
+    node_bytes.assign(n_nodes, 0);
+    for (int i = 0; i < n_nodes; ++i) node_bytes[i] = (size_t)desc.node_elements[i] * 4;
+    inputs.assign(desc.inputs, desc.inputs + desc.n_inputs);
+    outputs.assign(desc.outputs, desc.outputs + desc.n_outputs);
+    for (auto& io : inputs)
+        if (io.node < 0 || io.node >= n_nodes || io.param < 0 || io.param >= n_params) return fail(DSC_ERR_INVALID, "schedule: bad input entry");
+    for (auto& io : outputs)
+        if (io.node < 0 || io.node >= n_nodes || io.param < 0 || io.param >= n_params) return fail(DSC_ERR_INVALID, "schedule: bad output entry");
+
+    std::vector<bool> is_graph_output(n_nodes, false), is_graph_input(n_nodes, false);
+    for (auto& io : outputs) is_graph_output[io.node] = true;
+    for (auto& io : inputs) is_graph_input[io.node] = true;
+
+    // one draft per reference cluster
+    std::vector<Draft> drafts(desc.n_clusters);
+    for (int c = 0; c < desc.n_clusters; ++c) {
+        const dsc_cluster& cl = desc.clusters[c];
+        std::string err = validate(cl.kernel);
+        if (!err.empty()) return fail(DSC_ERR_INVALID, "schedule: cluster " + std::to_string(c) + ": " + err);
+        const int want_in = cl.kernel.kind == DSC_KERNEL_FILL ? 0 : cl.kernel.n_inputs;
+        const int want_out = cl.kernel.kind == DSC_KERNEL_PER_ELEMENT ? cl.kernel.n_outputs : 1;
+        if (cl.n_inputs != want_in || cl.n_outputs != want_out)
+            return fail(DSC_ERR_INVALID, "schedule: cluster " + std::to_string(c) + " binds the wrong number of nodes");
+        Draft& d = drafts[c];
+        d.fk = FusedKernel::plain(cl.kernel);
+        for (int i = 0; i < cl.n_inputs; ++i) {
+            if (cl.inputs[i] < 0 || cl.inputs[i] >= n_nodes) return fail(DSC_ERR_INVALID, "schedule: bad node id");
+            d.params.push_back(cl.inputs[i]);
+        }
+        for (int o = 0; o < cl.n_outputs; ++o) {
+            const dsc_cluster_output& co = cl.outputs[o];
+            if (co.node < 0 || co.node >= n_nodes || co.copy_from >= n_nodes) return fail(DSC_ERR_INVALID, "schedule: bad node id");
+            d.params.push_back(co.node);
+            d.outs.push_back(StepOutput{co.node, co.copy_from, co.copy_from_is_literal != 0, co.literal_bits});
+        }
+        d.covers.push_back(c);
+    }
+
+    if (!(flags & DSC_SCHEDULE_NO_FUSION)) {
+        Planner planner{flags, n_nodes, node_bytes, drafts, is_graph_output, is_graph_input};
+        planner.run();
     }
 
     // materialise the steps

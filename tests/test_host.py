@@ -368,3 +368,16 @@ def test_code_object_cache_hit_miss_and_damaged_files(tmp_path, monkeypatch):
     monkeypatch.setenv("DSC_CACHE_DIR", "off")
     _, delta = compile_once()
     assert delta == (0, 1, 0) and len(list(cache.iterdir())) == 2
+
+
+def test_every_environment_variable_the_library_reads_is_documented():
+    read = set()
+    csrc = os.path.join(ROOT, "descent_amd", "csrc")
+    for name in os.listdir(csrc):
+        if name.endswith((".cpp", ".hpp")):
+            read |= set(re.findall(r'getenv\("(DSC_[A-Z_0-9]+)"\)', open(os.path.join(csrc, name)).read()))
+            # names reached through a loop over a list of strings
+            read |= set(re.findall(r'"(DSC_(?:MM|ROWS|FUSE)_[A-Z_0-9]+)"', open(os.path.join(csrc, name)).read()))
+    assert len(read) >= 15
+    documented = set(re.findall(r"`(DSC_[A-Z_0-9]+)", open(os.path.join(ROOT, "INTEGRATION.md")).read()))
+    assert read <= documented, sorted(read - documented)

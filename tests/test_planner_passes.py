@@ -1,0 +1,99 @@
+"""One small graph per pass of the fusion planner (descent_amd/csrc/schedule.cpp, struct Planner), planned and compiled
+for gfx950 without a GPU; each test reads the listing for the launches the pass must have produced, next to the
+cluster-by-cluster listing of the same graph.  The convolution passes, the row-fused launch and the max-pool fusion
+are read off the ConvNet's listing in test_host.py."""
+import re
+
+from descent_amd import Environment, hip_backend, workloads
+from oracle.cpu_backend import CpuBackend
+
+
+def _env():
+    return Environment(CpuBackend())  # graphs are only built and planned here, never run
+
+
+def _listings(shapes, build):
+    env = _env()
+    params = [env.static_parameter(s, f"p{i}") for i, s in enumerate(shapes)]
+    graph = env.build_graph(lambda scope: build(scope, *params))
+    unfused = hip_backend.check_schedule(graph, fused=False)
+    assert int(unfused.split()[0]) == len(graph.clusters_sorted)
+    return unfused, hip_backend.check_schedule(graph, fused=True)
+
+
+def _value(scope, p):
+    return scope.parameter_value(p)
+
+
+def _chunks(listing):
+    return [int(c) for c in re.findall(r"chunks (\d+)", listing)]
+
+
+def test_a_long_k_over_a_small_product_is_split_over_more_workgroups():
+    unfused, fused = _listings([[8, 200000], [200000, 16], [8, 16]],
+                               lambda s, a, b, c: s.write_parameter_value(c, _value(s, a).matmul(_value(s, b))))
+    # the reference's ceil(k / 1024) chunks against a split that fills 256 compute units
+    assert _chunks(unfused) == [196]
+    assert _chunks(fused)[0] >= 512
+    # the partial products are summed by the Reduce the graph already had, which also takes the final copy
+    assert int(fused.split()[0]) == 2
+    assert re.search(r"Reduce \(k=\d+\) \[1, 1, 8, 16\] \+ PerElement", fused)
+
+
+def test_a_chain_of_reduces_over_neighbouring_axes_becomes_one_reduce():
+    unfused, fused = _listings([[64, 6, 6, 8], [8]], lambda s, x, o: s.write_parameter_value(
+        o, _value(s, x).reduce_sum(0, False).reduce_sum(0, False).reduce_sum(0, False)))
+    assert unfused.count("Reduce (k=") == 3
+    assert int(fused.split()[0]) == 1
+    assert "Reduce (k=2304) [1, 1, 1, 8] + PerElement (2 ops) [8]" in fused
+
+
+def test_a_long_reduce_with_few_outputs_is_split_in_two():
+    unfused, fused = _listings([[4, 1 << 20], [4]], lambda s, x, o: s.write_parameter_value(o, _value(s, x).reduce_sum(1, False)))
+    assert "Reduce (k=1048576) [4, 1]" in unfused and "grid 1x256" in unfused.splitlines()[1]
+    first, second = fused.splitlines()[1:3]
+    assert "Reduce (k=512) [4, 2048, 1]" in first and "grid 2048x256" in first
+    assert "Reduce (k=2048) [4, 1] + PerElement (2 ops) [4]" in second
+
+
+def test_light_producers_are_evaluated_inside_the_matmul_that_reads_them():
+    unfused, fused = _listings([[512, 512], [512, 512], [512, 512]], lambda s, a, b, c: s.write_parameter_value(
+        c, (_value(s, a) * 2.0).matmul(_value(s, b).transpose())))
+    assert unfused.splitlines()[1].startswith("0: PerElement (3 ops) [262144]")
+    first = fused.splitlines()[1]
+    assert first.startswith("0: MatMul (k=512)") and "<1 fused producers>" in first and first.rstrip().endswith("clusters 1 0")
+
+
+def test_a_reduce_applies_its_only_consumer_before_the_store():
+    unfused, fused = _listings([[4096, 256], [256], [256]], lambda s, x, m, o: s.write_parameter_value(
+        o, _value(s, m) * 0.9 + _value(s, x).reduce_sum(0, False)))
+    assert int(unfused.split()[0]) == 2
+    assert "[1, 256] + PerElement (5 ops) [256]" in fused
+    assert not any(line.split(": ")[1].startswith("PerElement") for line in fused.splitlines()[1:] if re.match(r"\d+: ", line))
+
+
+def test_matmul_takes_its_per_element_consumer_as_epilogue():
+    w = workloads.matmul_epilogue(_env(), 512, 256, 384, upload=False)
+    unfused = hip_backend.check_schedule(w.graph, fused=False)
+    fused = hip_backend.check_schedule(w.graph, fused=True)
+    assert int(unfused.split()[0]) == len(w.graph.clusters_sorted) >= 2
+    assert int(fused.split()[0]) == 1 and "+epilogue" in fused
+
+
+def test_bias_gradient_rides_on_the_weight_gradient_that_reads_the_same_array():
+    listing = hip_backend.check_schedule(workloads.convnet(_env(), batch=1000).graph, fused=True)
+    # conv1: filter gradient im2col^T x dC with the column sums of dC (the bias gradient) from the same pass
+    assert re.search(r"MatMul \(k=784000\) \[\d+, 1, 9, 16\] <1 fused producers>  \[tall-k mfma 16x16x4.*\+column sums of B\]", listing)
+    assert re.search(r"Reduce \(k=\d+\) \[1, 1, 1, 16\]; Reduce \(k=\d+\) \[1, 1, 9, 16\]", listing)
+
+
+def test_scatter_adds_into_one_accumulator_share_a_launch_and_small_launches_are_grouped():
+    w = workloads.hash_grid_fit(_env(), batch=1 << 12)
+    listing = hip_backend.check_schedule(w.graph, fused=True)
+    chains = [line for line in listing.splitlines() if "Multi (4 kernels: ScatterAdd" in line]
+    assert len(chains) == 16  # one per level: the four corner updates of a level add into one table gradient
+    assert all(line.count("scatter_add: global_atomic_add_f32") == 4 for line in chains)
+    # the sixteen zero fills of the table gradients: one launch ahead of the steps
+    assert "prefill: Multi (16 kernels: Fill(0x00000000)" in listing
+    # Adam updates of the sixteen tables and the MLP: a few shared launches, not one each
+    assert int(listing.split()[0]) <= 40 and len(w.graph.clusters_sorted) > 200
