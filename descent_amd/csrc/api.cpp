@@ -489,8 +489,8 @@ int dsc_kernel_launch(dsc_ctx* ctx, dsc_kernel* kernel, const dsc_buf* bufs, int
     if (!ctx || !kernel || (!bufs && n)) return fail(DSC_ERR_INVALID, "null argument");
     Kernel* k = reinterpret_cast<Kernel*>(kernel);
     if (n != k->gen.n_buffers) return fail(DSC_ERR_INVALID, "wrong number of buffers for '" + k->label + "'");
-    if (n > 64) return fail(DSC_ERR_UNSUPPORTED, "more than 64 buffers");
-    void* ptrs[64];
+    if (n > 256) return fail(DSC_ERR_UNSUPPORTED, "more than 256 buffers");
+    void* ptrs[256];
     // every bound buffer must hold at least what the kernel addresses
     const dsc_kernel_desc& d = k->fused.main.raw();
     for (int i = 0; i < n; ++i) {

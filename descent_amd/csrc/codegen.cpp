@@ -395,6 +395,7 @@ string entry_name(const FusedKernel& fk) {
                       : dot_kernel_applies(fk, g)    ? "dsc_matmul_dot"
                                                      : "dsc_matmul_mfma";
         if (fk.has_epilogue) base += "_epilogue";
+        if (fk.out_slice_width) base += "_slices" + count(fk.out_slice_width);
         return base + "_b" + count(g.batch) + "_m" + count(g.m) + "_n" + count(g.n) + "_k" + count(g.k);
     }
     case DSC_KERNEL_UNPAD: return string(fk.has_epilogue ? "dsc_unpad_epilogue_n" : "dsc_unpad_n") + count(element_count(d.shape));
@@ -862,8 +863,10 @@ string gen_scatter_add(Emitter& em, Generated* out) {
     auto emit_element = [&](const string& gid, const string& sfx) { emit_scatter_element(em, k, gid, sfx); };
     if (priv) {
         const int U = 4;  // elements per thread and trip: their loads are all issued before the first LDS atomic
-        k << "    __shared__ float acc[" << S(table) << "];\n";
-        k << "    for (int i = threadIdx.x; i < " << S(table) << "; i += 256) acc[i] = 0.f;\n    __syncthreads();\n";
+        // The sums are kept in double: on gfx950 ds_add_f64 runs seven times faster than ds_add_f32 (0.18 against
+        // 1.27 ns per add and CU, measured with random targets), and the rounding of the partial sums goes away.
+        k << "    __shared__ double acc[" << S(table) << "];\n";
+        k << "    for (int i = threadIdx.x; i < " << S(table) << "; i += 256) acc[i] = 0.0;\n    __syncthreads();\n";
         k << "    for (uint g0 = blockIdx.x * 256u + threadIdx.x; g0 < " << S(n) << "u; g0 += " << S(wgs * 256 * U) << "u) {\n";
         for (int u = 0; u < U; ++u) {
             k << "    const uint gid" << u << " = min(g0 + " << S(u * wgs * 256) << "u, " << S(n - 1) << "u);\n";
@@ -871,9 +874,9 @@ string gen_scatter_add(Emitter& em, Generated* out) {
         }
         k << "    __builtin_amdgcn_sched_barrier(0);\n";
         for (int u = 0; u < U; ++u)
-            k << "    if (ok" << u << " && g0 + " << S(u * wgs * 256) << "u < " << S(n) << "u) atomicAdd(&acc[at" << u << "], value" << u << ");\n";
+            k << "    if (ok" << u << " && g0 + " << S(u * wgs * 256) << "u < " << S(n) << "u) atomicAdd(&acc[at" << u << "], (double)value" << u << ");\n";
         k << "    }\n    __syncthreads();\n";
-        k << "    for (int i = threadIdx.x; i < " << S(table) << "; i += 256) {\n        const float total = acc[i];\n";
+        k << "    for (int i = threadIdx.x; i < " << S(table) << "; i += 256) {\n        const float total = (float)acc[i];\n";
         k << "        if (total != 0.f) unsafeAtomicAdd(&b" << fk.outputs[0] << "[i], total);\n    }\n}\n";
     } else {
         k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n";
@@ -883,7 +886,7 @@ string gen_scatter_add(Emitter& em, Generated* out) {
     out->grid = priv ? (unsigned)wgs : blocks_for(n, 256);
     out->block = 256;
     out->source = k.str();
-    out->note = priv ? "scatter_add: per-workgroup sums in LDS (ds_add_f32), then global_atomic_add_f32" : "scatter_add: global_atomic_add_f32";
+    out->note = priv ? "scatter_add: per-workgroup sums in LDS (ds_add_f64), then global_atomic_add_f32" : "scatter_add: global_atomic_add_f32";
     return "";
 }
 
@@ -1989,7 +1992,9 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
         k << "    __syncthreads();\n";
     }
     const int Q = (int)(g.n / 4);  // 16-byte pieces per row
-    const bool transposed_store = vec_store && (Q == 1 || Q == 2 || Q == 4 || Q == 8);
+    const int64_t W = fk.out_slice_width;  // slice-major store: a lane writes w floats of every slice, lanes on consecutive rows
+    if (W && (g.n % W != 0 || g.batch != 1 || fk.has_epilogue || rows)) return "matmul rows: slice-major store needs one batch, no epilogue and whole slices";
+    const bool transposed_store = !W && vec_store && (Q == 1 || Q == 2 || Q == 4 || Q == 8);
     // With at most 16 columns and a k of some length the products go through v_mfma_f32_16x16x4f32 instead of
     // scalar-operand FMAs (twice the fp32 rate with packed math off): a wave takes its 64 rows as four 16-row tiles,
     // lane l feeds A[row l % 16][k = 4 s + l / 16] straight from memory (the same generated load, so an im2col view
@@ -2090,7 +2095,18 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
     k << "#pragma unroll\n    for (int r = 0; r < " << R << "; ++r) {\n";
     k << "    const int cm = row0 + r * 256;\n    if (cm < " << S(g.m) << ") {\n";
     k << "    const int c_row = cb * " << S(batch_stride) << " + cm * " << S(row_stride) << ";\n";
-    if (vec_store) {
+    if (W) {
+        for (int64_t sl = 0; sl < g.n / W; ++sl) {
+            const string at = "b" + to_string(fk.outputs[0]) + " + (" + S(sl * g.m) + " + cm) * " + S(W);
+            const string a0 = "acc[r][" + S(sl * W) + "]";
+            if (W == 2) k << "    *(float2*)(" << at << ") = make_float2(acc[r][" << S(sl * W) << "], acc[r][" << S(sl * W + 1) << "]);\n";
+            else if (W == 4)
+                k << "    *(float4*)(" << at << ") = make_float4(acc[r][" << S(sl * W) << "], acc[r][" << S(sl * W + 1) << "], acc[r][" << S(sl * W + 2) << "], acc[r][" << S(sl * W + 3) << "]);\n";
+            else
+                for (int64_t j = 0; j < W; ++j) k << "    (" << at << ")[" << S(j) << "] = acc[r][" << S(sl * W + j) << "];\n";
+        }
+        k << "    (void)c_row;\n";
+    } else if (vec_store) {
         k << "#pragma unroll\n    for (int n = 0; n < " << S(g.n) << "; n += 4) {\n";
         if (fk.has_epilogue) {
             k << "        float res[4][" << n_out << "];\n";
@@ -2119,7 +2135,7 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
     out->source = k.str();
     out->note = (use_mfma ? string("row-per-thread store, mfma 16x16x4 from memory, B in registers")
                           : string("row-per-thread fma, B ") + (b_in_lds ? "in LDS" : "in SGPRs")) +
-                (fk.has_epilogue ? " +epilogue" : "");
+                (fk.has_epilogue ? " +epilogue" : "") + (W ? ", product stored as " + S(g.n / W) + " column slices of width " + S(W) : string());
     return "";
 }
 
@@ -2279,6 +2295,7 @@ string gen_matmul(Emitter& em, Generated* out) {
     const bool rows = d.output_mode == DSC_MATMUL_ROWS;
     if (fk.colsum_out >= 0 && (rows_kernel_applies(fk, g) || smallk_kernel_applies(fk, g)))
         return "matmul: column sums need the MFMA template or the tall-k kernel";
+    if (fk.out_slice_width && (!rows_kernel_applies(fk, g) || fk.dgrad.on || fk.cfwd.on)) return "matmul: only the row-per-thread kernel stores slice-major";
     if (rows_kernel_applies(fk, g)) return gen_matmul_rows(em, out);
     if (smallk_kernel_applies(fk, g)) return gen_matmul_smallk(em, out);
     if (tallk_kernel_applies(fk, g)) return gen_matmul_tallk(em, out);
@@ -2551,11 +2568,14 @@ std::string FusedKernel::key() const {
         }
     }
     if (shared_scatter) s += "|SS";
+    if (chain_group) s += "|CG";
+    if (binned_stage) s += "|BS" + to_string(binned_stage) + "," + to_string((long long)binned_table) + "," + to_string((long long)binned_total);
     for (size_t i = 0; i < parts.size(); ++i) {
         s += "|P{" + parts[i].key() + "}";
         for (int j : part_params[i]) s.append(reinterpret_cast<const char*>(&j), 4);
     }
     s += sum_chunks ? "|S1" : "|S0";
+    if (out_slice_width) s += "|OSW" + to_string((long long)out_slice_width);
     if (as_part) s += "|AP";
     if (colsum_out >= 0) s += "|CS" + to_string(colsum_out);
     s += "|O";
@@ -2572,6 +2592,9 @@ std::string FusedKernel::key() const {
 namespace {
 string generate_multi(const FusedKernel& fk, Generated* out);
 string generate_scatter_chain(const FusedKernel& fk, Generated* out);
+string generate_scatter_bin(const FusedKernel& fk, Generated* out);
+string generate_scatter_sum(const FusedKernel& fk, Generated* out);
+string generate_chain_group(const FusedKernel& fk, Generated* out);
 }
 
 bool conv_fwd_fits(const FusedKernel::ConvFwd& c, int64_t n) {
@@ -2588,7 +2611,7 @@ bool conv_dgrad_fits(const FusedKernel::ConvDgrad& c, int64_t k) {
 bool conv_bwd_fits(const FusedKernel::ConvDgrad& c, int64_t k) { return conv_bwd_fits_impl(c, k); }
 
 bool can_be_part(const FusedKernel& fk) {
-    if (!fk.parts.empty()) return false;
+    if (!fk.parts.empty() || fk.binned_stage || fk.chain_group) return false;
     if (fk.dgrad.on || fk.cfwd.on || !fk.row_stages.empty()) return true;
     if (fk.main.raw().kind != DSC_KERNEL_MATMUL) return true;
     // of the MatMul kernels, the row-per-thread, short-k and tall-k ones run 256 threads addressed by blockIdx.x
@@ -2604,6 +2627,9 @@ bool can_be_part(const FusedKernel& fk) {
 static std::string generate_one(const FusedKernel& fk, Generated* out, bool with_prelude);
 
 std::string generate(const FusedKernel& fk, Generated* out) {
+    if (fk.chain_group) return generate_chain_group(fk, out);
+    if (fk.binned_stage == 1) return generate_scatter_bin(fk, out);
+    if (fk.binned_stage == 2) return generate_scatter_sum(fk, out);
     if (!fk.parts.empty() && fk.shared_scatter) return generate_scatter_chain(fk, out);
     if (!fk.parts.empty()) return generate_multi(fk, out);
     return generate_one(fk, out, true);
@@ -2692,7 +2718,7 @@ string generate_scatter_chain(const FusedKernel& fk, Generated* out) {
         if (d.kind != DSC_KERNEL_SCATTER_ADD || !same_shape(d.shape, first.shape)) return "scatter chain: parts differ";
         total += element_count(d.inputs[0].out_shape);
     }
-    if (table * 4 > 144 * 1024) return "scatter chain: accumulator does not fit LDS";
+    if (table * 8 > 144 * 1024) return "scatter chain: accumulator does not fit LDS";
     // One workgroup per CU when there is work for that many: measured on hash-grid levels (2.1 M values), the LDS adds
     // take about 1 ns each per CU, so halving the workgroups costs more than the smaller flush (every workgroup
     // flushes the whole accumulator) gives back, up to the largest accumulator that fits.  A thread fetches U values
@@ -2703,7 +2729,8 @@ string generate_scatter_chain(const FusedKernel& fk, Generated* out) {
     const int64_t wgs = std::max<int64_t>(64, std::min<int64_t>(256, (nmax + 1024 * U - 1) / (1024 * U)));
     Generated g;
     std::ostringstream src, fetches, adds;
-    src << kPreludeSource << "\n";
+    if (!fk.as_part) src << kPreludeSource << "\n";
+    const string block_id = fk.as_part ? "dsc_block" : "blockIdx.x";
     int out_param = -1;
     for (size_t i = 0; i < fk.parts.size(); ++i) {
         const FusedKernel& part = fk.parts[i];
@@ -2722,39 +2749,277 @@ string generate_scatter_chain(const FusedKernel& fk, Generated* out) {
             fetches << "        part" << i << "::fetch(min(" << gid << ", " << S(n - 1) << "u), &v" << id << ", &a" << id << ", &k" << id;
             for (int j : fk.part_params[i]) fetches << ", b" << j;
             fetches << ", rand_seed);\n";
-            adds << "        if (k" << id << " && " << gid << " < " << S(n) << "u) atomicAdd(&acc[a" << id << "], v" << id << ");\n";
+            adds << "        if (k" << id << " && " << gid << " < " << S(n) << "u) atomicAdd(&acc[a" << id << "], (double)v" << id << ");\n";
         }
         out_param = fk.part_params[i][part.outputs[0]];
         Generated pg;  // for the work figures only
         if (generate_one(part, &pg, false).empty()) g.algo_bytes += pg.algo_bytes;
     }
     std::ostringstream body;
-    body << "    for (uint g0 = blockIdx.x * 1024u + threadIdx.x; g0 < " << S(nmax) << "u; g0 += " << S(wgs * 1024 * U) << "u) {\n"
+    body << "    for (uint g0 = " << block_id << " * 1024u + threadIdx.x; g0 < " << S(nmax) << "u; g0 += " << S(wgs * 1024 * U) << "u) {\n"
          << fetches.str() << "        __builtin_amdgcn_sched_barrier(0);\n" << adds.str() << "    }\n";
     Emitter em(fk);
     g.entry = "dsc_scatter_chain_l" + to_string(fk.parts.size()) + "_t" + S(table) + "_n" + S(total);
-    src << "extern \"C\" __global__ __launch_bounds__(1024) void " << g.entry << "(" << em.kernel_params_decl() << ") {\n";
+    if (fk.as_part) {
+        src << "DSC_INLINE void part_entry(const uint dsc_block, char* dsc_lds, " << em.kernel_params_decl() << ") {\n";
+        src << "    double* const acc = reinterpret_cast<double*>(dsc_lds);\n";
+    } else {
+        src << "extern \"C\" __global__ __launch_bounds__(1024) void " << g.entry << "(" << em.kernel_params_decl() << ") {\n";
+        src << "    __shared__ double acc[" << S(table) << "];\n";
+    }
+    g.lds_bytes = (size_t)table * 8;
     src << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
-    src << "    __shared__ float acc[" << S(table) << "];\n";
-    src << "    for (int i = threadIdx.x; i < " << S(table) << "; i += 1024) acc[i] = 0.f;\n    __syncthreads();\n";
+    src << "    for (int i = threadIdx.x; i < " << S(table) << "; i += 1024) acc[i] = 0.0;\n    __syncthreads();\n";
     src << body.str();
     src << "    __syncthreads();\n";
-    src << "    for (int i = threadIdx.x; i < " << S(table) << "; i += 1024) {\n        const float sum = acc[i];\n";
+    src << "    for (int i = threadIdx.x; i < " << S(table) << "; i += 1024) {\n        const float sum = (float)acc[i];\n";
     src << "        if (sum != 0.f) unsafeAtomicAdd(&b" << out_param << "[i], sum);\n    }\n}\n";
     g.source = src.str();
     g.grid = (unsigned)wgs;
     g.block = 1024;
     g.n_buffers = fk.n_buffers;
     g.note = "scatter chain: " + to_string(fk.parts.size()) + " links into one accumulator of " + S(table) +
-             " floats kept in LDS per workgroup (ds_add_f32), then global_atomic_add_f32";
+             " floats kept in LDS per workgroup (as doubles, ds_add_f64), then global_atomic_add_f32";
+    *out = g;
+    return "";
+}
+
+// Stage 1 of the two-launch ScatterAdd chain (FusedKernel::binned_stage): 1024 threads take 8192 values of one link,
+// count them per accumulator segment in LDS (the add returns each record's rank inside its segment), turn the
+// counts into offsets with one scan, reserve room in every segment's bin with one counter add per segment, order
+// the records by segment in LDS and copy them out: consecutive LDS slots of one segment land on consecutive
+// addresses, so the stores of a wave fall into a few runs instead of 64 places.
+string generate_scatter_bin(const FusedKernel& fk, Generated* out) {
+    const dsc_kernel_desc& first = fk.parts[0].main.raw();
+    const int64_t table = element_count(first.shape);
+    int64_t total = 0;
+    for (auto& part : fk.parts) {
+        const dsc_kernel_desc& d = part.main.raw();
+        if (d.kind != DSC_KERNEL_SCATTER_ADD || !same_shape(d.shape, first.shape)) return "binned scatter: parts differ";
+        total += element_count(d.inputs[0].out_shape);
+    }
+    if (table != fk.binned_table || total != fk.binned_total || fk.outputs.size() != 3) return "binned scatter: geometry differs from the plan";
+    const BinnedScatterPlan bp = binned_scatter_plan(table, total);
+    if (bp.nseg > 1024 || bp.nseg * bp.cap >= ((int64_t)1 << 31) || table >= ((int64_t)1 << 31)) return "binned scatter: accumulator too large";
+    if (bp.nseg != 256) return "binned scatter: the kernels take 256 segments";
+    const int U = 8;
+    const int64_t per_wg = 1024 * U;
+    const int rec = fk.outputs[0], cur = fk.outputs[1], acc = fk.outputs[2];
+    Generated g;
+    std::ostringstream src, fetches;
+    if (!fk.as_part) src << kPreludeSource << "\n";
+    const string block_id = fk.as_part ? "dsc_block" : "blockIdx.x";
+    int64_t first_wg = 0;
+    double rmw = 0;
+    for (size_t i = 0; i < fk.parts.size(); ++i) {
+        const FusedKernel& part = fk.parts[i];
+        if ((int)fk.part_params[i].size() != part.n_buffers) return "binned scatter: part parameter count";
+        Emitter em(part);
+        const int64_t n = element_count(part.main.raw().inputs[0].out_shape);
+        std::ostringstream fn;
+        fn << "DSC_INLINE void fetch(const uint gid, float* out_value, int* out_at, bool* out_ok, " << em.params_decl() << ") {\n";
+        emit_scatter_element(em, fn, "gid", "");
+        fn << "    *out_value = value;\n    *out_at = at;\n    *out_ok = ok;\n}\n";
+        src << "namespace part" << i << " {\n" << em.funcs.str() << fn.str() << "}  // namespace part" << i << "\n\n";
+        const int64_t wgs = (n + per_wg - 1) / per_wg;
+        fetches << "    " << (i ? "else " : "") << "if (" << block_id << " < " << S(first_wg + wgs) << "u) {\n";
+        fetches << "        const uint g0 = (" << block_id << " - " << S(first_wg) << "u) * " << S(per_wg) << "u + tid;\n";
+        for (int u = 0; u < U; ++u) {
+            fetches << "        part" << i << "::fetch(min(g0 + " << S(u * 1024) << "u, " << S(n - 1) << "u), &v" << u << ", &a" << u << ", &k" << u;
+            for (int j : fk.part_params[i]) fetches << ", b" << j;
+            fetches << ", rand_seed);\n";
+            fetches << "        k" << u << " = k" << u << " && g0 + " << S(u * 1024) << "u < " << S(n) << "u;\n";
+        }
+        fetches << "    }\n";
+        first_wg += wgs;
+        Generated pg;  // for the work figures only
+        if (generate_one(part, &pg, false).empty()) g.algo_bytes += pg.algo_bytes;
+        rmw += 8.0 * (double)std::min(table, n);
+    }
+    g.algo_bytes = std::max(0.0, g.algo_bytes - rmw);  // the accumulator's read-modify-write is stage 2's work
+    Emitter em(fk);
+    g.entry = "dsc_scatter_bin_l" + to_string(fk.parts.size()) + "_t" + S(table) + "_n" + S(total);
+    if (fk.as_part) {
+        src << "DSC_INLINE void part_entry(const uint dsc_block, char* dsc_lds, " << em.kernel_params_decl() << ") {\n";
+        src << "    float2* const stage = reinterpret_cast<float2*>(dsc_lds);\n";
+        src << "    uint* const cnt = reinterpret_cast<uint*>(dsc_lds + " << S(per_wg * 8) << ");\n";
+        src << "    uint* const lbase = cnt + " << S(bp.nseg) << ";\n    uint* const gbase = lbase + " << S(bp.nseg) << ";\n    uint* const wsum = gbase + " << S(bp.nseg) << ";\n";
+    } else {
+        src << "extern \"C\" __global__ __launch_bounds__(1024) void " << g.entry << "(" << em.kernel_params_decl() << ") {\n";
+        src << "    __shared__ uint cnt[" << S(bp.nseg) << "], lbase[" << S(bp.nseg) << "], gbase[" << S(bp.nseg) << "], wsum[16];\n";
+        src << "    __shared__ float2 stage[" << S(per_wg) << "];\n";
+    }
+    g.lds_bytes = (size_t)(per_wg * 8 + (3 * bp.nseg + 16) * 4);
+    src << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
+    src << "    const uint tid = threadIdx.x;\n";
+    src << "    for (uint i = tid; i < " << S(bp.nseg) << "u; i += 1024u) cnt[i] = 0u;\n    __syncthreads();\n";
+    for (int u = 0; u < U; ++u) src << "    float v" << u << " = 0.f; int a" << u << " = 0; bool k" << u << " = false;\n";
+    src << fetches.str();
+    src << "    __builtin_amdgcn_sched_barrier(0);\n";
+    for (int u = 0; u < U; ++u) src << "    const uint r" << u << " = k" << u << " ? atomicAdd(&cnt[(a" << u << " >> 4) & 255], 1u) : 0u;\n";
+    src << "    __syncthreads();\n";
+    src << "    const uint c = tid < " << S(bp.nseg) << "u ? cnt[tid] : 0u;\n";
+    src << "    uint incl = c;\n";
+    src << "#pragma unroll\n    for (int d = 1; d < 64; d <<= 1) {\n        const uint up = __shfl_up(incl, d);\n        if ((int)(tid & 63u) >= d) incl += up;\n    }\n";
+    src << "    if ((tid & 63u) == 63u) wsum[tid >> 6] = incl;\n    __syncthreads();\n";
+    src << "    uint before = 0u, filled = 0u;\n";
+    src << "#pragma unroll\n    for (uint w = 0; w < 16u; ++w) {\n        const uint s = wsum[w];\n        if (w < (tid >> 6)) before += s;\n        filled += s;\n    }\n";
+    src << "    uint* const cursor = reinterpret_cast<uint*>(b" << cur << ");\n";
+    src << "    if (tid < " << S(bp.nseg) << "u) {\n        lbase[tid] = before + incl - c;\n        gbase[tid] = c ? atomicAdd(&cursor[tid * 16u], c) : 0u;\n    }\n";
+    src << "    __syncthreads();\n";
+    for (int u = 0; u < U; ++u)
+        src << "    if (k" << u << ") stage[lbase[(a" << u << " >> 4) & 255] + r" << u << "] = make_float2(__int_as_float(a" << u << "), v" << u << ");\n";
+    src << "    __syncthreads();\n";
+    src << "    float2* const records = reinterpret_cast<float2*>(b" << rec << ");\n";
+    src << "    for (uint slot = tid; slot < filled; slot += 1024u) {\n";
+    src << "        const float2 r = stage[slot];\n        const int a = __float_as_int(r.x);\n        const uint bin = ((uint)a >> 4) & 255u;\n";
+    src << "        const uint pos = gbase[bin] + (slot - lbase[bin]);\n";
+    src << "        if (pos < " << S(bp.cap) << "u) records[bin * " << S(bp.cap) << "u + pos] = r;\n";
+    src << "        else unsafeAtomicAdd(&b" << acc << "[a], r.y);\n    }\n}\n";
+    g.source = src.str();
+    g.grid = (unsigned)first_wg;
+    g.block = 1024;
+    g.n_buffers = fk.n_buffers;
+    g.note = "scatter chain, stage 1 of 2: " + to_string(fk.parts.size()) + " links, (target, value) records ordered by segment in LDS (" + S(bp.nseg) +
+             " segments of " + S(bp.seg) + " floats, the accumulator's 64-byte lines dealt to them in turn), written in runs into bins of " + S(bp.cap) + " records";
+    *out = g;
+    return "";
+}
+
+// Stage 2: a workgroup sums the records of one segment (or of its slice of them) in LDS and adds the segment to the
+// accumulator, lanes on consecutive addresses.
+string generate_scatter_sum(const FusedKernel& fk, Generated* out) {
+    const dsc_kernel_desc& d = fk.main.raw();
+    const int64_t table = element_count(d.shape);
+    if (d.kind != DSC_KERNEL_SCATTER_ADD || table != fk.binned_table || fk.inputs.size() != 2 || fk.outputs.size() != 1 || fk.n_buffers != 3 ||
+        fk.inputs[0].buffer < 0 || fk.inputs[1].buffer < 0)
+        return "binned scatter: stage 2 binds records, counters and the accumulator";
+    const BinnedScatterPlan bp = binned_scatter_plan(table, fk.binned_total);
+    if (bp.nseg != 256 || bp.seg * 8 > 144 * 1024 || bp.nseg * bp.cap >= ((int64_t)1 << 31)) return "binned scatter: accumulator too large";
+    const int rec = fk.inputs[0].buffer, cur = fk.inputs[1].buffer, acc = fk.outputs[0];
+    const int U = 4;
+    Emitter em(fk);
+    Generated g;
+    std::ostringstream src;
+    if (!fk.as_part) src << kPreludeSource << "\n";
+    g.entry = "dsc_scatter_sum_t" + S(table) + "_n" + S(fk.binned_total);
+    src << "#ifndef LOCAL\n#define LOCAL(at) ((((at) >> 12) << 4) | ((at) & 15))\n#endif\n";
+    if (fk.as_part) {
+        src << "DSC_INLINE void part_entry(const uint dsc_block, char* dsc_lds, " << em.kernel_params_decl() << ") {\n";
+        src << "    double* const seg = reinterpret_cast<double*>(dsc_lds);\n";
+    } else {
+        src << "extern \"C\" __global__ __launch_bounds__(1024) void " << g.entry << "(" << em.kernel_params_decl() << ") {\n";
+        src << "    __shared__ double seg[" << S(bp.seg) << "];\n";
+    }
+    g.lds_bytes = (size_t)bp.seg * 8;
+    src << "    const uint tid = threadIdx.x;\n";
+    src << "    const uint s = " << (fk.as_part ? "dsc_block" : "blockIdx.x") << " / " << S(bp.slices) << "u, slice = " << (fk.as_part ? "dsc_block" : "blockIdx.x") << " % " << S(bp.slices) << "u;\n";
+    src << "    for (uint i = tid; i < " << S(bp.seg) << "u; i += 1024u) seg[i] = 0.0;\n    __syncthreads();\n";
+    src << "    const uint count = min(reinterpret_cast<const uint*>(b" << cur << ")[s * 16u], " << S(bp.cap) << "u);\n";
+    src << "    const uint lo = (uint)((unsigned long long)count * slice / " << S(bp.slices) << "u), hi = (uint)((unsigned long long)count * (slice + 1u) / " << S(bp.slices) << "u);\n";
+    src << "    const float2* const records = reinterpret_cast<const float2*>(b" << rec << ") + s * " << S(bp.cap) << "u;\n";
+    src << "    uint i = lo + tid;\n";
+    src << "    for (; i + " << S((U - 1) * 1024) << "u < hi; i += " << S(U * 1024) << "u) {\n";
+    for (int u = 0; u < U; ++u) src << "        const float2 r" << u << " = records[i + " << S(u * 1024) << "u];\n";
+    src << "        __builtin_amdgcn_sched_barrier(0);\n";
+    for (int u = 0; u < U; ++u) src << "        atomicAdd(&seg[LOCAL(__float_as_int(r" << u << ".x))], (double)r" << u << ".y);\n";
+    src << "    }\n";
+    src << "    for (; i < hi; i += 1024u) {\n        const float2 r = records[i];\n        atomicAdd(&seg[LOCAL(__float_as_int(r.x))], (double)r.y);\n    }\n";
+    src << "    __syncthreads();\n";
+    // local float j of segment s is float j % 16 of the accumulator's line (j / 16) * 256 + s
+    src << "    for (uint j = tid; j < " << S(bp.seg) << "u; j += 1024u) {\n        const float sum = (float)seg[j];\n";
+    src << "        const int at = (int)((((j >> 4) << 8) + s) << 4 | (j & 15u));\n";
+    if (bp.slices == 1)  // the segment has one owner in this launch
+        src << "        if (sum != 0.f && at < " << S(table) << ") b" << acc << "[at] += sum;\n    }\n}\n";
+    else
+        src << "        if (sum != 0.f && at < " << S(table) << ") unsafeAtomicAdd(&b" << acc << "[at], sum);\n    }\n}\n";
+    g.source = src.str();
+    g.grid = (unsigned)(bp.nseg * bp.slices);
+    g.block = 1024;
+    g.n_buffers = fk.n_buffers;
+    g.algo_bytes = 8.0 * (double)std::min(table, fk.binned_total);
+    g.note = "scatter chain, stage 2 of 2: a workgroup per segment (" + S(bp.nseg) + "), records summed in LDS (as doubles, ds_add_f64), the segment's lines added to the accumulator";
+    *out = g;
+    return "";
+}
+
+// Several chain kernels in one launch (FusedKernel::chain_group): each part is generated as a device function over
+// the launch's one LDS block; workgroup ids [first, first + grid) of the launch run part i.
+string generate_chain_group(const FusedKernel& fk, Generated* out) {
+    if (fk.parts.size() != fk.part_params.size() || fk.parts.empty()) return "chain group: part tables differ";
+    Generated g;
+    std::ostringstream src, body;
+    src << kPreludeSource << "\n";
+    unsigned first = 0;
+    size_t lds = 0;
+    string kinds;
+    for (size_t i = 0; i < fk.parts.size(); ++i) {
+        FusedKernel part = fk.parts[i];
+        if (!(part.binned_stage || (part.shared_scatter && !part.parts.empty())) || part.chain_group) return "chain group: a part is not a chain kernel";
+        part.as_part = true;
+        Generated pg;
+        string err = generate(part, &pg);
+        if (!err.empty()) return err;
+        if (pg.block != 1024 || pg.lds_bytes == 0) return "chain group: unexpected part form";
+        if ((int)fk.part_params[i].size() != part.n_buffers) return "chain group: part parameter count";
+        src << "namespace chain" << i << " {\n" << pg.source << "}  // namespace chain" << i << "\n\n";
+        body << "    if (blockIdx.x < " << first + pg.grid << "u) { chain" << i << "::part_entry(blockIdx.x - " << first << "u, dsc_lds";
+        for (int j : fk.part_params[i]) body << ", b" << j;
+        body << ", seed_cell, seed_value); return; }\n";
+        first += pg.grid;
+        lds = std::max(lds, pg.lds_bytes);
+        g.algo_bytes += pg.algo_bytes;
+        if (i == 0) kinds = pg.note;
+    }
+    Emitter em(fk);
+    g.entry = string(fk.parts[0].binned_stage == 1 ? "dsc_scatter_bin" : fk.parts[0].binned_stage == 2 ? "dsc_scatter_sum" : "dsc_scatter_chain") + "_group" +
+              to_string(fk.parts.size()) + "_g" + to_string(first);
+    src << "extern \"C\" __global__ __launch_bounds__(1024) void " << g.entry << "(" << em.kernel_params_decl() << ") {\n";
+    src << "    __shared__ __attribute__((aligned(16))) char dsc_lds[" << lds << "];\n";
+    src << body.str() << "}\n";
+    g.source = src.str();
+    g.grid = first;
+    g.block = 1024;
+    g.n_buffers = fk.n_buffers;
+    g.note = to_string(fk.parts.size()) + " chains in one launch, the first: " + kinds;
     *out = g;
     return "";
 }
 }  // namespace
 
 bool scatter_chain_in_lds(int64_t table_elements, int64_t total_values) {
-    return table_elements * 4 <= 144 * 1024 && total_values >= 16 * table_elements && total_values >= 65536;
+    static const bool binned = !(std::getenv("DSC_SCATTER_BINNED") && std::getenv("DSC_SCATTER_BINNED")[0] == '0');
+    // With the two-launch form available, accumulators above 32 KiB go there: measured on 2.1 M values, the LDS
+    // chain takes 28 us at 13122 floats and 38 us at 25088 (every workgroup adds its whole copy to memory at the
+    // end), the two launches 31 us at any size, and two workgroups of either launch fit a CU.
+    // (the LDS copy is kept in double, eight bytes per element)
+    const int64_t limit = binned && total_values >= (1 << 18) ? 64 * 1024 : 144 * 1024;
+    return table_elements * 8 <= limit && total_values >= 16 * table_elements && total_values >= 65536;
 }
+
+bool scatter_chain_binned(int64_t table_elements, int64_t total_values) {
+    static const bool enabled = !(std::getenv("DSC_SCATTER_BINNED") && std::getenv("DSC_SCATTER_BINNED")[0] == '0');
+    if (!enabled || scatter_chain_in_lds(table_elements, total_values)) return false;
+    // enough values that two launches pay, several per accumulator line (the closing adds touch every line of every
+    // segment that received something), and an accumulator the segment scan of stage 1 covers
+    return total_values >= (1 << 18) && total_values * 4 >= table_elements && table_elements >= 16 * 256 && table_elements <= 256 * 16384;
+}
+
+BinnedScatterPlan binned_scatter_plan(int64_t table_elements, int64_t total_values) {
+    // The accumulator's 64-byte lines are dealt to 256 segments in turn (line l belongs to segment l % 256): a hash
+    // or a row-major grid index spreads evenly over the low bits of the line number even where its high bits are
+    // skewed (measured on the reference's hash at 2^19 entries: contiguous segments received up to six times
+    // their share), and a segment is still stored in whole lines.
+    BinnedScatterPlan p;
+    p.nseg = 256;
+    const int64_t lines = (table_elements + 15) / 16;
+    p.seg = (lines + p.nseg - 1) / p.nseg * 16;
+    // a quarter more than an even spread needs; what does not fit goes to the accumulator directly
+    p.cap = ((total_values / p.nseg) * 5 / 4 + 2048 + 63) / 64 * 64;
+    p.slices = 1;
+    return p;
+}
+
 
 namespace {
 // One launch running several independent kernels: each part is generated as usual, its entry point turned into a

@@ -71,6 +71,22 @@ struct FusedKernel {
     // ONE copy of the accumulator in LDS, folds its share of every part's values into it and adds the non-zero
     // totals to memory once.
     bool shared_scatter = false;
+    // The same chain when the accumulator is too large for LDS, as two launches that replace one memory atomic per
+    // value (a 64-byte read-modify-write at a random address each) by streamed records:
+    // stage 1 ("bin", a multi-part kernel over the links): every workgroup sorts its share of (target, value)
+    //   records by accumulator segment in LDS, reserves room in each segment's bin with one counter add and writes
+    //   the records there in runs; records that find their bin full are added to the accumulator directly.
+    //   outputs = {records, bin counters (start at 0), accumulator}.
+    // stage 2 ("sum", inputs = {records, bin counters}, output = the accumulator taken over in place): workgroups
+    //   own one segment (or a slice of one segment's records), sum the records in LDS and add the segment to the
+    //   accumulator with consecutive addresses.
+    // Several chain kernels (LDS chains, or stage 1 / stage 2 kernels of binned chains) in one launch of 1024-thread
+    // workgroups: parts[] are those kernels, sharing one LDS block sized for the largest.  The chains of a step do
+    // not depend on one another, and one launch of all of them keeps every CU's two workgroup slots busy while a
+    // workgroup waits on its own chain of memory round trips.
+    bool chain_group = false;
+    int binned_stage = 0;
+    int64_t binned_table = 0, binned_total = 0;  // accumulator elements, values of all links together
     // Data gradient of a stride-1 convolution with few channels, as one kernel: `main` is the MatMul dC x filter^T
     // ([g][(img, oy, ox)][oc] x [g][oc][(fy, fx, c)]); the kernel also does what the reference's WindowsToImage
     // (sum of the windows covering each pixel of the padded image) and the two Unpads after it (fold the
@@ -110,6 +126,10 @@ struct FusedKernel {
         int epilogue_product_input = -1;
         std::vector<Source> epilogue_inputs;
     } pool;
+    // MatMul [m, n] (one batch) whose readers all take narrow column slices [m, w] of the product: the product is
+    // stored slice by slice, [n / w][m][w], so that a reader of one slice walks consecutive memory instead of w
+    // floats out of every row.  The readers' views are rewritten to that layout by the planner.
+    int64_t out_slice_width = 0;
     bool sum_chunks = false;               // MatMul: ignore the descriptor's chunk count, write one full sum
     int colsum_out = -1;                   // MatMul (MFMA template): buffer that takes the column sums of B per k chunk
     bool as_part = false;                  // generated as one part of a multi-part launch (set while the launch is generated)
@@ -129,6 +149,7 @@ struct Generated {
     unsigned block = 64;     // threads per workgroup
     int n_buffers = 0;       // pointer parameters, in order; followed by `const uint* seed_cell, uint seed_value`
     std::string note;        // strategy chosen (for schedule listings)
+    size_t lds_bytes = 0;    // (chain kernels generated as parts) LDS the part needs from the launch's shared block
     // Work one launch stands for, counted the way a roofline wants it: bytes = 4 * (distinct elements of every
     // buffer read, a broadcast or windowed operand at its own size, + elements written; a scatter accumulator is
     // read and written where values land), flops = 2*b*M*N*K of a MatMul (0 otherwise).
@@ -153,6 +174,16 @@ bool conv_fwd_fits(const FusedKernel::ConvFwd& c, int64_t n);
 // Whether a chain of ScatterAdds with this accumulator size and this many values in total runs as one kernel with
 // the accumulator in LDS (shared_scatter).
 bool scatter_chain_in_lds(int64_t table_elements, int64_t total_values);
+
+// The two-launch form of a chain (FusedKernel::binned_stage): whether a chain of this size takes it, and its geometry.
+struct BinnedScatterPlan {
+    int64_t seg = 0;     // accumulator elements per segment (whole 64-byte lines; line l belongs to segment l % nseg)
+    int64_t nseg = 0;    // segments = bins
+    int64_t cap = 0;     // records a bin holds
+    int64_t slices = 0;  // stage-2 workgroups per segment
+};
+bool scatter_chain_binned(int64_t table_elements, int64_t total_values);
+BinnedScatterPlan binned_scatter_plan(int64_t table_elements, int64_t total_values);
 
 // Whether a kernel can be one part of a multi-part launch (256 threads per workgroup, addressed by blockIdx.x only).
 bool can_be_part(const FusedKernel& k);

@@ -644,9 +644,10 @@ int launch_kernel(Context* ctx, Kernel* k, void* const* device_ptrs, int n, uint
     if (n != k->gen.n_buffers)
         return fail(DSC_ERR_INVALID, "kernel '" + k->label + "' takes " + std::to_string(k->gen.n_buffers) + " buffers, got " +
                                          std::to_string(n));
-    void* ptr_values[64];
-    void* args[66];
-    if (n > 64) return fail(DSC_ERR_UNSUPPORTED, "more than 64 buffers bound to one kernel");
+    // 256 pointers are 2 KiB of the 4 KiB a kernel's arguments may take; a launch shared by many chains binds the most
+    void* ptr_values[256];
+    void* args[258];
+    if (n > 256) return fail(DSC_ERR_UNSUPPORTED, "more than 256 buffers bound to one kernel");
     for (int i = 0; i < n; ++i) {
         ptr_values[i] = device_ptrs[i];
         args[i] = &ptr_values[i];

@@ -1556,6 +1556,95 @@ struct Planner {
         }
     }
 
+    // Pass 3d: a MatMul product [m, n] whose readers all take narrow column slices of it (the gradient of sixteen
+    // concatenated two-feature encodings, read back two columns at a time by sixty-four ScatterAdd links) is stored
+    // slice by slice instead of row by row: a reader of w columns then walks consecutive memory instead of w floats
+    // out of every n, which cost the whole product's lines once per reader.  Only the row-per-thread kernel has
+    // the store (a lane owns a row, so lanes write consecutive places of every slice), and every reader's view
+    // must be one whose rows and columns can be told apart: [.., m, n] with whole-slice column ranges, unclamped.
+    void slice_major_products() {
+        static const bool enabled = !(std::getenv("DSC_SLICE_MAJOR") && std::getenv("DSC_SLICE_MAJOR")[0] == '0');
+        if (!enabled) return;
+        for (int pi = 0; pi < (int)drafts.size(); ++pi) {
+            Draft& P = drafts[pi];
+            if (!P.alive || P.fk.main.raw().kind != DSC_KERNEL_MATMUL || P.fk.has_epilogue || P.fk.dgrad.on || P.fk.cfwd.on || !P.fk.parts.empty() ||
+                !P.fk.row_stages.empty() || P.fk.colsum_out >= 0 || P.outs.size() != 1 || P.outs[0].copy_from >= 0)
+                continue;
+            const MatMulDims g = matmul_dims(P.fk.main.raw());
+            if (g.batch != 1 || (g.chunks != 1 && !P.fk.sum_chunks) || g.m < 16384 || P.fk.main.raw().output_mode == DSC_MATMUL_ROWS) continue;
+            const int X = P.outs[0].node;
+            if (is_graph_output[X] || node_bytes[X] != (size_t)(g.m * g.n) * 4) continue;
+            // every view through which X is read
+            std::vector<dsc_view*> views;
+            bool ok = true;
+            for (int di = 0; di < (int)drafts.size() && ok; ++di) {
+                Draft& D = drafts[di];
+                if (!D.alive || di == pi) continue;
+                for (auto& o : D.outs)
+                    if (o.copy_from == X) ok = false;
+                bool reads = false;
+                for (size_t b = 0; b < D.params.size(); ++b)
+                    if (D.params[b] == X) reads = true;
+                if (!reads) continue;
+                FusedKernel& fk = D.fk;
+                if (fk.dgrad.on || fk.cfwd.on || fk.pool.on || !fk.row_stages.empty() || !fk.parts.empty() || fk.binned_stage) { ok = false; break; }
+                auto take = [&](KernelDesc& kd, std::vector<Source>& srcs, int skip) {
+                    if (srcs.size() != kd.inputs.size()) { ok = false; return; }
+                    for (size_t i = 0; i < srcs.size(); ++i) {
+                        if ((int)i == skip || srcs[i].buffer < 0 || D.params[srcs[i].buffer] != X) continue;
+                        for (auto& op : kd.ops)
+                            if (op.kind == DSC_PE_GATHER && op.input_index == (int)i) ok = false;  // indexed by data, not through the view
+                        if (kd.raw().kind != DSC_KERNEL_PER_ELEMENT && kd.raw().kind != DSC_KERNEL_SCATTER_ADD && kd.raw().kind != DSC_KERNEL_REDUCE) ok = false;
+                        views.push_back(&kd.inputs[i]);
+                    }
+                };
+                take(fk.main, fk.inputs, -1);
+                for (auto& v : fk.virtuals) take(v.pe, v.inputs, -1);
+                if (fk.has_epilogue) take(fk.epilogue, fk.epilogue_inputs, fk.epilogue_product_input);
+            }
+            if (!ok || views.size() < 2) continue;
+            // the slice width: the widest column range any reader takes, which must divide n and hold every range whole
+            int64_t W = 0;
+            for (const dsc_view* v : views) {
+                const int r = v->in_shape.rank;
+                if (r < 2 || r + 1 > DSC_MAX_DIM || v->in_shape.dims[r - 1] != g.n || v->in_shape.dims[r - 2] != g.m || any_clamp(*v)) { ok = false; break; }
+                for (int i = 0; i < r - 2; ++i)
+                    if (v->in_shape.dims[i] != 1) ok = false;
+                int64_t lo, hi;
+                axis_span(*v, r - 1, &lo, &hi);
+                W = std::max(W, hi - lo + 1);
+            }
+            if (!ok || W < 1 || W * 4 > 16 || W * 2 > g.n || g.n % W != 0) continue;
+            for (const dsc_view* v : views) {
+                int64_t lo, hi;
+                axis_span(*v, v->in_shape.rank - 1, &lo, &hi);
+                if (lo / W != hi / W) ok = false;
+            }
+            if (!ok) continue;
+            FusedKernel trial = P.fk;
+            trial.out_slice_width = W;
+            Generated probe;
+            if (!generate(trial, &probe).empty()) continue;
+            P.fk.out_slice_width = W;
+            for (dsc_view* v : views) {
+                // [.., m, n] -> [.., n / W, m, W]: rows keep their axis' mapping one place down, the slice becomes an offset
+                const int r = v->in_shape.rank;
+                int64_t lo, hi;
+                axis_span(*v, r - 1, &lo, &hi);
+                const int64_t slice = lo / W;
+                v->in_shape.rank = r + 1;
+                v->in_shape.dims[r - 2] = g.n / W;
+                v->in_shape.dims[r - 1] = g.m;
+                v->in_shape.dims[r] = W;
+                v->in_offset[r] = v->in_offset[r - 1] - slice * W;
+                v->in_offset[r - 1] = v->in_offset[r - 2];
+                v->in_offset[r - 2] = slice;
+                for (int j = 0; j < v->out_shape.rank; ++j)
+                    if (v->map_axis[j] >= r - 2) v->map_axis[j] += 1;
+            }
+        }
+    }
+
     // Pass 3c: max-pooling joins the convolution that feeds it.  By now the pooling is a Reduce(max) over four
     // window elements whose input is a fused producer -- the window copy of the convolution kernel's (activated)
     // output -- possibly with a per-element consumer of its own (pass 3: a dropout select).  The convolution
@@ -1752,10 +1841,147 @@ struct Planner {
             }
             StepOutput out = drafts[i].outs[0];  // the first link says where the accumulator comes from
             out.node = final_node;
+            int64_t total_values = 0;
+            for (int j : chain) total_values += element_count(drafts[j].fk.main.raw().inputs[0].out_shape);
+            const int64_t table = element_count(drafts[i].fk.main.raw().shape);
+            if (!multi.fk.shared_scatter && scatter_chain_binned(table, total_values) && (size_t)table * 4 == node_bytes[final_node]) {
+                // two launches: the links' values go to bins by accumulator segment, then every segment is summed in LDS
+                const BinnedScatterPlan bp = binned_scatter_plan(table, total_values);
+                auto new_node = [&](size_t bytes) {
+                    node_bytes.push_back(bytes);
+                    is_graph_output.push_back(false);
+                    is_graph_input.push_back(false);
+                    return n_nodes++;
+                };
+                const int records = new_node((size_t)(bp.nseg * bp.cap) * 8);
+                const int cursor = new_node((size_t)bp.nseg * 64);  // one counter per 64-byte line
+                const int zero = new_node(0);                       // stands for the literal the counters start from
+                const int mid = new_node(node_bytes[final_node]);   // the accumulator between the two launches
+                for (size_t p = 0; p < multi.params.size(); ++p)
+                    if (multi.params[p] == final_node && multi.fk.buffer_is_output[p]) multi.params[p] = mid;
+                multi.fk.binned_stage = 1;
+                multi.fk.binned_table = table;
+                multi.fk.binned_total = total_values;
+                multi.fk.outputs = {param_index(multi, records, true), param_index(multi, cursor, true), param_index(multi, mid, true)};
+                out.node = mid;
+                multi.outs = {StepOutput{records, -1, false, 0}, StepOutput{cursor, zero, true, 0}, out};
+                Draft sum;
+                sum.fk.main = drafts[i].fk.main;
+                sum.fk.binned_stage = 2;
+                sum.fk.binned_table = table;
+                sum.fk.binned_total = total_values;
+                sum.params = {records, cursor, final_node};
+                sum.fk.buffer_is_output = {false, false, true};
+                sum.fk.n_buffers = 3;
+                Source from_records, from_cursor;
+                from_records.buffer = 0;
+                from_cursor.buffer = 1;
+                sum.fk.inputs = {from_records, from_cursor};
+                sum.fk.outputs = {2};
+                sum.outs = {StepOutput{final_node, mid, false, 0}};
+                for (int j : chain) drafts[j].alive = false;
+                drafts[last] = multi;
+                drafts.insert(drafts.begin() + last + 1, sum);
+                continue;
+            }
             multi.outs.push_back(out);
             multi.fk.outputs.push_back(param_index(multi, final_node, true));
             for (int j : chain) drafts[j].alive = false;
             drafts[last] = multi;
+        }
+    }
+
+    // Pass 3e: the chain launches of a step (LDS chains, stage 1 and stage 2 kernels of binned chains) that stand
+    // next to one another and do not depend on one another share launches: one for the LDS chains, one for all
+    // first stages, one for all second stages.  Each of these kernels is a chain of memory round trips with
+    // barriers in between that occupies a CU with one workgroup; sixteen hash-grid levels launched one by one
+    // leave the machine waiting on those round trips sixteen (or thirty-two) times.
+    void group_chain_launches() {
+        static const bool enabled = !(std::getenv("DSC_CHAIN_GROUPS") && std::getenv("DSC_CHAIN_GROUPS")[0] == '0');
+        if (!enabled) return;
+        auto kind_of = [&](const Draft& d) {
+            if (d.fk.chain_group) return 0;
+            if (d.fk.binned_stage == 1) return 2;
+            if (d.fk.binned_stage == 2) return 3;
+            if (d.fk.shared_scatter && !d.fk.parts.empty()) return 1;
+            return 0;
+        };
+        size_t lo = 0;
+        while (lo < drafts.size()) {
+            if (!drafts[lo].alive || kind_of(drafts[lo]) == 0) { ++lo; continue; }
+            size_t hi = lo;
+            std::vector<int> run;
+            while (hi < drafts.size() && (!drafts[hi].alive || kind_of(drafts[hi]) != 0)) {
+                if (drafts[hi].alive) run.push_back((int)hi);
+                ++hi;
+            }
+            // nothing in the run may read or take over what another member writes, except a second stage its own first
+            std::vector<int> writer(n_nodes, -1);
+            for (int di : run)
+                for (auto& o : drafts[di].outs) writer[o.node] = di;
+            bool ok = run.size() >= 2;
+            int prev_bin = -1;
+            for (int di : run) {
+                const Draft& d = drafts[di];
+                const int kind = kind_of(d);
+                std::vector<int> reads = input_nodes(d);
+                for (auto& o : d.outs)
+                    if (o.copy_from >= 0 && !o.from_literal) reads.push_back(o.copy_from);
+                for (int nd : reads)
+                    if (writer[nd] >= 0 && !(kind == 3 && writer[nd] == prev_bin)) ok = false;
+                for (auto& o : d.outs) {
+                    if (o.copy_from < 0 || o.from_literal) continue;
+                    for (int dj : run) {
+                        if (dj == di) continue;
+                        auto ins = input_nodes(drafts[dj]);
+                        if (std::find(ins.begin(), ins.end(), o.copy_from) != ins.end()) ok = false;
+                    }
+                }
+                if (kind == 2) prev_bin = di;
+                else if (kind == 3) prev_bin = -1;
+            }
+            if (!ok) { lo = hi; continue; }
+            std::vector<Draft> grouped;
+            for (int kind = 1; kind <= 3; ++kind) {
+                std::vector<int> members;
+                for (int di : run)
+                    if (kind_of(drafts[di]) == kind) members.push_back(di);
+                if (members.empty()) continue;
+                size_t bound = 0;
+                for (int di : members) bound += drafts[di].params.size();
+                if (members.size() < 2 || bound > 240) {
+                    for (int di : members) grouped.push_back(drafts[di]);
+                    continue;
+                }
+                Draft G;
+                G.fk.chain_group = true;
+                G.fk.main = drafts[members[0]].fk.main;
+                std::set<int> seen;
+                for (int di : members) {
+                    const Draft& d = drafts[di];
+                    std::vector<int> map;
+                    for (size_t p = 0; p < d.params.size(); ++p) map.push_back(param_index(G, d.params[p], d.fk.buffer_is_output[p]));
+                    G.fk.parts.push_back(d.fk);
+                    G.fk.part_params.push_back(map);
+                    for (int nd : input_nodes(d))
+                        if (seen.insert(nd).second) G.part_inputs.push_back(nd);
+                    G.covers.insert(G.covers.end(), d.covers.begin(), d.covers.end());
+                    for (size_t k = 0; k < d.outs.size(); ++k) {
+                        G.outs.push_back(d.outs[k]);
+                        G.fk.outputs.push_back(map[d.fk.outputs[k]]);
+                    }
+                }
+                Generated probe;
+                if (!generate(G.fk, &probe).empty()) {
+                    for (int di : members) grouped.push_back(drafts[di]);
+                    continue;
+                }
+                grouped.push_back(G);
+            }
+            // the launches take the last places of the run, in the order LDS chains, first stages, second stages
+            for (int di : run) drafts[di].alive = false;
+            for (size_t k = 0; k < grouped.size(); ++k) drafts[run[run.size() - grouped.size() + k]] = grouped[k];
+            lo = hi;
         }
     }
 
@@ -1849,8 +2075,10 @@ struct Planner {
         row_kernels();                          // pass 1b
         inline_producers();                     // pass 2
         attach_epilogues();                     // pass 3
+        slice_major_products();                 // pass 3d
         pool_joins_conv_forward();              // pass 3c
         chain_scatter_adds();                   // pass 3b
+        group_chain_launches();                 // pass 3e
         share_launches();                       // pass 4
     }
 };

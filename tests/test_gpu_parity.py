@@ -350,14 +350,22 @@ def test_scatter_add_chains_vs_float64(hip_backend_session, n, entries, links):
     g, got, want = _scatter_chain_case(genv, n, entries, links, 40 + entries)
     _, oracle, _ = _scatter_chain_case(cenv, n, entries, links, 40 + entries)
     listing = next(iter(g.__dict__["_schedules"].values())).describe()
-    # the index conversions share one launch, the whole chain of scatter-adds another; the third is the Fill that
-    # zeroes the accumulator
-    assert int(listing.split()[0]) == 3 and "Multi (%d kernels: ScatterAdd" % links in listing, listing
-    # accumulators of up to 144 KiB with at least 16 values per entry: one LDS copy per workgroup takes every link
-    if entries * 2 * 4 <= 144 * 1024 and links * n * 2 >= 16 * entries * 2:
+    # the index conversions share one launch, the whole chain of scatter-adds another (two when the values are
+    # binned by accumulator segment first); the last is the Fill that zeroes the accumulator and the bin counters
+    assert "Multi (%d kernels: ScatterAdd" % links in listing, listing
+    # accumulators with at least 16 values per entry, of up to 8192 floats (18432 when the chain has too few values
+    # for the two-launch form): one LDS copy per workgroup takes every link
+    lds_limit = 64 * 1024 if links * n * 2 >= 1 << 18 else 144 * 1024  # the LDS copy is kept in double
+    if entries * 2 * 8 <= lds_limit and links * n * 2 >= 16 * entries * 2:
         assert "accumulator of %d floats kept in LDS" % (entries * 2) in listing, listing
+        assert int(listing.split()[0]) == 3, listing
+    elif links * n * 2 >= 1 << 18:
+        # larger accumulators with enough values: records ordered by segment, then summed segment by segment in LDS
+        assert "stage 1 of 2" in listing and "stage 2 of 2" in listing and "kept in LDS" not in listing, listing
+        assert int(listing.split()[0]) == 4, listing
     else:
-        assert "kept in LDS" not in listing, listing
+        assert "kept in LDS" not in listing and "stage 1 of 2" not in listing, listing
+        assert int(listing.split()[0]) == 3, listing
     assert rel_l2(got, want) <= TOL
     assert rel_l2(oracle, want) <= TOL
 

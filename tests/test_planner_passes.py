@@ -97,3 +97,41 @@ def test_scatter_adds_into_one_accumulator_share_a_launch_and_small_launches_are
     assert "prefill: Multi (16 kernels: Fill(0x00000000)" in listing
     # Adam updates of the sixteen tables and the MLP: a few shared launches, not one each
     assert int(listing.split()[0]) <= 40 and len(w.graph.clusters_sorted) > 200
+
+
+def test_full_size_hash_grid_chains_are_binned_grouped_and_read_a_slice_major_gradient():
+    w = workloads.hash_grid_fit(_env(), batch=1 << 18)
+    listing = hip_backend.check_schedule(w.graph, fused=True)
+    lines = listing.splitlines()
+    # the gradient of the sixteen concatenated two-feature encodings is read two columns at a time by 64 links:
+    # its MatMul stores it slice by slice
+    assert sum("product stored as 16 column slices of width 2" in line for line in lines) == 1, listing
+    # accumulators of up to 8192 floats keep a copy per workgroup in LDS; the five such chains share one launch
+    lds = [line for line in lines if "5 chains in one launch" in line]
+    assert len(lds) == 1 and "kept in LDS per workgroup (as doubles, ds_add_f64)" in lds[0] and "grid 1280x1024" in lds[0], listing
+    # the eleven larger ones go through records binned by accumulator segment: all first stages in one launch, all
+    # second stages in the next
+    first = [i for i, line in enumerate(lines) if "11 chains in one launch, the first: scatter chain, stage 1 of 2" in line]
+    second = [i for i, line in enumerate(lines) if "11 chains in one launch, the first: scatter chain, stage 2 of 2" in line]
+    assert len(first) == 1 and len(second) == 1 and second[0] == first[0] + 1, listing
+    assert "256 segments" in lines[first[0]] and "grid 2816x1024" in lines[first[0]] and "grid 2816x1024" in lines[second[0]]
+    assert int(listing.split()[0]) <= 28
+    # every reference cluster is still covered
+    covered = {int(c) for line in lines if " clusters " in line for c in line.split(" clusters ")[1].split()}
+    assert covered == set(range(len(w.graph.clusters_sorted)))
+
+
+def test_chain_switches_fall_back_to_one_launch_per_chain():
+    # the switches are read once per process, so the other settings are listed by a child process
+    import subprocess
+    import sys
+    code = ("import sys; sys.path.insert(0, %r); from descent_amd import Environment, hip_backend, workloads; "
+            "from oracle.cpu_backend import CpuBackend; "
+            "print(hip_backend.check_schedule(workloads.hash_grid_fit(Environment(CpuBackend()), batch=1 << 18).graph, fused=True))")
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, DSC_SCATTER_BINNED="0", DSC_CHAIN_GROUPS="0", DSC_SLICE_MAJOR="0")
+    listing = subprocess.run([sys.executable, "-c", code % root], env=env, check=True, capture_output=True, text=True).stdout
+    assert "chains in one launch" not in listing and "stage 1 of 2" not in listing and "column slices" not in listing
+    assert listing.count("kept in LDS per workgroup") == 6      # accumulators of up to 18432 floats
+    assert listing.count("scatter_add: global_atomic_add_f32 | scatter_add: global_atomic_add_f32") >= 10
