@@ -2719,14 +2719,14 @@ string generate_scatter_chain(const FusedKernel& fk, Generated* out) {
         total += element_count(d.inputs[0].out_shape);
     }
     if (table * 8 > 144 * 1024) return "scatter chain: accumulator does not fit LDS";
-    // One workgroup per CU when there is work for that many: measured on hash-grid levels (2.1 M values), the LDS adds
-    // take about 1 ns each per CU, so halving the workgroups costs more than the smaller flush (every workgroup
-    // flushes the whole accumulator) gives back, up to the largest accumulator that fits.  A thread fetches U values
-    // of every link before it adds any (one memory round trip per trip, not one per link).
+    // Up to one workgroup per CU.  A thread fetches U values of every link before it adds any (one memory round trip
+    // per trip, not one per link).
     int64_t nmax = 0;
     for (auto& part : fk.parts) nmax = std::max(nmax, element_count(part.main.raw().inputs[0].out_shape));
     const int U = 2;
-    const int64_t wgs = std::max<int64_t>(64, std::min<int64_t>(256, (nmax + 1024 * U - 1) / (1024 * U)));
+    // Every workgroup ends by adding its whole copy to memory, so an accumulator that is large against the values it
+    // receives gets fewer workgroups: at least sixteen values per element and workgroup.
+    const int64_t wgs = std::max<int64_t>(64, std::min<int64_t>(std::min<int64_t>(256, total / (16 * table)), (nmax + 1024 * U - 1) / (1024 * U)));
     Generated g;
     std::ostringstream src, fetches, adds;
     if (!fk.as_part) src << kPreludeSource << "\n";
@@ -2989,10 +2989,10 @@ string generate_chain_group(const FusedKernel& fk, Generated* out) {
 
 bool scatter_chain_in_lds(int64_t table_elements, int64_t total_values) {
     static const bool binned = !(std::getenv("DSC_SCATTER_BINNED") && std::getenv("DSC_SCATTER_BINNED")[0] == '0');
-    // With the two-launch form available, accumulators above 32 KiB go there: measured on 2.1 M values, the LDS
-    // chain takes 28 us at 13122 floats and 38 us at 25088 (every workgroup adds its whole copy to memory at the
-    // end), the two launches 31 us at any size, and two workgroups of either launch fit a CU.
-    // (the LDS copy is kept in double, eight bytes per element)
+    // With the two-launch form available, accumulators above 8192 floats go there (the LDS copy is kept in double:
+    // 64 KiB, so two workgroups still share a CU).  Measured on the hash grid's 2.1 M values per level with the
+    // launches grouped: the LDS chain costs about 4 us per level, the two launches 12 us at any size; moving the
+    // 13122-float level to LDS (105 KiB, one workgroup per CU for the whole group) gained 10 us there and lost 6 here.
     const int64_t limit = binned && total_values >= (1 << 18) ? 64 * 1024 : 144 * 1024;
     return table_elements * 8 <= limit && total_values >= 16 * table_elements && total_values >= 65536;
 }

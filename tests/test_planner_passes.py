@@ -108,7 +108,7 @@ def test_full_size_hash_grid_chains_are_binned_grouped_and_read_a_slice_major_gr
     assert sum("product stored as 16 column slices of width 2" in line for line in lines) == 1, listing
     # accumulators of up to 8192 floats keep a copy per workgroup in LDS; the five such chains share one launch
     lds = [line for line in lines if "5 chains in one launch" in line]
-    assert len(lds) == 1 and "kept in LDS per workgroup (as doubles, ds_add_f64)" in lds[0] and "grid 1280x1024" in lds[0], listing
+    assert len(lds) == 1 and "kept in LDS per workgroup (as doubles, ds_add_f64)" in lds[0] and "grid 545x1024" in lds[0], listing
     # the eleven larger ones go through records binned by accumulator segment: all first stages in one launch, all
     # second stages in the next
     first = [i for i, line in enumerate(lines) if "11 chains in one launch, the first: scatter chain, stage 1 of 2" in line]
