@@ -574,7 +574,7 @@ int dsc_schedule_create(dsc_ctx* ctx, const dsc_schedule_desc* desc, uint32_t fl
 }
 
 int dsc_schedule_destroy(dsc_ctx* ctx, dsc_schedule* s) {
-    (void)ctx;
+    if (ctx && s) s->s.release_replay_buffers(&ctx->c);  // the region and spares of a schedule that replays graphs
     delete s;
     return DSC_OK;
 }

@@ -2192,7 +2192,20 @@ int Schedule::build(Context* ctx, const dsc_schedule_desc& desc, uint32_t flags)
     return DSC_OK;
 }
 
+static bool graphs_by_env() {
+    static const bool on = [] {
+        const char* e = std::getenv("DSC_GRAPHS");
+        return e && e[0] == '1';
+    }();
+    return on;
+}
+
 int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
+    if ((graph_replay || graphs_by_env()) && replay_fixed && !ctx->profiling && launches_per_run() >= 4) {
+        bool handled = false;
+        const int rc = run_replayed(ctx, params, rand_seed, &handled);
+        if (handled) return rc;
+    }
     // environment.rs:326-516, over the fused steps.  Unlike the reference (which panics), a run that cannot be put
     // together leaves `params` and the caller's buffers as they were: until every launch's pointers are resolved
     // nothing the caller owns is released or handed on, and what the attempt allocated is given back.
@@ -2220,11 +2233,7 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
 
     // Pass 1: buffer bookkeeping only -- resolve every launch's pointers (allocation and release are host-side
     // and stream-ordered, so a buffer freed here may be handed to a later launch of the same step).
-    struct Launch {
-        Kernel* kernel;
-        size_t first;  // index into `pointers`
-        int n;
-    };
+    typedef PlannedLaunch Launch;
     std::vector<Launch> launches;
     std::vector<void*> pointers;
     launches.reserve(steps.size() + 4);
@@ -2324,17 +2333,23 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
         }
         return DSC_OK;
     };
-    // opt-in (DSC_SCHEDULE_GRAPH_REPLAY, or DSC_GRAPHS=1 for every schedule): replay needs a step's buffers to land
-    // on the same addresses again, which the shared best-fit heap does not guarantee (parameter buffers move every
-    // step), so by default launches are enqueued directly
-    static const bool graphs_by_env = [] {
-        const char* e = std::getenv("DSC_GRAPHS");
-        return e && e[0] == '1';
-    }();
-    if (ctx->profiling || !(graph_replay || graphs_by_env) || launches.size() < 4) {
+    // opt-in (DSC_SCHEDULE_GRAPH_REPLAY, or DSC_GRAPHS=1 for every schedule); a graph that run_replayed could not lay
+    // out at fixed addresses replays only when the heap happens to hand out the same buffers again
+    if (ctx->profiling || !(graph_replay || graphs_by_env()) || launches.size() < 4) {
         ++direct_runs;
         return enqueue_all();
     }
+    return replay_or_capture(ctx, launches, pointers, rand_seed);
+}
+
+int Schedule::replay_or_capture(Context* ctx, const std::vector<PlannedLaunch>& launches, const std::vector<void*>& pointers, uint32_t rand_seed) {
+    auto enqueue_all = [&]() -> int {
+        for (auto& l : launches) {
+            int rc = launch_kernel(ctx, l.kernel, pointers.data() + l.first, l.n, rand_seed);
+            if (rc != DSC_OK) return rc;
+        }
+        return DSC_OK;
+    };
     // captured launches read the seed from the context's device cell
     int rc = set_seed(ctx, rand_seed);
     if (rc != DSC_OK) return rc;
@@ -2373,6 +2388,44 @@ int Schedule::run(Context* ctx, dsc_buf* params, uint32_t rand_seed) {
     return DSC_OK;
 }
 
+int Schedule::run_replayed(Context* ctx, dsc_buf* params, uint32_t rand_seed, bool* handled) {
+    *handled = false;
+    auto give_back = [&]() {
+        if (replay_region) ctx->heap.free(replay_region);
+        for (dsc_buf h : replay_spare)
+            if (h) ctx->heap.free(h);
+        replay_region = 0;
+        replay_spare.clear();
+        replay_fixed = false;
+    };
+    if (replay_spare.empty()) {
+        // first run: a spare per written parameter, then the region, sized by a placement in an unbounded one
+        replay_spare.assign(n_params, 0);
+        for (auto& io : outputs) {
+            if (replay_spare[io.param]) continue;
+            replay_spare[io.param] = ctx->heap.alloc(std::max<size_t>(node_bytes[io.node], 4));
+            if (!replay_spare[io.param]) { give_back(); return DSC_OK; }
+        }
+        FixedPlan probe;
+        if (plan_fixed(ctx, params, replay_spare.data(), nullptr, (size_t)1 << 46, &probe) != DSC_OK) { give_back(); return DSC_OK; }
+        replay_region_bytes = std::max<size_t>(probe.high, DeviceHeap::kAlign);
+        replay_region = ctx->heap.alloc(replay_region_bytes);
+        if (!replay_region) { give_back(); return DSC_OK; }
+    }
+    void* base = nullptr;
+    if (!ctx->heap.info(replay_region, &base, nullptr)) { give_back(); return DSC_OK; }
+    FixedPlan plan;
+    if (plan_fixed(ctx, params, replay_spare.data(), static_cast<char*>(base), replay_region_bytes, &plan) != DSC_OK) {
+        // e.g. a parameter that was handed in without a buffer: let run() say so in its own words
+        return DSC_OK;
+    }
+    *handled = true;
+    const int rc = replay_or_capture(ctx, plan.launches, plan.pointers, rand_seed);
+    if (rc != DSC_OK) return rc;
+    for (int slot : plan.swapped) std::swap(params[slot], replay_spare[slot]);
+    return DSC_OK;
+}
+
 namespace {
 
 // Offsets inside a fixed region: first fit over the free ranges in address order, 256-byte granules, neighbours merged
@@ -2389,6 +2442,7 @@ class RegionPlanner {
             free_.erase(it);
             if (rest) free_[*offset + need] = rest;
             in_use_ += need;
+            high_ = std::max(high_, *offset + need);
             return true;
         }
         return false;
@@ -2411,15 +2465,16 @@ class RegionPlanner {
         free_[offset] = size;
     }
     size_t in_use() const { return in_use_; }
+    size_t high_water() const { return high_; }
 
   private:
     std::map<size_t, size_t> free_;  // offset -> size
-    size_t in_use_ = 0;
+    size_t in_use_ = 0, high_ = 0;
 };
 
 }  // namespace
 
-int Schedule::run_static(Context* ctx, dsc_buf* params, dsc_buf* spare, uint32_t rand_seed, char* scratch, size_t scratch_bytes) {
+int Schedule::plan_fixed(Context* ctx, const dsc_buf* params, const dsc_buf* spare, char* scratch, size_t scratch_bytes, FixedPlan* plan) {
     // Environment::run's bookkeeping (environment.rs:326-516) with the allocator taken out: where run() asks the heap,
     // a node that ends up as a parameter's new value is placed in the caller's spare buffer of that slot, and every
     // other node at an offset of `scratch`.  A buffer that one node hands to the next (ScatterAdd accumulators) is
@@ -2500,13 +2555,12 @@ int Schedule::run_static(Context* ctx, dsc_buf* params, dsc_buf* spare, uint32_t
         return fail(error.find("does not fit") != std::string::npos ? DSC_ERR_UNSUPPORTED : DSC_ERR_INVALID, error);
     };
 
-    struct Launch {
-        Kernel* kernel;
-        size_t first;
-        int n;
-    };
-    std::vector<Launch> launches;
-    std::vector<void*> pointers;
+    typedef PlannedLaunch Launch;
+    std::vector<Launch>& launches = plan->launches;
+    std::vector<void*>& pointers = plan->pointers;
+    launches.clear();
+    pointers.clear();
+    plan->swapped.clear();
     launches.reserve(steps.size() + 4);
     std::vector<Place> prefilled(prefills.empty() ? 0 : n_nodes);
     for (auto& pf : prefills) {
@@ -2566,19 +2620,36 @@ int Schedule::run_static(Context* ctx, dsc_buf* params, dsc_buf* spare, uint32_t
                                                  " would receive another parameter's buffer; use dsc_schedule_run for this graph");
     }
 
-    for (auto& l : launches) {
-        int rc = launch_kernel(ctx, l.kernel, pointers.data() + l.first, l.n, rand_seed);
+    for (auto& io : outputs)
+        if (place[io.node].where == kSpare) plan->swapped.push_back(io.param);
+    plan->peak = peak;
+    plan->high = region.high_water();
+    return DSC_OK;
+}
+
+int Schedule::run_static(Context* ctx, dsc_buf* params, dsc_buf* spare, uint32_t rand_seed, char* scratch, size_t scratch_bytes) {
+    FixedPlan plan;
+    if (int rc = plan_fixed(ctx, params, spare, scratch, scratch_bytes, &plan)) return rc;
+    for (auto& l : plan.launches) {
+        int rc = launch_kernel(ctx, l.kernel, plan.pointers.data() + l.first, l.n, rand_seed);
         if (rc != DSC_OK) return rc;
     }
-    for (auto& io : outputs)
-        if (place[io.node].where == kSpare) std::swap(params[io.param], spare[io.param]);
-    static_peak_bytes = std::max(static_peak_bytes, peak);
+    for (int slot : plan.swapped) std::swap(params[slot], spare[slot]);
+    static_peak_bytes = std::max(static_peak_bytes, plan.peak);
     return DSC_OK;
 }
 
 Schedule::~Schedule() {
     for (auto& c : captured)
         if (c.exec) (void)hipGraphExecDestroy(c.exec);
+}
+
+void Schedule::release_replay_buffers(Context* ctx) {
+    if (replay_region) ctx->heap.free(replay_region);
+    for (dsc_buf h : replay_spare)
+        if (h) ctx->heap.free(h);
+    replay_region = 0;
+    replay_spare.clear();
 }
 
 int Schedule::launches_per_run() const {

@@ -22,8 +22,25 @@ struct Step {
     std::vector<int> covers;   // reference cluster indices this launch stands for
 };
 
+// One launch of a planned run: `n` pointer arguments starting at `first` in the run's pointer table.
+struct PlannedLaunch {
+    Kernel* kernel = nullptr;
+    size_t first = 0;
+    int n = 0;
+};
+
+// A run whose buffers all sit at addresses known before anything is launched: intermediates at offsets of one
+// region, written parameters in the spare buffer of their slot.
+struct FixedPlan {
+    std::vector<PlannedLaunch> launches;
+    std::vector<void*> pointers;
+    std::vector<int> swapped;  // parameter slots whose new value sits in the spare buffer
+    size_t peak = 0;           // most bytes of the region in use at once
+    size_t high = 0;           // end of the highest placement in the region
+};
+
 // One step's launches with their resolved device pointers, captured once as a HIP graph and replayed whenever a
-// later step resolves to the same pointers (parameter buffers alternate between a few addresses).
+// later step resolves to the same pointers.
 struct CapturedStep {
     std::vector<void*> pointers;  // every pointer argument of every launch, in order
     hipGraphExec_t exec = nullptr;
@@ -35,6 +52,15 @@ struct Schedule {
     int64_t replays = 0, direct_runs = 0;
     size_t static_peak_bytes = 0;  // most scratch a run_static of this schedule has had in use at once
     bool graph_replay = false;  // DSC_SCHEDULE_GRAPH_REPLAY
+    // Graph replay needs a step's pointers to repeat, which buffers taken from the shared heap do not (measured on
+    // the ConvNet: no repeat within eight captures).  A schedule that replays therefore owns one region for its
+    // intermediates and one spare buffer per written parameter: a written parameter alternates between the
+    // caller's buffer and the spare, so the pointer table has period two and two captured graphs serve every step.
+    dsc_buf replay_region = 0;
+    size_t replay_region_bytes = 0;
+    std::vector<dsc_buf> replay_spare;  // per parameter slot, 0 where the slot is not written
+    bool replay_fixed = true;           // cleared when this graph cannot be laid out that way
+    void release_replay_buffers(Context* ctx);  // before the schedule goes, while its context is alive
     ~Schedule();
 
     int n_nodes = 0, n_params = 0, n_clusters = 0;
@@ -54,6 +80,12 @@ struct Schedule {
     // The same launches with every intermediate inside `scratch` (a fixed device array of `scratch_bytes`) and every
     // written parameter in the caller's `spare` buffer of its slot: no device allocation, no heap traffic.
     int run_static(Context* ctx, dsc_buf* params, dsc_buf* spare, uint32_t rand_seed, char* scratch, size_t scratch_bytes);
+    // The placement both of them use; launches nothing.
+    int plan_fixed(Context* ctx, const dsc_buf* params, const dsc_buf* spare, char* scratch, size_t scratch_bytes, FixedPlan* plan);
+    // run() for a schedule that replays graphs, over its own region and spares; *handled is false when the graph
+    // cannot be laid out at fixed addresses (run() then goes on as usual).
+    int run_replayed(Context* ctx, dsc_buf* params, uint32_t rand_seed, bool* handled);
+    int replay_or_capture(Context* ctx, const std::vector<PlannedLaunch>& launches, const std::vector<void*>& pointers, uint32_t rand_seed);
     std::string describe() const;
     // The schedule after fusion as a graphviz digraph (the reference exports its graph before scheduling,
     // src/graph.rs:656-760): one box per launch, one ellipse per parameter slot, one edge per buffer.

@@ -416,7 +416,9 @@ def test_graph_replay_matches_direct_launches_on_every_replay(hip_backend_sessio
     import re
     m = re.search(r"graph replays (\d+), captured (\d+), direct runs (\d+)", listing)
     assert m and int(m.group(1)) + int(m.group(2)) + int(m.group(3)) >= 10, listing
-    assert int(m.group(2)) >= 1, listing  # at least one capture happened
+    # the schedule keeps its intermediates in a region of its own and lets every written parameter alternate between
+    # its buffer and a spare, so a step's pointers repeat with period two: two captures, every other step a replay
+    assert (int(m.group(1)), int(m.group(2)), int(m.group(3))) == (8, 2, 0), listing
 
 
 def _conv_grad_case(env, m, h, w, c_in, c_out, fh, fw, pad, groups, seed):
