@@ -372,8 +372,8 @@ string entry_name(const FusedKernel& fk) {
     auto count = [](int64_t v) { return to_string((long long)v); };
     if (fk.dgrad.on) {
         const MatMulDims g = matmul_dims(d);
-        return string(fk.dgrad.wgrad ? "dsc_conv_bwd_img" : "dsc_conv_dgrad_img") + count(fk.dgrad.img) + "_" + count(fk.dgrad.oh) + "x" + count(fk.dgrad.ow) + "_g" + count(fk.dgrad.g) + "_k" +
-               count(g.k) + "_c" + count(fk.dgrad.c);
+        return string(fk.dgrad.wgrad_only ? "dsc_conv_wgrad_img" : fk.dgrad.wgrad ? "dsc_conv_bwd_img" : "dsc_conv_dgrad_img") + count(fk.dgrad.img) + "_" + count(fk.dgrad.oh) +
+               "x" + count(fk.dgrad.ow) + "_g" + count(fk.dgrad.g) + "_k" + count(fk.dgrad.wgrad_only ? g.n : g.k) + "_c" + count(fk.dgrad.c);
     }
     if (fk.cfwd.on)
         return string(fk.has_epilogue ? "dsc_conv_fwd_epilogue_img" : "dsc_conv_fwd_img") + count(fk.cfwd.img) + "_" + count(fk.cfwd.h) + "x" +
@@ -1140,7 +1140,9 @@ struct ConvBwdLayout {
     int64_t P, TQ, GS, GPR, GROUPS, TILES, TPW;
 };
 
-ConvBwdLayout conv_bwd_layout(const FusedKernel::ConvDgrad& c, int64_t K, int64_t cp_override = 0) {
+ConvBwdLayout conv_bwd_layout(const FusedKernel::ConvDgrad& full, int64_t K, int64_t cp_override = 0) {
+    FusedKernel::ConvDgrad c = full;
+    if (c.wgrad_only && c.bands > 1) c.oh = full.oh / c.bands;  // the tiles hold one band of output rows
     ConvBwdLayout L{};
     L.PH = c.oh + c.fh - 1;
     L.PW = c.ow + c.fw - 1;
@@ -1155,8 +1157,10 @@ ConvBwdLayout conv_bwd_layout(const FusedKernel::ConvDgrad& c, int64_t K, int64_
     L.GROUPS = L.PH * L.GPR;
     L.TILES = (L.GROUPS + 15) / 16;
     L.TPW = (L.TILES + 3) / 4;
-    L.mfma_dgrad = L.P > 0 && L.GS <= 96 && L.TPW <= 8;
-    L.PITCH = dgrad_pitch(K);  // the FMA form reads 16-byte pieces of a slot
+    L.mfma_dgrad = L.P > 0 && L.GS <= 96 && L.TPW <= 8 && !c.wgrad_only;
+    // the FMA form reads 16-byte pieces of a slot; the filter gradient alone reads four consecutive slots' words
+    // li .. li + 15, which K words per slot spread over all banks
+    L.PITCH = c.wgrad_only ? K : dgrad_pitch(K);
     if (L.mfma_dgrad) {
         // words per slot: the one (from k to k + 8) that spreads an A fragment load of the data gradient -- lane l reads
         // word l / 16 of the slot of group l % 16 -- over the most of the 64 banks
@@ -1188,15 +1192,16 @@ ConvBwdLayout conv_bwd_layout(const FusedKernel::ConvDgrad& c, int64_t K, int64_
     L.TOTAL = std::max<int64_t>(L.GB_AT + (L.mfma_dgrad ? L.GS * 64 : 0), (int64_t)4 * L.MT * L.NT * 256);
     // four workgroups per CU (160 KB of LDS) matter more than the input tile's bank spread
     if (cp_override == 0 && L.CP != c.c && L.TOTAL * 4 * 4 > 160 * 1024) {
-        const ConvBwdLayout tight = conv_bwd_layout(c, K, c.c);
+        const ConvBwdLayout tight = conv_bwd_layout(full, K, c.c);
         if (tight.TOTAL * 4 * 4 <= 160 * 1024) return tight;
     }
     return L;
 }
 
 bool conv_bwd_fits_impl(const FusedKernel::ConvDgrad& c, int64_t k) {
-    if (!conv_dgrad_fits(c, k)) return false;
+    if (c.wgrad_only ? (k % 4 != 0 || c.g * c.c > 64) : !conv_dgrad_fits(c, k)) return false;
     const ConvBwdLayout L = conv_bwd_layout(c, k);
+    if (c.bands < 1 || (c.bands > 1 && (!c.wgrad_only || c.oh % c.bands != 0))) return false;
     return L.TOTAL * 4 <= 64 * 1024 && L.MT * L.NT <= 8 && c.chunks >= 8 && c.chunks % 8 == 0;
 }
 
@@ -1205,25 +1210,31 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     const dsc_kernel_desc& d = fk.main.raw();
     const FusedKernel::ConvDgrad& cv = fk.dgrad;
     const MatMulDims g = matmul_dims(d);
-    const int64_t K = g.k, G = cv.g, C = cv.c, FH = cv.fh, FW = cv.fw, OH = cv.oh, OW = cv.ow, IMG = cv.img;
-    if (g.batch != G || g.m != IMG * OH * OW || g.n != FH * FW * C || g.chunks != 1) return "conv backward: geometry mismatch";
+    const bool wonly = cv.wgrad_only;
+    const int64_t BANDS = wonly ? cv.bands : 1, OHF = cv.oh;  // OH below: the output rows a workgroup's tiles hold
+    const int64_t K = wonly ? g.n : g.k, G = cv.g, C = cv.c, FH = cv.fh, FW = cv.fw, OH = OHF / BANDS, OW = cv.ow, IMG = cv.img;
+    if (wonly ? (g.batch != G || g.k != IMG * OHF * OW || g.m != FH * FW * C) : (g.batch != G || g.m != IMG * OH * OW || g.n != FH * FW * C || g.chunks != 1))
+        return "conv backward: geometry mismatch";
     if (fk.inputs.size() != 3 || fk.inputs[2].buffer < 0) return "conv backward: the image must be a buffer";
-    if ((int)fk.outputs.size() != 2 + (cv.bias ? 1 : 0)) return "conv backward: output count";
+    if ((int)fk.outputs.size() != (wonly ? 1 : 2) + (cv.bias ? 1 : 0)) return "conv backward: output count";
+    const int DC = wonly ? 1 : 0;  // which operand of `main` is dC: [g][(img, oy, ox)][oc] either way
     if (!conv_bwd_fits_impl(cv, K)) return "conv backward: geometry does not fit";
     const ConvBwdLayout L = conv_bwd_layout(cv, K);
     const int64_t PH = L.PH, PW = L.PW, KD = L.KD, PITCH = L.PITCH, CP = L.CP, GC = G * C;
-    const int64_t H = PH - 2 * cv.pad_h, W = PW - 2 * cv.pad_w;
+    const int64_t H = OHF + FH - 1 - 2 * cv.pad_h, W = PW - 2 * cv.pad_w;
     const bool unpad = cv.pad_h > 0 || cv.pad_w > 0;
     const int MT = L.MT, NT = L.NT;
     if (H < 1 || W < 1 || K % 4 != 0) return "conv backward: unsupported geometry";
 
-    const string la = em.load_view(fk.inputs[0], d.inputs[0], {"cb", "cm", "ck"});
+    const string la = em.load_view(fk.inputs[DC], d.inputs[DC], {"cb", "cm", "ck"});
     em.funcs << "DSC_INLINE float load_a(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return " << la << ";\n}\n";
-    const string lb = em.load_view(fk.inputs[1], d.inputs[1], {"cb", "ck", "cn"});
-    em.funcs << "DSC_INLINE float load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb << ";\n}\n";
+    if (!wonly) {
+        const string lb = em.load_view(fk.inputs[1], d.inputs[1], {"cb", "ck", "cn"});
+        em.funcs << "DSC_INLINE float load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb << ";\n}\n";
+    }
 
     std::ostringstream k;
-    const string out_ptr = "b" + to_string(fk.outputs[0]), part_ptr = "b" + to_string(fk.outputs[1]);
+    const string out_ptr = "b" + to_string(fk.outputs[0]), part_ptr = "b" + to_string(fk.outputs[wonly ? 0 : 1]);
     const string img_ptr = "b" + to_string(fk.inputs[2].buffer);
     k << "typedef float cb_float4 __attribute__((ext_vector_type(4)));\n";
     k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
@@ -1232,7 +1243,11 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     k << "    float* const lds = smem;\n    float* const xt = smem + " << S(L.XT_AT) << ";\n";
     // the groups of a set of images sit 8 workgroups apart: same XCD, same L2 (they share the lines of dC, of the
     // image and of the output)
-    k << "    const int cb = (blockIdx.x / 8) % " << S(G) << ", chunk = (blockIdx.x / " << S(8 * G) << ") * 8 + blockIdx.x % 8;\n";
+    if (BANDS > 1)
+        k << "    const int band = blockIdx.x / " << S(cv.chunks * G) << ", in_band = blockIdx.x % " << S(cv.chunks * G) << ";\n";
+    else
+        k << "    const int band = 0, in_band = blockIdx.x;\n";
+    k << "    const int cb = (in_band / 8) % " << S(G) << ", chunk = (in_band / " << S(8 * G) << ") * 8 + in_band % 8;\n";
     k << "    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 15, lk = lane >> 4;\n";
     // what stays zero for the whole kernel: slots without a pixel, the zero row, the tile words behind the last pixel
     k << "    for (int i = threadIdx.x; i < " << S(L.ONE_AT) << "; i += 256) smem[i] = 0.f;\n";
@@ -1276,7 +1291,7 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     // second convolution -- the registers that hold them cost a wave of occupancy.)
     // dC in 16-byte pieces when the operand is a buffer whose k runs along memory
     int64_t dc_base = 0, dc_coef[DSC_MAX_DIM] = {0};
-    const bool vec_dc = fk.inputs[0].buffer >= 0 && K % 4 == 0 && affine_form(d.inputs[0], &dc_base, dc_coef) && dc_coef[2] == 1 && dc_base % 4 == 0 &&
+    const bool vec_dc = fk.inputs[DC].buffer >= 0 && K % 4 == 0 && affine_form(d.inputs[DC], &dc_base, dc_coef) && dc_coef[2] == 1 && dc_base % 4 == 0 &&
                         dc_coef[1] % 4 == 0 && (G == 1 || dc_coef[0] % 4 == 0);
     const int64_t dunit = vec_dc ? 4 : 1;
     const int64_t fill_n = OH * OW * K / dunit, NC = (fill_n + 255) / 256;
@@ -1287,14 +1302,14 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NC) << "; ++u) {\n";
         k << ind << "    const int i = min((int)threadIdx.x + u * 256, " << S(fill_n - 1) << ") * " << S(dunit) << ";\n";
         if (vec_dc)
-            k << ind << "    pv[u] = *(const float4*)(b" << fk.inputs[0].buffer << " + " << S(dc_base) << " + cb * " << S(G == 1 ? 0 : dc_coef[0]) << " + (" << img << " * "
-              << S(OH * OW) << " + i / " << S(K) << ") * " << S(dc_coef[1]) << " + i % " << S(K) << ");\n" << ind << "}\n";
+            k << ind << "    pv[u] = *(const float4*)(b" << fk.inputs[DC].buffer << " + " << S(dc_base) << " + cb * " << S(G == 1 ? 0 : dc_coef[0]) << " + (" << img << " * "
+              << S(OHF * OW) << " + band * " << S(OH * OW) << " + i / " << S(K) << ") * " << S(dc_coef[1]) << " + i % " << S(K) << ");\n" << ind << "}\n";
         else
-            k << ind << "    pv[u] = load_a(cb, " << img << " * " << S(OH * OW) << " + i / " << S(K) << ", i % " << S(K) << ", " << em.params_pass() << ");\n" << ind << "}\n";
+            k << ind << "    pv[u] = load_a(cb, " << img << " * " << S(OHF * OW) << " + band * " << S(OH * OW) << " + i / " << S(K) << ", i % " << S(K) << ", " << em.params_pass() << ");\n" << ind << "}\n";
         k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NX) << "; ++u) {\n";
         k << ind << "    const int e = min((int)threadIdx.x + u * 256, " << S(xn - 1) << ") * " << S(unit) << ";\n";
         k << ind << "    const int ch = e % " << S(C) << ", px = (e / " << S(C) << ") % " << S(PW) << ", py = e / " << S(C * PW) << ";\n";
-        k << ind << "    const int sy = clampi(py - " << S(cv.pad_h) << ", 0, " << S(H - 1) << "), sx = clampi(px - " << S(cv.pad_w) << ", 0, " << S(W - 1) << ");\n";
+        k << ind << "    const int sy = clampi(py + band * " << S(OH) << " - " << S(cv.pad_h) << ", 0, " << S(H - 1) << "), sx = clampi(px - " << S(cv.pad_w) << ", 0, " << S(W - 1) << ");\n";
         k << ind << "    xv[u] = *(const " << vt << "*)(" << img_ptr << " + ((" << img << " * " << S(H) << " + sy) * " << S(W) << " + sx) * " << S(GC) << " + cb * " << S(C)
           << " + ch);\n" << ind << "}\n";
         k << ind << "__builtin_amdgcn_sched_barrier(0);\n";
@@ -1303,7 +1318,9 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NC) << "; ++u) {\n";
         k << ind << "    const int i = ((int)threadIdx.x + u * 256) * " << S(dunit) << ", pi = i / " << S(K) << ";\n";
         k << ind << "    float* const at = lds + ((pi / " << S(OW) << ") * " << S(PW) << " + pi % " << S(OW) << ") * " << S(PITCH) << " + i % " << S(K) << ";\n";
-        if (vec_dc)
+        if (vec_dc && PITCH % 4 == 0)
+            k << ind << "    if ((int)threadIdx.x + u * 256 < " << S(fill_n) << ") *(float4*)at = pv[u];\n" << ind << "}\n";
+        else if (vec_dc)
             k << ind << "    if ((int)threadIdx.x + u * 256 < " << S(fill_n) << ") { at[0] = pv[u].x; at[1] = pv[u].y; at[2] = pv[u].z; at[3] = pv[u].w; }\n" << ind << "}\n";
         else
             k << ind << "    if ((int)threadIdx.x + u * 256 < " << S(fill_n) << ") at[0] = pv[u];\n" << ind << "}\n";
@@ -1329,7 +1346,9 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     k << "                    wacc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[mt], fb[nt], wacc[mt][nt], 0, 0, 0);\n";
     k << "        }\n";
     const int64_t passes = (PH * PW + 255) / 256;
-    if (mfma_dgrad) {
+    if (wonly) {
+        k << "        __syncthreads();\n";  // the next image's fills overwrite what the fragments read
+    } else if (mfma_dgrad) {
         // 2b. data gradient: every wave takes every fourth tile of 16 pixel groups
         k << "        cb_float4 dacc[" << S(TPW) << "];\n";
         k << "#pragma unroll\n        for (int t = 0; t < " << S(TPW) << "; ++t) {\n";
@@ -1406,7 +1425,7 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         k << "        __syncthreads();\n";
     }
     }
-    if (unpad) {
+    if (unpad && !wonly) {
         k << "        for (int i = threadIdx.x; i < " << S(H * W * C) << "; i += 256) {\n";
         k << "            const int c = i % " << S(C) << ", x = (i / " << S(C) << ") % " << S(W) << ", y = i / " << S(C * W) << ";\n";
         k << "            float sum = 0.f;\n";
@@ -1451,17 +1470,17 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     k << "        const float sum = (smem[i] + smem[" << S(R) << " + i]) + (smem[" << S(2 * R) << " + i] + smem[" << S(3 * R) << " + i]);\n";
     k << "        const int tile = i >> 8, r = (i >> 6) & 3, l = i & 63;\n";
     k << "        const int cm = (tile / " << NT << ") * 16 + 4 * (l >> 4) + r, cn = (tile % " << NT << ") * 16 + (l & 15);\n";
-    k << "        if (cm < " << S(KD) << " && cn < " << S(K) << ") " << part_ptr << "[(chunk * " << S(G) << " + cb) * " << S(KD * K) << " + cm * " << S(K) << " + cn] = sum;\n";
+    k << "        if (cm < " << S(KD) << " && cn < " << S(K) << ") " << part_ptr << "[((band * " << S(cv.chunks) << " + chunk) * " << S(G) << " + cb) * " << S(KD * K) << " + cm * " << S(K) << " + cn] = sum;\n";
     if (cv.bias)
-        k << "        if (cm == " << S(KD) << " && cn < " << S(K) << ") b" << fk.outputs[2] << "[(chunk * " << S(G) << " + cb) * " << S(K) << " + cn] = sum;\n";
+        k << "        if (cm == " << S(KD) << " && cn < " << S(K) << ") b" << fk.outputs[wonly ? 1 : 2] << "[((band * " << S(cv.chunks) << " + chunk) * " << S(G) << " + cb) * " << S(K) << " + cn] = sum;\n";
     k << "    }\n}\n";
-    if (cv.chunks * G >= kMaxIndex) return "conv backward: grid too large";
-    out->grid = (unsigned)(cv.chunks * G);
+    if (cv.chunks * G * BANDS >= kMaxIndex) return "conv backward: grid too large";
+    out->grid = (unsigned)(cv.chunks * G * BANDS);
     out->block = 256;
     out->source = k.str();
-    out->note = "conv backward: workgroup per group and image set (" + S(cv.chunks) + " sets), dC and input tile in LDS, data gradient " + S(FH) + "x" + S(FW) +
-                " taps x " + S(K) + " channels" + (unpad ? " with border folds" : "") + ", filter gradient mfma 16x16x4 " + to_string(MT) + "x" + to_string(NT) +
-                " tiles" + (cv.bias ? " +column sums of dC" : "");
+    out->note = "conv backward: workgroup per group and image set (" + S(cv.chunks) + " sets), dC and input tile in LDS, " +
+                (wonly ? "no data gradient, " + S(BANDS) + " bands of " + S(OH) + " output rows" : "data gradient " + S(FH) + "x" + S(FW) + " taps x " + S(K) + " channels" + (unpad ? " with border folds" : "")) +
+                ", filter gradient mfma 16x16x4 " + to_string(MT) + "x" + to_string(NT) + " tiles" + (cv.bias ? " +column sums of dC" : "");
     return "";
 }
 
@@ -2458,7 +2477,15 @@ void count_work(const FusedKernel& fk, Generated* g) {
         out_each = (double)(m.batch * m.m * m.n) * (double)(fk.sum_chunks ? 1 : m.chunks);
         g->algo_flops = 2.0 * (double)m.batch * (double)m.m * (double)m.n * (double)m.k;
     }
-    if (fk.dgrad.on) {
+    if (fk.dgrad.on && fk.dgrad.wgrad_only) {
+        // dC and the image in (both counted above: dC through its view, the image through the im2col view, capped at
+        // its size), one partial product and one row of column sums per image set out
+        const FusedKernel::ConvDgrad& c = fk.dgrad;
+        const MatMulDims m = matmul_dims(d);
+        out_each = 0;
+        elements += (double)(c.chunks * c.bands) * (double)c.g * ((double)(c.fh * c.fw * c.c) * (double)m.n + (c.bias ? (double)m.n : 0.0));
+        g->algo_flops = 2.0 * (double)c.g * (double)(c.fh * c.fw * c.c) * (double)m.n * (double)(c.img * c.oh * c.ow);
+    } else if (fk.dgrad.on) {
         const FusedKernel::ConvDgrad& c = fk.dgrad;
         const MatMulDims m = matmul_dims(d);
         const double ph = (double)(c.oh + c.fh - 1), pw = (double)(c.ow + c.fw - 1);
@@ -2569,6 +2596,7 @@ std::string FusedKernel::key() const {
     }
     if (shared_scatter) s += "|SS";
     if (chain_group) s += "|CG";
+    if (dgrad.wgrad_only) s += "|WO" + to_string((long long)dgrad.bands);
     if (binned_stage) s += "|BS" + to_string(binned_stage) + "," + to_string((long long)binned_table) + "," + to_string((long long)binned_total);
     for (size_t i = 0; i < parts.size(); ++i) {
         s += "|P{" + parts[i].key() + "}";

@@ -104,6 +104,13 @@ struct FusedKernel {
         // and the outputs are {data gradient, partials [chunks, g, fh*fw*c, k], (column sums [chunks, g*k])}.
         bool wgrad = false, bias = false;
         int64_t chunks = 0;
+        // The filter gradient alone (a first layer, whose input needs no gradient): `main` is then the filter
+        // gradient's own MatMul, im2col^T [g][(fy, fx, c)][(img, oy, ox)] x dC [g][(img, oy, ox)][oc]; inputs[1] is dC
+        // (a buffer or a fused producer), inputs[0] and inputs[2] the image, outputs {partials, (column sums)}.
+        bool wgrad_only = false;
+        // (filter gradient alone) bands of output rows an image is cut into, one workgroup each: a band's tiles are a
+        // fraction of the image's, so more workgroups share a CU; partials then number chunks x bands
+        int64_t bands = 1;
     } dgrad;
     // MatMul whose A operand is the im2col of a stride-1 convolution's (replicate-padded) input: the kernel reads the
     // image [img, h, w, g*c] itself, one workgroup per (image, group) with the group's channels of the image in LDS,

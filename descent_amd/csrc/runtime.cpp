@@ -440,7 +440,7 @@ Kernel* get_kernel(Context* ctx, const FusedKernel& fk, int* status) {
     if (fk.dgrad.on) {
         const auto& c = fk.dgrad;
         char text[160];
-        std::snprintf(text, sizeof text, "%s [%lld, %lld, %lld, %lld] %lldx%lld taps, %lld groups", c.wgrad ? "ConvBackward" : "ConvDataGrad", (long long)c.img,
+        std::snprintf(text, sizeof text, "%s [%lld, %lld, %lld, %lld] %lldx%lld taps, %lld groups", c.wgrad_only ? "ConvFilterGrad" : c.wgrad ? "ConvBackward" : "ConvDataGrad", (long long)c.img,
                       (long long)(c.oh + c.fh - 1 - 2 * c.pad_h), (long long)(c.ow + c.fw - 1 - 2 * c.pad_w), (long long)(c.g * c.c),
                       (long long)c.fh, (long long)c.fw, (long long)c.g);
         k->label = text;
@@ -457,7 +457,7 @@ Kernel* get_kernel(Context* ctx, const FusedKernel& fk, int* status) {
     if (!fk.parts.empty()) {
         k->label = "Multi (" + std::to_string(fk.parts.size()) + " kernels:";
         for (auto& part : fk.parts)
-            k->label += " " + std::string(part.dgrad.on ? (part.dgrad.wgrad ? "ConvBackward" : "ConvDataGrad") : part.cfwd.on ? "ConvForward" : part.row_stages.empty() ? label_name(part.main.raw()) : "RowFused") + ";";
+            k->label += " " + std::string(part.dgrad.on ? (part.dgrad.wgrad_only ? "ConvFilterGrad" : part.dgrad.wgrad ? "ConvBackward" : "ConvDataGrad") : part.cfwd.on ? "ConvForward" : part.row_stages.empty() ? label_name(part.main.raw()) : "RowFused") + ";";
         k->label += ")";
     }
     k->reference_groups = reference_group_count(fk.main.raw());

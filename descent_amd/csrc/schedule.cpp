@@ -1162,6 +1162,128 @@ struct Planner {
         }
     }
 
+    // The filter gradient of a convolution whose input needs no gradient (a first layer): the tall-k MatMul
+    // im2col^T x dC becomes the convolution backward kernel without its data-gradient phase.  dC may later become a
+    // fused producer (pass 2): with no data gradient to compute from it, nothing else needs it in memory.
+    void filter_gradient_alone(const ConvSite& site) {
+        static const bool enabled = !(std::getenv("DSC_FUSE_CONV_WGRAD") && std::getenv("DSC_FUSE_CONV_WGRAD")[0] == '0');
+        if (!enabled) return;
+        const FusedKernel::ConvFwd& f = site.geo;
+        int ti = -1;
+        for (int q = 0; q < (int)drafts.size() && ti < 0; ++q) {
+            const Draft& T = drafts[q];
+            const dsc_kernel_desc& td = T.fk.main.raw();
+            if (!T.alive || td.kind != DSC_KERNEL_MATMUL || !T.keep_split || !T.fk.virtuals.empty() || T.fk.has_epilogue ||
+                td.output_mode != DSC_MATMUL_BATCHES || T.fk.dgrad.on || T.fk.cfwd.on || T.fk.inputs[0].buffer < 0 || T.fk.inputs[1].buffer < 0)
+                continue;
+            if (T.params[T.fk.inputs[0].buffer] != site.a_node) continue;
+            const MatMulDims gt = matmul_dims(td);
+            if (gt.batch != f.g || gt.m != f.fh * f.fw * f.c || gt.k != f.img * f.oh * f.ow || gt.n > 16 || gt.n % 4 != 0) continue;
+            // its A is the forward's A transposed; its B is read as [g][(img, oy, ox)][oc] with nothing clamped
+            int64_t bt, bf, ct[DSC_MAX_DIM], cf[DSC_MAX_DIM];
+            if (!affine_form(td.inputs[0], &bt, ct) || !affine_form(site.a_view, &bf, cf) || bt != bf || ct[1] != cf[2] || ct[2] != cf[1] ||
+                (gt.batch > 1 && ct[0] != cf[0]))
+                continue;
+            if (any_clamp(td.inputs[1])) continue;
+            ti = q;
+        }
+        if (ti < 0) return;
+        Draft& T = drafts[ti];
+        const MatMulDims gt = matmul_dims(T.fk.main.raw());
+        const bool bias = T.fk.colsum_out >= 0;
+        if ((int)T.outs.size() != (bias ? 2 : 1) || T.outs[0].copy_from >= 0 || is_graph_output[T.outs[0].node]) return;
+        auto only_reduce_of = [&](int node) {
+            auto cons = consumers_of(node);
+            if (cons.size() != 1 || cons[0] <= ti) return -1;
+            const Draft& r = drafts[cons[0]];
+            const dsc_kernel_desc& rd = r.fk.main.raw();
+            if (rd.kind != DSC_KERNEL_REDUCE || rd.reduce_op != DSC_REDUCE_SUM || !r.fk.virtuals.empty() || r.fk.has_epilogue) return -1;
+            return cons[0];
+        };
+        const int r1 = only_reduce_of(T.outs[0].node);
+        if (r1 < 0) return;
+        {
+            const dsc_kernel_desc& rd = drafts[r1].fk.main.raw();
+            if (rd.axis != 0 || !is_identity(rd.inputs[0]) || rd.inputs[0].in_shape.dims[0] != gt.chunks ||
+                element_count(rd.inputs[0].in_shape) != gt.chunks * gt.batch * gt.m * gt.n)
+                return;
+        }
+        int r2 = -1;
+        if (bias) {
+            if (is_graph_output[T.outs[1].node]) return;
+            r2 = only_reduce_of(T.outs[1].node);
+            if (r2 < 0) return;
+            const dsc_kernel_desc& rd = drafts[r2].fk.main.raw();
+            const dsc_view& pv = rd.inputs[0];
+            if (pv.in_shape.rank != 2 || pv.in_shape.dims[0] != gt.chunks || pv.in_shape.dims[1] != gt.batch * gt.n ||
+                pv.out_shape.dims[rd.axis] != gt.chunks || (gt.chunks > 1 && pv.map_axis[rd.axis] != 0))
+                return;
+        }
+        // the image must still be what the forward convolution read
+        {
+            bool image_ok = true;
+            for (int q = 0; q <= ti && image_ok; ++q) {
+                if (!drafts[q].alive) continue;
+                for (auto& o : drafts[q].outs)
+                    if (o.copy_from == site.image_node) image_ok = false;
+            }
+            if (!image_ok) return;
+        }
+        // bands of at least four output rows: the tiles of a band are small enough for eight workgroups to share a CU,
+        // which is what hides each workgroup's fill -> barrier -> products -> reduction chain
+        const int64_t bands = (f.oh % 4 == 0 && f.oh >= 16) ? 4 : (f.oh % 2 == 0 && f.oh >= 8) ? 2 : 1;
+        // image sets: about a thousand workgroups, a multiple of eight sets (measured on the ConvNet's first
+        // convolution together with the Reduce over the partials that follows: 4096 workgroups 5354 steps/s, 2048
+        // 5350, 1024 5379, 512 clearly slower)
+        const int64_t per_group = std::max<int64_t>(8, 1024 / (f.g * bands));
+        const int64_t images_per_set = (f.img + per_group - 1) / per_group;
+        const int64_t sets = ((f.img + images_per_set - 1) / images_per_set + 7) / 8 * 8;
+        Draft fused = T;
+        fused.keep_split = false;
+        FusedKernel::ConvDgrad& cv = fused.fk.dgrad;
+        cv.on = true;
+        cv.img = f.img; cv.oh = f.oh; cv.ow = f.ow; cv.g = f.g; cv.fh = f.fh; cv.fw = f.fw; cv.c = f.c;
+        cv.pad_h = f.pad_h; cv.pad_w = f.pad_w;
+        cv.wgrad = true;
+        cv.wgrad_only = true;
+        cv.bias = bias;
+        cv.chunks = sets;
+        cv.bands = bands;
+        const int64_t partials = sets * cv.bands;
+        fused.fk.colsum_out = -1;
+        fused.fk.outputs.clear();
+        for (auto& o : T.outs) fused.fk.outputs.push_back(param_index(fused, o.node, true));
+        {
+            Source xs;
+            xs.buffer = param_index(fused, site.image_node, false);
+            fused.fk.inputs[0] = xs;  // the im2col operand of the MatMul is read from the image itself
+            fused.fk.inputs.push_back(xs);
+        }
+        compact(fused);
+        if (!conv_bwd_fits(fused.fk.dgrad, gt.n)) return;
+        {
+            Generated probe;
+            if (!generate(fused.fk, &probe).empty()) return;
+        }
+        node_bytes[T.outs[0].node] = (size_t)(partials * gt.batch * gt.m * gt.n) * 4;
+        drafts[r1].fk.main.inputs[0].in_shape.dims[0] = partials;
+        drafts[r1].fk.main.inputs[0].out_shape.dims[0] = partials;
+        if (bias) {
+            node_bytes[T.outs[1].node] = (size_t)(partials * gt.batch * gt.n) * 4;
+            const int axis = drafts[r2].fk.main.raw().axis;
+            dsc_view& pv = drafts[r2].fk.main.inputs[0];
+            pv.in_shape.dims[0] = partials;
+            pv.out_shape.dims[axis] = partials;
+            pv.map_axis[axis] = 0;
+            pv.map_step[axis] = 1;
+        }
+        drafts[ti] = fused;
+        if (drafts[site.copy_idx].alive && consumers_of(site.a_node).empty()) {
+            drafts[ti].covers.insert(drafts[ti].covers.end(), drafts[site.copy_idx].covers.begin(), drafts[site.copy_idx].covers.end());
+            drafts[site.copy_idx].alive = false;
+        }
+    }
+
     // Pass 1e: both gradients of a convolution in one kernel.  The data-gradient kernel (pass 1c) holds dC of an
     // image in LDS; the filter gradient im2col^T x dC of the same convolution -- by now a MatMul whose k (images x
     // output pixels) pass 0 split into many chunks, summed by a Reduce, possibly with the bias gradient's column
@@ -1182,7 +1304,10 @@ struct Planner {
                     cv.pad_h == f.pad_h && cv.pad_w == f.pad_w)
                     di = q;
             }
-            if (di < 0) continue;
+            if (di < 0) {
+                filter_gradient_alone(site);
+                continue;
+            }
             const MatMulDims gd = matmul_dims(drafts[di].fk.main.raw());  // [g][(img, oy, ox)][oc] x [g][oc][(fy, fx, c)]
             const int dc_node = drafts[di].params[drafts[di].fk.inputs[0].buffer];
             int ti = -1;
@@ -1288,6 +1413,58 @@ struct Planner {
                 drafts[at].covers.insert(drafts[at].covers.end(), drafts[site.copy_idx].covers.begin(), drafts[site.copy_idx].covers.end());
                 drafts[site.copy_idx].alive = false;
             }
+        }
+    }
+
+    // Pass 1g: a WindowsToImage whose windows neither overlap nor leave gaps (the backward of a pooling: stride =
+    // window size) adds nothing up -- every image element is one window element.  It becomes a per-element copy
+    // through the window view with its axes reordered: [.., oy, ox, g, fy, fx, c] read as [.., oy, fy, ox, fx, g, c],
+    // whose row-major order is the image's.  Pass 2 then evaluates the copy inside whoever reads the image.
+    void disjoint_windows_to_copies() {
+        static const bool enabled = !(std::getenv("DSC_WINDOW_COPIES") && std::getenv("DSC_WINDOW_COPIES")[0] == '0');
+        if (!enabled) return;
+        for (auto& D : drafts) {
+            const dsc_kernel_desc& d = D.fk.main.raw();
+            if (!D.alive || d.kind != DSC_KERNEL_WINDOWS_TO_IMAGE || !D.fk.virtuals.empty() || D.fk.has_epilogue || !D.fk.parts.empty() ||
+                D.outs.size() != 1 || D.outs[0].copy_from >= 0 || D.fk.inputs.size() != 1)
+                continue;
+            const dsc_view& v = d.inputs[0];
+            const int r = v.out_shape.rank, bd = d.shape.rank - 3;
+            if (r < 6 || bd != r - 6) continue;
+            const int64_t oh = v.out_shape.dims[r - 6], ow = v.out_shape.dims[r - 5], fh = v.out_shape.dims[r - 3], fw = v.out_shape.dims[r - 2];
+            if (d.stride_h != fh || d.stride_w != fw || d.shape.dims[bd] != oh * fh || d.shape.dims[bd + 1] != ow * fw) continue;
+            // output axis -> window-view axis
+            int from[DSC_MAX_DIM];
+            for (int i = 0; i < bd; ++i) from[i] = i;
+            from[bd + 0] = bd + 0;  // oy
+            from[bd + 1] = bd + 3;  // fy
+            from[bd + 2] = bd + 1;  // ox
+            from[bd + 3] = bd + 4;  // fx
+            from[bd + 4] = bd + 2;  // g
+            from[bd + 5] = bd + 5;  // c
+            dsc_view nv = v;
+            dsc_kernel_desc nd{};
+            nd.kind = DSC_KERNEL_PER_ELEMENT;
+            nd.shape.rank = 1;  // a per-element kernel is described over its linear element count
+            nd.shape.dims[0] = element_count(d.shape);
+            for (int j = 0; j < r; ++j) {
+                nv.out_shape.dims[j] = v.out_shape.dims[from[j]];
+                nv.map_axis[j] = v.map_axis[from[j]];
+                nv.map_step[j] = v.map_step[from[j]];
+            }
+            dsc_pe_op ops[2] = {pe_op(DSC_PE_LOAD), pe_op(DSC_PE_UNARY, DSC_UN_MOV, 0)};
+            ops[0].input_index = 0;
+            int32_t outputs[1] = {1};
+            nd.n_inputs = 1;
+            nd.inputs = &nv;
+            nd.n_ops = 2;
+            nd.ops = ops;
+            nd.n_outputs = 1;
+            nd.outputs = outputs;
+            if (!validate(nd).empty()) continue;
+            FusedKernel fk = FusedKernel::plain(nd);
+            if (fk.n_buffers != (int)D.params.size()) continue;
+            D.fk = fk;
         }
     }
 
@@ -1475,6 +1652,8 @@ struct Planner {
                     if (q.fk.colsum_out >= 0 && q.fk.inputs[1].buffer >= 0 && q.params[q.fk.inputs[1].buffer] == node) ok = false;
                     // the kernel that takes both gradients of a convolution requests dC of its next image while it
                     // works on the current one: plain loads, nothing evaluated in between
+                    // (the filter gradient alone has one round trip per image anyway and takes dC as a producer; its
+                    // image has to be a buffer)
                     if (q.fk.dgrad.on && q.fk.dgrad.wgrad && q.fk.inputs[0].buffer >= 0 && q.params[q.fk.inputs[0].buffer] == node) ok = false;
                     // an epilogue reads its product from the accumulator, never through a producer
                     if (q.fk.has_epilogue && q.fk.epilogue_product_input >= 0) {
@@ -2072,6 +2251,7 @@ struct Planner {
         conv_data_gradient();                   // pass 1c
         conv_forward();                         // pass 1d
         conv_backward();                        // pass 1e
+        disjoint_windows_to_copies();           // pass 1g
         row_kernels();                          // pass 1b
         inline_producers();                     // pass 2
         attach_epilogues();                     // pass 3

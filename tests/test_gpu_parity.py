@@ -483,6 +483,59 @@ def test_conv2d_gradients_over_geometries(hip_backend_session, geom, fused):
     assert rel_l2(gdf, cdf) <= TOL, (rel_l2(gdf, cdf), listing)
 
 
+def _first_layer_case(env, m, h, w, c_in, c_out, fh, fw, pad, pool, seed):
+    """data -> conv2d + bias -> leaky_relu (-> 2x2 max-pool) -> 0.5 * sum(y^2), the data a plain parameter: only the
+    filter and the bias have gradients, as for the first layer of a network."""
+    from descent_amd import Initializer
+
+    rng = np.random.default_rng(seed)
+    xp = env.static_parameter_with_data([m, h, w, c_in], "x", rng.standard_normal((m, h, w, c_in), dtype=np.float32))
+    fp = env.trainable_parameter([1, c_out, fh, fw, c_in], "f", Initializer.zero())
+    bp = env.trainable_parameter([c_out], "b", Initializer.zero())
+    env.write_parameter(fp, rng.standard_normal((1, c_out, fh, fw, c_in), dtype=np.float32) * 0.3)
+    env.write_parameter(bp, rng.standard_normal(c_out, dtype=np.float32) * 0.1)
+    df, db = env.static_parameter(list(fp.shape), "df"), env.static_parameter([c_out], "db")
+
+    def build(s):
+        f, b = s.parameter(fp), s.parameter(bp)
+        y = (s.parameter(xp).conv2d(f, pad) + b).leaky_relu(0.01)
+        if pool:
+            y = y.max_pool2d((2, 2), (2, 2))
+        (y.square() * 0.5).set_loss()
+        s.write_parameter_value(df, f.loss_grad())
+        s.write_parameter_value(db, b.loss_grad())
+
+    g = env.build_graph(build)
+    env.run(g, 0)
+    return g, env.read_parameter(df), env.read_parameter(db)
+
+
+@pytest.mark.parametrize("geom", [
+    # m, h, w, c_in, c_out, fh, fw, pad, pool
+    (600, 28, 28, 1, 16, 3, 3, 1, True),    # the ConvNet's first layer: four bands of seven rows
+    (500, 20, 12, 1, 8, 3, 3, 1, True),     # not square, eight outputs
+    (700, 10, 10, 3, 16, 3, 3, 1, True),    # three channels, two bands of five rows
+    (900, 9, 9, 2, 12, 5, 5, 2, False),     # one band, 5x5 taps, no pooling: dC comes from the activation derivative alone
+    (800, 16, 16, 4, 16, 3, 3, 0, True),    # no padding: 14 output rows, two bands
+], ids=lambda g: "x".join(map(str, g)))
+@pytest.mark.parametrize("fused", [True, "split-conv-grads"])
+def test_first_layer_filter_gradient(hip_backend_session, geom, fused):
+    genv, cenv = _envs(hip_backend_session, fused=fused)
+    g, gdf, gdb = _first_layer_case(genv, *geom, seed=77)
+    _, cdf, cdb = _first_layer_case(cenv, *geom, seed=77)
+    listing = next(iter(g.__dict__["_schedules"].values())).describe()
+    if fused is True:
+        # the filter gradient (k = images x output pixels, long enough to be split) on the convolution backward kernel
+        # without its data-gradient phase, dC evaluated where the kernel fills its tile
+        assert "ConvFilterGrad" in listing and "no data gradient" in listing, listing
+        if geom[-1]:
+            assert "WindowsToImage" not in listing, listing
+    else:
+        assert "ConvFilterGrad" not in listing, listing
+    assert rel_l2(gdf, cdf) <= TOL, (rel_l2(gdf, cdf), listing)
+    assert rel_l2(gdb, cdb) <= TOL, (rel_l2(gdb, cdb), listing)
+
+
 def _random_conv_geometry(rng):
     while True:
         groups = int(rng.choice([1, 1, 2, 3, 4]))

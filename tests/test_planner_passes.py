@@ -81,10 +81,30 @@ def test_matmul_takes_its_per_element_consumer_as_epilogue():
 
 
 def test_bias_gradient_rides_on_the_weight_gradient_that_reads_the_same_array():
-    listing = hip_backend.check_schedule(workloads.convnet(_env(), batch=1000).graph, fused=True)
+    graph = workloads.convnet(_env(), batch=1000).graph
+    listing = hip_backend.check_schedule(graph, fused="split-conv-grads")
     # conv1: filter gradient im2col^T x dC with the column sums of dC (the bias gradient) from the same pass
     assert re.search(r"MatMul \(k=784000\) \[\d+, 1, 9, 16\] <1 fused producers>  \[tall-k mfma 16x16x4.*\+column sums of B\]", listing)
     assert re.search(r"Reduce \(k=\d+\) \[1, 1, 1, 16\]; Reduce \(k=\d+\) \[1, 1, 9, 16\]", listing)
+
+
+def test_first_layer_filter_gradient_takes_the_pooling_gradient_as_a_producer():
+    graph = workloads.convnet(_env(), batch=1000).graph
+    listing = hip_backend.check_schedule(graph, fused=True)
+    assert int(listing.split()[0]) == 12
+    # conv1 needs no data gradient: its filter gradient (and the bias gradient's column sums) run on the convolution
+    # backward kernel, bands of 7 output rows; dC is never written -- the max-pool gradient (a WindowsToImage over
+    # 2x2 windows that do not overlap, turned into a copy), the selects around it and the activation derivative are
+    # evaluated where the kernel fills its dC tile
+    line = next(l for l in listing.splitlines() if "ConvFilterGrad" in l)
+    assert "no data gradient, 4 bands of 7 output rows, filter gradient mfma 16x16x4 1x1 tiles +column sums of dC" in line, line
+    for cluster in (44, 45, 46, 50):  # select_eq, WindowsToImage, leaky', the filter gradient's MatMul
+        assert str(cluster) in line.split(" clusters ")[1].split(), (cluster, line)
+    assert "WindowsToImage" not in listing
+    assert re.search(r"Reduce \(k=1024\) \[1, 1, 1, 16\]; Reduce \(k=1024\) \[1, 1, 9, 16\]", listing)
+    # with the switch the second convolution keeps its own two kernels and the first its tall-k product
+    split = hip_backend.check_schedule(graph, fused="split-conv-grads")
+    assert "ConvFilterGrad" not in split and "ConvBackward" not in split
 
 
 def test_scatter_adds_into_one_accumulator_share_a_launch_and_small_launches_are_grouped():
