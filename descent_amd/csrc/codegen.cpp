@@ -1293,18 +1293,26 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     int64_t dc_base = 0, dc_coef[DSC_MAX_DIM] = {0};
     const bool vec_dc = fk.inputs[DC].buffer >= 0 && K % 4 == 0 && affine_form(d.inputs[DC], &dc_base, dc_coef) && dc_coef[2] == 1 && dc_base % 4 == 0 &&
                         dc_coef[1] % 4 == 0 && (G == 1 || dc_coef[0] % 4 == 0);
-    const int64_t dunit = vec_dc ? 4 : 1;
+    // Four consecutive output channels of a pixel per thread also when dC is a fused producer: the producers' index
+    // arithmetic (divisions by the extents of every view on the way) is then shared by the four evaluations, whose
+    // element ids differ in their two lowest bits only.
+    const bool quad_dc = K % 4 == 0;
+    const int64_t dunit = quad_dc ? 4 : 1;
     const int64_t fill_n = OH * OW * K / dunit, NC = (fill_n + 255) / 256;
     const bool vec_fill = C % 4 == 0;
     const int64_t unit = vec_fill ? 4 : 1, xn = PH * PW * C / unit, NX = (xn + 255) / 256;
-    const string vt = vec_fill ? "float4" : "float", dvt = vec_dc ? "float4" : "float";
+    const string vt = vec_fill ? "float4" : "float", dvt = quad_dc ? "float4" : "float";
     auto emit_issue = [&](const string& img, const string& ind) {
         k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NC) << "; ++u) {\n";
         k << ind << "    const int i = min((int)threadIdx.x + u * 256, " << S(fill_n - 1) << ") * " << S(dunit) << ";\n";
         if (vec_dc)
             k << ind << "    pv[u] = *(const float4*)(b" << fk.inputs[DC].buffer << " + " << S(dc_base) << " + cb * " << S(G == 1 ? 0 : dc_coef[0]) << " + (" << img << " * "
               << S(OHF * OW) << " + band * " << S(OH * OW) << " + i / " << S(K) << ") * " << S(dc_coef[1]) << " + i % " << S(K) << ");\n" << ind << "}\n";
-        else
+        else if (quad_dc) {
+            k << ind << "    const int pix = " << img << " * " << S(OHF * OW) << " + band * " << S(OH * OW) << " + i / " << S(K) << ", oc = i % " << S(K) << ";\n";
+            k << ind << "    pv[u] = make_float4(load_a(cb, pix, oc, " << em.params_pass() << "), load_a(cb, pix, oc + 1, " << em.params_pass() << "), load_a(cb, pix, oc + 2, "
+              << em.params_pass() << "), load_a(cb, pix, oc + 3, " << em.params_pass() << "));\n" << ind << "}\n";
+        } else
             k << ind << "    pv[u] = load_a(cb, " << img << " * " << S(OHF * OW) << " + band * " << S(OH * OW) << " + i / " << S(K) << ", i % " << S(K) << ", " << em.params_pass() << ");\n" << ind << "}\n";
         k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NX) << "; ++u) {\n";
         k << ind << "    const int e = min((int)threadIdx.x + u * 256, " << S(xn - 1) << ") * " << S(unit) << ";\n";
@@ -1318,9 +1326,9 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NC) << "; ++u) {\n";
         k << ind << "    const int i = ((int)threadIdx.x + u * 256) * " << S(dunit) << ", pi = i / " << S(K) << ";\n";
         k << ind << "    float* const at = lds + ((pi / " << S(OW) << ") * " << S(PW) << " + pi % " << S(OW) << ") * " << S(PITCH) << " + i % " << S(K) << ";\n";
-        if (vec_dc && PITCH % 4 == 0)
+        if (quad_dc && PITCH % 4 == 0)
             k << ind << "    if ((int)threadIdx.x + u * 256 < " << S(fill_n) << ") *(float4*)at = pv[u];\n" << ind << "}\n";
-        else if (vec_dc)
+        else if (quad_dc)
             k << ind << "    if ((int)threadIdx.x + u * 256 < " << S(fill_n) << ") { at[0] = pv[u].x; at[1] = pv[u].y; at[2] = pv[u].z; at[3] = pv[u].w; }\n" << ind << "}\n";
         else
             k << ind << "    if ((int)threadIdx.x + u * 256 < " << S(fill_n) << ") at[0] = pv[u];\n" << ind << "}\n";
