@@ -446,6 +446,97 @@ struct Planner {
             return loads == 1;
     }
 
+    // Pass 00: the sign of a pre-activation read off the activation.  A cluster that stores both z and
+    // a = (z > 0) ? z : z * c with a literal c > 0 (a leaky ReLU beside its input, kept for the backward pass) and whose
+    // z is read elsewhere only as the left side of "(z > 0) ? .. : .." selects: a > 0 exactly when z > 0 (z * c is
+    // negative, a negative zero or a NaN whenever z is not positive), so those readers take a instead and z is not
+    // stored.  One array less written by the forward kernel and one less read by the backward one, bit for bit the same
+    // results.
+    void sign_through_activation() {
+        static const bool enabled = !(std::getenv("DSC_SIGN_THROUGH_ACTIVATION") && std::getenv("DSC_SIGN_THROUGH_ACTIVATION")[0] == '0');
+        if (!enabled) return;
+        auto is_zero = [](const dsc_pe_op& o) { return o.kind == DSC_PE_LITERAL_F32 && (o.bits & 0x7fffffffu) == 0; };
+        auto plain_pe = [](const Draft& d) {
+            return d.alive && d.fk.main.raw().kind == DSC_KERNEL_PER_ELEMENT && d.fk.virtuals.empty() && !d.fk.has_epilogue && d.fk.parts.empty() &&
+                   d.fk.row_stages.empty() && (int)d.fk.inputs.size() == d.fk.main.raw().n_inputs;
+        };
+        for (int pi = 0; pi < (int)drafts.size(); ++pi) {
+            if (!plain_pe(drafts[pi]) || drafts[pi].fk.main.raw().n_outputs < 2) continue;
+            const dsc_kernel_desc& pd = drafts[pi].fk.main.raw();
+            int oz = -1, oa = -1;  // which outputs are z and a
+            for (int i = 0; i < pd.n_outputs && oz < 0; ++i)
+                for (int j = 0; j < pd.n_outputs && oz < 0; ++j) {
+                    if (i == j) continue;
+                    const int z = pd.outputs[i];
+                    const dsc_pe_op& sel = pd.ops[pd.outputs[j]];
+                    if (sel.kind != DSC_PE_SELECT || sel.op != DSC_CMP_GT || sel.args[0] != z || sel.args[2] != z || !is_zero(pd.ops[sel.args[1]])) continue;
+                    const dsc_pe_op& mul = pd.ops[sel.args[3]];
+                    if (mul.kind != DSC_PE_BINARY || mul.op != DSC_BIN_MUL) continue;
+                    const int c = mul.args[0] == z ? mul.args[1] : mul.args[1] == z ? mul.args[0] : -1;
+                    if (c < 0 || pd.ops[c].kind != DSC_PE_LITERAL_F32) continue;
+                    float cv;
+                    std::memcpy(&cv, &pd.ops[c].bits, 4);
+                    if (!(cv > 0.f) || !(cv < 3.0e38f)) continue;
+                    oz = i;
+                    oa = j;
+                }
+            if (oz < 0) continue;
+            const int z_node = drafts[pi].outs[oz].node, a_node = drafts[pi].outs[oa].node;
+            if (is_graph_output[z_node] || drafts[pi].outs[oz].copy_from >= 0 || node_bytes[z_node] != node_bytes[a_node]) continue;
+            // every reader of z: a plain per-element cluster that uses it only as the left side of (z > 0) selects
+            bool ok = true;
+            std::vector<std::pair<int, int>> uses;  // (draft, pointer parameter)
+            for (int qi = 0; qi < (int)drafts.size() && ok; ++qi) {
+                Draft& Q = drafts[qi];
+                if (!Q.alive || qi == pi) continue;
+                for (auto& o : Q.outs)
+                    if (o.copy_from == z_node) ok = false;
+                for (size_t b = 0; b < Q.params.size() && ok; ++b) {
+                    if (Q.params[b] != z_node || Q.fk.buffer_is_output[b]) continue;
+                    if (!plain_pe(Q) || qi < pi) { ok = false; break; }
+                    const dsc_kernel_desc& qd = Q.fk.main.raw();
+                    for (int in = 0; in < qd.n_inputs && ok; ++in) {
+                        if (Q.fk.inputs[in].buffer != (int)b) continue;
+                        for (int l = 0; l < qd.n_ops && ok; ++l) {
+                            const dsc_pe_op& lo = qd.ops[l];
+                            if (lo.kind == DSC_PE_GATHER && lo.input_index == in) ok = false;
+                            if (lo.kind != DSC_PE_LOAD || lo.input_index != in) continue;
+                            for (int o = 0; o < qd.n_outputs; ++o)
+                                if (qd.outputs[o] == l) ok = false;
+                            for (int u = 0; u < qd.n_ops && ok; ++u) {
+                                const dsc_pe_op& uo = qd.ops[u];
+                                const int nargs = uo.kind == DSC_PE_UNARY || uo.kind == DSC_PE_GATHER ? 1 : uo.kind == DSC_PE_BINARY ? 2 : uo.kind == DSC_PE_SELECT ? 4 : 0;
+                                for (int a = 0; a < nargs; ++a) {
+                                    if (uo.args[a] != l) continue;
+                                    if (!(uo.kind == DSC_PE_SELECT && uo.op == DSC_CMP_GT && a == 0 && is_zero(qd.ops[uo.args[1]]))) ok = false;
+                                }
+                            }
+                        }
+                    }
+                    uses.emplace_back(qi, (int)b);
+                }
+            }
+            if (!ok || uses.empty()) continue;
+            for (auto& u : uses) drafts[u.first].params[u.second] = a_node;
+            // z is no output any more
+            dsc_kernel_desc trimmed = pd;
+            std::vector<int32_t> kept(pd.outputs, pd.outputs + pd.n_outputs);
+            kept.erase(kept.begin() + oz);
+            trimmed.outputs = kept.data();
+            trimmed.n_outputs = (int32_t)kept.size();
+            KernelDesc fixed(trimmed);
+            if (!validate(fixed.raw()).empty()) {
+                for (auto& u : uses) drafts[u.first].params[u.second] = z_node;
+                continue;
+            }
+            Draft& P = drafts[pi];
+            const int n_in = fixed.raw().n_inputs;
+            P.params.erase(P.params.begin() + n_in + oz);
+            P.outs.erase(P.outs.begin() + oz);
+            P.fk = FusedKernel::plain(fixed.raw());
+        }
+    }
+
     // Pass 0: a MatMul whose output is small but whose k is long gets its k range split over many more
     // workgroups than the reference's ceil(K/1024) chunks; the partial products go to an internal buffer and
     // are summed by a Reduce (which pass 2 then inlines into the consumer when the split is small).
@@ -2243,6 +2334,7 @@ struct Planner {
 
     // The order matters: each pass names the ones it relies on.
     void run() {
+        sign_through_activation();              // pass 00
         split_long_k();                         // pass 0
         bias_sums_ride_on_weight_gradients();   // pass 0c
         merge_reduce_chains();                  // pass 0a

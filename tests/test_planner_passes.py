@@ -155,3 +155,23 @@ def test_chain_switches_fall_back_to_one_launch_per_chain():
     assert "chains in one launch" not in listing and "stage 1 of 2" not in listing and "column slices" not in listing
     assert listing.count("kept in LDS per workgroup") == 6      # accumulators of up to 18432 floats
     assert listing.count("scatter_add: global_atomic_add_f32 | scatter_add: global_atomic_add_f32") >= 10
+
+
+def test_the_sign_of_a_pre_activation_is_read_off_the_stored_activation():
+    graph = workloads.convnet(_env(), batch=1000).graph
+    fused = hip_backend.check_schedule(graph, fused=True)
+    lines = [l for l in fused.splitlines() if re.match(r"\d+: ", l)]
+
+    def moved(line):
+        return float(re.search(r"grid \S+ ([0-9.]+) MB", line).group(1))
+
+    # The reference's convolution clusters store z = conv + bias beside a = leaky_relu(z), and the backward pass reads
+    # z again for "(z > 0) ? g : 0.01 g".  a has the sign of z, so the readers test a > 0 and z is never written:
+    # conv1's kernel writes a (50.2 MB) and the pooled a (12.5 MB) for its 3.1 MB image, conv2's a (25.1), the pooled
+    # and dropped-out a (2 x 6.3) for 12.5 MB in
+    assert "ConvForward" in lines[0] and 65.0 < moved(lines[0]) < 66.5, lines[0]     # 116.0 with z stored
+    assert lines[1].split(": ")[1].startswith("ConvForward") and 49.5 < moved(lines[1]) < 51.0, lines[1]  # 75.3 with z stored
+    assert "414." in fused.splitlines()[-1], fused.splitlines()[-1]                  # MB per step; 565 with z stored
+    # cluster by cluster nothing is rewritten
+    unfused = hip_backend.check_schedule(graph, fused=False)
+    assert "PerElement (7 ops) [12544000]" in unfused and "2316." in unfused.splitlines()[-1], unfused.splitlines()[-1]
