@@ -333,7 +333,12 @@ typedef struct dsc_schedule dsc_schedule;
 #define DSC_SCHEDULE_NO_FUSION 1u /* launch exactly one kernel per reference cluster (for parity tests) */
 #define DSC_SCHEDULE_GRAPH_REPLAY 4u /* capture each run's launches as a HIP graph and replay it whenever a later run's
                                         buffers land on the same addresses (the Submit half of the reference's
-                                        command buffer, device/command_buffer.rs:64-123, recorded once) */
+                                        command buffer, device/command_buffer.rs:64-123, recorded once).  For the
+                                        addresses to repeat, such a schedule keeps its intermediates in one region
+                                        of its own and holds one spare buffer per written parameter slot: a run
+                                        returns the spare as the slot's new buffer and keeps the old one as the
+                                        next spare (the region and the spares go back to the heap in
+                                        dsc_schedule_destroy) */
 #define DSC_SCHEDULE_NO_CONV_KERNELS 2u /* keep convolutions (forward and data gradient) on the generic MatMul path
                                            (fused producers) instead of the dedicated LDS-tiled kernels (for
                                            parity tests) */
