@@ -447,7 +447,7 @@ struct Planner {
     }
 
     // Pass 00: the sign of a pre-activation read off the activation.  A cluster that stores both z and
-    // a = (z > 0) ? z : z * c with a literal c > 0 (a leaky ReLU beside its input, kept for the backward pass) and whose
+    // a = (z > 0) ? z : z * c with a literal c >= 0, or : 0 (a leaky or plain ReLU beside its input, kept for the backward pass) and whose
     // z is read elsewhere only as the left side of "(z > 0) ? .. : .." selects: a > 0 exactly when z > 0 (z * c is
     // negative, a negative zero or a NaN whenever z is not positive), so those readers take a instead and z is not
     // stored.  One array less written by the forward kernel and one less read by the backward one, bit for bit the same
@@ -471,12 +471,14 @@ struct Planner {
                     const dsc_pe_op& sel = pd.ops[pd.outputs[j]];
                     if (sel.kind != DSC_PE_SELECT || sel.op != DSC_CMP_GT || sel.args[0] != z || sel.args[2] != z || !is_zero(pd.ops[sel.args[1]])) continue;
                     const dsc_pe_op& mul = pd.ops[sel.args[3]];
-                    if (mul.kind != DSC_PE_BINARY || mul.op != DSC_BIN_MUL) continue;
-                    const int c = mul.args[0] == z ? mul.args[1] : mul.args[1] == z ? mul.args[0] : -1;
-                    if (c < 0 || pd.ops[c].kind != DSC_PE_LITERAL_F32) continue;
-                    float cv;
-                    std::memcpy(&cv, &pd.ops[c].bits, 4);
-                    if (!(cv > 0.f) || !(cv < 3.0e38f)) continue;
+                    if (!is_zero(mul)) {  // a plain ReLU stores zero there; a leaky one z times a positive literal
+                        if (mul.kind != DSC_PE_BINARY || mul.op != DSC_BIN_MUL) continue;
+                        const int c = mul.args[0] == z ? mul.args[1] : mul.args[1] == z ? mul.args[0] : -1;
+                        if (c < 0 || pd.ops[c].kind != DSC_PE_LITERAL_F32) continue;
+                        float cv;
+                        std::memcpy(&cv, &pd.ops[c].bits, 4);
+                        if (!(cv >= 0.f) || !(cv < 3.0e38f)) continue;  // (z * 0 is a zero or a NaN: not positive either)
+                    }
                     oz = i;
                     oa = j;
                 }

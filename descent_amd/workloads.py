@@ -183,8 +183,9 @@ def positional_encoding(x, freq_count: int):
 class ReluMlp(Module):
     """examples/image_fit/main.rs:52-87 (`Relu`; its activation is leaky_relu(0.01))."""
 
-    def __init__(self, env, freq_count: int, hidden_units, n_in: int = 2):
+    def __init__(self, env, freq_count: int, hidden_units, n_in: int = 2, leakiness: float = 0.01):
         self.freq_count = freq_count
+        self.leakiness = leakiness
         prev = n_in if freq_count == 0 else 2 * n_in * freq_count
         self.hidden = []
         for h in hidden_units:
@@ -196,7 +197,7 @@ class ReluMlp(Module):
         if self.freq_count:
             x = positional_encoding(x, self.freq_count)
         for layer in self.hidden:
-            x = x.apply(layer, ctx).leaky_relu(0.01)
+            x = x.apply(layer, ctx).leaky_relu(self.leakiness)
         return x.apply(self.final, ctx)
 
 
@@ -329,13 +330,13 @@ def _image_fit_workload(env: Environment, module: Module, points01: np.ndarray, 
 
 
 def coordinate_mlp(env: Environment, side: int = 512, variant: str = "relu-pe", hidden=(256, 256, 256, 256),
-                   freq_count: int = 16, seed: int = 5) -> Workload:
+                   freq_count: int = 16, seed: int = 5, leakiness: float = 0.01) -> Workload:
     """Coordinate MLP image fit: every point of a side x side grid in [0,1]^2; "relu-pe" = positional encoding
     (freq_count sin/cos pairs per axis) + leaky_relu(0.01) hidden layers, "siren" = sin activations; Adam lr 1e-3."""
     rng = np.random.Generator(np.random.PCG64(seed))
     axis = (np.arange(side, dtype=np.float64) + 0.5) / side
     pts = np.stack(np.meshgrid(axis, axis, indexing="xy"), axis=-1).reshape(-1, 2)
-    module = Siren(env, hidden) if variant == "siren" else ReluMlp(env, freq_count, hidden)
+    module = Siren(env, hidden) if variant == "siren" else ReluMlp(env, freq_count, hidden, leakiness=leakiness)
     # the SIREN consumes coordinates in [-1, 1] as the reference feeds them (examples/image_fit/main.rs:372-375)
     return _image_fit_workload(env, module, pts, rng, 1e-3, (0.9, 0.999), signed_inputs=variant == "siren")
 

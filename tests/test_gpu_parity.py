@@ -186,14 +186,17 @@ def test_bias_gradient_rides_on_the_weight_gradient_matmul(hip_backend_session):
         assert err <= TOL, f"{key}: rel L2 {err}"
 
 
-@pytest.mark.parametrize("variant", ["relu-pe", "siren"])
+@pytest.mark.parametrize("variant", ["relu-pe", "siren", "plain-relu"])
 def test_coordinate_mlp_steps_vs_oracle(hip_backend_session, variant):
-    """Config 4 at reduced size (64x64 grid, two hidden layers of 64): three Adam steps."""
+    """Config 4 at reduced size (64x64 grid, two hidden layers of 64): three Adam steps.  "plain-relu" is the leaky
+    variant with slope 0: the schedule reads the sign of a pre-activation off the stored activation either way."""
     from descent_amd import workloads
 
     genv, cenv = _envs(hip_backend_session)
-    gw = workloads.coordinate_mlp(genv, side=64, variant=variant, hidden=(64, 64), freq_count=8, seed=21)
-    cw = workloads.coordinate_mlp(cenv, side=64, variant=variant, hidden=(64, 64), freq_count=8, seed=21)
+    kw = dict(side=64, variant="relu-pe" if variant == "plain-relu" else variant, hidden=(64, 64), freq_count=8, seed=21,
+              leakiness=0.0 if variant == "plain-relu" else 0.01)
+    gw = workloads.coordinate_mlp(genv, **kw)
+    cw = workloads.coordinate_mlp(cenv, **kw)
     for step in range(3):
         genv.run(gw.graph, step)
         cenv.run(cw.graph, step)
