@@ -2603,6 +2603,7 @@ std::string FusedKernel::key() const {
         }
     }
     if (shared_scatter) s += "|SS";
+    if (binned_pairs) s += "|BP";
     if (chain_group) s += "|CG";
     if (dgrad.wgrad_only) s += "|WO" + to_string((long long)dgrad.bands);
     if (binned_stage) s += "|BS" + to_string(binned_stage) + "," + to_string((long long)binned_table) + "," + to_string((long long)binned_total);
@@ -2835,11 +2836,15 @@ string generate_scatter_bin(const FusedKernel& fk, Generated* out) {
         total += element_count(d.inputs[0].out_shape);
     }
     if (table != fk.binned_table || total != fk.binned_total || fk.outputs.size() != 3) return "binned scatter: geometry differs from the plan";
-    const BinnedScatterPlan bp = binned_scatter_plan(table, total);
+    const bool pairs = fk.binned_pairs;
+    if (pairs)
+        for (auto& part : fk.parts)
+            if (!scatter_rows_of_two(part.main.raw())) return "binned scatter: a link does not add rows of two";
+    const BinnedScatterPlan bp = binned_scatter_plan(table, total, pairs);
     if (bp.nseg > 1024 || bp.nseg * bp.cap >= ((int64_t)1 << 31) || table >= ((int64_t)1 << 31)) return "binned scatter: accumulator too large";
     if (bp.nseg != 256) return "binned scatter: the kernels take 256 segments";
-    const int U = 8;
-    const int64_t per_wg = 1024 * U;
+    const int U = pairs ? 4 : 8;          // records per thread: 8192 values per workgroup either way
+    const int64_t per_wg = 1024 * U;      // records per workgroup
     const int rec = fk.outputs[0], cur = fk.outputs[1], acc = fk.outputs[2];
     Generated g;
     std::ostringstream src, fetches;
@@ -2857,14 +2862,26 @@ string generate_scatter_bin(const FusedKernel& fk, Generated* out) {
         emit_scatter_element(em, fn, "gid", "");
         fn << "    *out_value = value;\n    *out_at = at;\n    *out_ok = ok;\n}\n";
         src << "namespace part" << i << " {\n" << em.funcs.str() << fn.str() << "}  // namespace part" << i << "\n\n";
-        const int64_t wgs = (n + per_wg - 1) / per_wg;
+        const int64_t nrec = pairs ? n / 2 : n;  // records of this link
+        const int64_t wgs = (nrec + per_wg - 1) / per_wg;
         fetches << "    " << (i ? "else " : "") << "if (" << block_id << " < " << S(first_wg + wgs) << "u) {\n";
         fetches << "        const uint g0 = (" << block_id << " - " << S(first_wg) << "u) * " << S(per_wg) << "u + tid;\n";
         for (int u = 0; u < U; ++u) {
-            fetches << "        part" << i << "::fetch(min(g0 + " << S(u * 1024) << "u, " << S(n - 1) << "u), &v" << u << ", &a" << u << ", &k" << u;
-            for (int j : fk.part_params[i]) fetches << ", b" << j;
-            fetches << ", rand_seed);\n";
-            fetches << "        k" << u << " = k" << u << " && g0 + " << S(u * 1024) << "u < " << S(n) << "u;\n";
+            const string r = "min(g0 + " + S(u * 1024) + "u, " + S(nrec - 1) + "u)";
+            if (pairs) {
+                fetches << "        { int a_second; bool k_second;\n";
+                fetches << "        part" << i << "::fetch(2u * " << r << ", &v" << u << ", &a" << u << ", &k" << u;
+                for (int j : fk.part_params[i]) fetches << ", b" << j;
+                fetches << ", rand_seed);\n";
+                fetches << "        part" << i << "::fetch(2u * " << r << " + 1u, &w" << u << ", &a_second, &k_second";
+                for (int j : fk.part_params[i]) fetches << ", b" << j;
+                fetches << ", rand_seed); }\n";
+            } else {
+                fetches << "        part" << i << "::fetch(" << r << ", &v" << u << ", &a" << u << ", &k" << u;
+                for (int j : fk.part_params[i]) fetches << ", b" << j;
+                fetches << ", rand_seed);\n";
+            }
+            fetches << "        k" << u << " = k" << u << " && g0 + " << S(u * 1024) << "u < " << S(nrec) << "u;\n";
         }
         fetches << "    }\n";
         first_wg += wgs;
@@ -2880,16 +2897,18 @@ string generate_scatter_bin(const FusedKernel& fk, Generated* out) {
         src << "    float2* const stage = reinterpret_cast<float2*>(dsc_lds);\n";
         src << "    uint* const cnt = reinterpret_cast<uint*>(dsc_lds + " << S(per_wg * 8) << ");\n";
         src << "    uint* const lbase = cnt + " << S(bp.nseg) << ";\n    uint* const gbase = lbase + " << S(bp.nseg) << ";\n    uint* const wsum = gbase + " << S(bp.nseg) << ";\n";
+        if (pairs) src << "    int* const stage_at = reinterpret_cast<int*>(wsum + 16);\n";
     } else {
         src << "extern \"C\" __global__ __launch_bounds__(1024) void " << g.entry << "(" << em.kernel_params_decl() << ") {\n";
         src << "    __shared__ uint cnt[" << S(bp.nseg) << "], lbase[" << S(bp.nseg) << "], gbase[" << S(bp.nseg) << "], wsum[16];\n";
         src << "    __shared__ float2 stage[" << S(per_wg) << "];\n";
+        if (pairs) src << "    __shared__ int stage_at[" << S(per_wg) << "];\n";
     }
-    g.lds_bytes = (size_t)(per_wg * 8 + (3 * bp.nseg + 16) * 4);
+    g.lds_bytes = (size_t)(per_wg * (pairs ? 12 : 8) + (3 * bp.nseg + 16) * 4);
     src << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
     src << "    const uint tid = threadIdx.x;\n";
     src << "    for (uint i = tid; i < " << S(bp.nseg) << "u; i += 1024u) cnt[i] = 0u;\n    __syncthreads();\n";
-    for (int u = 0; u < U; ++u) src << "    float v" << u << " = 0.f; int a" << u << " = 0; bool k" << u << " = false;\n";
+    for (int u = 0; u < U; ++u) src << "    float v" << u << " = 0.f, w" << u << " = 0.f; int a" << u << " = 0; bool k" << u << " = false;\n";
     src << fetches.str();
     src << "    __builtin_amdgcn_sched_barrier(0);\n";
     for (int u = 0; u < U; ++u) src << "    const uint r" << u << " = k" << u << " ? atomicAdd(&cnt[(a" << u << " >> 4) & 255], 1u) : 0u;\n";
@@ -2903,6 +2922,20 @@ string generate_scatter_bin(const FusedKernel& fk, Generated* out) {
     src << "    uint* const cursor = reinterpret_cast<uint*>(b" << cur << ");\n";
     src << "    if (tid < " << S(bp.nseg) << "u) {\n        lbase[tid] = before + incl - c;\n        gbase[tid] = c ? atomicAdd(&cursor[tid * 16u], c) : 0u;\n    }\n";
     src << "    __syncthreads();\n";
+    if (pairs) {
+        // a record is a row: both values in one array, the target of the first in another behind it
+        for (int u = 0; u < U; ++u)
+            src << "    if (k" << u << ") { const uint at_slot = lbase[(a" << u << " >> 4) & 255] + r" << u << "; stage[at_slot] = make_float2(v" << u << ", w" << u
+                << "); stage_at[at_slot] = a" << u << "; }\n";
+        src << "    __syncthreads();\n";
+        src << "    float2* const records = reinterpret_cast<float2*>(b" << rec << ");\n";
+        src << "    int* const targets = reinterpret_cast<int*>(b" << rec << ") + " << S(2 * bp.nseg * bp.cap) << ";\n";
+        src << "    for (uint slot = tid; slot < filled; slot += 1024u) {\n";
+        src << "        const float2 r = stage[slot];\n        const int a = stage_at[slot];\n        const uint bin = ((uint)a >> 4) & 255u;\n";
+        src << "        const uint pos = gbase[bin] + (slot - lbase[bin]);\n";
+        src << "        if (pos < " << S(bp.cap) << "u) { records[bin * " << S(bp.cap) << "u + pos] = r; targets[bin * " << S(bp.cap) << "u + pos] = a; }\n";
+        src << "        else { unsafeAtomicAdd(&b" << acc << "[a], r.x); unsafeAtomicAdd(&b" << acc << "[a + 1], r.y); }\n    }\n}\n";
+    } else {
     for (int u = 0; u < U; ++u)
         src << "    if (k" << u << ") stage[lbase[(a" << u << " >> 4) & 255] + r" << u << "] = make_float2(__int_as_float(a" << u << "), v" << u << ");\n";
     src << "    __syncthreads();\n";
@@ -2912,11 +2945,12 @@ string generate_scatter_bin(const FusedKernel& fk, Generated* out) {
     src << "        const uint pos = gbase[bin] + (slot - lbase[bin]);\n";
     src << "        if (pos < " << S(bp.cap) << "u) records[bin * " << S(bp.cap) << "u + pos] = r;\n";
     src << "        else unsafeAtomicAdd(&b" << acc << "[a], r.y);\n    }\n}\n";
+    }
     g.source = src.str();
     g.grid = (unsigned)first_wg;
     g.block = 1024;
     g.n_buffers = fk.n_buffers;
-    g.note = "scatter chain, stage 1 of 2: " + to_string(fk.parts.size()) + " links, (target, value) records ordered by segment in LDS (" + S(bp.nseg) +
+    g.note = "scatter chain, stage 1 of 2: " + to_string(fk.parts.size()) + " links, " + (pairs ? "(target, two values)" : "(target, value)") + " records ordered by segment in LDS (" + S(bp.nseg) +
              " segments of " + S(bp.seg) + " floats, the accumulator's 64-byte lines dealt to them in turn), written in runs into bins of " + S(bp.cap) + " records";
     *out = g;
     return "";
@@ -2930,7 +2964,8 @@ string generate_scatter_sum(const FusedKernel& fk, Generated* out) {
     if (d.kind != DSC_KERNEL_SCATTER_ADD || table != fk.binned_table || fk.inputs.size() != 2 || fk.outputs.size() != 1 || fk.n_buffers != 3 ||
         fk.inputs[0].buffer < 0 || fk.inputs[1].buffer < 0)
         return "binned scatter: stage 2 binds records, counters and the accumulator";
-    const BinnedScatterPlan bp = binned_scatter_plan(table, fk.binned_total);
+    const bool pairs = fk.binned_pairs;
+    const BinnedScatterPlan bp = binned_scatter_plan(table, fk.binned_total, pairs);
     if (bp.nseg != 256 || bp.seg * 8 > 144 * 1024 || bp.nseg * bp.cap >= ((int64_t)1 << 31)) return "binned scatter: accumulator too large";
     const int rec = fk.inputs[0].buffer, cur = fk.inputs[1].buffer, acc = fk.outputs[0];
     const int U = 4;
@@ -2955,12 +2990,25 @@ string generate_scatter_sum(const FusedKernel& fk, Generated* out) {
     src << "    const uint lo = (uint)((unsigned long long)count * slice / " << S(bp.slices) << "u), hi = (uint)((unsigned long long)count * (slice + 1u) / " << S(bp.slices) << "u);\n";
     src << "    const float2* const records = reinterpret_cast<const float2*>(b" << rec << ") + s * " << S(bp.cap) << "u;\n";
     src << "    uint i = lo + tid;\n";
+    if (pairs) {
+        // a row's two values sit side by side in one line of the accumulator, so side by side in the segment too
+        src << "    const int* const targets = reinterpret_cast<const int*>(b" << rec << ") + " << S(2 * bp.nseg * bp.cap) << " + s * " << S(bp.cap) << "u;\n";
+        src << "    for (; i + " << S((U - 1) * 1024) << "u < hi; i += " << S(U * 1024) << "u) {\n";
+        for (int u = 0; u < U; ++u) src << "        const float2 r" << u << " = records[i + " << S(u * 1024) << "u]; const int t" << u << " = targets[i + " << S(u * 1024) << "u];\n";
+        src << "        __builtin_amdgcn_sched_barrier(0);\n";
+        for (int u = 0; u < U; ++u)
+            src << "        { double* const at = &seg[LOCAL(t" << u << ")]; atomicAdd(at, (double)r" << u << ".x); atomicAdd(at + 1, (double)r" << u << ".y); }\n";
+        src << "    }\n";
+        src << "    for (; i < hi; i += 1024u) {\n        const float2 r = records[i];\n        double* const at = &seg[LOCAL(targets[i])];\n";
+        src << "        atomicAdd(at, (double)r.x); atomicAdd(at + 1, (double)r.y);\n    }\n";
+    } else {
     src << "    for (; i + " << S((U - 1) * 1024) << "u < hi; i += " << S(U * 1024) << "u) {\n";
     for (int u = 0; u < U; ++u) src << "        const float2 r" << u << " = records[i + " << S(u * 1024) << "u];\n";
     src << "        __builtin_amdgcn_sched_barrier(0);\n";
     for (int u = 0; u < U; ++u) src << "        atomicAdd(&seg[LOCAL(__float_as_int(r" << u << ".x))], (double)r" << u << ".y);\n";
     src << "    }\n";
     src << "    for (; i < hi; i += 1024u) {\n        const float2 r = records[i];\n        atomicAdd(&seg[LOCAL(__float_as_int(r.x))], (double)r.y);\n    }\n";
+    }
     src << "    __syncthreads();\n";
     // local float j of segment s is float j % 16 of the accumulator's line (j / 16) * 256 + s
     src << "    for (uint j = tid; j < " << S(bp.seg) << "u; j += 1024u) {\n        const float sum = (float)seg[j];\n";
@@ -3041,7 +3089,12 @@ bool scatter_chain_binned(int64_t table_elements, int64_t total_values) {
     return total_values >= (1 << 18) && total_values * 4 >= table_elements && table_elements >= 16 * 256 && table_elements <= 256 * 16384;
 }
 
-BinnedScatterPlan binned_scatter_plan(int64_t table_elements, int64_t total_values) {
+bool scatter_rows_of_two(const dsc_kernel_desc& d) {
+    return d.kind == DSC_KERNEL_SCATTER_ADD && d.axis == 0 && d.shape.rank == 2 && d.shape.dims[1] == 2 && d.n_inputs == 2 &&
+           d.inputs[0].out_shape.rank == 2 && d.inputs[0].out_shape.dims[1] == 2;
+}
+
+BinnedScatterPlan binned_scatter_plan(int64_t table_elements, int64_t total_values, bool pairs) {
     // The accumulator's 64-byte lines are dealt to 256 segments in turn (line l belongs to segment l % 256): a hash
     // or a row-major grid index spreads evenly over the low bits of the line number even where its high bits are
     // skewed (measured on the reference's hash at 2^19 entries: contiguous segments received up to six times
@@ -3051,7 +3104,9 @@ BinnedScatterPlan binned_scatter_plan(int64_t table_elements, int64_t total_valu
     const int64_t lines = (table_elements + 15) / 16;
     p.seg = (lines + p.nseg - 1) / p.nseg * 16;
     // a quarter more than an even spread needs; what does not fit goes to the accumulator directly
-    p.cap = ((total_values / p.nseg) * 5 / 4 + 2048 + 63) / 64 * 64;
+    const int64_t records = pairs ? total_values / 2 : total_values;
+    p.cap = ((records / p.nseg) * 5 / 4 + 2048 + 63) / 64 * 64;
+    p.record_bytes = pairs ? 12 : 8;
     p.slices = 1;
     return p;
 }

@@ -87,6 +87,9 @@ struct FusedKernel {
     bool chain_group = false;
     int binned_stage = 0;
     int64_t binned_table = 0, binned_total = 0;  // accumulator elements, values of all links together
+    // The accumulator is [entries, 2] and every link adds rows of two along axis 0: a record is then (target of the
+    // row's first value, both values), twelve bytes for two values instead of sixteen, and one count per row.
+    bool binned_pairs = false;
     // Data gradient of a stride-1 convolution with few channels, as one kernel: `main` is the MatMul dC x filter^T
     // ([g][(img, oy, ox)][oc] x [g][oc][(fy, fx, c)]); the kernel also does what the reference's WindowsToImage
     // (sum of the windows covering each pixel of the padded image) and the two Unpads after it (fold the
@@ -186,11 +189,14 @@ bool scatter_chain_in_lds(int64_t table_elements, int64_t total_values);
 struct BinnedScatterPlan {
     int64_t seg = 0;     // accumulator elements per segment (whole 64-byte lines; line l belongs to segment l % nseg)
     int64_t nseg = 0;    // segments = bins
-    int64_t cap = 0;     // records a bin holds
+    int64_t cap = 0;     // records a bin holds (a record is one value, or one row of two)
+    int64_t record_bytes = 8;
     int64_t slices = 0;  // stage-2 workgroups per segment
 };
 bool scatter_chain_binned(int64_t table_elements, int64_t total_values);
-BinnedScatterPlan binned_scatter_plan(int64_t table_elements, int64_t total_values);
+BinnedScatterPlan binned_scatter_plan(int64_t table_elements, int64_t total_values, bool pairs = false);
+// Whether a ScatterAdd adds rows of two values that share an index (accumulator [entries, 2], axis 0).
+bool scatter_rows_of_two(const dsc_kernel_desc& d);
 
 // Whether a kernel can be one part of a multi-part launch (256 threads per workgroup, addressed by blockIdx.x only).
 bool can_be_part(const FusedKernel& k);

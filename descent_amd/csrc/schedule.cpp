@@ -2118,14 +2118,16 @@ struct Planner {
             const int64_t table = element_count(drafts[i].fk.main.raw().shape);
             if (!multi.fk.shared_scatter && scatter_chain_binned(table, total_values) && (size_t)table * 4 == node_bytes[final_node]) {
                 // two launches: the links' values go to bins by accumulator segment, then every segment is summed in LDS
-                const BinnedScatterPlan bp = binned_scatter_plan(table, total_values);
+                bool pairs = true;
+                for (int j : chain) pairs = pairs && scatter_rows_of_two(drafts[j].fk.main.raw());
+                const BinnedScatterPlan bp = binned_scatter_plan(table, total_values, pairs);
                 auto new_node = [&](size_t bytes) {
                     node_bytes.push_back(bytes);
                     is_graph_output.push_back(false);
                     is_graph_input.push_back(false);
                     return n_nodes++;
                 };
-                const int records = new_node((size_t)(bp.nseg * bp.cap) * 8);
+                const int records = new_node((size_t)(bp.nseg * bp.cap) * (size_t)bp.record_bytes);
                 const int cursor = new_node((size_t)bp.nseg * 64);  // one counter per 64-byte line
                 const int zero = new_node(0);                       // stands for the literal the counters start from
                 const int mid = new_node(node_bytes[final_node]);   // the accumulator between the two launches
@@ -2134,6 +2136,7 @@ struct Planner {
                 multi.fk.binned_stage = 1;
                 multi.fk.binned_table = table;
                 multi.fk.binned_total = total_values;
+                multi.fk.binned_pairs = pairs;
                 multi.fk.outputs = {param_index(multi, records, true), param_index(multi, cursor, true), param_index(multi, mid, true)};
                 out.node = mid;
                 multi.outs = {StepOutput{records, -1, false, 0}, StepOutput{cursor, zero, true, 0}, out};
@@ -2142,6 +2145,7 @@ struct Planner {
                 sum.fk.binned_stage = 2;
                 sum.fk.binned_table = table;
                 sum.fk.binned_total = total_values;
+                sum.fk.binned_pairs = pairs;
                 sum.params = {records, cursor, final_node};
                 sum.fk.buffer_is_output = {false, false, true};
                 sum.fk.n_buffers = 3;
