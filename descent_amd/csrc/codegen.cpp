@@ -2384,9 +2384,32 @@ string gen_matmul(Emitter& em, Generated* out) {
         k << "#define MM_COLSUM 0\n";
     }
 
+    // k-tiles straight from memory into LDS (see MM_DIRECT in the template), for the tile shapes of up to four waves:
+    // measured on MI355X, two tile buffers, 1024^3 (64x64x64 tiles) 63.3 -> 77.4 TFLOP/s, 2048^3 (128x128x16) 89.8 ->
+    // 100.8; the sixteen-wave 256x256x16 tile loses 1.6 % with it (8192^3 137.9 -> 135.5, 4096^3 131.4 -> 129.2) and
+    // keeps its pass through registers.  A third buffer (two tiles requested ahead) measured the same as two.
+    // DSC_MM_DIRECT_LDS=0 switches the path off, =2 / =3 force it with that many buffers wherever a product allows it.
+    int direct = 0;
+    {
+        const char* e = std::getenv("DSC_MM_DIRECT_LDS");
+        const int nt = 64 * c.wm * c.wn;
+        const int nbuf = !e ? (nt <= 256 ? 2 : 0) : e[0] == '2' ? 2 : e[0] == '3' ? 3 : 0;
+        const bool whole = g.m % c.bm == 0 && g.n % c.bn == 0 && chunk_k % c.bk == 0 && g.k % chunk_k == 0;
+        const bool even = (c.bm * c.bk / 4) % nt == 0 && (c.bn * c.bk / 4) % nt == 0 && (c.bk & (c.bk - 1)) == 0;
+        if (nbuf && a_mode && b_mode && fk.colsum_out < 0 && whole && even && chunk_k / c.bk >= nbuf &&
+            (int64_t)nbuf * (c.bm + c.bn) * c.bk * 4 <= 160 * 1024)
+            direct = nbuf;
+    }
+    k << "#define MM_DIRECT " << direct << "\n";
+
     // results leave through LDS as 16-byte row pieces when the output allows it
     bool vec_store = g.n % 4 == 0 && batch_stride % 4 == 0 && row_stride % 4 == 0 && (g.batch * g.m * g.n) % 4 == 0;
-    {
+    if (direct) {
+        // every wave's corner has to fit the one tile buffer that is free at the end of a unit
+        if ((int64_t)c.wm * c.wn * 32 * 36 > (int64_t)(c.bm + c.bn) * c.bk) vec_store = false;
+        if (const char* e = std::getenv("DSC_MM_VEC_STORE"))
+            if (e[0] == '0') vec_store = false;
+    } else {
         const int64_t sa = a_mode == 1 ? c.bm * (c.bk + 4) : c.bk * (c.bm + 8), sb = b_mode == 2 ? c.bn * (c.bk + 4) : c.bk * (c.bn + 8);
         const int64_t per_wave = 32 * 36, waves = (int64_t)c.wm * c.wn;
         const int64_t in_a = std::min(waves, 2 * sa / per_wave);
@@ -2441,10 +2464,10 @@ string gen_matmul(Emitter& em, Generated* out) {
         const char* e = std::getenv("DSC_MM_PERSISTENT");
         out->persistent_ok = !(e && e[0] == '0') && !fk.as_part && grid > 256 && chunk_k / c.bk <= 128;
     }
-    char note[160];
-    std::snprintf(note, sizeof note, "mfma 32x32x2 tile %dx%dx%d waves %dx%d A%d B%d chunks %lld%s%s%s", c.bm, c.bn, c.bk, c.wm, c.wn,
+    char note[224];
+    std::snprintf(note, sizeof note, "mfma 32x32x2 tile %dx%dx%d waves %dx%d A%d B%d chunks %lld%s%s%s%s", c.bm, c.bn, c.bk, c.wm, c.wn,
                   a_mode, b_mode, (long long)kchunks, fk.has_epilogue ? " +epilogue" : "", fk.colsum_out >= 0 ? " +column sums of B" : "",
-                  out->persistent_ok ? " persistent" : "");
+                  out->persistent_ok ? " persistent" : "", direct == 3 ? " tiles straight into LDS x3" : direct == 2 ? " tiles straight into LDS x2" : "");
     out->note = note;
     return "";
 }
@@ -2620,7 +2643,7 @@ std::string FusedKernel::key() const {
     s.append(reinterpret_cast<const char*>(&n_buffers), 4);
     if (const char* env = std::getenv("DSC_MM_TILE"))
         if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|T") + env;
-    for (const char* name : {"DSC_MM_SMALLK", "DSC_MM_VEC_STORE", "DSC_MM_PERSISTENT", "DSC_MM_DEEP_K", "DSC_MM_ROWS", "DSC_MM_DOT", "DSC_ROWS_MFMA", "DSC_MM_TALLK"})
+    for (const char* name : {"DSC_MM_SMALLK", "DSC_MM_VEC_STORE", "DSC_MM_PERSISTENT", "DSC_MM_DEEP_K", "DSC_MM_DIRECT_LDS", "DSC_MM_ROWS", "DSC_MM_DOT", "DSC_ROWS_MFMA", "DSC_MM_TALLK"})
         if (const char* env = std::getenv(name))
             if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|") + name + env;
     return s;

@@ -78,6 +78,43 @@ def test_matmul_transposed_operands(hip_backend_session, ta, tb, m, n, k):
     assert rel_l2(got, want) <= TOL
 
 
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("m,n,k,tile,buffers", [
+    (256, 256, 64, "32x32x16", None), (1024, 512, 128, "64x32x16", None), (1024, 1024, 128, "64x64x16", None),
+    (1024, 1024, 1024, "64x64x64", None), (2048, 1024, 128, "128x64x16", None), (2048, 2048, 64, "128x128x16", None),
+    (2048, 2048, 64, "128x128x16", "3"), (4096, 2048, 64, "256x128x16", "2"), (4096, 4096, 64, "256x256x16", "2"),
+    (4096, 4096, 48, "256x256x16", "3"),
+    # more tiles than workgroups: a workgroup's stream of k-tiles runs on into its next unit
+    (2048, 3072, 64, "128x128x16", None), (2048, 3072, 64, "128x128x16", "3"), (1024, 1536, 512, "64x64x64", None),
+    (1024, 1536, 512, "64x64x64", "3"), (8192, 4096, 48, "256x256x16", "3"),
+])
+def test_matmul_tiles_loaded_straight_into_lds(hip_backend_session, monkeypatch, m, n, k, tile, buffers, ta, tb):
+    """Whole-tile products take their k-tiles from memory straight into LDS: every tile shape, both operand
+    layouts on either side, two and three tile buffers, against the oracle."""
+    from descent_amd import hip_backend
+
+    if buffers is None:
+        monkeypatch.delenv("DSC_MM_DIRECT_LDS", raising=False)
+    else:
+        monkeypatch.setenv("DSC_MM_DIRECT_LDS", buffers)  # read when a kernel is generated; part of the kernel cache key
+    genv, cenv = _envs(hip_backend_session)
+    got = _transposed_case(genv, np.random.default_rng(m + k), m, n, k, ta, tb)
+    want = _transposed_case(cenv, np.random.default_rng(m + k), m, n, k, ta, tb)
+    assert rel_l2(got, want) <= TOL
+    # the launch that ran is the one the listing describes
+    a = genv.static_parameter([k, m] if ta else [m, k], "a")
+    b = genv.static_parameter([n, k] if tb else [k, n], "b")
+    c = genv.static_parameter([m, n], "c")
+
+    def build(s):
+        av, bv = s.parameter_value(a), s.parameter_value(b)
+        s.write_parameter_value(c, (av.transpose() if ta else av).matmul(bv.transpose() if tb else bv))
+
+    listing = hip_backend.check_schedule(genv.build_graph(build), fused=True)
+    assert f"tile {tile} " in listing and f"A{2 if ta else 1} B{2 if tb else 1}" in listing, listing
+    assert f"tiles straight into LDS x{buffers or 2}" in listing, listing
+
+
 @pytest.mark.parametrize("mode", ["fused", "unfused", "kernel_by_kernel"])
 def test_convnet_train_steps_vs_oracle(hip_backend_session, mode):
     """Three Adam steps of the ConvNet at batch 16: every parameter, optimiser state and the loss/accuracy sums."""
