@@ -2384,16 +2384,17 @@ string gen_matmul(Emitter& em, Generated* out) {
         k << "#define MM_COLSUM 0\n";
     }
 
-    // k-tiles straight from memory into LDS (see MM_DIRECT in the template), for the tile shapes of up to four waves:
-    // measured on MI355X, two tile buffers, 1024^3 (64x64x64 tiles) 63.3 -> 77.4 TFLOP/s, 2048^3 (128x128x16) 89.8 ->
-    // 100.8; the sixteen-wave 256x256x16 tile loses 1.6 % with it (8192^3 137.9 -> 135.5, 4096^3 131.4 -> 129.2) and
-    // keeps its pass through registers.  A third buffer (two tiles requested ahead) measured the same as two.
-    // DSC_MM_DIRECT_LDS=0 switches the path off, =2 / =3 force it with that many buffers wherever a product allows it.
+    // k-tiles straight from memory into LDS (see MM_DIRECT in the template) wherever a product consists of whole tiles.
+    // Measured on MI355X with two tile buffers against the pass through registers (TFLOP/s): 1024^3 (64x64x64 tiles)
+    // 64.9 -> 78.4, 2048^3 (128x128x16) 92.0 -> 101.2, 2048x4096x1024 101.6 -> 107.2 and 4096x2048x4096 116.5 -> 120.1
+    // (256x128x16), 262144x256x256 101.9 -> 103.5, 4096^3 131.9 -> 131.9, 8192^3 138.2 -> 138.6 (256x256x16).  A third
+    // buffer (two tiles requested ahead) measured 1-2 % below two.
+    // DSC_MM_DIRECT_LDS=0 switches the path off, =2 / =3 choose the number of buffers.
     int direct = 0;
     {
         const char* e = std::getenv("DSC_MM_DIRECT_LDS");
         const int nt = 64 * c.wm * c.wn;
-        const int nbuf = !e ? (nt <= 256 ? 2 : 0) : e[0] == '2' ? 2 : e[0] == '3' ? 3 : 0;
+        const int nbuf = !e ? 2 : e[0] == '2' ? 2 : e[0] == '3' ? 3 : 0;
         const bool whole = g.m % c.bm == 0 && g.n % c.bn == 0 && chunk_k % c.bk == 0 && g.k % chunk_k == 0;
         const bool even = (c.bm * c.bk / 4) % nt == 0 && (c.bn * c.bk / 4) % nt == 0 && (c.bk & (c.bk - 1)) == 0;
         if (nbuf && a_mode && b_mode && fk.colsum_out < 0 && whole && even && chunk_k / c.bk >= nbuf &&
@@ -2405,8 +2406,8 @@ string gen_matmul(Emitter& em, Generated* out) {
     // results leave through LDS as 16-byte row pieces when the output allows it
     bool vec_store = g.n % 4 == 0 && batch_stride % 4 == 0 && row_stride % 4 == 0 && (g.batch * g.m * g.n) % 4 == 0;
     if (direct) {
-        // every wave's corner has to fit the one tile buffer that is free at the end of a unit
-        if ((int64_t)c.wm * c.wn * 32 * 36 > (int64_t)(c.bm + c.bn) * c.bk) vec_store = false;
+        // every wave's corner (eight rows of a block) has to fit the one tile buffer that is free at the end of a unit
+        if ((int64_t)c.wm * c.wn * 8 * 40 > (int64_t)(c.bm + c.bn) * c.bk) vec_store = false;
         if (const char* e = std::getenv("DSC_MM_VEC_STORE"))
             if (e[0] == '0') vec_store = false;
     } else {
@@ -2418,6 +2419,20 @@ string gen_matmul(Emitter& em, Generated* out) {
             if (e[0] == '0') vec_store = false;
     }
     k << "#define MM_VEC_STORE " << (vec_store ? 1 : 0) << "\n";
+    {
+        bool long_epilogue = false;
+        if (fk.has_epilogue) {
+            const dsc_kernel_desc& pe = fk.epilogue.raw();
+            for (int o = 0; o < pe.n_ops; ++o) {
+                const dsc_pe_op& op = pe.ops[o];
+                if (op.kind == DSC_PE_UNARY && (op.op == DSC_UN_SIN || op.op == DSC_UN_COS || op.op == DSC_UN_EXP || op.op == DSC_UN_LOG)) long_epilogue = true;
+                if (op.kind == DSC_PE_BINARY && op.op == DSC_BIN_POW) long_epilogue = true;
+                if (op.kind == DSC_PE_RAND || op.kind == DSC_PE_GATHER) long_epilogue = true;
+            }
+            if (pe.n_ops > 24 || !fk.virtuals.empty()) long_epilogue = true;
+        }
+        k << "#define MM_LONG_EPILOGUE " << (long_epilogue ? 1 : 0) << "\n";
+    }
     if (fk.has_epilogue) {
         const dsc_kernel_desc& pe = fk.epilogue.raw();
         std::ostringstream body;
