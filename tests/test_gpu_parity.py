@@ -115,6 +115,48 @@ def test_matmul_tiles_loaded_straight_into_lds(hip_backend_session, monkeypatch,
     assert f"tiles straight into LDS x{buffers or 2}" in listing, listing
 
 
+@pytest.mark.parametrize("case", ["k-chunks", "batches", "rows-mode", "batches-transposed"])
+def test_direct_lds_tiles_over_k_chunks_and_batches(hip_backend_session, case):
+    """The same path where a unit is a (k-chunk, batch, tile) triple: the reference's 1024-deep k-chunks written as
+    separate partial products (cluster by cluster), and batched products in both output modes."""
+    from descent_amd import hip_backend
+    from descent_amd.array import BATCHES, ROWS
+
+    fused = case != "k-chunks"
+    genv, cenv = _envs(hip_backend_session, fused=fused)
+
+    def run(env):
+        rng = np.random.default_rng(11)
+        if case == "k-chunks":
+            m, n, k = 512, 512, 4096
+            a = env.static_parameter_with_data([m, k], "a", rng.standard_normal(m * k, dtype=np.float32))
+            b = env.static_parameter_with_data([k, n], "b", rng.standard_normal(k * n, dtype=np.float32))
+            c = env.static_parameter([m, n], "c")
+            build = lambda s: s.write_parameter_value(c, s.parameter_value(a).matmul(s.parameter_value(b)))
+        else:
+            g, m, n, k = 3, 1024, 512, 96
+            tb = case == "batches-transposed"
+            a = env.static_parameter_with_data([g, m, k], "a", rng.standard_normal(g * m * k, dtype=np.float32))
+            b = env.static_parameter_with_data([g, n, k] if tb else [g, k, n], "b", rng.standard_normal(g * k * n, dtype=np.float32))
+            c = env.static_parameter([g, m, n], "c")
+
+            def build(s):
+                bv = s.parameter_value(b)
+                s.write_parameter_value(c, s.parameter_value(a).batched_matmul(bv.transpose() if tb else bv, ROWS if case == "rows-mode" else BATCHES))
+
+        graph = env.build_graph(build)
+        env.run(graph, 0)
+        return env.read_parameter(c), graph
+
+    got, graph = run(genv)
+    want, _ = run(cenv)
+    assert rel_l2(got, want) <= TOL
+    listing = hip_backend.check_schedule(graph, fused=fused)
+    assert "tiles straight into LDS" in listing, listing
+    if case == "k-chunks":
+        assert "chunks 4" in listing, listing
+
+
 @pytest.mark.parametrize("mode", ["fused", "unfused", "kernel_by_kernel"])
 def test_convnet_train_steps_vs_oracle(hip_backend_session, mode):
     """Three Adam steps of the ConvNet at batch 16: every parameter, optimiser state and the loss/accuracy sums."""
