@@ -1687,6 +1687,87 @@ struct Planner {
         }
     }
 
+    // Pass 1h: a per-element cluster that reads nothing but small arrays (all of its inputs together fit the L2 of
+    // one XCD: the coordinates of a mini-batch) and writes large ones is evaluated again by each of its readers, and
+    // its outputs are neither written nor read back.  The hashed corner indices and bilinear weights of a grid level
+    // are such outputs: a megabyte each, four of each per level, read by the forward gather and again by the four
+    // ScatterAdds of the backward pass, all of them integer and float arithmetic on two coordinates.
+    void recompute_from_small_inputs() {
+        if (const char* e = std::getenv("DSC_RECOMPUTE_SMALL"))
+            if (e[0] == '0') return;
+        const size_t kInputLimit = (size_t)4 << 20, kOutputFloor = (size_t)256 << 10;
+        for (int i = 0; i < (int)drafts.size(); ++i) {
+            Draft& p = drafts[i];
+            if (!p.alive || !p.fk.parts.empty() || !p.fk.row_stages.empty() || !p.fk.virtuals.empty() || p.fk.has_epilogue || p.keep_output) continue;
+            const dsc_kernel_desc& pd = p.fk.main.raw();
+            if (pd.kind != DSC_KERNEL_PER_ELEMENT || pd.n_ops > 40) continue;
+            bool plain = true;
+            for (int o = 0; o < pd.n_ops && plain; ++o) {
+                const dsc_pe_op& op = pd.ops[o];
+                if (op.kind == DSC_PE_GATHER || op.kind == DSC_PE_RAND) plain = false;
+                if (op.kind == DSC_PE_UNARY && (op.op == DSC_UN_SQRT || op.op == DSC_UN_EXP || op.op == DSC_UN_LOG || op.op == DSC_UN_SIN || op.op == DSC_UN_COS)) plain = false;
+                if (op.kind == DSC_PE_BINARY && (op.op == DSC_BIN_POW || op.op == DSC_BIN_DIV)) plain = false;
+            }
+            if (!plain) continue;
+            size_t in_bytes = 0;
+            bool ok = true;
+            for (auto& src : p.fk.inputs) {
+                if (src.buffer < 0) { ok = false; break; }
+                in_bytes += node_bytes[p.params[src.buffer]];
+            }
+            if (!ok || p.fk.inputs.empty() || in_bytes > kInputLimit) continue;
+            std::set<int> readers;
+            for (auto& out : p.outs) {
+                if (is_graph_output[out.node] || out.copy_from >= 0 || node_bytes[out.node] < kOutputFloor) { ok = false; break; }
+                for (int ci : consumers_of(out.node)) readers.insert(ci);
+            }
+            if (!ok || readers.empty()) continue;
+            for (int ci : readers) {
+                Draft& q = drafts[ci];
+                const int qk = q.fk.main.raw().kind;
+                if (ci <= i || !q.fk.parts.empty() || !q.fk.row_stages.empty() || q.fk.dgrad.on || q.fk.cfwd.on || q.fk.pool.on) ok = false;
+                if (qk != DSC_KERNEL_PER_ELEMENT && qk != DSC_KERNEL_REDUCE && qk != DSC_KERNEL_SCATTER_ADD) ok = false;
+                if ((int)q.fk.virtuals.size() + (int)p.outs.size() > 12) ok = false;
+                for (auto& o : q.outs)
+                    for (auto& out : p.outs)
+                        if (o.copy_from == out.node) ok = false;  // updated in place by the reader
+                if (ok && taken_in_place_between(i, ci, input_nodes(p))) ok = false;
+                if (q.fk.has_epilogue && q.fk.epilogue_product_input >= 0) {
+                    const Source& ps = q.fk.epilogue_inputs[q.fk.epilogue_product_input];
+                    for (auto& out : p.outs)
+                        if (ps.buffer >= 0 && q.params[ps.buffer] == out.node) ok = false;
+                }
+            }
+            if (!ok) continue;
+            for (int ci : readers) {
+                Draft& q = drafts[ci];
+                for (size_t o = 0; o < p.outs.size(); ++o) {
+                    const int node = p.outs[o].node;
+                    bool reads = false;
+                    for_each_source(q.fk, [&](Source& src) {
+                        if (src.buffer >= 0 && q.params[src.buffer] == node && !q.fk.buffer_is_output[src.buffer]) reads = true;
+                    });
+                    if (!reads) continue;
+                    const int new_virt = (int)q.fk.virtuals.size();
+                    Virtual nv;
+                    nv.pe = p.fk.main;
+                    nv.out_op = pd.outputs[o];
+                    for (auto& src : p.fk.inputs) nv.inputs.push_back(import_source(q, p, src, 0));
+                    q.fk.virtuals.push_back(nv);
+                    for_each_source(q.fk, [&](Source& src) {
+                        if (src.buffer >= 0 && q.params[src.buffer] == node && !q.fk.buffer_is_output[src.buffer]) {
+                            src.buffer = -1;
+                            src.virt = new_virt;
+                        }
+                    });
+                }
+                q.covers.insert(q.covers.end(), p.covers.begin(), p.covers.end());
+                compact(q);
+            }
+            p.alive = false;
+        }
+    }
+
     // Pass 2: per-element producers whose result need not exist in memory are evaluated inside their
     // consumers: pure copies (materialised im2col / pooling windows) into every consumer, light arithmetic
     // into a single consumer.
@@ -2351,6 +2432,7 @@ struct Planner {
         conv_backward();                        // pass 1e
         disjoint_windows_to_copies();           // pass 1g
         row_kernels();                          // pass 1b
+        recompute_from_small_inputs();          // pass 1h
         inline_producers();                     // pass 2
         attach_epilogues();                     // pass 3
         slice_major_products();                 // pass 3d
