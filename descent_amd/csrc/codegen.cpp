@@ -196,11 +196,49 @@ struct Emitter {
         return f;
     }
 
+    // The index as one term per axis of the view's input (clamped where the view pads), for views index_form gives up on.
+    bool axis_form(const dsc_view& v, const std::vector<string>& coord, IndexForm* f, std::vector<string>* args) const {
+        int64_t st[DSC_MAX_DIM];
+        strides_of(v.in_shape, st);
+        for (int i = 0; i < v.in_shape.rank; ++i) {
+            if (v.in_shape.dims[i] <= 1) continue;
+            string e = S(v.in_offset[i]);
+            bool driven = false;
+            for (int j = 0; j < v.out_shape.rank; ++j)
+                if (v.map_axis[j] == i && v.out_shape.dims[j] > 1) {
+                    e += " + (" + S(v.map_step[j]) + ")*" + coord[j];
+                    driven = true;
+                }
+            if (!driven) {
+                if (v.in_offset[i] != 0) return false;  // a fixed slice of the producer: the linear form handles it
+                continue;
+            }
+            if (needs_clamp(v, i)) e = "clampi(" + e + ", 0, " + S(v.in_shape.dims[i] - 1) + ")";
+            args->push_back("(" + e + ")");
+            f->names.push_back("axis" + to_string(i));
+            f->coefs.push_back(st[i]);
+            f->extents.push_back(v.in_shape.dims[i]);
+        }
+        if (args->empty()) return false;
+        f->valid = true;
+        return true;
+    }
+
     // Expression for the element of source `s` that view `v` selects at coordinates `coord`.
     string load_view(const Source& s, const dsc_view& v, const std::vector<string>& coord) {
         if (s.buffer >= 0) return "b" + to_string(s.buffer) + "[" + index_expr(v, coord) + "]";
         IndexForm form = index_form(v, coord);
         if (!form.valid) {
+            // a padded (clamped) view: one argument per axis of the producer, the clamp applied here, so that a
+            // coordinate that is a constant at the call stays one inside the producer
+            IndexForm per_axis;
+            std::vector<string> args;
+            if (axis_form(v, coord, &per_axis, &args)) {
+                const string fn = instantiate(s.virt, per_axis);
+                string list;
+                for (auto& a : args) list += a + ", ";
+                return fn + "(" + list + params_pass() + ")";
+            }
             const string fn = instantiate(s.virt, IndexForm{});
             return fn + "(" + index_expr(v, coord) + ", " + params_pass() + ")";
         }
@@ -382,7 +420,7 @@ string entry_name(const FusedKernel& fk) {
     if (!fk.row_stages.empty()) return "dsc_row_fused_m" + count(fk.row_m) + "_n" + count(fk.row_n) + "_s" + count((int64_t)fk.row_stages.size());
     switch (d.kind) {
     case DSC_KERNEL_FILL: return "dsc_fill_n" + count(d.shape.dims[0]);
-    case DSC_KERNEL_PER_ELEMENT: return "dsc_per_element_n" + count(d.shape.dims[0]);
+    case DSC_KERNEL_PER_ELEMENT: return "dsc_per_element_n" + count(d.shape.dims[0]) + (fk.row_width ? "_rows" + count(fk.row_width) : string());
     case DSC_KERNEL_REDUCE: {
         return string(fk.has_epilogue ? "dsc_reduce_epilogue_k" : "dsc_reduce_k") + count(d.inputs[0].out_shape.dims[d.axis]) + "_n" +
                count(element_count(d.shape));
@@ -522,9 +560,77 @@ string gen_fill(Emitter& em, Generated* out) {
     return "";
 }
 
+}  // namespace
+
+int64_t column_partition_width(const dsc_kernel_desc& d) {
+    if (d.kind != DSC_KERNEL_PER_ELEMENT) return 0;
+    for (int i = 0; i < d.n_ops; ++i) {
+        const dsc_pe_op& op = d.ops[i];
+        if (op.kind != DSC_PE_SELECT || op.op != DSC_CMP_GT) continue;
+        const dsc_pe_op& lhs = d.ops[op.args[0]];
+        const dsc_pe_op& rhs = d.ops[op.args[1]];
+        if (lhs.kind != DSC_PE_COORD || (rhs.kind != DSC_PE_LITERAL_F32 && rhs.kind != DSC_PE_LITERAL_U32)) continue;
+        const dsc_view& v = d.builtin_views[lhs.view_index];
+        const int last = v.out_shape.rank - 1;
+        if (last < 1 || element_count(v.out_shape) != d.shape.dims[0]) continue;
+        int64_t base = 0, coef[DSC_MAX_DIM];
+        if (!affine_form(v, &base, coef) || coef[last] == 0) continue;
+        bool only_last = true;
+        for (int a = 0; a < last; ++a)
+            if (coef[a] != 0 && v.out_shape.dims[a] > 1) only_last = false;
+        const int64_t w = v.out_shape.dims[last];
+        if (only_last && w >= 2 && w <= 64) return w;
+    }
+    return 0;
+}
+
+namespace {
+// One thread per row of a [rows, w] per-element kernel (see FusedKernel::row_width).
+string gen_per_element_rows(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const int64_t n = d.shape.dims[0], W = fk.row_width;
+    if (W < 2 || W > 64 || n % W != 0 || column_partition_width(d) != W) return "per-element rows: not a column partition of this width";
+    const int64_t rows = n / W;
+    if (rows >= kMaxIndex) return "per-element rows: too many rows";
+    std::ostringstream k;
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
+    k << "    const int dsc_row = (int)(blockIdx.x * 256u + threadIdx.x);\n";
+    k << "    if (dsc_row >= " << S(rows) << ") return;\n";
+    for (int o = 0; o < d.n_outputs; ++o) k << "    float o" << o << "[" << S(W) << "];\n";
+    for (int64_t c = 0; c < W; ++c) {
+        k << "    {\n    const int dsc_col = " << S(c) << ";\n";
+        IndexForm form;
+        form.valid = true;
+        form.names = {"dsc_row", "dsc_col"};
+        form.coefs = {W, 1};
+        form.extents = {rows, W};
+        em.emit_pe(k, d, fk.inputs, "(uint)(dsc_row * " + S(W) + " + dsc_col)", "", {}, &form);
+        for (int o = 0; o < d.n_outputs; ++o) k << "    o" << o << "[" << S(c) << "] = t" << d.outputs[o] << ";\n";
+        k << "    }\n";
+    }
+    for (int o = 0; o < d.n_outputs; ++o) {
+        k << "    float* const row" << o << " = b" << fk.outputs[o] << " + (size_t)dsc_row * " << S(W) << ";\n";
+        if (W % 4 == 0) {
+            for (int64_t c = 0; c < W; c += 4)
+                k << "    *(float4*)(row" << o << " + " << S(c) << ") = make_float4(o" << o << "[" << S(c) << "], o" << o << "[" << S(c + 1) << "], o" << o << "["
+                  << S(c + 2) << "], o" << o << "[" << S(c + 3) << "]);\n";
+        } else {
+            for (int64_t c = 0; c < W; ++c) k << "    row" << o << "[" << S(c) << "] = o" << o << "[" << S(c) << "];\n";
+        }
+    }
+    k << "}\n";
+    out->grid = blocks_for(rows, 256);
+    out->block = 256;
+    out->source = k.str();
+    out->note = "per-element: a thread per row of " + S(W) + " columns, the column a constant of each evaluation";
+    return "";
+}
+
 string gen_per_element(Emitter& em, Generated* out) {
     const FusedKernel& fk = em.fk;
     const dsc_kernel_desc& d = fk.main.raw();
+    if (fk.row_width) return gen_per_element_rows(em, out);
     const int64_t n = d.shape.dims[0];
     const int vec = (n % 4 == 0 && n >= 4096) ? 4 : 1;
     std::ostringstream k;
@@ -2651,6 +2757,7 @@ std::string FusedKernel::key() const {
     }
     s += sum_chunks ? "|S1" : "|S0";
     if (out_slice_width) s += "|OSW" + to_string((long long)out_slice_width);
+    if (row_width) s += "|RW" + to_string((long long)row_width);
     if (as_part) s += "|AP";
     if (colsum_out >= 0) s += "|CS" + to_string(colsum_out);
     s += "|O";

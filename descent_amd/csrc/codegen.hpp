@@ -140,6 +140,10 @@ struct FusedKernel {
     // stored slice by slice, [n / w][m][w], so that a reader of one slice walks consecutive memory instead of w
     // floats out of every row.  The readers' views are rewritten to that layout by the planner.
     int64_t out_slice_width = 0;
+    // A per-element kernel over [rows, w] whose value is chosen by comparing the column with literals (a chain of
+    // concats): w > 0 makes a thread evaluate one whole row with the column a constant of each of its w evaluations,
+    // so the compiler keeps, per column, only the branch that column takes.
+    int64_t row_width = 0;
     bool sum_chunks = false;               // MatMul: ignore the descriptor's chunk count, write one full sum
     int colsum_out = -1;                   // MatMul (MFMA template): buffer that takes the column sums of B per k chunk
     bool as_part = false;                  // generated as one part of a multi-part launch (set while the launch is generated)
@@ -197,6 +201,8 @@ bool scatter_chain_binned(int64_t table_elements, int64_t total_values);
 BinnedScatterPlan binned_scatter_plan(int64_t table_elements, int64_t total_values, bool pairs = false);
 // Whether a ScatterAdd adds rows of two values that share an index (accumulator [entries, 2], axis 0).
 bool scatter_rows_of_two(const dsc_kernel_desc& d);
+// Width of the last axis if the per-element kernel selects by comparing that axis' coordinate with a literal, else 0.
+int64_t column_partition_width(const dsc_kernel_desc& d);
 
 // Whether a kernel can be one part of a multi-part launch (256 threads per workgroup, addressed by blockIdx.x only).
 bool can_be_part(const FusedKernel& k);

@@ -1687,6 +1687,22 @@ struct Planner {
         }
     }
 
+    // Pass 1i: per-element clusters over [rows, w] that pick their value by comparing the column with literals (each
+    // concat of the reference is one: select(column > n - 1, pad(b), pad(a))) are marked to run a thread per row,
+    // the column a constant of each of the row's w evaluations.  A chain of concats inlined into the last one then
+    // costs each column only the branch it takes, not one load per link.
+    void column_partitions() {
+        if (const char* e = std::getenv("DSC_ROW_PARTITIONS"))
+            if (e[0] == '0') return;
+        for (Draft& d : drafts) {
+            if (!d.alive || !d.fk.parts.empty() || !d.fk.row_stages.empty() || d.fk.has_epilogue || !d.fk.virtuals.empty()) continue;
+            const dsc_kernel_desc& pd = d.fk.main.raw();
+            if (pd.kind != DSC_KERNEL_PER_ELEMENT) continue;
+            const int64_t w = column_partition_width(pd);
+            if (w && pd.shape.dims[0] / w >= 16384) d.fk.row_width = w;
+        }
+    }
+
     // Pass 1h: a per-element cluster that reads nothing but small arrays (all of its inputs together fit the L2 of
     // one XCD: the coordinates of a mini-batch) and writes large ones is evaluated again by each of its readers, and
     // its outputs are neither written nor read back.  The hashed corner indices and bilinear weights of a grid level
@@ -1788,9 +1804,13 @@ struct Planner {
                 if ((!is_pe && !is_red) || p.keep_output) continue;
                 const int node = p.outs[0].node;
                 if (is_graph_output[node] || p.outs[0].copy_from >= 0) continue;
-                if (is_pe && !is_cheap_producer(pd)) continue;
                 auto cons = consumers_of(node);
                 if (cons.empty()) continue;
+                // A reader that evaluates whole rows with the column a constant (see column_partitions) runs, per
+                // column, only the producers that column selects: there a producer need not be light (a gather of
+                // four table entries), and the chain of producers may be as long as the row is wide.
+                const bool into_rows = is_pe && cons.size() == 1 && drafts[cons[0]].fk.row_width > 0 && drafts[cons[0]].fk.main.raw().kind == DSC_KERNEL_PER_ELEMENT;
+                if (is_pe && !into_rows && (!is_cheap_producer(pd) || p.fk.virtuals.size() > 8)) continue;
                 if (is_pe && cons.size() > 1 && !is_pure_copy(pd)) continue;
                 bool ok = true;
                 if (is_pe && !fuse_into_matmul)
@@ -1819,7 +1839,7 @@ struct Planner {
                     for (auto& o : q.outs)
                         if (o.copy_from == node) ok = false;  // updated in place by the consumer
                     if (taken_in_place_between(i, ci, input_nodes(p))) ok = false;
-                    if ((int)q.fk.virtuals.size() + (int)p.fk.virtuals.size() + 1 > 8) ok = false;
+                    if ((int)q.fk.virtuals.size() + (int)p.fk.virtuals.size() + 1 > (into_rows ? 512 : 8)) ok = false;
                     if (!q.fk.row_stages.empty()) ok = false;
                     // a MatMul that sums its B operand's columns on the side took over the operand's other reader: the
                     // operand stays a buffer, as it was when two launches read it
@@ -2433,6 +2453,7 @@ struct Planner {
         disjoint_windows_to_copies();           // pass 1g
         row_kernels();                          // pass 1b
         recompute_from_small_inputs();          // pass 1h
+        column_partitions();                    // pass 1i
         inline_producers();                     // pass 2
         attach_epilogues();                     // pass 3
         slice_major_products();                 // pass 3d

@@ -157,6 +157,39 @@ def test_direct_lds_tiles_over_k_chunks_and_batches(hip_backend_session, case):
         assert "chunks 4" in listing, listing
 
 
+@pytest.mark.parametrize("rows", [16384, 40000])
+def test_concat_chain_with_gathers_as_one_row_kernel(hip_backend_session, rows):
+    """Four pieces of different widths joined by three concats, one of them gathered from a table through indices
+    computed from a small array, another scaled: one launch that evaluates a row per thread.  Bit-exact against the
+    oracle (nothing is summed)."""
+    genv, cenv = _envs(hip_backend_session)
+
+    def run(env):
+        rng = np.random.default_rng(rows)
+        a = env.static_parameter_with_data([rows, 2], "a", rng.standard_normal(rows * 2, dtype=np.float32))
+        t = env.static_parameter_with_data([1000, 3], "t", rng.standard_normal(3000, dtype=np.float32))
+        i = env.static_parameter_with_data([rows], "i", rng.integers(0, 5000, rows).astype(np.float32))
+        c = env.static_parameter_with_data([rows, 2], "c", rng.standard_normal(rows * 2, dtype=np.float32))
+        d = env.static_parameter_with_data([rows, 5], "d", rng.standard_normal(rows * 5, dtype=np.float32))
+        out = env.static_parameter([rows, 12], "out")
+
+        def build(s):
+            index = (s.parameter_value(i).into_u32() * 7) % 1000
+            gathered = s.parameter_value(t).gather(-2, index)
+            joined = (s.parameter_value(a) * 2.0).concat(gathered, -1).concat(s.parameter_value(c) + 1.0, -1).concat(s.parameter_value(d), -1)
+            s.write_parameter_value(out, joined)
+
+        graph = env.build_graph(build)
+        env.run(graph, 0)
+        return env.read_parameter(out), graph
+
+    got, graph = run(genv)
+    want, _ = run(cenv)
+    assert np.array_equal(got, want)
+    listing = next(iter(graph.__dict__["_schedules"].values())).describe()
+    assert int(listing.split()[0]) == 1 and "a thread per row of 12 columns" in listing, listing
+
+
 @pytest.mark.parametrize("mode", ["fused", "unfused", "kernel_by_kernel"])
 def test_convnet_train_steps_vs_oracle(hip_backend_session, mode):
     """Three Adam steps of the ConvNet at batch 16: every parameter, optimiser state and the loss/accuracy sums."""

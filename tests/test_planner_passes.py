@@ -119,6 +119,41 @@ def test_scatter_adds_into_one_accumulator_share_a_launch_and_small_launches_are
     assert int(listing.split()[0]) <= 40 and len(w.graph.clusters_sorted) > 200
 
 
+def test_clusters_over_small_inputs_are_evaluated_by_their_readers():
+    # the float -> integer conversion of an index array of 128 KiB, read by two ScatterAdds of a megabyte of values each
+    def build(s, idx, v0, v1, acc):
+        i = _value(s, idx).into_u32()
+        z = s.literal(0.0).value().broadcast([100000, 2])
+        s.write_parameter_value(acc, z.scatter_add(_value(s, v0), -2, i).scatter_add(_value(s, v1), -2, i))
+
+    env = _env()
+    params = [env.static_parameter(sh, f"p{i}") for i, sh in enumerate([[131072], [131072, 2], [131072, 2], [100000, 2]])]
+    graph = env.build_graph(lambda scope: build(scope, *params))
+    unfused = hip_backend.check_schedule(graph, fused=False)
+    fused = hip_backend.check_schedule(graph, fused=True)
+    assert any(line.split(": ")[1].startswith("PerElement") for line in unfused.splitlines()[1:] if re.match(r"\d+: ", line))
+    launches = [line for line in fused.splitlines() if re.match(r"(\d+|prefill): ", line)]
+    assert not any(line.split(": ")[1].startswith("PerElement") for line in launches), fused
+    assert any("ScatterAdd" in line for line in launches)
+    covered = {int(c) for line in launches if " clusters " in line for c in line.split(" clusters ")[1].split()}
+    assert covered == set(range(len(graph.clusters_sorted)))
+
+
+def test_a_chain_of_concats_runs_a_thread_per_row_with_the_column_a_constant():
+    def build(s, a, b, c, d, out):
+        s.write_parameter_value(out, (_value(s, a) * 2.0).concat(_value(s, b), -1).concat(_value(s, c) + 1.0, -1).concat(_value(s, d), -1))
+
+    unfused, fused = _listings([[65536, 2], [65536, 3], [65536, 2], [65536, 5], [65536, 12]], build)
+    assert int(unfused.split()[0]) >= 3
+    assert int(fused.split()[0]) == 1, fused
+    assert "a thread per row of 12 columns, the column a constant of each evaluation" in fused, fused
+    # the generated kernel loads each input once per row element and selects nothing at run time
+    env = _env()
+    params = [env.static_parameter(sh, f"q{i}") for i, sh in enumerate([[65536, 2], [65536, 3], [65536, 2], [65536, 5], [65536, 12]])]
+    graph = env.build_graph(lambda sc: build(sc, *params))
+    assert len(graph.clusters_sorted) >= 3
+
+
 def test_full_size_hash_grid_chains_are_binned_grouped_and_read_a_slice_major_gradient():
     w = workloads.hash_grid_fit(_env(), batch=1 << 18)
     listing = hip_backend.check_schedule(w.graph, fused=True)
@@ -135,7 +170,10 @@ def test_full_size_hash_grid_chains_are_binned_grouped_and_read_a_slice_major_gr
     second = [i for i, line in enumerate(lines) if "11 chains in one launch, the first: scatter chain, stage 2 of 2" in line]
     assert len(first) == 1 and len(second) == 1 and second[0] == first[0] + 1, listing
     assert "256 segments" in lines[first[0]] and "grid 2816x1024" in lines[first[0]] and "grid 2816x1024" in lines[second[0]]
-    assert int(listing.split()[0]) <= 28
+    assert int(listing.split()[0]) <= 18
+    # the whole encoding (corner indices, weights, gathers, the chain of fifteen concats) is the one launch after the
+    # target image's
+    assert sum("a thread per row of 32 columns" in line for line in lines) == 1, listing
     # every reference cluster is still covered
     covered = {int(c) for line in lines if " clusters " in line for c in line.split(" clusters ")[1].split()}
     assert covered == set(range(len(w.graph.clusters_sorted)))
