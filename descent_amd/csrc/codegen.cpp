@@ -2435,7 +2435,7 @@ string gen_matmul(Emitter& em, Generated* out) {
     if (dot_kernel_applies(fk, g)) return gen_matmul_dot(em, out);
     MmPlan plan;
     if (!plan_mfma(fk, g, &plan, fk.as_part)) return "matmul: invalid tile configuration";
-    const MmConfig c = plan.c;
+    MmConfig c = plan.c;
     const int64_t kchunks = plan.kchunks, chunk_k = plan.chunk_k;
     if (fk.as_part && 64 * c.wm * c.wn != 256) return "matmul: a part of a multi-part launch runs 256 threads";
 
@@ -2458,6 +2458,34 @@ string gen_matmul(Emitter& em, Generated* out) {
     k << "#define MM_B " << S(g.batch) << "\n#define MM_M " << S(g.m) << "\n#define MM_N " << S(g.n) << "\n#define MM_K "
       << S(g.k) << "\n";
     k << "#define MM_KCHUNKS " << S(kchunks) << "\n#define MM_CHUNK_K " << S(chunk_k) << "\n";
+    // k-tiles straight from memory into LDS (see MM_DIRECT in the template) wherever a product consists of whole tiles.
+    // Measured on MI355X with two tile buffers against the pass through registers (TFLOP/s): 1024^3 (64x64x64 tiles)
+    // 64.9 -> 78.4, 2048^3 (128x128x16) 92.0 -> 101.2, 2048x4096x1024 101.6 -> 107.2 and 4096x2048x4096 116.5 -> 120.1
+    // (256x128x16), 262144x256x256 101.9 -> 103.5, 4096^3 131.9 -> 131.9, 8192^3 138.2 -> 138.6 (256x256x16).  A third
+    // buffer (two tiles requested ahead) measured 1-2 % below two.
+    // DSC_MM_DIRECT_LDS=0 switches the path off, =2 / =3 choose the number of buffers.
+    auto direct_buffers = [&](const MmConfig& t) {
+        const char* e = std::getenv("DSC_MM_DIRECT_LDS");
+        const int nt = 64 * t.wm * t.wn;
+        const int nbuf = !e ? 2 : e[0] == '2' ? 2 : e[0] == '3' ? 3 : 0;
+        const bool whole = g.m % t.bm == 0 && g.n % t.bn == 0 && chunk_k % t.bk == 0 && g.k % chunk_k == 0;
+        const bool even = (t.bm * t.bk / 4) % nt == 0 && (t.bn * t.bk / 4) % nt == 0 && (t.bk & (t.bk - 1)) == 0;
+        if (nbuf && a_mode && b_mode && fk.colsum_out < 0 && whole && even && chunk_k / t.bk >= nbuf &&
+            (int64_t)nbuf * (t.bm + t.bn) * t.bk * 4 <= 160 * 1024)
+            return nbuf;
+        return 0;
+    };
+    // Without padding two buffers of a 32-deep 256x256 tile are 128 KiB: half the barriers per product.  8192^3
+    // 137.9 -> 144.2 TFLOP/s (91.7 % of peak), 4096^3 131.8 -> 135.4, 262144x256x256 101.9 -> 103.6; eight waves on
+    // the same tile 142.7, the 256x128 and 128x128 tiles gained nothing from 32-deep steps.
+    // (a unit of two 32-deep tiles lost: 262144x256x64 124 us against 117.5, so k ranges under 128 keep 16-deep steps)
+    if (c.bm == 256 && c.bn == 256 && c.bk == 16 && c.wm * c.wn == 16 && chunk_k >= 128 && !std::getenv("DSC_MM_TILE")) {
+        MmConfig deep = c;
+        deep.bk = 32;
+        deep.group_m = 8;
+        if (direct_buffers(deep) == 2) c = deep;
+    }
+    const int direct = direct_buffers(c);
     k << "#define BM " << c.bm << "\n#define BN " << c.bn << "\n#define BK " << c.bk << "\n#define WAVES_M " << c.wm
       << "\n#define WAVES_N " << c.wn << "\n#define GROUP_M " << c.group_m << "\n";
     k << "#define A_MODE " << a_mode << "\n#define B_MODE " << b_mode << "\n";
@@ -2490,23 +2518,6 @@ string gen_matmul(Emitter& em, Generated* out) {
         k << "#define MM_COLSUM 0\n";
     }
 
-    // k-tiles straight from memory into LDS (see MM_DIRECT in the template) wherever a product consists of whole tiles.
-    // Measured on MI355X with two tile buffers against the pass through registers (TFLOP/s): 1024^3 (64x64x64 tiles)
-    // 64.9 -> 78.4, 2048^3 (128x128x16) 92.0 -> 101.2, 2048x4096x1024 101.6 -> 107.2 and 4096x2048x4096 116.5 -> 120.1
-    // (256x128x16), 262144x256x256 101.9 -> 103.5, 4096^3 131.9 -> 131.9, 8192^3 138.2 -> 138.6 (256x256x16).  A third
-    // buffer (two tiles requested ahead) measured 1-2 % below two.
-    // DSC_MM_DIRECT_LDS=0 switches the path off, =2 / =3 choose the number of buffers.
-    int direct = 0;
-    {
-        const char* e = std::getenv("DSC_MM_DIRECT_LDS");
-        const int nt = 64 * c.wm * c.wn;
-        const int nbuf = !e ? 2 : e[0] == '2' ? 2 : e[0] == '3' ? 3 : 0;
-        const bool whole = g.m % c.bm == 0 && g.n % c.bn == 0 && chunk_k % c.bk == 0 && g.k % chunk_k == 0;
-        const bool even = (c.bm * c.bk / 4) % nt == 0 && (c.bn * c.bk / 4) % nt == 0 && (c.bk & (c.bk - 1)) == 0;
-        if (nbuf && a_mode && b_mode && fk.colsum_out < 0 && whole && even && chunk_k / c.bk >= nbuf &&
-            (int64_t)nbuf * (c.bm + c.bn) * c.bk * 4 <= 160 * 1024)
-            direct = nbuf;
-    }
     k << "#define MM_DIRECT " << direct << "\n";
 
     // results leave through LDS as 16-byte row pieces when the output allows it

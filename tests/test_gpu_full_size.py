@@ -96,7 +96,7 @@ def test_matmul_8192_cubed_sampled_rows_and_columns(hip_backend_session):
     """The launch bench.py times: 64 sampled rows (every tile column) and 64 sampled columns (every tile row)."""
     n = 8192
     listing, a, b, bias, c = _matmul_case(hip_backend_session, n, n, n, 7)
-    assert "mfma 32x32x2 tile 256x256x16" in listing and int(listing.split()[0]) == 1, listing
+    assert "mfma 32x32x2 tile 256x256x32" in listing and "tiles straight into LDS x2" in listing and int(listing.split()[0]) == 1, listing
     rng = np.random.default_rng(0)
     rows = rng.choice(n, 64, replace=False)
     cols = rng.choice(n, 64, replace=False)

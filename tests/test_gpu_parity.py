@@ -82,11 +82,11 @@ def test_matmul_transposed_operands(hip_backend_session, ta, tb, m, n, k):
 @pytest.mark.parametrize("m,n,k,tile,buffers", [
     (256, 256, 64, "32x32x16", None), (1024, 512, 128, "64x32x16", None), (1024, 1024, 128, "64x64x16", None),
     (1024, 1024, 1024, "64x64x64", None), (2048, 1024, 128, "128x64x16", None), (2048, 2048, 64, "128x128x16", None),
-    (2048, 2048, 64, "128x128x16", "3"), (4096, 2048, 64, "256x128x16", "2"), (4096, 4096, 64, "256x256x16", "2"),
-    (4096, 4096, 48, "256x256x16", "3"),
+    (2048, 2048, 64, "128x128x16", "3"), (4096, 2048, 64, "256x128x16", "2"), (4096, 4096, 128, "256x256x32", "2"),
+    (4096, 4096, 48, "256x256x16", "3"), (4096, 4096, 160, "256x256x32", None),
     # more tiles than workgroups: a workgroup's stream of k-tiles runs on into its next unit
     (2048, 3072, 64, "128x128x16", None), (2048, 3072, 64, "128x128x16", "3"), (1024, 1536, 512, "64x64x64", None),
-    (1024, 1536, 512, "64x64x64", "3"), (8192, 4096, 48, "256x256x16", "3"),
+    (1024, 1536, 512, "64x64x64", "3"), (8192, 4096, 48, "256x256x16", "3"), (8192, 8192, 128, "256x256x32", None), (4096, 4096, 64, "256x256x16", None),
 ])
 def test_matmul_tiles_loaded_straight_into_lds(hip_backend_session, monkeypatch, m, n, k, tile, buffers, ta, tb):
     """Whole-tile products take their k-tiles from memory straight into LDS: every tile shape, both operand
