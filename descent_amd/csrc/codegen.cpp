@@ -2785,6 +2785,8 @@ std::string FusedKernel::key() const {
 namespace {
 string generate_multi(const FusedKernel& fk, Generated* out);
 string generate_scatter_chain(const FusedKernel& fk, Generated* out);
+// threads of a first-stage workgroup; measured on the hash grid's eleven binned levels: 1024 88.8 us, 512 82.0, 256 85.9
+int scatter_bin_threads() { return 512; }
 string generate_scatter_bin(const FusedKernel& fk, Generated* out);
 string generate_scatter_sum(const FusedKernel& fk, Generated* out);
 string generate_chain_group(const FusedKernel& fk, Generated* out);
@@ -2999,8 +3001,11 @@ string generate_scatter_bin(const FusedKernel& fk, Generated* out) {
     const BinnedScatterPlan bp = binned_scatter_plan(table, total, pairs);
     if (bp.nseg > 1024 || bp.nseg * bp.cap >= ((int64_t)1 << 31) || table >= ((int64_t)1 << 31)) return "binned scatter: accumulator too large";
     if (bp.nseg != 256) return "binned scatter: the kernels take 256 segments";
-    const int U = pairs ? 4 : 8;          // records per thread: 8192 values per workgroup either way
-    const int64_t per_wg = 1024 * U;      // records per workgroup
+    // 8192 values per workgroup (runs of 16 records per segment on average) on 512 threads: a workgroup waits for
+    // the round trip of its reservations, and three of these fit a CU where two of 1024 threads did
+    const int NTH = scatter_bin_threads();
+    const int U = (pairs ? 4096 : 8192) / NTH;  // records per thread
+    const int64_t per_wg = (int64_t)NTH * U;     // records per workgroup
     const int rec = fk.outputs[0], cur = fk.outputs[1], acc = fk.outputs[2];
     Generated g;
     std::ostringstream src, fetches;
@@ -3023,7 +3028,7 @@ string generate_scatter_bin(const FusedKernel& fk, Generated* out) {
         fetches << "    " << (i ? "else " : "") << "if (" << block_id << " < " << S(first_wg + wgs) << "u) {\n";
         fetches << "        const uint g0 = (" << block_id << " - " << S(first_wg) << "u) * " << S(per_wg) << "u + tid;\n";
         for (int u = 0; u < U; ++u) {
-            const string r = "min(g0 + " + S(u * 1024) + "u, " + S(nrec - 1) + "u)";
+            const string r = "min(g0 + " + S(u * NTH) + "u, " + S(nrec - 1) + "u)";
             if (pairs) {
                 fetches << "        { int a_second; bool k_second;\n";
                 fetches << "        part" << i << "::fetch(2u * " << r << ", &v" << u << ", &a" << u << ", &k" << u;
@@ -3037,7 +3042,7 @@ string generate_scatter_bin(const FusedKernel& fk, Generated* out) {
                 for (int j : fk.part_params[i]) fetches << ", b" << j;
                 fetches << ", rand_seed);\n";
             }
-            fetches << "        k" << u << " = k" << u << " && g0 + " << S(u * 1024) << "u < " << S(nrec) << "u;\n";
+            fetches << "        k" << u << " = k" << u << " && g0 + " << S(u * NTH) << "u < " << S(nrec) << "u;\n";
         }
         fetches << "    }\n";
         first_wg += wgs;
@@ -3055,7 +3060,7 @@ string generate_scatter_bin(const FusedKernel& fk, Generated* out) {
         src << "    uint* const lbase = cnt + " << S(bp.nseg) << ";\n    uint* const gbase = lbase + " << S(bp.nseg) << ";\n    uint* const wsum = gbase + " << S(bp.nseg) << ";\n";
         if (pairs) src << "    int* const stage_at = reinterpret_cast<int*>(wsum + 16);\n";
     } else {
-        src << "extern \"C\" __global__ __launch_bounds__(1024) void " << g.entry << "(" << em.kernel_params_decl() << ") {\n";
+        src << "extern \"C\" __global__ __launch_bounds__(" << NTH << ") void " << g.entry << "(" << em.kernel_params_decl() << ") {\n";
         src << "    __shared__ uint cnt[" << S(bp.nseg) << "], lbase[" << S(bp.nseg) << "], gbase[" << S(bp.nseg) << "], wsum[16];\n";
         src << "    __shared__ float2 stage[" << S(per_wg) << "];\n";
         if (pairs) src << "    __shared__ int stage_at[" << S(per_wg) << "];\n";
@@ -3063,18 +3068,19 @@ string generate_scatter_bin(const FusedKernel& fk, Generated* out) {
     g.lds_bytes = (size_t)(per_wg * (pairs ? 12 : 8) + (3 * bp.nseg + 16) * 4);
     src << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
     src << "    const uint tid = threadIdx.x;\n";
-    src << "    for (uint i = tid; i < " << S(bp.nseg) << "u; i += 1024u) cnt[i] = 0u;\n    __syncthreads();\n";
+    src << "    for (uint i = tid; i < " << S(bp.nseg) << "u; i += " << NTH << "u) cnt[i] = 0u;\n    __syncthreads();\n";
     for (int u = 0; u < U; ++u) src << "    float v" << u << " = 0.f, w" << u << " = 0.f; int a" << u << " = 0; bool k" << u << " = false;\n";
     src << fetches.str();
     src << "    __builtin_amdgcn_sched_barrier(0);\n";
     for (int u = 0; u < U; ++u) src << "    const uint r" << u << " = k" << u << " ? atomicAdd(&cnt[(a" << u << " >> 4) & 255], 1u) : 0u;\n";
     src << "    __syncthreads();\n";
+    if (NTH < bp.nseg) return "binned scatter: fewer threads than segments";
     src << "    const uint c = tid < " << S(bp.nseg) << "u ? cnt[tid] : 0u;\n";
     src << "    uint incl = c;\n";
     src << "#pragma unroll\n    for (int d = 1; d < 64; d <<= 1) {\n        const uint up = __shfl_up(incl, d);\n        if ((int)(tid & 63u) >= d) incl += up;\n    }\n";
     src << "    if ((tid & 63u) == 63u) wsum[tid >> 6] = incl;\n    __syncthreads();\n";
     src << "    uint before = 0u, filled = 0u;\n";
-    src << "#pragma unroll\n    for (uint w = 0; w < 16u; ++w) {\n        const uint s = wsum[w];\n        if (w < (tid >> 6)) before += s;\n        filled += s;\n    }\n";
+    src << "#pragma unroll\n    for (uint w = 0; w < " << NTH / 64 << "u; ++w) {\n        const uint s = wsum[w];\n        if (w < (tid >> 6)) before += s;\n        filled += s;\n    }\n";
     src << "    uint* const cursor = reinterpret_cast<uint*>(b" << cur << ");\n";
     src << "    if (tid < " << S(bp.nseg) << "u) {\n        lbase[tid] = before + incl - c;\n        gbase[tid] = c ? atomicAdd(&cursor[tid * 16u], c) : 0u;\n    }\n";
     src << "    __syncthreads();\n";
@@ -3086,7 +3092,7 @@ string generate_scatter_bin(const FusedKernel& fk, Generated* out) {
         src << "    __syncthreads();\n";
         src << "    float2* const records = reinterpret_cast<float2*>(b" << rec << ");\n";
         src << "    int* const targets = reinterpret_cast<int*>(b" << rec << ") + " << S(2 * bp.nseg * bp.cap) << ";\n";
-        src << "    for (uint slot = tid; slot < filled; slot += 1024u) {\n";
+        src << "    for (uint slot = tid; slot < filled; slot += " << NTH << "u) {\n";
         src << "        const float2 r = stage[slot];\n        const int a = stage_at[slot];\n        const uint bin = ((uint)a >> 4) & 255u;\n";
         src << "        const uint pos = gbase[bin] + (slot - lbase[bin]);\n";
         src << "        if (pos < " << S(bp.cap) << "u) { records[bin * " << S(bp.cap) << "u + pos] = r; targets[bin * " << S(bp.cap) << "u + pos] = a; }\n";
@@ -3096,7 +3102,7 @@ string generate_scatter_bin(const FusedKernel& fk, Generated* out) {
         src << "    if (k" << u << ") stage[lbase[(a" << u << " >> 4) & 255] + r" << u << "] = make_float2(__int_as_float(a" << u << "), v" << u << ");\n";
     src << "    __syncthreads();\n";
     src << "    float2* const records = reinterpret_cast<float2*>(b" << rec << ");\n";
-    src << "    for (uint slot = tid; slot < filled; slot += 1024u) {\n";
+    src << "    for (uint slot = tid; slot < filled; slot += " << NTH << "u) {\n";
     src << "        const float2 r = stage[slot];\n        const int a = __float_as_int(r.x);\n        const uint bin = ((uint)a >> 4) & 255u;\n";
     src << "        const uint pos = gbase[bin] + (slot - lbase[bin]);\n";
     src << "        if (pos < " << S(bp.cap) << "u) records[bin * " << S(bp.cap) << "u + pos] = r;\n";
@@ -3104,7 +3110,7 @@ string generate_scatter_bin(const FusedKernel& fk, Generated* out) {
     }
     g.source = src.str();
     g.grid = (unsigned)first_wg;
-    g.block = 1024;
+    g.block = NTH;
     g.n_buffers = fk.n_buffers;
     g.note = "scatter chain, stage 1 of 2: " + to_string(fk.parts.size()) + " links, " + (pairs ? "(target, two values)" : "(target, value)") + " records ordered by segment in LDS (" + S(bp.nseg) +
              " segments of " + S(bp.seg) + " floats, the accumulator's 64-byte lines dealt to them in turn), written in runs into bins of " + S(bp.cap) + " records";
@@ -3200,7 +3206,8 @@ string generate_chain_group(const FusedKernel& fk, Generated* out) {
         Generated pg;
         string err = generate(part, &pg);
         if (!err.empty()) return err;
-        if (pg.block != 1024 || pg.lds_bytes == 0) return "chain group: unexpected part form";
+        if ((pg.block != 1024 && pg.block != 512 && pg.block != 256) || pg.lds_bytes == 0 || (i && pg.block != g.block)) return "chain group: unexpected part form";
+        g.block = pg.block;
         if ((int)fk.part_params[i].size() != part.n_buffers) return "chain group: part parameter count";
         src << "namespace chain" << i << " {\n" << pg.source << "}  // namespace chain" << i << "\n\n";
         body << "    if (blockIdx.x < " << first + pg.grid << "u) { chain" << i << "::part_entry(blockIdx.x - " << first << "u, dsc_lds";
@@ -3214,12 +3221,11 @@ string generate_chain_group(const FusedKernel& fk, Generated* out) {
     Emitter em(fk);
     g.entry = string(fk.parts[0].binned_stage == 1 ? "dsc_scatter_bin" : fk.parts[0].binned_stage == 2 ? "dsc_scatter_sum" : "dsc_scatter_chain") + "_group" +
               to_string(fk.parts.size()) + "_g" + to_string(first);
-    src << "extern \"C\" __global__ __launch_bounds__(1024) void " << g.entry << "(" << em.kernel_params_decl() << ") {\n";
+    src << "extern \"C\" __global__ __launch_bounds__(" << g.block << ") void " << g.entry << "(" << em.kernel_params_decl() << ") {\n";
     src << "    __shared__ __attribute__((aligned(16))) char dsc_lds[" << lds << "];\n";
     src << body.str() << "}\n";
     g.source = src.str();
     g.grid = first;
-    g.block = 1024;
     g.n_buffers = fk.n_buffers;
     g.note = to_string(fk.parts.size()) + " chains in one launch, the first: " + kinds;
     *out = g;

@@ -169,7 +169,7 @@ def test_full_size_hash_grid_chains_are_binned_grouped_and_read_a_slice_major_gr
     first = [i for i, line in enumerate(lines) if "11 chains in one launch, the first: scatter chain, stage 1 of 2" in line]
     second = [i for i, line in enumerate(lines) if "11 chains in one launch, the first: scatter chain, stage 2 of 2" in line]
     assert len(first) == 1 and len(second) == 1 and second[0] == first[0] + 1, listing
-    assert "256 segments" in lines[first[0]] and "grid 2816x1024" in lines[first[0]] and "grid 2816x1024" in lines[second[0]]
+    assert "256 segments" in lines[first[0]] and "grid 2816x512" in lines[first[0]] and "grid 2816x1024" in lines[second[0]]
     assert int(listing.split()[0]) <= 18
     # the whole encoding (corner indices, weights, gathers, the chain of fifteen concats) is the one launch after the
     # target image's
