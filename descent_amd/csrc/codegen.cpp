@@ -1859,24 +1859,36 @@ bool config_ok(const MmConfig& c) {
     return acc <= 256;
 }
 
-// Largest tile whose grid still fills the 256 CUs; small products fall back to small tiles so that more
-// workgroups exist (they are latency bound, not MFMA bound).  Measured on MI355X at 8192^3: 256x256x16 with
-// 16 waves 137 TFLOP/s, 256x128x16 with 8 waves 134, 128x128x16 with 4 waves 127.
+// The tile shape with the best predicted rate: how evenly its tiles deal out over the 256 CUs (the CU with the most
+// tiles sets the time: 288 tiles of 256x128 on 3072^3 ran at 74.8 TFLOP/s, 2304 tiles of 64x64 at 105.4) times what
+// the shape reaches on a CU, which grows with the number of tiles a CU works through (co-resident workgroups cover one
+// another's barriers and first loads).  The two rates per shape are measurements on MI355X, TFLOP/s with exactly one
+// tile per CU and with many: 256x256 144 / 144 (one workgroup fills a CU), 256x128 125 / 137, 128x128 108 / 134,
+// 128x64 93 / 127, 64x64 78 / 117, 64x32 36 / 78, 32x32 30 / 77.  The prediction was within 5 % of the measurement on 2560^3, 3072^3, 5120^3 and
+// 6144^3 for every shape (20 cases) and picks the fastest measured shape on each.
 MmConfig pick_config(int64_t M, int64_t N, int64_t K /* per chunk */, int64_t groups /* batch * k-chunks */) {
-    static const MmConfig candidates[] = {
-        {256, 256, 16, 4, 4, 4}, {256, 128, 16, 4, 2, 4}, {128, 128, 16, 2, 2, 8}, {128, 64, 16, 2, 2, 8},
-        {64, 64, 16, 2, 2, 8},   {64, 32, 16, 2, 1, 8},   {32, 32, 16, 1, 1, 8},
+    struct Rated { MmConfig c; double one, many; };
+    static const Rated candidates[] = {
+        {{256, 256, 16, 4, 4, 4}, 144, 144}, {{256, 128, 16, 4, 2, 4}, 125, 137}, {{128, 128, 16, 2, 2, 8}, 108, 134}, {{128, 64, 16, 2, 2, 8}, 93, 127},
+        {{64, 64, 16, 2, 2, 8}, 78, 117},    {{64, 32, 16, 2, 1, 8}, 36, 78},     {{32, 32, 16, 1, 1, 8}, 30, 77},
     };
     auto tiles = [&](const MmConfig& c) { return ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn) * groups; };
-    MmConfig best = candidates[6];
-    bool found = false;
-    for (const MmConfig& c : candidates) {
+    MmConfig best = candidates[6].c;
+    double best_rate = -1.0;
+    for (const Rated& r : candidates) {
+        const MmConfig& c = r.c;
         // do not pad an extent to more than twice its size
         if (c.bm > 32 && M * 2 <= c.bm) continue;
         if (c.bn > 32 && N * 2 <= c.bn) continue;
-        if (!found) { best = c; found = true; }
-        if (tiles(c) >= 256) { best = c; break; }
-        if (tiles(c) > tiles(best)) best = c;
+        const int64_t t = tiles(c), rounds = (t + 255) / 256;
+        const double fill = (double)t / (double)(rounds * 256);
+        // the work inside the padded tiles that is real
+        const double real = ((double)M * (double)N) / ((double)((M + c.bm - 1) / c.bm * c.bm) * (double)((N + c.bn - 1) / c.bn * c.bn));
+        const double rate = fill * real * (r.many - (r.many - r.one) / (double)rounds);
+        if (rate > best_rate * 1.02) {  // a smaller tile has to win by more than the model's noise
+            best_rate = rate;
+            best = c;
+        }
     }
     MmConfig c = best;
     // narrow outputs: keep all four waves along m
@@ -2479,10 +2491,12 @@ string gen_matmul(Emitter& em, Generated* out) {
     // 137.9 -> 144.2 TFLOP/s (91.7 % of peak), 4096^3 131.8 -> 135.4, 262144x256x256 101.9 -> 103.6; eight waves on
     // the same tile 142.7, the 256x128 and 128x128 tiles gained nothing from 32-deep steps.
     // (a unit of two 32-deep tiles lost: 262144x256x64 124 us against 117.5, so k ranges under 128 keep 16-deep steps)
-    if (c.bm == 256 && c.bn == 256 && c.bk == 16 && c.wm * c.wn == 16 && chunk_k >= 128 && !std::getenv("DSC_MM_TILE")) {
+    // The smaller tiles gain from 32-deep steps as well: 128x128 on 2048^3 100.6 -> 106-108, 256x128 on 4096x2048x4096
+    // 121.7 -> 124.5, 128x64 on 3072^3 97.2 -> 103.4 and on 2048x1024x2048 84.8 -> 92.6.
+    if (c.bm * c.bn >= 128 * 64 && c.bk == 16 && chunk_k >= 128 && !std::getenv("DSC_MM_TILE")) {
         MmConfig deep = c;
         deep.bk = 32;
-        deep.group_m = 8;
+        if (c.bm == 256 && c.bn == 256) deep.group_m = 8;
         if (direct_buffers(deep) == 2) c = deep;
     }
     const int direct = direct_buffers(c);

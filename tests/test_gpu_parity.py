@@ -79,16 +79,18 @@ def test_matmul_transposed_operands(hip_backend_session, ta, tb, m, n, k):
 
 
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
-@pytest.mark.parametrize("m,n,k,tile,buffers", [
-    (256, 256, 64, "32x32x16", None), (1024, 512, 128, "64x32x16", None), (1024, 1024, 128, "64x64x16", None),
-    (1024, 1024, 1024, "64x64x64", None), (2048, 1024, 128, "128x64x16", None), (2048, 2048, 64, "128x128x16", None),
-    (2048, 2048, 64, "128x128x16", "3"), (4096, 2048, 64, "256x128x16", "2"), (4096, 4096, 128, "256x256x32", "2"),
-    (4096, 4096, 48, "256x256x16", "3"), (4096, 4096, 160, "256x256x32", None),
+@pytest.mark.parametrize("m,n,k,tile,buffers,force", [
+    (256, 256, 64, "32x32x16", None, None), (1024, 512, 128, "64x32x16", None, "64,32,16,2,1,8"), (1024, 1024, 128, "64x64x16", None, None),
+    (1024, 1024, 1024, "64x64x64", None, None), (2048, 1024, 128, "128x64x16", None, "128,64,16,2,2,8"), (2048, 2048, 64, "128x128x16", None, None),
+    (2048, 2048, 64, "128x128x16", "3", None), (4096, 2048, 64, "256x128x16", "2", None), (4096, 4096, 128, "256x256x32", "2", None),
+    (4096, 4096, 48, "256x256x16", "3", None), (4096, 4096, 160, "256x256x32", None, None), (2048, 2048, 256, "128x128x32", None, None),
+    (4096, 1024, 256, "128x64x32", None, "128,64,32,2,2,8"), (4096, 2048, 128, "256x128x32", None, None),
     # more tiles than workgroups: a workgroup's stream of k-tiles runs on into its next unit
-    (2048, 3072, 64, "128x128x16", None), (2048, 3072, 64, "128x128x16", "3"), (1024, 1536, 512, "64x64x64", None),
-    (1024, 1536, 512, "64x64x64", "3"), (8192, 4096, 48, "256x256x16", "3"), (8192, 8192, 128, "256x256x32", None), (4096, 4096, 64, "256x256x16", None),
+    (2048, 3072, 64, "128x64x16", None, None), (2048, 3072, 64, "128x64x16", "3", None), (1024, 1536, 512, "64x64x64", None, None),
+    (1024, 1536, 512, "64x64x64", "3", None), (8192, 4096, 48, "256x256x16", "3", None), (8192, 8192, 128, "256x256x32", None, None),
+    (4096, 4096, 64, "256x256x16", None, None),
 ])
-def test_matmul_tiles_loaded_straight_into_lds(hip_backend_session, monkeypatch, m, n, k, tile, buffers, ta, tb):
+def test_matmul_tiles_loaded_straight_into_lds(hip_backend_session, monkeypatch, m, n, k, tile, buffers, force, ta, tb):
     """Whole-tile products take their k-tiles from memory straight into LDS: every tile shape, both operand
     layouts on either side, two and three tile buffers, against the oracle."""
     from descent_amd import hip_backend
@@ -97,6 +99,10 @@ def test_matmul_tiles_loaded_straight_into_lds(hip_backend_session, monkeypatch,
         monkeypatch.delenv("DSC_MM_DIRECT_LDS", raising=False)
     else:
         monkeypatch.setenv("DSC_MM_DIRECT_LDS", buffers)  # read when a kernel is generated; part of the kernel cache key
+    if force is None:
+        monkeypatch.delenv("DSC_MM_TILE", raising=False)
+    else:
+        monkeypatch.setenv("DSC_MM_TILE", force)  # a tile shape the choice by predicted rate does not take for this product
     genv, cenv = _envs(hip_backend_session)
     got = _transposed_case(genv, np.random.default_rng(m + k), m, n, k, ta, tb)
     want = _transposed_case(cenv, np.random.default_rng(m + k), m, n, k, ta, tb)
