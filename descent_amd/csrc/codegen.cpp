@@ -2480,7 +2480,9 @@ string gen_matmul(Emitter& em, Generated* out) {
         const char* e = std::getenv("DSC_MM_DIRECT_LDS");
         const int nt = 64 * t.wm * t.wn;
         const int nbuf = !e ? 2 : e[0] == '2' ? 2 : e[0] == '3' ? 3 : 0;
-        const bool whole = g.m % t.bm == 0 && g.n % t.bn == 0 && chunk_k % t.bk == 0 && g.k % chunk_k == 0;
+        // every k range whole k-tiles; a tile may reach past M or N (it repeats the last row / the last four columns),
+        // as long as the product is at least one piece wide and tall
+        const bool whole = chunk_k % t.bk == 0 && g.k % chunk_k == 0 && g.m >= 4 && g.n >= 4;
         const bool even = (t.bm * t.bk / 4) % nt == 0 && (t.bn * t.bk / 4) % nt == 0 && (t.bk & (t.bk - 1)) == 0;
         if (nbuf && a_mode && b_mode && fk.colsum_out < 0 && whole && even && chunk_k / t.bk >= nbuf &&
             (int64_t)nbuf * (t.bm + t.bn) * t.bk * 4 <= 160 * 1024)

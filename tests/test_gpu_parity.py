@@ -89,6 +89,9 @@ def test_matmul_transposed_operands(hip_backend_session, ta, tb, m, n, k):
     (2048, 3072, 64, "128x64x16", None, None), (2048, 3072, 64, "128x64x16", "3", None), (1024, 1536, 512, "64x64x64", None, None),
     (1024, 1536, 512, "64x64x64", "3", None), (8192, 4096, 48, "256x256x16", "3", None), (8192, 8192, 128, "256x256x32", None, None),
     (4096, 4096, 64, "256x256x16", None, None),
+    # tiles that reach past M or N repeat the last row / the last four columns and store only what exists
+    (1000, 1000, 512, "64x64x64", None, None), (1000, 1000, 512, "64x64x64", "3", None), (2500, 1100, 128, "128x128x32", None, "128,128,32,2,2,8"),
+    (5000, 3000, 128, "256x256x32", None, "256,256,32,4,4,8"), (4100, 2052, 64, "256x128x16", None, "256,128,16,4,2,4"), (36, 20, 64, "32x32x16", None, None),
 ])
 def test_matmul_tiles_loaded_straight_into_lds(hip_backend_session, monkeypatch, m, n, k, tile, buffers, force, ta, tb):
     """Whole-tile products take their k-tiles from memory straight into LDS: every tile shape, both operand
