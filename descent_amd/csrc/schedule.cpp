@@ -1714,24 +1714,29 @@ struct Planner {
         const size_t kInputLimit = (size_t)4 << 20, kOutputFloor = (size_t)256 << 10;
         for (int i = 0; i < (int)drafts.size(); ++i) {
             Draft& p = drafts[i];
-            if (!p.alive || !p.fk.parts.empty() || !p.fk.row_stages.empty() || !p.fk.virtuals.empty() || p.fk.has_epilogue || p.keep_output) continue;
+            if (!p.alive || !p.fk.parts.empty() || !p.fk.row_stages.empty() || p.fk.has_epilogue || p.keep_output) continue;
+            if (p.fk.row_width) continue;  // a link of a concat chain: pass 2 inlines it into the chain's row kernel
             const dsc_kernel_desc& pd = p.fk.main.raw();
-            if (pd.kind != DSC_KERNEL_PER_ELEMENT || pd.n_ops > 40) continue;
-            bool plain = true;
-            for (int o = 0; o < pd.n_ops && plain; ++o) {
-                const dsc_pe_op& op = pd.ops[o];
-                if (op.kind == DSC_PE_GATHER || op.kind == DSC_PE_RAND) plain = false;
-                if (op.kind == DSC_PE_UNARY && (op.op == DSC_UN_SQRT || op.op == DSC_UN_EXP || op.op == DSC_UN_LOG || op.op == DSC_UN_SIN || op.op == DSC_UN_COS)) plain = false;
-                if (op.kind == DSC_PE_BINARY && (op.op == DSC_BIN_POW || op.op == DSC_BIN_DIV)) plain = false;
-            }
+            if (pd.kind != DSC_KERNEL_PER_ELEMENT) continue;
+            // the cluster and whatever was already inlined into it (an earlier cluster of this kind)
+            auto is_plain = [](const dsc_kernel_desc& d) {
+                if (d.kind != DSC_KERNEL_PER_ELEMENT || d.n_ops > 40) return false;
+                for (int o = 0; o < d.n_ops; ++o) {
+                    const dsc_pe_op& op = d.ops[o];
+                    if (op.kind == DSC_PE_GATHER || op.kind == DSC_PE_RAND) return false;
+                    if (op.kind == DSC_PE_UNARY && (op.op == DSC_UN_SQRT || op.op == DSC_UN_EXP || op.op == DSC_UN_LOG || op.op == DSC_UN_SIN || op.op == DSC_UN_COS)) return false;
+                    if (op.kind == DSC_PE_BINARY && (op.op == DSC_BIN_POW || op.op == DSC_BIN_DIV)) return false;
+                }
+                return true;
+            };
+            bool plain = is_plain(pd) && p.fk.virtuals.size() <= 8;
+            for (auto& v : p.fk.virtuals) plain = plain && is_plain(v.pe.raw());
             if (!plain) continue;
             size_t in_bytes = 0;
             bool ok = true;
-            for (auto& src : p.fk.inputs) {
-                if (src.buffer < 0) { ok = false; break; }
-                in_bytes += node_bytes[p.params[src.buffer]];
-            }
-            if (!ok || p.fk.inputs.empty() || in_bytes > kInputLimit) continue;
+            const std::vector<int> p_inputs = input_nodes(p);
+            for (int node : p_inputs) in_bytes += node_bytes[node];
+            if (p_inputs.empty() || in_bytes > kInputLimit) continue;
             std::set<int> readers;
             for (auto& out : p.outs) {
                 if (is_graph_output[out.node] || out.copy_from >= 0 || node_bytes[out.node] < kOutputFloor) { ok = false; break; }
@@ -1743,7 +1748,7 @@ struct Planner {
                 const int qk = q.fk.main.raw().kind;
                 if (ci <= i || !q.fk.parts.empty() || !q.fk.row_stages.empty() || q.fk.dgrad.on || q.fk.cfwd.on || q.fk.pool.on) ok = false;
                 if (qk != DSC_KERNEL_PER_ELEMENT && qk != DSC_KERNEL_REDUCE && qk != DSC_KERNEL_SCATTER_ADD) ok = false;
-                if ((int)q.fk.virtuals.size() + (int)p.outs.size() > 12) ok = false;
+                if ((int)q.fk.virtuals.size() + (int)p.fk.virtuals.size() + (int)p.outs.size() > 24) ok = false;
                 for (auto& o : q.outs)
                     for (auto& out : p.outs)
                         if (o.copy_from == out.node) ok = false;  // updated in place by the reader
@@ -1757,6 +1762,7 @@ struct Planner {
             if (!ok) continue;
             for (int ci : readers) {
                 Draft& q = drafts[ci];
+                const int voff = import_virtuals(q, p);
                 for (size_t o = 0; o < p.outs.size(); ++o) {
                     const int node = p.outs[o].node;
                     bool reads = false;
@@ -1768,7 +1774,7 @@ struct Planner {
                     Virtual nv;
                     nv.pe = p.fk.main;
                     nv.out_op = pd.outputs[o];
-                    for (auto& src : p.fk.inputs) nv.inputs.push_back(import_source(q, p, src, 0));
+                    for (auto& src : p.fk.inputs) nv.inputs.push_back(import_source(q, p, src, voff));
                     q.fk.virtuals.push_back(nv);
                     for_each_source(q.fk, [&](Source& src) {
                         if (src.buffer >= 0 && q.params[src.buffer] == node && !q.fk.buffer_is_output[src.buffer]) {
@@ -2452,8 +2458,8 @@ struct Planner {
         conv_backward();                        // pass 1e
         disjoint_windows_to_copies();           // pass 1g
         row_kernels();                          // pass 1b
-        recompute_from_small_inputs();          // pass 1h
         column_partitions();                    // pass 1i
+        recompute_from_small_inputs();          // pass 1h
         inline_producers();                     // pass 2
         attach_epilogues();                     // pass 3
         slice_major_products();                 // pass 3d

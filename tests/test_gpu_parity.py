@@ -346,6 +346,29 @@ def test_hash_grid_steps_vs_oracle(hip_backend_session):
         assert err <= 1e-3, f"{key}: rel L2 {err}"
 
 
+def test_hash_grid_steps_vs_oracle_with_the_encoding_as_one_kernel(hip_backend_session):
+    """Config 5 at a size where the planner's large-array passes apply: the corner indices and weights are evaluated
+    by their readers (outputs of 256 KiB), the chain of concats and gathers is one row kernel (65536 rows), the
+    hashed levels' ScatterAdd chains go through binned records of rows of two.  Same bound as the smaller case."""
+    from descent_amd import workloads
+
+    genv, cenv = _envs(hip_backend_session)
+    kw = dict(batch=1 << 16, levels=(16, 40, 100, 300), entry_count=1 << 14, hidden=(32,), seed=23)
+    gw = workloads.hash_grid_fit(genv, **kw)
+    cw = workloads.hash_grid_fit(cenv, **kw)
+    for step in range(2):
+        genv.run(gw.graph, step)
+        cenv.run(cw.graph, step)
+    listing = next(iter(gw.graph.__dict__["_schedules"].values())).describe()
+    assert "a thread per row of 8 columns" in listing, listing
+    assert "(target, two values) records" in listing, listing
+    assert not any(line.split(": ")[1].startswith("PerElement (20 ops)") for line in listing.splitlines() if ": " in line), listing
+    got, want = gw.snapshot(), cw.snapshot()
+    for key in want:
+        err = rel_l2(got[key], want[key])
+        assert err <= 1e-3, f"{key}: rel L2 {err}"
+
+
 def test_gather_indices_are_bit_exact(hip_backend_session):
     """The hash index arithmetic (u32 xor / mul / rem on bit-cast floats) and the gathered values must match
     the oracle bit for bit."""
