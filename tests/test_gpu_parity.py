@@ -166,8 +166,8 @@ def test_direct_lds_tiles_over_k_chunks_and_batches(hip_backend_session, case):
         assert "chunks 4" in listing, listing
 
 
-@pytest.mark.parametrize("rows", [16384, 40000])
-def test_concat_chain_with_gathers_as_one_row_kernel(hip_backend_session, rows):
+@pytest.mark.parametrize("rows,with_last", [(16384, True), (40000, True), (20000, False)])
+def test_concat_chain_with_gathers_as_one_row_kernel(hip_backend_session, rows, with_last):
     """Four pieces of different widths joined by three concats, one of them gathered from a table through indices
     computed from a small array, another scaled: one launch that evaluates a row per thread.  Bit-exact against the
     oracle (nothing is summed)."""
@@ -180,12 +180,15 @@ def test_concat_chain_with_gathers_as_one_row_kernel(hip_backend_session, rows):
         i = env.static_parameter_with_data([rows], "i", rng.integers(0, 5000, rows).astype(np.float32))
         c = env.static_parameter_with_data([rows, 2], "c", rng.standard_normal(rows * 2, dtype=np.float32))
         d = env.static_parameter_with_data([rows, 5], "d", rng.standard_normal(rows * 5, dtype=np.float32))
-        out = env.static_parameter([rows, 12], "out")
+        width = 12 if with_last else 7  # 7: rows that are not whole 16-byte pieces
+        out = env.static_parameter([rows, width], "out")
 
         def build(s):
             index = (s.parameter_value(i).into_u32() * 7) % 1000
             gathered = s.parameter_value(t).gather(-2, index)
-            joined = (s.parameter_value(a) * 2.0).concat(gathered, -1).concat(s.parameter_value(c) + 1.0, -1).concat(s.parameter_value(d), -1)
+            joined = (s.parameter_value(a) * 2.0).concat(gathered, -1).concat(s.parameter_value(c) + 1.0, -1)
+            if with_last:
+                joined = joined.concat(s.parameter_value(d), -1)
             s.write_parameter_value(out, joined)
 
         graph = env.build_graph(build)
@@ -196,7 +199,7 @@ def test_concat_chain_with_gathers_as_one_row_kernel(hip_backend_session, rows):
     want, _ = run(cenv)
     assert np.array_equal(got, want)
     listing = next(iter(graph.__dict__["_schedules"].values())).describe()
-    assert int(listing.split()[0]) == 1 and "a thread per row of 12 columns" in listing, listing
+    assert int(listing.split()[0]) == 1 and "a thread per row of %d columns" % (12 if with_last else 7) in listing, listing
 
 
 @pytest.mark.parametrize("mode", ["fused", "unfused", "kernel_by_kernel"])
