@@ -2552,8 +2552,8 @@ string gen_matmul(Emitter& em, Generated* out) {
             if (e[0] == '0') vec_store = false;
     }
     k << "#define MM_VEC_STORE " << (vec_store ? 1 : 0) << "\n";
+    bool long_epilogue = false;
     {
-        bool long_epilogue = false;
         if (fk.has_epilogue) {
             const dsc_kernel_desc& pe = fk.epilogue.raw();
             for (int o = 0; o < pe.n_ops; ++o) {
@@ -2597,9 +2597,81 @@ string gen_matmul(Emitter& em, Generated* out) {
         em.funcs << one.str() << four.str();
         k << "#define MM_STORE(v, idx, b, m, n) mm_store(v, idx, b, m, n, " << em.params_pass() << ")\n";
         k << "#define MM_STORE4(v, idx, b, m, n) mm_store4(v, idx, b, m, n, " << em.params_pass() << ")\n";
+        // Operands of the epilogue that the 16-byte store path can request ahead of the staging rounds (each round's
+        // own load would wait on vmcnt(0), i.e. also for the previous round's store to be acknowledged): a
+        // per-column operand (a bias: the view reads element base + column) once per block column, a per-element
+        // operand (an activation the gradient is masked with: an identity view) one block ahead.
+        std::vector<int> pre_col, pre_elem;
+        std::vector<int64_t> pre_col_base;
+        if (direct && vec_store && !long_epilogue) {
+            for (int i = 0; i < pe.n_inputs; ++i) {
+                if (i == fk.epilogue_product_input || fk.epilogue_inputs[i].buffer < 0) continue;
+                const dsc_view& v = pe.inputs[i];
+                int loads = 0;
+                for (int o = 0; o < pe.n_ops; ++o)
+                    if (pe.ops[o].kind == DSC_PE_LOAD && pe.ops[o].input_index == i) ++loads;
+                    else if (pe.ops[o].kind == DSC_PE_GATHER && pe.ops[o].input_index == i) loads = -100;
+                if (loads < 1) continue;
+                int64_t base = 0, coef[DSC_MAX_DIM];
+                if (is_identity(v) && element_count(v.out_shape) == g.batch * g.m * g.n) {
+                    if (pre_elem.size() < 2) pre_elem.push_back(i);
+                    continue;
+                }
+                const int last = v.out_shape.rank - 1;
+                if (last < 0 || !affine_form(v, &base, coef) || v.out_shape.dims[last] != g.n || coef[last] != 1 || base % 4 != 0) continue;
+                bool column_only = element_count(v.out_shape) == g.batch * g.m * g.n;
+                for (int ax = 0; ax < last; ++ax)
+                    if (v.out_shape.dims[ax] > 1 && coef[ax] != 0) column_only = false;
+                if (column_only && pre_col.size() < 2) {
+                    pre_col.push_back(i);
+                    pre_col_base.push_back(base);
+                }
+            }
+        }
+        if (!pre_col.empty() || !pre_elem.empty()) {
+            std::ostringstream pb, fn;
+            std::map<int, string> pov;
+            pov[fk.epilogue_product_input] = "product";
+            string scalars, scalar_args[4];
+            for (size_t q = 0; q < pre_col.size(); ++q) {
+                pov[pre_col[q]] = "pc" + to_string(q);
+                scalars += "float pc" + to_string(q) + ", ";
+            }
+            for (size_t q = 0; q < pre_elem.size(); ++q) {
+                pov[pre_elem[q]] = "pe" + to_string(q);
+                scalars += "float pe" + to_string(q) + ", ";
+            }
+            em.emit_pe(pb, pe, fk.epilogue_inputs, "gid", "e", pov, &form);
+            for (int o = 0; o < pe.n_outputs; ++o) pb << "    result[" << o << "] = et" << pe.outputs[o] << ";\n";
+            em.funcs << "DSC_INLINE void mm_epilogue_pre(float product, int gid, int cb, int cm, int cn, float* result, " << scalars << em.params_decl() << ") {\n"
+                     << pb.str() << "}\n";
+            fn << "DSC_INLINE void mm_store4_pre(float4 p, int gid, int cb, int cm, int cn, const float4* colv, const float4* elv, " << em.params_decl() << ") {\n";
+            fn << "    const float pv[4] = {p.x, p.y, p.z, p.w};\n    float res[4][" << pe.n_outputs << "];\n";
+            for (size_t q = 0; q < pre_col.size(); ++q) fn << "    const float c" << q << "[4] = {colv[" << q << "].x, colv[" << q << "].y, colv[" << q << "].z, colv[" << q << "].w};\n";
+            for (size_t q = 0; q < pre_elem.size(); ++q) fn << "    const float e" << q << "[4] = {elv[" << q << "].x, elv[" << q << "].y, elv[" << q << "].z, elv[" << q << "].w};\n";
+            fn << "#pragma unroll\n    for (int j = 0; j < 4; ++j) mm_epilogue_pre(pv[j], gid + j, cb, cm, cn + j, res[j], ";
+            for (size_t q = 0; q < pre_col.size(); ++q) fn << "c" << q << "[j], ";
+            for (size_t q = 0; q < pre_elem.size(); ++q) fn << "e" << q << "[j], ";
+            fn << em.params_pass() << ");\n";
+            for (int o = 0; o < pe.n_outputs; ++o)
+                fn << "    *(float4*)(b" << fk.outputs[o] << " + gid) = make_float4(res[0][" << o << "], res[1][" << o << "], res[2][" << o
+                   << "], res[3][" << o << "]);\n";
+            fn << "}\n";
+            em.funcs << fn.str();
+            k << "#define MM_NPRE_COL " << pre_col.size() << "\n#define MM_NPRE_ELEM " << pre_elem.size() << "\n";
+            k << "#define MM_LOAD_COL4(dst, cn) {";
+            for (size_t q = 0; q < pre_col.size(); ++q)
+                k << " (dst)[" << q << "] = *(const float4*)(b" << fk.epilogue_inputs[pre_col[q]].buffer << " + " << S(pre_col_base[q]) << " + (cn));";
+            k << " }\n#define MM_LOAD_ELEM4(dst, gid) {";
+            for (size_t q = 0; q < pre_elem.size(); ++q) k << " (dst)[" << q << "] = *(const float4*)(b" << fk.epilogue_inputs[pre_elem[q]].buffer << " + (gid));";
+            k << " }\n#define MM_STORE4P(v, idx, b, m, n, colv, elv) mm_store4_pre(v, idx, b, m, n, colv, elv, " << em.params_pass() << ")\n";
+        } else {
+            k << "#define MM_NPRE_COL 0\n#define MM_NPRE_ELEM 0\n";
+        }
     } else {
         k << "#define MM_STORE(v, idx, b, m, n) b" << fk.outputs[0] << "[idx] = (v)\n";
         k << "#define MM_STORE4(v, idx, b, m, n) *(float4*)(b" << fk.outputs[0] << " + (idx)) = (v)\n";
+        k << "#define MM_NPRE_COL 0\n#define MM_NPRE_ELEM 0\n";
     }
     k << kMatmulMfmaSource;
 
