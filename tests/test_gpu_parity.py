@@ -124,6 +124,35 @@ def test_matmul_tiles_loaded_straight_into_lds(hip_backend_session, monkeypatch,
     assert f"tiles straight into LDS x{buffers or 2}" in listing, listing
 
 
+@pytest.mark.parametrize("m,n,k", [(2048, 1024, 128), (1000, 520, 256), (4096, 4096, 64), (300, 36, 64)])
+def test_matmul_epilogue_with_a_per_element_and_a_per_column_operand(hip_backend_session, m, n, k):
+    """The store path requests the epilogue's own operands ahead of its staging rounds: a bias (per column) and a mask
+    (per element), on whole and on ragged products, against the oracle."""
+    genv, cenv = _envs(hip_backend_session)
+
+    def run(env):
+        rng = np.random.default_rng(m + n)
+        a = env.static_parameter_with_data([m, k], "a", rng.standard_normal(m * k, dtype=np.float32))
+        b = env.static_parameter_with_data([k, n], "b", rng.standard_normal(k * n, dtype=np.float32))
+        bias = env.static_parameter_with_data([n], "bias", rng.standard_normal(n, dtype=np.float32))
+        mask = env.static_parameter_with_data([m, n], "mask", rng.standard_normal(m * n, dtype=np.float32))
+        c = env.static_parameter([m, n], "c")
+
+        def build(s):
+            z = s.parameter_value(a).matmul(s.parameter_value(b)) + s.parameter_value(bias)
+            s.write_parameter_value(c, s.parameter_value(mask).select_gt(0.0, z, z * 0.01))
+
+        graph = env.build_graph(build)
+        env.run(graph, 0)
+        return env.read_parameter(c), graph
+
+    got, graph = run(genv)
+    want, _ = run(cenv)
+    assert rel_l2(got, want) <= TOL
+    listing = next(iter(graph.__dict__["_schedules"].values())).describe()
+    assert int(listing.split()[0]) == 1 and "+epilogue" in listing and "tiles straight into LDS" in listing, listing
+
+
 @pytest.mark.parametrize("case", ["k-chunks", "batches", "rows-mode", "batches-transposed"])
 def test_direct_lds_tiles_over_k_chunks_and_batches(hip_backend_session, case):
     """The same path where a unit is a (k-chunk, batch, tile) triple: the reference's 1024-deep k-chunks written as
