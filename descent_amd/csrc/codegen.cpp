@@ -1002,7 +1002,22 @@ string gen_row_fused(Emitter& em, Generated* out) {
     const FusedKernel& fk = em.fk;
     const int64_t m = fk.row_m, n = fk.row_n;
     if (m < 1 || n < 2 || n > 64) return "row-fused: bad row shape";
-    const int64_t G = pow2_ceil(n), per_block = 256 / G;
+    int64_t G = pow2_ceil(n);
+    // A MatMul as stage 0: the lanes of a row share its k range as in the dot-product kernel (B in LDS, blocks of four k
+    // per lane, a shuffle butterfly), after which lane `col` keeps the sum of its column.
+    const bool mm0 = !fk.row_stages.empty() && fk.row_stages[0].k.raw().kind == DSC_KERNEL_MATMUL;
+    int64_t K = 0, kblocks = 0, J = 0;
+    if (mm0) {
+        const MatMulDims g = matmul_dims(fk.row_stages[0].k.raw());
+        if (g.batch != 1 || g.chunks != 1 || g.m != m || g.n != n || g.k * g.n > 8192) return "row-fused: the MatMul stage does not match the rows";
+        K = g.k;
+        kblocks = (K + 3) / 4;
+        int64_t L = 4;
+        while (L < 64 && L * 2 < kblocks) L *= 2;
+        G = std::max(G, L);
+        J = (kblocks + G - 1) / G;
+    }
+    const int64_t per_block = 256 / G;
     std::ostringstream k;
     k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
     k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
@@ -1024,7 +1039,7 @@ string gen_row_fused(Emitter& em, Generated* out) {
     // variable holding output `o` of stage `s`
     auto stage_var = [&](int s_idx, int o) {
         const dsc_kernel_desc& sd = fk.row_stages[s_idx].k.raw();
-        if (sd.kind == DSC_KERNEL_REDUCE) return "s" + to_string(s_idx) + "_r";
+        if (sd.kind == DSC_KERNEL_REDUCE || sd.kind == DSC_KERNEL_MATMUL) return "s" + to_string(s_idx) + "_r";
         return "s" + to_string(s_idx) + "_t" + to_string(sd.outputs[o]);
     };
     auto stage_is_wide = [&](int s_idx) {
@@ -1036,7 +1051,31 @@ string gen_row_fused(Emitter& em, Generated* out) {
         const dsc_kernel_desc& sd = st.k.raw();
         const string pfx = "s" + to_string(si) + "_";
         k << "    // stage " << si << ": " << label_name(sd) << "\n";
-        if (sd.kind == DSC_KERNEL_PER_ELEMENT) {
+        if (sd.kind == DSC_KERNEL_MATMUL) {
+            if (si != 0 || !mm0) return "row-fused: a MatMul can only be the first stage";
+            const string la = em.load_view(st.inputs[0], sd.inputs[0], {"cb", "cm", "ck"});
+            em.funcs << "DSC_INLINE float rows_load_a(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return " << la << ";\n}\n";
+            const string lb = em.load_view(st.inputs[1], sd.inputs[1], {"cb", "ck", "cn"});
+            em.funcs << "DSC_INLINE float rows_load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb << ";\n}\n";
+            k << "    __shared__ float sB[" << S(kblocks * 4 * n) << "];\n";
+            k << "    for (int e = threadIdx.x; e < " << S(kblocks * 4 * n) << "; e += 256) {\n";
+            k << "        const int kk = e / " << S(n) << ", nn = e % " << S(n) << ";\n";
+            k << "        const float v = rows_load_b(0, min(kk, " << S(K - 1) << "), nn, " << em.params_pass() << ");\n";
+            k << "        sB[e] = kk < " << S(K) << " ? v : 0.f;\n    }\n";
+            // every block of the lane requested before anything is used; beyond k the clamped loads meet zeros of B
+            k << "    float mm_a[" << S(J) << "][4];\n";
+            k << "#pragma unroll\n    for (int j = 0; j < " << S(J) << "; ++j)\n#pragma unroll\n        for (int i = 0; i < 4; ++i)\n";
+            k << "            mm_a[j][i] = rows_load_a(0, rowc, min(4 * (col + j * " << S(G) << ") + i, " << S(K - 1) << "), " << em.params_pass() << ");\n";
+            k << "    __syncthreads();\n";
+            k << "    float mm_acc[" << S(n) << "];\n#pragma unroll\n    for (int nn = 0; nn < " << S(n) << "; ++nn) mm_acc[nn] = 0.f;\n";
+            k << "#pragma unroll\n    for (int j = 0; j < " << S(J) << "; ++j) {\n";
+            k << "        const int blk = col + j * " << S(G) << ";\n        if (blk < " << S(kblocks) << ") {\n";
+            k << "#pragma unroll\n            for (int i = 0; i < 4; ++i)\n#pragma unroll\n                for (int nn = 0; nn < " << S(n) << "; ++nn)\n";
+            k << "                    mm_acc[nn] = fmaf(mm_a[j][i], sB[(4 * blk + i) * " << S(n) << " + nn], mm_acc[nn]);\n        }\n    }\n";
+            k << "#pragma unroll\n    for (int nn = 0; nn < " << S(n) << "; ++nn)\n#pragma unroll\n        for (int sft = 1; sft < " << S(G) << "; sft *= 2) mm_acc[nn] += __shfl_xor(mm_acc[nn], sft, 64);\n";
+            k << "    float " << pfx << "r = 0.f;\n#pragma unroll\n    for (int nn = 0; nn < " << S(n) << "; ++nn) if (col == nn) " << pfx << "r = mm_acc[nn];\n";
+            if (st.outputs[0] >= 0) k << "    if (row_ok && col_ok) b" << fk.outputs[st.outputs[0]] << "[row * " << S(n) << " + col] = " << pfx << "r;\n";
+        } else if (sd.kind == DSC_KERNEL_PER_ELEMENT) {
             const bool is_wide = stage_is_wide(si);
             if (!is_wide && sd.shape.dims[0] != m) return "row-fused: per-element stage of the wrong size";
             std::map<int, string> ov;
@@ -1069,7 +1108,7 @@ string gen_row_fused(Emitter& em, Generated* out) {
     out->grid = blocks_for(m, (int)per_block);
     out->block = 256;
     out->source = k.str();
-    out->note = "row-fused: " + S(G) + " lanes per row, " + to_string(fk.row_stages.size()) + " stages";
+    out->note = "row-fused: " + S(G) + " lanes per row, " + to_string(fk.row_stages.size()) + " stages" + (mm0 ? ", the first a MatMul over k=" + S(K) + " shared by the row's lanes" : "");
     return "";
 }
 
@@ -2014,6 +2053,16 @@ bool dot_kernel_applies(const FusedKernel& fk, const MatMulDims& g) {
     return fk.colsum_out < 0 && dot_shape(whole);
 }
 
+}  // namespace
+
+bool matmul_fits_row_stage(const FusedKernel& fk) {
+    const dsc_kernel_desc& d = fk.main.raw();
+    if (d.kind != DSC_KERNEL_MATMUL || d.output_mode != DSC_MATMUL_BATCHES || fk.colsum_out >= 0 || fk.dgrad.on || fk.cfwd.on || fk.out_slice_width) return false;
+    const MatMulDims g = matmul_dims(d);
+    return g.batch == 1 && g.chunks == 1 && g.n >= 2 && dot_kernel_applies(fk, g);
+}
+
+namespace {
 string gen_matmul_dot(Emitter& em, Generated* out) {
     const FusedKernel& fk = em.fk;
     const dsc_kernel_desc& d = fk.main.raw();

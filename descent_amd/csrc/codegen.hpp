@@ -33,7 +33,8 @@ struct Virtual {
 
 // One cluster of a row-fused kernel (see FusedKernel::row_stages).
 struct RowStage {
-    KernelDesc k;                // PerElement over [m, n] or [m] elements, or Reduce of [m, n] along n
+    KernelDesc k;                // PerElement over [m, n] or [m] elements, or Reduce of [m, n] along n, or (stage 0
+                                 // only) the MatMul whose [m, n] product the other stages start from
     std::vector<Source> inputs;  // one per input view of k
     std::vector<int> outputs;    // per output of k: index into FusedKernel::outputs when stored, else -1
 };
@@ -201,6 +202,9 @@ bool scatter_chain_binned(int64_t table_elements, int64_t total_values);
 BinnedScatterPlan binned_scatter_plan(int64_t table_elements, int64_t total_values, bool pairs = false);
 // Whether a ScatterAdd adds rows of two values that share an index (accumulator [entries, 2], axis 0).
 bool scatter_rows_of_two(const dsc_kernel_desc& d);
+// A MatMul small enough to run as the first stage of a row-fused kernel over its [m, n] product: the shape the
+// dot-product kernel takes (few columns, a moderate number of rows, B of a few KB), one batch, no k chunks.
+bool matmul_fits_row_stage(const FusedKernel& fk);
 // Width of the last axis if the per-element kernel selects by comparing that axis' coordinate with a literal, else 0.
 int64_t column_partition_width(const dsc_kernel_desc& d);
 

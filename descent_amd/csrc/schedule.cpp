@@ -1684,7 +1684,119 @@ struct Planner {
             if (fused.fk.outputs.empty()) continue;
             for (int j : members) drafts[j].alive = false;
             drafts[seed] = fused;
+            absorb_matmul_into_rows(seed);
         }
+    }
+
+    // The [m, n] product a row-fused launch starts from (the logits of a classifier head) joins it as its first
+    // stage when it is small enough for the dot-product kernel and has no other reader: one launch less, and the
+    // product never leaves registers.  DSC_FUSE_ROWS_MATMUL=0 keeps the two launches.
+    void absorb_matmul_into_rows(int ri) {
+        if (const char* e = std::getenv("DSC_FUSE_ROWS_MATMUL"))
+            if (e[0] == '0') return;
+        Draft& r = drafts[ri];
+        const int64_t m = r.fk.row_m, n = r.fk.row_n;
+        // the producer of a buffer the stages read
+        int pi = -1;
+        for (auto& st : r.fk.row_stages)
+            for (auto& src : st.inputs) {
+                if (src.buffer < 0) continue;
+                const int node = r.params[src.buffer];
+                for (int j = 0; j < ri; ++j) {
+                    if (!drafts[j].alive || drafts[j].fk.main.raw().kind != DSC_KERNEL_MATMUL) continue;
+                    for (auto& o : drafts[j].outs)
+                        if (o.node == node) pi = j;
+                }
+            }
+        if (pi < 0) return;
+        Draft& p = drafts[pi];
+        if (!p.fk.parts.empty() || !p.fk.row_stages.empty() || !p.fk.virtuals.empty() || p.keep_split || p.keep_output || !matmul_fits_row_stage(p.fk)) return;
+        const MatMulDims g = matmul_dims(p.fk.main.raw());
+        if (g.m != m || g.n != n) return;
+        for (auto& src : p.fk.inputs)
+            if (src.buffer < 0) return;
+        if (p.fk.has_epilogue)
+            for (size_t i = 0; i < p.fk.epilogue_inputs.size(); ++i)
+                if ((int)i != p.fk.epilogue_product_input && p.fk.epilogue_inputs[i].buffer < 0) return;
+        for (auto& o : p.outs) {
+            if (is_graph_output[o.node] || o.copy_from >= 0) return;
+            for (int c : consumers_of(o.node))
+                if (c != ri) return;
+        }
+        if (taken_in_place_between(pi, ri, input_nodes(p))) return;
+        // every stage that reads one of the product's arrays reads it element for element
+        for (auto& st : r.fk.row_stages) {
+            const dsc_kernel_desc& k = st.k.raw();
+            for (int i = 0; i < k.n_inputs; ++i) {
+                if (st.inputs[i].buffer < 0) continue;
+                const int node = r.params[st.inputs[i].buffer];
+                bool from_p = false;
+                for (auto& o : p.outs) from_p = from_p || o.node == node;
+                if (!from_p) continue;
+                const dsc_view& v = k.inputs[i];
+                int64_t base, coef[DSC_MAX_DIM];
+                const bool wide_reader = k.kind == DSC_KERNEL_REDUCE || (k.kind == DSC_KERNEL_PER_ELEMENT && k.shape.dims[0] == m * n);
+                if (!wide_reader || element_count(v.in_shape) != m * n || v.out_shape.rank != 2 || !affine_form(v, &base, coef) || base != 0 || coef[0] != n || coef[1] != 1) return;
+            }
+        }
+        Draft fused;
+        fused.fk.main = r.fk.main;
+        fused.fk.row_m = m;
+        fused.fk.row_n = n;
+        const int shift = p.fk.has_epilogue ? 2 : 1;
+        {
+            RowStage mm;
+            mm.k = p.fk.main;
+            for (auto& src : p.fk.inputs) mm.inputs.push_back(import_source(fused, p, src, 0));
+            mm.outputs.push_back(-1);
+            fused.fk.row_stages.push_back(mm);
+        }
+        if (p.fk.has_epilogue) {
+            RowStage ep;
+            ep.k = p.fk.epilogue;
+            for (size_t i = 0; i < p.fk.epilogue_inputs.size(); ++i) {
+                Source src;
+                if ((int)i == p.fk.epilogue_product_input) src.stage = 0;
+                else src = import_source(fused, p, p.fk.epilogue_inputs[i], 0);
+                ep.inputs.push_back(src);
+            }
+            for (int o = 0; o < p.fk.epilogue.raw().n_outputs; ++o) ep.outputs.push_back(-1);
+            fused.fk.row_stages.push_back(ep);
+        }
+        for (auto& st : r.fk.row_stages) {
+            RowStage ns;
+            ns.k = st.k;
+            for (auto& src : st.inputs) {
+                Source s2;
+                if (src.stage >= 0) {
+                    s2.stage = src.stage + shift;
+                    s2.stage_out = src.stage_out;
+                } else {
+                    const int node = r.params[src.buffer];
+                    int from = -1;
+                    for (size_t o = 0; o < p.outs.size(); ++o)
+                        if (p.outs[o].node == node) from = (int)o;
+                    if (from >= 0) {
+                        s2.stage = shift - 1;  // the epilogue's output `from`, or the product itself
+                        s2.stage_out = from;
+                    } else {
+                        s2.buffer = param_index(fused, node, false);
+                    }
+                }
+                ns.inputs.push_back(s2);
+            }
+            for (int oi : st.outputs) {
+                if (oi < 0) { ns.outputs.push_back(-1); continue; }
+                ns.outputs.push_back((int)fused.fk.outputs.size());
+                fused.fk.outputs.push_back(param_index(fused, r.params[r.fk.outputs[oi]], true));
+                fused.outs.push_back(r.outs[oi]);
+            }
+            fused.fk.row_stages.push_back(ns);
+        }
+        fused.covers = p.covers;
+        fused.covers.insert(fused.covers.end(), r.covers.begin(), r.covers.end());
+        p.alive = false;
+        drafts[ri] = fused;
     }
 
     // Pass 1i: per-element clusters over [rows, w] that pick their value by comparing the column with literals (each

@@ -456,6 +456,44 @@ def _softmax_case(env, m, n, seed, quantised):
     return g, env.read_parameter(loss_rows), env.read_parameter(acc_rows), env.read_parameter(dz)
 
 
+@pytest.mark.parametrize("m,k,n", [(1000, 128, 10), (300, 64, 7), (5000, 200, 16), (65, 33, 3), (1000, 400, 10)])
+def test_classifier_head_product_is_the_first_stage_of_the_row_fused_launch(hip_backend_session, m, k, n):
+    """features x weights + bias -> softmax cross-entropy and accuracy: the small MatMul runs inside the row-fused launch
+    (lanes of a row share its k range); loss rows, accuracy flags and the gradient of the logits against the oracle."""
+    from descent_amd import Initializer
+    from descent_amd.loss import softmax_cross_entropy_accuracy, softmax_cross_entropy_loss
+
+    genv, cenv = _envs(hip_backend_session)
+
+    def run(env):
+        rng = np.random.default_rng(m + k + n)
+        x = env.static_parameter_with_data([m, k], "x", rng.standard_normal(m * k, dtype=np.float32))
+        w = env.trainable_parameter([k, n], "w", Initializer.zero())
+        env.write_parameter(w, rng.standard_normal(k * n, dtype=np.float32) * 0.3)
+        b = env.static_parameter_with_data([n], "b", rng.standard_normal(n, dtype=np.float32))
+        y = env.static_parameter_with_data([m, 1], "y", rng.integers(0, n, (m, 1)).astype(np.float32))
+        loss_rows, acc_rows, dw = env.static_parameter([m, 1], "l"), env.static_parameter([m, 1], "a"), env.static_parameter([k, n], "dw")
+
+        def build(s):
+            wd = s.parameter(w)
+            z = s.parameter(x).next_colour().matmul(wd) + s.parameter(b)
+            loss = softmax_cross_entropy_loss(z, y).set_loss()
+            s.write_parameter_value(loss_rows, loss)
+            s.write_parameter_value(acc_rows, softmax_cross_entropy_accuracy(z, y))
+            s.write_parameter_value(dw, wd.loss_grad())
+
+        g = env.build_graph(build)
+        env.run(g, 0)
+        return g, env.read_parameter(loss_rows), env.read_parameter(acc_rows), env.read_parameter(dw)
+
+    g, gl, ga, gdw = run(genv)
+    _, cl, ca, cdw = run(cenv)
+    listing = next(iter(g.__dict__["_schedules"].values())).describe()
+    assert "the first a MatMul over k=%d shared by the row's lanes" % k in listing, listing
+    assert rel_l2(gl, cl) <= TOL and rel_l2(gdw, cdw) <= TOL
+    assert np.mean(ga != ca) <= 0.002  # a logit pair closer than the two sums' rounding may swap the arg-max
+
+
 @pytest.mark.parametrize("m,n", [(1000, 10), (37, 3), (64, 64), (5, 33), (4097, 2), (300, 17)])
 @pytest.mark.parametrize("quantised", [False, True])
 def test_softmax_cross_entropy_runs_as_one_row_fused_launch(hip_backend_session, m, n, quantised):

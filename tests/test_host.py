@@ -211,8 +211,10 @@ def test_convnet_graph_shape():
     listing = hip_backend.check_schedule(w.graph, fused=True)
     launches = int(listing.split()[0])
     assert launches < 30, listing
-    # softmax cross-entropy and the accuracy count: one row-fused launch over the [1000, 10] logits
-    assert "RowFused [1000, 10] (8 clusters)" in listing
+    # the classifier head (1000 x 128 -> 10), softmax cross-entropy and the accuracy count: one row-fused launch over the
+    # [1000, 10] logits, whose first stage is the MatMul (the lanes of a row share its k range)
+    assert "RowFused [1000, 10] (10 clusters)" in listing
+    assert "10 stages, the first a MatMul over k=128 shared by the row's lanes" in listing
     # small independent launches (optimiser updates of small tensors, short reductions) share launches
     assert listing.count("Multi (") >= 3
     # every reference cluster is covered exactly once, except producers inlined into several consumers
@@ -224,8 +226,10 @@ def test_convnet_graph_shape():
     split = hip_backend.check_schedule(w.graph, fused="split-conv-grads")
     assert "ConvDataGrad" in split and "conv data gradient: workgroup per image and group, tile in LDS, 3x3 taps x 16 channels, border folds fused" in split
     assert "tall-k mfma 16x16x4, 5x1 tiles" in split and "ConvBackward" not in split
-    # the classifier head (1000 x 128 -> 10): lanes share a row's k range, no MFMA tile grid of 32 single-wave workgroups
-    assert "MatMul (k=128) [1, 1, 1000, 10] + PerElement (3 ops) [10000]  [dot products: 16 lanes per row, B in LDS +epilogue]" in listing
+    # on its own the same product is the dot-product kernel: lanes share a row's k range, no MFMA tile grid of 32
+    # single-wave workgroups
+    head = workloads.matmul_epilogue(_env(), 1000, 10, 128, upload=False)
+    assert "[dot products: 16 lanes per row, B in LDS +epilogue]" in hip_backend.check_schedule(head.graph, fused=True)
     # both forward convolutions: the image tile goes to LDS, the im2col copy stays only for the filter gradient
     assert listing.count("ConvForward") == 2
     assert "conv forward: workgroup per image and group, padded image tile in LDS, mfma 16x16x4, 3x3 taps x 8 channels +epilogue" in listing

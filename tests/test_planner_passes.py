@@ -91,7 +91,7 @@ def test_bias_gradient_rides_on_the_weight_gradient_that_reads_the_same_array():
 def test_first_layer_filter_gradient_takes_the_pooling_gradient_as_a_producer():
     graph = workloads.convnet(_env(), batch=1000).graph
     listing = hip_backend.check_schedule(graph, fused=True)
-    assert int(listing.split()[0]) == 12
+    assert int(listing.split()[0]) == 11
     # conv1 needs no data gradient: its filter gradient (and the bias gradient's column sums) run on the convolution
     # backward kernel, bands of 7 output rows; dC is never written -- the max-pool gradient (a WindowsToImage over
     # 2x2 windows that do not overlap, turned into a copy), the selects around it and the activation derivative are
@@ -105,6 +105,23 @@ def test_first_layer_filter_gradient_takes_the_pooling_gradient_as_a_producer():
     # with the switch the second convolution keeps its own two kernels and the first its tall-k product
     split = hip_backend.check_schedule(graph, fused="split-conv-grads")
     assert "ConvFilterGrad" not in split and "ConvBackward" not in split
+
+
+def test_the_product_a_row_fused_launch_starts_from_is_its_first_stage():
+    def build(s, x, w, b, labels, loss):
+        logits = _value(s, x).matmul(_value(s, w)) + _value(s, b)
+        t = logits - logits.reduce_max(-1, True)
+        e = t.exp()
+        p = e / e.reduce_sum(-1, True)
+        s.write_parameter_value(loss, (p * _value(s, labels)).reduce_sum(-1, True))
+
+    unfused, fused = _listings([[1000, 128], [128, 10], [10], [1000, 10], [1000, 1]], build)
+    assert "MatMul (k=128) [1, 1, 1000, 10]" in unfused and int(unfused.split()[0]) >= 4
+    assert int(fused.split()[0]) == 1, fused
+    assert "the first a MatMul over k=128 shared by the row's lanes" in fused, fused
+    # a product too large for that (B would not fit a few KB of LDS per workgroup) keeps its own launch
+    _, big = _listings([[1000, 2048], [2048, 10], [10], [1000, 10], [1000, 1]], build)
+    assert int(big.split()[0]) >= 2 and "the first a MatMul" not in big, big
 
 
 def test_scatter_adds_into_one_accumulator_share_a_launch_and_small_launches_are_grouped():
