@@ -639,13 +639,36 @@ string gen_per_element(Emitter& em, Generated* out) {
     k << "    if (base >= " << S(n) << "u) return;\n";
     std::map<int, string> override_load;
     if (vec == 4) {
-        // identity-view loads of real buffers become one 16-byte load per thread
+        // identity-view loads of real buffers become one 16-byte load per thread; so do the loads through any view
+        // whose innermost output axis walks the innermost input axis one to one in whole groups of four (a bias
+        // broadcast over rows, the window of a pooling gradient over channels-last data): the thread's four elements
+        // share every other coordinate, so the view's index is evaluated once, at the first of them
+        auto quad_contiguous = [&](const dsc_view& v) {
+            const int L = v.out_shape.rank - 1;
+            if (L < 0 || element_count(v.out_shape) != n || v.out_shape.dims[L] % 4 != 0) return false;
+            const int a = v.map_axis[L];
+            if (a < 0 || v.map_step[L] != 1 || needs_clamp(v, a) || v.in_offset[a] % 4 != 0 || v.in_shape.dims[a] % 4 != 0) return false;
+            for (int i = a + 1; i < v.in_shape.rank; ++i)
+                if (v.in_shape.dims[i] != 1) return false;
+            for (int j = 0; j < L; ++j)
+                if (v.map_axis[j] == a && v.out_shape.dims[j] > 1) return false;
+            return true;
+        };
         for (int i = 0; i < d.n_inputs; ++i) {
-            if (fk.inputs[i].buffer >= 0 && is_identity(d.inputs[i])) {
+            if (fk.inputs[i].buffer < 0) continue;
+            bool loaded = false;
+            for (int o = 0; o < d.n_ops; ++o) loaded = loaded || (d.ops[o].kind == DSC_PE_LOAD && d.ops[o].input_index == i);
+            if (!loaded) continue;
+            if (is_identity(d.inputs[i])) {
                 k << "    const float4 q" << i << " = *(const float4*)(b" << fk.inputs[i].buffer << " + base);\n";
-                k << "    const float l" << i << "[4] = {q" << i << ".x, q" << i << ".y, q" << i << ".z, q" << i << ".w};\n";
-                override_load[i] = "l" + to_string(i) + "[e]";
+            } else if (quad_contiguous(d.inputs[i])) {
+                auto c = em.emit_coords(k, d.inputs[i].out_shape, "base", "qb" + to_string(i) + "_");
+                k << "    const float4 q" << i << " = *(const float4*)(b" << fk.inputs[i].buffer << " + " << em.index_expr(d.inputs[i], c) << ");\n";
+            } else {
+                continue;
             }
+            k << "    const float l" << i << "[4] = {q" << i << ".x, q" << i << ".y, q" << i << ".z, q" << i << ".w};\n";
+            override_load[i] = "l" + to_string(i) + "[e]";
         }
         for (int o = 0; o < d.n_outputs; ++o) k << "    float o" << o << "[4];\n";
         k << "#pragma unroll\n    for (int e = 0; e < 4; ++e) {\n    const uint gid = base + e;\n";
