@@ -331,7 +331,10 @@ struct Emitter {
                 auto ov = override_load.find(op.input_index);
                 if (ov != override_load.end()) { rhs = ov->second; break; }
                 const dsc_view& v = pe.inputs[op.input_index];
-                if (is_identity(v)) rhs = load_linear(srcs[op.input_index], "(int)(" + gid + ")");
+                // (a fused producer behind an identity view is handed the coordinates when the caller has them taken
+                // apart already: it then divides nothing either)
+                if (is_identity(v) && !(form && form->valid && srcs[op.input_index].virt >= 0 && v.out_shape.rank > 1))
+                    rhs = load_linear(srcs[op.input_index], "(int)(" + gid + ")");
                 else rhs = load_view(srcs[op.input_index], v, coords_for(v.out_shape));
                 break;
             }
@@ -638,6 +641,9 @@ string gen_per_element(Emitter& em, Generated* out) {
     k << "    const uint base = (blockIdx.x * 256u + threadIdx.x) * " << vec << "u;\n";
     k << "    if (base >= " << S(n) << "u) return;\n";
     std::map<int, string> override_load;
+    dsc_shape quad_shape{};
+    IndexForm quad_form;
+    string quad_inner;
     if (vec == 4) {
         // identity-view loads of real buffers become one 16-byte load per thread; so do the loads through any view
         // whose innermost output axis walks the innermost input axis one to one in whole groups of four (a bias
@@ -671,11 +677,35 @@ string gen_per_element(Emitter& em, Generated* out) {
             override_load[i] = "l" + to_string(i) + "[e]";
         }
         for (int o = 0; o < d.n_outputs; ++o) k << "    float o" << o << "[4];\n";
+        // The thread's four elements differ in the innermost coordinate only (when that axis is a multiple of four
+        // long): the coordinates of the first are taken apart once, outside the loop, and handed to the views and
+        // fused producers as names, so nothing divides the element id per element, and what the four evaluations
+        // load from consecutive addresses can be merged by the compiler.
+        for (int i = 0; i < d.n_inputs + d.n_builtin_views && quad_shape.rank == 0; ++i) {
+            const dsc_view& v = i < d.n_inputs ? d.inputs[i] : d.builtin_views[i - d.n_inputs];
+            if (i < d.n_inputs && override_load.count(i)) continue;
+            const int L = v.out_shape.rank - 1;
+            if (L >= 1 && element_count(v.out_shape) == n && v.out_shape.dims[L] % 4 == 0) quad_shape = v.out_shape;
+        }
+        if (quad_shape.rank) {
+            auto c = em.emit_coords(k, quad_shape, "base", "qs_");
+            int64_t st[DSC_MAX_DIM];
+            strides_of(quad_shape, st);
+            quad_form.valid = true;
+            for (int j = 0; j < quad_shape.rank; ++j) {
+                if (quad_shape.dims[j] <= 1) continue;
+                quad_form.names.push_back(j == quad_shape.rank - 1 ? string("qs_inner") : c[j]);
+                quad_form.coefs.push_back(st[j]);
+                quad_form.extents.push_back(quad_shape.dims[j]);
+            }
+            quad_inner = c[quad_shape.rank - 1];
+        }
         k << "#pragma unroll\n    for (int e = 0; e < 4; ++e) {\n    const uint gid = base + e;\n";
+        if (quad_shape.rank) k << "    const int qs_inner = " << quad_inner << " + e;\n";
     } else {
         k << "    const uint gid = base;\n    {\n";
     }
-    em.emit_pe(k, d, fk.inputs, "gid", "", override_load);
+    em.emit_pe(k, d, fk.inputs, "gid", "", override_load, quad_form.valid ? &quad_form : nullptr);
     for (int o = 0; o < d.n_outputs; ++o) {
         if (vec == 4) k << "    o" << o << "[e] = t" << d.outputs[o] << ";\n";
         else k << "    b" << fk.outputs[o] << "[gid] = t" << d.outputs[o] << ";\n";
