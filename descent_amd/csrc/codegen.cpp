@@ -2586,7 +2586,10 @@ string gen_matmul(Emitter& em, Generated* out) {
         // as long as the product is at least one piece wide and tall
         const bool whole = chunk_k % t.bk == 0 && g.k % chunk_k == 0 && g.m >= 4 && g.n >= 4;
         const bool even = (t.bm * t.bk / 4) % nt == 0 && (t.bn * t.bk / 4) % nt == 0 && (t.bk & (t.bk - 1)) == 0;
-        if (nbuf && a_mode && b_mode && fk.colsum_out < 0 && whole && even && chunk_k / t.bk >= nbuf &&
+        // (column sums are combined through the one free tile buffer: a 16-byte partial per thread has to fit it)
+        // (weight gradients with their bias sums: 1024x1024 grid, layers of 256, 309 -> 318 steps/s)
+        const bool sums_fit = fk.colsum_out < 0 || (int64_t)nt * 4 <= (int64_t)(t.bm + t.bn) * t.bk;
+        if (nbuf && a_mode && b_mode && sums_fit && whole && even && chunk_k / t.bk >= nbuf &&
             (int64_t)nbuf * (t.bm + t.bn) * t.bk * 4 <= 160 * 1024)
             return nbuf;
         return 0;

@@ -153,6 +153,52 @@ def test_matmul_epilogue_with_a_per_element_and_a_per_column_operand(hip_backend
     assert int(listing.split()[0]) == 1 and "+epilogue" in listing and "tiles straight into LDS" in listing, listing
 
 
+@pytest.mark.parametrize("rows,m,n,force,buffers", [
+    (16384, 128, 260, "64,64,16,1,1,8", None), (32768, 128, 132, "128,64,32,2,2,8", None), (16384, 256, 388, "256,256,32,4,4,8", None),
+    (8192, 512, 512, None, None), (16384, 256, 256, None, "3"), (16384, 256, 256, "128,128,32,2,2,8", None),
+])
+def test_column_sums_from_tiles_loaded_straight_into_lds(hip_backend_session, monkeypatch, rows, m, n, force, buffers):
+    """A weight gradient x^T dz with the bias gradient (the column sums of dz) taken from the B tiles as they pass
+    through LDS: whole and ragged products, a thread's pieces on one and on both sides of the swapped row halves,
+    two and three tile buffers, against the oracle."""
+    if buffers is None:
+        monkeypatch.delenv("DSC_MM_DIRECT_LDS", raising=False)
+    else:
+        monkeypatch.setenv("DSC_MM_DIRECT_LDS", buffers)
+    if force is None:
+        monkeypatch.delenv("DSC_MM_TILE", raising=False)
+    else:
+        monkeypatch.setenv("DSC_MM_TILE", force)
+    genv, cenv = _envs(hip_backend_session)
+
+    def run(env):
+        rng = np.random.default_rng(rows + n)
+        x = env.static_parameter_with_data([rows, m], "x", rng.standard_normal(rows * m, dtype=np.float32))
+        dz = env.static_parameter_with_data([rows, n], "dz", rng.standard_normal(rows * n, dtype=np.float32))
+        dw = env.static_parameter([m, n], "dw")
+        db = env.static_parameter([n], "db")
+
+        def build(s):
+            d = s.parameter_value(dz)
+            s.write_parameter_value(db, d.reduce_sum(0, False) * 0.5)
+            # (the sine keeps x a stored operand of the product and puts the product behind the sum in the schedule)
+            s.write_parameter_value(dw, s.parameter_value(x).sin().transpose().matmul(d))
+
+        graph = env.build_graph(build)
+        env.run(graph, 0)
+        return env.read_parameter(dw), env.read_parameter(db), graph
+
+    got_w, got_b, graph = run(genv)
+    want_w, want_b, _ = run(cenv)
+    listing = next(iter(graph.__dict__["_schedules"].values())).describe()
+    assert "+column sums of B" in listing and f"tiles straight into LDS x{buffers or 2}" in listing, listing
+    if force is not None:
+        bm, bn, bk = force.split(",")[:3]
+        assert f"tile {bm}x{bn}x{bk} " in listing, listing
+    assert rel_l2(got_w, want_w) <= TOL
+    assert rel_l2(got_b, want_b) <= TOL
+
+
 @pytest.mark.parametrize("case", ["k-chunks", "batches", "rows-mode", "batches-transposed"])
 def test_direct_lds_tiles_over_k_chunks_and_batches(hip_backend_session, case):
     """The same path where a unit is a (k-chunk, batch, tile) triple: the reference's 1024-deep k-chunks written as
