@@ -405,6 +405,7 @@ bool rows_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
 bool smallk_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
 bool tallk_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
 bool dot_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
+bool dot_kernel_for_many_rows(const FusedKernel& fk, const MatMulDims& g);
 
 // Entry points carry the kernel kind and its size, so that a profiler's per-name statistics tell the kernels of
 // a schedule apart: dsc_matmul_mfma_epilogue_b1_m8192_n8192_k8192, dsc_reduce_k4084_n144, dsc_per_element_n12544000.
@@ -822,8 +823,10 @@ string gen_reduce(Emitter& em, Generated* out) {
         // k optionally split over TK thread rows combined through LDS
         const int64_t n_vec = n_out / 4;
         int64_t TK = 1;
-        if (n_vec < 32768 && K >= 8) {
-            while (TK < 64 && n_vec * TK < 32768 && TK * 4 <= K) TK *= 2;
+        // (a workgroup per compute unit at least: the sum of 256 partial 256x256 products took 23.4 us with 128 workgroups)
+        const int64_t want_threads = 65536;
+        if (n_vec < want_threads && K >= 8) {
+            while (TK < 64 && n_vec * TK < want_threads && TK * 4 <= K) TK *= 2;
         }
         const int64_t TO = 256 / TK;
         k << "    const int to = threadIdx.x % " << TO << ", tk = threadIdx.x / " << TO << ";\n";
@@ -2005,6 +2008,21 @@ MmConfig pick_config(int64_t M, int64_t N, int64_t K /* per chunk */, int64_t gr
     return c;
 }
 
+// Tall products with a few columns whose rows lie contiguous in memory and are long (the output layer of a coordinate
+// network: 262144 x 256 -> 3) go to the dot-product kernel instead of the row-per-thread one: with a lane per row the
+// 64 lanes of a load touch 64 different cache lines, eight loads before a line is used up, and a row of 1 KB per
+// lane is more than L1 keeps.  With L lanes along a row every line is requested once.  Measured on MI355X:
+// 262144 x 256 -> 3 77.4 -> 53 us, 262144 x 64 -> 3 23.6 -> 19.4 us.
+bool dot_kernel_for_many_rows(const FusedKernel& fk, const MatMulDims& g) {
+    if (const char* e = std::getenv("DSC_MM_DOT"))
+        if (e[0] == '0') return false;
+    if (g.chunks != 1 && !fk.sum_chunks) return false;
+    if (fk.colsum_out >= 0 || fk.out_slice_width || fk.dgrad.on || fk.cfwd.on || fk.pool.on) return false;
+    if (!(g.n <= 16 && g.k >= 64 && g.k <= 256 && g.k * g.n <= 4096 && g.m * g.batch >= 16384)) return false;
+    int64_t base = 0, coef[DSC_MAX_DIM] = {0};
+    return fk.inputs[0].buffer >= 0 && affine_form(fk.main.raw().inputs[0], &base, coef) && coef[2] == 1;
+}
+
 // Row-per-thread matmul for tall products with a narrow output (N <= 32, K <= 256): the HBM-bound GEMMs of the
 // convolutions (N = 16, K = 9 / 72) and of the narrow output layers.  Every thread owns one row of C in
 // registers.  B's address is the same for every lane of a wave, so the compiler fetches it with scalar loads
@@ -2015,6 +2033,7 @@ bool rows_kernel_applies(const FusedKernel& fk, const MatMulDims& g) {
     if (const char* e = std::getenv("DSC_MM_ROWS"))
         if (e[0] == '0') return false;
     if (g.chunks != 1 && !fk.sum_chunks) return false;
+    if (dot_kernel_for_many_rows(fk, g)) return false;
     return g.n <= 32 && g.k <= 256 && g.k * g.n <= 8192 && g.m * g.batch >= 16384;
 }
 
@@ -2103,7 +2122,7 @@ bool dot_kernel_applies(const FusedKernel& fk, const MatMulDims& g) {
         if (e[0] == '0') return false;
     MatMulDims whole = g;
     if (fk.sum_chunks) whole.chunks = 1;  // one full sum over k is what this kernel computes anyway
-    return fk.colsum_out < 0 && dot_shape(whole);
+    return fk.colsum_out < 0 && (dot_shape(whole) || dot_kernel_for_many_rows(fk, g));
 }
 
 }  // namespace
@@ -2152,20 +2171,34 @@ string gen_matmul_dot(Emitter& em, Generated* out) {
     // B of this workgroup's batch: [k][n], zero beyond k (a workgroup's rows may straddle two batches only when
     // the batch has fewer rows than a workgroup, which the row -> batch split below rules out by using one batch
     // per workgroup)
-    const int64_t wgs_per_batch = (g.m + RPW - 1) / RPW;
+    // Many rows: a workgroup walks T groups of RPW rows with B staged once, the next group's A requested before the
+    // current one is multiplied.
+    const int64_t T = total_rows >= 16384 ? 8 : 1;
+    const int64_t wgs_per_batch = (g.m + RPW * T - 1) / (RPW * T);
     k << "    __shared__ float sB[" << S(blocks * 4 * N) << "];\n";
-    k << "    const int cb = blockIdx.x / " << S(wgs_per_batch) << ", row0 = (blockIdx.x % " << S(wgs_per_batch) << ") * " << S(RPW) << ";\n";
+    k << "    const int cb = blockIdx.x / " << S(wgs_per_batch) << ", row0 = (blockIdx.x % " << S(wgs_per_batch) << ") * " << S(RPW * T) << ";\n";
     k << "    for (int e = threadIdx.x; e < " << S(blocks * 4 * N) << "; e += 256) {\n";
     k << "        const int kk = e / " << S(N) << ", nn = e % " << S(N) << ";\n";
     k << "        const float v = load_b(cb, min(kk, " << S(K - 1) << "), nn, " << em.params_pass() << ");\n";
     k << "        sB[e] = kk < " << S(K) << " ? v : 0.f;\n    }\n";
-    k << "    const int lg = threadIdx.x % " << S(L) << ", cm = row0 + threadIdx.x / " << S(L) << ", cml = min(cm, " << S(g.m - 1) << ");\n";
+    k << "    const int lg = threadIdx.x % " << S(L) << ", rl = row0 + threadIdx.x / " << S(L) << ";\n";
     // A: every block of the lane requested before anything is used; beyond k the clamped loads repeat valid
     // elements, which meet zeros of B
-    k << "    float a[" << S(J) << "][4];\n";
-    k << "#pragma unroll\n    for (int j = 0; j < " << S(J) << "; ++j)\n#pragma unroll\n        for (int i = 0; i < 4; ++i)\n";
-    k << "            a[j][i] = load_a(cb, cml, min(4 * (lg + j * " << S(L) << ") + i, " << S(K - 1) << "), " << em.params_pass() << ");\n";
+    k << "    float a[" << S(J) << "][4], an[" << S(J) << "][4];\n";
+    auto load_group = [&](const char* dst, const string& row) {
+        k << "#pragma unroll\n    for (int j = 0; j < " << S(J) << "; ++j)\n#pragma unroll\n        for (int i = 0; i < 4; ++i)\n";
+        k << "            " << dst << "[j][i] = load_a(cb, min(" << row << ", " << S(g.m - 1) << "), min(4 * (lg + j * " << S(L) << ") + i, " << S(K - 1) << "), "
+          << em.params_pass() << ");\n";
+    };
+    load_group("a", "rl");
     k << "    __syncthreads();\n";
+    k << "#pragma unroll\n    for (int it = 0; it < " << S(T) << "; ++it) {\n";
+    k << "    const int cm = rl + it * " << S(RPW) << ";\n";
+    if (T > 1) {
+        k << "    if (it + 1 < " << S(T) << ") {\n";
+        load_group("an", "cm + " + S(RPW));
+        k << "    }\n";
+    }
     k << "    float acc[" << S(N) << "];\n#pragma unroll\n    for (int n = 0; n < " << S(N) << "; ++n) acc[n] = 0.f;\n";
     k << "#pragma unroll\n    for (int j = 0; j < " << S(J) << "; ++j) {\n";
     k << "        const int blk = lg + j * " << S(L) << ";\n";
@@ -2183,13 +2216,15 @@ string gen_matmul_dot(Emitter& em, Generated* out) {
     } else {
         k << "                b" << fk.outputs[0] << "[c_at] = acc[n];\n";
     }
-    k << "            }\n    }\n}\n";
+    k << "            }\n    }\n";
+    if (T > 1) k << "#pragma unroll\n    for (int j = 0; j < " << S(J) << "; ++j)\n#pragma unroll\n        for (int i = 0; i < 4; ++i) a[j][i] = an[j][i];\n";
+    k << "    }\n}\n";
     (void)total_rows;
     if (wgs_per_batch * g.batch >= kMaxIndex) return "matmul: grid too large";
     out->grid = (unsigned)(wgs_per_batch * g.batch);
     out->block = 256;
     out->source = k.str();
-    out->note = "dot products: " + S(L) + " lanes per row, B in LDS" + (fk.has_epilogue ? " +epilogue" : "");
+    out->note = "dot products: " + S(L) + " lanes per row, " + (T > 1 ? S(T) + " row groups per workgroup, " : string()) + "B in LDS" + (fk.has_epilogue ? " +epilogue" : "");
     return "";
 }
 

@@ -2487,7 +2487,13 @@ struct Planner {
     // small parts start at once and finish in its shadow).
     void share_launches() {
         static const int64_t small_grid = std::getenv("DSC_MULTI_GRID") ? std::atoll(std::getenv("DSC_MULTI_GRID")) : 1024;
+        // A kernel that moves this much is a launch's worth of work whatever its grid (a tall-k MatMul walks 268 MB with
+        // 1024 workgroups): sharing a launch with another large kernel would only tie the two to the registers and
+        // LDS of the hungrier one.
+        static const double heavy_bytes = std::getenv("DSC_MULTI_BYTES") ? std::atof(std::getenv("DSC_MULTI_BYTES")) : 128e6;
         std::vector<int64_t> grid_of(drafts.size(), -1);
+        std::vector<char> heavy(drafts.size(), 0);
+        auto is_large = [&](int i) { return grid_of[i] > small_grid || heavy[i]; };
         auto partable = [&](int i) {
             const Draft& d = drafts[i];
             if (!d.alive || !can_be_part(d.fk)) return false;
@@ -2499,6 +2505,7 @@ struct Planner {
                 probe.as_part = true;  // a kernel may pick another workgroup shape inside a shared launch
                 if (!generate(probe, &g).empty() || g.block != 256) { grid_of[i] = (int64_t)1 << 40; return false; }
                 grid_of[i] = g.grid;
+                heavy[i] = g.algo_bytes > heavy_bytes;
             }
             return grid_of[i] < ((int64_t)1 << 30);
         };
@@ -2506,7 +2513,7 @@ struct Planner {
         for (int i = 0; i < (int)drafts.size() && small_grid > 0; ++i) {
             if (taken[i] || !partable(i)) continue;
             std::vector<int> batch{i};
-            int large = grid_of[i] > small_grid ? 1 : 0;
+            int large = is_large(i) ? 1 : 0;
             int64_t total_grid = grid_of[i];
             std::set<int> blocked, bound;
             for (auto& o : drafts[i].outs) blocked.insert(o.node);
@@ -2518,11 +2525,11 @@ struct Planner {
                     if (blocked.count(nd)) depends = true;
                 std::set<int> would = bound;
                 for (int nd : drafts[j].params) would.insert(nd);
-                if (!depends && batch.size() < 16 && would.size() <= 48 && partable(j) && (grid_of[j] <= small_grid || large == 0) &&
+                if (!depends && batch.size() < 16 && would.size() <= 48 && partable(j) && (!is_large(j) || large == 0) &&
                     total_grid + grid_of[j] < ((int64_t)1 << 30)) {
                     batch.push_back(j);
                     bound = would;
-                    large += grid_of[j] > small_grid ? 1 : 0;
+                    large += is_large(j) ? 1 : 0;
                     total_grid += grid_of[j];
                 }
                 for (auto& o : drafts[j].outs) blocked.insert(o.node);

@@ -153,6 +153,42 @@ def test_matmul_epilogue_with_a_per_element_and_a_per_column_operand(hip_backend
     assert int(listing.split()[0]) == 1 and "+epilogue" in listing and "tiles straight into LDS" in listing, listing
 
 
+@pytest.mark.parametrize("m,n,k,tb,epilogue", [
+    (16384, 3, 256, False, True), (20000, 5, 64, False, False), (40001, 16, 200, True, True), (16390, 2, 66, False, False),
+    (262144, 3, 256, True, True), (70000, 1, 128, False, True),
+])
+def test_tall_products_with_long_contiguous_rows_and_few_columns(hip_backend_session, m, n, k, tb, epilogue):
+    """The output layer of a coordinate network: many rows, each long and contiguous, a few columns.  Lanes share a
+    row (every cache line requested once) and a workgroup walks several groups of rows with B staged once; row
+    counts that end inside a group, k off the 16-byte grid, B in either layout, with and without a fused consumer."""
+    genv, cenv = _envs(hip_backend_session)
+
+    def run(env):
+        rng = np.random.default_rng(m + k)
+        a = env.static_parameter_with_data([m, k], "a", rng.standard_normal(m * k, dtype=np.float32))
+        b = env.static_parameter_with_data([n, k] if tb else [k, n], "b", rng.standard_normal(k * n, dtype=np.float32))
+        bias = env.static_parameter_with_data([n], "bias", rng.standard_normal(n, dtype=np.float32))
+        c = env.static_parameter([m, n], "c")
+
+        def build(s):
+            bv = s.parameter_value(b)
+            z = s.parameter_value(a).matmul(bv.transpose() if tb else bv)
+            if epilogue:
+                z = z + s.parameter_value(bias)
+                z = z.select_gt(0.0, z, z * 0.01)
+            s.write_parameter_value(c, z)
+
+        graph = env.build_graph(build)
+        env.run(graph, 0)
+        return env.read_parameter(c), graph
+
+    got, graph = run(genv)
+    want, _ = run(cenv)
+    listing = next(iter(graph.__dict__["_schedules"].values())).describe()
+    assert "dot products:" in listing and int(listing.split()[0]) == 1, listing
+    assert rel_l2(got, want) <= TOL
+
+
 @pytest.mark.parametrize("rows,m,n,force,buffers", [
     (16384, 128, 260, "64,64,16,1,1,8", None), (32768, 128, 132, "128,64,32,2,2,8", None), (16384, 256, 388, "256,256,32,4,4,8", None),
     (8192, 512, 512, None, None), (16384, 256, 256, None, "3"), (16384, 256, 256, "128,128,32,2,2,8", None),
