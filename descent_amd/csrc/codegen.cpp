@@ -431,11 +431,13 @@ string entry_name(const FusedKernel& fk) {
     }
     case DSC_KERNEL_MATMUL: {
         const MatMulDims g = matmul_dims(d);
-        string base = rows_kernel_applies(fk, g)     ? "dsc_matmul_rows"
+        string base = fk.pair.on                     ? "dsc_matmul_shortk"
+                      : rows_kernel_applies(fk, g)   ? "dsc_matmul_rows"
                       : smallk_kernel_applies(fk, g) ? "dsc_matmul_shortk"
                       : tallk_kernel_applies(fk, g)  ? "dsc_matmul_tallk"
                       : dot_kernel_applies(fk, g)    ? "dsc_matmul_dot"
                                                      : "dsc_matmul_mfma";
+        if (fk.pair.on) base += "_wgrad";
         if (fk.has_epilogue) base += "_epilogue";
         if (fk.out_slice_width) base += "_slices" + count(fk.out_slice_width);
         return base + "_b" + count(g.batch) + "_m" + count(g.m) + "_n" + count(g.n) + "_k" + count(g.k);
@@ -2105,6 +2107,88 @@ string gen_matmul_smallk(Emitter& em, Generated* out) {
     return "";
 }
 
+// The short-k kernel of a layer's data gradient that computes the layer's weight gradient as well (see
+// FusedKernel::GradPair).  256 threads = n/4 column quads x (1024 / n) row lanes; a workgroup owns `chunk_rows` rows.
+// Per row a thread loads dY's k values, 16 bytes of X and computes what the short-k kernel computes, with X handed
+// to the consumer as a value; X times dY goes into 4k accumulators, which meet in LDS at the end.  Up to eight rows
+// are requested before the first is used.
+string gen_matmul_smallk_pair(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const MatMulDims g = matmul_dims(d);
+    const dsc_kernel_desc& pe = fk.epilogue.raw();
+    const int n_out = pe.n_outputs;
+    const int64_t N = g.n, KS = g.k, NQ = N / 4, RL = 256 / NQ, R = fk.pair.chunk_rows, C = fk.pair.chunks;
+    if (!fk.has_epilogue || g.batch != 1 || KS > 4 || N % 4 != 0 || NQ > 256 || 256 % NQ != 0 || R < 1 || C < 1 || (C - 1) * R >= g.m || C * R < g.m ||
+        C >= kMaxIndex || fk.pair.x_buffer < 0 || fk.pair.out < 0)
+        return "matmul: not a data/weight gradient pair";
+    // rows in flight per thread (262144 x 256, k = 3, 1024 workgroups: 2 rows 105.6 us, 4 103.5, 8 97.7, 16 96.1)
+    const int U = (int)std::max<int64_t>(1, std::min<int64_t>(8, R / RL));
+    const string la = em.load_view(fk.inputs[0], d.inputs[0], {"cb", "cm", "ck"});
+    em.funcs << "DSC_INLINE float load_a(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return " << la << ";\n}\n";
+    const string lb = em.load_view(fk.inputs[1], d.inputs[1], {"cb", "ck", "cn"});
+    em.funcs << "DSC_INLINE float load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb << ";\n}\n";
+    {
+        std::ostringstream body;
+        std::map<int, string> ov;
+        ov[fk.epilogue_product_input] = "product";
+        for (int i = 0; i < pe.n_inputs; ++i)
+            if (i != fk.epilogue_product_input && fk.epilogue_inputs[i].buffer == fk.pair.x_buffer && is_identity(pe.inputs[i]) &&
+                element_count(pe.inputs[i].out_shape) == g.m * N)
+                ov[i] = "xval";
+        IndexForm form;
+        form.valid = true;
+        form.names = {"cb", "cm", "cn"};
+        form.coefs = {g.m * N, N, 1};
+        form.extents = {g.batch, g.m, g.n};
+        em.emit_pe(body, pe, fk.epilogue_inputs, "gid", "e", ov, &form);
+        for (int o = 0; o < pe.n_outputs; ++o) body << "    result[" << o << "] = et" << pe.outputs[o] << ";\n";
+        em.funcs << "DSC_INLINE void mm_epilogue(float product, float xval, int gid, int cb, int cm, int cn, float* result, " << em.params_decl() << ") {\n"
+                 << body.str() << "}\n";
+    }
+    std::ostringstream k;
+    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
+    k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
+    k << "    __shared__ float red[" << S(RL * N * KS) << "];\n";
+    k << "    const int q = threadIdx.x % " << S(NQ) << ", rl = threadIdx.x / " << S(NQ) << ", cn = q * 4, cb = 0;\n";
+    k << "    const int row_begin = blockIdx.x * " << S(R) << ", row_end = min(row_begin + " << S(R) << ", " << S(g.m) << ");\n";
+    k << "    float bq[" << S(KS) << "][4], wg[" << S(KS) << "][4];\n";
+    k << "#pragma unroll\n    for (int ck = 0; ck < " << S(KS) << "; ++ck)\n#pragma unroll\n        for (int j = 0; j < 4; ++j) {\n";
+    k << "            bq[ck][j] = load_b(cb, ck, cn + j, " << em.params_pass() << ");\n            wg[ck][j] = 0.f;\n        }\n";
+    k << "    for (int r0 = row_begin + rl; r0 < row_end; r0 += " << S(RL * U) << ") {\n";
+    k << "        float a[" << U << "][" << S(KS) << "];\n        float4 x[" << U << "];\n";
+    // rows past the chunk's end repeat its last row's loads and take no part in the sums or the stores
+    k << "#pragma unroll\n        for (int u = 0; u < " << U << "; ++u) {\n";
+    k << "            const int cm = min(r0 + u * " << S(RL) << ", row_end - 1);\n";
+    k << "#pragma unroll\n            for (int ck = 0; ck < " << S(KS) << "; ++ck) a[u][ck] = load_a(cb, cm, ck, " << em.params_pass() << ");\n";
+    k << "            x[u] = *(const float4*)(b" << fk.pair.x_buffer << " + (cm * " << S(N) << " + cn));\n        }\n";
+    k << "#pragma unroll\n        for (int u = 0; u < " << U << "; ++u) {\n";
+    k << "            const int cm = r0 + u * " << S(RL) << ";\n            if (cm < row_end) {\n";
+    k << "                const float xs[4] = {x[u].x, x[u].y, x[u].z, x[u].w};\n";
+    k << "                const int c_at = cm * " << S(N) << " + cn;\n";
+    k << "                float res[4][" << n_out << "];\n";
+    k << "#pragma unroll\n                for (int j = 0; j < 4; ++j) {\n                    float acc = 0.f;\n";
+    k << "#pragma unroll\n                    for (int ck = 0; ck < " << S(KS) << "; ++ck) acc = fmaf(a[u][ck], bq[ck][j], acc);\n";
+    k << "                    mm_epilogue(acc, xs[j], c_at + j, cb, cm, cn + j, res[j], " << em.params_pass() << ");\n";
+    k << "#pragma unroll\n                    for (int ck = 0; ck < " << S(KS) << "; ++ck) wg[ck][j] = fmaf(xs[j], a[u][ck], wg[ck][j]);\n                }\n";
+    for (int o = 0; o < n_out; ++o)
+        k << "                *(float4*)(b" << fk.outputs[o] << " + c_at) = make_float4(res[0][" << o << "], res[1][" << o << "], res[2][" << o << "], res[3]["
+          << o << "]);\n";
+    k << "            }\n        }\n    }\n";
+    // partial[chunk][column][k]: the row lanes' sums meet in LDS
+    k << "#pragma unroll\n    for (int j = 0; j < 4; ++j)\n#pragma unroll\n        for (int ck = 0; ck < " << S(KS) << "; ++ck) red[rl * " << S(N * KS)
+      << " + (cn + j) * " << S(KS) << " + ck] = wg[ck][j];\n";
+    k << "    __syncthreads();\n";
+    k << "    for (int i = threadIdx.x; i < " << S(N * KS) << "; i += 256) {\n        float sum = red[i];\n";
+    k << "        for (int r = 1; r < " << S(RL) << "; ++r) sum += red[r * " << S(N * KS) << " + i];\n";
+    k << "        b" << fk.pair.out << "[blockIdx.x * " << S(N * KS) << " + i] = sum;\n    }\n}\n";
+    out->grid = (unsigned)C;
+    out->block = 256;
+    out->source = k.str();
+    out->note = "short-k fma, four columns per thread +epilogue, +the weight gradient X^T A over " + S(C) + " chunks of " + S(R) + " rows";
+    return "";
+}
+
 // Dot-product kernel for products with few columns and not many rows (a classifier head: 1000 x 128 -> 10): too
 // small to fill the MFMA template's tiles -- a 32x32 tile grid of such a product is a few dozen single-wave
 // workgroups, each walking k in eight sequential load -> LDS -> MFMA round trips.  Here L lanes share one row: lane l
@@ -2578,6 +2662,8 @@ string gen_matmul(Emitter& em, Generated* out) {
     if (fk.colsum_out >= 0 && (rows_kernel_applies(fk, g) || smallk_kernel_applies(fk, g)))
         return "matmul: column sums need the MFMA template or the tall-k kernel";
     if (fk.out_slice_width && (!rows_kernel_applies(fk, g) || fk.dgrad.on || fk.cfwd.on)) return "matmul: only the row-per-thread kernel stores slice-major";
+    // (a gradient pair is a short-k kernel whatever else the product's shape would allow)
+    if (fk.pair.on) return smallk_kernel_applies(fk, g) && !fk.out_slice_width ? gen_matmul_smallk_pair(em, out) : string("matmul: a gradient pair needs the short-k kernel");
     if (rows_kernel_applies(fk, g)) return gen_matmul_rows(em, out);
     if (smallk_kernel_applies(fk, g)) return gen_matmul_smallk(em, out);
     if (tallk_kernel_applies(fk, g)) return gen_matmul_tallk(em, out);
@@ -2899,6 +2985,12 @@ void count_work(const FusedKernel& fk, Generated* g) {
     if (d.kind == DSC_KERNEL_SCATTER_ADD)  // read-modify-write of the entries that receive a value
         out_each = 2.0 * std::min((double)element_count(d.shape), (double)element_count(d.inputs[0].out_shape));
     if (fk.row_stages.empty()) elements += out_each * (double)fk.outputs.size();
+    if (fk.pair.on) {
+        // the last output is the weight gradient's partials, and its flops are those of the MatMul it stands for
+        const MatMulDims m = matmul_dims(d);
+        elements += (double)(fk.pair.chunks * m.n * m.k) - out_each;
+        g->algo_flops *= 2.0;
+    }
     for (auto& st : fk.row_stages)
         for (int o : st.outputs)
             if (o >= 0) elements += (double)element_count(st.k.raw().shape);
@@ -2908,6 +3000,30 @@ void count_work(const FusedKernel& fk, Generated* g) {
 }  // namespace
 
 bool tallk_shape(const MatMulDims& g) { return tallk_shape_impl(g); }
+
+bool grad_pair_shapes(const FusedKernel& s, const FusedKernel& t, int64_t* chunk_rows, int64_t* chunks) {
+    const dsc_kernel_desc& sd = s.main.raw();
+    const dsc_kernel_desc& td = t.main.raw();
+    if (sd.kind != DSC_KERNEL_MATMUL || td.kind != DSC_KERNEL_MATMUL || sd.output_mode != DSC_MATMUL_BATCHES || td.output_mode != DSC_MATMUL_BATCHES) return false;
+    auto plain = [](const FusedKernel& f) {
+        return f.virtuals.empty() && f.colsum_out < 0 && !f.dgrad.on && !f.cfwd.on && !f.pool.on && !f.out_slice_width && f.parts.empty() &&
+               f.row_stages.empty() && !f.pair.on && f.inputs.size() >= 2 && f.inputs[0].buffer >= 0 && f.inputs[1].buffer >= 0;
+    };
+    if (!plain(s) || !plain(t) || !s.has_epilogue || t.has_epilogue || t.sum_chunks) return false;
+    const MatMulDims gs = matmul_dims(sd), gt = matmul_dims(td);
+    if (!smallk_kernel_applies(s, gs) || !tallk_kernel_applies(t, gt)) return false;
+    if (gs.batch != 1 || gt.batch != 1 || gs.k > 4 || gs.n > 1024 || 256 % (gs.n / 4) != 0) return false;
+    if (gt.m != gs.n || gt.n != gs.k || gt.k != gs.m) return false;
+    int64_t base = 0, coef[DSC_MAX_DIM] = {0};
+    // dY [m, k] in order, as the short-k product's A and as the tall-k product's B
+    if (!affine_form(sd.inputs[0], &base, coef) || base != 0 || coef[1] != gs.k || coef[2] != 1) return false;
+    if (!affine_form(td.inputs[1], &base, coef) || base != 0 || coef[1] != gs.k || coef[2] != 1) return false;
+    // X [m, n] in order, transposed by the tall-k product's view
+    if (!affine_form(td.inputs[0], &base, coef) || base != 0 || coef[1] != 1 || coef[2] != gs.n) return false;
+    *chunk_rows = chunk_k_of(gt);
+    *chunks = gt.chunks;
+    return (*chunks - 1) * *chunk_rows < gt.k && *chunks * *chunk_rows >= gt.k;
+}
 bool dot_kernel_shape(const MatMulDims& g) {
     const char* e = std::getenv("DSC_MM_DOT");
     return !(e && e[0] == '0') && dot_shape(g);
@@ -2999,6 +3115,7 @@ std::string FusedKernel::key() const {
     if (row_width) s += "|RW" + to_string((long long)row_width);
     if (as_part) s += "|AP";
     if (colsum_out >= 0) s += "|CS" + to_string(colsum_out);
+    if (pair.on) s += "|GP" + to_string(pair.x_buffer) + "," + to_string(pair.out) + "," + to_string((long long)pair.chunk_rows) + "," + to_string((long long)pair.chunks);
     s += "|O";
     for (int o : outputs) s.append(reinterpret_cast<const char*>(&o), 4);
     s.append(reinterpret_cast<const char*>(&n_buffers), 4);
@@ -3076,7 +3193,7 @@ static std::string generate_one(const FusedKernel& fk, Generated* out, bool with
             return "this kernel kind takes no epilogue";
         if (fk.epilogue_permuted && mk != DSC_KERNEL_REDUCE) return "only a Reduce takes an epilogue through a permuting view";
         if (fk.epilogue_keeps_product && (mk == DSC_KERNEL_MATMUL || fk.epilogue_permuted)) return "this epilogue cannot keep its product";
-        if (!fk.pool.on && (int)fk.outputs.size() != fk.epilogue.raw().n_outputs + (fk.epilogue_keeps_product ? 1 : 0)) return "epilogue output count";
+        if (!fk.pool.on && (int)fk.outputs.size() != fk.epilogue.raw().n_outputs + (fk.epilogue_keeps_product ? 1 : 0) + (fk.pair.on ? 1 : 0)) return "epilogue output count";
     }
     if (fk.pool.on) {
         if (!fk.cfwd.on) return "pooling rides on the convolution-forward kernel only";

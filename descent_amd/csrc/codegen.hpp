@@ -145,6 +145,17 @@ struct FusedKernel {
     // concats): w > 0 makes a thread evaluate one whole row with the column a constant of each of its w evaluations,
     // so the compiler keeps, per column, only the branch that column takes.
     int64_t row_width = 0;
+    // Short-k MatMul with a per-element consumer -- the data gradient dY x W^T of a layer with a few outputs, masked by
+    // the stored activation X -- that also computes the layer's weight gradient X^T dY, the tall-k MatMul that reads
+    // the same X [m, n] and the same dY [m, k]: a workgroup walks `chunk_rows` rows, a thread multiplies the 16 bytes
+    // of X it holds anyway with the row's k values of dY, and the workgroup writes one partial [n, k] per chunk, the
+    // layout the tall-k kernel's k chunks had (the Reduce over them stays as it is).  `x_buffer` is X's pointer
+    // parameter, `out` the partials'.
+    struct GradPair {
+        bool on = false;
+        int x_buffer = -1, out = -1;
+        int64_t chunk_rows = 0, chunks = 0;
+    } pair;
     bool sum_chunks = false;               // MatMul: ignore the descriptor's chunk count, write one full sum
     int colsum_out = -1;                   // MatMul (MFMA template): buffer that takes the column sums of B per k chunk
     bool as_part = false;                  // generated as one part of a multi-part launch (set while the launch is generated)
@@ -216,6 +227,9 @@ bool can_be_part(const FusedKernel& k);
 bool tallk_shape(const MatMulDims& g);
 // the dot-product kernel takes this product (rows x few columns over a k of moderate length)
 bool dot_kernel_shape(const MatMulDims& g);
+// `s` is a short-k MatMul with a consumer and `t` a plain tall-k MatMul shaped like the data and weight gradient of
+// one layer with a few outputs (see FusedKernel::GradPair; which buffers they read is the caller's to compare)
+bool grad_pair_shapes(const FusedKernel& s, const FusedKernel& t, int64_t* chunk_rows, int64_t* chunks);
 
 // hipRTC options every kernel is compiled with (after --offload-arch=<arch>).
 const std::vector<std::string>& compile_options();

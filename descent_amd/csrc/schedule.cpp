@@ -2480,6 +2480,68 @@ struct Planner {
         }
     }
 
+    // Pass 3f: the two gradients of a layer with a few outputs (the last layer of a coordinate network, 256 -> 3) read
+    // the same two arrays: the data gradient dY x W^T, a short-k MatMul whose consumer masks it with the stored
+    // activation X, and the weight gradient X^T dY, a tall-k MatMul over the rows.  One kernel computes both from one
+    // pass over X (FusedKernel::GradPair); the tall-k product's chunks become the row chunks of that kernel, so the
+    // Reduce over its partials stays as it is.  The pair runs where the earlier of the two ran.
+    void pair_output_layer_gradients() {
+        static const bool enabled = !(std::getenv("DSC_FUSE_GRAD_PAIR") && std::getenv("DSC_FUSE_GRAD_PAIR")[0] == '0');
+        if (!enabled) return;
+        for (int si = 0; si < (int)drafts.size(); ++si) {
+            if (!drafts[si].alive || drafts[si].fk.main.raw().kind != DSC_KERNEL_MATMUL || !drafts[si].fk.has_epilogue) continue;
+            bool in_place = false;
+            for (auto& o : drafts[si].outs)
+                if (o.copy_from >= 0) in_place = true;
+            if (in_place) continue;
+            for (int ti = 0; ti < (int)drafts.size(); ++ti) {
+                const Draft& S = drafts[si];
+                const Draft& T = drafts[ti];
+                if (ti == si || !T.alive || T.fk.main.raw().kind != DSC_KERNEL_MATMUL || T.outs.size() != 1 || T.outs[0].copy_from >= 0) continue;
+                int64_t rows = 0, chunks = 0;
+                if (!grad_pair_shapes(S.fk, T.fk, &rows, &chunks)) continue;
+                const int dy = S.params[S.fk.inputs[0].buffer], x = T.params[T.fk.inputs[0].buffer];
+                if (T.params[T.fk.inputs[1].buffer] != dy) continue;
+                // X has to be something the data gradient's consumer reads anyway, element for element
+                int x_param = -1;
+                for (size_t p = 0; p < S.params.size(); ++p)
+                    if (S.params[p] == x && !S.fk.buffer_is_output[p]) x_param = (int)p;
+                const dsc_kernel_desc& pe = S.fk.epilogue.raw();
+                bool reads_x = false;
+                for (int i = 0; i < pe.n_inputs && x_param >= 0; ++i)
+                    if (i != S.fk.epilogue_product_input && S.fk.epilogue_inputs[i].buffer == x_param && is_identity(pe.inputs[i])) reads_x = true;
+                if (!reads_x) continue;
+                // everything the later of the two reads must exist where the earlier one runs
+                const int first = std::min(si, ti), last = std::max(si, ti);
+                std::set<int> needed;
+                for (int nd : input_nodes(drafts[last])) needed.insert(nd);
+                bool ok = true;
+                for (int q = first; q < last && ok; ++q) {
+                    if (!drafts[q].alive) continue;
+                    for (auto& o : drafts[q].outs)
+                        if (needed.count(o.node)) ok = false;
+                }
+                if (!ok) continue;
+                Draft F = S;
+                F.fk.pair.on = true;
+                F.fk.pair.x_buffer = x_param;
+                F.fk.pair.chunk_rows = rows;
+                F.fk.pair.chunks = chunks;
+                F.fk.pair.out = param_index(F, T.outs[0].node, true);
+                F.fk.outputs.push_back(F.fk.pair.out);
+                F.outs.push_back(T.outs[0]);
+                F.covers.insert(F.covers.end(), T.covers.begin(), T.covers.end());
+                {
+                    Generated probe;
+                    if (!generate(F.fk, &probe).empty()) continue;
+                }
+                drafts[last].alive = false;
+                drafts[first] = F;
+                break;
+            }
+        }
+    }
+
     // Pass 4: launches of a few workgroups each (optimiser updates of small tensors, short reductions, scalar
     // bookkeeping) cost a launch apiece while using a fraction of the machine.  Runs of them that do not
     // depend on one another become one multi-part launch; a later launch is hoisted into the run when nothing
@@ -2585,6 +2647,7 @@ struct Planner {
         pool_joins_conv_forward();              // pass 3c
         chain_scatter_adds();                   // pass 3b
         group_chain_launches();                 // pass 3e
+        pair_output_layer_gradients();          // pass 3f
         share_launches();                       // pass 4
     }
 };

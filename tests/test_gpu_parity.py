@@ -189,6 +189,38 @@ def test_tall_products_with_long_contiguous_rows_and_few_columns(hip_backend_ses
     assert rel_l2(got, want) <= TOL
 
 
+@pytest.mark.parametrize("m,n,k", [(65536, 128, 2), (100000, 64, 3), (70000, 256, 4), (262144, 256, 3), (132072, 64, 3), (65536, 32, 3), (131072, 16, 3)])
+def test_data_and_weight_gradient_of_a_layer_with_few_outputs_as_one_kernel(hip_backend_session, m, n, k):
+    """dZ = (dY W^T) masked by the stored activation X, and dW = X^T dY: one kernel reads X once for both (the weight
+    gradient's k chunks become the kernel's row chunks; the last chunk of a ragged row count is short)."""
+    genv, cenv = _envs(hip_backend_session)
+
+    def run(env):
+        rng = np.random.default_rng(m + n)
+        dy = env.static_parameter_with_data([m, k], "dy", rng.standard_normal(m * k, dtype=np.float32))
+        x = env.static_parameter_with_data([m, n], "x", rng.standard_normal(m * n, dtype=np.float32))
+        w = env.static_parameter_with_data([n, k], "w", rng.standard_normal(n * k, dtype=np.float32))
+        dz = env.static_parameter([m, n], "dz")
+        dw = env.static_parameter([n, k], "dw")
+
+        def build(s):
+            d, xv = s.parameter_value(dy), s.parameter_value(x)
+            p = d.matmul(s.parameter_value(w).transpose())
+            s.write_parameter_value(dz, xv.select_gt(0.0, p, p * 0.01))
+            s.write_parameter_value(dw, xv.transpose().matmul(d))
+
+        graph = env.build_graph(build)
+        env.run(graph, 0)
+        return env.read_parameter(dz), env.read_parameter(dw), graph
+
+    got_z, got_w, graph = run(genv)
+    want_z, want_w, _ = run(cenv)
+    listing = next(iter(graph.__dict__["_schedules"].values())).describe()
+    assert "+the weight gradient X^T A over" in listing and int(listing.split()[0]) == 2, listing
+    assert rel_l2(got_z, want_z) <= TOL
+    assert rel_l2(got_w, want_w) <= TOL
+
+
 @pytest.mark.parametrize("rows,m,n,force,buffers", [
     (16384, 128, 260, "64,64,16,1,1,8", None), (32768, 128, 132, "128,64,32,2,2,8", None), (16384, 256, 388, "256,256,32,4,4,8", None),
     (8192, 512, 512, None, None), (16384, 256, 256, None, "3"), (16384, 256, 256, "128,128,32,2,2,8", None),

@@ -230,3 +230,27 @@ def test_the_sign_of_a_pre_activation_is_read_off_the_stored_activation():
     # cluster by cluster nothing is rewritten
     unfused = hip_backend.check_schedule(graph, fused=False)
     assert "PerElement (7 ops) [12544000]" in unfused and "2316." in unfused.splitlines()[-1], unfused.splitlines()[-1]
+
+
+def test_data_and_weight_gradient_of_a_layer_with_few_outputs_share_one_pass_over_the_activation():
+    def build(masked_by_x):
+        def fn(s, dy, x, w, other, dz, dw):
+            d, xv = _value(s, dy), _value(s, x)
+            p = d.matmul(_value(s, w).transpose())
+            mask = xv if masked_by_x else _value(s, other)
+            s.write_parameter_value(dz, mask.select_gt(0.0, p, p * 0.01))
+            s.write_parameter_value(dw, xv.transpose().matmul(d))
+        return fn
+
+    shapes = [[65536, 2], [65536, 128], [128, 2], [65536, 128], [65536, 128], [128, 2]]
+    unfused, fused = _listings(shapes, build(True))
+    # cluster by cluster: a short-k product, its consumer, the product over the rows in the reference's 1024-deep chunks
+    # and the sum of those
+    assert "short-k fma" in unfused and "chunks 64" in unfused and int(unfused.split()[0]) == 5
+    # fused: the weight gradient's 256 chunks are the row chunks of the data gradient's kernel; their sum is untouched
+    assert int(fused.split()[0]) == 2
+    assert "+the weight gradient X^T A over 256 chunks of 256 rows" in fused and "tall-k" not in fused
+    assert re.search(r"Reduce \(k=256\) \[1, 1, 128, 2\]", fused)
+    # a consumer that does not read the activation gains nothing from the pairing: both products stay as they are
+    _, apart = _listings(shapes, build(False))
+    assert "+the weight gradient" not in apart and "tall-k mfma 16x16x4" in apart
