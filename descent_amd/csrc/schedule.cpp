@@ -559,9 +559,13 @@ struct Planner {
             int64_t S = std::min<int64_t>(split_target / t64, g.k / 64);
             {
                 // a small output over a long k runs on the tall-k kernel, one workgroup of four waves per
-                // (chunk, batch): a thousand workgroups with at least 256 k each
+                // (chunk, batch): a thousand workgroups with at least 256 k each.  With eight or more 16x16 tiles the
+                // four waves' partial tiles take 32 KB or more of LDS and each workgroup ends with that much of a
+                // reduction: half as many workgroups with twice the rows (64x64 over k = 262144: 35.1 -> 30.5 us,
+                // 32x64 20.9 -> 19.0; 256 workgroups 39.7)
                 MatMulDims t = g;
-                t.chunks = std::min<int64_t>(std::max<int64_t>(1024 / g.batch, 1), g.k / 256);
+                const int64_t tk_target = ((g.m + 15) / 16) * ((g.n + 15) / 16) >= 8 ? 512 : 1024;
+                t.chunks = std::min<int64_t>(std::max<int64_t>(tk_target / g.batch, 1), g.k / 256);
                 if (t.chunks >= 2 && tallk_shape(t)) S = t.chunks;
             }
             if (S < 2) continue;
