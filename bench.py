@@ -81,6 +81,7 @@ def bench_matmul(env, m, n, k, steps, warmup, verify=False):
     w = workloads.matmul_epilogue(env, m, n, k, seed=2)
     wall = time_graph(env, w.graph, steps, warmup)
     avg_us, launches = env.backend.timing_query("MatMul")
+    all_us, _, _, all_n = env.backend.timing_work("")  # every launch of the step (a re-split product has two)
     report = env.backend.timing_report(0)
     env.backend.profile_reset()
     rel_err = verify_matmul_rows(env, w) if verify else None
@@ -96,6 +97,7 @@ def bench_matmul(env, m, n, k, steps, warmup, verify=False):
         "ms_per_step": 1e3 * wall / steps,
         "tflops_wall": w.flops * steps / wall / 1e12,
         "kernel_avg_us": avg_us,
+        "kernel_us_per_step": all_us / steps if all_n else None,
         "kernel_launches": launches,
         "tflops_kernel": (w.flops / (avg_us * 1e-6) / 1e12) if avg_us else None,
         "launches_per_step": sched.launch_count()[0],
@@ -228,12 +230,14 @@ def bench_elementwise(env, n, steps, warmup):
             "gbs_wall": nbytes * steps / wall / 1e9, "frac_hbm": nbytes / (avg_us * 1e-6) / 1e9 / HBM_PEAK_GBS}
 
 
-def bench_workload(env, build, steps, warmup, topn=8):
+def bench_workload(env, build, steps, warmup, topn=8, read_loss=False):
     """Step rate of one of the image-fit configurations, with the per-kernel table."""
     w = build(env)
     wall = time_then_profile(env, w.graph, steps, warmup)
     be = env.backend
     out = {"steps_per_s": steps / wall, "ms_per_step": 1e3 * wall / steps}
+    if read_loss:
+        out["loss_finite"] = bool(all(np.all(np.isfinite(env.read_parameter(p))) for p in w.scalars.values()))
     out["kernel_classes"] = class_rooflines(be, steps) if EVENT_PASS else {}
     report = be.timing_report(topn)
     be.profile_reset()
@@ -297,6 +301,46 @@ def bench_upload(env, n):
     return {"upload_gbs": a.nbytes / up / 1e9, "matmul_with_upload_tflops": w.flops / dt / 1e12, "ms_per_step_with_upload": dt * 1e3}
 
 
+def _compact_classes(classes):
+    """Kernel classes of a step, compact: microseconds per step, launches, and the fraction of the roof each class's
+    algorithmic work reaches (HBM always; fp32 MFMA where the class multiplies matrices)."""
+    out = {}
+    for name, row in classes.items():
+        c = {"us": round(row["us_per_step"], 1), "launches": round(row["launches_per_step"], 2), "frac_hbm": round(row["frac_hbm"], 3)}
+        if "frac_mfma" in row:
+            c["frac_mfma"] = round(row["frac_mfma"], 3)
+        out[name.split(" (")[0] if name.startswith("Multi (") else name] = c
+    return out
+
+
+def bench_configs(env, warmup=3):
+    """The configurations the headline does not cover, compact enough for the one JSON line: the other four
+    standalone matmul shapes (each verified on sampled rows against float64 after its timed region), the linear
+    classifier, both coordinate MLPs and the hash-grid fit (step rate, launches, per-class roofline fractions,
+    and the summed loss of the timed steps, which must be finite)."""
+    from descent_amd import workloads as _w
+
+    out = {"matmul": {}}
+    for (m, n, k), steps in (((1024, 1024, 1024), 50), ((4096, 4096, 4096), 20), ((1000, 128, 784), 50), ((262144, 256, 256), 20)):
+        r = bench_matmul(env, m, n, k, steps, warmup, verify=True)
+        ok = r["rel_l2_error_sampled_rows"] <= 1e-4
+        # a product of one launch: rate of that launch; of several (k re-split + the sum of its partials): of all of them
+        us = r["kernel_us_per_step"]
+        out["matmul"]["%dx%dx%d" % (m, n, k)] = {
+            "tflops_kernels": round(r["flops"] / (us * 1e-6) / 1e12, 2), "frac_mfma": round(r["flops"] / (us * 1e-6) / 1e12 / MFMA_FP32_PEAK_TFLOPS, 3),
+            "kernels_us": round(us, 2), "tflops_wall": round(r["tflops_wall"], 2), "launches": r["launches_per_step"],
+            "rel_l2_error_sampled_rows": r["rel_l2_error_sampled_rows"], "verified": bool(ok)}
+    builds = (("cfg1_linear_classifier_bs1000", lambda e: _w.linear_classifier(e), 200),
+              ("cfg4_coordinate_mlp_relu_pe_512", lambda e: _w.coordinate_mlp(e), 10),
+              ("cfg4_coordinate_mlp_siren_512", lambda e: _w.coordinate_mlp(e, variant="siren"), 10),
+              ("cfg5_hash_grid_2p18", lambda e: _w.hash_grid_fit(e), 20))
+    for name, build, steps in builds:
+        r, _ = bench_workload(env, build, steps, 2, read_loss=True)
+        out[name] = {"steps_per_s": round(r["steps_per_s"], 1), "ms_per_step": round(r["ms_per_step"], 4), "launches": r["launches_per_step"],
+                     "clusters": r["clusters"], "loss_sum_finite": r["loss_finite"], "kernel_classes": _compact_classes(r["kernel_classes"])}
+    return out
+
+
 def cpu_baseline_matmul(n: int, rows: int):
     """The CPU oracle (restatement of the reference's algorithm; the reference itself needs Rust + Vulkan) on
     a slab of `rows` rows of the same n^3 product, epilogue included, and on a few ConvNet train steps, all host
@@ -341,6 +385,7 @@ def main():
                                                   "alone and print its line (e.g. under rocprofv3 --pmc)")
     ap.add_argument("--all", action="store_true", help="also time the other matmul shapes and the ConvNet step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true", help="leave the other configurations out of the headline line")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only the streaming c=a*2+b kernel over 2^26 elements (counter calibration)")
     ap.add_argument("--cpu-rows", type=int, default=8192,
@@ -431,6 +476,7 @@ def main():
         # the other half of the headline metric: ConvNet (batch 1000) train steps per second
         conv = bench_convnet(env, max(args.steps, 200), args.warmup)
         sys.stderr.write(conv.pop("report"))
+    configs = bench_configs(env) if args.workload == "headline" and not args.no_configs else None
 
     cpu = None
     if not args.no_cpu_baseline:
@@ -464,12 +510,15 @@ def main():
         },
         "cpu_baseline": cpu,
         # 64 sampled rows of the C the timed launches wrote, against a float64 product of the operands read back
-        "verified": True,
+        "verified": bool(head["rel_l2_error_sampled_rows"] <= 1e-4),
         "rel_l2_error_sampled_rows": head["rel_l2_error_sampled_rows"],
     }
     if conv is not None:
         # the first half of the headline metric: ConvNet (batch 1000) train steps per second, with the step's own roofline
         line["convnet_bs1000"] = conv
+    if configs is not None:
+        # the remaining configurations, timed in this same run (matmul shapes verified on sampled rows)
+        line["configs"] = configs
     if extra:
         line["extra"] = extra
     print(json.dumps(line))

@@ -574,7 +574,11 @@ int dsc_schedule_create(dsc_ctx* ctx, const dsc_schedule_desc* desc, uint32_t fl
 }
 
 int dsc_schedule_destroy(dsc_ctx* ctx, dsc_schedule* s) {
-    if (ctx && s) s->s.release_replay_buffers(&ctx->c);  // the region and spares of a schedule that replays graphs
+    if (ctx && s) {
+        // captured graphs may still be running, and the region they write goes back to the heap here
+        if (s->s.has_captured_graphs()) (void)hipStreamSynchronize(ctx->c.stream);
+        s->s.release_replay_buffers(&ctx->c);  // the region and spares of a schedule that replays graphs
+    }
     delete s;
     return DSC_OK;
 }

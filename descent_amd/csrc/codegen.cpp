@@ -2705,7 +2705,9 @@ string gen_matmul(Emitter& em, Generated* out) {
         const int nbuf = !e ? 2 : e[0] == '2' ? 2 : e[0] == '3' ? 3 : 0;
         // every k range whole k-tiles; a tile may reach past M or N (it repeats the last row / the last four columns),
         // as long as the product is at least one piece wide and tall
-        const bool whole = chunk_k % t.bk == 0 && g.k % chunk_k == 0 && g.m >= 4 && g.n >= 4;
+        // (a descriptor may name more chunks than k has tiles for: the last chunks then start at or past k and the
+        // reference writes zero partials for them; this path does not clamp k, so they stay on the register path)
+        const bool whole = chunk_k % t.bk == 0 && kchunks * chunk_k == g.k && g.m >= 4 && g.n >= 4;
         const bool even = (t.bm * t.bk / 4) % nt == 0 && (t.bn * t.bk / 4) % nt == 0 && (t.bk & (t.bk - 1)) == 0;
         // (column sums are combined through the one free tile buffer: a 16-byte partial per thread has to fit it)
         // (weight gradients with their bias sums: 1024x1024 grid, layers of 256, 309 -> 318 steps/s)

@@ -2996,6 +2996,16 @@ int Schedule::run_replayed(Context* ctx, dsc_buf* params, uint32_t rand_seed, bo
     const int rc = replay_or_capture(ctx, plan.launches, plan.pointers, rand_seed);
     if (rc != DSC_OK) return rc;
     for (int slot : plan.swapped) std::swap(params[slot], replay_spare[slot]);
+    // a written parameter that came in without a buffer (an output nobody wrote before the first run) leaves no old
+    // buffer behind to be the next run's spare: give its slot a new one, or every later placement would fail
+    for (auto& io : outputs) {
+        if (replay_spare[io.param] || !params[io.param]) continue;
+        replay_spare[io.param] = ctx->heap.alloc(std::max<size_t>(node_bytes[io.node], 4));
+        if (!replay_spare[io.param]) {
+            give_back();  // out of memory: the allocating run() serves this schedule from now on
+            break;
+        }
+    }
     return DSC_OK;
 }
 

@@ -61,6 +61,7 @@ struct Schedule {
     std::vector<dsc_buf> replay_spare;  // per parameter slot, 0 where the slot is not written
     bool replay_fixed = true;           // cleared when this graph cannot be laid out that way
     void release_replay_buffers(Context* ctx);  // before the schedule goes, while its context is alive
+    bool has_captured_graphs() const { return !captured.empty(); }
     ~Schedule();
 
     int n_nodes = 0, n_params = 0, n_clusters = 0;

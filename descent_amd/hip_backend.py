@@ -7,6 +7,7 @@ present, constructing `HipBackend` raises.
 from __future__ import annotations
 
 import ctypes as C
+import weakref
 import os
 from typing import List
 
@@ -170,6 +171,21 @@ class HipSchedule:
         flags = schedule_flags(fused)
         check(lib().dsc_schedule_create(backend._ctx, C.byref(self._ms.desc), flags, C.byref(self._handle)))
         self._slots = (C.c_uint64 * max(1, len(self.params)))()
+        backend._schedules.add(self)
+
+    def close(self) -> None:
+        """dsc_schedule_destroy, while the context the schedule was created on is still alive (the backend closes its
+        live schedules before it destroys the context): graph executables, the replay region and the spare buffers of
+        a schedule that replays HIP graphs go back with it."""
+        handle, self._handle = self._handle, C.c_void_p()
+        if handle and self._backend._ctx:
+            lib().dsc_schedule_destroy(self._backend._ctx, handle)
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
     def run(self, handles: List[int], rand_seed: int) -> List[int]:
         for i, h in enumerate(handles):
@@ -215,8 +231,11 @@ class HipBackend:
         check(lib().dsc_ctx_create(device, C.byref(self._ctx)))
         self._kernels = {}
         self._pinned = {}
+        self._schedules = weakref.WeakSet()
 
     def close(self):
+        for schedule in list(self._schedules):
+            schedule.close()
         if self._ctx:
             lib().dsc_ctx_destroy(self._ctx)
             self._ctx = C.c_void_p()

@@ -348,6 +348,10 @@ typedef struct dsc_schedule dsc_schedule;
                                            the one that holds dC and the input tile in LDS (for parity tests) */
 
 int dsc_schedule_create(dsc_ctx* ctx, const dsc_schedule_desc* desc, uint32_t flags, dsc_schedule** out);
+/* Destroy every schedule BEFORE the context it was created on: dsc_schedule_destroy returns the schedule's replay
+   region and spare buffers to that context's heap, and dsc_ctx_destroy does not know the context's schedules.  A
+   schedule destroyed after its context is a use of freed memory.  (The reference has no such object: its
+   Environment owns device and kernel cache together and drops them in one place, src/environment.rs:523-528.) */
 int dsc_schedule_destroy(dsc_ctx* ctx, dsc_schedule* s);
 /* Environment::run (environment.rs:326-516). `params[slot]` holds each parameter's current buffer (0 if
  * none) and is updated in place with the buffers the run leaves in the parameters. */

@@ -246,8 +246,21 @@ fn take_string(p: *mut c_char) -> String {
 #[derive(Debug, Clone, Copy, PartialEq, Eq, Hash)]
 pub struct BufferId(pub dsc_buf);
 
+/// Owner of the library context.  `HipDevice` and every `HipSchedule` created on it share one of these, so the
+/// context is destroyed after the last of them: `dsc_schedule_destroy` hands a schedule's buffers back to the
+/// context's heap and must find it alive.
+struct ContextHandle(*mut dsc_ctx);
+
+impl Drop for ContextHandle {
+    /// `Drop for Environment` waits for the device (src/environment.rs:523-528); dsc_ctx_destroy does and frees all.
+    fn drop(&mut self) {
+        unsafe { dsc_ctx_destroy(self.0) };
+    }
+}
+
 pub struct HipDevice {
     ctx: *mut dsc_ctx,
+    owner: std::rc::Rc<ContextHandle>,
 }
 
 impl HipDevice {
@@ -259,7 +272,7 @@ impl HipDevice {
         check(unsafe { dsc_ctx_caps(ctx, caps.as_mut_ptr()) }, "dsc_ctx_caps");
         // src/kernel.rs:954 asserts shader float atomics when a ScatterAdd module is built; always present here
         assert_eq!(unsafe { caps.assume_init() }.has_float_atomic_add, 1);
-        Self { ctx }
+        Self { ctx, owner: std::rc::Rc::new(ContextHandle(ctx)) }
     }
 
     pub fn raw(&self) -> *mut dsc_ctx {
@@ -321,25 +334,19 @@ impl HipDevice {
     }
 }
 
-impl Drop for HipDevice {
-    /// `Drop for Environment` waits for the device (src/environment.rs:523-528); dsc_ctx_destroy does and frees all.
-    fn drop(&mut self) {
-        unsafe { dsc_ctx_destroy(self.ctx) };
-    }
-}
-
 /// A whole `Graph` handed to the library once (see `kernel_marshal::MarshalledSchedule`); `run` is what
 /// `Environment::run` calls per step.
 pub struct HipSchedule {
     handle: *mut dsc_schedule,
     ctx: *mut dsc_ctx,
+    _owner: std::rc::Rc<ContextHandle>, // keeps the context alive until this schedule has been destroyed
 }
 
 impl HipSchedule {
     pub fn new(device: &HipDevice, desc: &dsc_schedule_desc, flags: u32) -> Self {
         let mut handle = std::ptr::null_mut();
         check(unsafe { dsc_schedule_create(device.raw(), desc, flags, &mut handle) }, "dsc_schedule_create");
-        Self { handle, ctx: device.raw() }
+        Self { handle, ctx: device.raw(), _owner: device.owner.clone() }
     }
 
     /// `params[slot]` = current buffer of each parameter (0 = none); updated in place (src/environment.rs:506-515).
@@ -364,6 +371,7 @@ impl HipSchedule {
 }
 
 impl Drop for HipSchedule {
+    /// Runs before `_owner` is released (fields drop after `drop` returns), so the context is still there.
     fn drop(&mut self) {
         unsafe { dsc_schedule_destroy(self.ctx, self.handle) };
     }

@@ -20,7 +20,7 @@
 
 use crate::common::*;
 use crate::device::hip::*;
-use crate::kernel_marshal::MarshalledSchedule;
+use crate::kernel_marshal::{graph_fingerprint, MarshalledSchedule};
 use slotmap::SlotMap;
 use std::{
     cell::RefCell,
@@ -94,9 +94,10 @@ impl io::BufRead for ParameterReader {
     }
 }
 
-/// One schedule per `Graph`, created the first time the graph runs.  The key is the address of the graph's cluster
-/// list, which is stable for the life of a `Graph` (graphs are built once and run many times: examples/fashion_mnist/
-/// main.rs:360-448).
+/// One schedule per distinct graph, created the first time such a graph runs (graphs are built once and run many
+/// times: examples/fashion_mnist/main.rs:360-448).  The key is `graph_fingerprint`, a hash of the graph's content:
+/// nothing of the `Graph` is held, so a graph that is dropped and rebuilt finds its schedule again, and a different
+/// graph that happens to reuse the old one's memory cannot be mistaken for it.
 struct GraphSchedule {
     marshalled: Box<MarshalledSchedule>,
     schedule: HipSchedule,
@@ -106,7 +107,7 @@ struct GraphSchedule {
 pub struct Environment {
     device: HipDevice,
     parameters: SharedParameters,
-    schedules: HashMap<usize, GraphSchedule>,
+    schedules: HashMap<u64, GraphSchedule>,
 }
 
 impl Default for Environment {
@@ -152,7 +153,7 @@ impl Environment {
     /// inside `dsc_schedule_run`, over the fused launch list; this side only passes the parameters' buffers in and
     /// takes the new ones back.
     pub fn run(&mut self, graph: &Graph, rand_seed: u32) {
-        let key = graph.clusters_sorted.as_ptr() as usize;
+        let key = graph_fingerprint(graph);
         let device = &self.device;
         let entry = self.schedules.entry(key).or_insert_with(|| {
             let marshalled = MarshalledSchedule::new(graph);

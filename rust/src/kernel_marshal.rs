@@ -290,6 +290,57 @@ pub(crate) struct MarshalledSchedule {
     outputs: Vec<dsc_param_io>,
 }
 
+/// Identifies a graph by content: a hash over everything `MarshalledSchedule::new` reads (the element count of
+/// every node, the parameter behind each Input / Output node, and per cluster its kernel descriptor, its input and
+/// output nodes and their initial states).  Two graphs with the same fingerprint marshal to the same schedule and
+/// the same parameter slots, so a schedule cached under it is valid for either.  An address of something inside the
+/// `Graph` is not: a graph dropped and rebuilt (per epoch, in a loop) can put its vectors where the old one's were.
+/// The reference pays the same kind of cost per run: one `HashMap<GenericKernel, _>` lookup per cluster
+/// (src/kernel.rs:1050).
+pub(crate) fn graph_fingerprint(graph: &Graph) -> u64 {
+    use std::hash::{Hash, Hasher};
+    let mut h = std::collections::hash_map::DefaultHasher::new();
+    graph.ops.node_bound().hash(&mut h);
+    for node_ref in graph.ops.node_references() {
+        let node_id = node_ref.id();
+        node_id.index().hash(&mut h);
+        node_ref.weight().shape.element_count().hash(&mut h);
+        match node_ref.weight().op {
+            Op::Input { parameter_id } => (1u8, parameter_id).hash(&mut h),
+            Op::Output { parameter_id } => {
+                (2u8, parameter_id).hash(&mut h);
+                for source in get_arg_sources(&graph.ops, node_id).iter() {
+                    source.node_id.index().hash(&mut h);
+                }
+            }
+            _ => 0u8.hash(&mut h),
+        }
+    }
+    graph.clusters_sorted.len().hash(&mut h);
+    for cluster_id in graph.clusters_sorted.iter().copied() {
+        let cluster = &graph.clusters[cluster_id];
+        cluster.kernel.hash(&mut h);
+        cluster.inputs.len().hash(&mut h);
+        for n in cluster.inputs.iter() {
+            n.index().hash(&mut h);
+        }
+        cluster.outputs.len().hash(&mut h);
+        for output in cluster.outputs.iter() {
+            output.node_id.index().hash(&mut h);
+            match output.initial_state {
+                InitialState::CopyFrom(src_node_id) => {
+                    (1u8, src_node_id.index()).hash(&mut h);
+                    if let Op::Literal(value) = graph.ops[src_node_id].op {
+                        literal_bits(value).hash(&mut h);
+                    }
+                }
+                _ => 0u8.hash(&mut h),
+            }
+        }
+    }
+    h.finish()
+}
+
 impl MarshalledSchedule {
     pub(crate) fn new(graph: &Graph) -> Box<Self> {
         let mut params: Vec<ParameterId> = Vec::new();

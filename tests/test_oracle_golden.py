@@ -362,6 +362,191 @@ def test_concat_along_each_axis():
         assert np.array_equal(env.read_parameter(cp), want)
 
 
+# ---- u32 arithmetic, conversions, transcendentals (src/kernel.rs:470-520 per-element op table) ----------------
+def _u32_param(env, name, bits):
+    return env.static_parameter_with_data([bits.size], name, bits.astype(np.uint32).view(np.float32))
+
+
+def test_u32_ops_wrap_and_are_unsigned():
+    """UAdd / UMul / URem / UBitXor on bit-cast words: full-range operands, so a signed remainder, a missing
+    wrap-around or swapped operands of `%` give different bits than numpy's uint32 arithmetic."""
+    rng = np.random.default_rng(21)
+    n = 4096
+    a = rng.integers(0, 1 << 32, n, dtype=np.uint64).astype(np.uint32)
+    b = rng.integers(1, 1 << 32, n, dtype=np.uint64).astype(np.uint32)
+    b[: n // 2] = rng.integers(1, 1 << 20, n // 2)  # small moduli beside full-range ones
+    a[:8] = [0, 1, 0x7FFFFFFF, 0x80000000, 0xFFFFFFFF, 0xFFFFFFFE, 0x80000001, 12345]
+    env = _env()
+    ap, bp = _u32_param(env, "a", a), _u32_param(env, "b", b)
+    outs = {k: env.static_parameter([n], k) for k in ("add", "mul", "rem", "xor", "mixed")}
+
+    def build(s):
+        x, y = s.parameter_value(ap).to_u32_bits(), s.parameter_value(bp).to_u32_bits()
+        s.write_parameter_value(outs["add"], (x + y).to_f32_bits())
+        s.write_parameter_value(outs["mul"], (x * y).to_f32_bits())
+        s.write_parameter_value(outs["rem"], (x % y).to_f32_bits())
+        s.write_parameter_value(outs["xor"], (x ^ y).to_f32_bits())
+        s.write_parameter_value(outs["mixed"], (((x + 1) ^ (y * 1526263 + 1526263)) % (1 << 19)).to_f32_bits())
+
+    env.run(env.build_graph(build), 0)
+    got = {k: env.read_parameter(v).view(np.uint32) for k, v in outs.items()}
+    with np.errstate(over="ignore"):
+        assert np.array_equal(got["add"], a + b)
+        assert np.array_equal(got["mul"], a * b)
+        assert np.array_equal(got["rem"], a % b)
+        assert np.array_equal(got["xor"], a ^ b)
+        assert np.array_equal(got["mixed"], ((a + np.uint32(1)) ^ (b * np.uint32(1526263) + np.uint32(1526263))) % np.uint32(1 << 19))
+    assert not np.array_equal(a % b, (a.view(np.int32) % b.view(np.int32)).view(np.uint32))  # signedness is visible
+
+
+def test_uint_float_conversions():
+    """FloatToUint truncates toward zero; UintToFloat reads the word as unsigned (values above 2^31 stay
+    positive) and rounds to nearest even above 2^24 -- both against numpy's conversions."""
+    rng = np.random.default_rng(22)
+    n = 2048
+    bits = rng.integers(0, 1 << 32, n, dtype=np.uint64).astype(np.uint32)
+    bits[:6] = [0, 1, (1 << 24) + 1, (1 << 24) + 3, 0x80000000, 0xFFFFFFFF]
+    vals = (rng.random(n, dtype=np.float32) * np.float32(4.0e9)).astype(np.float32)
+    vals[:5] = [0.0, 0.99999994, 1.0, 16777217.0, 2147483648.0]
+    env = _env()
+    bp = _u32_param(env, "b", bits)
+    vp = env.static_parameter_with_data([n], "v", vals)
+    as_float, as_uint = env.static_parameter([n], "f"), env.static_parameter([n], "u")
+
+    def build(s):
+        s.write_parameter_value(as_float, s.parameter_value(bp).to_u32_bits().into_f32())
+        s.write_parameter_value(as_uint, s.parameter_value(vp).into_u32().to_f32_bits())
+
+    env.run(env.build_graph(build), 0)
+    assert np.array_equal(env.read_parameter(as_float), bits.astype(np.float32))
+    assert np.array_equal(env.read_parameter(as_uint).view(np.uint32), vals.astype(np.uint32))
+
+
+@pytest.mark.parametrize("grid_size,entry_count", [(16, 1 << 19), (80, 1 << 19), (111, 1 << 14), (2048, 1 << 19)])
+def test_hash_grid_corner_indices_and_fractions_against_numpy(grid_size, entry_count):
+    """The four corner indices and the fractional position of a hash-grid level
+    (examples/image_fit/main.rs:132-170) for a dense level (stride = points per side) and for hashed ones
+    (stride = 1526263), bit for bit against numpy uint32 / float32 arithmetic written from the formula."""
+    rng = np.random.default_rng(grid_size)
+    m = 5000
+    x = (rng.random((m, 2), dtype=np.float32) * np.float32(2.0 * (1.0 - 1e-6)) - np.float32(1.0)).astype(np.float32)
+    points = grid_size + 1
+    dense = entry_count >= points * points
+    entries = min(entry_count, points * points)
+    stride = points if dense else workloads.HASH_PRIME
+    assert workloads.HASH_PRIME == 1526263
+    env = _env()
+    xp = env.static_parameter_with_data([m, 2], "x", x)
+    idx = [env.static_parameter([m], "i%d" % i) for i in range(4)]
+    frac = env.static_parameter([m, 2], "f")
+
+    def build(s):
+        cf = (s.parameter_value(xp) * 0.5 + 0.5) * float(grid_size)
+        c = cf.into_u32()
+        s.write_parameter_value(frac, cf - c.into_f32())
+        c0, c1 = c.lock_axis(-1, 0, False), c.lock_axis(-1, 1, False)
+        corners = (((c0 + 0) ^ (c1 * stride + 0)), ((c0 + 1) ^ (c1 * stride + 0)),
+                   ((c0 + 0) ^ (c1 * stride + stride)), ((c0 + 1) ^ (c1 * stride + stride)))
+        for out, corner in zip(idx, corners):
+            s.write_parameter_value(out, (corner % entries).to_f32_bits())
+
+    env.run(env.build_graph(build), 0)
+    cf = ((x * np.float32(0.5) + np.float32(0.5)) * np.float32(grid_size)).astype(np.float32)
+    c = cf.astype(np.uint32)
+    assert np.array_equal(env.read_parameter(frac), cf - c.astype(np.float32))
+    c0, c1, st = c[:, 0], c[:, 1], np.uint32(stride)
+    with np.errstate(over="ignore"):
+        want = [(c0 + np.uint32(di)) ^ (c1 * st + np.uint32(dj) * st) for dj in (0, 1) for di in (0, 1)]
+    for out, w in zip(idx, want):
+        got = env.read_parameter(out).view(np.uint32).ravel()
+        assert np.array_equal(got, w % np.uint32(entries))
+    if dense:  # a dense level's index is the row-major grid point: y * points + x, never wrapped
+        got = env.read_parameter(idx[3]).view(np.uint32).ravel()
+        assert np.array_equal(got, (c0 + 1) ^ ((c1 + 1) * st)) and got.max() < entries + points
+
+
+def test_hash_level_sizes_fixture():
+    """The sixteen level resolutions are committed as data with the f32 evaluation of the reference's formula
+    beside them (examples/image_fit/main.rs:222-228: b = exp((ln 2048 - ln 16) / 15), size = trunc(16 * b^i) with
+    `powi` as repeated squaring).  The last product lands within one f32 step of 2048, so the top level is 2047
+    or 2048 depending on the libm in use; the first fifteen are fixed."""
+    import json
+    import os
+
+    fixture = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "hash_level_sizes.json")))
+    assert tuple(fixture["sizes"]) == workloads.HASH_LEVEL_SIZES
+    f = np.float32
+    b = f(np.exp(f((np.log(f(2048)) - np.log(f(16))) / f(15))))
+
+    def powi(a, n):
+        r = f(1)
+        while True:
+            if n & 1:
+                r = f(r * a)
+            n //= 2
+            if n == 0:
+                return r
+            a = f(a * a)
+
+    products = [float(f(16) * powi(b, i)) for i in range(16)]
+    assert [int(v) for v in products[:15]] == fixture["sizes"][:15]
+    assert int(products[15]) in (2047, 2048) and fixture["sizes"][15] == 2048
+    assert np.allclose(products, fixture["f32_products"], rtol=1e-6)
+
+
+def test_positional_encoding_sin_and_pow_against_numpy():
+    """sin(x * 2^i * pi + {0, pi/2}) (examples/image_fit/main.rs:259-275): `pow(2, i)` must be the exact power of
+    two, the feature order [coordinate][phase][frequency], and Sin within an ulp or two of float64's sine of the
+    same f32 argument."""
+    rng = np.random.default_rng(23)
+    m, freq_count = 300, 16
+    x = rng.random((m, 2), dtype=np.float32)
+    env = _env()
+    xp = env.static_parameter_with_data([m, 2], "x", x)
+    out = env.static_parameter([m, 4 * freq_count], "pe")
+    powers = env.static_parameter([freq_count], "p")
+
+    def build(s):
+        s.write_parameter_value(out, workloads.positional_encoding(s.parameter(xp), freq_count).value())
+        s.write_parameter_value(powers, s.literal(2.0).pow(s.coord(freq_count)).value())
+
+    env.run(env.build_graph(build), 0)
+    assert np.array_equal(env.read_parameter(powers), 2.0 ** np.arange(freq_count, dtype=np.float32))
+    pi32 = np.float32(np.pi)
+    freq = (np.float32(2.0) ** np.arange(freq_count, dtype=np.float32)) * pi32
+    phase = (np.arange(2, dtype=np.float32) * np.float32(0.5) * pi32).astype(np.float32)
+    arg = (x[:, :, None, None] * freq[None, None, None, :]).astype(np.float32) + phase[None, None, :, None]
+    want = np.sin(arg.astype(np.float32).astype(np.float64)).reshape(m, 4 * freq_count)
+    got = env.read_parameter(out).astype(np.float64)
+    assert np.max(np.abs(got - want)) <= 2.5e-7
+    # the phase-pi/2 half is the cosine of the same product: a dropped phase or swapped axes fails here
+    cos_half = got.reshape(m, 2, 2, freq_count)[:, :, 1, :3]
+    assert np.max(np.abs(cos_half - np.cos((x[:, :, None] * freq[None, None, :3]).astype(np.float64)))) <= 1e-5
+
+
+def test_sin_cos_pow_ops_against_numpy():
+    rng = np.random.default_rng(24)
+    n = 4096
+    x = (rng.standard_normal(n) * 40).astype(np.float32)
+    base = (rng.random(n, dtype=np.float32) * 3 + np.float32(0.1)).astype(np.float32)
+    expo = (rng.standard_normal(n) * 2).astype(np.float32)
+    env = _env()
+    xp, bp, ep = (env.static_parameter_with_data([n], k, v) for k, v in (("x", x), ("b", base), ("e", expo)))
+    sp, cp, pp = (env.static_parameter([n], k) for k in ("s", "c", "p"))
+
+    def build(s):
+        s.write_parameter_value(sp, s.parameter_value(xp).sin())
+        s.write_parameter_value(cp, s.parameter_value(xp).cos())
+        s.write_parameter_value(pp, s.parameter_value(bp).pow(s.parameter_value(ep)))
+
+    env.run(env.build_graph(build), 0)
+    x64 = x.astype(np.float64)
+    assert np.max(np.abs(env.read_parameter(sp) - np.sin(x64))) <= 1.5e-7
+    assert np.max(np.abs(env.read_parameter(cp) - np.cos(x64))) <= 1.5e-7
+    assert rel_l2(env.read_parameter(pp), base.astype(np.float64) ** expo.astype(np.float64)) <= 2e-7
+    assert env.read_parameter(pp)[0] != np.float32(expo[0].astype(np.float64) ** base[0].astype(np.float64))  # base ^ exponent, not swapped
+
+
 # ---- optimisers ------------------------------------------------------------------------------------------------
 def _quadratic_problem(env, opt_factory, steps):
     """loss = sum((theta * x)^2) / m with fixed x; returns theta after `steps` updates."""

@@ -254,3 +254,20 @@ def test_data_and_weight_gradient_of_a_layer_with_few_outputs_share_one_pass_ove
     # a consumer that does not read the activation gains nothing from the pairing: both products stay as they are
     _, apart = _listings(shapes, build(False))
     assert "+the weight gradient" not in apart and "tall-k mfma 16x16x4" in apart
+
+
+def test_surplus_k_chunks_keep_the_bounds_checked_register_path():
+    """A MatMul descriptor may name more k chunks than k has tiles for (k = 64 in 3 chunks of 32: the third starts at
+    k).  The tiles-straight-into-LDS path does not clamp k, so such a product must not take it; the same product with
+    chunks that cover k exactly does."""
+    from descent_amd import kernel as K
+    from descent_amd.shape import BATCHES, Shape
+
+    def direct(chunks, k):
+        kern = K.MatMulKernel(Shape((chunks, 1, 256, 256)), BATCHES, Shape((1, 256, k)).identity_view(), Shape((1, k, 256)).identity_view())
+        return int(re.search(r"#define MM_DIRECT (\d+)", hip_backend.codegen_source(kern)).group(1))
+
+    assert direct(2, 64) > 0
+    assert direct(3, 64) == 0
+    assert direct(3, 96) > 0
+    assert direct(5, 128) == 0  # chunks of 32: 5 * 32 > 128
