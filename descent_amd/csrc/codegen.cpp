@@ -4,6 +4,7 @@
 #include <cctype>
 #include <cstdio>
 #include <cstdlib>
+#include <functional>
 #include <map>
 #include <sstream>
 
@@ -303,6 +304,161 @@ struct Emitter {
         }
         funcs << "DSC_INLINE float " << name << "(" << decl << params_decl() << ") {\n" << body.str() << "}\n\n";
         return name;
+    }
+
+    // ---- four consecutive elements at once ------------------------------------------------------------
+    // A consumer that wants elements id .. id + 3 of a source, id a multiple of four and the four of them inside one
+    // run of the innermost axis of every view on the way, gets them from ONE evaluation: the index arithmetic of each
+    // view (the divisions by its extents) is done once for the quad, a buffer is read with one 16-byte load where its
+    // innermost axis walks memory (or one word, where the view repeats an element along that axis), and only the
+    // arithmetic is done four times.  The reference has no counterpart: it evaluates one element per invocation
+    // (src/kernel.rs:196-383).  Everything returns "" where a quad cannot be formed; callers then fall back on four
+    // single evaluations.
+    //
+    // The view's element for the quad that starts at coordinates `coord` (the last one a multiple of four).
+    string load_view4(const Source& s, const dsc_view& v, const std::vector<string>& coord) {
+        const int L = v.out_shape.rank - 1;
+        if (L < 0 || v.out_shape.dims[L] % 4 != 0) return "";
+        int64_t base = 0, coef[DSC_MAX_DIM];
+        if (!affine_form(v, &base, coef)) return "";
+        if (v.out_shape.dims[L] > 1 && coef[L] == 0) {  // the same element four times
+            const string one = load_view(s, v, coord);
+            return "dsc_splat4(" + one + ")";
+        }
+        if (coef[L] != 1) return "";
+        if (s.buffer >= 0) {
+            bool aligned = base % 4 == 0;
+            for (int j = 0; j < L; ++j)
+                if (v.out_shape.dims[j] > 1 && coef[j] % 4 != 0) aligned = false;
+            const string idx = index_expr(v, coord);
+            const string b = "b" + to_string(s.buffer);
+            if (aligned) return "*(const float4*)(" + b + " + " + idx + ")";
+            return "dsc_load4_unaligned(" + b + " + " + idx + ")";
+        }
+        IndexForm form = index_form(v, coord);
+        if (!form.valid || form.names.empty() || form.names.back() != coord[L] || form.coefs.back() != 1) return "";
+        const string fn = instantiate4(s.virt, form);
+        if (fn.empty()) return "";
+        string args;
+        for (auto& n : form.names) args += n + ", ";
+        return fn + "(" + args + params_pass() + ")";
+    }
+
+    // The float4 counterpart of `instantiate`: elements id .. id + 3 of virtual producer `virt`, where the form's last
+    // term is the quad's coordinate (coefficient one, a multiple of four at every call) and every other term moves the
+    // id by a multiple of four.  "" when the producer cannot be evaluated that way.
+    string instantiate4(int virt, const IndexForm& form) {
+        if (!form.valid || form.names.empty() || form.coefs.back() != 1 || form.extents.back() % 4 != 0 || form.base % 4 != 0) return "";
+        for (size_t t = 0; t + 1 < form.names.size(); ++t)
+            if (form.coefs[t] % 4 != 0) return "";
+        string sig = "q" + to_string(virt) + "|" + S(form.base);
+        for (size_t t = 0; t < form.names.size(); ++t) sig += "," + S(form.coefs[t]) + "x" + S(form.extents[t]);
+        auto it = instances.find(sig);
+        if (it != instances.end()) return it->second;
+        const Virtual& vi = fk.virtuals[virt];
+        const dsc_kernel_desc& pd = vi.pe.raw();
+        if (pd.kind != DSC_KERNEL_PER_ELEMENT) return instances[sig] = "";
+        const string name = "virt" + to_string(virt) + "_" + to_string(instances.size()) + "_x4";
+        instances[sig] = name;  // (a producer never reads itself: the graph of virtuals is acyclic)
+        IndexForm local = form;
+        string decl, gid = S(form.base);
+        for (size_t t = 0; t < form.names.size(); ++t) {
+            local.names[t] = "a" + to_string(t);
+            decl += "int a" + to_string(t) + ", ";
+            gid += " + (" + S(form.coefs[t]) + ")*a" + to_string(t);
+        }
+        std::ostringstream body;
+        body << "    const int gid = " << gid << ";\n";
+        if (!emit_pe4(body, pd, vi.inputs, "gid", "v", &local)) return instances[sig] = "";
+        body << "    return make_float4(vt" << vi.out_op << "[0], vt" << vi.out_op << "[1], vt" << vi.out_op << "[2], vt" << vi.out_op << "[3]);\n";
+        funcs << "DSC_INLINE float4 " << name << "(" << decl << params_decl() << ") {\n" << body.str() << "}\n\n";
+        return name;
+    }
+
+    // emit_pe for the quad gid .. gid + 3 (gid a multiple of four): op i is left in the array <pfx>t<i>[4].  False
+    // when an op or a load cannot be done for a quad (nothing usable has been emitted then).
+    bool emit_pe4(std::ostream& out, const dsc_kernel_desc& pe, const std::vector<Source>& srcs, const string& gid, const string& pfx,
+                  const IndexForm* form) {
+        std::ostringstream o;
+        std::vector<std::pair<dsc_shape, std::vector<string>>> sets;
+        auto coords_for = [&](const dsc_shape& shape) -> std::vector<string> {
+            for (auto& s : sets)
+                if (same_shape(s.first, shape)) return s.second;
+            const string cp = pfx + "c" + to_string(sets.size()) + "_";
+            std::vector<string> names;
+            if (form) names = emit_coords_separable(o, shape, *form, cp);
+            if (names.empty()) names = emit_coords(o, shape, gid, cp);
+            sets.emplace_back(shape, names);
+            return names;
+        };
+        auto T = [&](int i) { return pfx + "t" + to_string(i); };
+        auto each = [&](int i, const std::function<string(int)>& rhs) {
+            o << "    const float " << T(i) << "[4] = {" << rhs(0) << ", " << rhs(1) << ", " << rhs(2) << ", " << rhs(3) << "};\n";
+        };
+        auto E = [&](int i, int e) { return T(i) + "[" + to_string(e) + "]"; };
+        for (int i = 0; i < pe.n_ops; ++i) {
+            const dsc_pe_op& op = pe.ops[i];
+            switch (op.kind) {
+            case DSC_PE_LOAD: {
+                const dsc_view& v = pe.inputs[op.input_index];
+                const int L = v.out_shape.rank - 1;
+                if (L < 0 || v.out_shape.dims[L] % 4 != 0) return false;
+                const Source& src = srcs[op.input_index];
+                string q;
+                if (is_identity(v) && src.buffer >= 0) q = "*(const float4*)(b" + to_string(src.buffer) + " + " + gid + ")";
+                else if (is_identity(v) && form && form->valid) {
+                    // the producer's ids are this function's: hand the coordinates on as they came
+                    const string fn = instantiate4(src.virt, *form);
+                    if (!fn.empty()) {
+                        string args;
+                        for (auto& n : form->names) args += n + ", ";
+                        q = fn + "(" + args + params_pass() + ")";
+                    }
+                }
+                if (q.empty()) q = load_view4(src, v, coords_for(v.out_shape));
+                if (q.empty()) return false;
+                o << "    const float4 " << T(i) << "q = " << q << ";\n";
+                o << "    const float " << T(i) << "[4] = {" << T(i) << "q.x, " << T(i) << "q.y, " << T(i) << "q.z, " << T(i) << "q.w};\n";
+                break;
+            }
+            case DSC_PE_LITERAL_F32:
+            case DSC_PE_LITERAL_U32: each(i, [&](int) { return "U2F(" + hex32(op.bits) + ")"; }); break;
+            case DSC_PE_UNARY: {
+                const int a = op.args[0];
+                switch (op.op) {
+                case DSC_UN_MOV: each(i, [&](int e) { return E(a, e); }); break;
+                case DSC_UN_NEG: each(i, [&](int e) { return "-" + E(a, e); }); break;
+                case DSC_UN_SQRT: each(i, [&](int e) { return "sqrtf(" + E(a, e) + ")"; }); break;
+                case DSC_UN_FLOAT_TO_UINT: each(i, [&](int e) { return "U2F((uint)" + E(a, e) + ")"; }); break;
+                case DSC_UN_UINT_TO_FLOAT: each(i, [&](int e) { return "(float)F2U(" + E(a, e) + ")"; }); break;
+                default: return false;  // transcendental producers stay on the single-element path
+                }
+                break;
+            }
+            case DSC_PE_BINARY: {
+                const int a = op.args[0], b = op.args[1];
+                switch (op.op) {
+                case DSC_BIN_ADD: each(i, [&](int e) { return E(a, e) + " + " + E(b, e); }); break;
+                case DSC_BIN_SUB: each(i, [&](int e) { return E(a, e) + " - " + E(b, e); }); break;
+                case DSC_BIN_MUL: each(i, [&](int e) { return E(a, e) + " * " + E(b, e); }); break;
+                case DSC_BIN_DIV: each(i, [&](int e) { return E(a, e) + " / " + E(b, e); }); break;
+                case DSC_BIN_UADD: each(i, [&](int e) { return "U2F(F2U(" + E(a, e) + ") + F2U(" + E(b, e) + "))"; }); break;
+                case DSC_BIN_UMUL: each(i, [&](int e) { return "U2F(F2U(" + E(a, e) + ") * F2U(" + E(b, e) + "))"; }); break;
+                case DSC_BIN_UBITXOR: each(i, [&](int e) { return "U2F(F2U(" + E(a, e) + ") ^ F2U(" + E(b, e) + "))"; }); break;
+                default: return false;
+                }
+                break;
+            }
+            case DSC_PE_SELECT:
+                each(i, [&](int e) {
+                    return "(" + E(op.args[0], e) + (op.op == DSC_CMP_EQ ? " == " : " > ") + E(op.args[1], e) + ") ? " + E(op.args[2], e) + " : " + E(op.args[3], e);
+                });
+                break;
+            default: return false;  // coordinates, random numbers and gathers differ per element in more than a value
+            }
+        }
+        out << o.str();
+        return true;
     }
 
     // ---- per-element bodies ---------------------------------------------------------------------------
@@ -1408,6 +1564,23 @@ bool conv_bwd_fits_impl(const FusedKernel::ConvDgrad& c, int64_t k) {
     return L.TOTAL * 4 <= 64 * 1024 && L.MT * L.NT <= 8 && c.chunks >= 8 && c.chunks % 8 == 0;
 }
 
+// Whether the convolution backward kernel of this geometry runs with loader waves.  Without them a workgroup is one
+// chain per image -- request the tiles, wait, store them to LDS, barrier, matrix phases, folds -- and the workgroups
+// that share a CU walk it in step, so fill time and matrix time add up.  With them a workgroup has eight waves and two
+// tile buffers: waves 4-7 only ever fill the buffer of the set's next image (their registers hold the loads in
+// flight; they own no accumulators), waves 0-3 only ever run the matrix phases and the folds of the current one, and
+// one barrier per image hands the buffers over.  Two such workgroups have to fit a CU's 160 KB of LDS.
+bool conv_bwd_loader_waves_impl(const FusedKernel& fk) {
+    const FusedKernel::ConvDgrad& cv = fk.dgrad;
+    if (!cv.on || !cv.wgrad || cv.wgrad_only || fk.as_part) return false;
+    if (const char* e = std::getenv("DSC_CONV_BWD_LOADERS"))
+        if (e[0] == '0') return false;
+    const MatMulDims g = matmul_dims(fk.main.raw());
+    const ConvBwdLayout L = conv_bwd_layout(cv, g.k);
+    const int64_t total = std::max<int64_t>(2 * L.ONE_AT + 4 + (L.mfma_dgrad ? L.GS * 64 : 0), (int64_t)4 * L.MT * L.NT * 256);
+    return total * 4 <= 80 * 1024 && cv.img >= 2 * cv.chunks - cv.chunks / 2;  // most sets hold two images or more
+}
+
 string gen_conv_bwd(Emitter& em, Generated* out) {
     const FusedKernel& fk = em.fk;
     const dsc_kernel_desc& d = fk.main.raw();
@@ -1428,9 +1601,20 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     const bool unpad = cv.pad_h > 0 || cv.pad_w > 0;
     const int MT = L.MT, NT = L.NT;
     if (H < 1 || W < 1 || K % 4 != 0) return "conv backward: unsupported geometry";
+    // Loader waves (see conv_bwd_loader_waves): 512 threads, the upper four waves fill the other of two tile buffers
+    // with the set's next image while the lower four run the matrix phases of the current one.
+    const bool spec = conv_bwd_loader_waves_impl(fk);
+    const int64_t BLOCK = spec ? 512 : 256;
+    const int64_t BUFSZ = L.ONE_AT;  // one buffer: dC slots, the zero row, the input tile
+    const int64_t ONE_AT = spec ? 2 * BUFSZ : L.ONE_AT, ZW_AT = ONE_AT + 1, GB_AT = ONE_AT + 4;
+    const int64_t TOTAL = spec ? std::max<int64_t>(GB_AT + (L.mfma_dgrad ? L.GS * 64 : 0), (int64_t)4 * MT * NT * 256) : L.TOTAL;
 
     const string la = em.load_view(fk.inputs[DC], d.inputs[DC], {"cb", "cm", "ck"});
     em.funcs << "DSC_INLINE float load_a(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return " << la << ";\n}\n";
+    // four consecutive output channels of a pixel from one evaluation of the producers, where they allow it
+    const string la4 = fk.inputs[DC].virt >= 0 && K % 4 == 0 ? em.load_view4(fk.inputs[DC], d.inputs[DC], {"cb", "cm", "ck"}) : string();
+    if (!la4.empty())
+        em.funcs << "DSC_INLINE float4 load_a4(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return " << la4 << ";\n}\n";
     if (!wonly) {
         const string lb = em.load_view(fk.inputs[1], d.inputs[1], {"cb", "ck", "cn"});
         em.funcs << "DSC_INLINE float load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb << ";\n}\n";
@@ -1440,9 +1624,9 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     const string out_ptr = "b" + to_string(fk.outputs[0]), part_ptr = "b" + to_string(fk.outputs[wonly ? 0 : 1]);
     const string img_ptr = "b" + to_string(fk.inputs[2].buffer);
     k << "typedef float cb_float4 __attribute__((ext_vector_type(4)));\n";
-    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
+    k << "extern \"C\" __global__ __launch_bounds__(" << S(BLOCK) << (spec ? ", 4" : "") << ") void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
     k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
-    k << "    __shared__ __attribute__((aligned(16))) float smem[" << S(L.TOTAL) << "];\n";
+    k << "    __shared__ __attribute__((aligned(16))) float smem[" << S(TOTAL) << "];\n";
     k << "    float* const lds = smem;\n    float* const xt = smem + " << S(L.XT_AT) << ";\n";
     // the groups of a set of images sit 8 workgroups apart: same XCD, same L2 (they share the lines of dC, of the
     // image and of the output)
@@ -1451,17 +1635,22 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     else
         k << "    const int band = 0, in_band = blockIdx.x;\n";
     k << "    const int cb = (in_band / 8) % " << S(G) << ", chunk = (in_band / " << S(8 * G) << ") * 8 + in_band % 8;\n";
-    k << "    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 15, lk = lane >> 4;\n";
+    // tid / wave: a thread's place among the 256 that share a role (all of them without loader waves)
+    // (the role comes through readfirstlane: a branch the compiler knows to be uniform is a scalar branch, so no wave
+    // ever walks the other role's barriers with an empty execution mask)
+    if (spec) k << "    const int tid = threadIdx.x & 255;\n    const bool loader = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8)) != 0;\n";
+    else k << "    const int tid = threadIdx.x;\n";
+    k << "    const int lane = tid & 63, wave = tid >> 6, li = lane & 15, lk = lane >> 4;\n";
     // what stays zero for the whole kernel: slots without a pixel, the zero row, the tile words behind the last pixel
-    k << "    for (int i = threadIdx.x; i < " << S(L.ONE_AT) << "; i += 256) smem[i] = 0.f;\n";
-    k << "    if (threadIdx.x == 0) { smem[" << S(L.ONE_AT) << "] = 1.f; smem[" << S(L.ZW_AT) << "] = 0.f; }\n";
+    k << "    for (int i = threadIdx.x; i < " << S(ONE_AT) << "; i += " << S(BLOCK) << ") smem[i] = 0.f;\n";
+    k << "    if (threadIdx.x == 0) { smem[" << S(ONE_AT) << "] = 1.f; smem[" << S(ZW_AT) << "] = 0.f; }\n";
     // fragment addresses of this lane: a constant, plus the step's slot term where the mask says so
     k << "    int a_off[" << MT << "], a_msk[" << MT << "], b_off[" << NT << "], b_msk[" << NT << "];\n";
     k << "#pragma unroll\n    for (int mt = 0; mt < " << MT << "; ++mt) {\n";
     k << "        const int kidx = mt * 16 + li, tap = kidx / " << S(C) << ";\n";
     k << "        const bool real = kidx < " << S(KD) << ";\n";
     k << "        a_off[mt] = real ? " << S(L.XT_AT) << " + ((tap / " << S(FW) << ") * " << S(PW) << " + tap % " << S(FW) << ") * " << S(CP) << " + kidx % " << S(C)
-      << " : (" << (cv.bias ? "kidx == " + S(KD) : string("false")) << " ? " << S(L.ONE_AT) << " : " << S(L.ZW_AT) << ");\n";
+      << " : (" << (cv.bias ? "kidx == " + S(KD) : string("false")) << " ? " << S(ONE_AT) << " : " << S(ZW_AT) << ");\n";
     k << "        a_msk[mt] = real ? -1 : 0;\n    }\n";
     k << "#pragma unroll\n    for (int nt = 0; nt < " << NT << "; ++nt) {\n";
     k << "        const int oc = nt * 16 + li;\n";
@@ -1483,7 +1672,7 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         for (int64_t s = 0; s < GS; ++s) {
             const int64_t oc0 = (4 * s) % K, tt = (4 * s) / K, ty = tt / TQ, tq = tt % TQ - (P - 1);
             k << "        { const int tx = " << S(tq) << " + par; const float w = load_b(cb, " << S(oc0) << " + lk, (" << S(ty * FW) << " + clampi(tx, 0, " << S(FW - 1)
-              << ")) * " << S(C) << " + gc, " << em.params_pass() << "); smem[" << S(L.GB_AT + s * 64) << " + lane] = (tx >= 0 && tx < " << S(FW) << ") ? w : 0.f; }\n";
+              << ")) * " << S(C) << " + gc, " << em.params_pass() << "); smem[" << S(GB_AT + s * 64) << " + lane] = (tx >= 0 && tx < " << S(FW) << ") ? w : 0.f; }\n";
         }
         k << "    }\n";
     }
@@ -1507,79 +1696,145 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     const string vt = vec_fill ? "float4" : "float", dvt = quad_dc ? "float4" : "float";
     auto emit_issue = [&](const string& img, const string& ind) {
         k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NC) << "; ++u) {\n";
-        k << ind << "    const int i = min((int)threadIdx.x + u * 256, " << S(fill_n - 1) << ") * " << S(dunit) << ";\n";
+        k << ind << "    const int i = min(tid + u * 256, " << S(fill_n - 1) << ") * " << S(dunit) << ";\n";
         if (vec_dc)
             k << ind << "    pv[u] = *(const float4*)(b" << fk.inputs[DC].buffer << " + " << S(dc_base) << " + cb * " << S(G == 1 ? 0 : dc_coef[0]) << " + (" << img << " * "
               << S(OHF * OW) << " + band * " << S(OH * OW) << " + i / " << S(K) << ") * " << S(dc_coef[1]) << " + i % " << S(K) << ");\n" << ind << "}\n";
-        else if (quad_dc) {
+        else if (quad_dc && !la4.empty()) {
+            k << ind << "    const int pix = " << img << " * " << S(OHF * OW) << " + band * " << S(OH * OW) << " + i / " << S(K) << ", oc = i % " << S(K) << ";\n";
+            k << ind << "    pv[u] = load_a4(cb, pix, oc, " << em.params_pass() << ");\n" << ind << "}\n";
+        } else if (quad_dc) {
             k << ind << "    const int pix = " << img << " * " << S(OHF * OW) << " + band * " << S(OH * OW) << " + i / " << S(K) << ", oc = i % " << S(K) << ";\n";
             k << ind << "    pv[u] = make_float4(load_a(cb, pix, oc, " << em.params_pass() << "), load_a(cb, pix, oc + 1, " << em.params_pass() << "), load_a(cb, pix, oc + 2, "
               << em.params_pass() << "), load_a(cb, pix, oc + 3, " << em.params_pass() << "));\n" << ind << "}\n";
         } else
             k << ind << "    pv[u] = load_a(cb, " << img << " * " << S(OHF * OW) << " + band * " << S(OH * OW) << " + i / " << S(K) << ", i % " << S(K) << ", " << em.params_pass() << ");\n" << ind << "}\n";
         k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NX) << "; ++u) {\n";
-        k << ind << "    const int e = min((int)threadIdx.x + u * 256, " << S(xn - 1) << ") * " << S(unit) << ";\n";
+        k << ind << "    const int e = min(tid + u * 256, " << S(xn - 1) << ") * " << S(unit) << ";\n";
         k << ind << "    const int ch = e % " << S(C) << ", px = (e / " << S(C) << ") % " << S(PW) << ", py = e / " << S(C * PW) << ";\n";
         k << ind << "    const int sy = clampi(py + band * " << S(OH) << " - " << S(cv.pad_h) << ", 0, " << S(H - 1) << "), sx = clampi(px - " << S(cv.pad_w) << ", 0, " << S(W - 1) << ");\n";
         k << ind << "    xv[u] = *(const " << vt << "*)(" << img_ptr << " + ((" << img << " * " << S(H) << " + sy) * " << S(W) << " + sx) * " << S(GC) << " + cb * " << S(C)
           << " + ch);\n" << ind << "}\n";
         k << ind << "__builtin_amdgcn_sched_barrier(0);\n";
     };
-    auto emit_tile_stores = [&](const string& ind) {
+    auto emit_tile_stores = [&](const string& ind, const string& buf) {
         k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NC) << "; ++u) {\n";
-        k << ind << "    const int i = ((int)threadIdx.x + u * 256) * " << S(dunit) << ", pi = i / " << S(K) << ";\n";
-        k << ind << "    float* const at = lds + ((pi / " << S(OW) << ") * " << S(PW) << " + pi % " << S(OW) << ") * " << S(PITCH) << " + i % " << S(K) << ";\n";
+        k << ind << "    const int i = (tid + u * 256) * " << S(dunit) << ", pi = i / " << S(K) << ";\n";
+        k << ind << "    float* const at = lds + " << buf << " + ((pi / " << S(OW) << ") * " << S(PW) << " + pi % " << S(OW) << ") * " << S(PITCH) << " + i % " << S(K) << ";\n";
         if (quad_dc && PITCH % 4 == 0)
-            k << ind << "    if ((int)threadIdx.x + u * 256 < " << S(fill_n) << ") *(float4*)at = pv[u];\n" << ind << "}\n";
+            k << ind << "    if (tid + u * 256 < " << S(fill_n) << ") *(float4*)at = pv[u];\n" << ind << "}\n";
         else if (quad_dc)
-            k << ind << "    if ((int)threadIdx.x + u * 256 < " << S(fill_n) << ") { at[0] = pv[u].x; at[1] = pv[u].y; at[2] = pv[u].z; at[3] = pv[u].w; }\n" << ind << "}\n";
+            k << ind << "    if (tid + u * 256 < " << S(fill_n) << ") { at[0] = pv[u].x; at[1] = pv[u].y; at[2] = pv[u].z; at[3] = pv[u].w; }\n" << ind << "}\n";
         else
-            k << ind << "    if ((int)threadIdx.x + u * 256 < " << S(fill_n) << ") at[0] = pv[u];\n" << ind << "}\n";
+            k << ind << "    if (tid + u * 256 < " << S(fill_n) << ") at[0] = pv[u];\n" << ind << "}\n";
         k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NX) << "; ++u) {\n";
-        k << ind << "    const int e = ((int)threadIdx.x + u * 256) * " << S(unit) << ";\n";
-        k << ind << "    if ((int)threadIdx.x + u * 256 < " << S(xn) << ") *(" << vt << "*)(xt + (e / " << S(C) << ") * " << S(CP) << " + e % " << S(C) << ") = xv[u];\n"
+        k << ind << "    const int e = (tid + u * 256) * " << S(unit) << ";\n";
+        k << ind << "    if (tid + u * 256 < " << S(xn) << ") *(" << vt << "*)(xt + " << buf << " + (e / " << S(C) << ") * " << S(CP) << " + e % " << S(C) << ") = xv[u];\n"
           << ind << "}\n";
     };
     k << "    __syncthreads();\n";
-    k << "    for (int img = chunk; img < " << S(IMG) << "; img += " << S(cv.chunks) << ") {\n";
-    k << "        {\n            " << dvt << " pv[" << S(NC) << "];\n            " << vt << " xv[" << S(NX) << "];\n";
-    emit_issue("img", "            ");
-    emit_tile_stores("            ");
-    k << "        }\n";
-    k << "        __syncthreads();\n";
+    // Barriers the lower waves pass inside one image's matrix phases: the loader waves pass as many.
+    int phase_syncs = 0;
+    auto sync = [&]() {
+        k << "        __syncthreads();\n";
+        ++phase_syncs;
+    };
+    if (spec) {
+        // the set's first image, then per image: loader waves fill the other buffer while the lower waves work
+        k << "    if (loader && chunk < " << S(IMG) << ") {\n        " << dvt << " pv[" << S(NC) << "];\n        " << vt << " xv[" << S(NX) << "];\n";
+        emit_issue("chunk", "        ");
+        emit_tile_stores("        ", "0");
+        k << "    }\n    __syncthreads();\n";
+        k << "    int bo = 0;\n";
+        k << "    for (int img = chunk; img < " << S(IMG) << "; img += " << S(cv.chunks) << ", bo ^= " << S(BUFSZ) << ") {\n";
+        k << "        if (!loader) {\n";
+    } else {
+        k << "    constexpr int bo = 0;\n";
+        k << "    for (int img = chunk; img < " << S(IMG) << "; img += " << S(cv.chunks) << ") {\n";
+        k << "        {\n            " << dvt << " pv[" << S(NC) << "];\n            " << vt << " xv[" << S(NX) << "];\n";
+        emit_issue("img", "            ");
+        emit_tile_stores("            ", "0");
+        k << "        }\n";
+        k << "        __syncthreads();\n";
+    }
     // 2a. filter gradient: this wave's steps of four slots
+    if (spec) {
+        // Two waves per SIMD run these products (the other two are loader waves), so a wave has to keep the matrix
+        // pipe busy by itself: the fragments of two steps are requested before the first product is issued.
+        k << "#pragma unroll 1\n        for (int s = wave; s < " << S(L.steps) << "; s += 8) {\n";
+        k << "            const bool two = s + 4 < " << S(L.steps) << ";\n";
+        k << "            const int q0 = 4 * s + lk, q1 = 4 * min(s + 4, " << S(L.steps - 1) << ") + lk;\n";
+        k << "            float fa[2][" << MT << "], fb[2][" << NT << "];\n";
+        k << "#pragma unroll\n            for (int h = 0; h < 2; ++h) {\n";
+        k << "                const int qa = (h ? q1 : q0) * " << S(CP) << ", qb = (h ? q1 : q0) * " << S(PITCH) << ";\n";
+        k << "#pragma unroll\n                for (int mt = 0; mt < " << MT << "; ++mt) fa[h][mt] = smem[a_off[mt] + ((qa + bo) & a_msk[mt])];\n";
+        k << "#pragma unroll\n                for (int nt = 0; nt < " << NT << "; ++nt) fb[h][nt] = smem[b_off[nt] + bo + (qb & b_msk[nt])];\n";
+        k << "            }\n";
+        k << "#pragma unroll\n            for (int nt = 0; nt < " << NT << "; ++nt) fb[1][nt] = two ? fb[1][nt] : 0.f;\n";
+        k << "            __builtin_amdgcn_sched_barrier(0);\n";
+        k << "#pragma unroll\n            for (int h = 0; h < 2; ++h)\n#pragma unroll\n                for (int mt = 0; mt < " << MT << "; ++mt)\n#pragma unroll\n                    for (int nt = 0; nt < " << NT << "; ++nt)\n";
+        k << "                        wacc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[h][mt], fb[h][nt], wacc[mt][nt], 0, 0, 0);\n";
+        k << "            __builtin_amdgcn_sched_barrier(0);\n";
+        k << "        }\n";
+    }
+    if (!spec) {
     k << "#pragma unroll 2\n        for (int s = wave; s < " << S(L.steps) << "; s += 4) {\n";
     k << "            const int q = 4 * s + lk, qa = q * " << S(CP) << ", qb = q * " << S(PITCH) << ";\n";
     k << "            float fa[" << MT << "], fb[" << NT << "];\n";
-    k << "#pragma unroll\n            for (int mt = 0; mt < " << MT << "; ++mt) fa[mt] = smem[a_off[mt] + (qa & a_msk[mt])];\n";
-    k << "#pragma unroll\n            for (int nt = 0; nt < " << NT << "; ++nt) fb[nt] = smem[b_off[nt] + (qb & b_msk[nt])];\n";
+    k << "#pragma unroll\n            for (int mt = 0; mt < " << MT << "; ++mt) fa[mt] = smem[a_off[mt] + ((qa + bo) & a_msk[mt])];\n";
+    k << "#pragma unroll\n            for (int nt = 0; nt < " << NT << "; ++nt) fb[nt] = smem[b_off[nt] + bo + (qb & b_msk[nt])];\n";
     k << "#pragma unroll\n            for (int mt = 0; mt < " << MT << "; ++mt)\n#pragma unroll\n                for (int nt = 0; nt < " << NT << "; ++nt)\n";
     k << "                    wacc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[mt], fb[nt], wacc[mt][nt], 0, 0, 0);\n";
     k << "        }\n";
+    }
     const int64_t passes = (PH * PW + 255) / 256;
     if (wonly) {
         k << "        __syncthreads();\n";  // the next image's fills overwrite what the fragments read
     } else if (mfma_dgrad) {
         // 2b. data gradient: every wave takes every fourth tile of 16 pixel groups
         k << "        cb_float4 dacc[" << S(TPW) << "];\n";
+        if (spec) {
+            // the wave's tiles side by side: independent accumulators, one B fragment serves all of them, and the
+            // fragments of a filter row are all requested before its first product
+            const int64_t K4 = K / 4, NF = TQ * K4;
+            k << "#pragma unroll\n        for (int t = 0; t < " << S(TPW) << "; ++t) dacc[t] = (cb_float4){0.f, 0.f, 0.f, 0.f};\n";
+            k << "#pragma unroll 1\n        for (int ty = 0; ty < " << S(FH) << "; ++ty) {\n";
+            k << "            const float* const gbp = smem + " << S(GB_AT) << " + ty * " << S(NF * 64) << " + lane;\n";
+            k << "            float fa[" << S(TPW) << "][" << S(NF) << "], fb[" << S(NF) << "];\n";
+            k << "#pragma unroll\n            for (int i = 0; i < " << S(NF) << "; ++i) fb[i] = gbp[i * 64];\n";
+            k << "#pragma unroll\n            for (int t = 0; t < " << S(TPW) << "; ++t) {\n";
+            k << "                const int grp = (t * 4 + wave) * 16 + li, oy = grp / " << S(GPR) << " - ty, gx0 = (grp % " << S(GPR) << ") * " << S(P) << ";\n";
+            k << "#pragma unroll\n                for (int tqi = 0; tqi < " << S(TQ) << "; ++tqi) {\n";
+            k << "                    const int ox = gx0 - (tqi - " << S(P - 1) << ");\n";
+            k << "                    const int at = bo + ((oy >= 0 && oy < " << S(OH) << " && ox >= 0 && ox < " << S(OW) << ") ? (oy * " << S(PW) << " + ox) * " << S(PITCH) << " : " << S(L.ZERO_AT) << ");\n";
+            k << "#pragma unroll\n                    for (int o4 = 0; o4 < " << S(K4) << "; ++o4) fa[t][tqi * " << S(K4) << " + o4] = lds[at + 4 * o4 + lk];\n";
+            k << "                }\n            }\n";
+            k << "            __builtin_amdgcn_sched_barrier(0);\n";
+            k << "#pragma unroll\n            for (int i = 0; i < " << S(NF) << "; ++i)\n#pragma unroll\n                for (int t = 0; t < " << S(TPW) << "; ++t)\n";
+            k << "                    dacc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[t][i], fb[i], dacc[t], 0, 0, 0);\n";
+            k << "            __builtin_amdgcn_sched_barrier(0);\n";
+            k << "        }\n";
+        }
+        if (!spec) {
         k << "#pragma unroll\n        for (int t = 0; t < " << S(TPW) << "; ++t) {\n";
         k << "            const int grp = (t * 4 + wave) * 16 + li, gy = grp / " << S(GPR) << ", gx0 = (grp % " << S(GPR) << ") * " << S(P) << ";\n";
         k << "            cb_float4 d = (cb_float4){0.f, 0.f, 0.f, 0.f};\n";
         // (the filter rows stay a loop: unrolled whole, the scheduler hoists every LDS load of a tile and the kernel
         // loses a wave of occupancy to the registers that hold them)
         k << "#pragma unroll 1\n            for (int ty = 0; ty < " << S(FH) << "; ++ty) {\n";
-        k << "                const int oy = gy - ty;\n                const float* const gbp = smem + " << S(L.GB_AT) << " + ty * " << S(TQ * (K / 4) * 64) << " + lane;\n";
+        k << "                const int oy = gy - ty;\n                const float* const gbp = smem + " << S(GB_AT) << " + ty * " << S(TQ * (K / 4) * 64) << " + lane;\n";
         for (int64_t tqi = 0; tqi < TQ; ++tqi) {
             const int64_t tq = tqi - (P - 1);
             k << "                {\n                    const int ox = gx0 - " << S(tq) << ";\n";
-            k << "                    const int at = (oy >= 0 && oy < " << S(OH) << " && ox >= 0 && ox < " << S(OW) << ") ? (oy * " << S(PW) << " + ox) * " << S(PITCH) << " : "
-              << S(L.ZERO_AT) << ";\n";
+            k << "                    const int at = bo + ((oy >= 0 && oy < " << S(OH) << " && ox >= 0 && ox < " << S(OW) << ") ? (oy * " << S(PW) << " + ox) * " << S(PITCH) << " : "
+              << S(L.ZERO_AT) << ");\n";
             for (int64_t o4 = 0; o4 < K / 4; ++o4)
                 k << "                    d = __builtin_amdgcn_mfma_f32_16x16x4f32(lds[at + " << S(4 * o4) << " + lk], gbp[" << S((tqi * (K / 4) + o4) * 64) << "], d, 0, 0, 0);\n";
             k << "                }\n";
         }
         k << "            }\n";
         k << "            dacc[t] = d;\n        }\n";
+        }
         // register r of lane l is D[group 4 * (l / 16) + r][(pixel of the group, channel) = l % 16]
         auto emit_dacc_stores = [&](const string& target_of_p) {
             k << "#pragma unroll\n        for (int t = 0; t < " << S(TPW) << "; ++t)\n#pragma unroll\n            for (int r = 0; r < 4; ++r) {\n";
@@ -1590,11 +1845,10 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         };
         if (!unpad) {
             emit_dacc_stores(out_ptr + "[(img * " + S(PH * PW) + " + p) * " + S(GC) + " + cb * " + S(C) + " + gc]");
-            k << "        __syncthreads();\n";
         } else {
-            k << "        __syncthreads();\n";
-            emit_dacc_stores("xt[p * " + S(C) + " + gc]");
-            k << "        __syncthreads();\n";
+            sync();
+            emit_dacc_stores("xt[bo + p * " + S(C) + " + gc]");
+            sync();
         }
     } else {
     // 2b. data gradient: one padded-image pixel per thread and pass, taps x output channels, the filter element
@@ -1602,14 +1856,14 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     const int64_t OCB = K % 8 == 0 ? 8 : 4;
     k << "        float acc[" << passes << "][" << S(C) << "];\n";
     k << "#pragma unroll\n        for (int ps = 0; ps < " << passes << "; ++ps) {\n";
-    k << "            const int p = min(ps * 256 + (int)threadIdx.x, " << S(PH * PW - 1) << ");\n";
+    k << "            const int p = min(ps * 256 + tid, " << S(PH * PW - 1) << ");\n";
     k << "            const int py = p / " << S(PW) << ", px = p % " << S(PW) << ";\n";
     k << "#pragma unroll\n            for (int c = 0; c < " << S(C) << "; ++c) acc[ps][c] = 0.f;\n";
     k << "#pragma unroll 1\n            for (int tap = 0; tap < " << S(FH * FW) << "; ++tap) {\n";
     k << "                const int fy = tap / " << S(FW) << ", fx = tap % " << S(FW) << ";\n";
     k << "                const int oy = py - fy, ox = px - fx;\n";
     k << "                const bool inside = oy >= 0 && oy < " << S(OH) << " && ox >= 0 && ox < " << S(OW) << ";\n";
-    k << "                const float* src = &lds[inside ? (oy * " << S(PW) << " + ox) * " << S(PITCH) << " : " << S(L.ZERO_AT) << "];\n";
+    k << "                const float* src = &lds[bo + (inside ? (oy * " << S(PW) << " + ox) * " << S(PITCH) << " : " << S(L.ZERO_AT) << ")];\n";
     k << "#pragma unroll\n                for (int oc = 0; oc < " << S(K) << "; oc += " << OCB << ") {\n";
     k << "                    float a[" << OCB << "];\n";
     k << "#pragma unroll\n                    for (int q = 0; q < " << OCB << "; q += 4) {\n";
@@ -1622,22 +1876,21 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     k << "                }\n            }\n        }\n";
     if (!unpad) {
         k << "#pragma unroll\n        for (int ps = 0; ps < " << passes << "; ++ps) {\n";
-        k << "            const int p = ps * 256 + (int)threadIdx.x;\n            if (p < " << S(PH * PW) << ") {\n";
+        k << "            const int p = ps * 256 + tid;\n            if (p < " << S(PH * PW) << ") {\n";
         k << "#pragma unroll\n                for (int c = 0; c < " << S(C) << "; ++c) " << out_ptr << "[(img * " << S(PH * PW) << " + p) * " << S(GC)
           << " + cb * " << S(C) << " + c] = acc[ps][c];\n            }\n        }\n";
-        k << "        __syncthreads();\n";
     } else {
         // 3. the padded-image gradient goes through the input tile's memory (dead by now); each pixel of the image sums
         // the padded pixels that replicate it
-        k << "        __syncthreads();\n";
+        sync();
         k << "#pragma unroll\n        for (int ps = 0; ps < " << passes << "; ++ps) {\n";
-        k << "            const int p = ps * 256 + (int)threadIdx.x;\n            if (p < " << S(PH * PW) << ") {\n";
-        k << "#pragma unroll\n                for (int c = 0; c < " << S(C) << "; ++c) xt[p * " << S(C) << " + c] = acc[ps][c];\n            }\n        }\n";
-        k << "        __syncthreads();\n";
+        k << "            const int p = ps * 256 + tid;\n            if (p < " << S(PH * PW) << ") {\n";
+        k << "#pragma unroll\n                for (int c = 0; c < " << S(C) << "; ++c) xt[bo + p * " << S(C) << " + c] = acc[ps][c];\n            }\n        }\n";
+        sync();
     }
     }
     if (unpad && !wonly) {
-        k << "        for (int i = threadIdx.x; i < " << S(H * W * C) << "; i += 256) {\n";
+        k << "        for (int i = tid; i < " << S(H * W * C) << "; i += 256) {\n";
         k << "            const int c = i % " << S(C) << ", x = (i / " << S(C) << ") % " << S(W) << ", y = i / " << S(C * W) << ";\n";
         k << "            float sum = 0.f;\n";
         const string outer = cv.rows_first ? "jx" : "jy", inner = cv.rows_first ? "jy" : "jx";
@@ -1656,7 +1909,7 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
             k << "#pragma unroll\n                " << slots(qi, cv.rows_first) << " {\n";
             k << "                    const bool ok = (edge_y || qy == 0) && (edge_x || qx == 0);\n";
             k << "                    const int ky = base_y + (edge_y ? qy : 0), kx = base_x + (edge_x ? qx : 0);\n";
-            k << "                    const float w = xt[(ky * " << S(PW) << " + kx) * " << S(C) << " + c];\n";
+            k << "                    const float w = xt[bo + (ky * " << S(PW) << " + kx) * " << S(C) << " + c];\n";
             k << "                    part += ok ? w : 0.f;\n                }\n                sum += part;\n            }\n";
         } else {
             k << "#pragma unroll\n            " << range(outer) << " {\n                float part = 0.f;\n";
@@ -1665,19 +1918,32 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
             k << "                    const bool ok_x = jx == 0 || (jx < 0 && x == 0) || (jx > 0 && x == " << S(W - 1) << ");\n";
             k << "                    const int ky = clampi(y + " << S(cv.pad_h) << " + jy, 0, " << S(PH - 1) << "), kx = clampi(x + " << S(cv.pad_w)
               << " + jx, 0, " << S(PW - 1) << ");\n";
-            k << "                    const float w = xt[(ky * " << S(PW) << " + kx) * " << S(C) << " + c];\n";
+            k << "                    const float w = xt[bo + (ky * " << S(PW) << " + kx) * " << S(C) << " + c];\n";
             k << "                    part += (ok_y && ok_x) ? w : 0.f;\n                }\n                sum += part;\n            }\n";
         }
         k << "            " << out_ptr << "[((img * " << S(H) << " + y) * " << S(W) << " + x) * " << S(GC) << " + cb * " << S(C) << " + c] = sum;\n        }\n";
-        k << "        __syncthreads();\n";  // the next image's fills overwrite what the folds read
     }
+    if (spec) {
+        // the loader waves: the next image of the set into the other buffer, then the barriers of the matrix phases
+        k << "        } else {\n";
+        k << "            const int nimg = img + " << S(cv.chunks) << ";\n";
+        k << "            if (nimg < " << S(IMG) << ") {\n                " << dvt << " pv[" << S(NC) << "];\n                " << vt << " xv[" << S(NX) << "];\n";
+        emit_issue("nimg", "                ");
+        emit_tile_stores("                ", "(bo ^ " + S(BUFSZ) + ")");
+        k << "            }\n";
+        for (int i = 0; i < phase_syncs; ++i) k << "            __syncthreads();\n";
+        k << "        }\n";
+    }
+    // the next image's fills overwrite what the matrix phases and the folds read (with loader waves: the buffer the
+    // lower waves turn to next has been filled)
+    if (!wonly) k << "        __syncthreads();\n";
     k << "    }\n";
     // 4. the four waves' accumulators are summed through LDS; register r of lane l is D[4 * (l / 16) + r][l % 16]
     const int64_t R = (int64_t)MT * NT * 256;
     k << "#pragma unroll\n    for (int mt = 0; mt < " << MT << "; ++mt)\n#pragma unroll\n        for (int nt = 0; nt < " << NT
-      << "; ++nt)\n#pragma unroll\n            for (int r = 0; r < 4; ++r) smem[wave * " << S(R) << " + (mt * " << NT << " + nt) * 256 + r * 64 + lane] = wacc[mt][nt][r];\n";
+      << "; ++nt)\n#pragma unroll\n            for (int r = 0; r < 4; ++r) " << (spec ? "if (!loader) " : "") << "smem[wave * " << S(R) << " + (mt * " << NT << " + nt) * 256 + r * 64 + lane] = wacc[mt][nt][r];\n";
     k << "    __syncthreads();\n";
-    k << "    for (int i = threadIdx.x; i < " << S(R) << "; i += 256) {\n";
+    k << "    for (int i = threadIdx.x; i < " << S(R) << "; i += " << S(BLOCK) << ") {\n";
     k << "        const float sum = (smem[i] + smem[" << S(R) << " + i]) + (smem[" << S(2 * R) << " + i] + smem[" << S(3 * R) << " + i]);\n";
     k << "        const int tile = i >> 8, r = (i >> 6) & 3, l = i & 63;\n";
     k << "        const int cm = (tile / " << NT << ") * 16 + 4 * (l >> 4) + r, cn = (tile % " << NT << ") * 16 + (l & 15);\n";
@@ -1687,9 +1953,9 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     k << "    }\n}\n";
     if (cv.chunks * G * BANDS >= kMaxIndex) return "conv backward: grid too large";
     out->grid = (unsigned)(cv.chunks * G * BANDS);
-    out->block = 256;
+    out->block = (unsigned)BLOCK;
     out->source = k.str();
-    out->note = "conv backward: workgroup per group and image set (" + S(cv.chunks) + " sets), dC and input tile in LDS, " +
+    out->note = "conv backward: workgroup per group and image set (" + S(cv.chunks) + " sets), dC and input tile in LDS, " + (spec ? "loader waves fill the next image's tiles, " : "") +
                 (wonly ? "no data gradient, " + S(BANDS) + " bands of " + S(OH) + " output rows" : "data gradient " + S(FH) + "x" + S(FW) + " taps x " + S(K) + " channels" + (unpad ? " with border folds" : "")) +
                 ", filter gradient mfma 16x16x4 " + to_string(MT) + "x" + to_string(NT) + " tiles" + (cv.bias ? " +column sums of dC" : "");
     return "";
@@ -3126,6 +3392,8 @@ std::string FusedKernel::key() const {
     for (const char* name : {"DSC_MM_SMALLK", "DSC_MM_VEC_STORE", "DSC_MM_PERSISTENT", "DSC_MM_DEEP_K", "DSC_MM_DIRECT_LDS", "DSC_MM_ROWS", "DSC_MM_DOT", "DSC_ROWS_MFMA", "DSC_MM_TALLK"})
         if (const char* env = std::getenv(name))
             if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|") + name + env;
+    if (dgrad.on && dgrad.wgrad && !dgrad.wgrad_only)
+        if (const char* env = std::getenv("DSC_CONV_BWD_LOADERS")) s += string("|LW") + env;
     return s;
 }
 
@@ -3151,9 +3419,11 @@ bool conv_dgrad_fits(const FusedKernel::ConvDgrad& c, int64_t k) {
 }
 
 bool conv_bwd_fits(const FusedKernel::ConvDgrad& c, int64_t k) { return conv_bwd_fits_impl(c, k); }
+bool conv_bwd_loader_waves(const FusedKernel& fk) { return conv_bwd_loader_waves_impl(fk); }
 
 bool can_be_part(const FusedKernel& fk) {
     if (!fk.parts.empty() || fk.binned_stage || fk.chain_group) return false;
+    if (fk.dgrad.on && conv_bwd_loader_waves_impl(fk)) return false;  // 512 threads per workgroup
     if (fk.dgrad.on || fk.cfwd.on || !fk.row_stages.empty()) return true;
     if (fk.main.raw().kind != DSC_KERNEL_MATMUL) return true;
     // of the MatMul kernels, the row-per-thread, short-k and tall-k ones run 256 threads addressed by blockIdx.x

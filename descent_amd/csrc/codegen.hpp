@@ -194,6 +194,9 @@ std::string generate(const FusedKernel& k, Generated* out);
 bool conv_dgrad_fits(const FusedKernel::ConvDgrad& c, int64_t k);
 // The same for the kernel that also takes the filter gradient (c.wgrad, c.bias and c.chunks set).
 bool conv_bwd_fits(const FusedKernel::ConvDgrad& c, int64_t k);
+// Whether that kernel runs with loader waves (512 threads: four waves fill the next image's tiles while four run the
+// matrix phases of the current one); the planner deals the images into fewer, larger sets then.
+bool conv_bwd_loader_waves(const FusedKernel& fk);
 // Whether the convolution-forward kernel takes this geometry with n output channels per group.
 bool conv_fwd_fits(const FusedKernel::ConvFwd& c, int64_t n);
 

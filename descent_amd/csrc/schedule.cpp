@@ -1468,12 +1468,19 @@ struct Planner {
             }
             // image sets: about a thousand workgroups, a multiple of eight sets
             // (measured on the ConvNet's second convolution, 2000 image-groups: ~1000 workgroups 38.8 us, ~2000 43.9, ~500 43.1)
-            const int64_t per_group = std::max<int64_t>(8, 1024 / f.g);
-            const int64_t images_per_set = (f.img + per_group - 1) / per_group;
-            const int64_t sets = ((f.img + images_per_set - 1) / images_per_set + 7) / 8 * 8;
             Draft fused = drafts[di];
             fused.fk.dgrad.wgrad = true;
             fused.fk.dgrad.bias = bias;
+            auto sets_for = [&](int64_t workgroups) {
+                const int64_t per_group = std::max<int64_t>(8, workgroups / f.g);
+                const int64_t images_per_set = (f.img + per_group - 1) / per_group;
+                return ((f.img + images_per_set - 1) / images_per_set + 7) / 8 * 8;
+            };
+            // with loader waves two workgroups of eight waves share a CU: one round of 512 workgroups, whose sets are
+            // long enough for the fills to run beside the matrix phases
+            int64_t sets = sets_for(512);
+            fused.fk.dgrad.chunks = sets;
+            if (!conv_bwd_loader_waves(fused.fk)) sets = sets_for(1024);
             fused.fk.dgrad.chunks = sets;
             {
                 Source xs;
@@ -1913,6 +1920,9 @@ struct Planner {
         // tuning hook: DSC_FUSE_INTO_MATMUL=0 keeps producers of MatMul operands materialised
         const char* fim = std::getenv("DSC_FUSE_INTO_MATMUL");
         const bool fuse_into_matmul = !(fim && fim[0] == '0');
+        // DSC_CONV_BWD_LOADERS=2: loader waves, but dC of the convolution backward kernel stays a buffer
+        const char* lw = std::getenv("DSC_CONV_BWD_LOADERS");
+        const bool no_dc_producer = lw && lw[0] == '2';
         bool changed = true;
         while (changed) {
             changed = false;
@@ -1970,7 +1980,11 @@ struct Planner {
                     // works on the current one: plain loads, nothing evaluated in between
                     // (the filter gradient alone has one round trip per image anyway and takes dC as a producer; its
                     // image has to be a buffer)
-                    if (q.fk.dgrad.on && q.fk.dgrad.wgrad && q.fk.inputs[0].buffer >= 0 && q.params[q.fk.inputs[0].buffer] == node) ok = false;
+                    // (with loader waves the fills run beside the matrix phases, on waves of their own: there dC is a
+                    // producer again, and the pooling gradient it usually is never goes through memory)
+                    if (q.fk.dgrad.on && q.fk.dgrad.wgrad && q.fk.inputs[0].buffer >= 0 && q.params[q.fk.inputs[0].buffer] == node &&
+                        !(conv_bwd_loader_waves(q.fk) && !no_dc_producer))
+                        ok = false;
                     // an epilogue reads its product from the accumulator, never through a producer
                     if (q.fk.has_epilogue && q.fk.epilogue_product_input >= 0) {
                         const Source& ps = q.fk.epilogue_inputs[q.fk.epilogue_product_input];

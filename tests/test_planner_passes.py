@@ -226,7 +226,7 @@ def test_the_sign_of_a_pre_activation_is_read_off_the_stored_activation():
     # and dropped-out a (2 x 6.3) for 12.5 MB in
     assert "ConvForward" in lines[0] and 65.0 < moved(lines[0]) < 66.5, lines[0]     # 116.0 with z stored
     assert lines[1].split(": ")[1].startswith("ConvForward") and 49.5 < moved(lines[1]) < 51.0, lines[1]  # 75.3 with z stored
-    assert "414." in fused.splitlines()[-1], fused.splitlines()[-1]                  # MB per step; 565 with z stored
+    assert "409." in fused.splitlines()[-1], fused.splitlines()[-1]                  # MB per step; 565 with z stored
     # cluster by cluster nothing is rewritten
     unfused = hip_backend.check_schedule(graph, fused=False)
     assert "PerElement (7 ops) [12544000]" in unfused and "2316." in unfused.splitlines()[-1], unfused.splitlines()[-1]
