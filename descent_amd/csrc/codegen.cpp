@@ -1640,7 +1640,7 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     // ever walks the other role's barriers with an empty execution mask)
     if (spec) k << "    const int tid = threadIdx.x & 255;\n    const bool loader = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8)) != 0;\n";
     else k << "    const int tid = threadIdx.x;\n";
-    k << "    const int lane = tid & 63, wave = tid >> 6, li = lane & 15, lk = lane >> 4;\n";
+    k << "    const int lane = tid & 63, wave = " << (spec ? "__builtin_amdgcn_readfirstlane(tid >> 6)" : "tid >> 6") << ", li = lane & 15, lk = lane >> 4;\n";
     // what stays zero for the whole kernel: slots without a pixel, the zero row, the tile words behind the last pixel
     k << "    for (int i = threadIdx.x; i < " << S(ONE_AT) << "; i += " << S(BLOCK) << ") smem[i] = 0.f;\n";
     k << "    if (threadIdx.x == 0) { smem[" << S(ONE_AT) << "] = 1.f; smem[" << S(ZW_AT) << "] = 0.f; }\n";
@@ -1739,15 +1739,12 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         k << "        __syncthreads();\n";
         ++phase_syncs;
     };
+    const string loop_head = "    int bo = 0;\n    for (int img = chunk; img < " + S(IMG) + "; img += " + S(cv.chunks) + ", bo ^= " + S(BUFSZ) + ") {\n";
     if (spec) {
-        // the set's first image, then per image: loader waves fill the other buffer while the lower waves work
-        k << "    if (loader && chunk < " << S(IMG) << ") {\n        " << dvt << " pv[" << S(NC) << "];\n        " << vt << " xv[" << S(NX) << "];\n";
-        emit_issue("chunk", "        ");
-        emit_tile_stores("        ", "0");
-        k << "    }\n    __syncthreads();\n";
-        k << "    int bo = 0;\n";
-        k << "    for (int img = chunk; img < " << S(IMG) << "; img += " << S(cv.chunks) << ", bo ^= " << S(BUFSZ) << ") {\n";
-        k << "        if (!loader) {\n";
+        // The two roles are two loops, so that neither carries the other's registers (the accumulators and fragment
+        // addresses of the matrix phases, the addresses the fills keep): the loader waves then have room to request
+        // all of an image's loads in one go.  Both pass the same barriers.
+        k << "    if (!loader) {\n    __syncthreads();\n" << loop_head;
     } else {
         k << "    constexpr int bo = 0;\n";
         k << "    for (int img = chunk; img < " << S(IMG) << "; img += " << S(cv.chunks) << ") {\n";
@@ -1923,21 +1920,26 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         }
         k << "            " << out_ptr << "[((img * " << S(H) << " + y) * " << S(W) << " + x) * " << S(GC) << " + cb * " << S(C) << " + c] = sum;\n        }\n";
     }
-    if (spec) {
-        // the loader waves: the next image of the set into the other buffer, then the barriers of the matrix phases
-        k << "        } else {\n";
-        k << "            const int nimg = img + " << S(cv.chunks) << ";\n";
-        k << "            if (nimg < " << S(IMG) << ") {\n                " << dvt << " pv[" << S(NC) << "];\n                " << vt << " xv[" << S(NX) << "];\n";
-        emit_issue("nimg", "                ");
-        emit_tile_stores("                ", "(bo ^ " + S(BUFSZ) + ")");
-        k << "            }\n";
-        for (int i = 0; i < phase_syncs; ++i) k << "            __syncthreads();\n";
-        k << "        }\n";
-    }
     // the next image's fills overwrite what the matrix phases and the folds read (with loader waves: the buffer the
     // lower waves turn to next has been filled)
     if (!wonly) k << "        __syncthreads();\n";
     k << "    }\n";
+    if (spec) {
+        // the loader waves: the set's first image, then per image the next one into the other buffer and the
+        // barriers of the matrix phases
+        k << "    } else {\n";
+        k << "    if (chunk < " << S(IMG) << ") {\n        " << dvt << " pv[" << S(NC) << "];\n        " << vt << " xv[" << S(NX) << "];\n";
+        emit_issue("chunk", "        ");
+        emit_tile_stores("        ", "0");
+        k << "    }\n    __syncthreads();\n" << loop_head;
+        k << "        const int nimg = img + " << S(cv.chunks) << ";\n";
+        k << "        if (nimg < " << S(IMG) << ") {\n            " << dvt << " pv[" << S(NC) << "];\n            " << vt << " xv[" << S(NX) << "];\n";
+        emit_issue("nimg", "            ");
+        emit_tile_stores("            ", "(bo ^ " + S(BUFSZ) + ")");
+        k << "        }\n";
+        for (int i = 0; i < phase_syncs + 1; ++i) k << "        __syncthreads();\n";
+        k << "    }\n    }\n";
+    }
     // 4. the four waves' accumulators are summed through LDS; register r of lane l is D[4 * (l / 16) + r][l % 16]
     const int64_t R = (int64_t)MT * NT * 256;
     k << "#pragma unroll\n    for (int mt = 0; mt < " << MT << "; ++mt)\n#pragma unroll\n        for (int nt = 0; nt < " << NT

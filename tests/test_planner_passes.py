@@ -91,7 +91,11 @@ def test_bias_gradient_rides_on_the_weight_gradient_that_reads_the_same_array():
 def test_first_layer_filter_gradient_takes_the_pooling_gradient_as_a_producer():
     graph = workloads.convnet(_env(), batch=1000).graph
     listing = hip_backend.check_schedule(graph, fused=True)
-    assert int(listing.split()[0]) == 11
+    assert int(listing.split()[0]) == 10
+    # conv2's backward kernel runs with loader waves and takes its dC the same way: the pooling gradient behind it is
+    # a producer of that kernel's fills and no launch of its own
+    line = next(l for l in listing.splitlines() if ": ConvBackward" in l)
+    assert "fused producers>" in line and "loader waves fill the next image's tiles" in line and "grid 512x512" in line, line
     # conv1 needs no data gradient: its filter gradient (and the bias gradient's column sums) run on the convolution
     # backward kernel, bands of 7 output rows; dC is never written -- the max-pool gradient (a WindowsToImage over
     # 2x2 windows that do not overlap, turned into a copy), the selects around it and the activation derivative are
@@ -226,7 +230,7 @@ def test_the_sign_of_a_pre_activation_is_read_off_the_stored_activation():
     # and dropped-out a (2 x 6.3) for 12.5 MB in
     assert "ConvForward" in lines[0] and 65.0 < moved(lines[0]) < 66.5, lines[0]     # 116.0 with z stored
     assert lines[1].split(": ")[1].startswith("ConvForward") and 49.5 < moved(lines[1]) < 51.0, lines[1]  # 75.3 with z stored
-    assert "409." in fused.splitlines()[-1], fused.splitlines()[-1]                  # MB per step; 565 with z stored
+    assert "359." in fused.splitlines()[-1], fused.splitlines()[-1]                  # MB per step; 565 with z stored, 414 before conv2's dC became a producer
     # cluster by cluster nothing is rewritten
     unfused = hip_backend.check_schedule(graph, fused=False)
     assert "PerElement (7 ops) [12544000]" in unfused and "2316." in unfused.splitlines()[-1], unfused.splitlines()[-1]
