@@ -357,7 +357,7 @@ struct Emitter {
         if (it != instances.end()) return it->second;
         const Virtual& vi = fk.virtuals[virt];
         const dsc_kernel_desc& pd = vi.pe.raw();
-        if (pd.kind != DSC_KERNEL_PER_ELEMENT) return instances[sig] = "";
+        if (pd.kind != DSC_KERNEL_PER_ELEMENT && pd.kind != DSC_KERNEL_REDUCE) return instances[sig] = "";
         const string name = "virt" + to_string(virt) + "_" + to_string(instances.size()) + "_x4";
         instances[sig] = name;  // (a producer never reads itself: the graph of virtuals is acyclic)
         IndexForm local = form;
@@ -369,6 +369,27 @@ struct Emitter {
         }
         std::ostringstream body;
         body << "    const int gid = " << gid << ";\n";
+        if (pd.kind == DSC_KERNEL_REDUCE) {
+            // four neighbouring results of a reduction along another axis than the innermost: one loop, quads added up
+            const dsc_view& v = pd.inputs[0];
+            const int L = pd.shape.rank - 1;
+            if (L < 1 || pd.axis == L || pd.shape.dims[L] % 4 != 0) return instances[sig] = "";
+            std::vector<string> oc = emit_coords_separable(body, pd.shape, local, "vo");
+            if (oc.empty()) oc = emit_coords(body, pd.shape, "gid", "vo");
+            auto ic = oc;
+            ic[pd.axis] = "kk";
+            const string x = load_view4(vi.inputs[0], v, ic);
+            if (x.empty()) return instances[sig] = "";
+            const bool is_max = pd.reduce_op == DSC_REDUCE_MAX;
+            const string init = is_max ? "U2F(0xff800000u)" : "0.f";
+            body << "    float4 acc = make_float4(" << init << ", " << init << ", " << init << ", " << init << ");\n";
+            body << "    for (int kk = 0; kk < " << S(v.out_shape.dims[pd.axis]) << "; ++kk) {\n        const float4 x = " << x << ";\n";
+            if (is_max) body << "        acc = make_float4(glsl_max(acc.x, x.x), glsl_max(acc.y, x.y), glsl_max(acc.z, x.z), glsl_max(acc.w, x.w));\n    }\n";
+            else body << "        acc = make_float4(acc.x + x.x, acc.y + x.y, acc.z + x.z, acc.w + x.w);\n    }\n";
+            body << "    return acc;\n";
+            funcs << "DSC_INLINE float4 " << name << "(" << decl << params_decl() << ") {\n" << body.str() << "}\n\n";
+            return name;
+        }
         if (!emit_pe4(body, pd, vi.inputs, "gid", "v", &local)) return instances[sig] = "";
         body << "    return make_float4(vt" << vi.out_op << "[0], vt" << vi.out_op << "[1], vt" << vi.out_op << "[2], vt" << vi.out_op << "[3]);\n";
         funcs << "DSC_INLINE float4 " << name << "(" << decl << params_decl() << ") {\n" << body.str() << "}\n\n";
@@ -1231,9 +1252,12 @@ string gen_row_fused(Emitter& em, Generated* out) {
         G = std::max(G, L);
         J = (kblocks + G - 1) / G;
     }
-    const int64_t per_block = 256 / G;
+    // (one wave per workgroup, to spread 1000 rows over four times as many compute units, measured slower: 13.9 us
+    // against 10.1 for the ConvNet's head -- every workgroup stages B for itself)
+    const int64_t BT = 256;
+    const int64_t per_block = BT / G;
     std::ostringstream k;
-    k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
+    k << "extern \"C\" __global__ __launch_bounds__(" << S(BT) << ") void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
     k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
     k << "    const int col = threadIdx.x % " << G << ";\n";
     k << "    const int row = blockIdx.x * " << per_block << " + threadIdx.x / " << G << ";\n";
@@ -1272,14 +1296,35 @@ string gen_row_fused(Emitter& em, Generated* out) {
             const string lb = em.load_view(st.inputs[1], sd.inputs[1], {"cb", "ck", "cn"});
             em.funcs << "DSC_INLINE float rows_load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb << ";\n}\n";
             k << "    __shared__ float sB[" << S(kblocks * 4 * n) << "];\n";
-            k << "    for (int e = threadIdx.x; e < " << S(kblocks * 4 * n) << "; e += 256) {\n";
+            k << "    for (int e = threadIdx.x; e < " << S(kblocks * 4 * n) << "; e += " << S(BT) << ") {\n";
             k << "        const int kk = e / " << S(n) << ", nn = e % " << S(n) << ";\n";
             k << "        const float v = rows_load_b(0, min(kk, " << S(K - 1) << "), nn, " << em.params_pass() << ");\n";
             k << "        sB[e] = kk < " << S(K) << " ? v : 0.f;\n    }\n";
             // every block of the lane requested before anything is used; beyond k the clamped loads meet zeros of B
             k << "    float mm_a[" << S(J) << "][4];\n";
+            // a lane's block is four consecutive k: one evaluation of A's producers where they can be taken in quads
+            const string la4 = st.inputs[0].virt >= 0 && K % 4 == 0 ? em.load_view4(st.inputs[0], sd.inputs[0], {"cb", "cm", "ck"}) : string();
+            if (!la4.empty()) {
+                em.funcs << "DSC_INLINE float4 rows_load_a4(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return " << la4 << ";\n}\n";
+                k << "#pragma unroll\n    for (int j = 0; j < " << S(J) << "; ++j) {\n";
+                k << "        const float4 q = rows_load_a4(0, rowc, min(4 * (col + j * " << S(G) << "), " << S(K - 4) << "), " << em.params_pass() << ");\n";
+                k << "        mm_a[j][0] = q.x; mm_a[j][1] = q.y; mm_a[j][2] = q.z; mm_a[j][3] = q.w;\n    }\n";
+            } else {
             k << "#pragma unroll\n    for (int j = 0; j < " << S(J) << "; ++j)\n#pragma unroll\n        for (int i = 0; i < 4; ++i)\n";
             k << "            mm_a[j][i] = rows_load_a(0, rowc, min(4 * (col + j * " << S(G) << ") + i, " << S(K - 1) << "), " << em.params_pass() << ");\n";
+            }
+            if (st.store_a >= 0) {
+                // A is evaluated here and nowhere else: the launches that read it later find it in memory
+                int64_t ab = 0, ac[DSC_MAX_DIM];
+                if (sd.inputs[0].out_shape.rank != 3 || !affine_form(sd.inputs[0], &ab, ac) || ab != 0 || ac[1] != K || ac[2] != 1)
+                    return "row-fused: an A operand that is stored must be a plain [m, k] array";
+                const string ap = "b" + to_string(fk.outputs[st.store_a]);
+                k << "#pragma unroll\n    for (int j = 0; j < " << S(J) << "; ++j) {\n        const int kb = 4 * (col + j * " << S(G) << ");\n";
+                if (K % 4 == 0)
+                    k << "        if (row_ok && kb < " << S(K) << ") *(float4*)(" << ap << " + row * " << S(K) << " + kb) = make_float4(mm_a[j][0], mm_a[j][1], mm_a[j][2], mm_a[j][3]);\n    }\n";
+                else
+                    k << "#pragma unroll\n        for (int i = 0; i < 4; ++i)\n            if (row_ok && kb + i < " << S(K) << ") " << ap << "[row * " << S(K) << " + kb + i] = mm_a[j][i];\n    }\n";
+            }
             k << "    __syncthreads();\n";
             k << "    float mm_acc[" << S(n) << "];\n#pragma unroll\n    for (int nn = 0; nn < " << S(n) << "; ++nn) mm_acc[nn] = 0.f;\n";
             k << "#pragma unroll\n    for (int j = 0; j < " << S(J) << "; ++j) {\n";
@@ -1320,7 +1365,7 @@ string gen_row_fused(Emitter& em, Generated* out) {
     }
     k << "}\n";
     out->grid = blocks_for(m, (int)per_block);
-    out->block = 256;
+    out->block = (unsigned)BT;
     out->source = k.str();
     out->note = "row-fused: " + S(G) + " lanes per row, " + to_string(fk.row_stages.size()) + " stages" + (mm0 ? ", the first a MatMul over k=" + S(K) + " shared by the row's lanes" : "");
     return "";
@@ -3261,9 +3306,11 @@ void count_work(const FusedKernel& fk, Generated* g) {
         elements += (double)(fk.pair.chunks * m.n * m.k) - out_each;
         g->algo_flops *= 2.0;
     }
-    for (auto& st : fk.row_stages)
+    for (auto& st : fk.row_stages) {
         for (int o : st.outputs)
             if (o >= 0) elements += (double)element_count(st.k.raw().shape);
+        if (st.store_a >= 0) elements += (double)element_count(st.k.raw().inputs[0].out_shape);
+    }
     g->algo_bytes = 4.0 * elements;
 }
 
@@ -3345,6 +3392,7 @@ std::string FusedKernel::key() const {
             s.append(reinterpret_cast<const char*>(&x.stage_out), 4);
         }
         for (int o : st.outputs) s.append(reinterpret_cast<const char*>(&o), 4);
+        s.append(reinterpret_cast<const char*>(&st.store_a), 4);
     }
     if (!row_stages.empty()) {
         s.append(reinterpret_cast<const char*>(&row_m), 8);

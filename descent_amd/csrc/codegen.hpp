@@ -37,6 +37,10 @@ struct RowStage {
                                  // only) the MatMul whose [m, n] product the other stages start from
     std::vector<Source> inputs;  // one per input view of k
     std::vector<int> outputs;    // per output of k: index into FusedKernel::outputs when stored, else -1
+    // (stage 0 MatMul only) index into FusedKernel::outputs of the buffer that takes the A operand [m, k] as the stage
+    // evaluates it -- each element exactly once, by the lane that multiplies it -- when A is a fused producer whose
+    // result other launches read as well; -1 otherwise
+    int store_a = -1;
 };
 
 struct FusedKernel {

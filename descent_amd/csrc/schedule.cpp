@@ -1810,6 +1810,67 @@ struct Planner {
         drafts[ri] = fused;
     }
 
+    // The A operand [m, k] of the product a row-fused launch starts from is often a light per-element cluster's only
+    // output -- the hidden layer's activation: bias and leaky_relu over the sum of the previous product's k chunks --
+    // that later launches read as well (the backward pass).  The row-fused launch evaluates every element of A exactly
+    // once, so it can run that cluster itself and store the result on the way: one launch less.
+    // DSC_FUSE_ROWS_OPERAND=0 keeps the cluster a launch of its own.
+    void rows_take_their_operands_producer(int ri) {
+        if (const char* e = std::getenv("DSC_FUSE_ROWS_OPERAND"))
+            if (e[0] == '0') return;
+        Draft& r = drafts[ri];
+        if (r.fk.row_stages.empty() || r.fk.row_stages[0].k.raw().kind != DSC_KERNEL_MATMUL) return;
+        RowStage& mm = r.fk.row_stages[0];
+        if (mm.inputs[0].buffer < 0 || mm.store_a >= 0) return;
+        const int node = r.params[mm.inputs[0].buffer];
+        const dsc_kernel_desc& md = mm.k.raw();
+        const MatMulDims g = matmul_dims(md);
+        int64_t base = 0, coef[DSC_MAX_DIM];
+        if (md.inputs[0].out_shape.rank != 3 || !affine_form(md.inputs[0], &base, coef) || base != 0 || coef[1] != g.k || coef[2] != 1 ||
+            element_count(md.inputs[0].in_shape) != g.m * g.k)
+            return;
+        int qi = -1;
+        for (int j = 0; j < ri; ++j)
+            if (drafts[j].alive)
+                for (auto& o : drafts[j].outs)
+                    if (o.node == node) qi = j;
+        if (qi < 0) return;
+        const Draft& q = drafts[qi];
+        const dsc_kernel_desc& qd = q.fk.main.raw();
+        if (qd.kind != DSC_KERNEL_PER_ELEMENT || qd.n_outputs != 1 || q.fk.has_epilogue || !q.fk.row_stages.empty() || !q.fk.parts.empty() || q.keep_output ||
+            q.fk.row_width || q.outs.size() != 1 || q.outs[0].copy_from >= 0 || qd.shape.dims[0] != g.m * g.k || !is_cheap_producer(qd) ||
+            q.fk.virtuals.size() + r.fk.virtuals.size() + 1 > 8)
+            return;
+        for (int c : consumers_of(node))
+            if (c < ri) return;  // someone ahead of the row-fused launch needs the array in memory
+        if (taken_in_place_between(qi, ri, input_nodes(q))) return;
+        Draft fused = r;
+        {
+            const int new_virt = (int)fused.fk.virtuals.size();
+            fused.fk.virtuals.emplace_back();
+            const int voff = import_virtuals(fused, q);
+            Virtual nv;
+            nv.pe = q.fk.main;
+            nv.out_op = qd.outputs[0];
+            for (auto& s : q.fk.inputs) nv.inputs.push_back(import_source(fused, q, s, voff));
+            fused.fk.virtuals[new_virt] = nv;
+            RowStage& fm = fused.fk.row_stages[0];
+            fm.inputs[0] = Source{};
+            fm.inputs[0].virt = new_virt;
+            fm.store_a = (int)fused.fk.outputs.size();
+            fused.fk.outputs.push_back(param_index(fused, node, true));
+            fused.outs.push_back(q.outs[0]);
+        }
+        compact(fused);
+        {
+            Generated probe;
+            if (!generate(fused.fk, &probe).empty()) return;
+        }
+        fused.covers.insert(fused.covers.end(), q.covers.begin(), q.covers.end());
+        drafts[qi].alive = false;
+        drafts[ri] = fused;
+    }
+
     // Pass 1i: per-element clusters over [rows, w] that pick their value by comparing the column with literals (each
     // concat of the reference is one: select(column > n - 1, pad(b), pad(a))) are marked to run a thread per row,
     // the column a constant of each of the row's w evaluations.  A chain of concats inlined into the last one then
@@ -2660,6 +2721,8 @@ struct Planner {
         column_partitions();                    // pass 1i
         recompute_from_small_inputs();          // pass 1h
         inline_producers();                     // pass 2
+        for (int i = 0; i < (int)drafts.size(); ++i)
+            if (drafts[i].alive) rows_take_their_operands_producer(i);  // pass 2b
         attach_epilogues();                     // pass 3
         slice_major_products();                 // pass 3d
         pool_joins_conv_forward();              // pass 3c
