@@ -1300,6 +1300,13 @@ string gen_row_fused(Emitter& em, Generated* out) {
             k << "        const int kk = e / " << S(n) << ", nn = e % " << S(n) << ";\n";
             k << "        const float v = rows_load_b(0, min(kk, " << S(K - 1) << "), nn, " << em.params_pass() << ");\n";
             k << "        sB[e] = kk < " << S(K) << " ? v : 0.f;\n    }\n";
+            if (fk.row_tail.on) {
+                const FusedKernel::RowTail& rt = fk.row_tail;
+                const string lb2 = em.load_view(rt.b, rt.mm.raw().inputs[1], {"cb", "ck", "cn"});
+                em.funcs << "DSC_INLINE float tail_load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb2 << ";\n}\n";
+                k << "    __shared__ __attribute__((aligned(16))) float sB2[" << S(n * K) << "];\n";
+                k << "    for (int e = threadIdx.x; e < " << S(n * K) << "; e += " << S(BT) << ") sB2[e] = tail_load_b(0, e / " << S(K) << ", e % " << S(K) << ", " << em.params_pass() << ");\n";
+            }
             // every block of the lane requested before anything is used; beyond k the clamped loads meet zeros of B
             k << "    float mm_a[" << S(J) << "][4];\n";
             // a lane's block is four consecutive k: one evaluation of A's producers where they can be taken in quads
@@ -1363,11 +1370,49 @@ string gen_row_fused(Emitter& em, Generated* out) {
             return "row-fused: stage must be a per-element or reduce kernel";
         }
     }
+    if (fk.row_tail.on) {
+        const FusedKernel::RowTail& rt = fk.row_tail;
+        const dsc_kernel_desc& td = rt.mm.raw();
+        const MatMulDims tg = matmul_dims(td);
+        if (!mm0 || tg.batch != 1 || tg.chunks != 1 || tg.m != m || tg.k != n || tg.n != K || K % 4 != 0 || rt.b.buffer < 0 || rt.x_stage < 0 ||
+            rt.x_stage >= (int)fk.row_stages.size() || !stage_is_wide(rt.x_stage))
+            return "row-fused: the trailing product does not match the rows";
+        if (rt.epilogue_a_input >= 0 && fk.row_stages[0].store_a < 0) return "row-fused: the trailing product's consumer reads an operand that is not stored";
+        k << "    // trailing product: [m, " << n << "] x [" << n << ", " << K << "], a lane's blocks of four columns as in stage 0\n";
+        const string x = stage_var(rt.x_stage, rt.x_stage_out);
+        k << "    const int tl_base = (threadIdx.x & 63) / " << S(G) << " * " << S(G) << ";\n";
+        k << "    float tl_x[" << S(n) << "];\n#pragma unroll\n    for (int c = 0; c < " << S(n) << "; ++c) tl_x[c] = __shfl(" << x << ", tl_base + c, 64);\n";
+        std::ostringstream body;
+        int n_res = 1;
+        if (rt.has_epilogue) {
+            const dsc_kernel_desc& pe = rt.epilogue.raw();
+            n_res = pe.n_outputs;
+            std::map<int, string> ov;
+            ov[rt.epilogue_product_input] = "product";
+            if (rt.epilogue_a_input >= 0) ov[rt.epilogue_a_input] = "operand";
+            em.emit_pe(body, pe, rt.epilogue_inputs, "gid", "e", ov);
+            for (int o = 0; o < pe.n_outputs; ++o) body << "    result[" << o << "] = et" << pe.outputs[o] << ";\n";
+            em.funcs << "DSC_INLINE void tail_epilogue(float product, float operand, int gid, float* result, " << em.params_decl() << ") {\n" << body.str() << "}\n";
+        }
+        if ((int)rt.outputs.size() != n_res) return "row-fused: trailing product output count";
+        k << "#pragma unroll\n    for (int j = 0; j < " << S(J) << "; ++j) {\n        const int blk = col + j * " << S(G) << ";\n";
+        k << "        if (blk < " << S(kblocks) << ") {\n            float acc[4] = {0.f, 0.f, 0.f, 0.f};\n";
+        k << "#pragma unroll\n            for (int c = 0; c < " << S(n) << "; ++c) {\n                const float4 b4 = *(const float4*)&sB2[c * " << S(K) << " + 4 * blk];\n";
+        k << "                acc[0] = fmaf(tl_x[c], b4.x, acc[0]); acc[1] = fmaf(tl_x[c], b4.y, acc[1]); acc[2] = fmaf(tl_x[c], b4.z, acc[2]); acc[3] = fmaf(tl_x[c], b4.w, acc[3]);\n            }\n";
+        if (rt.has_epilogue) {
+            k << "            float res[4][" << n_res << "];\n#pragma unroll\n            for (int i = 0; i < 4; ++i) tail_epilogue(acc[i], mm_a[j][i], rowc * " << S(K) << " + 4 * blk + i, res[i], " << em.params_pass() << ");\n";
+            for (int o = 0; o < n_res; ++o)
+                k << "            if (row_ok) *(float4*)(b" << fk.outputs[rt.outputs[o]] << " + row * " << S(K) << " + 4 * blk) = make_float4(res[0][" << o << "], res[1][" << o << "], res[2][" << o << "], res[3][" << o << "]);\n";
+        } else {
+            k << "            if (row_ok) *(float4*)(b" << fk.outputs[rt.outputs[0]] << " + row * " << S(K) << " + 4 * blk) = make_float4(acc[0], acc[1], acc[2], acc[3]);\n";
+        }
+        k << "        }\n    }\n";
+    }
     k << "}\n";
     out->grid = blocks_for(m, (int)per_block);
     out->block = (unsigned)BT;
     out->source = k.str();
-    out->note = "row-fused: " + S(G) + " lanes per row, " + to_string(fk.row_stages.size()) + " stages" + (mm0 ? ", the first a MatMul over k=" + S(K) + " shared by the row's lanes" : "");
+    out->note = string(fk.row_tail.on ? "row-fused with the first stage's data gradient behind the last: " : "row-fused: ") + S(G) + " lanes per row, " + to_string(fk.row_stages.size()) + " stages" + (mm0 ? ", the first a MatMul over k=" + S(K) + " shared by the row's lanes" : "");
     return "";
 }
 
@@ -3311,6 +3356,11 @@ void count_work(const FusedKernel& fk, Generated* g) {
             if (o >= 0) elements += (double)element_count(st.k.raw().shape);
         if (st.store_a >= 0) elements += (double)element_count(st.k.raw().inputs[0].out_shape);
     }
+    if (fk.row_tail.on) {
+        const MatMulDims tg = matmul_dims(fk.row_tail.mm.raw());
+        elements += (double)(tg.k * tg.n) + (double)(tg.m * tg.n) * (double)fk.row_tail.outputs.size();
+        g->algo_flops += 2.0 * (double)tg.m * (double)tg.n * (double)tg.k;
+    }
     g->algo_bytes = 4.0 * elements;
 }
 
@@ -3397,6 +3447,16 @@ std::string FusedKernel::key() const {
     if (!row_stages.empty()) {
         s.append(reinterpret_cast<const char*>(&row_m), 8);
         s.append(reinterpret_cast<const char*>(&row_n), 8);
+    }
+    if (row_tail.on) {
+        s += "|RT" + row_tail.mm.key();
+        put_src(row_tail.b);
+        for (int v : {row_tail.x_stage, row_tail.x_stage_out, row_tail.epilogue_product_input, row_tail.epilogue_a_input}) s.append(reinterpret_cast<const char*>(&v), 4);
+        if (row_tail.has_epilogue) {
+            s += "E" + row_tail.epilogue.key();
+            for (auto& x : row_tail.epilogue_inputs) put_src(x);
+        }
+        for (int o : row_tail.outputs) s.append(reinterpret_cast<const char*>(&o), 4);
     }
     if (dgrad.on) {
         s += "|D";
@@ -3531,6 +3591,15 @@ static std::string generate_one(const FusedKernel& fk, Generated* out, bool with
         if ((int)st.inputs.size() != st.k.raw().n_inputs) return "row stage: input binding count";
         const int n_out = st.k.raw().kind == DSC_KERNEL_PER_ELEMENT ? st.k.raw().n_outputs : 1;
         if ((int)st.outputs.size() != n_out) return "row stage: output binding count";
+    }
+    if (fk.row_tail.on) {
+        err = validate(fk.row_tail.mm.raw());
+        if (!err.empty()) return "row tail: " + err;
+        if (fk.row_tail.has_epilogue) {
+            err = validate(fk.row_tail.epilogue.raw());
+            if (!err.empty()) return "row tail consumer: " + err;
+            if ((int)fk.row_tail.epilogue_inputs.size() != fk.row_tail.epilogue.raw().n_inputs) return "row tail consumer: input binding count";
+        }
     }
     if (fk.row_stages.empty() && (int)fk.inputs.size() != fk.main.raw().n_inputs + (fk.dgrad.on && fk.dgrad.wgrad ? 1 : 0)) return "input binding count";
     if ((int)fk.buffer_is_output.size() != fk.n_buffers) return "buffer table size";

@@ -67,6 +67,23 @@ struct FusedKernel {
     // `main` is the first stage's descriptor (for the label), only the outputs someone else needs are stored.
     std::vector<RowStage> row_stages;
     int64_t row_m = 0, row_n = 0;
+    // Row-fused kernel whose first stage is a MatMul over k: after the last stage, the product of one of the stages'
+    // [m, n] values X with a small matrix B2 [n, k] -- the data gradient of the layer the launch starts from, dZ x W^T
+    // -- with its per-element consumer.  A lane owns the same blocks of four k it multiplied in stage 0: X's columns
+    // come to it through shuffles, B2 sits in LDS, and where the consumer reads the A operand that stage 0 evaluated
+    // and stored (the activation the gradient is masked with), it takes it from the lane's registers.
+    struct RowTail {
+        bool on = false;
+        KernelDesc mm;                 // the MatMul [m, n] x [n, k]; inputs[1] is B2's view
+        int x_stage = -1, x_stage_out = 0;
+        Source b;                      // B2: a buffer
+        bool has_epilogue = false;
+        KernelDesc epilogue;
+        int epilogue_product_input = -1;
+        int epilogue_a_input = -1;     // epilogue input that reads stage 0's stored A operand element for element
+        std::vector<Source> epilogue_inputs;
+        std::vector<int> outputs;      // per output of the epilogue (or the product): index into FusedKernel::outputs
+    } row_tail;
     // Several independent small kernels in one launch: workgroup ids [0, g0) run parts[0], [g0, g0 + g1) run
     // parts[1], ...  part_params[i][j] is the pointer parameter of this kernel that part i's parameter j binds.
     // `main` is parts[0].main (for the label); inputs/outputs of the launch are those of the parts.

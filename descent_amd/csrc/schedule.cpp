@@ -79,6 +79,12 @@ void for_each_source(FusedKernel& fk, F f) {
     if (fk.pool.on && fk.pool.has_epilogue)
         for (size_t i = 0; i < fk.pool.epilogue_inputs.size(); ++i)
             if ((int)i != fk.pool.epilogue_product_input) f(fk.pool.epilogue_inputs[i]);
+    if (fk.row_tail.on) {
+        f(fk.row_tail.b);
+        if (fk.row_tail.has_epilogue)
+            for (size_t i = 0; i < fk.row_tail.epilogue_inputs.size(); ++i)
+                if ((int)i != fk.row_tail.epilogue_product_input && (int)i != fk.row_tail.epilogue_a_input) f(fk.row_tail.epilogue_inputs[i]);
+    }
 }
 
 // Drops pointer parameters nothing refers to and renumbers the rest.
@@ -1871,6 +1877,122 @@ struct Planner {
         drafts[ri] = fused;
     }
 
+    // Pass 2c: the data gradient of the layer a row-fused launch starts from.  The launch begins with Z = A x W
+    // ([m, k] x [k, n], n <= 64) and, in a training graph, produces dZ [m, n] among its outputs; the backward pass then
+    // wants dA = dZ x W^T [m, k], usually masked by the stored activation A (a short-k MatMul with a per-element
+    // consumer).  A lane of the row-fused kernel still owns the blocks of four k it multiplied in stage 0, dZ's row is
+    // in the registers of its row's lanes and W is small: the product runs behind the last stage, and its launch --
+    // on which the gradients of the layer below wait -- goes.  DSC_FUSE_ROWS_DGRAD=0 keeps it.
+    void rows_take_the_data_gradient(int ri) {
+        if (const char* e = std::getenv("DSC_FUSE_ROWS_DGRAD"))
+            if (e[0] == '0') return;
+        Draft& r = drafts[ri];
+        if (r.fk.row_stages.empty() || r.fk.row_stages[0].k.raw().kind != DSC_KERNEL_MATMUL || r.fk.row_tail.on) return;
+        const int64_t m = r.fk.row_m, n = r.fk.row_n;
+        const MatMulDims g0 = matmul_dims(r.fk.row_stages[0].k.raw());
+        if (g0.k % 4 != 0 || n * g0.k > 8192) return;
+        for (int ti = ri + 1; ti < (int)drafts.size(); ++ti) {
+            Draft& t = drafts[ti];
+            if (!t.alive || t.fk.main.raw().kind != DSC_KERNEL_MATMUL || !t.fk.virtuals.empty() || !t.fk.parts.empty() || !t.fk.row_stages.empty() ||
+                t.keep_split || t.keep_output || t.fk.dgrad.on || t.fk.cfwd.on || t.fk.pair.on || t.fk.colsum_out >= 0 || t.fk.out_slice_width)
+                continue;
+            const dsc_kernel_desc& td = t.fk.main.raw();
+            const MatMulDims g = matmul_dims(td);
+            if (g.batch != 1 || (g.chunks != 1 && !t.fk.sum_chunks) || g.m != m || g.k != n || g.n != g0.k || td.output_mode == DSC_MATMUL_ROWS) continue;
+            if (t.fk.inputs[0].buffer < 0 || t.fk.inputs[1].buffer < 0) continue;
+            // A = a wide value of the launch, read element for element
+            const int x_node = t.params[t.fk.inputs[0].buffer];
+            int xs = -1, xo = 0;
+            for (int si = 0; si < (int)r.fk.row_stages.size(); ++si) {
+                const RowStage& st = r.fk.row_stages[si];
+                const dsc_kernel_desc& sd = st.k.raw();
+                if (sd.kind != DSC_KERNEL_PER_ELEMENT || sd.shape.dims[0] != m * n) continue;
+                for (size_t o = 0; o < st.outputs.size(); ++o)
+                    if (st.outputs[o] >= 0 && r.params[r.fk.outputs[st.outputs[o]]] == x_node) { xs = si; xo = (int)o; }
+            }
+            if (xs < 0) continue;
+            int64_t base = 0, coef[DSC_MAX_DIM];
+            if (td.inputs[0].out_shape.rank != 3 || !affine_form(td.inputs[0], &base, coef) || base != 0 || coef[1] != n || coef[2] != 1) continue;
+            // B must exist when the row-fused launch runs
+            const int b_node = t.params[t.fk.inputs[1].buffer];
+            bool early = true;
+            for (int j = ri; j < ti; ++j)
+                if (drafts[j].alive)
+                    for (auto& o : drafts[j].outs)
+                        if (o.node == b_node) early = false;
+            if (!early) continue;
+            // the consumer's other operands: the A operand the launch stores (element for element), or arrays that
+            // exist before the launch
+            const int a_node = r.fk.row_stages[0].store_a >= 0 ? r.params[r.fk.outputs[r.fk.row_stages[0].store_a]] : -1;
+            int a_input = -1;
+            bool ok = true;
+            if (t.fk.has_epilogue) {
+                const dsc_kernel_desc& ed = t.fk.epilogue.raw();
+                if (ed.shape.dims[0] != m * g.n) continue;
+                for (int i = 0; i < ed.n_inputs && ok; ++i) {
+                    if (i == t.fk.epilogue_product_input) {
+                        ok = is_identity(ed.inputs[i]) || reads_in_order(ed.inputs[i]);
+                        continue;
+                    }
+                    const Source& src = t.fk.epilogue_inputs[i];
+                    if (src.buffer < 0) { ok = false; break; }
+                    const int nd = t.params[src.buffer];
+                    if (nd == a_node) {
+                        if (a_input >= 0 || !reads_in_order(ed.inputs[i])) ok = false;
+                        a_input = i;
+                        continue;
+                    }
+                    for (int j = ri; j < ti; ++j)
+                        if (drafts[j].alive)
+                            for (auto& o : drafts[j].outs)
+                                if (o.node == nd) ok = false;
+                }
+                for (int i = 0; i < ed.n_ops && ok; ++i)
+                    if (ed.ops[i].kind == DSC_PE_RAND || ed.ops[i].kind == DSC_PE_COORD || ed.ops[i].kind == DSC_PE_GATHER) ok = false;
+            }
+            if (!ok) continue;
+            for (auto& o : t.outs)
+                if (o.copy_from >= 0) ok = false;
+            if (!ok) continue;
+            {
+                std::vector<int> reads = input_nodes(t);
+                if (taken_in_place_between(ri, ti, reads)) continue;
+            }
+            Draft fused = r;
+            FusedKernel::RowTail& rt = fused.fk.row_tail;
+            rt.on = true;
+            rt.mm = t.fk.main;
+            rt.mm.d.shape.dims[0] = 1;  // one full sum over the n columns
+            rt.x_stage = xs;
+            rt.x_stage_out = xo;
+            rt.b = import_source(fused, t, t.fk.inputs[1], 0);
+            rt.has_epilogue = t.fk.has_epilogue;
+            if (t.fk.has_epilogue) {
+                rt.epilogue = t.fk.epilogue;
+                rt.epilogue_product_input = t.fk.epilogue_product_input;
+                rt.epilogue_a_input = a_input;
+                for (size_t i = 0; i < t.fk.epilogue_inputs.size(); ++i) {
+                    if ((int)i == t.fk.epilogue_product_input || (int)i == a_input) rt.epilogue_inputs.push_back(Source{});
+                    else rt.epilogue_inputs.push_back(import_source(fused, t, t.fk.epilogue_inputs[i], 0));
+                }
+            }
+            for (size_t o = 0; o < t.outs.size(); ++o) {
+                rt.outputs.push_back((int)fused.fk.outputs.size());
+                fused.fk.outputs.push_back(param_index(fused, t.outs[o].node, true));
+                fused.outs.push_back(t.outs[o]);
+            }
+            compact(fused);
+            {
+                Generated probe;
+                if (!generate(fused.fk, &probe).empty()) continue;
+            }
+            fused.covers.insert(fused.covers.end(), t.covers.begin(), t.covers.end());
+            t.alive = false;
+            drafts[ri] = fused;
+            return;
+        }
+    }
+
     // Pass 1i: per-element clusters over [rows, w] that pick their value by comparing the column with literals (each
     // concat of the reference is one: select(column > n - 1, pad(b), pad(a))) are marked to run a thread per row,
     // the column a constant of each of the row's w evaluations.  A chain of concats inlined into the last one then
@@ -2723,6 +2845,8 @@ struct Planner {
         inline_producers();                     // pass 2
         for (int i = 0; i < (int)drafts.size(); ++i)
             if (drafts[i].alive) rows_take_their_operands_producer(i);  // pass 2b
+        for (int i = 0; i < (int)drafts.size(); ++i)
+            if (drafts[i].alive) rows_take_the_data_gradient(i);        // pass 2c
         attach_epilogues();                     // pass 3
         slice_major_products();                 // pass 3d
         pool_joins_conv_forward();              // pass 3c

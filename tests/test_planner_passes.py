@@ -94,7 +94,7 @@ def test_bias_gradient_rides_on_the_weight_gradient_that_reads_the_same_array():
 def test_first_layer_filter_gradient_takes_the_pooling_gradient_as_a_producer():
     graph = workloads.convnet(_env(), batch=1000).graph
     listing = hip_backend.check_schedule(graph, fused=True)
-    assert int(listing.split()[0]) == 9
+    assert int(listing.split()[0]) == 8
     # conv2's backward kernel runs with loader waves and takes its dC the same way: the pooling gradient behind it is
     # a producer of that kernel's fills and no launch of its own
     line = next(l for l in listing.splitlines() if ": ConvBackward" in l)
@@ -127,7 +127,14 @@ def test_a_row_fused_launch_runs_the_light_cluster_that_produces_its_operand():
            "print(hip_backend.check_schedule(workloads.convnet(Environment(CpuBackend()), batch=1000).graph, fused=True))"
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     off = subprocess.run([sys.executable, "-c", code % root], env=dict(os.environ, DSC_FUSE_ROWS_OPERAND="0"), check=True, capture_output=True, text=True).stdout
-    assert int(off.split()[0]) == 10 and re.search(r"\d+: PerElement \(7 ops\) \[128000\] <1 fused producers>", off), off
+    assert int(off.split()[0]) == 9 and re.search(r"\d+: PerElement \(7 ops\) \[128000\] <1 fused producers>", off), off
+    # the same launch ends with the head's data gradient, dZ x W^T masked by the hidden layer it has just stored: the
+    # short-k MatMul is no launch part any more, and the gradients of the layer below share one launch with the head's
+    assert "row-fused with the first stage's data gradient behind the last" in line, line
+    assert "MatMul (k=10)" not in listing
+    assert re.search(r"Multi \(7 kernels: .*MatMul \(k=1000\) \[13, 1, 128, 10\]; MatMul \(k=128\) \[1, 1, 1000, 1568\]; MatMul \(k=1000\) \[13, 1, 1568, 128\];\)", listing), listing
+    no_tail = subprocess.run([sys.executable, "-c", code % root], env=dict(os.environ, DSC_FUSE_ROWS_DGRAD="0"), check=True, capture_output=True, text=True).stdout
+    assert int(no_tail.split()[0]) == 9 and "MatMul (k=10) [1, 1, 1000, 128]" in no_tail, no_tail
 
 
 def test_the_product_a_row_fused_launch_starts_from_is_its_first_stage():
@@ -249,7 +256,7 @@ def test_the_sign_of_a_pre_activation_is_read_off_the_stored_activation():
     # and dropped-out a (2 x 6.3) for 12.5 MB in
     assert "ConvForward" in lines[0] and 65.0 < moved(lines[0]) < 66.5, lines[0]     # 116.0 with z stored
     assert lines[1].split(": ")[1].startswith("ConvForward") and 49.5 < moved(lines[1]) < 51.0, lines[1]  # 75.3 with z stored
-    assert "358.9" in fused.splitlines()[-1], fused.splitlines()[-1]                  # MB per step; 565 with z stored, 414 before conv2's dC became a producer
+    assert "358.3" in fused.splitlines()[-1] or "358.4" in fused.splitlines()[-1], fused.splitlines()[-1]                  # MB per step; 565 with z stored, 414 before conv2's dC became a producer
     # cluster by cluster nothing is rewritten
     unfused = hip_backend.check_schedule(graph, fused=False)
     assert "PerElement (7 ops) [12544000]" in unfused and "2316." in unfused.splitlines()[-1], unfused.splitlines()[-1]
