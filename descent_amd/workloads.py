@@ -71,6 +71,17 @@ class Linear(Module):
         return x.flatten().apply(self.fc, ctx)
 
 
+class SingleLayer(Module):
+    """examples/fashion_mnist/main.rs:146-169: one hidden layer with leaky_relu(0.01)."""
+
+    def __init__(self, env, n_in=784, hidden_units=300, classes=10):
+        self.fc1 = Dense(env, n_in, hidden_units)
+        self.fc2 = Dense(env, hidden_units, classes)
+
+    def eval(self, x, ctx):
+        return x.flatten().apply(self.fc1, ctx).leaky_relu(0.01).apply(self.fc2, ctx)
+
+
 def _classifier_workload(env: Environment, module: Module, batch: int, side: int, optimizer: str,
                          rng: np.random.Generator, init: str = "he") -> Workload:
     """Train-graph assembly of examples/fashion_mnist/main.rs:235-287 (weight decay 0)."""
@@ -121,6 +132,13 @@ def convnet(env: Environment, batch: int = 1000, seed: int = 3, side: int = 28) 
     softmax cross-entropy."""
     rng = np.random.Generator(np.random.PCG64(seed))
     return _classifier_workload(env, ConvNet(env, side=side), batch, side, "adam", rng)
+
+
+def single_layer_classifier(env: Environment, batch: int = 1000, seed: int = 2, side: int = 28, hidden_units: int = 300,
+                            optimizer: str = "sgd") -> Workload:
+    """The reference's single-hidden-layer classifier (side*side -> hidden_units -> 10)."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    return _classifier_workload(env, SingleLayer(env, side * side, hidden_units), batch, side, optimizer, rng)
 
 
 def linear_classifier(env: Environment, batch: int = 1000, seed: int = 1) -> Workload:

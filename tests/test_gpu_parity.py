@@ -805,6 +805,64 @@ def test_graph_replay_with_an_output_that_starts_without_a_buffer(hip_backend_se
     assert m and (int(m.group(1)), int(m.group(2)), int(m.group(3))) == (4, 2, 0), listing
 
 
+@pytest.mark.parametrize("batch,side,hidden", [(1000, 28, 128), (333, 24, 300), (64, 28, 64)])
+@pytest.mark.parametrize("switch", [None, "DSC_FUSE_ROWS_DGRAD", "DSC_FUSE_ROWS_OPERAND"])
+def test_hidden_layer_classifier_head_in_one_row_fused_launch(hip_backend_session, monkeypatch, batch, side, hidden, switch):
+    """The reference's single-hidden-layer classifier, three momentum steps: the row-fused launch of the head evaluates
+    and stores the hidden activation (bias + leaky_relu over the first product's k chunks) and ends with the head's
+    data gradient masked by it; each of the two can be switched off, and all three ways match the oracle."""
+    from descent_amd import workloads
+
+    if switch:
+        monkeypatch.setenv(switch, "0")
+    genv, cenv = _envs(hip_backend_session)
+    gw = workloads.single_layer_classifier(genv, batch=batch, side=side, hidden_units=hidden)
+    cw = workloads.single_layer_classifier(cenv, batch=batch, side=side, hidden_units=hidden)
+    for step in range(3):
+        genv.run(gw.graph, 40 + step)
+        cenv.run(cw.graph, 40 + step)
+    listing = next(iter(gw.graph.__dict__["_schedules"].values())).describe()
+    line = next(l for l in listing.splitlines() if "RowFused" in l)
+    assert ("data gradient behind the last" in line) == (switch != "DSC_FUSE_ROWS_DGRAD"), listing
+    assert ("fused producers>" in line) == (switch != "DSC_FUSE_ROWS_OPERAND"), listing
+    got, want = gw.snapshot(), cw.snapshot()
+    for key in want:
+        if key == "accuracy":
+            assert np.array_equal(got[key], want[key]), key
+        else:
+            assert rel_l2(got[key], want[key]) <= TOL, (key, rel_l2(got[key], want[key]), listing)
+
+
+@pytest.mark.parametrize("loaders", ["0", "1", "2"])
+@pytest.mark.parametrize("batch,side", [(520, 28), (777, 20)])
+def test_convnet_backward_with_and_without_loader_waves(hip_backend_session, monkeypatch, loaders, batch, side):
+    """Two Adam steps of the ConvNet with the second convolution's backward kernel in its three forms: 256 threads that
+    fill, multiply and fold in turn (0), loader waves with the pooling gradient as a producer of their fills (1), loader
+    waves over a dC that stays a buffer (2)."""
+    from descent_amd import workloads
+
+    monkeypatch.setenv("DSC_CONV_BWD_LOADERS", loaders)
+    genv, cenv = _envs(hip_backend_session)
+    gw = workloads.convnet(genv, batch=batch, seed=31, side=side)
+    cw = workloads.convnet(cenv, batch=batch, seed=31, side=side)
+    for step in range(2):
+        genv.run(gw.graph, 7 + step)
+        cenv.run(cw.graph, 7 + step)
+    listing = next(iter(gw.graph.__dict__["_schedules"].values())).describe()
+    line = next(l for l in listing.splitlines() if "ConvBackward" in l)
+    assert ("loader waves" in line) == (loaders != "0"), listing
+    # (the pooling gradient becomes a producer of the fills only where the kernel is dC's one reader, which it is when
+    # the bias gradient's column sums ride on it: batch 1000, tests/test_gpu_full_size.py)
+    if loaders != "1":
+        assert "fused producers>" not in line.split("[conv backward")[0], listing
+    got, want = gw.snapshot(), cw.snapshot()
+    for key in want:
+        if key == "accuracy":
+            assert np.array_equal(got[key], want[key]), key
+        else:
+            assert rel_l2(got[key], want[key]) <= TOL, (key, rel_l2(got[key], want[key]), listing)
+
+
 def _conv_grad_case(env, m, h, w, c_in, c_out, fh, fw, pad, groups, seed):
     """x -> conv2d -> 0.5 * sum(y^2): the gradients with respect to the image and the filter."""
     from descent_amd import Initializer
