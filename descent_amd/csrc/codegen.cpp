@@ -581,6 +581,7 @@ struct Emitter {
 bool rows_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
 bool smallk_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
 bool tallk_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
+bool ksplit_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
 bool dot_kernel_applies(const FusedKernel& fk, const MatMulDims& g);
 bool dot_kernel_for_many_rows(const FusedKernel& fk, const MatMulDims& g);
 
@@ -612,6 +613,7 @@ string entry_name(const FusedKernel& fk) {
                       : rows_kernel_applies(fk, g)   ? "dsc_matmul_rows"
                       : smallk_kernel_applies(fk, g) ? "dsc_matmul_shortk"
                       : tallk_kernel_applies(fk, g)  ? "dsc_matmul_tallk"
+                      : ksplit_kernel_applies(fk, g) ? "dsc_matmul_ksplit"
                       : dot_kernel_applies(fk, g)    ? "dsc_matmul_dot"
                                                      : "dsc_matmul_mfma";
         if (fk.pair.on) base += "_wgrad";
@@ -2981,6 +2983,146 @@ string gen_matmul_tallk(Emitter& em, Generated* out) {
     return "";
 }
 
+// k split inside the workgroup: a product whose output is small (a few hundred 16x16 tiles) and whose k is a few
+// hundred to a few thousand long -- the first layer of a classifier at batch 1000, 1000 x 784 -> 128.  Tiled for the
+// MFMA template it is a few dozen workgroups walking k in sequential load -> LDS -> multiply round trips; split over k
+// into partial products it is two launches and a pass over the partials.  Here a workgroup owns a block of 16 rows x
+// NTB*16 columns for the WHOLE k: its waves take a slice of k each, load the 16x4 / 4x16 fragments of
+// v_mfma_f32_16x16x4f32 straight from memory (A in 16-byte pieces along k, B a word per lane and row, a batch of
+// k blocks requested before the first product), and meet in LDS, where the per-element consumer is applied before
+// the one store.  One launch, no partials in memory.
+struct KsplitPlan {
+    int ntb = 0, waves = 0;
+    int64_t blocks_m = 0, blocks_n = 0;
+};
+bool ksplit_plan(const FusedKernel& fk, const MatMulDims& g, KsplitPlan* p) {
+    if (const char* e = std::getenv("DSC_MM_KSPLIT"))
+        if (e[0] == '0') return false;
+    if (!(fk.sum_chunks || g.chunks == 1) || fk.colsum_out >= 0 || fk.out_slice_width || fk.pair.on || fk.dgrad.on || fk.cfwd.on) return false;
+    if (g.k < 512 || g.k > 2048 || g.m < 64 || g.n < 32 || g.n > 256) return false;
+    {
+        // both operands plain arrays, A's k along memory (16-byte pieces): a transposed or generated A would be
+        // fetched a word at a time by every one of the block's column workgroups
+        const dsc_kernel_desc& d = fk.main.raw();
+        int64_t ab = 0, ac[DSC_MAX_DIM] = {0};
+        if (fk.inputs.size() < 2 || fk.inputs[0].buffer < 0 || fk.inputs[1].buffer < 0 || d.inputs[0].out_shape.rank != 3 || !affine_form(d.inputs[0], &ab, ac) ||
+            ac[2] != 1 || ab % 4 != 0 || ac[1] % 4 != 0 || (g.batch > 1 && ac[0] % 4 != 0) || g.k % 4 != 0)
+            return false;
+    }
+    const int64_t bm = (g.m + 15) / 16;
+    // columns per workgroup: the widest block that still leaves about one workgroup per compute unit
+    int best = 0;
+    for (int ntb : {4, 2, 1}) {
+        if (16 * ntb > (g.n + 15) / 16 * 16) continue;  // no block wider than the product
+        const int64_t wgs = bm * ((g.n + 16 * ntb - 1) / (16 * ntb)) * g.batch;
+        if (wgs >= 192 && wgs <= 1024) { best = ntb; break; }
+    }
+    if (!best) return false;
+    // the MFMA template's tiles must be few for this to pay: otherwise its reuse of operands through LDS wins
+    if (((g.m + 63) / 64) * ((g.n + 63) / 64) * g.batch >= 128) return false;
+    p->ntb = best;
+    // (sixteen waves, one batch of loads each, measured the same as eight with two: 1000 x 128 over k = 784 8.6 us
+    // either way -- the 38 MB the 252 blocks pull out of L2 between them is what bounds it, not the round trips)
+    p->waves = 8;
+    p->blocks_m = bm;
+    p->blocks_n = (g.n + 16 * best - 1) / (16 * best);
+    return true;
+}
+bool ksplit_kernel_applies(const FusedKernel& fk, const MatMulDims& g) {
+    KsplitPlan p;
+    return ksplit_plan(fk, g, &p);
+}
+
+string gen_matmul_ksplit(Emitter& em, Generated* out) {
+    const FusedKernel& fk = em.fk;
+    const dsc_kernel_desc& d = fk.main.raw();
+    const MatMulDims g = matmul_dims(d);
+    KsplitPlan p;
+    if (!ksplit_plan(fk, g, &p)) return "matmul k-split: shape does not apply";
+    const bool rows = d.output_mode == DSC_MATMUL_ROWS;
+    const int64_t batch_stride = rows ? g.n : g.m * g.n, row_stride = rows ? g.batch * g.n : g.n;
+    const int NTB = p.ntb, W = p.waves;
+    const int64_t kw = ((g.k + W - 1) / W + 15) / 16 * 16;  // k per wave, whole blocks of 16
+    const int64_t nblk = kw / 16;
+    const int U = (int)std::min<int64_t>(nblk, NTB >= 4 ? 3 : 4);  // blocks of 16 k requested together
+
+    const string la = em.load_view(fk.inputs[0], d.inputs[0], {"cb", "cm", "ck"});
+    em.funcs << "DSC_INLINE float load_a(int cb, int cm, int ck, " << em.params_decl() << ") {\n    return " << la << ";\n}\n";
+    const string lb = em.load_view(fk.inputs[1], d.inputs[1], {"cb", "ck", "cn"});
+    em.funcs << "DSC_INLINE float load_b(int cb, int ck, int cn, " << em.params_decl() << ") {\n    return " << lb << ";\n}\n";
+    // A in 16-byte pieces where k runs along memory
+    int64_t ab = 0, ac[DSC_MAX_DIM] = {0};
+    const bool a_vec = fk.inputs[0].buffer >= 0 && d.inputs[0].out_shape.rank == 3 && affine_form(d.inputs[0], &ab, ac) && ac[2] == 1 && ab % 4 == 0 &&
+                       ac[1] % 4 == 0 && (g.batch == 1 || ac[0] % 4 == 0) && g.k % 4 == 0;
+    int n_out = 1;
+    if (fk.has_epilogue) {
+        const dsc_kernel_desc& pe = fk.epilogue.raw();
+        n_out = pe.n_outputs;
+        std::ostringstream body;
+        std::map<int, string> ov;
+        ov[fk.epilogue_product_input] = "product";
+        em.emit_pe(body, pe, fk.epilogue_inputs, "gid", "e", ov);
+        for (int o = 0; o < pe.n_outputs; ++o) body << "    result[" << o << "] = et" << pe.outputs[o] << ";\n";
+        em.funcs << "DSC_INLINE void mm_epilogue(float product, int gid, float* result, " << em.params_decl() << ") {\n" << body.str() << "}\n";
+    }
+    std::ostringstream k;
+    k << "typedef float ks_float4 __attribute__((ext_vector_type(4)));\n";
+    k << "extern \"C\" __global__ __launch_bounds__(" << 64 * W << ") void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
+    k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
+    k << "    __shared__ float red[" << W << "][" << NTB * 256 << "];\n";
+    k << "    const int bn = blockIdx.x % " << S(p.blocks_n) << ", bm = (blockIdx.x / " << S(p.blocks_n) << ") % " << S(p.blocks_m) << ", cb = blockIdx.x / " << S(p.blocks_n * p.blocks_m) << ";\n";
+    k << "    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), li = lane & 15, lk = lane >> 4;\n";
+    k << "    const int row = min(bm * 16 + li, " << S(g.m - 1) << ");\n";
+    k << "    const int k_begin = wave * " << S(kw) << ", k_end = min(k_begin + " << S(kw) << ", " << S(g.k) << ");\n";
+    k << "    ks_float4 acc[" << NTB << "];\n#pragma unroll\n    for (int nt = 0; nt < " << NTB << "; ++nt) acc[nt] = (ks_float4){0.f, 0.f, 0.f, 0.f};\n";
+    k << "    for (int k0 = k_begin; k0 < k_end; k0 += " << 16 * U << ") {\n";
+    k << "        float fa[" << U << "][4], fb[" << U << "][" << NTB << "][4];\n";
+    // a lane's four k of a block: 16 * u + 4 * lk + j.  Out-of-range k repeat a valid element's load and are zeroed
+    // after the fence; nothing before the fence consumes a loaded value, so the whole batch is in flight at once.
+    k << "#pragma unroll\n        for (int u = 0; u < " << U << "; ++u) {\n            const int kq = k0 + 16 * u + 4 * lk;\n";
+    if (a_vec) {
+        k << "            { const float4 q = *(const float4*)(b" << fk.inputs[0].buffer << " + " << S(ab) << " + cb * " << S(g.batch == 1 ? 0 : ac[0]) << " + row * " << S(ac[1])
+          << " + min(kq, " << S(g.k - 4) << ")); fa[u][0] = q.x; fa[u][1] = q.y; fa[u][2] = q.z; fa[u][3] = q.w; }\n";
+    } else {
+        k << "#pragma unroll\n            for (int j = 0; j < 4; ++j) fa[u][j] = load_a(cb, row, min(kq + j, " << S(g.k - 1) << "), " << em.params_pass() << ");\n";
+    }
+    k << "#pragma unroll\n            for (int nt = 0; nt < " << NTB << "; ++nt)\n#pragma unroll\n                for (int j = 0; j < 4; ++j)\n";
+    k << "                    fb[u][nt][j] = load_b(cb, min(kq + j, " << S(g.k - 1) << "), min((bn * " << NTB << " + nt) * 16 + li, " << S(g.n - 1) << "), " << em.params_pass() << ");\n";
+    k << "        }\n        __builtin_amdgcn_sched_barrier(0);\n";
+    k << "#pragma unroll\n        for (int u = 0; u < " << U << "; ++u)\n#pragma unroll\n            for (int j = 0; j < 4; ++j) {\n";
+    k << "                const bool k_ok = k0 + 16 * u + 4 * lk + j < k_end;\n";
+    if (a_vec) k << "                const float a = (k_ok && k0 + 16 * u + 4 * lk <= " << S(g.k - 4) << ") ? fa[u][j] : 0.f;\n";
+    else k << "                const float a = k_ok ? fa[u][j] : 0.f;\n";
+    k << "#pragma unroll\n                for (int nt = 0; nt < " << NTB << "; ++nt)\n";
+    k << "                    acc[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, k_ok ? fb[u][nt][j] : 0.f, acc[nt], 0, 0, 0);\n            }\n";
+    k << "    }\n";
+    // the waves' partial blocks meet in LDS; register r of lane l is D[4 * (l / 16) + r][l % 16]
+    k << "#pragma unroll\n    for (int nt = 0; nt < " << NTB << "; ++nt)\n#pragma unroll\n        for (int r = 0; r < 4; ++r) red[wave][nt * 256 + r * 64 + lane] = acc[nt][r];\n";
+    k << "    __syncthreads();\n";
+    k << "    for (int i = threadIdx.x; i < " << NTB * 256 << "; i += " << 64 * W << ") {\n        float sum = red[0][i];\n";
+    k << "#pragma unroll\n        for (int w = 1; w < " << W << "; ++w) sum += red[w][i];\n";
+    k << "        const int nt = i >> 8, r = (i >> 6) & 3, l = i & 63;\n";
+    k << "        const int cm = bm * 16 + 4 * (l >> 4) + r, cn = (bn * " << NTB << " + nt) * 16 + (l & 15);\n";
+    k << "        if (cm < " << S(g.m) << " && cn < " << S(g.n) << ") {\n            const int gid = cb * " << S(batch_stride) << " + cm * " << S(row_stride) << " + cn;\n";
+    if (fk.has_epilogue) {
+        k << "            float res[" << n_out << "];\n            mm_epilogue(sum, gid, res, " << em.params_pass() << ");\n";
+        for (int o = 0; o < n_out; ++o) k << "            b" << fk.outputs[o] << "[gid] = res[" << o << "];\n";
+    } else {
+        k << "            b" << fk.outputs[0] << "[gid] = sum;\n";
+    }
+    k << "        }\n    }\n}\n";
+    const int64_t grid = p.blocks_m * p.blocks_n * g.batch;
+    if (grid >= kMaxIndex) return "matmul: grid too large";
+    out->grid = (unsigned)grid;
+    out->block = (unsigned)(64 * W);
+    out->source = k.str();
+    char note[200];
+    std::snprintf(note, sizeof note, "k split over the %d waves of a workgroup, mfma 16x16x4 on a 16x%d block, operands from memory, %d blocks of 16 k in flight%s",
+                  W, 16 * NTB, U, fk.has_epilogue ? " +epilogue" : "");
+    out->note = note;
+    return "";
+}
+
 // Tile configuration, k chunking and grid of the MFMA template for one product.
 struct MmPlan {
     MmConfig c;
@@ -3026,6 +3168,7 @@ string gen_matmul(Emitter& em, Generated* out) {
     if (smallk_kernel_applies(fk, g)) return gen_matmul_smallk(em, out);
     if (tallk_kernel_applies(fk, g)) return gen_matmul_tallk(em, out);
     if (dot_kernel_applies(fk, g)) return gen_matmul_dot(em, out);
+    if (ksplit_kernel_applies(fk, g)) return gen_matmul_ksplit(em, out);
     MmPlan plan;
     if (!plan_mfma(fk, g, &plan, fk.as_part)) return "matmul: invalid tile configuration";
     MmConfig c = plan.c;
@@ -3391,6 +3534,12 @@ bool grad_pair_shapes(const FusedKernel& s, const FusedKernel& t, int64_t* chunk
     *chunks = gt.chunks;
     return (*chunks - 1) * *chunk_rows < gt.k && *chunks * *chunk_rows >= gt.k;
 }
+bool ksplit_kernel_shape(const FusedKernel& fk) {
+    FusedKernel probe = fk;
+    probe.sum_chunks = true;  // the planner asks before it has folded the sum over the reference's chunks in
+    return ksplit_kernel_applies(probe, matmul_dims(fk.main.raw()));
+}
+
 bool dot_kernel_shape(const MatMulDims& g) {
     const char* e = std::getenv("DSC_MM_DOT");
     return !(e && e[0] == '0') && dot_shape(g);
@@ -3499,7 +3648,7 @@ std::string FusedKernel::key() const {
     s.append(reinterpret_cast<const char*>(&n_buffers), 4);
     if (const char* env = std::getenv("DSC_MM_TILE"))
         if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|T") + env;
-    for (const char* name : {"DSC_MM_SMALLK", "DSC_MM_VEC_STORE", "DSC_MM_PERSISTENT", "DSC_MM_DEEP_K", "DSC_MM_DIRECT_LDS", "DSC_MM_ROWS", "DSC_MM_DOT", "DSC_ROWS_MFMA", "DSC_MM_TALLK"})
+    for (const char* name : {"DSC_MM_SMALLK", "DSC_MM_VEC_STORE", "DSC_MM_PERSISTENT", "DSC_MM_DEEP_K", "DSC_MM_DIRECT_LDS", "DSC_MM_ROWS", "DSC_MM_DOT", "DSC_ROWS_MFMA", "DSC_MM_TALLK", "DSC_MM_KSPLIT"})
         if (const char* env = std::getenv(name))
             if (main.raw().kind == DSC_KERNEL_MATMUL) s += string("|") + name + env;
     if (dgrad.on && dgrad.wgrad && !dgrad.wgrad_only)
@@ -3539,6 +3688,7 @@ bool can_be_part(const FusedKernel& fk) {
     // of the MatMul kernels, the row-per-thread, short-k and tall-k ones run 256 threads addressed by blockIdx.x
     const MatMulDims g = matmul_dims(fk.main.raw());
     if (rows_kernel_applies(fk, g) || smallk_kernel_applies(fk, g) || tallk_kernel_applies(fk, g) || dot_kernel_applies(fk, g)) return true;
+    if (ksplit_kernel_applies(fk, g)) return false;  // eight waves per workgroup
     if (fk.colsum_out >= 0) return false;
     // the MFMA template, when its tile choice runs four waves: small products only (large ones want their
     // workgroups persistent and the CU's whole LDS, which a shared launch cannot give them)

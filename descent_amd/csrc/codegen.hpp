@@ -249,6 +249,8 @@ bool can_be_part(const FusedKernel& k);
 // Whether a MatMul of these dimensions (already split into its chunks) runs on the tall-k kernel: a small output
 // summed over a long k, one workgroup per (chunk, batch).  The schedule sizes its k re-split for that kernel.
 bool tallk_shape(const MatMulDims& g);
+// the kernel that splits k over the waves of a workgroup takes this product whole (no k re-split, no partials)
+bool ksplit_kernel_shape(const FusedKernel& fk);
 // the dot-product kernel takes this product (rows x few columns over a k of moderate length)
 bool dot_kernel_shape(const MatMulDims& g);
 // `s` is a short-k MatMul with a consumer and `t` a plain tall-k MatMul shaped like the data and weight gradient of

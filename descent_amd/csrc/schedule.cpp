@@ -554,6 +554,7 @@ struct Planner {
             const MatMulDims g = matmul_dims(drafts[i].fk.main.raw());
             if (g.k < 512) continue;
             if (((g.m + 63) / 64) * ((g.n + 63) / 64) * g.batch >= 128) continue;  // the tile grid is already wide
+            if (ksplit_kernel_shape(drafts[i].fk)) continue;  // k is split inside the workgroups of one launch
             {
                 // rows of k-contiguous memory times a few columns: the dot-product kernel spreads k over lanes itself
                 const dsc_view& av = drafts[i].fk.main.raw().inputs[0];

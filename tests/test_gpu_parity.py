@@ -406,6 +406,23 @@ def test_large_matmul_sampled_rows(hip_backend_session):
     assert rel_l2(c[rows], want) <= TOL
 
 
+@pytest.mark.parametrize("m,n,k", [(1000, 128, 784), (1000, 128, 1568), (777, 100, 600), (3000, 36, 516), (257, 200, 2048), (4099, 32, 1024)])
+def test_matmul_with_k_split_inside_the_workgroups(hip_backend_session, m, n, k):
+    """Small products over a moderate k run as one launch, the eight waves of a workgroup a slice of k each: ragged row
+    and column counts, k that is no multiple of 16 or of the waves' slices, against a float64 product."""
+    from descent_amd import Environment, workloads
+
+    env = Environment(hip_backend_session)
+    w = workloads.matmul_epilogue(env, m, n, k, seed=m + n + k)
+    env.run(w.graph, 0)
+    listing = next(iter(w.graph.__dict__["_schedules"].values())).describe()
+    assert int(listing.split()[0]) == 1 and "k split over the 8 waves of a workgroup" in listing, listing
+    a = env.read_parameter(w.a).astype(np.float64)
+    b = env.read_parameter(w.b).astype(np.float64)
+    z = a @ b + env.read_parameter(w.bias).astype(np.float64)
+    assert rel_l2(env.read_parameter(w.c), np.where(z > 0, z, 0.01 * z)) <= 2e-6, listing
+
+
 def test_heap_reuse_and_errors(hip_backend_session):
     from descent_amd.hip_backend import DescentHipError
 
@@ -815,6 +832,9 @@ def test_hidden_layer_classifier_head_in_one_row_fused_launch(hip_backend_sessio
 
     if switch:
         monkeypatch.setenv(switch, "0")
+    # (the first product's k stays split into chunks here: on the kernel that splits k inside its workgroups the hidden
+    # activation is that kernel's epilogue and there is no cluster for the row-fused launch to take)
+    monkeypatch.setenv("DSC_MM_KSPLIT", "0")
     genv, cenv = _envs(hip_backend_session)
     gw = workloads.single_layer_classifier(genv, batch=batch, side=side, hidden_units=hidden)
     cw = workloads.single_layer_classifier(cenv, batch=batch, side=side, hidden_units=hidden)
