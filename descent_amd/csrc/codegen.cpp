@@ -1583,7 +1583,7 @@ string gen_conv_dgrad(Emitter& em, Generated* out) {
 // of dC: the bias gradient.  The accumulators live across the workgroup's images; the four waves take every fourth
 // step and are summed through LDS at the end, one partial product per workgroup.
 struct ConvBwdLayout {
-    int64_t PH, PW, KD, PITCH, CP, SLP, steps, ZERO_AT, XT_AT, XT_FLOATS, ONE_AT, ZW_AT, GB_AT, TOTAL;
+    int64_t PH, PW, KD, PITCH, CP, SLP, steps, DC_AT, ZERO_AT, XT_AT, XT_FLOATS, ONE_AT, ZW_AT, GB_AT, TOTAL;
     int MT, NT;
     // data gradient on the matrix cores (see gen_conv_bwd): pixels per group, shifted taps per filter row, B fragments
     // per lane, groups per image row, groups, tiles of 16 groups, tiles per wave
@@ -1631,8 +1631,13 @@ ConvBwdLayout conv_bwd_layout(const FusedKernel::ConvDgrad& full, int64_t K, int
     }
     L.SLP = (c.oh * L.PW + 3) / 4 * 4;
     L.steps = L.SLP / 4;
-    L.ZERO_AT = L.SLP * L.PITCH;
-    L.XT_AT = (L.ZERO_AT + L.PITCH + 3) / 4 * 4;
+    // With the data gradient on the matrix cores the slots start behind fw - 1 slots that stay zero and the zero row is
+    // as long as a filter row's taps reach: a lane's fragments of a filter row then lie at literal distances from one
+    // address (a tap left of the image falls on the zero slots that end the row above, or on the head), and a filter
+    // row outside the image takes that address to the zero row as a whole.
+    L.DC_AT = L.mfma_dgrad ? ((c.fw - 1) * L.PITCH + 3) / 4 * 4 : 0;
+    L.ZERO_AT = L.DC_AT + L.SLP * L.PITCH;
+    L.XT_AT = (L.ZERO_AT + (L.mfma_dgrad ? (L.TQ - 1) * L.PITCH + K + 4 : L.PITCH) + 3) / 4 * 4;
     const int64_t pixels = std::max(L.PH * L.PW, L.SLP + (c.fh - 1) * L.PW + c.fw - 1);  // what a fragment load may address
     L.XT_FLOATS = (pixels * L.CP + 3) / 4 * 4;
     L.ONE_AT = L.XT_AT + L.XT_FLOATS;
@@ -1746,7 +1751,7 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     k << "        a_msk[mt] = real ? -1 : 0;\n    }\n";
     k << "#pragma unroll\n    for (int nt = 0; nt < " << NT << "; ++nt) {\n";
     k << "        const int oc = nt * 16 + li;\n";
-    k << "        b_off[nt] = oc < " << S(K) << " ? oc : " << S(L.ZERO_AT) << ";\n        b_msk[nt] = oc < " << S(K) << " ? -1 : 0;\n    }\n";
+    k << "        b_off[nt] = oc < " << S(K) << " ? " << S(L.DC_AT) << " + oc : " << S(L.ZERO_AT) << ";\n        b_msk[nt] = oc < " << S(K) << " ? -1 : 0;\n    }\n";
     k << "    cb_float4 wacc[" << MT << "][" << NT << "];\n";
     k << "#pragma unroll\n    for (int mt = 0; mt < " << MT << "; ++mt)\n#pragma unroll\n        for (int nt = 0; nt < " << NT
       << "; ++nt) wacc[mt][nt] = (cb_float4){0.f, 0.f, 0.f, 0.f};\n";
@@ -1758,6 +1763,13 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     // the B fragments are the same for every group: they stay in registers for the whole kernel.
     const int64_t P = L.P, TQ = L.TQ, GS = L.GS, GPR = L.GPR, GROUPS = L.GROUPS, TPW = L.TPW;
     const bool mfma_dgrad = L.mfma_dgrad;
+    if (mfma_dgrad && spec) {
+        // this lane's pixel group in each of the wave's tiles: its row, and the word of its first tap in filter row 0
+        k << "    int dgy[" << S(TPW) << "], dbase[" << S(TPW) << "];\n";
+        k << "#pragma unroll\n    for (int t = 0; t < " << S(TPW) << "; ++t) {\n";
+        k << "        const int grp = (t * 4 + wave) * 16 + li;\n        dgy[t] = grp / " << S(GPR) << ";\n";
+        k << "        dbase[t] = " << S(L.DC_AT) << " + (dgy[t] * " << S(PW) << " + (grp % " << S(GPR) << ") * " << S(P) << " - " << S(FW - 1) << ") * " << S(PITCH) << " + lk;\n    }\n";
+    }
     if (mfma_dgrad) {
         k << "    {\n";
         k << "        const int par = li / " << S(C) << ", gc = li % " << S(C) << ";\n";
@@ -1812,7 +1824,7 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     auto emit_tile_stores = [&](const string& ind, const string& buf) {
         k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NC) << "; ++u) {\n";
         k << ind << "    const int i = (tid + u * 256) * " << S(dunit) << ", pi = i / " << S(K) << ";\n";
-        k << ind << "    float* const at = lds + " << buf << " + ((pi / " << S(OW) << ") * " << S(PW) << " + pi % " << S(OW) << ") * " << S(PITCH) << " + i % " << S(K) << ";\n";
+        k << ind << "    float* const at = lds + " << buf << " + " << S(L.DC_AT) << " + ((pi / " << S(OW) << ") * " << S(PW) << " + pi % " << S(OW) << ") * " << S(PITCH) << " + i % " << S(K) << ";\n";
         if (quad_dc && PITCH % 4 == 0)
             k << ind << "    if (tid + u * 256 < " << S(fill_n) << ") *(float4*)at = pv[u];\n" << ind << "}\n";
         else if (quad_dc)
@@ -1850,20 +1862,42 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     if (spec) {
         // Two waves per SIMD run these products (the other two are loader waves), so a wave has to keep the matrix
         // pipe busy by itself: the fragments of two steps are requested before the first product is issued.
-        k << "#pragma unroll 1\n        for (int s = wave; s < " << S(L.steps) << "; s += 8) {\n";
-        k << "            const bool two = s + 4 < " << S(L.steps) << ";\n";
-        k << "            const int q0 = 4 * s + lk, q1 = 4 * min(s + 4, " << S(L.steps - 1) << ") + lk;\n";
+        // The fragment addresses are running registers: a step is an add per fragment (none for the second step of
+        // a pair in the tiles whose rows are all real: its distance is a literal in the read), where a slot term
+        // computed from the step number cost two to three vector instructions per read -- and vector instructions
+        // do not hide behind the products of the other wave on the SIMD, they take turns with them.
+        auto full_a = [&](int mt) { return (int64_t)(mt + 1) * 16 <= KD; };
+        auto full_b = [&](int nt) { return (int64_t)(nt + 1) * 16 <= K; };
+        k << "        const char* const sbytes = (const char*)smem;\n        int aw[" << MT << "], bw[" << NT << "];  // in bytes\n";
+        k << "#pragma unroll\n        for (int mt = 0; mt < " << MT << "; ++mt) aw[mt] = 4 * (a_off[mt] + ((((4 * wave + lk) * " << S(CP) << ") + bo) & a_msk[mt]));\n";
+        k << "#pragma unroll\n        for (int nt = 0; nt < " << NT << "; ++nt) bw[nt] = 4 * (b_off[nt] + bo + (((4 * wave + lk) * " << S(PITCH) << ") & b_msk[nt]));\n";
+        auto emit_reads = [&](const string& ind, int halves) {
+            for (int h = 0; h < halves; ++h) {
+                for (int mt = 0; mt < MT; ++mt)
+                    k << ind << "fa[" << h << "][" << mt << "] = *(const float*)(sbytes + aw[" << mt << "]" << (h ? (full_a(mt) ? " + " + S(64 * CP) : " + (" + S(64 * CP) + " & a_msk[" + to_string(mt) + "])") : string()) << ");\n";
+                for (int nt = 0; nt < NT; ++nt)
+                    k << ind << "fb[" << h << "][" << nt << "] = *(const float*)(sbytes + bw[" << nt << "]" << (h ? (full_b(nt) ? " + " + S(64 * PITCH) : " + (" + S(64 * PITCH) + " & b_msk[" + to_string(nt) + "])") : string()) << ");\n";
+            }
+        };
+        k << "        int s = wave;\n";
+        k << "#pragma unroll 1\n        for (; s + 4 < " << S(L.steps) << "; s += 8) {\n";
         k << "            float fa[2][" << MT << "], fb[2][" << NT << "];\n";
-        k << "#pragma unroll\n            for (int h = 0; h < 2; ++h) {\n";
-        k << "                const int qa = (h ? q1 : q0) * " << S(CP) << ", qb = (h ? q1 : q0) * " << S(PITCH) << ";\n";
-        k << "#pragma unroll\n                for (int mt = 0; mt < " << MT << "; ++mt) fa[h][mt] = smem[a_off[mt] + ((qa + bo) & a_msk[mt])];\n";
-        k << "#pragma unroll\n                for (int nt = 0; nt < " << NT << "; ++nt) fb[h][nt] = smem[b_off[nt] + bo + (qb & b_msk[nt])];\n";
-        k << "            }\n";
-        k << "#pragma unroll\n            for (int nt = 0; nt < " << NT << "; ++nt) fb[1][nt] = two ? fb[1][nt] : 0.f;\n";
+        emit_reads("            ", 2);
         k << "            __builtin_amdgcn_sched_barrier(0);\n";
         k << "#pragma unroll\n            for (int h = 0; h < 2; ++h)\n#pragma unroll\n                for (int mt = 0; mt < " << MT << "; ++mt)\n#pragma unroll\n                    for (int nt = 0; nt < " << NT << "; ++nt)\n";
         k << "                        wacc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[h][mt], fb[h][nt], wacc[mt][nt], 0, 0, 0);\n";
         k << "            __builtin_amdgcn_sched_barrier(0);\n";
+        for (int mt = 0; mt < MT; ++mt)
+            k << "            aw[" << mt << "] += " << (full_a(mt) ? S(128 * CP) : "(" + S(128 * CP) + " & a_msk[" + to_string(mt) + "])") << ";\n";
+        for (int nt = 0; nt < NT; ++nt)
+            k << "            bw[" << nt << "] += " << (full_b(nt) ? S(128 * PITCH) : "(" + S(128 * PITCH) + " & b_msk[" + to_string(nt) + "])") << ";\n";
+        k << "        }\n";
+        // the wave's odd step, where it has one
+        k << "        if (s < " << S(L.steps) << ") {\n";
+        k << "            float fa[1][" << MT << "], fb[1][" << NT << "];\n";
+        emit_reads("            ", 1);
+        k << "#pragma unroll\n            for (int mt = 0; mt < " << MT << "; ++mt)\n#pragma unroll\n                for (int nt = 0; nt < " << NT << "; ++nt)\n";
+        k << "                    wacc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[0][mt], fb[0][nt], wacc[mt][nt], 0, 0, 0);\n";
         k << "        }\n";
     }
     if (!spec) {
@@ -1891,13 +1925,13 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
             k << "            const float* const gbp = smem + " << S(GB_AT) << " + ty * " << S(NF * 64) << " + lane;\n";
             k << "            float fa[" << S(TPW) << "][" << S(NF) << "], fb[" << S(NF) << "];\n";
             k << "#pragma unroll\n            for (int i = 0; i < " << S(NF) << "; ++i) fb[i] = gbp[i * 64];\n";
+            // one address per tile and filter row: the row's first tap of this lane's group, or the zero row
             k << "#pragma unroll\n            for (int t = 0; t < " << S(TPW) << "; ++t) {\n";
-            k << "                const int grp = (t * 4 + wave) * 16 + li, oy = grp / " << S(GPR) << " - ty, gx0 = (grp % " << S(GPR) << ") * " << S(P) << ";\n";
-            k << "#pragma unroll\n                for (int tqi = 0; tqi < " << S(TQ) << "; ++tqi) {\n";
-            k << "                    const int ox = gx0 - (tqi - " << S(P - 1) << ");\n";
-            k << "                    const int at = bo + ((oy >= 0 && oy < " << S(OH) << " && ox >= 0 && ox < " << S(OW) << ") ? (oy * " << S(PW) << " + ox) * " << S(PITCH) << " : " << S(L.ZERO_AT) << ");\n";
-            k << "#pragma unroll\n                    for (int o4 = 0; o4 < " << S(K4) << "; ++o4) fa[t][tqi * " << S(K4) << " + o4] = lds[at + 4 * o4 + lk];\n";
-            k << "                }\n            }\n";
+            k << "                const int oy = dgy[t] - ty;\n";
+            k << "                const int at = bo + ((unsigned)oy < " << S(OH) << "u ? dbase[t] - ty * " << S(PW * PITCH) << " : " << S(L.ZERO_AT) << " + lk);\n";
+            k << "#pragma unroll\n                for (int tqi = 0; tqi < " << S(TQ) << "; ++tqi)\n";
+            k << "#pragma unroll\n                    for (int o4 = 0; o4 < " << S(K4) << "; ++o4) fa[t][tqi * " << S(K4) << " + o4] = lds[at + (" << S(TQ - 1) << " - tqi) * " << S(PITCH) << " + 4 * o4];\n";
+            k << "            }\n";
             k << "            __builtin_amdgcn_sched_barrier(0);\n";
             k << "#pragma unroll\n            for (int i = 0; i < " << S(NF) << "; ++i)\n#pragma unroll\n                for (int t = 0; t < " << S(TPW) << "; ++t)\n";
             k << "                    dacc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[t][i], fb[i], dacc[t], 0, 0, 0);\n";
@@ -1915,7 +1949,7 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         for (int64_t tqi = 0; tqi < TQ; ++tqi) {
             const int64_t tq = tqi - (P - 1);
             k << "                {\n                    const int ox = gx0 - " << S(tq) << ";\n";
-            k << "                    const int at = bo + ((oy >= 0 && oy < " << S(OH) << " && ox >= 0 && ox < " << S(OW) << ") ? (oy * " << S(PW) << " + ox) * " << S(PITCH) << " : "
+            k << "                    const int at = bo + ((oy >= 0 && oy < " << S(OH) << " && ox >= 0 && ox < " << S(OW) << ") ? " << S(L.DC_AT) << " + (oy * " << S(PW) << " + ox) * " << S(PITCH) << " : "
               << S(L.ZERO_AT) << ");\n";
             for (int64_t o4 = 0; o4 < K / 4; ++o4)
                 k << "                    d = __builtin_amdgcn_mfma_f32_16x16x4f32(lds[at + " << S(4 * o4) << " + lk], gbp[" << S((tqi * (K / 4) + o4) * 64) << "], d, 0, 0, 0);\n";
@@ -1952,7 +1986,7 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     k << "                const int fy = tap / " << S(FW) << ", fx = tap % " << S(FW) << ";\n";
     k << "                const int oy = py - fy, ox = px - fx;\n";
     k << "                const bool inside = oy >= 0 && oy < " << S(OH) << " && ox >= 0 && ox < " << S(OW) << ";\n";
-    k << "                const float* src = &lds[bo + (inside ? (oy * " << S(PW) << " + ox) * " << S(PITCH) << " : " << S(L.ZERO_AT) << ")];\n";
+    k << "                const float* src = &lds[bo + (inside ? " << S(L.DC_AT) << " + (oy * " << S(PW) << " + ox) * " << S(PITCH) << " : " << S(L.ZERO_AT) << ")];\n";
     k << "#pragma unroll\n                for (int oc = 0; oc < " << S(K) << "; oc += " << OCB << ") {\n";
     k << "                    float a[" << OCB << "];\n";
     k << "#pragma unroll\n                    for (int q = 0; q < " << OCB << "; q += 4) {\n";
