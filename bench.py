@@ -136,7 +136,9 @@ def bench_convnet(env, steps, warmup, batch=1000, repeats=5):
     from descent_amd import workloads
 
     w = workloads.convnet(env, batch=batch, seed=3)
-    walls = [time_graph(env, w.graph, steps, warmup if r == 0 else 0, seed0=1 + r * steps, profile=False) for r in range(repeats)]
+    # (the warm-up is long enough for the device to reach the clock it holds under this load: the first region of a run
+    # that starts from idle reads 1.5 % low)
+    walls = [time_graph(env, w.graph, steps, max(warmup, 1000) if r == 0 else 0, seed0=1 + r * steps, profile=False) for r in range(repeats)]
     wall = sorted(walls)[len(walls) // 2]
     if EVENT_PASS:
         time_graph(env, w.graph, min(steps, 50), 0, seed0=100000, profile=True)
@@ -313,31 +315,39 @@ def _compact_classes(classes):
     return out
 
 
-def bench_configs(env, warmup=3):
+def bench_configs(env):
     """The configurations the headline does not cover, compact enough for the one JSON line: the other four
     standalone matmul shapes (each verified on sampled rows against float64 after its timed region), the linear
     classifier, both coordinate MLPs and the hash-grid fit (step rate, launches, per-class roofline fractions,
-    and the summed loss of the timed steps, which must be finite)."""
+    and the summed loss of the timed steps, which must be finite).
+
+    Every timed region follows a warm-up of the same launches that lasts a quarter of a second or so, and lasts about
+    as long itself: the device raises its clock over the first milliseconds of a burst of work, and a launch of tens or
+    hundreds of microseconds timed twenty times from idle is measured on the ramp (262144x256x256: 345 us per launch
+    over 20 launches from idle, 288 over 200, 275 over 3000; 4096^3 1099 us over 10, 977 over 300; the 8192^3 headline
+    takes 7.6 ms per launch and reads the same over 5 launches and over 100)."""
     from descent_amd import workloads as _w
 
     out = {"matmul": {}}
-    for (m, n, k), steps in (((1024, 1024, 1024), 50), ((4096, 4096, 4096), 20), ((1000, 128, 784), 50), ((262144, 256, 256), 20)):
+    for (m, n, k), warmup, steps in (((1024, 1024, 1024), 4000, 6000), ((4096, 4096, 4096), 150, 250), ((1000, 128, 784), 4000, 6000),
+                                     ((262144, 256, 256), 600, 900)):
         r = bench_matmul(env, m, n, k, steps, warmup, verify=True)
         ok = r["rel_l2_error_sampled_rows"] <= 1e-4
         # a product of one launch: rate of that launch; of several (k re-split + the sum of its partials): of all of them
         us = r["kernel_us_per_step"]
         out["matmul"]["%dx%dx%d" % (m, n, k)] = {
             "tflops_kernels": round(r["flops"] / (us * 1e-6) / 1e12, 2), "frac_mfma": round(r["flops"] / (us * 1e-6) / 1e12 / MFMA_FP32_PEAK_TFLOPS, 3),
-            "kernels_us": round(us, 2), "tflops_wall": round(r["tflops_wall"], 2), "launches": r["launches_per_step"],
+            "kernels_us": round(us, 2), "tflops_wall": round(r["tflops_wall"], 2), "launches": r["launches_per_step"], "steps": steps, "warmup": warmup,
             "rel_l2_error_sampled_rows": r["rel_l2_error_sampled_rows"], "verified": bool(ok)}
-    builds = (("cfg1_linear_classifier_bs1000", lambda e: _w.linear_classifier(e), 200),
-              ("cfg4_coordinate_mlp_relu_pe_512", lambda e: _w.coordinate_mlp(e), 10),
-              ("cfg4_coordinate_mlp_siren_512", lambda e: _w.coordinate_mlp(e, variant="siren"), 10),
-              ("cfg5_hash_grid_2p18", lambda e: _w.hash_grid_fit(e), 20))
-    for name, build, steps in builds:
-        r, _ = bench_workload(env, build, steps, 2, read_loss=True)
+    builds = (("cfg1_linear_classifier_bs1000", lambda e: _w.linear_classifier(e), 2000, 5000),
+              ("cfg4_coordinate_mlp_relu_pe_512", lambda e: _w.coordinate_mlp(e), 40, 80),
+              ("cfg4_coordinate_mlp_siren_512", lambda e: _w.coordinate_mlp(e, variant="siren"), 40, 80),
+              ("cfg5_hash_grid_2p18", lambda e: _w.hash_grid_fit(e), 200, 400))
+    for name, build, warmup, steps in builds:
+        r, _ = bench_workload(env, build, steps, warmup, read_loss=True)
         out[name] = {"steps_per_s": round(r["steps_per_s"], 1), "ms_per_step": round(r["ms_per_step"], 4), "launches": r["launches_per_step"],
-                     "clusters": r["clusters"], "loss_sum_finite": r["loss_finite"], "kernel_classes": _compact_classes(r["kernel_classes"])}
+                     "clusters": r["clusters"], "steps": steps, "warmup": warmup, "loss_sum_finite": r["loss_finite"],
+                     "kernel_classes": _compact_classes(r["kernel_classes"])}
     return out
 
 
@@ -459,15 +469,15 @@ def main():
                            bench_reduce(env, 262144, 256, 0, 20, 3)]
         from descent_amd import workloads as _w
 
-        mlp, rep = bench_workload(env, lambda e: _w.coordinate_mlp(e), 10, 2)
+        mlp, rep = bench_workload(env, lambda e: _w.coordinate_mlp(e), 80, 40)
         sys.stderr.write("cfg4 coordinate MLP (relu-pe):\n" + rep)
         extra["coordinate_mlp_relu_pe_512"] = mlp
-        siren, rep = bench_workload(env, lambda e: _w.coordinate_mlp(e, variant="siren"), 10, 2)
+        siren, rep = bench_workload(env, lambda e: _w.coordinate_mlp(e, variant="siren"), 80, 40)
         extra["coordinate_mlp_siren_512"] = siren
-        lin, rep = bench_workload(env, lambda e: _w.linear_classifier(e), 50, 5)
+        lin, rep = bench_workload(env, lambda e: _w.linear_classifier(e), 5000, 2000)
         sys.stderr.write("cfg1 linear classifier:\n" + rep)
         extra["linear_classifier_bs1000"] = lin
-        hg, rep = bench_workload(env, lambda e: _w.hash_grid_fit(e), 10, 2)
+        hg, rep = bench_workload(env, lambda e: _w.hash_grid_fit(e), 400, 200)
         sys.stderr.write("cfg5 hash grid:\n" + rep)
         sc = hg["kernel_classes"].get("Multi (4 kernels: ScatterAdd") or hg["kernel_classes"].get("ScatterAdd")
         hg["scatter_atomics_per_s"] = 16 * 4 * 2 * (1 << 18) / (sc["us_per_step"] * 1e-6) if sc else None
