@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes one launch of the headline kernel moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same
 # command, each counter scaled by what it reads for the streaming kernel of known size (--copy-calibration); the
 # summary is profiles/matmul_mfma_8192.txt.  Only the 8192^3 workload has been counted.
-MEASURED_TRAFFIC_BYTES = {8192: 3.550e9}
+MEASURED_TRAFFIC_BYTES = {8192: 3.546e9}
 
 
 def time_graph(env, graph, steps: int, warmup: int, seed0: int = 1, profile: bool = True):
@@ -303,6 +303,11 @@ def bench_upload(env, n):
     return {"upload_gbs": a.nbytes / up / 1e9, "matmul_with_upload_tflops": w.flops / dt / 1e12, "ms_per_step_with_upload": dt * 1e3}
 
 
+# the cfg2 shapes beside the headline, each with the warm-up and the number of timed launches that put about a quarter of
+# a second of the same work before and inside the timed region
+CFG2_OTHER_SHAPES = (((1024, 1024, 1024), 4000, 6000), ((4096, 4096, 4096), 150, 250), ((1000, 128, 784), 4000, 6000), ((262144, 256, 256), 600, 900))
+
+
 def _compact_classes(classes):
     """Kernel classes of a step, compact: microseconds per step, launches, and the fraction of the roof each class's
     algorithmic work reaches (HBM always; fp32 MFMA where the class multiplies matrices)."""
@@ -329,8 +334,7 @@ def bench_configs(env):
     from descent_amd import workloads as _w
 
     out = {"matmul": {}}
-    for (m, n, k), warmup, steps in (((1024, 1024, 1024), 4000, 6000), ((4096, 4096, 4096), 150, 250), ((1000, 128, 784), 4000, 6000),
-                                     ((262144, 256, 256), 600, 900)):
+    for (m, n, k), warmup, steps in CFG2_OTHER_SHAPES:
         r = bench_matmul(env, m, n, k, steps, warmup, verify=True)
         ok = r["rel_l2_error_sampled_rows"] <= 1e-4
         # a product of one launch: rate of that launch; of several (k re-split + the sum of its partials): of all of them
@@ -456,17 +460,16 @@ def main():
     extra = {}
     conv = None
     if args.all:
-        shapes = [(1024, 1024, 1024), (4096, 4096, 4096), (1000, 128, 784), (262144, 256, 256)]
         extra["matmul"] = []
-        for (m, nn, k) in shapes:
-            r = bench_matmul(env, m, nn, k, max(args.steps, 20), args.warmup)
+        for (m, nn, k), shape_warmup, shape_steps in CFG2_OTHER_SHAPES:
+            r = bench_matmul(env, m, nn, k, shape_steps, shape_warmup)
             r.pop("report")
             extra["matmul"].append(r)
-        extra["elementwise_axpb_64M"] = bench_elementwise(env, 1 << 26, max(args.steps, 20), args.warmup)
+        extra["elementwise_axpb_64M"] = bench_elementwise(env, 1 << 26, 1500, 1000)
         extra["host_operands"] = bench_upload(env, n)
         extra["convnet_bs1000_minibatch_uploads"] = bench_convnet_minibatch_uploads(env)
-        extra["reduce"] = [bench_reduce(env, 8192, 8192, 1, 20, 3), bench_reduce(env, 8192, 8192, 0, 20, 3),
-                           bench_reduce(env, 262144, 256, 0, 20, 3)]
+        extra["reduce"] = [bench_reduce(env, 8192, 8192, 1, 3000, 2000), bench_reduce(env, 8192, 8192, 0, 3000, 2000),
+                           bench_reduce(env, 262144, 256, 0, 3000, 2000)]
         from descent_amd import workloads as _w
 
         mlp, rep = bench_workload(env, lambda e: _w.coordinate_mlp(e), 80, 40)

@@ -3104,7 +3104,13 @@ string gen_matmul_ksplit(Emitter& em, Generated* out) {
     k << "extern \"C\" __global__ __launch_bounds__(" << 64 * W << ") void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
     k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
     k << "    __shared__ float red[" << W << "][" << NTB * 256 << "];\n";
-    k << "    const int bn = blockIdx.x % " << S(p.blocks_n) << ", bm = (blockIdx.x / " << S(p.blocks_n) << ") % " << S(p.blocks_m) << ", cb = blockIdx.x / " << S(p.blocks_n * p.blocks_m) << ";\n";
+    // Consecutive workgroup ids go to consecutive XCDs: the column blocks of a row block (which read the same rows of
+    // A) get ids 8 apart, so that they share one L2 (measured for 1000x128x1568: 26.8 MB fetched from memory per launch
+    // with neighbouring ids, for 7.1 MB of operands).
+    const int64_t ks_total = p.blocks_n * p.blocks_m * g.batch, ks_per_xcd = (ks_total + 7) / 8;
+    k << "    const int ks_block = (int)(blockIdx.x & 7u) * " << S(ks_per_xcd) << " + (int)(blockIdx.x >> 3);\n";
+    k << "    if (ks_block >= " << S(ks_total) << ") return;\n";
+    k << "    const int bn = ks_block % " << S(p.blocks_n) << ", bm = (ks_block / " << S(p.blocks_n) << ") % " << S(p.blocks_m) << ", cb = ks_block / " << S(p.blocks_n * p.blocks_m) << ";\n";
     k << "    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), li = lane & 15, lk = lane >> 4;\n";
     k << "    const int row = min(bm * 16 + li, " << S(g.m - 1) << ");\n";
     k << "    const int k_begin = wave * " << S(kw) << ", k_end = min(k_begin + " << S(kw) << ", " << S(g.k) << ");\n";
@@ -3145,7 +3151,7 @@ string gen_matmul_ksplit(Emitter& em, Generated* out) {
         k << "            b" << fk.outputs[0] << "[gid] = sum;\n";
     }
     k << "        }\n    }\n}\n";
-    const int64_t grid = p.blocks_m * p.blocks_n * g.batch;
+    const int64_t grid = ks_per_xcd * 8;
     if (grid >= kMaxIndex) return "matmul: grid too large";
     out->grid = (unsigned)grid;
     out->block = (unsigned)(64 * W);
