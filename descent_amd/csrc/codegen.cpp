@@ -1793,6 +1793,11 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     // arithmetic (divisions by the extents of every view on the way) is then shared by the four evaluations, whose
     // element ids differ in their two lowest bits only.
     const bool quad_dc = K % 4 == 0;
+    // dC read off the pooling windows' words (ConvDgrad::PoolMasks): a word and the window's four dP values per quad
+    const bool pmask = cv.pm.on;
+    if (pmask && (K % 4 != 0 || OHF % 2 != 0 || OW % 2 != 0 || fk.inputs[DC].buffer < 0 || cv.pm.masks.buffer < 0))
+        return "conv backward: pooling words need channel quads, even extents and buffers";
+    const string pm_leak = "U2F(0x" + [&] { char b[16]; std::snprintf(b, sizeof b, "%08x", cv.pm.leak_bits); return string(b); }() + "u)";
     const int64_t dunit = quad_dc ? 4 : 1;
     const int64_t fill_n = OH * OW * K / dunit, NC = (fill_n + 255) / 256;
     const bool vec_fill = C % 4 == 0;
@@ -1801,7 +1806,13 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     auto emit_issue = [&](const string& img, const string& ind) {
         k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NC) << "; ++u) {\n";
         k << ind << "    const int i = min(tid + u * 256, " << S(fill_n - 1) << ") * " << S(dunit) << ";\n";
-        if (vec_dc)
+        if (pmask) {
+            k << ind << "    const int pi = i / " << S(K) << ", oc = i % " << S(K) << ", wy = (band * " << S(OH) << " + pi / " << S(OW) << ") >> 1, wx = (pi % " << S(OW) << ") >> 1;\n";
+            k << ind << "    pw[u] = ((const uint*)b" << cv.pm.masks.buffer << ")[((cb * " << S(IMG) << " + " << img << ") * " << S((OHF / 2) * (OW / 2)) << " + wy * " << S(OW / 2)
+              << " + wx) * " << S(K / 4) << " + (oc >> 2)];\n";
+            k << ind << "    pv[u] = *(const float4*)(b" << fk.inputs[DC].buffer << " + ((" << img << " * " << S(OHF / 2) << " + wy) * " << S(OW / 2) << " + wx) * " << S(G * K)
+              << " + cb * " << S(K) << " + oc);\n" << ind << "}\n";
+        } else if (vec_dc)
             k << ind << "    pv[u] = *(const float4*)(b" << fk.inputs[DC].buffer << " + " << S(dc_base) << " + cb * " << S(G == 1 ? 0 : dc_coef[0]) << " + (" << img << " * "
               << S(OHF * OW) << " + band * " << S(OH * OW) << " + i / " << S(K) << ") * " << S(dc_coef[1]) << " + i % " << S(K) << ");\n" << ind << "}\n";
         else if (quad_dc && !la4.empty()) {
@@ -1824,6 +1835,14 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     auto emit_tile_stores = [&](const string& ind, const string& buf) {
         k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NC) << "; ++u) {\n";
         k << ind << "    const int i = (tid + u * 256) * " << S(dunit) << ", pi = i / " << S(K) << ";\n";
+        if (pmask) {
+            k << ind << "    {\n" << ind << "        const uint bits = pw[u] >> (2 * (((pi % " << S(OW) << ") & 1) | (((band * " << S(OH) << " + pi / " << S(OW) << ") & 1) << 1)));\n";
+            const char* comp[4] = {"x", "y", "z", "w"};
+            for (int j = 0; j < 4; ++j)
+                k << ind << "        { const float v = (bits & " << (1u << (8 * j)) << "u) ? pv[u]." << comp[j] << " : 0.f; pv[u]." << comp[j] << " = (bits & " << (2u << (8 * j))
+                  << "u) ? v : v * " << pm_leak << "; }\n";
+            k << ind << "    }\n";
+        }
         k << ind << "    float* const at = lds + " << buf << " + " << S(L.DC_AT) << " + ((pi / " << S(OW) << ") * " << S(PW) << " + pi % " << S(OW) << ") * " << S(PITCH) << " + i % " << S(K) << ";\n";
         if (quad_dc && PITCH % 4 == 0)
             k << ind << "    if (tid + u * 256 < " << S(fill_n) << ") *(float4*)at = pv[u];\n" << ind << "}\n";
@@ -1853,6 +1872,7 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         k << "    constexpr int bo = 0;\n";
         k << "    for (int img = chunk; img < " << S(IMG) << "; img += " << S(cv.chunks) << ") {\n";
         k << "        {\n            " << dvt << " pv[" << S(NC) << "];\n            " << vt << " xv[" << S(NX) << "];\n";
+        if (pmask) k << "            uint pw[" << S(NC) << "];\n";
         emit_issue("img", "            ");
         emit_tile_stores("            ", "0");
         k << "        }\n";
@@ -2055,11 +2075,13 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         // barriers of the matrix phases
         k << "    } else {\n";
         k << "    if (chunk < " << S(IMG) << ") {\n        " << dvt << " pv[" << S(NC) << "];\n        " << vt << " xv[" << S(NX) << "];\n";
+        if (pmask) k << "        uint pw[" << S(NC) << "];\n";
         emit_issue("chunk", "        ");
         emit_tile_stores("        ", "0");
         k << "    }\n    __syncthreads();\n" << loop_head;
         k << "        const int nimg = img + " << S(cv.chunks) << ";\n";
         k << "        if (nimg < " << S(IMG) << ") {\n            " << dvt << " pv[" << S(NC) << "];\n            " << vt << " xv[" << S(NX) << "];\n";
+        if (pmask) k << "            uint pw[" << S(NC) << "];\n";
         emit_issue("nimg", "            ");
         emit_tile_stores("            ", "(bo ^ " + S(BUFSZ) + ")");
         k << "        }\n";
@@ -2083,7 +2105,8 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     out->grid = (unsigned)(cv.chunks * G * BANDS);
     out->block = (unsigned)BLOCK;
     out->source = k.str();
-    out->note = "conv backward: workgroup per group and image set (" + S(cv.chunks) + " sets), dC and input tile in LDS, " + (spec ? "loader waves fill the next image's tiles, " : "") +
+    out->note = "conv backward: workgroup per group and image set (" + S(cv.chunks) + " sets), dC and input tile in LDS, " + (pmask ? "dC read off the pooling windows' words, " : "") +
+                (spec ? "loader waves fill the next image's tiles, " : "") +
                 (wonly ? "no data gradient, " + S(BANDS) + " bands of " + S(OH) + " output rows" : "data gradient " + S(FH) + "x" + S(FW) + " taps x " + S(K) + " channels" + (unpad ? " with border folds" : "")) +
                 ", filter gradient mfma 16x16x4 " + to_string(MT) + "x" + to_string(NT) + " tiles" + (cv.bias ? " +column sums of dC" : "");
     return "";
@@ -2266,6 +2289,7 @@ string gen_conv_fwd(Emitter& em, Generated* out) {
         }
         auto val = [&](int i, int o) { return fk.has_epilogue ? "res[" + to_string(i) + "][" + to_string(o) + "]" : "acc[j][" + to_string(i) + "]"; };
         for (int o = 0; o < n_out; ++o) {
+            if (pooled && fk.pool.masks && o == fk.pool.source) continue;  // its readers take the window words below
             const string ptr = "b" + to_string(fk.outputs[o]);
             if (vec_store) {
                 k << ind << "        " << (pooled ? "if (valid) " : "") << "*(float4*)(" << ptr << " + c_at) = make_float4(" << val(0, o) << ", " << val(1, o) << ", " << val(2, o) << ", "
@@ -2282,7 +2306,19 @@ string gen_conv_fwd(Emitter& em, Generated* out) {
                 k << ind << "        { float v = " << val(i, fk.pool.source) << "; v = glsl_max(v, __shfl_xor(v, 1, 64)); pm[" << i << "] = glsl_max(v, __shfl_xor(v, 8, 64)); }\n";
             }
             const int64_t pbs = rows ? g.n : (int64_t)cv.img * OH2 * OW2 * g.n, prs = rows ? g.batch * g.n : g.n;
+            if (fk.pool.masks) {
+                // two bits per element: equals its window's maximum, is positive; the four pixels of a window meet in
+                // one word per four channels (lanes l, l ^ 1, l ^ 8, l ^ 9)
+                k << ind << "        uint mw = 0u;\n";
+                for (int i = 0; i < 4; ++i)
+                    k << ind << "        { const float v = " << val(i, fk.pool.source) << "; mw |= ((v == pm[" << i << "] ? 1u : 0u) | (v > 0.f ? 2u : 0u)) << " << 8 * i << "; }\n";
+                k << ind << "        mw <<= 2 * ((li & 1) | ((li >> 3) << 1));\n";
+                k << ind << "        mw |= (uint)__shfl_xor((int)mw, 1, 64);\n" << ind << "        mw |= (uint)__shfl_xor((int)mw, 8, 64);\n";
+            }
             k << ind << "        if (valid && (li & 9) == 0) {\n";
+            if (fk.pool.masks)
+                k << ind << "            ((uint*)b" << fk.outputs[fk.pool.source] << ")[((cb * " << S(cv.img) << " + img) * " << S(OH2 * OW2) << " + (t / " << S(TPR) << ") * " << S(OW2)
+                  << " + (xr >> 1)) * " << S(g.n / 4) << " + lk] = mw;\n";
             k << ind << "            const int p_at = cb * " << S(pbs) << " + (img * " << S(OH2 * OW2) << " + (t / " << S(TPR) << ") * " << S(OW2) << " + (xr >> 1)) * " << S(prs) << " + cn;\n";
             if (fk.pool.has_epilogue) {
                 k << ind << "            float pres[4][" << n_pool_out << "];\n";
@@ -2327,7 +2363,7 @@ string gen_conv_fwd(Emitter& em, Generated* out) {
     out->source = k.str();
     out->note = "conv forward: workgroup per image and group, padded image tile in LDS, mfma 16x16x4, " + S(cv.fh) + "x" + S(cv.fw) + " taps x " + S(C) +
                 " channels" + (fk.has_epilogue ? " +epilogue" : "") +
-                (pooled ? string(" +2x2 max-pool") + (fk.pool.has_epilogue ? " with its consumer" : "") : string());
+                (pooled ? string(" +2x2 max-pool") + (fk.pool.has_epilogue ? " with its consumer" : "") + (fk.pool.masks ? ", window words in place of its source" : "") : string());
     return "";
 }
 
@@ -3520,10 +3556,20 @@ void count_work(const FusedKernel& fk, Generated* g) {
             elements -= out_each * (double)(fk.outputs.size() - 1);  // only the first output has the image's size
         }
     }
+    if (fk.dgrad.on && fk.dgrad.pm.on) {
+        // dC was counted through its view at the convolution's output size: what is read is the pooled gradient (a
+        // quarter of that) and one word per window and four channels
+        const FusedKernel::ConvDgrad& c = fk.dgrad;
+        const MatMulDims m = matmul_dims(d);
+        const double dc = (double)c.img * (double)c.oh * (double)c.ow * (double)c.g * (double)(c.wgrad_only ? m.n : m.k);
+        elements -= dc * (1.0 - 0.25 - 1.0 / 16.0);
+    }
     if (fk.pool.on) {
         // the pooled array and what its consumer writes have a quarter of the convolution's elements
         const double extra = (double)((fk.pool.has_epilogue ? fk.pool.epilogue.raw().n_outputs : 0) + (fk.pool.store_pooled ? 1 : 0));
         elements -= out_each * extra * 0.75;
+        // one word per window and four channels in place of the source array
+        if (fk.pool.masks) elements -= out_each * (1.0 - 1.0 / 16.0);
     }
     if (d.kind == DSC_KERNEL_SCATTER_ADD)  // read-modify-write of the entries that receive a value
         out_each = 2.0 * std::min((double)element_count(d.shape), (double)element_count(d.inputs[0].out_shape));
@@ -3652,6 +3698,11 @@ std::string FusedKernel::key() const {
         for (int64_t v : {dgrad.img, dgrad.oh, dgrad.ow, dgrad.g, dgrad.fh, dgrad.fw, dgrad.c, dgrad.pad_h, dgrad.pad_w, (int64_t)dgrad.rows_first,
                           (int64_t)dgrad.wgrad, (int64_t)dgrad.bias, dgrad.chunks})
             s.append(reinterpret_cast<const char*>(&v), 8);
+        if (dgrad.pm.on) {
+            s += "|PM";
+            put_src(dgrad.pm.masks);
+            s.append(reinterpret_cast<const char*>(&dgrad.pm.leak_bits), 4);
+        }
     }
     if (cfwd.on) {
         s += "|CF";
@@ -3662,6 +3713,7 @@ std::string FusedKernel::key() const {
         s += "|PL";
         s.append(reinterpret_cast<const char*>(&pool.source), 4);
         s += pool.store_pooled ? "S" : "-";
+        s += pool.masks ? "M" : "-";
         if (pool.has_epilogue) {
             s += "E" + pool.epilogue.key();
             s.append(reinterpret_cast<const char*>(&pool.epilogue_product_input), 4);

@@ -136,6 +136,15 @@ struct FusedKernel {
         // (filter gradient alone) bands of output rows an image is cut into, one workgroup each: a band's tiles are a
         // fraction of the image's, so more workgroups share a CU; partials then number chunks x bands
         int64_t bands = 1;
+        // dC is the gradient of a 2x2 max-pooling behind an activation with slope `leak` below zero, read off the words a
+        // pooling convolution-forward kernel wrote (ConvPool::masks): dC[pixel][oc] = (equals its window's maximum ?
+        // dP[window][oc] : 0) x (positive ? 1 : leak).  Then the dC operand of `main` is dP -- the pooled array's
+        // gradient [img, oh/2, ow/2, g*k], a buffer -- and `masks` the words' buffer.
+        struct PoolMasks {
+            bool on = false;
+            Source masks;
+            uint32_t leak_bits = 0;
+        } pm;
     } dgrad;
     // MatMul whose A operand is the im2col of a stride-1 convolution's (replicate-padded) input: the kernel reads the
     // image [img, h, w, g*c] itself, one workgroup per (image, group) with the group's channels of the image in LDS,
@@ -154,6 +163,13 @@ struct FusedKernel {
         int source = 0;                 // which of the convolution's outputs is pooled
         bool has_epilogue = false;      // the Reduce carried a per-element consumer
         bool store_pooled = true;       // the pooled array itself is written (no consumer, or a consumer that keeps it)
+        // The pooled output's source is read by nothing but the backward pass of this pooling and of the activation in
+        // front of it, which ask two things of each element: does it equal its window's maximum, and is it positive.
+        // The kernel then writes those two bits per element in place of the element -- one word per pooling window and
+        // four channels, [g][img * oh/2 * ow/2][n / 4], byte j of a word for channel 4q + j, bits 2p and 2p + 1 of a
+        // byte for the window's pixel p = (x & 1) + 2 (y & 1) -- through the pointer that stood for the source, which
+        // is never stored (see ConvDgrad::masks for the reader).
+        bool masks = false;
         KernelDesc epilogue;
         int epilogue_product_input = -1;
         std::vector<Source> epilogue_inputs;

@@ -79,6 +79,7 @@ void for_each_source(FusedKernel& fk, F f) {
     if (fk.pool.on && fk.pool.has_epilogue)
         for (size_t i = 0; i < fk.pool.epilogue_inputs.size(); ++i)
             if ((int)i != fk.pool.epilogue_product_input) f(fk.pool.epilogue_inputs[i]);
+    if (fk.dgrad.on && fk.dgrad.pm.on) f(fk.dgrad.pm.masks);
     if (fk.row_tail.on) {
         f(fk.row_tail.b);
         if (fk.row_tail.has_epilogue)
@@ -2475,6 +2476,159 @@ struct Planner {
         }
     }
 
+    // Pass 3g: the gradient of a 2x2 max-pooling read off two bits per element.  The backward pass of "convolution,
+    // activation, 2x2 max-pool" reads the activation A twice -- (A == its window's maximum P) ? dP : 0, then
+    // (A > 0) ? that : that x c -- and nothing else does once the pooling itself runs inside the convolution kernel
+    // (pass 3c).  That kernel has A and P in registers: it writes the two comparisons' outcomes, one word per window
+    // and four channels, and A is never stored; the convolution backward kernel that evaluated the four producers of
+    // this chain where it fills dC (pass 2) reads a word and the window's dP instead (ConvPool::masks,
+    // ConvDgrad::PoolMasks).  Bit for bit the same gradient: the comparisons are made on the same values.
+    // The chain is matched op by op, and its index arithmetic is checked element by element on three images.
+    void pooling_gradients_read_window_words() {
+        const char* sw = std::getenv("DSC_POOL_WORDS");
+        if ((sw && sw[0] == '0') || (flags & DSC_SCHEDULE_NO_CONV_KERNELS)) return;
+        auto strip = [](const dsc_kernel_desc& pe, int op) {
+            while (pe.ops[op].kind == DSC_PE_UNARY && pe.ops[op].op == DSC_UN_MOV) op = pe.ops[op].args[0];
+            return op;
+        };
+        auto is_zero = [&](const dsc_kernel_desc& pe, int op) {
+            op = strip(pe, op);
+            return pe.ops[op].kind == DSC_PE_LITERAL_F32 && pe.ops[op].bits == 0u;
+        };
+        // element id of a per-element cluster -> the element its input `in` reads there
+        auto through = [](const dsc_kernel_desc& pe, int in, int64_t gid) {
+            const dsc_view& v = pe.inputs[in];
+            int64_t c[DSC_MAX_DIM];
+            for (int a = v.out_shape.rank - 1; a >= 0; --a) {
+                c[a] = gid % v.out_shape.dims[a];
+                gid /= v.out_shape.dims[a];
+            }
+            return view_index_clamped(v, c);
+        };
+        for (int fi = 0; fi < (int)drafts.size(); ++fi) {
+            Draft& F = drafts[fi];
+            if (!F.alive || !F.fk.cfwd.on || !F.fk.pool.on || F.fk.pool.masks || !F.fk.pool.store_pooled || !F.fk.parts.empty()) continue;
+            const FusedKernel::ConvFwd& cv = F.fk.cfwd;
+            const dsc_kernel_desc& fd = F.fk.main.raw();
+            const MatMulDims g = matmul_dims(fd);
+            const bool rows = fd.output_mode == DSC_MATMUL_ROWS;
+            const int64_t batch_stride = rows ? g.n : g.m * g.n, row_stride = rows ? g.batch * g.n : g.n;
+            const int64_t OH2 = cv.oh / 2, OW2 = cv.ow / 2, K = g.n, G = g.batch;
+            const int64_t pbs = rows ? g.n : cv.img * OH2 * OW2 * g.n, prs = rows ? g.batch * g.n : g.n;
+            const int n_out = F.fk.has_epilogue ? F.fk.epilogue.raw().n_outputs : 1;
+            const int n_epi = F.fk.pool.has_epilogue ? F.fk.pool.epilogue.raw().n_outputs : 0;
+            if (K % 4 != 0 || (int)F.outs.size() != n_out + n_epi + 1) continue;
+            const int a_node = F.outs[F.fk.pool.source].node, p_node = F.outs[n_out + n_epi].node;
+            if (is_graph_output[a_node] || F.outs[F.fk.pool.source].copy_from >= 0) continue;
+            const auto cons = consumers_of(a_node);
+            if (cons.size() != 1 || cons[0] <= fi) continue;
+            const int qi = cons[0];
+            Draft& Q = drafts[qi];
+            const FusedKernel::ConvDgrad& dg = Q.fk.dgrad;
+            if (!dg.on || !dg.wgrad || dg.pm.on || !Q.fk.parts.empty() || Q.fk.has_epilogue) continue;
+            const int DC = dg.wgrad_only ? 1 : 0;
+            const dsc_kernel_desc& qd = Q.fk.main.raw();
+            const MatMulDims gq = matmul_dims(qd);
+            if (dg.img != cv.img || dg.oh != cv.oh || dg.ow != cv.ow || dg.g != G || (dg.wgrad_only ? gq.n : gq.k) != K) continue;
+            if (Q.fk.inputs[DC].virt < 0 || Q.fk.virtuals.size() != 4) continue;
+            // every other operand of the kernel is a buffer that is not A
+            bool clean = true;
+            for (size_t in = 0; in < Q.fk.inputs.size(); ++in)
+                if ((int)in != DC && (Q.fk.inputs[in].buffer < 0 || Q.params[Q.fk.inputs[in].buffer] == a_node)) clean = false;
+            if (!clean) continue;
+            // V0 = (A > 0) ? X : X x c
+            const int v0 = Q.fk.inputs[DC].virt;
+            const Virtual& V0 = Q.fk.virtuals[v0];
+            const dsc_kernel_desc& d0 = V0.pe.raw();
+            if (d0.kind != DSC_KERNEL_PER_ELEMENT || d0.n_inputs != 2) continue;
+            const dsc_pe_op& sel0 = d0.ops[strip(d0, V0.out_op)];
+            if (sel0.kind != DSC_PE_SELECT || sel0.op != DSC_CMP_GT || !is_zero(d0, sel0.args[1])) continue;
+            const int a_op = strip(d0, sel0.args[0]), x_op = strip(d0, sel0.args[2]), y_op = strip(d0, sel0.args[3]);
+            if (d0.ops[a_op].kind != DSC_PE_LOAD || d0.ops[x_op].kind != DSC_PE_LOAD || d0.ops[y_op].kind != DSC_PE_BINARY || d0.ops[y_op].op != DSC_BIN_MUL) continue;
+            const int a_in0 = d0.ops[a_op].input_index, x_in0 = d0.ops[x_op].input_index;
+            if (a_in0 == x_in0 || V0.inputs[a_in0].buffer < 0 || Q.params[V0.inputs[a_in0].buffer] != a_node || V0.inputs[x_in0].virt < 0) continue;
+            uint32_t leak_bits = 0;
+            {
+                const int m0 = strip(d0, d0.ops[y_op].args[0]), m1 = strip(d0, d0.ops[y_op].args[1]);
+                const bool x_first = d0.ops[m0].kind == DSC_PE_LOAD && d0.ops[m0].input_index == x_in0 && d0.ops[m1].kind == DSC_PE_LITERAL_F32;
+                const bool x_second = d0.ops[m1].kind == DSC_PE_LOAD && d0.ops[m1].input_index == x_in0 && d0.ops[m0].kind == DSC_PE_LITERAL_F32;
+                if (!x_first && !x_second) continue;
+                leak_bits = d0.ops[x_first ? m1 : m0].bits;
+            }
+            // V1 = copy of V2
+            const Virtual& V1 = Q.fk.virtuals[V0.inputs[x_in0].virt];
+            const dsc_kernel_desc& d1 = V1.pe.raw();
+            if (d1.kind != DSC_KERNEL_PER_ELEMENT || d1.n_inputs != 1 || !is_pure_copy(d1) || V1.inputs[0].virt < 0) continue;
+            // V2 = (V3 == P) ? dP : 0
+            const Virtual& V2 = Q.fk.virtuals[V1.inputs[0].virt];
+            const dsc_kernel_desc& d2 = V2.pe.raw();
+            if (d2.kind != DSC_KERNEL_PER_ELEMENT || d2.n_inputs != 3) continue;
+            const dsc_pe_op& sel2 = d2.ops[strip(d2, V2.out_op)];
+            if (sel2.kind != DSC_PE_SELECT || sel2.op != DSC_CMP_EQ || !is_zero(d2, sel2.args[3])) continue;
+            const int w_op = strip(d2, sel2.args[0]), p_op = strip(d2, sel2.args[1]), dp_op = strip(d2, sel2.args[2]);
+            if (d2.ops[w_op].kind != DSC_PE_LOAD || d2.ops[p_op].kind != DSC_PE_LOAD || d2.ops[dp_op].kind != DSC_PE_LOAD) continue;
+            const int w_in = d2.ops[w_op].input_index, p_in = d2.ops[p_op].input_index, dp_in = d2.ops[dp_op].input_index;
+            if (w_in == p_in || w_in == dp_in || p_in == dp_in) continue;
+            if (V2.inputs[w_in].virt < 0 || V2.inputs[p_in].buffer < 0 || V2.inputs[dp_in].buffer < 0 || Q.params[V2.inputs[p_in].buffer] != p_node) continue;
+            const int dp_node = Q.params[V2.inputs[dp_in].buffer];
+            if (dp_node == a_node || dp_node == p_node) continue;
+            // V3 = copy of A
+            const Virtual& V3 = Q.fk.virtuals[V2.inputs[w_in].virt];
+            const dsc_kernel_desc& d3 = V3.pe.raw();
+            if (d3.kind != DSC_KERNEL_PER_ELEMENT || d3.n_inputs != 1 || !is_pure_copy(d3) || V3.inputs[0].buffer < 0 || Q.params[V3.inputs[0].buffer] != a_node) continue;
+            if ((int64_t)node_bytes[dp_node] != cv.img * OH2 * OW2 * G * K * 4) continue;
+            // the indices, element by element: A at the pixel itself (both reads), P and dP at the pixel's window
+            const dsc_view& dcv = qd.inputs[DC];
+            bool ok = dcv.out_shape.rank == 3;
+            for (int64_t img : {(int64_t)0, cv.img / 2, cv.img - 1})
+                for (int64_t y = 0; y < cv.oh && ok; ++y)
+                    for (int64_t x = 0; x < cv.ow && ok; ++x)
+                        for (int64_t cb = 0; cb < G && ok; ++cb)
+                            for (int64_t oc = 0; oc < K && ok; ++oc) {
+                                const int64_t pix = (img * cv.oh + y) * cv.ow + x;
+                                const int64_t c3[3] = {cb, dg.wgrad_only ? pix : pix, oc};
+                                const int64_t gid0 = view_index_clamped(dcv, c3);
+                                const int64_t a_at = cb * batch_stride + pix * row_stride + oc;
+                                const int64_t win = (img * OH2 + y / 2) * OW2 + x / 2;
+                                if (through(d0, a_in0, gid0) != a_at) ok = false;
+                                const int64_t gid1 = through(d0, x_in0, gid0), gid2 = through(d1, 0, gid1);
+                                const int64_t gid3 = through(d2, w_in, gid2);
+                                if (through(d3, 0, gid3) != a_at) ok = false;
+                                if (through(d2, p_in, gid2) != cb * pbs + win * prs + oc) ok = false;
+                                if (through(d2, dp_in, gid2) != win * (G * K) + cb * K + oc) ok = false;
+                            }
+            if (!ok) continue;
+            // rewire: the forward kernel writes the words through the pointer that stood for A, the backward kernel reads
+            // them and dP
+            node_bytes.push_back((size_t)(G * cv.img * OH2 * OW2 * (K / 4)) * 4);
+            is_graph_output.push_back(false);
+            is_graph_input.push_back(false);
+            const int words = n_nodes++;
+            Draft f2 = F, q2 = Q;
+            f2.fk.pool.masks = true;
+            f2.params[f2.fk.outputs[f2.fk.pool.source]] = words;
+            f2.outs[f2.fk.pool.source].node = words;
+            q2.fk.virtuals.clear();
+            q2.fk.inputs[DC] = Source{};
+            q2.fk.inputs[DC].buffer = param_index(q2, dp_node, false);
+            q2.fk.dgrad.pm.on = true;
+            q2.fk.dgrad.pm.masks = Source{};
+            q2.fk.dgrad.pm.masks.buffer = param_index(q2, words, false);
+            q2.fk.dgrad.pm.leak_bits = leak_bits;
+            compact(q2);
+            Generated probe_f, probe_q;
+            if (!generate(f2.fk, &probe_f).empty() || !generate(q2.fk, &probe_q).empty()) {
+                node_bytes.pop_back();
+                is_graph_output.pop_back();
+                is_graph_input.pop_back();
+                --n_nodes;
+                continue;
+            }
+            drafts[fi] = f2;
+            drafts[qi] = q2;
+        }
+    }
+
     // Pass 3b: ScatterAdds chained through one accumulator (each takes the previous one's result in place:
     // the four corner updates of one hash-grid level) commute, so the chain runs as one multi-part launch
     // whose parts all add into the same buffer.  It runs where the last one ran.
@@ -2851,6 +3005,7 @@ struct Planner {
         attach_epilogues();                     // pass 3
         slice_major_products();                 // pass 3d
         pool_joins_conv_forward();              // pass 3c
+        pooling_gradients_read_window_words();  // pass 3g
         chain_scatter_adds();                   // pass 3b
         group_chain_launches();                 // pass 3e
         pair_output_layer_gradients();          // pass 3f

@@ -883,6 +883,32 @@ def test_convnet_backward_with_and_without_loader_waves(hip_backend_session, mon
             assert rel_l2(got[key], want[key]) <= TOL, (key, rel_l2(got[key], want[key]), listing)
 
 
+@pytest.mark.parametrize("batch,side,loaders", [(1000, 28, "1"), (1000, 28, "0"), (1536, 20, "1")])
+def test_pooling_gradients_read_off_window_words_are_bit_equal(hip_backend_session, monkeypatch, batch, side, loaders):
+    """Two Adam steps of the ConvNet with the pooling gradients evaluated from the stored activations (DSC_POOL_WORDS=0)
+    and read off the two bits per element the forward kernels write in their place: the comparisons are made on the
+    same values, so every parameter, optimiser state and loss comes out bit for bit the same."""
+    from descent_amd import Environment, workloads
+
+    monkeypatch.setenv("DSC_CONV_BWD_LOADERS", loaders)
+    results, listings = [], []
+    for words in ("0", "1"):
+        monkeypatch.setenv("DSC_POOL_WORDS", words)
+        env = Environment(hip_backend_session)
+        w = workloads.convnet(env, batch=batch, seed=17, side=side)
+        for step in range(2):
+            env.run(w.graph, 3 + step)
+        results.append(w.snapshot())
+        listings.append(next(iter(w.graph.__dict__["_schedules"].values())).describe())
+    assert "pooling windows' words" not in listings[0] and "window words in place of its source" not in listings[0], listings[0]
+    # the first convolution's filter gradient always reads the words; the second one's backward kernel where it took the
+    # pooling gradient as a producer of its fills (loader waves)
+    assert listings[1].count("dC read off the pooling windows' words") == (2 if loaders == "1" else 1), listings[1]
+    assert listings[1].count("window words in place of its source") == (2 if loaders == "1" else 1), listings[1]
+    for key in results[0]:
+        assert np.array_equal(results[0][key], results[1][key]), (key, listings[1])
+
+
 def _conv_grad_case(env, m, h, w, c_in, c_out, fh, fw, pad, groups, seed):
     """x -> conv2d -> 0.5 * sum(y^2): the gradients with respect to the image and the filter."""
     from descent_amd import Initializer

@@ -91,9 +91,16 @@ def test_bias_gradient_rides_on_the_weight_gradient_that_reads_the_same_array():
     assert re.search(r"Reduce \(k=\d+\) \[1, 1, 1, 16\]; Reduce \(k=\d+\) \[1, 1, 9, 16\]", listing)
 
 
+def _convnet_plan(fused="True", **env):
+    """The ConvNet's schedule listing from a process of its own (the planner reads its switches once per process)."""
+    code = "import sys; sys.path.insert(0, %r); from descent_amd import Environment, hip_backend, workloads; from oracle.cpu_backend import CpuBackend; " \
+           "print(hip_backend.check_schedule(workloads.convnet(Environment(CpuBackend()), batch=1000).graph, fused=%s))"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    return subprocess.run([sys.executable, "-c", code % (root, fused)], env=dict(os.environ, **env), check=True, capture_output=True, text=True).stdout
+
+
 def test_first_layer_filter_gradient_takes_the_pooling_gradient_as_a_producer():
-    graph = workloads.convnet(_env(), batch=1000).graph
-    listing = hip_backend.check_schedule(graph, fused=True)
+    listing = _convnet_plan(DSC_POOL_WORDS="0")
     assert int(listing.split()[0]) == 8
     # conv2's backward kernel runs with loader waves and takes its dC the same way: the pooling gradient behind it is
     # a producer of that kernel's fills and no launch of its own
@@ -109,9 +116,26 @@ def test_first_layer_filter_gradient_takes_the_pooling_gradient_as_a_producer():
         assert str(cluster) in line.split(" clusters ")[1].split(), (cluster, line)
     assert "WindowsToImage" not in listing
     assert re.search(r"Reduce \(k=1024\) \[1, 1, 1, 16\]; Reduce \(k=1024\) \[1, 1, 9, 16\]", listing)
+    assert "338.4" in listing.strip().splitlines()[-1], listing.strip().splitlines()[-1]
     # with the switch the second convolution keeps its own two kernels and the first its tall-k product
-    split = hip_backend.check_schedule(graph, fused="split-conv-grads")
+    split = _convnet_plan(fused="'split-conv-grads'")
     assert "ConvFilterGrad" not in split and "ConvBackward" not in split
+
+
+def test_pooling_gradients_are_read_off_the_window_words_the_forward_kernels_write():
+    """Both convolutions' activations are read by nothing but their pooling's and their activation's backward: the
+    forward kernels write two bits per element (equals the window's maximum, is positive) in place of the activation,
+    the backward kernels read those words and the pooled gradient instead of evaluating four producers."""
+    listing = _convnet_plan()
+    assert int(listing.split()[0]) == 8
+    forward = [l for l in listing.splitlines() if "conv forward:" in l]
+    assert len(forward) == 2 and all("window words in place of its source" in l for l in forward), forward
+    line = next(l for l in listing.splitlines() if ": ConvBackward" in l)
+    assert "dC read off the pooling windows' words" in line and "fused producers" not in line and "loader waves" in line, line
+    line = next(l for l in listing.splitlines() if "ConvFilterGrad" in l)
+    assert "dC read off the pooling windows' words, no data gradient, 4 bands of 7 output rows" in line, line
+    # 75 MB of activations are neither written nor read back; 4.7 MB of words are
+    assert "178.49" in listing.strip().splitlines()[-1], listing.strip().splitlines()[-1]
 
 
 def test_a_small_product_over_a_moderate_k_is_one_launch_with_k_split_inside_the_workgroups():
@@ -270,9 +294,11 @@ def test_the_sign_of_a_pre_activation_is_read_off_the_stored_activation():
     # z again for "(z > 0) ? g : 0.01 g".  a has the sign of z, so the readers test a > 0 and z is never written:
     # conv1's kernel writes a (50.2 MB) and the pooled a (12.5 MB) for its 3.1 MB image, conv2's a (25.1), the pooled
     # and dropped-out a (2 x 6.3) for 12.5 MB in
-    assert "ConvForward" in lines[0] and 65.0 < moved(lines[0]) < 66.5, lines[0]     # 116.0 with z stored
-    assert lines[1].split(": ")[1].startswith("ConvForward") and 49.5 < moved(lines[1]) < 51.0, lines[1]  # 75.3 with z stored
-    assert "338.4" in fused.splitlines()[-1], fused.splitlines()[-1]  # MB per step; 565 with z stored, 414 before conv2's dC became a producer, 358 with fc1's k chunks in memory
+    # (and a itself gives way to two bits per element once the pooling gradients read those: 15.7 MB out for conv1,
+    # 14.1 MB for conv2)
+    assert "ConvForward" in lines[0] and 18.0 < moved(lines[0]) < 19.5, lines[0]     # 116.0 with z stored, 65.9 with a stored
+    assert lines[1].split(": ")[1].startswith("ConvForward") and 26.0 < moved(lines[1]) < 27.5, lines[1]  # 75.3 with z stored, 50.2 with a stored
+    assert "178.49" in fused.splitlines()[-1], fused.splitlines()[-1]  # MB per step; 565 with z stored, 414 before conv2's dC became a producer, 358 with fc1's k chunks in memory, 338.4 with the activations stored for the pooling gradients
     # cluster by cluster nothing is rewritten
     unfused = hip_backend.check_schedule(graph, fused=False)
     assert "PerElement (7 ops) [12544000]" in unfused and "2316." in unfused.splitlines()[-1], unfused.splitlines()[-1]

@@ -81,7 +81,7 @@ def test_static_run_refuses_what_does_not_fit_and_what_it_cannot_place(hip_backe
 
     be = hip_backend_session
     env = Environment(be)
-    w = workloads.convnet(env, batch=1000, seed=3)  # conv1's activations alone exceed the 64 MiB array
+    w = workloads.convnet(env, batch=8000, seed=3)  # conv1's pooled activations alone exceed the 64 MiB array
     before = {id(p): p.buffer for p in w.trainable + w.state}
     with pytest.raises(DescentHipError) as err:
         env.run_static(w.graph, 1)
