@@ -2303,7 +2303,7 @@ string gen_conv_fwd(Emitter& em, Generated* out) {
             // the window's maximum: across the column pair, then across the row pair
             k << ind << "        float pm[4];\n";
             for (int i = 0; i < 4; ++i) {
-                k << ind << "        { float v = " << val(i, fk.pool.source) << "; v = glsl_max(v, __shfl_xor(v, 1, 64)); pm[" << i << "] = glsl_max(v, __shfl_xor(v, 8, 64)); }\n";
+                k << ind << "        { float v = " << val(i, fk.pool.source) << "; v = glsl_max(v, dsc_lane_xor1(v)); pm[" << i << "] = glsl_max(v, dsc_lane_xor8(v)); }\n";
             }
             const int64_t pbs = rows ? g.n : (int64_t)cv.img * OH2 * OW2 * g.n, prs = rows ? g.batch * g.n : g.n;
             if (fk.pool.masks) {
@@ -2313,20 +2313,24 @@ string gen_conv_fwd(Emitter& em, Generated* out) {
                 for (int i = 0; i < 4; ++i)
                     k << ind << "        { const float v = " << val(i, fk.pool.source) << "; mw |= ((v == pm[" << i << "] ? 1u : 0u) | (v > 0.f ? 2u : 0u)) << " << 8 * i << "; }\n";
                 k << ind << "        mw <<= 2 * ((li & 1) | ((li >> 3) << 1));\n";
-                k << ind << "        mw |= (uint)__shfl_xor((int)mw, 1, 64);\n" << ind << "        mw |= (uint)__shfl_xor((int)mw, 8, 64);\n";
+                k << ind << "        mw |= (uint)dsc_lane_xor1((int)mw);\n" << ind << "        mw |= (uint)dsc_lane_xor8((int)mw);\n";
+            }
+            k << ind << "        const int p_at = cb * " << S(pbs) << " + (img * " << S(OH2 * OW2) << " + (t / " << S(TPR) << ") * " << S(OW2) << " + (xr >> 1)) * " << S(prs) << " + cn;\n";
+            if (fk.pool.has_epilogue) {
+                // the window's four lanes all hold its four maxima: each runs the consumer for one of the four channels
+                // (all four in one lane, the other three idle, cost this issue-bound kernel four times the instructions)
+                k << ind << "        if (valid) {\n";
+                k << ind << "            const int wq = (li & 1) | ((li >> 3) << 1);\n";
+                k << ind << "            const float pmq = wq == 0 ? pm[0] : wq == 1 ? pm[1] : wq == 2 ? pm[2] : pm[3];\n";
+                k << ind << "            float pres[" << n_pool_out << "];\n";
+                k << ind << "            pool_epilogue(pmq, p_at + wq, pres, " << em.params_pass() << ");\n";
+                for (int o = 0; o < n_pool_out; ++o) k << ind << "            b" << fk.outputs[n_out + o] << "[p_at + wq] = pres[" << o << "];\n";
+                k << ind << "        }\n";
             }
             k << ind << "        if (valid && (li & 9) == 0) {\n";
             if (fk.pool.masks)
                 k << ind << "            ((uint*)b" << fk.outputs[fk.pool.source] << ")[((cb * " << S(cv.img) << " + img) * " << S(OH2 * OW2) << " + (t / " << S(TPR) << ") * " << S(OW2)
                   << " + (xr >> 1)) * " << S(g.n / 4) << " + lk] = mw;\n";
-            k << ind << "            const int p_at = cb * " << S(pbs) << " + (img * " << S(OH2 * OW2) << " + (t / " << S(TPR) << ") * " << S(OW2) << " + (xr >> 1)) * " << S(prs) << " + cn;\n";
-            if (fk.pool.has_epilogue) {
-                k << ind << "            float pres[4][" << n_pool_out << "];\n";
-                k << "#pragma unroll\n" << ind << "            for (int i = 0; i < 4; ++i) pool_epilogue(pm[i], p_at + i, pres[i], " << em.params_pass() << ");\n";
-                for (int o = 0; o < n_pool_out; ++o)
-                    k << ind << "            *(float4*)(b" << fk.outputs[n_out + o] << " + p_at) = make_float4(pres[0][" << o << "], pres[1][" << o << "], pres[2][" << o
-                      << "], pres[3][" << o << "]);\n";
-            }
             if (fk.pool.store_pooled)
                 k << ind << "            *(float4*)(b" << fk.outputs[n_out + n_pool_out] << " + p_at) = make_float4(pm[0], pm[1], pm[2], pm[3]);\n";
             k << ind << "        }\n";
