@@ -2301,10 +2301,14 @@ string gen_conv_fwd(Emitter& em, Generated* out) {
         }
         if (pooled) {
             // the window's maximum: across the column pair, then across the row pair
-            k << ind << "        float pm[4];\n";
-            for (int i = 0; i < 4; ++i) {
-                k << ind << "        { float v = " << val(i, fk.pool.source) << "; v = glsl_max(v, dsc_lane_xor1(v)); pm[" << i << "] = glsl_max(v, dsc_lane_xor8(v)); }\n";
-            }
+            // (the four channels side by side, step by step: a lane exchange may not follow the instruction that wrote
+            // its operand, and written channel by channel every exchange waited out that distance)
+            k << ind << "        float pm[4], px[4];\n";
+            for (int i = 0; i < 4; ++i) k << ind << "        pm[" << i << "] = " << val(i, fk.pool.source) << ";\n";
+            k << "#pragma unroll\n" << ind << "        for (int i = 0; i < 4; ++i) px[i] = dsc_lane_xor1(pm[i]);\n";
+            k << "#pragma unroll\n" << ind << "        for (int i = 0; i < 4; ++i) pm[i] = glsl_max(pm[i], px[i]);\n";
+            k << "#pragma unroll\n" << ind << "        for (int i = 0; i < 4; ++i) px[i] = dsc_lane_xor8(pm[i]);\n";
+            k << "#pragma unroll\n" << ind << "        for (int i = 0; i < 4; ++i) pm[i] = glsl_max(pm[i], px[i]);\n";
             const int64_t pbs = rows ? g.n : (int64_t)cv.img * OH2 * OW2 * g.n, prs = rows ? g.batch * g.n : g.n;
             if (fk.pool.masks) {
                 // two bits per element: equals its window's maximum, is positive; the four pixels of a window meet in
