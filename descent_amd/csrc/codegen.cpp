@@ -45,6 +45,24 @@ bool is_identifier(const string& s) {
     return true;
 }
 
+// A leaky ReLU as the reference writes it, select(x > 0, x, x * c) with a literal 0 < c < 1: the larger of x and x * c
+// (for x > 0 that is x, for x < 0 it is x * c, and where the two are equal -- zeros, infinities -- either is the
+// value; a NaN x gives NaN both ways).  One v_max_f32 where the select is a compare, a wait for its mask and a
+// conditional move.
+bool leaky_relu_select(const dsc_kernel_desc& pe, const dsc_pe_op& op) {
+    if (op.kind != DSC_PE_SELECT || op.op != DSC_CMP_GT || op.args[2] != op.args[0]) return false;
+    const dsc_pe_op& zero = pe.ops[op.args[1]];
+    const dsc_pe_op& scaled = pe.ops[op.args[3]];
+    if (zero.kind != DSC_PE_LITERAL_F32 || zero.bits != 0u || scaled.kind != DSC_PE_BINARY || scaled.op != DSC_BIN_MUL) return false;
+    int lit = -1;
+    if (scaled.args[0] == op.args[0]) lit = scaled.args[1];
+    else if (scaled.args[1] == op.args[0]) lit = scaled.args[0];
+    if (lit < 0 || pe.ops[lit].kind != DSC_PE_LITERAL_F32) return false;
+    float c;
+    std::memcpy(&c, &pe.ops[lit].bits, 4);
+    return c > 0.f && c < 1.f;
+}
+
 struct Emitter {
     const FusedKernel& fk;
     std::ostringstream funcs;  // device functions, emitted before the kernel
@@ -471,6 +489,10 @@ struct Emitter {
                 break;
             }
             case DSC_PE_SELECT:
+                if (leaky_relu_select(pe, op)) {
+                    each(i, [&](int e) { return "fmaxf(" + E(op.args[0], e) + ", " + E(op.args[3], e) + ")"; });
+                    break;
+                }
                 each(i, [&](int e) {
                     return "(" + E(op.args[0], e) + (op.op == DSC_CMP_EQ ? " == " : " > ") + E(op.args[1], e) + ") ? " + E(op.args[2], e) + " : " + E(op.args[3], e);
                 });
@@ -559,6 +581,10 @@ struct Emitter {
                 break;
             }
             case DSC_PE_SELECT:
+                if (leaky_relu_select(pe, op)) {
+                    rhs = "fmaxf(" + T(op.args[0]) + ", " + T(op.args[3]) + ")";
+                    break;
+                }
                 rhs = "(" + T(op.args[0]) + (op.op == DSC_CMP_EQ ? " == " : " > ") + T(op.args[1]) + ") ? " +
                       T(op.args[2]) + " : " + T(op.args[3]);
                 break;
