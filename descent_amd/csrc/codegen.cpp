@@ -3432,10 +3432,16 @@ string gen_matmul(Emitter& em, Generated* out) {
         for (int o = 0; o < pe.n_outputs; ++o)
             four << "    *(float4*)(b" << fk.outputs[o] << " + gid) = make_float4(res[0][" << o << "], res[1][" << o << "], res[2][" << o
                  << "], res[3][" << o << "]);\n";
+        const string sign_store = fk.sign_out < 0 ? string() :
+            "    ((unsigned char*)b" + to_string(fk.sign_out) + ")[gid >> 2] = (unsigned char)((res[0][" + to_string(fk.sign_source) + "] > 0.f ? 1 : 0) | (res[1][" +
+            to_string(fk.sign_source) + "] > 0.f ? 2 : 0) | (res[2][" + to_string(fk.sign_source) + "] > 0.f ? 4 : 0) | (res[3][" + to_string(fk.sign_source) + "] > 0.f ? 8 : 0));\n";
+        four << sign_store;
         four << "}\n";
         em.funcs << one.str() << four.str();
         k << "#define MM_STORE(v, idx, b, m, n) mm_store(v, idx, b, m, n, " << em.params_pass() << ")\n";
         k << "#define MM_STORE4(v, idx, b, m, n) mm_store4(v, idx, b, m, n, " << em.params_pass() << ")\n";
+        if ((fk.sign_out >= 0 || fk.epilogue_sign_input >= 0) && !(direct && vec_store && !long_epilogue && g.n % 4 == 0))
+            return "matmul: sign bytes need the 16-byte store path over whole tiles";
         // Operands of the epilogue that the 16-byte store path can request ahead of the staging rounds (each round's
         // own load would wait on vmcnt(0), i.e. also for the previous round's store to be acknowledged): a
         // per-column operand (a bias: the view reads element base + column) once per block column, a per-element
@@ -3456,6 +3462,7 @@ string gen_matmul(Emitter& em, Generated* out) {
                     if (pre_elem.size() < 2) pre_elem.push_back(i);
                     continue;
                 }
+                if (i == fk.epilogue_sign_input) return "matmul: the sign bytes stand for an operand read element for element";
                 const int last = v.out_shape.rank - 1;
                 if (last < 0 || !affine_form(v, &base, coef) || v.out_shape.dims[last] != g.n || coef[last] != 1 || base % 4 != 0) continue;
                 bool column_only = element_count(v.out_shape) == g.batch * g.m * g.n;
@@ -3487,7 +3494,13 @@ string gen_matmul(Emitter& em, Generated* out) {
             fn << "DSC_INLINE void mm_store4_pre(float4 p, int gid, int cb, int cm, int cn, const float4* colv, const float4* elv, " << em.params_decl() << ") {\n";
             fn << "    const float pv[4] = {p.x, p.y, p.z, p.w};\n    float res[4][" << pe.n_outputs << "];\n";
             for (size_t q = 0; q < pre_col.size(); ++q) fn << "    const float c" << q << "[4] = {colv[" << q << "].x, colv[" << q << "].y, colv[" << q << "].z, colv[" << q << "].w};\n";
-            for (size_t q = 0; q < pre_elem.size(); ++q) fn << "    const float e" << q << "[4] = {elv[" << q << "].x, elv[" << q << "].y, elv[" << q << "].z, elv[" << q << "].w};\n";
+            for (size_t q = 0; q < pre_elem.size(); ++q) {
+                if (pre_elem[q] == fk.epilogue_sign_input)  // a byte of four sign bits: the selects see +1 or -1
+                    fn << "    const uint sb" << q << " = F2U(elv[" << q << "].x);\n    const float e" << q << "[4] = {(sb" << q << " & 1u) ? 1.f : -1.f, (sb" << q << " & 2u) ? 1.f : -1.f, (sb" << q
+                       << " & 4u) ? 1.f : -1.f, (sb" << q << " & 8u) ? 1.f : -1.f};\n";
+                else
+                    fn << "    const float e" << q << "[4] = {elv[" << q << "].x, elv[" << q << "].y, elv[" << q << "].z, elv[" << q << "].w};\n";
+            }
             fn << "#pragma unroll\n    for (int j = 0; j < 4; ++j) mm_epilogue_pre(pv[j], gid + j, cb, cm, cn + j, res[j], ";
             for (size_t q = 0; q < pre_col.size(); ++q) fn << "c" << q << "[j], ";
             for (size_t q = 0; q < pre_elem.size(); ++q) fn << "e" << q << "[j], ";
@@ -3495,6 +3508,7 @@ string gen_matmul(Emitter& em, Generated* out) {
             for (int o = 0; o < pe.n_outputs; ++o)
                 fn << "    *(float4*)(b" << fk.outputs[o] << " + gid) = make_float4(res[0][" << o << "], res[1][" << o << "], res[2][" << o
                    << "], res[3][" << o << "]);\n";
+            fn << sign_store;
             fn << "}\n";
             em.funcs << fn.str();
             k << "#define MM_NPRE_COL " << pre_col.size() << "\n#define MM_NPRE_ELEM " << pre_elem.size() << "\n";
@@ -3502,15 +3516,26 @@ string gen_matmul(Emitter& em, Generated* out) {
             for (size_t q = 0; q < pre_col.size(); ++q)
                 k << " (dst)[" << q << "] = *(const float4*)(b" << fk.epilogue_inputs[pre_col[q]].buffer << " + " << S(pre_col_base[q]) << " + (cn));";
             k << " }\n#define MM_LOAD_ELEM4(dst, gid) {";
-            for (size_t q = 0; q < pre_elem.size(); ++q) k << " (dst)[" << q << "] = *(const float4*)(b" << fk.epilogue_inputs[pre_elem[q]].buffer << " + (gid));";
-            k << " }\n#define MM_STORE4P(v, idx, b, m, n, colv, elv) mm_store4_pre(v, idx, b, m, n, colv, elv, " << em.params_pass() << ")\n";
+            bool all_signs = !pre_elem.empty();
+            for (size_t q = 0; q < pre_elem.size(); ++q) {
+                if (pre_elem[q] == fk.epilogue_sign_input)
+                    k << " (dst)[" << q << "].x = U2F((uint)((const unsigned char*)b" << fk.epilogue_inputs[pre_elem[q]].buffer << ")[(gid) >> 2]);";
+                else {
+                    k << " (dst)[" << q << "] = *(const float4*)(b" << fk.epilogue_inputs[pre_elem[q]].buffer << " + (gid));";
+                    all_signs = false;
+                }
+            }
+            // (a byte per round: all of a unit's rounds are requested before the first)
+            k << " }\n#define MM_PRE_ALL " << (all_signs ? 1 : 0) << "\n";
+            k << "#define MM_STORE4P(v, idx, b, m, n, colv, elv) mm_store4_pre(v, idx, b, m, n, colv, elv, " << em.params_pass() << ")\n";
         } else {
-            k << "#define MM_NPRE_COL 0\n#define MM_NPRE_ELEM 0\n";
+            k << "#define MM_NPRE_COL 0\n#define MM_NPRE_ELEM 0\n#define MM_PRE_ALL 0\n";
+            if (fk.epilogue_sign_input >= 0) return "matmul: the sign bytes' operand is not requested ahead";
         }
     } else {
         k << "#define MM_STORE(v, idx, b, m, n) b" << fk.outputs[0] << "[idx] = (v)\n";
         k << "#define MM_STORE4(v, idx, b, m, n) *(float4*)(b" << fk.outputs[0] << " + (idx)) = (v)\n";
-        k << "#define MM_NPRE_COL 0\n#define MM_NPRE_ELEM 0\n";
+        k << "#define MM_NPRE_COL 0\n#define MM_NPRE_ELEM 0\n#define MM_PRE_ALL 0\n";
     }
     k << kMatmulMfmaSource;
 
@@ -3528,6 +3553,8 @@ string gen_matmul(Emitter& em, Generated* out) {
                   a_mode, b_mode, (long long)kchunks, fk.has_epilogue ? " +epilogue" : "", fk.colsum_out >= 0 ? " +column sums of B" : "",
                   out->persistent_ok ? " persistent" : "", direct == 3 ? " tiles straight into LDS x3" : direct == 2 ? " tiles straight into LDS x2" : "");
     out->note = note;
+    if (fk.sign_out >= 0) out->note += ", writes its output's sign bytes";
+    if (fk.epilogue_sign_input >= 0) out->note += ", masks by sign bytes";
     return "";
 }
 
@@ -3608,6 +3635,9 @@ void count_work(const FusedKernel& fk, Generated* g) {
     if (d.kind == DSC_KERNEL_SCATTER_ADD)  // read-modify-write of the entries that receive a value
         out_each = 2.0 * std::min((double)element_count(d.shape), (double)element_count(d.inputs[0].out_shape));
     if (fk.row_stages.empty()) elements += out_each * (double)fk.outputs.size();
+    // a byte per four elements written beside the activation / read in place of it
+    if (fk.sign_out >= 0) elements -= out_each * (15.0 / 16.0);
+    if (fk.epilogue_sign_input >= 0) elements -= out_each * (15.0 / 16.0);
     if (fk.pair.on) {
         // the last output is the weight gradient's partials, and its flops are those of the MatMul it stands for
         const MatMulDims m = matmul_dims(d);
@@ -3768,6 +3798,8 @@ std::string FusedKernel::key() const {
     if (row_width) s += "|RW" + to_string((long long)row_width);
     if (as_part) s += "|AP";
     if (colsum_out >= 0) s += "|CS" + to_string(colsum_out);
+    if (sign_out >= 0) s += "|SG" + to_string(sign_out) + "," + to_string(sign_source);
+    if (epilogue_sign_input >= 0) s += "|SI" + to_string(epilogue_sign_input);
     if (pair.on) s += "|GP" + to_string(pair.x_buffer) + "," + to_string(pair.out) + "," + to_string((long long)pair.chunk_rows) + "," + to_string((long long)pair.chunks);
     s += "|O";
     for (int o : outputs) s.append(reinterpret_cast<const char*>(&o), 4);
@@ -3851,7 +3883,7 @@ static std::string generate_one(const FusedKernel& fk, Generated* out, bool with
             return "this kernel kind takes no epilogue";
         if (fk.epilogue_permuted && mk != DSC_KERNEL_REDUCE) return "only a Reduce takes an epilogue through a permuting view";
         if (fk.epilogue_keeps_product && (mk == DSC_KERNEL_MATMUL || fk.epilogue_permuted)) return "this epilogue cannot keep its product";
-        if (!fk.pool.on && (int)fk.outputs.size() != fk.epilogue.raw().n_outputs + (fk.epilogue_keeps_product ? 1 : 0) + (fk.pair.on ? 1 : 0)) return "epilogue output count";
+        if (!fk.pool.on && (int)fk.outputs.size() != fk.epilogue.raw().n_outputs + (fk.epilogue_keeps_product ? 1 : 0) + (fk.pair.on ? 1 : 0) + (fk.sign_out >= 0 ? 1 : 0)) return "epilogue output count";
     }
     if (fk.pool.on) {
         if (!fk.cfwd.on) return "pooling rides on the convolution-forward kernel only";

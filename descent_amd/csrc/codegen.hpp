@@ -195,6 +195,14 @@ struct FusedKernel {
     } pair;
     bool sum_chunks = false;               // MatMul: ignore the descriptor's chunk count, write one full sum
     int colsum_out = -1;                   // MatMul (MFMA template): buffer that takes the column sums of B per k chunk
+    // MatMul (MFMA template, 16-byte store path) with an epilogue: `sign_out` is a buffer that takes one byte per four
+    // consecutive results of the epilogue's output `sign_source`, bit j set where result 4i + j is positive -- what the
+    // backward pass asks of a stored activation when all it does with it is "(a > 0) ? x : y".  `epilogue_sign_input`
+    // names an epilogue input that is read from such bytes instead of the activation itself (every use of that input
+    // is the left side of a "> 0" select): one byte per lane and store round, requested for all of a unit's rounds
+    // before the first, in place of a 16-byte load per round that the round then waited for.
+    int sign_out = -1, sign_source = 0;
+    int epilogue_sign_input = -1;
     bool as_part = false;                  // generated as one part of a multi-part launch (set while the launch is generated)
     std::vector<int> outputs;              // pointer parameter index of each output of main (or of the epilogue)
     int n_buffers = 0;                     // number of pointer parameters

@@ -105,6 +105,7 @@ void compact(Draft& d) {
     for_each_source(d.fk, [&](Source& s) { if (s.buffer >= 0) s.buffer = remap[s.buffer]; });
     for (int& o : d.fk.outputs) o = remap[o];
     if (d.fk.colsum_out >= 0) d.fk.colsum_out = remap[d.fk.colsum_out];
+    if (d.fk.sign_out >= 0) d.fk.sign_out = remap[d.fk.sign_out];
     d.params = params;
     d.fk.buffer_is_output = is_out;
     d.fk.n_buffers = (int)params.size();
@@ -2898,6 +2899,100 @@ struct Planner {
         }
     }
 
+    // Pass 3h: what a dense layer's backward pass asks of the stored activation.  The data gradient of the layer
+    // above, dX = (a > 0) ? g : g x c, is the epilogue of a MatMul and reads the activation a [m, n] element for element
+    // -- as many bytes again as the product it masks -- to look at one bit of each.  The MatMul that wrote a has every
+    // element in registers when it stores it: it writes a byte per four consecutive elements beside them (bit j set
+    // where element 4i + j is positive), and the masked product reads those bytes, a sixteenth of the activation, all
+    // of a unit's store rounds requested before the first (FusedKernel::sign_out / epilogue_sign_input).  a itself stays:
+    // the next layer reads it.  Bit for bit the same results: "(a > 0)" is evaluated once, by the writer, on the same a.
+    void activation_signs_as_bytes() {
+        const char* sw = std::getenv("DSC_SIGN_BYTES");
+        if (sw && sw[0] == '0') return;
+        for (int di = 0; di < (int)drafts.size(); ++di) {
+            Draft& D = drafts[di];
+            const dsc_kernel_desc& dd = D.fk.main.raw();
+            if (!D.alive || dd.kind != DSC_KERNEL_MATMUL || !D.fk.has_epilogue || D.fk.epilogue_sign_input >= 0 || !D.fk.parts.empty() || !D.fk.row_stages.empty() ||
+                D.fk.dgrad.on || D.fk.cfwd.on || D.fk.pair.on || D.fk.out_slice_width || D.fk.colsum_out >= 0 || !D.fk.virtuals.empty())
+                continue;
+            const dsc_kernel_desc& pe = D.fk.epilogue.raw();
+            const MatMulDims g = matmul_dims(dd);
+            const int64_t count = g.batch * g.m * g.n;
+            if (dd.output_mode != DSC_MATMUL_BATCHES || count % 4 != 0 || count < (1 << 20)) continue;
+            for (int in = 0; in < pe.n_inputs; ++in) {
+                if (in == D.fk.epilogue_product_input || D.fk.epilogue_inputs[in].buffer < 0) continue;
+                if (!is_identity(pe.inputs[in]) || element_count(pe.inputs[in].out_shape) != count) continue;
+                // every load of the input is the left side of a "> 0" select and nothing else
+                bool only_signs = true, any = false;
+                for (int q = 0; q < pe.n_ops && only_signs; ++q) {
+                    if (pe.ops[q].kind != DSC_PE_LOAD || pe.ops[q].input_index != in) continue;
+                    any = true;
+                    for (int o = 0; o < pe.n_outputs; ++o)
+                        if (pe.outputs[o] == q) only_signs = false;
+                    for (int r = 0; r < pe.n_ops && only_signs; ++r) {
+                        const dsc_pe_op& u = pe.ops[r];
+                        const int nargs = u.kind == DSC_PE_UNARY || u.kind == DSC_PE_GATHER ? 1 : u.kind == DSC_PE_BINARY ? 2 : u.kind == DSC_PE_SELECT ? 4 : 0;
+                        for (int a = 0; a < nargs; ++a) {
+                            if (u.args[a] != q) continue;
+                            const bool as_sign = u.kind == DSC_PE_SELECT && u.op == DSC_CMP_GT && a == 0 && pe.ops[u.args[1]].kind == DSC_PE_LITERAL_F32 &&
+                                                 pe.ops[u.args[1]].bits == 0u && u.args[2] != q && u.args[3] != q;
+                            if (!as_sign) only_signs = false;
+                        }
+                    }
+                }
+                if (!any || !only_signs) continue;
+                const int a_node = D.params[D.fk.epilogue_inputs[in].buffer];
+                // the MatMul that writes a, element for element in product order
+                int fi = -1, src = -1;
+                for (int q = 0; q < di && fi < 0; ++q) {
+                    const Draft& F = drafts[q];
+                    if (!F.alive || F.fk.main.raw().kind != DSC_KERNEL_MATMUL || !F.fk.has_epilogue || !F.fk.parts.empty() || !F.fk.row_stages.empty() || F.fk.dgrad.on ||
+                        F.fk.cfwd.on || F.fk.pair.on || F.fk.out_slice_width || F.fk.main.raw().output_mode != DSC_MATMUL_BATCHES)
+                        continue;
+                    const MatMulDims gf = matmul_dims(F.fk.main.raw());
+                    if (gf.batch * gf.m * gf.n != count) continue;
+                    const int n_epi = F.fk.epilogue.raw().n_outputs;
+                    for (int o = 0; o < n_epi && o < (int)F.outs.size(); ++o)
+                        if (F.outs[o].node == a_node && F.outs[o].copy_from < 0) { fi = q; src = o; }
+                }
+                if (fi < 0) continue;
+                Draft f2 = drafts[fi], d2 = D;
+                int bytes_node = -1;
+                bool fresh = false;
+                if (f2.fk.sign_out >= 0) {
+                    if (f2.fk.sign_source != src) continue;
+                    bytes_node = f2.params[f2.fk.sign_out];
+                } else {
+                    node_bytes.push_back((size_t)((count / 4 + 3) / 4 * 4));
+                    is_graph_output.push_back(false);
+                    is_graph_input.push_back(false);
+                    bytes_node = n_nodes++;
+                    fresh = true;
+                    f2.fk.sign_out = param_index(f2, bytes_node, true);
+                    f2.fk.sign_source = src;
+                    f2.fk.outputs.push_back(f2.fk.sign_out);
+                    f2.outs.push_back(StepOutput{bytes_node, -1, false, 0});
+                }
+                d2.fk.epilogue_inputs[in].buffer = param_index(d2, bytes_node, false);
+                d2.fk.epilogue_sign_input = in;
+                compact(d2);
+                Generated probe_f, probe_d;
+                if (!generate(f2.fk, &probe_f).empty() || !generate(d2.fk, &probe_d).empty()) {
+                    if (fresh) {
+                        node_bytes.pop_back();
+                        is_graph_output.pop_back();
+                        is_graph_input.pop_back();
+                        --n_nodes;
+                    }
+                    continue;
+                }
+                drafts[fi] = f2;
+                drafts[di] = d2;
+                break;  // one such operand per product
+            }
+        }
+    }
+
     // Pass 4: launches of a few workgroups each (optimiser updates of small tensors, short reductions, scalar
     // bookkeeping) cost a launch apiece while using a fraction of the machine.  Runs of them that do not
     // depend on one another become one multi-part launch; a later launch is hoisted into the run when nothing
@@ -3009,6 +3104,7 @@ struct Planner {
         chain_scatter_adds();                   // pass 3b
         group_chain_launches();                 // pass 3e
         pair_output_layer_gradients();          // pass 3f
+        activation_signs_as_bytes();            // pass 3h
         share_launches();                       // pass 4
     }
 };

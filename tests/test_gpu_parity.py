@@ -909,6 +909,29 @@ def test_pooling_gradients_read_off_window_words_are_bit_equal(hip_backend_sessi
         assert np.array_equal(results[0][key], results[1][key]), (key, listings[1])
 
 
+@pytest.mark.parametrize("side", [128, 100])
+def test_masked_data_gradients_read_sign_bytes_bit_equal(hip_backend_session, monkeypatch, side):
+    """Two Adam steps of the coordinate MLP (leaky_relu layers of 256) with the data gradients masked by the stored
+    activations (DSC_SIGN_BYTES=0) and by the bytes of sign bits the forward products write beside them: "(a > 0)" is
+    evaluated on the same values either way, so everything comes out bit for bit the same.  side 100: 10000 rows, the
+    last tile reaches past them."""
+    from descent_amd import Environment, workloads
+
+    results, listings = [], []
+    for on in ("0", "1"):
+        monkeypatch.setenv("DSC_SIGN_BYTES", on)
+        env = Environment(hip_backend_session)
+        w = workloads.coordinate_mlp(env, side=side)
+        for step in range(2):
+            env.run(w.graph, 5 + step)
+        results.append(w.snapshot())
+        listings.append(next(iter(w.graph.__dict__["_schedules"].values())).describe())
+    assert "sign bytes" not in listings[0], listings[0]
+    assert listings[1].count("masks by sign bytes") == 3 and listings[1].count("writes its output's sign bytes") == 3, listings[1]
+    for key in results[0]:
+        assert np.array_equal(results[0][key], results[1][key]), (key, listings[1])
+
+
 def _conv_grad_case(env, m, h, w, c_in, c_out, fh, fw, pad, groups, seed):
     """x -> conv2d -> 0.5 * sum(y^2): the gradients with respect to the image and the filter."""
     from descent_amd import Initializer

@@ -343,3 +343,20 @@ def test_surplus_k_chunks_keep_the_bounds_checked_register_path():
     assert direct(3, 64) == 0
     assert direct(3, 96) > 0
     assert direct(5, 128) == 0  # chunks of 32: 5 * 32 > 128
+
+
+def test_masked_data_gradients_read_the_sign_bytes_the_forward_products_write():
+    """cfg4: the three hidden layers whose data gradient is needed are masked by (a > 0) of the stored activation; the
+    forward products that write those activations add a byte per four elements, the gradients read the bytes."""
+    code = "import sys; sys.path.insert(0, %r); from descent_amd import Environment, hip_backend, workloads; from oracle.cpu_backend import CpuBackend; " \
+           "print(hip_backend.check_schedule(workloads.coordinate_mlp(Environment(CpuBackend())).graph, fused=True))"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+    def plan(**env):
+        return subprocess.run([sys.executable, "-c", code % root], env=dict(os.environ, **env), check=True, capture_output=True, text=True).stdout
+
+    on, off = plan(), plan(DSC_SIGN_BYTES="0")
+    assert on.count("masks by sign bytes") == 3 and on.count("writes its output's sign bytes") == 3, on
+    assert "sign bytes" not in off
+    # 3 x 268 MB of activations not read again, 3 x 16.8 MB of bytes written and read
+    assert "7318.3" in on.strip().splitlines()[-1] and "8022.9" in off.strip().splitlines()[-1], (on.strip().splitlines()[-1], off.strip().splitlines()[-1])
