@@ -3274,6 +3274,10 @@ string gen_matmul(Emitter& em, Generated* out) {
     if (fk.out_slice_width && (!rows_kernel_applies(fk, g) || fk.dgrad.on || fk.cfwd.on)) return "matmul: only the row-per-thread kernel stores slice-major";
     // (a gradient pair is a short-k kernel whatever else the product's shape would allow)
     if (fk.pair.on) return smallk_kernel_applies(fk, g) && !fk.out_slice_width ? gen_matmul_smallk_pair(em, out) : string("matmul: a gradient pair needs the short-k kernel");
+    // (sign bytes are written and read by the MFMA template's 16-byte store path only)
+    if ((fk.sign_out >= 0 || fk.epilogue_sign_input >= 0) &&
+        (rows_kernel_applies(fk, g) || smallk_kernel_applies(fk, g) || tallk_kernel_applies(fk, g) || dot_kernel_applies(fk, g) || ksplit_kernel_applies(fk, g)))
+        return "matmul: sign bytes need the MFMA kernel";
     if (rows_kernel_applies(fk, g)) return gen_matmul_rows(em, out);
     if (smallk_kernel_applies(fk, g)) return gen_matmul_smallk(em, out);
     if (tallk_kernel_applies(fk, g)) return gen_matmul_tallk(em, out);
