@@ -2950,7 +2950,7 @@ struct Planner {
                         F.fk.cfwd.on || F.fk.pair.on || F.fk.out_slice_width || F.fk.main.raw().output_mode != DSC_MATMUL_BATCHES)
                         continue;
                     const MatMulDims gf = matmul_dims(F.fk.main.raw());
-                    if (gf.batch * gf.m * gf.n != count) continue;
+                    if (gf.batch != g.batch || gf.m != g.m || gf.n != g.n) continue;  // the same rows of the same width: one byte layout
                     const int n_epi = F.fk.epilogue.raw().n_outputs;
                     for (int o = 0; o < n_epi && o < (int)F.outs.size(); ++o)
                         if (F.outs[o].node == a_node && F.outs[o].copy_from < 0) { fi = q; src = o; }
