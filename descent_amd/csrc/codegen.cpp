@@ -2058,7 +2058,28 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         sync();
     }
     }
-    if (unpad && !wonly) {
+    // (four channels of a pixel per evaluation where the layouts allow 16-byte pieces; the sums keep their order)
+    const bool fold4 = unpad && !wonly && H > 1 && W > 1 && C % 4 == 0 && GC % 4 == 0 && L.XT_AT % 4 == 0 && BUFSZ % 4 == 0;
+    if (fold4) {
+        const int64_t CQ = C / 4;
+        k << "        for (int i = tid; i < " << S(H * W * CQ) << "; i += 256) {\n";
+        k << "            const int c = (i % " << S(CQ) << ") * 4, x = (i / " << S(CQ) << ") % " << S(W) << ", y = i / " << S(CQ * W) << ";\n";
+        k << "            float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);\n";
+        auto slots = [&](const string& q, bool is_y) {
+            return "for (int " + q + " = 0; " + q + " <= " + S(is_y ? cv.pad_h : cv.pad_w) + "; ++" + q + ")";
+        };
+        const string qo = cv.rows_first ? "qx" : "qy", qi = cv.rows_first ? "qy" : "qx";
+        k << "            const bool edge_y = y == 0 || y == " << S(H - 1) << ", edge_x = x == 0 || x == " << S(W - 1) << ";\n";
+        k << "            const int base_y = y == 0 ? 0 : y + " << S(cv.pad_h) << ", base_x = x == 0 ? 0 : x + " << S(cv.pad_w) << ";\n";
+        k << "#pragma unroll\n            " << slots(qo, !cv.rows_first) << " {\n                float4 part = make_float4(0.f, 0.f, 0.f, 0.f);\n";
+        k << "#pragma unroll\n                " << slots(qi, cv.rows_first) << " {\n";
+        k << "                    const bool ok = (edge_y || qy == 0) && (edge_x || qx == 0);\n";
+        k << "                    const int ky = base_y + (edge_y ? qy : 0), kx = base_x + (edge_x ? qx : 0);\n";
+        k << "                    const float4 w = *(const float4*)(xt + bo + (ky * " << S(PW) << " + kx) * " << S(C) << " + c);\n";
+        k << "                    part.x += ok ? w.x : 0.f; part.y += ok ? w.y : 0.f; part.z += ok ? w.z : 0.f; part.w += ok ? w.w : 0.f;\n                }\n";
+        k << "                sum.x += part.x; sum.y += part.y; sum.z += part.z; sum.w += part.w;\n            }\n";
+        k << "            *(float4*)(" << out_ptr << " + ((img * " << S(H) << " + y) * " << S(W) << " + x) * " << S(GC) << " + cb * " << S(C) << " + c) = sum;\n        }\n";
+    } else if (unpad && !wonly) {
         k << "        for (int i = tid; i < " << S(H * W * C) << "; i += 256) {\n";
         k << "            const int c = i % " << S(C) << ", x = (i / " << S(C) << ") % " << S(W) << ", y = i / " << S(C * W) << ";\n";
         k << "            float sum = 0.f;\n";
