@@ -1789,6 +1789,10 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     // the B fragments are the same for every group: they stay in registers for the whole kernel.
     const int64_t P = L.P, TQ = L.TQ, GS = L.GS, GPR = L.GPR, GROUPS = L.GROUPS, TPW = L.TPW;
     const bool mfma_dgrad = L.mfma_dgrad;
+    // the geometry whose border folds are lane exchanges (below): pairs of 8 channels, 8 pairs per padded row (two rows
+    // per tile of 16 pairs), one replicated pixel on every side
+    const bool reg_fold = mfma_dgrad && !wonly && C == 8 && PW == 16 && PH % 2 == 0 && cv.pad_h == 1 && cv.pad_w == 1 && H > 1 && W > 1 &&
+                          !(std::getenv("DSC_CONV_BWD_REGFOLD") && std::getenv("DSC_CONV_BWD_REGFOLD")[0] == '0');
     if (mfma_dgrad && spec) {
         // this lane's pixel group in each of the wave's tiles: its row, and the word of its first tap in filter row 0
         k << "    int dgy[" << S(TPW) << "], dbase[" << S(TPW) << "];\n";
@@ -2014,6 +2018,24 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         };
         if (!unpad) {
             emit_dacc_stores(out_ptr + "[(img * " + S(PH * PW) + " + p) * " + S(GC) + " + cb * " + S(C) + " + gc]");
+        } else if (reg_fold) {
+            // Border folds in registers.  Register r of lane (li, lk) of tile T is padded pixel row 2 T + lk / 2, pixel
+            // pair 4 (lk % 2) + r, pixel li / 8 of the pair, channel li % 8: the two padded columns that replicate an
+            // image's edge column are the two pixels of the row's first / last pair (lanes 8 apart), the two padded rows
+            // that replicate an edge row are the two rows of the first / last tile (lanes 32 apart).  Sums in the order
+            // of the Unpads; the lane whose padded pixel is the image's own stores.
+            const string yfold = "                if (T == 0 || T == " + S(L.TILES - 1) + ") {\n#pragma unroll\n                    for (int r = 0; r < 4; ++r) v[r] += __shfl_xor(v[r], 32, 64);\n                }\n";
+            const string xfold = "                {\n                    const float f0 = v[0] + dsc_lane_xor8(v[0]), f3 = v[3] + dsc_lane_xor8(v[3]);\n"
+                                 "                    v[0] = (lk & 1) ? v[0] : f0;\n                    v[3] = (lk & 1) ? f3 : v[3];\n                }\n";
+            k << "        {\n            const int par = li >> 3, gc = li & 7;\n";
+            k << "#pragma unroll\n            for (int t = 0; t < " << S(TPW) << "; ++t) {\n";
+            k << "                const int T = t * 4 + wave;\n                float v[4] = {dacc[t][0], dacc[t][1], dacc[t][2], dacc[t][3]};\n";
+            k << (cv.rows_first ? yfold + xfold : xfold + yfold);
+            k << "                const int gy = 2 * T + (lk >> 1);\n";
+            k << "#pragma unroll\n                for (int r = 0; r < 4; ++r) {\n";
+            k << "                    const int gx = 2 * (4 * (lk & 1) + r) + par;\n";
+            k << "                    if (T < " << S(L.TILES) << " && gy >= 1 && gy <= " << S(PH - 2) << " && gx >= 1 && gx <= " << S(PW - 2) << ") " << out_ptr << "[((img * " << S(H)
+              << " + gy - 1) * " << S(W) << " + gx - 1) * " << S(GC) << " + cb * " << S(C) << " + gc] = v[r];\n                }\n            }\n        }\n";
         } else {
             sync();
             emit_dacc_stores("xt[bo + p * " + S(C) + " + gc]");
@@ -2060,7 +2082,9 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     }
     // (four channels of a pixel per evaluation where the layouts allow 16-byte pieces; the sums keep their order)
     const bool fold4 = unpad && !wonly && H > 1 && W > 1 && C % 4 == 0 && GC % 4 == 0 && L.XT_AT % 4 == 0 && BUFSZ % 4 == 0;
-    if (fold4) {
+    if (reg_fold) {
+        // (folded in registers above)
+    } else if (fold4) {
         const int64_t CQ = C / 4;
         k << "        for (int i = tid; i < " << S(H * W * CQ) << "; i += 256) {\n";
         k << "            const int c = (i % " << S(CQ) << ") * 4, x = (i / " << S(CQ) << ") % " << S(W) << ", y = i / " << S(CQ * W) << ";\n";
