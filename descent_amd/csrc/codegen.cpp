@@ -1765,7 +1765,27 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
     else k << "    const int tid = threadIdx.x;\n";
     k << "    const int lane = tid & 63, wave = " << (spec ? "__builtin_amdgcn_readfirstlane(tid >> 6)" : "tid >> 6") << ", li = lane & 15, lk = lane >> 4;\n";
     // what stays zero for the whole kernel: slots without a pixel, the zero row, the tile words behind the last pixel
-    k << "    for (int i = threadIdx.x; i < " << S(ONE_AT) << "; i += " << S(BLOCK) << ") smem[i] = 0.f;\n";
+    if (spec) {
+        // (with loader waves no barrier stands between this and the first image's fills: only the words no fill writes
+        // and a fragment may read are cleared -- the head, the slots right of the output's columns, the slots behind
+        // its last row with the zero row, the tile words behind the last pixel)
+        const int64_t RB = (PW - OW) * PITCH;
+        auto clear_range = [&](int64_t from, int64_t to) {
+            for (int64_t b2 = 0; b2 < 2; ++b2)
+                if (to > from)
+                    k << "    for (int i = threadIdx.x; i < " << S(to - from) << "; i += " << S(BLOCK) << ") smem[" << S(b2 * BUFSZ + from) << " + i] = 0.f;\n";
+        };
+        clear_range(0, L.DC_AT);
+        clear_range(L.DC_AT + OH * PW * PITCH, L.XT_AT);
+        clear_range(L.XT_AT + PH * PW * CP, BUFSZ);
+        if (RB > 0) {
+            k << "    for (int i = threadIdx.x; i < " << S(2 * OH * RB) << "; i += " << S(BLOCK) << ") {\n";
+            k << "        const int r = i % " << S(OH * RB) << ";\n";
+            k << "        smem[(i / " << S(OH * RB) << ") * " << S(BUFSZ) << " + " << S(L.DC_AT) << " + ((r / " << S(RB) << ") * " << S(PW) << " + " << S(OW) << ") * " << S(PITCH) << " + r % " << S(RB) << "] = 0.f;\n    }\n";
+        }
+    } else {
+        k << "    for (int i = threadIdx.x; i < " << S(ONE_AT) << "; i += " << S(BLOCK) << ") smem[i] = 0.f;\n";
+    }
     k << "    if (threadIdx.x == 0) { smem[" << S(ONE_AT) << "] = 1.f; smem[" << S(ZW_AT) << "] = 0.f; }\n";
     // fragment addresses of this lane: a constant, plus the step's slot term where the mask says so
     k << "    int a_off[" << MT << "], a_msk[" << MT << "], b_off[" << NT << "], b_msk[" << NT << "];\n";
@@ -1800,16 +1820,23 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         k << "        const int grp = (t * 4 + wave) * 16 + li;\n        dgy[t] = grp / " << S(GPR) << ";\n";
         k << "        dbase[t] = " << S(L.DC_AT) << " + (dgy[t] * " << S(PW) << " + (grp % " << S(GPR) << ") * " << S(P) << " - " << S(FW - 1) << ") * " << S(PITCH) << " + lk;\n    }\n";
     }
-    if (mfma_dgrad) {
+    // (with loader waves the four matrix waves take a quarter of the fragments each, while the loader waves already
+    // have the set's first image requested: one round trip to memory before the first product, not two)
+    auto emit_b_fragments = [&](bool shared_out) {
         k << "    {\n";
         k << "        const int par = li / " << S(C) << ", gc = li % " << S(C) << ";\n";
-        for (int64_t s = 0; s < GS; ++s) {
-            const int64_t oc0 = (4 * s) % K, tt = (4 * s) / K, ty = tt / TQ, tq = tt % TQ - (P - 1);
-            k << "        { const int tx = " << S(tq) << " + par; const float w = load_b(cb, " << S(oc0) << " + lk, (" << S(ty * FW) << " + clampi(tx, 0, " << S(FW - 1)
-              << ")) * " << S(C) << " + gc, " << em.params_pass() << "); smem[" << S(GB_AT + s * 64) << " + lane] = (tx >= 0 && tx < " << S(FW) << ") ? w : 0.f; }\n";
+        for (int64_t w4 = 0; w4 < (shared_out ? 4 : 1); ++w4) {
+            if (shared_out) k << "        " << (w4 ? "else " : "") << "if (wave == " << S(w4) << ") {\n";
+            for (int64_t s = shared_out ? w4 : 0; s < GS; s += shared_out ? 4 : 1) {
+                const int64_t oc0 = (4 * s) % K, tt = (4 * s) / K, ty = tt / TQ, tq = tt % TQ - (P - 1);
+                k << "        { const int tx = " << S(tq) << " + par; const float w = load_b(cb, " << S(oc0) << " + lk, (" << S(ty * FW) << " + clampi(tx, 0, " << S(FW - 1)
+                  << ")) * " << S(C) << " + gc, " << em.params_pass() << "); smem[" << S(GB_AT + s * 64) << " + lane] = (tx >= 0 && tx < " << S(FW) << ") ? w : 0.f; }\n";
+            }
+            if (shared_out) k << "        }\n";
         }
         k << "    }\n";
-    }
+    };
+    if (mfma_dgrad && !spec) emit_b_fragments(false);
     // Fills.  The loads of an image -- dC of the image and group, and the image's padded input tile,
     // xt[py][px][c] = image[clamp(py - pad_h)][clamp(px - pad_w)][c] -- are all issued before the first of them is
     // stored to LDS: one round trip to memory per image.  (Requesting the next image's loads before the matrix phases
@@ -1885,7 +1912,7 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         k << ind << "    if (tid + u * 256 < " << S(xn) << ") *(" << vt << "*)(xt + " << buf << " + (e / " << S(C) << ") * " << S(CP) << " + e % " << S(C) << ") = xv[u];\n"
           << ind << "}\n";
     };
-    k << "    __syncthreads();\n";
+    if (!spec) k << "    __syncthreads();\n";
     // Barriers the lower waves pass inside one image's matrix phases: the loader waves pass as many.
     int phase_syncs = 0;
     auto sync = [&]() {
@@ -1897,7 +1924,9 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         // The two roles are two loops, so that neither carries the other's registers (the accumulators and fragment
         // addresses of the matrix phases, the addresses the fills keep): the loader waves then have room to request
         // all of an image's loads in one go.  Both pass the same barriers.
-        k << "    if (!loader) {\n    __syncthreads();\n" << loop_head;
+        k << "    if (!loader) {\n";
+        if (mfma_dgrad) emit_b_fragments(true);
+        k << "    __syncthreads();\n" << loop_head;
     } else {
         k << "    constexpr int bo = 0;\n";
         k << "    for (int img = chunk; img < " << S(IMG) << "; img += " << S(cv.chunks) << ") {\n";
