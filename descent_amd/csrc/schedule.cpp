@@ -2617,6 +2617,18 @@ struct Planner {
             q2.fk.dgrad.pm.masks.buffer = param_index(q2, words, false);
             q2.fk.dgrad.pm.leak_bits = leak_bits;
             compact(q2);
+            // the pooled array itself, kept beside its consumer's output for this chain alone, is no longer written
+            if (f2.fk.pool.has_epilogue && !is_graph_output[p_node] && F.outs[n_out + n_epi].copy_from < 0) {
+                bool only_q = true;
+                for (int c : consumers_of(p_node))
+                    if (c != qi) only_q = false;
+                if (only_q) {
+                    f2.fk.pool.store_pooled = false;
+                    f2.fk.outputs.pop_back();
+                    f2.outs.pop_back();
+                    compact(f2);
+                }
+            }
             Generated probe_f, probe_q;
             if (!generate(f2.fk, &probe_f).empty() || !generate(q2.fk, &probe_q).empty()) {
                 node_bytes.pop_back();
