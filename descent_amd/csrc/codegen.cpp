@@ -2295,7 +2295,8 @@ string gen_conv_fwd(Emitter& em, Generated* out) {
     k << "    const int lane = threadIdx.x & 63, li = lane & 15, lk = lane >> 4;\n";
     // the 16-pixel tiles are dealt to the four waves in turn; which wave takes the odd ones out rotates with the
     // workgroup, so that no SIMD of a CU collects all of them
-    k << "    const int wv = ((threadIdx.x >> 6) + blockIdx.x) & 3;\n";
+    // (through readfirstlane: the tile numbers and what the addresses take from them are then scalar arithmetic)
+    k << "    const int wv = __builtin_amdgcn_readfirstlane((int)(((threadIdx.x >> 6) + blockIdx.x) & 3));\n";
     // 1. B goes through LDS: every wave needs all of it in MFMA fragment order, and when each wave of every
     // workgroup fetched its fragments itself (K/4 loads per lane, the same few cache lines for the whole grid) those
     // loads alone cost a third of the kernel.  Zero beyond k and n.
@@ -2403,12 +2404,10 @@ string gen_conv_fwd(Emitter& em, Generated* out) {
             // the window's maximum: across the column pair, then across the row pair
             // (the four channels side by side, step by step: a lane exchange may not follow the instruction that wrote
             // its operand, and written channel by channel every exchange waited out that distance)
-            k << ind << "        float pm[4], px[4];\n";
+            k << ind << "        float pm[4];\n";
             for (int i = 0; i < 4; ++i) k << ind << "        pm[" << i << "] = " << val(i, fk.pool.source) << ";\n";
-            k << "#pragma unroll\n" << ind << "        for (int i = 0; i < 4; ++i) px[i] = dsc_lane_xor1(pm[i]);\n";
-            k << "#pragma unroll\n" << ind << "        for (int i = 0; i < 4; ++i) pm[i] = glsl_max(pm[i], px[i]);\n";
-            k << "#pragma unroll\n" << ind << "        for (int i = 0; i < 4; ++i) px[i] = dsc_lane_xor8(pm[i]);\n";
-            k << "#pragma unroll\n" << ind << "        for (int i = 0; i < 4; ++i) pm[i] = glsl_max(pm[i], px[i]);\n";
+            k << "#pragma unroll\n" << ind << "        for (int i = 0; i < 4; ++i) pm[i] = dsc_max_xor1(pm[i]);\n";
+            k << "#pragma unroll\n" << ind << "        for (int i = 0; i < 4; ++i) pm[i] = dsc_max_xor8(pm[i]);\n";
             const int64_t pbs = rows ? g.n : (int64_t)cv.img * OH2 * OW2 * g.n, prs = rows ? g.batch * g.n : g.n;
             if (fk.pool.masks) {
                 // two bits per element: equals its window's maximum, is positive; the four pixels of a window meet in
@@ -2423,9 +2422,10 @@ string gen_conv_fwd(Emitter& em, Generated* out) {
             if (fk.pool.has_epilogue) {
                 // the window's four lanes all hold its four maxima: each runs the consumer for one of the four channels
                 // (all four in one lane, the other three idle, cost this issue-bound kernel four times the instructions)
+                k << ind << "        const int wq = (li & 1) | ((li >> 3) << 1);\n";
+                k << ind << "        float pmq = pm[0];\n";
+                k << ind << "        pmq = wq == 1 ? pm[1] : pmq;\n" << ind << "        pmq = wq == 2 ? pm[2] : pmq;\n" << ind << "        pmq = wq == 3 ? pm[3] : pmq;\n";
                 k << ind << "        if (valid) {\n";
-                k << ind << "            const int wq = (li & 1) | ((li >> 3) << 1);\n";
-                k << ind << "            const float pmq = wq == 0 ? pm[0] : wq == 1 ? pm[1] : wq == 2 ? pm[2] : pm[3];\n";
                 k << ind << "            float pres[" << n_pool_out << "];\n";
                 k << ind << "            pool_epilogue(pmq, p_at + wq, pres, " << em.params_pass() << ");\n";
                 for (int o = 0; o < n_pool_out; ++o) k << ind << "            b" << fk.outputs[n_out + o] << "[p_at + wq] = pres[" << o << "];\n";
