@@ -1893,10 +1893,10 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         k << "#pragma unroll\n" << ind << "for (int u = 0; u < " << S(NC) << "; ++u) {\n";
         k << ind << "    const int i = (tid + u * 256) * " << S(dunit) << ", pi = i / " << S(K) << ";\n";
         if (pmask) {
-            k << ind << "    {\n" << ind << "        const uint bits = pw[u] >> (2 * (((pi % " << S(OW) << ") & 1) | (((band * " << S(OH) << " + pi / " << S(OW) << ") & 1) << 1)));\n";
+            k << ind << "    {\n" << ind << "        const uint bits = pw[u] >> (8 * (((pi % " << S(OW) << ") & 1) | (((band * " << S(OH) << " + pi / " << S(OW) << ") & 1) << 1)));\n";
             const char* comp[4] = {"x", "y", "z", "w"};
             for (int j = 0; j < 4; ++j)
-                k << ind << "        { const float v = (bits & " << (1u << (8 * j)) << "u) ? pv[u]." << comp[j] << " : 0.f; pv[u]." << comp[j] << " = (bits & " << (2u << (8 * j))
+                k << ind << "        { const float v = (bits & " << (1u << (2 * j)) << "u) ? pv[u]." << comp[j] << " : 0.f; pv[u]." << comp[j] << " = (bits & " << (2u << (2 * j))
                   << "u) ? v : v * " << pm_leak << "; }\n";
             k << ind << "    }\n";
         }
@@ -2405,17 +2405,14 @@ string gen_conv_fwd(Emitter& em, Generated* out) {
             // (the four channels side by side, step by step: a lane exchange may not follow the instruction that wrote
             // its operand, and written channel by channel every exchange waited out that distance)
             k << ind << "        float pm[4];\n";
-            for (int i = 0; i < 4; ++i) k << ind << "        pm[" << i << "] = " << val(i, fk.pool.source) << ";\n";
-            k << "#pragma unroll\n" << ind << "        for (int i = 0; i < 4; ++i) pm[i] = dsc_max_xor1(pm[i]);\n";
-            k << "#pragma unroll\n" << ind << "        for (int i = 0; i < 4; ++i) pm[i] = dsc_max_xor8(pm[i]);\n";
+            k << ind << "        dsc_window_max4(" << val(0, fk.pool.source) << ", " << val(1, fk.pool.source) << ", " << val(2, fk.pool.source) << ", " << val(3, fk.pool.source) << ", pm);\n";
             const int64_t pbs = rows ? g.n : (int64_t)cv.img * OH2 * OW2 * g.n, prs = rows ? g.batch * g.n : g.n;
             if (fk.pool.masks) {
                 // two bits per element: equals its window's maximum, is positive; the four pixels of a window meet in
                 // one word per four channels (lanes l, l ^ 1, l ^ 8, l ^ 9)
-                k << ind << "        uint mw = 0u;\n";
-                for (int i = 0; i < 4; ++i)
-                    k << ind << "        { const float v = " << val(i, fk.pool.source) << "; mw |= ((v == pm[" << i << "] ? 1u : 0u) | (v > 0.f ? 2u : 0u)) << " << 8 * i << "; }\n";
-                k << ind << "        mw <<= 2 * ((li & 1) | ((li >> 3) << 1));\n";
+                k << ind << "        uint mw = dsc_window_bits4(" << val(0, fk.pool.source) << ", " << val(1, fk.pool.source) << ", " << val(2, fk.pool.source) << ", " << val(3, fk.pool.source)
+                  << ", pm[0], pm[1], pm[2], pm[3]);\n";
+                k << ind << "        mw <<= 8 * ((li & 1) | ((li >> 3) << 1));\n";
                 k << ind << "        mw |= (uint)dsc_lane_xor1((int)mw);\n" << ind << "        mw |= (uint)dsc_lane_xor8((int)mw);\n";
             }
             k << ind << "        const int p_at = cb * " << S(pbs) << " + (img * " << S(OH2 * OW2) << " + (t / " << S(TPR) << ") * " << S(OW2) << " + (xr >> 1)) * " << S(prs) << " + cn;\n";

@@ -166,8 +166,8 @@ struct FusedKernel {
         // The pooled output's source is read by nothing but the backward pass of this pooling and of the activation in
         // front of it, which ask two things of each element: does it equal its window's maximum, and is it positive.
         // The kernel then writes those two bits per element in place of the element -- one word per pooling window and
-        // four channels, [g][img * oh/2 * ow/2][n / 4], byte j of a word for channel 4q + j, bits 2p and 2p + 1 of a
-        // byte for the window's pixel p = (x & 1) + 2 (y & 1) -- through the pointer that stood for the source, which
+        // four channels, [g][img * oh/2 * ow/2][n / 4], byte p of a word for the window's pixel p = (x & 1) + 2 (y & 1),
+        // bits 2j and 2j + 1 of a byte for channel 4q + j -- through the pointer that stood for the source, which
         // is never stored (see ConvDgrad::masks for the reader).
         bool masks = false;
         KernelDesc epilogue;
