@@ -1938,9 +1938,9 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         k << "        __syncthreads();\n";
     }
     // 2a. filter gradient: this wave's steps of four slots
-    if (spec) {
-        // Two waves per SIMD run these products (the other two are loader waves), so a wave has to keep the matrix
-        // pipe busy by itself: the fragments of two steps are requested before the first product is issued.
+    {
+        // With loader waves two waves per SIMD run these products (the other two are loader waves), so a wave has to
+        // keep the matrix pipe busy by itself: the fragments of two steps are requested before the first product is issued.
         // The fragment addresses are running registers: a step is an add per fragment (none for the second step of
         // a pair in the tiles whose rows are all real: its distance is a literal in the read), where a slot term
         // computed from the step number cost two to three vector instructions per read -- and vector instructions
@@ -1978,16 +1978,6 @@ string gen_conv_bwd(Emitter& em, Generated* out) {
         k << "#pragma unroll\n            for (int mt = 0; mt < " << MT << "; ++mt)\n#pragma unroll\n                for (int nt = 0; nt < " << NT << "; ++nt)\n";
         k << "                    wacc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[0][mt], fb[0][nt], wacc[mt][nt], 0, 0, 0);\n";
         k << "        }\n";
-    }
-    if (!spec) {
-    k << "#pragma unroll 2\n        for (int s = wave; s < " << S(L.steps) << "; s += 4) {\n";
-    k << "            const int q = 4 * s + lk, qa = q * " << S(CP) << ", qb = q * " << S(PITCH) << ";\n";
-    k << "            float fa[" << MT << "], fb[" << NT << "];\n";
-    k << "#pragma unroll\n            for (int mt = 0; mt < " << MT << "; ++mt) fa[mt] = smem[a_off[mt] + ((qa + bo) & a_msk[mt])];\n";
-    k << "#pragma unroll\n            for (int nt = 0; nt < " << NT << "; ++nt) fb[nt] = smem[b_off[nt] + bo + (qb & b_msk[nt])];\n";
-    k << "#pragma unroll\n            for (int mt = 0; mt < " << MT << "; ++mt)\n#pragma unroll\n                for (int nt = 0; nt < " << NT << "; ++nt)\n";
-    k << "                    wacc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[mt], fb[nt], wacc[mt][nt], 0, 0, 0);\n";
-    k << "        }\n";
     }
     const int64_t passes = (PH * PW + 255) / 256;
     if (wonly) {
