@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes one launch of the headline kernel moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same
 # command, each counter scaled by what it reads for the streaming kernel of known size (--copy-calibration); the
 # summary is profiles/matmul_mfma_8192.txt.  Only the 8192^3 workload has been counted.
-MEASURED_TRAFFIC_BYTES = {8192: 3.692e9}
+MEASURED_TRAFFIC_BYTES = {8192: 3.705e9}
 
 
 def time_graph(env, graph, steps: int, warmup: int, seed0: int = 1, profile: bool = True):
