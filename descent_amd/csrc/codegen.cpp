@@ -4392,6 +4392,7 @@ string generate_multi(const FusedKernel& fk, Generated* out) {
     std::ostringstream src, body;
     src << kPreludeSource << "\n";
     unsigned first = 0;
+    string pool_terms;
     for (size_t i = 0; i < fk.parts.size(); ++i) {
         const FusedKernel& part = fk.parts[i];
         if (!can_be_part(part)) return "multi: kernel cannot be a part";
@@ -4407,12 +4408,48 @@ string generate_multi(const FusedKernel& fk, Generated* out) {
             const string head = "extern \"C\" __global__ __launch_bounds__(256) void " + pg.entry + "(";
             const size_t at = text.find(head);
             if (at == string::npos) return "multi: unexpected entry point form";
-            text.replace(at, head.size(), "DSC_INLINE void part_entry(const uint dsc_block, ");
+            text.replace(at, head.size(), "DSC_INLINE void part_entry(char* const dsc_pool, const uint dsc_block, ");
             for (size_t pos = text.find("blockIdx.x"); pos != string::npos; pos = text.find("blockIdx.x", pos)) text.replace(pos, 10, "dsc_block");
             if (text.find("gridDim") != string::npos) return "multi: part depends on the grid size";
+            // The parts' LDS arrays overlie one another in the launch's one block (a kernel's distinct __shared__ arrays
+            // are laid out side by side whether or not they are ever live together: three MatMul parts of 16-26 KB each
+            // made a 62 KB launch of two workgroups per CU).  Every `__shared__ [aligned] T name[n]...;` becomes a
+            // reference into the block.
+            size_t used = 0;
+            for (size_t pos = text.find("__shared__"); pos != string::npos; pos = text.find("__shared__", pos)) {
+                size_t q = pos + 10;
+                auto skip = [&]() { while (q < text.size() && (text[q] == ' ' || text[q] == '\t')) ++q; };
+                auto word = [&]() { const size_t b = q; while (q < text.size() && (std::isalnum((unsigned char)text[q]) || text[q] == '_')) ++q; return text.substr(b, q - b); };
+                skip();
+                const string attr = "__attribute__((aligned(16)))";
+                if (text.compare(q, attr.size(), attr) == 0) q += attr.size();
+                skip();
+                const string type = word();
+                skip();
+                const string name = word();
+                const size_t size = type == "float" || type == "int" || type == "uint" ? 4 : type == "double" || type == "float2" ? 8 : type == "float4" ? 16 : 0;
+                string dims;
+                size_t count = 1;
+                bool ok = size != 0 && !name.empty();
+                while (ok && q < text.size() && text[q] == '[') {
+                    const size_t b = ++q;
+                    while (q < text.size() && std::isdigit((unsigned char)text[q])) ++q;
+                    if (q == b || q >= text.size() || text[q] != ']') { ok = false; break; }
+                    dims += "[" + text.substr(b, q - b) + "]";
+                    count *= (size_t)std::stoll(text.substr(b, q - b));
+                    ++q;
+                }
+                if (!ok || dims.empty() || q >= text.size() || text[q] != ';') return "multi: a part declares LDS in a form the launch's block cannot take";
+                const string ref = type + " (&" + name + ")" + dims + " = *reinterpret_cast<" + type + " (*)" + dims + ">(dsc_pool + " + to_string(used) + ");";
+                text.replace(pos, q + 1 - pos, ref);
+                used = (used + count * size + 15) / 16 * 16;
+                pos += ref.size();
+            }
+            text += "constexpr int dsc_part_lds_bytes = " + to_string(used) + ";\n";
         }
+        pool_terms += (i ? ", " : "") + string("part") + to_string(i) + "::dsc_part_lds_bytes";
         src << "namespace part" << i << " {\n" << text << "}  // namespace part" << i << "\n\n";
-        body << "    if (blockIdx.x < " << first + pg.grid << "u) { part" << i << "::part_entry(blockIdx.x - " << first << "u";
+        body << "    if (blockIdx.x < " << first + pg.grid << "u) { part" << i << "::part_entry(dsc_pool, blockIdx.x - " << first << "u";
         for (int j : fk.part_params[i]) body << ", b" << j;
         body << ", seed_cell, seed_value); return; }\n";
         first += pg.grid;
@@ -4422,7 +4459,10 @@ string generate_multi(const FusedKernel& fk, Generated* out) {
     }
     Emitter em(fk);
     g.entry = "dsc_multi_p" + to_string(fk.parts.size()) + "_g" + to_string(first);
-    src << "extern \"C\" __global__ __launch_bounds__(256) void " << g.entry << "(" << em.kernel_params_decl() << ") {\n" << body.str() << "}\n";
+    src << "constexpr int dsc_pool_sizes[] = {" << pool_terms << "};\n";
+    src << "constexpr int dsc_pool_bytes() { int m = 16; for (int v : dsc_pool_sizes) m = v > m ? v : m; return m; }\n";
+    src << "extern \"C\" __global__ __launch_bounds__(256) void " << g.entry << "(" << em.kernel_params_decl() << ") {\n";
+    src << "    __shared__ __attribute__((aligned(16))) char dsc_pool[dsc_pool_bytes()];\n" << body.str() << "}\n";
     g.source = src.str();
     g.grid = first;
     g.block = 256;
