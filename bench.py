@@ -128,14 +128,14 @@ def class_rooflines(be, steps):
     return out
 
 
-def bench_convnet(env, steps, warmup, batch=1000, repeats=5):
+def bench_convnet(env, steps, warmup, batch=1000, repeats=5, blur_pool=False):
     """ConvNet train steps per second: `repeats` timed regions of `steps` steps each (no per-launch events), the
     median reported with the spread beside it; then one more pass with events for the per-kernel table."""
     import re
 
     from descent_amd import workloads
 
-    w = workloads.convnet(env, batch=batch, seed=3)
+    w = workloads.convnet(env, batch=batch, seed=3, blur_pool=blur_pool)
     # (the warm-up is long enough for the device to reach the clock it holds under this load: the first region of a run
     # that starts from idle reads 1.5 % low)
     walls = [time_graph(env, w.graph, steps, max(warmup, 1000) if r == 0 else 0, seed0=1 + r * steps, profile=False) for r in range(repeats)]
@@ -405,7 +405,7 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=8192,
                     help="rows of the headline product the CPU baseline computes (a bounded sample of the same workload)")
     ap.add_argument("--workload", default="headline",
-                    choices=["headline", "matmul", "convnet", "convnet-uploads", "linear", "relu-pe", "siren", "hash-grid"],
+                    choices=["headline", "matmul", "convnet", "conv-blur-net", "convnet-uploads", "linear", "relu-pe", "siren", "hash-grid"],
                     help="headline: the 8192^3 matmul line with the ConvNet step rate beside it (default); matmul: "
                          "that line without the ConvNet; the others run one workload alone, e.g. under rocprofv3")
     ap.add_argument("--no-events", action="store_true", help="no per-launch HIP events (wall time only)")
@@ -430,8 +430,8 @@ def main():
     if args.workload not in ("headline", "matmul"):
         from descent_amd import workloads as _w
 
-        if args.workload == "convnet":
-            out = bench_convnet(env, args.steps, args.warmup)
+        if args.workload in ("convnet", "conv-blur-net"):
+            out = bench_convnet(env, args.steps, args.warmup, blur_pool=args.workload == "conv-blur-net")
             sys.stderr.write(out.pop("report"))
         elif args.workload == "convnet-uploads":
             out = bench_convnet_minibatch_uploads(env, steps=max(args.steps, 20))

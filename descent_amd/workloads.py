@@ -17,7 +17,7 @@ from .array import Parameter
 from .environment import Environment
 from .graph import Graph
 from .loss import softmax_cross_entropy_accuracy, softmax_cross_entropy_loss
-from .module import Conv2D, Dense, Dropout, EvalContext, MaxPool2D, Module
+from .module import Conv2D, Dense, Dropout, EvalContext, MaxBlurPool2D, MaxPool2D, Module
 from .optimizer import Adam, StochasticGradientDescent
 
 
@@ -44,13 +44,14 @@ class Workload:
 
 
 class ConvNet(Module):
-    """examples/fashion_mnist/main.rs:171-222 (max-pool variant)."""
+    """examples/fashion_mnist/main.rs:171-222: the max-pool network, or with `blur_pool` the ConvBlurNet whose pools
+    are a stride-1 max pool followed by a stride-2 depthwise blur (main.rs:187-199)."""
 
-    def __init__(self, env, c1=16, c2=32, hidden=128, classes=10, side=28):
+    def __init__(self, env, c1=16, c2=32, hidden=128, classes=10, side=28, blur_pool=False):
         self.conv1 = Conv2D(env, 1, c1, 3, 3, pad=1)
-        self.pool1 = MaxPool2D()
+        self.pool1 = MaxBlurPool2D(env, c1) if blur_pool else MaxPool2D()
         self.conv2 = Conv2D(env, c1, c2, 3, 3, pad=1, groups=2)
-        self.pool2 = MaxPool2D()
+        self.pool2 = MaxBlurPool2D(env, c2) if blur_pool else MaxPool2D()
         self.fc1 = Dense(env, (side // 4) * (side // 4) * c2, hidden)
         self.fc2 = Dense(env, hidden, classes)
 
@@ -126,12 +127,12 @@ def _classifier_workload(env: Environment, module: Module, batch: int, side: int
                     {"loss": loss_sum, "accuracy": accuracy_sum}, test_graph)
 
 
-def convnet(env: Environment, batch: int = 1000, seed: int = 3, side: int = 28) -> Workload:
+def convnet(env: Environment, batch: int = 1000, seed: int = 3, side: int = 28, blur_pool: bool = False) -> Workload:
     """ConvNet full training step with Adam (lr 1e-3): conv3x3 1->16 pad 1, leaky_relu, maxpool 2x2; conv3x3
     16->32 pad 1 groups 2, leaky_relu, maxpool; flatten; dropout 0.5; dense ->128 leaky_relu; dense ->10;
-    softmax cross-entropy."""
+    softmax cross-entropy.  `blur_pool` makes each pool a 2x2 stride-1 max pool and a fixed 3x3 stride-2 blur."""
     rng = np.random.Generator(np.random.PCG64(seed))
-    return _classifier_workload(env, ConvNet(env, side=side), batch, side, "adam", rng)
+    return _classifier_workload(env, ConvNet(env, side=side, blur_pool=blur_pool), batch, side, "adam", rng)
 
 
 def single_layer_classifier(env: Environment, batch: int = 1000, seed: int = 2, side: int = 28, hidden_units: int = 300,

@@ -368,6 +368,30 @@ def test_convnet_train_steps_vs_oracle(hip_backend_session, mode):
             assert err <= TOL, f"{key} [{mode}]: rel L2 {err}"
 
 
+@pytest.mark.parametrize("mode,batch", [("fused", 16), ("unfused", 16), ("fused", 64)])
+def test_conv_blur_net_train_steps_vs_oracle(hip_backend_session, mode, batch):
+    """Three Adam steps of the ConvBlurNet (examples/fashion_mnist/main.rs:187-199: every pool a 2x2 stride-1 max pool
+    and a fixed 3x3 stride-2 depthwise blur, src/module.rs:219-246): parameters, optimiser state, loss and accuracy."""
+    from descent_amd import Environment, workloads
+    from oracle.cpu_backend import CpuBackend
+
+    genv = Environment(hip_backend_session, fused=mode == "fused")
+    cenv = Environment(CpuBackend())
+    gw = workloads.convnet(genv, batch=batch, seed=19, blur_pool=True)
+    cw = workloads.convnet(cenv, batch=batch, seed=19, blur_pool=True)
+    for step in range(3):
+        genv.run(gw.graph, 2000 + step)
+        cenv.run(cw.graph, 2000 + step)
+    got, want = gw.snapshot(), cw.snapshot()
+    assert got.keys() == want.keys()
+    for key in want:
+        if key == "accuracy":
+            assert np.array_equal(got[key], want[key]), key
+        else:
+            err = rel_l2(got[key], want[key])
+            assert err <= TOL, f"{key} [{mode}, batch {batch}]: rel L2 {err}"
+
+
 def test_linear_classifier_steps_vs_oracle(hip_backend_session):
     """Config 1: single-layer softmax classifier, batch 1000, SGD momentum; 10 steps then one eval pass."""
     from descent_amd import workloads
