@@ -306,6 +306,65 @@ struct Emitter {
         if (pd.kind == DSC_KERNEL_PER_ELEMENT) {
             emit_pe(body, pd, vi.inputs, "gid", "v", {}, form.valid ? &local : nullptr);
             body << "    return vt" << vi.out_op << ";\n";
+        } else if (pd.kind == DSC_KERNEL_UNPAD) {
+            // one element of an Unpad on demand: the padded elements that the replicate padding took from it, in the
+            // standalone kernel's order (src/kernel.rs:645-710); one of them away from the border
+            const dsc_view& v = pd.inputs[0];
+            std::vector<string> oc;
+            if (form.valid) oc = emit_coords_separable(body, pd.shape, local, "vo");
+            if (oc.empty()) oc = emit_coords(body, pd.shape, "gid", "vo");
+            body << "    const int in_c = " << oc[pd.axis] << " + " << pd.pad << ";\n";
+            body << "    const int k_min = in_c - ((" << oc[pd.axis] << " == 0) ? " << pd.pad << " : 0);\n";
+            body << "    const int k_max = in_c + ((" << oc[pd.axis] << " == " << S(pd.shape.dims[pd.axis] - 1) << ") ? " << pd.pad << " : 0);\n";
+            body << "    float acc = 0.f;\n    for (int kk = k_min; kk <= k_max; ++kk) {\n";
+            auto ic = oc;
+            ic[pd.axis] = "kk";
+            body << "        acc += " << load_view(vi.inputs[0], v, ic) << ";\n    }\n    return acc;\n";
+        } else if (pd.kind == DSC_KERNEL_WINDOWS_TO_IMAGE) {
+            // one pixel of a WindowsToImage on demand: the windows that cover it, in the standalone kernel's order
+            // (src/kernel.rs:713-810, with the test that the window exists)
+            const dsc_view& v = pd.inputs[0];
+            const int r = v.out_shape.rank, bd = pd.shape.rank - 3;
+            const int64_t out_h = v.out_shape.dims[r - 6], out_w = v.out_shape.dims[r - 5];
+            const int64_t fh = v.out_shape.dims[r - 3], fw = v.out_shape.dims[r - 2], group_nc = v.out_shape.dims[r - 1];
+            const int64_t sw = pd.stride_w, sh = pd.stride_h;
+            std::vector<string> oc;
+            if (form.valid) oc = emit_coords_separable(body, pd.shape, local, "vo");
+            if (oc.empty()) oc = emit_coords(body, pd.shape, "gid", "vo");
+            body << "    const int in_y = " << oc[bd] << ", in_x = " << oc[bd + 1] << ", in_c = " << oc[bd + 2] << ";\n";
+            body << "    const int group_index = in_c / " << S(group_nc) << ", group_c = in_c % " << S(group_nc) << ";\n";
+            body << "    const int fbx = in_x % " << S(sw) << ", fby = in_y % " << S(sh) << ";\n";
+            body << "    const int oxb = in_x / " << S(sw) << ", oyb = in_y / " << S(sh) << ";\n";
+            body << "    float acc = 0.f;\n";
+            body << "#pragma unroll\n    for (int iy = 0; iy < " << S((fh + sh - 1) / sh) << "; ++iy)\n";
+            body << "#pragma unroll\n    for (int ix = 0; ix < " << S((fw + sw - 1) / sw) << "; ++ix) {\n";
+            body << "        const int fx = fbx + " << S(sw) << " * ix, fy = fby + " << S(sh) << " * iy;\n";
+            body << "        const int ox = oxb - ix, oy = oyb - iy;\n";
+            // (as in the standalone kernel, a tap without a window reads a valid element and adds zero: the taps' loads
+            // are then independent of the tests and in flight together -- behind a branch each, they were four round
+            // trips one after another)
+            body << "        const bool ok = fx < " << S(fw) << " && fy < " << S(fh) << " && ox >= 0 && ox < " << S(out_w) << " && oy >= 0 && oy < " << S(out_h) << ";\n";
+            body << "        const int fxc = min(fx, " << S(fw - 1) << "), fyc = min(fy, " << S(fh - 1) << "), oxc = clampi(ox, 0, " << S(out_w - 1)
+                 << "), oyc = clampi(oy, 0, " << S(out_h - 1) << ");\n";
+            std::vector<string> ic(r);
+            for (int i = 0; i < bd; ++i) ic[i] = oc[i];
+            ic[bd] = "oyc"; ic[bd + 1] = "oxc"; ic[bd + 2] = "group_index"; ic[bd + 3] = "fyc"; ic[bd + 4] = "fxc"; ic[bd + 5] = "group_c";
+            body << "        const float w = " << load_view(vi.inputs[0], v, ic) << ";\n        acc += ok ? w : 0.f;\n    }\n    return acc;\n";
+        } else if (pd.kind == DSC_KERNEL_MATMUL) {
+            // one element of a product over a very short k on demand (an outer product: the gradient of a depthwise
+            // filter's windows), summed in k order with fused multiply-adds like the row-per-thread kernel
+            const MatMulDims g = matmul_dims(pd);
+            dsc_shape os{};  // the product as the kernel stores it
+            os.rank = 3;
+            const bool by_rows = pd.output_mode == DSC_MATMUL_ROWS;
+            os.dims[0] = by_rows ? g.m : g.batch; os.dims[1] = by_rows ? g.batch : g.m; os.dims[2] = g.n;
+            std::vector<string> oc;
+            if (form.valid) oc = emit_coords_separable(body, os, local, "vo");
+            if (oc.empty()) oc = emit_coords(body, os, "gid", "vo");
+            body << "    const int cn = " << oc[2] << ", cm = " << oc[by_rows ? 0 : 1] << ", cb = " << oc[by_rows ? 1 : 0] << ";\n";
+            body << "    float acc = 0.f;\n#pragma unroll\n    for (int ck = 0; ck < " << S(g.k) << "; ++ck)\n";
+            body << "        acc = fmaf(" << load_view(vi.inputs[0], pd.inputs[0], {"cb", "cm", "ck"}) << ", " << load_view(vi.inputs[1], pd.inputs[1], {"cb", "ck", "cn"}) << ", acc);\n";
+            body << "    return acc;\n";
         } else {  // DSC_KERNEL_REDUCE evaluated on demand: one output element = a loop over the reduced axis
             const dsc_view& v = pd.inputs[0];
             std::vector<string> oc;
@@ -1133,12 +1192,19 @@ string gen_unpad(Emitter& em, Generated* out) {
     k << "    const int k_max = in_c + ((" << oc << " == " << S(d.shape.dims[d.axis] - 1) << ") ? " << d.pad << " : 0);\n";
     // the candidates in_c - pad .. in_c + pad are all loaded (clamped into [k_min, k_max]) and the ones outside
     // that range add zero: no loop with a data-dependent trip count, every load in flight at once
+    auto ic = c;
+    if (fk.inputs[0].virt >= 0) {
+        // (an input that is evaluated on demand -- sums of gathered elements themselves -- is evaluated only where it counts:
+        // once away from the border, where the masked candidates would cost 2 pad + 1 evaluations)
+        ic[d.axis] = "kk";
+        k << "    float sum = 0.f;\n    for (int kk = k_min; kk <= k_max; ++kk) sum += " << em.load_view(fk.inputs[0], v, ic) << ";\n";
+    } else {
     k << "    float sum = 0.f;\n#pragma unroll\n    for (int j = " << -d.pad << "; j <= " << d.pad << "; ++j) {\n";
     k << "        const int kk = in_c + j;\n        const int kc = clampi(kk, k_min, k_max);\n";
-    auto ic = c;
     ic[d.axis] = "kc";
     k << "        const float w = " << em.load_view(fk.inputs[0], v, ic) << ";\n";
     k << "        sum += (kk >= k_min && kk <= k_max) ? w : 0.f;\n    }\n";
+    }
     k << "    " << ResultStore(em).one("sum", "gid") << "\n}\n";
     out->grid = blocks_for(n, 256);
     out->block = 256;
@@ -2874,8 +2940,19 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
     std::ostringstream k;
     k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(fk) << "(" << em.kernel_params_decl() << ") {\n";
     k << "    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
+    // A depthwise product (one column per batch, the batches innermost in memory: [m][batch][1], the channels of an
+    // image) with consecutive lanes on consecutive batches of a row: the loads of A and the store then walk memory,
+    // where a lane per row of one batch reads and writes words `batch` apart (measured on a 3x3 blur of [1000, 27,
+    // 27, 16]: 134 us with a lane per row).  B is then a vector load per lane, from a few cache lines.
+    const bool batch_lanes = rows && g.n == 1 && g.batch > 1 && g.batch * g.m < kMaxIndex && R == 1 && !b_in_lds && !fk.out_slice_width;
+    if (batch_lanes) {
+        k << "    const int flat = min((int)(blockIdx.x * 256u + threadIdx.x), " << S(g.batch * g.m - 1) << ");\n";
+        k << "    const int cb = flat % " << S(g.batch) << ";\n";
+        k << "    const int row0 = blockIdx.x * 256u + threadIdx.x < " << S(g.batch * g.m) << "u ? flat / " << S(g.batch) << " : " << S(g.m) << ";\n";
+    } else {
     k << "    const int cb = blockIdx.x / " << S(blocks_per_batch) << ";\n";
     k << "    const int row0 = (blockIdx.x % " << S(blocks_per_batch) << ") * " << S(256 * R) << " + threadIdx.x;\n";
+    }
     if (b_in_lds) {
         k << "    __shared__ __attribute__((aligned(16))) float sB[" << S(g.k * g.n) << "];\n";
         k << "    for (int i = threadIdx.x; i < " << S(g.k * g.n) << "; i += 256) sB[i] = load_b(cb, i / " << S(g.n) << ", i % " << S(g.n)
@@ -3021,10 +3098,11 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
     }
     k << "    }\n    }\n}\n";
     }
-    out->grid = (unsigned)(blocks_per_batch * g.batch);
+    out->grid = batch_lanes ? (unsigned)((g.batch * g.m + 255) / 256) : (unsigned)(blocks_per_batch * g.batch);
     out->block = 256;
     out->source = k.str();
     out->note = (use_mfma ? string("row-per-thread store, mfma 16x16x4 from memory, B in registers")
+                 : batch_lanes ? string("row-per-thread fma, lanes along the batches of a row")
                           : string("row-per-thread fma, B ") + (b_in_lds ? "in LDS" : "in SGPRs")) +
                 (fk.has_epilogue ? " +epilogue" : "") + (W ? ", product stored as " + S(g.n / W) + " column slices of width " + S(W) : string());
     return "";
@@ -3936,8 +4014,11 @@ static std::string generate_one(const FusedKernel& fk, Generated* out, bool with
     for (auto& v : fk.virtuals) {
         err = validate(v.pe.raw());
         if (!err.empty()) return "fused producer: " + err;
-        if (v.pe.raw().kind != DSC_KERNEL_PER_ELEMENT && v.pe.raw().kind != DSC_KERNEL_REDUCE)
-            return "fused producer must be a per-element or reduce kernel";
+        const int vk = v.pe.raw().kind;
+        if (vk != DSC_KERNEL_PER_ELEMENT && vk != DSC_KERNEL_REDUCE && vk != DSC_KERNEL_UNPAD && vk != DSC_KERNEL_WINDOWS_TO_IMAGE && vk != DSC_KERNEL_MATMUL)
+            return "fused producer must be a per-element, reduce, unpad, windows-to-image or short matmul kernel";
+        if (vk == DSC_KERNEL_MATMUL && (matmul_dims(v.pe.raw()).chunks != 1 || matmul_dims(v.pe.raw()).k > 4))
+            return "fused producer: a matmul evaluated on demand has one chunk of at most four k";
         if ((int)v.inputs.size() != v.pe.raw().n_inputs) return "fused producer: input binding count";
     }
     if (fk.has_epilogue) {

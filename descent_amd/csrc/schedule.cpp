@@ -138,11 +138,27 @@ bool is_cheap_producer(const dsc_kernel_desc& pe) {
 
 // Loads issued per evaluated element, following fused producers (a Reduce producer multiplies by its k).
 double source_cost(const FusedKernel& fk, const Source& s);
+// Elements of its input that one element of a kernel evaluated on demand reads: the reduced axis of a Reduce, the k of a
+// MatMul, the windows that cover a pixel of a WindowsToImage (on average), the padded elements behind an element
+// of an Unpad (one, away from the border).
+double on_demand_reads(const dsc_kernel_desc& d) {
+    switch (d.kind) {
+    case DSC_KERNEL_REDUCE: return (double)d.inputs[0].out_shape.dims[d.axis];
+    case DSC_KERNEL_MATMUL: return (double)matmul_dims(d).k;
+    case DSC_KERNEL_UNPAD: return 1.0 + 2.0 * (double)d.pad / (double)d.shape.dims[d.axis];
+    case DSC_KERNEL_WINDOWS_TO_IMAGE: {
+        const dsc_view& v = d.inputs[0];
+        const int r = v.out_shape.rank;
+        return std::max(1.0, (double)(v.out_shape.dims[r - 3] * v.out_shape.dims[r - 2]) / (double)(d.stride_w * d.stride_h));
+    }
+    default: return 1.0;
+    }
+}
 double virtual_cost(const FusedKernel& fk, const Virtual& v) {
     const dsc_kernel_desc& d = v.pe.raw();
     double c = 0;
     for (auto& s : v.inputs) c += source_cost(fk, s);
-    if (d.kind == DSC_KERNEL_REDUCE) return c * (double)d.inputs[0].out_shape.dims[d.axis];
+    if (d.kind != DSC_KERNEL_PER_ELEMENT) return c * on_demand_reads(d);
     return c + d.n_ops / 4.0;
 }
 double source_cost(const FusedKernel& fk, const Source& s) { return s.buffer >= 0 ? 1.0 : virtual_cost(fk, fk.virtuals[s.virt]); }
@@ -160,7 +176,7 @@ double node_multiplicity(const Draft& d, int node) {
         if (s.buffer >= 0) return d.params[s.buffer] == node ? m : 0.0;
         const Virtual& v = d.fk.virtuals[s.virt];
         const dsc_kernel_desc& vd = v.pe.raw();
-        const double inner = m * (vd.kind == DSC_KERNEL_REDUCE ? (double)vd.inputs[0].out_shape.dims[vd.axis] : 1.0);
+        const double inner = m * (vd.kind != DSC_KERNEL_PER_ELEMENT ? on_demand_reads(vd) : 1.0);
         double best = 0.0;
         for (auto& in : v.inputs) best = std::max(best, self(in, inner, self));
         return best;
@@ -2109,6 +2125,27 @@ struct Planner {
         // DSC_CONV_BWD_LOADERS=2: loader waves, but dC of the convolution backward kernel stays a buffer
         const char* lw = std::getenv("DSC_CONV_BWD_LOADERS");
         const bool no_dc_producer = lw && lw[0] == '2';
+        // tuning hook: DSC_FUSE_GATHER_SUMS=0 keeps every Unpad, WindowsToImage and outer product a launch of its own
+        const char* fgs = std::getenv("DSC_FUSE_GATHER_SUMS");
+        const bool sum_on_demand = !(fgs && fgs[0] == '0');
+        auto on_demand_sum_kind = [](const Draft& p) {
+            const FusedKernel& f = p.fk;
+            const dsc_kernel_desc& d = f.main.raw();
+            if (f.has_epilogue || !f.parts.empty() || !f.row_stages.empty() || f.dgrad.on || f.cfwd.on || f.pool.on || f.pair.on || f.colsum_out >= 0 ||
+                f.sign_out >= 0 || f.out_slice_width || p.keep_split || p.outs.size() != 1 || f.outputs.size() != 1)
+                return false;
+            if (d.kind == DSC_KERNEL_UNPAD || d.kind == DSC_KERNEL_WINDOWS_TO_IMAGE) return true;
+            if (d.kind != DSC_KERNEL_MATMUL) return false;
+            const MatMulDims g = matmul_dims(d);
+            return g.chunks == 1 && g.k <= 2;
+        };
+        auto carries_on_demand_sum = [](const FusedKernel& f) {
+            for (auto& v : f.virtuals) {
+                const int k = v.pe.raw().kind;
+                if (k == DSC_KERNEL_UNPAD || k == DSC_KERNEL_WINDOWS_TO_IMAGE || k == DSC_KERNEL_MATMUL) return true;
+            }
+            return false;
+        };
         bool changed = true;
         while (changed) {
             changed = false;
@@ -2119,7 +2156,12 @@ struct Planner {
                 if (!p.fk.row_stages.empty()) continue;
                 const bool is_pe = pd.kind == DSC_KERNEL_PER_ELEMENT && pd.n_outputs == 1 && !p.fk.has_epilogue;
                 const bool is_red = pd.kind == DSC_KERNEL_REDUCE;
-                if ((!is_pe && !is_red) || p.keep_output) continue;
+                // An Unpad, a WindowsToImage or a product over a k of one or two (an outer product): each of their
+                // elements is a short sum of gathered elements, which a single consumer can evaluate where it reads it.
+                // (The backward pass of a strided convolution arrives as MatMul -> copy -> WindowsToImage -> Unpad ->
+                // Unpad, src/array.rs:954-975,989-1031: five arrays through memory for one.)
+                const bool is_sum = sum_on_demand && on_demand_sum_kind(p);
+                if ((!is_pe && !is_red && !is_sum) || p.keep_output) continue;
                 const int node = p.outs[0].node;
                 if (is_graph_output[node] || p.outs[0].copy_from >= 0) continue;
                 auto cons = consumers_of(node);
@@ -2131,6 +2173,25 @@ struct Planner {
                 if (is_pe && !into_rows && (!is_cheap_producer(pd) || p.fk.virtuals.size() > 8)) continue;
                 if (is_pe && cons.size() > 1 && !is_pure_copy(pd)) continue;
                 bool ok = true;
+                if (is_sum) {
+                    if (cons.size() != 1) continue;
+                    const Draft& q = drafts[cons[0]];
+                    const dsc_kernel_desc& cd = q.fk.main.raw();
+                    const bool plain = q.fk.parts.empty() && q.fk.row_stages.empty() && q.fk.row_width == 0 && !q.fk.has_epilogue;
+                    if (!plain || (cd.kind != DSC_KERNEL_PER_ELEMENT && cd.kind != DSC_KERNEL_UNPAD && cd.kind != DSC_KERNEL_WINDOWS_TO_IMAGE)) continue;
+                    // a per-element consumer that reads each element several times over (a broadcast) leaves it in memory
+                    if (cd.kind == DSC_KERNEL_PER_ELEMENT && 2 * element_count(cd.shape) > 3 * element_count(pd.shape)) continue;
+                    // loads per element the consumer stores: what one evaluation costs, times the evaluations behind each of
+                    // the consumer's own reads, times those reads (a WindowsToImage over overlapping windows evaluates each
+                    // element once per window: measured on the gradient of a 2x2 stride-1 max pooling, 30 loads per stored
+                    // element took as long as the four launches they replaced)
+                    const double fan_in = cd.kind == DSC_KERNEL_PER_ELEMENT ? 1.0 : on_demand_reads(cd);
+                    const double per_read = draft_unit_cost(p) * on_demand_reads(pd) * node_multiplicity(q, node);
+                    if (per_read > 24.0 || per_read * fan_in > 16.0) continue;
+                }
+                if (is_pe && carries_on_demand_sum(p.fk))
+                    for (int ci : cons)
+                        if (drafts[ci].fk.main.raw().kind == DSC_KERNEL_MATMUL || cons.size() > 1) ok = false;
                 if (is_pe && !fuse_into_matmul)
                     for (int ci : cons)
                         if (drafts[ci].fk.main.raw().kind == DSC_KERNEL_MATMUL) ok = false;
@@ -2186,7 +2247,7 @@ struct Planner {
                     {
                         Virtual nv;
                         nv.pe = p.fk.main;
-                        nv.out_op = is_pe ? pd.outputs[0] : 0;
+                        nv.out_op = is_pe ? pd.outputs[0] : 0;  // (kinds evaluated on demand have one result)
                         for (auto& s : p.fk.inputs) nv.inputs.push_back(import_source(q, p, s, voff));
                         q.fk.virtuals[new_virt] = nv;
                     }

@@ -361,3 +361,23 @@ def test_masked_data_gradients_read_the_sign_bytes_the_forward_products_write():
     assert "sign bytes" not in off
     # 3 x 268 MB of activations not read again, 3 x 16.8 MB of bytes written and read
     assert "7318.3" in on.strip().splitlines()[-1] and "8022.9" in off.strip().splitlines()[-1], (on.strip().splitlines()[-1], off.strip().splitlines()[-1])
+
+
+def test_the_backward_of_a_strided_depthwise_convolution_is_one_launch_of_gathered_sums(monkeypatch):
+    """The blur of a MaxBlurPool2D (src/module.rs:219-246: 3x3, stride 2, a group per channel) leaves, in the backward
+    pass, MatMul(k=1) -> copy -> WindowsToImage -> Unpad -> Unpad (src/array.rs:954-975,989-1031).  One launch evaluates
+    the chain per element of the last Unpad; the gradient of the stride-1 max pooling behind it, which would evaluate it
+    once per window, reads it from memory.  The forward product of one column per channel runs with its lanes along
+    the channels."""
+    env = _env()
+    w = workloads.convnet(env, batch=16, seed=1, blur_pool=True)
+    fused = hip_backend.check_schedule(w.graph, fused=True)
+    assert fused.count("lanes along the batches of a row") == 2, fused
+    assert "MatMul (k=1)" not in fused and fused.count("Unpad [") == 2 and fused.count("WindowsToImage [") == 2, fused
+    for line in fused.splitlines():
+        if "Unpad [" in line:
+            # the chain behind each remaining Unpad: its producers' clusters are covered by its launch
+            assert len(re.search(r"clusters ([\d ]+)$", line).group(1).split()) >= 5, line
+    monkeypatch.setenv("DSC_FUSE_GATHER_SUMS", "0")
+    apart = hip_backend.check_schedule(workloads.convnet(_env(), batch=16, seed=1, blur_pool=True).graph, fused=True)
+    assert apart.count("Unpad [") == 4 and apart.count("MatMul (k=1)") == 2 and int(apart.split()[0]) > int(fused.split()[0])
