@@ -1031,6 +1031,19 @@ string gen_reduce(Emitter& em, Generated* out) {
         }
     }
 
+    // ... or, from a fused producer, with one evaluation of a quad (a pooling over a window copy of an image whose
+    // channels walk memory: the copy's index arithmetic once per four channels, 16-byte loads)
+    bool vec_virtual = false;
+    if (!k_fastest && !vec_outputs && fk.inputs[0].virt >= 0 && n_out % 4 == 0 && v.out_shape.rank == d.shape.rank) {
+        const int L = d.shape.rank - 1;
+        if (L >= 1 && d.axis != L && d.shape.dims[L] % 4 == 0) {
+            std::vector<string> pc;
+            for (int i = 0; i < d.shape.rank; ++i) pc.push_back(d.shape.dims[i] == 1 && i != d.axis ? "0" : "oc" + to_string(i));
+            pc[d.axis] = "kq0";
+            vec_virtual = vec_outputs = !em.load_view4(fk.inputs[0], v, pc).empty();
+        }
+    }
+
     std::ostringstream k;
     k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
     // The k loop runs over groups of U independent accumulators: the U loads of a group are issued before any of
@@ -1102,7 +1115,7 @@ string gen_reduce(Emitter& em, Generated* out) {
         k << "    if (vid < " << S(n_vec) << "u) {\n";
         k << "    const uint oid = vid * 4u;\n";
         auto oc = em.emit_coords(k, d.shape, "oid", "oc");
-        const int U = pick_unroll(TK, 16);
+        const int U = pick_unroll(TK, vec_virtual ? 4 : 16);
         const char* comps[4] = {"x", "y", "z", "w"};
         for (int u = 0; u < U; ++u) k << (u ? ", a" : "    float4 a") << u << " = result";
         k << ";\n    int kb = " << (TK > 1 ? "tk" : "0") << ";\n";
@@ -1112,6 +1125,14 @@ string gen_reduce(Emitter& em, Generated* out) {
             for (int u = 0; u < lvl; ++u) {
                 auto ic = oc;
                 ic[d.axis] = "(kb + " + S(u * TK) + ")";
+                if (vec_virtual) {  // (a producer takes its coordinates by name)
+                    ic[d.axis] = "kq" + to_string(u);
+                    for (int i = 0; i < d.shape.rank; ++i)
+                        if (d.shape.dims[i] == 1 && i != d.axis) ic[i] = "0";
+                    k << "        const int kq" << u << " = kb + " << S(u * TK) << ";\n";
+                    k << "        const float4 x" << u << " = " << em.load_view4(fk.inputs[0], v, ic) << ";\n";
+                }
+                else
                 k << "        const float4 x" << u << " = *(const float4*)(b" << fk.inputs[0].buffer << " + " << em.index_expr(v, ic) << ");\n";
             }
             for (int u = 0; u < lvl; ++u) {
@@ -1225,6 +1246,41 @@ string gen_windows_to_image(Emitter& em, Generated* out) {
     const int64_t n = element_count(d.shape);
     std::ostringstream k;
     k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
+    // Four channels of a pixel per thread where a group's channels come in fours: they share the pixel's windows, so the
+    // index arithmetic is done once per quad and the loads are 16 bytes (a kernel of this kind is bound by the number
+    // of load instructions it issues, not by their bytes).
+    if (group_nc % 4 == 0 && n % 4 == 0) {
+        std::vector<string> pc(r);
+        for (int i = 0; i < bd; ++i) pc[i] = "c" + to_string(i);
+        pc[bd] = "oyc"; pc[bd + 1] = "oxc"; pc[bd + 2] = "group_index"; pc[bd + 3] = "fyc"; pc[bd + 4] = "fxc"; pc[bd + 5] = "group_c";
+        for (int i = 0; i < bd; ++i)
+            if (d.shape.dims[i] == 1) pc[i] = "0";
+        const string w4 = em.load_view4(fk.inputs[0], v, pc);
+        if (!w4.empty()) {
+            k << "    const uint gid = (blockIdx.x * 256u + threadIdx.x) * 4u;\n    if (gid >= " << S(n) << "u) return;\n";
+            auto c = em.emit_coords(k, d.shape, "gid", "c");
+            k << "    const int in_y = " << c[bd] << ", in_x = " << c[bd + 1] << ", in_c = " << c[bd + 2] << ";\n";
+            k << "    const int group_index = in_c / " << S(group_nc) << ", group_c = in_c % " << S(group_nc) << ";\n";
+            k << "    const int fbx = in_x % " << S(sw) << ", fby = in_y % " << S(sh) << ";\n";
+            k << "    const int oxb = in_x / " << S(sw) << ", oyb = in_y / " << S(sh) << ";\n";
+            k << "    float4 tmp = make_float4(0.f, 0.f, 0.f, 0.f);\n";
+            k << "#pragma unroll\n    for (int iy = 0; iy < " << S((fh + sh - 1) / sh) << "; ++iy)\n";
+            k << "#pragma unroll\n    for (int ix = 0; ix < " << S((fw + sw - 1) / sw) << "; ++ix) {\n";
+            k << "        const int fx = fbx + " << S(sw) << " * ix, fy = fby + " << S(sh) << " * iy;\n";
+            k << "        const int ox = oxb - ix, oy = oyb - iy;\n";
+            k << "        const bool ok = fx < " << S(fw) << " && fy < " << S(fh) << " && ox >= 0 && ox < " << S(out_w) << " && oy >= 0 && oy < " << S(out_h) << ";\n";
+            k << "        const int fxc = min(fx, " << S(fw - 1) << "), fyc = min(fy, " << S(fh - 1) << "), oxc = clampi(ox, 0, " << S(out_w - 1)
+              << "), oyc = clampi(oy, 0, " << S(out_h - 1) << ");\n";
+            k << "        const float4 w = " << w4 << ";\n";
+            k << "        tmp.x += ok ? w.x : 0.f; tmp.y += ok ? w.y : 0.f; tmp.z += ok ? w.z : 0.f; tmp.w += ok ? w.w : 0.f;\n    }\n";
+            k << "    " << ResultStore(em).four("tmp", "gid") << "\n}\n";
+            out->grid = blocks_for(n / 4, 256);
+            out->block = 256;
+            out->source = k.str();
+            out->note = fk.has_epilogue ? "windows_to_image x4 +epilogue" : "windows_to_image x4";
+            return "";
+        }
+    }
     k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n";
     auto c = em.emit_coords(k, d.shape, "gid", "c");
     k << "    const int in_y = " << c[bd] << ", in_x = " << c[bd + 1] << ", in_c = " << c[bd + 2] << ";\n";
