@@ -323,7 +323,7 @@ def _compact_classes(classes):
 def bench_configs(env):
     """The configurations the headline does not cover, compact enough for the one JSON line: the other four
     standalone matmul shapes (each verified on sampled rows against float64 after its timed region), the linear
-    classifier, both coordinate MLPs and the hash-grid fit (step rate, launches, per-class roofline fractions,
+    classifier, the ConvBlurNet, both coordinate MLPs and the hash-grid fit (step rate, launches, per-class roofline fractions,
     and the summed loss of the timed steps, which must be finite).
 
     Every timed region follows a warm-up of the same launches that lasts a quarter of a second or so, and lasts about
@@ -343,7 +343,10 @@ def bench_configs(env):
             "tflops_kernels": round(r["flops"] / (us * 1e-6) / 1e12, 2), "frac_mfma": round(r["flops"] / (us * 1e-6) / 1e12 / MFMA_FP32_PEAK_TFLOPS, 3),
             "kernels_us": round(us, 2), "tflops_wall": round(r["tflops_wall"], 2), "launches": r["launches_per_step"], "steps": steps, "warmup": warmup,
             "rel_l2_error_sampled_rows": r["rel_l2_error_sampled_rows"], "verified": bool(ok)}
+    # (the ConvBlurNet is the reference example's other convolutional network -- strided depthwise blurs behind stride-1
+    # max pools, examples/fashion_mnist/main.rs:187-199 -- and not one of the five configurations)
     builds = (("cfg1_linear_classifier_bs1000", lambda e: _w.linear_classifier(e), 2000, 5000),
+              ("conv_blur_net_bs1000", lambda e: _w.convnet(e, blur_pool=True), 300, 600),
               ("cfg4_coordinate_mlp_relu_pe_512", lambda e: _w.coordinate_mlp(e), 40, 80),
               ("cfg4_coordinate_mlp_siren_512", lambda e: _w.coordinate_mlp(e, variant="siren"), 40, 80),
               ("cfg5_hash_grid_2p18", lambda e: _w.hash_grid_fit(e), 200, 400))
