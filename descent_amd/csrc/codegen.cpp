@@ -6,6 +6,7 @@
 #include <cstdlib>
 #include <functional>
 #include <map>
+#include <set>
 #include <sstream>
 
 namespace dsc {
@@ -805,6 +806,44 @@ struct ResultStore {
 
 unsigned blocks_for(int64_t threads, int block) { return (unsigned)((threads + block - 1) / block); }
 
+// Read-only inputs of at most `max_floats` elements that a kernel and its fused producers read through plain views
+// (a depthwise filter, a bias): (buffer, elements).  A kernel whose lanes read such a table at lane-dependent places
+// pays a vector memory instruction per read -- a quarter wave per cycle through the address unit whatever the bytes --
+// and can keep the table in LDS instead (`stage_small_tables`).
+std::vector<std::pair<int, int64_t>> small_tables(const FusedKernel& fk, int64_t max_floats) {
+    std::map<int, int64_t> extent;
+    std::set<int> barred;
+    auto visit = [&](const dsc_kernel_desc& d, const std::vector<Source>& srcs) {
+        for (int i = 0; i < d.n_inputs && i < (int)srcs.size(); ++i) {
+            if (srcs[i].buffer < 0) continue;
+            const int b = srcs[i].buffer;
+            extent[b] = std::max(extent[b], element_count(d.inputs[i].in_shape));
+            if (d.kind == DSC_KERNEL_PER_ELEMENT)
+                for (int o = 0; o < d.n_ops; ++o)
+                    if (d.ops[o].kind == DSC_PE_GATHER && d.ops[o].input_index == i) barred.insert(b);
+            if (d.kind == DSC_KERNEL_SCATTER_ADD) barred.insert(b);
+        }
+    };
+    visit(fk.main.raw(), fk.inputs);
+    for (auto& v : fk.virtuals) visit(v.pe.raw(), v.inputs);
+    if (fk.has_epilogue) visit(fk.epilogue.raw(), fk.epilogue_inputs);
+    std::vector<std::pair<int, int64_t>> out;
+    for (auto& e : extent)
+        if (e.second <= max_floats && !barred.count(e.first) && e.first < fk.n_buffers && !fk.buffer_is_output[e.first]) out.push_back(e);
+    return out;
+}
+
+// Opens a block in which the names of the given buffers mean copies of them in LDS (every later read of b<i>, in the
+// kernel and in the producers' functions it passes b<i> to, is then an LDS read); the caller closes the block with
+// one more "}".  All 256 threads of the workgroup must reach this point.
+void stage_small_tables(std::ostream& k, const std::vector<std::pair<int, int64_t>>& tables) {
+    for (auto& t : tables) k << "    __shared__ float sb" << t.first << "[" << S(t.second) << "];\n";
+    for (auto& t : tables)
+        k << "    for (int i = threadIdx.x; i < " << S(t.second) << "; i += 256) sb" << t.first << "[i] = b" << t.first << "[i];\n";
+    k << "    __syncthreads();\n    {\n";
+    for (auto& t : tables) k << "    const float* const b" << t.first << " = sb" << t.first << ";\n";
+}
+
 // ---------------------------------------------------------------------------------------------------------
 
 string gen_fill(Emitter& em, Generated* out) {
@@ -1205,6 +1244,10 @@ string gen_unpad(Emitter& em, Generated* out) {
     const int64_t n = element_count(d.shape);
     std::ostringstream k;
     k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
+    // (a chain of gathered sums evaluated on demand reads the small tables at its end -- a depthwise filter -- once per
+    // evaluation and lane: from LDS)
+    const auto tables = fk.inputs[0].virt >= 0 ? small_tables(fk, 1024) : std::vector<std::pair<int, int64_t>>();
+    if (!tables.empty()) stage_small_tables(k, tables);
     k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n";
     auto c = em.emit_coords(k, d.shape, "gid", "c");
     const string oc = c[d.axis];
@@ -1226,11 +1269,11 @@ string gen_unpad(Emitter& em, Generated* out) {
     k << "        const float w = " << em.load_view(fk.inputs[0], v, ic) << ";\n";
     k << "        sum += (kk >= k_min && kk <= k_max) ? w : 0.f;\n    }\n";
     }
-    k << "    " << ResultStore(em).one("sum", "gid") << "\n}\n";
+    k << "    " << ResultStore(em).one("sum", "gid") << "\n" << (tables.empty() ? "" : "    }\n") << "}\n";
     out->grid = blocks_for(n, 256);
     out->block = 256;
     out->source = k.str();
-    out->note = fk.has_epilogue ? "unpad +epilogue" : "unpad";
+    out->note = string(fk.has_epilogue ? "unpad +epilogue" : "unpad") + (tables.empty() ? "" : ", small tables in LDS");
     return "";
 }
 
@@ -3001,6 +3044,8 @@ string gen_matmul_rows(Emitter& em, Generated* out) {
     // where a lane per row of one batch reads and writes words `batch` apart (measured on a 3x3 blur of [1000, 27,
     // 27, 16]: 134 us with a lane per row).  B is then a vector load per lane, from a few cache lines.
     const bool batch_lanes = rows && g.n == 1 && g.batch > 1 && g.batch * g.m < kMaxIndex && R == 1 && !b_in_lds && !fk.out_slice_width;
+    // (the filters, read per lane here, stay in memory: staged in LDS -- a fill and a barrier per workgroup -- the blur of
+    // [1000, 27, 27, 16] took 16.2 us against 14.0)
     if (batch_lanes) {
         k << "    const int flat = min((int)(blockIdx.x * 256u + threadIdx.x), " << S(g.batch * g.m - 1) << ");\n";
         k << "    const int cb = flat % " << S(g.batch) << ";\n";
