@@ -128,7 +128,7 @@ def class_rooflines(be, steps):
     return out
 
 
-def bench_convnet(env, steps, warmup, batch=1000, repeats=5, blur_pool=False):
+def bench_convnet(env, steps, warmup, batch=1000, repeats=5, blur_pool=False, min_warmup=1000):
     """ConvNet train steps per second: `repeats` timed regions of `steps` steps each (no per-launch events), the
     median reported with the spread beside it; then one more pass with events for the per-kernel table."""
     import re
@@ -138,7 +138,7 @@ def bench_convnet(env, steps, warmup, batch=1000, repeats=5, blur_pool=False):
     w = workloads.convnet(env, batch=batch, seed=3, blur_pool=blur_pool)
     # (the warm-up is long enough for the device to reach the clock it holds under this load: the first region of a run
     # that starts from idle reads 1.5 % low)
-    walls = [time_graph(env, w.graph, steps, max(warmup, 1000) if r == 0 else 0, seed0=1 + r * steps, profile=False) for r in range(repeats)]
+    walls = [time_graph(env, w.graph, steps, max(warmup, min_warmup) if r == 0 else 0, seed0=1 + r * steps, profile=False) for r in range(repeats)]
     wall = sorted(walls)[len(walls) // 2]
     if EVENT_PASS:
         time_graph(env, w.graph, min(steps, 50), 0, seed0=100000, profile=True)
@@ -412,6 +412,9 @@ def main():
                     help="headline: the 8192^3 matmul line with the ConvNet step rate beside it (default); matmul: "
                          "that line without the ConvNet; the others run one workload alone, e.g. under rocprofv3")
     ap.add_argument("--no-events", action="store_true", help="no per-launch HIP events (wall time only)")
+    ap.add_argument("--min-warmup", type=int, default=1000,
+                    help="convnet / conv-blur-net: warm-up steps at least (1000 bring the device to its sustained clock; a counter "
+                         "run, which serialises every dispatch, wants a handful)")
     ap.add_argument("--markers", action="store_true",
                     help="wrap every launch in a ROCTx range named by the kernel's label (rocprofv3 --marker-trace)")
     args = ap.parse_args()
@@ -434,7 +437,7 @@ def main():
         from descent_amd import workloads as _w
 
         if args.workload in ("convnet", "conv-blur-net"):
-            out = bench_convnet(env, args.steps, args.warmup, blur_pool=args.workload == "conv-blur-net")
+            out = bench_convnet(env, args.steps, args.warmup, blur_pool=args.workload == "conv-blur-net", min_warmup=args.min_warmup)
             sys.stderr.write(out.pop("report"))
         elif args.workload == "convnet-uploads":
             out = bench_convnet_minibatch_uploads(env, steps=max(args.steps, 20))
