@@ -1018,6 +1018,63 @@ def test_conv2d_gradients_over_geometries(hip_backend_session, geom, fused):
     assert rel_l2(gdf, cdf) <= TOL, (rel_l2(gdf, cdf), listing)
 
 
+def _strided_conv_grad_case(env, m, h, w, c_in, c_out, fh, fw, pad, stride, groups, seed):
+    """x -> conv2d with a stride -> 0.5 * sum(y^2): the product and the gradients with respect to the image and the filter."""
+    from descent_amd import Initializer
+
+    rng = np.random.default_rng(seed)
+    xp = env.trainable_parameter([m, h, w, c_in], "x", Initializer.zero())
+    fp = env.trainable_parameter([groups, c_out // groups, fh, fw, c_in // groups], "f", Initializer.zero())
+    env.write_parameter(xp, rng.standard_normal((m, h, w, c_in), dtype=np.float32))
+    env.write_parameter(fp, rng.standard_normal(tuple(fp.shape), dtype=np.float32) * 0.2)
+    dx, df = env.static_parameter([m, h, w, c_in], "dx"), env.static_parameter(list(fp.shape), "df")
+    oh, ow = (h + 2 * pad - fh) // stride[1] + 1, (w + 2 * pad - fw) // stride[0] + 1
+    y_out = env.static_parameter([m, oh, ow, c_out], "y")
+
+    def build(s):
+        x, f = s.parameter(xp), s.parameter(fp)
+        y = x.conv2d(f, pad, stride)
+        s.write_parameter_value(y_out, y.value() * 1.0)
+        (y.square() * 0.5).set_loss()
+        s.write_parameter_value(dx, x.loss_grad())
+        s.write_parameter_value(df, f.loss_grad())
+
+    g = env.build_graph(build)
+    env.run(g, 0)
+    return g, env.read_parameter(y_out), env.read_parameter(dx), env.read_parameter(df)
+
+
+@pytest.mark.parametrize("geom", [
+    # m, h, w, c_in, c_out, fh, fw, pad, stride (w, h), groups
+    (300, 27, 27, 16, 16, 3, 3, 1, (2, 2), 16),  # the blur of a MaxBlurPool2D: one group per channel, the chain one launch
+    (200, 13, 13, 32, 32, 3, 3, 1, (2, 2), 32),
+    (120, 12, 12, 8, 16, 2, 2, 0, (2, 2), 1),    # windows that tile the image: a copy, no sums
+    (90, 11, 9, 4, 8, 3, 3, 0, (2, 2), 2),       # no padding: no Unpads
+    (80, 11, 13, 6, 6, 4, 3, 1, (2, 3), 3),      # strides that differ, an even filter height
+    (70, 16, 16, 8, 8, 5, 5, 2, (3, 3), 8),      # depthwise, stride 3, two replicated pixels per side
+], ids=lambda g: "x".join(str(v) for v in g[:8]) + "s%dx%dg%d" % (g[8][0], g[8][1], g[9]))
+def test_strided_conv2d_gradients_with_gathered_sums_on_demand(hip_backend_session, monkeypatch, geom):
+    """Strided convolutions (src/array.rs:989-1031) take no dedicated kernel: the data gradient's WindowsToImage and
+    Unpads, and the outer product in front of them where a group has one output channel, are evaluated on demand by
+    the last of them.  Against the oracle within the tolerance, and bit for bit against the same kernels launched one
+    by one (the sums are made in the standalone kernels' order)."""
+    genv, cenv = _envs(hip_backend_session, fused=True)
+    g, gy, gdx, gdf = _strided_conv_grad_case(genv, *geom, seed=41)
+    _, cy, cdx, cdf = _strided_conv_grad_case(cenv, *geom, seed=41)
+    listing = next(iter(g.__dict__["_schedules"].values())).describe()
+    assert rel_l2(gy, cy) <= TOL, listing
+    assert rel_l2(gdx, cdx) <= TOL, (rel_l2(gdx, cdx), listing)
+    assert rel_l2(gdf, cdf) <= TOL, (rel_l2(gdf, cdf), listing)
+    monkeypatch.setenv("DSC_FUSE_GATHER_SUMS", "0")
+    aenv, _ = _envs(hip_backend_session, fused=True)
+    a, ay, adx, adf = _strided_conv_grad_case(aenv, *geom, seed=41)
+    apart = next(iter(a.__dict__["_schedules"].values())).describe()
+    assert int(apart.split()[0]) >= int(listing.split()[0]), (listing, apart)
+    if geom[7] > 0:  # with padding there are Unpads, and the first of them is evaluated by the second
+        assert apart.count("Unpad [") > listing.count("Unpad ["), (listing, apart)
+    assert np.array_equal(gdx, adx) and np.array_equal(gy, ay) and np.array_equal(gdf, adf), (listing, apart)
+
+
 def _first_layer_case(env, m, h, w, c_in, c_out, fh, fw, pad, pool, seed):
     """data -> conv2d + bias -> leaky_relu (-> 2x2 max-pool) -> 0.5 * sum(y^2), the data a plain parameter: only the
     filter and the bias have gradients, as for the first layer of a network."""
