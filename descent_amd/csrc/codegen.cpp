@@ -904,6 +904,8 @@ string gen_per_element_rows(Emitter& em, Generated* out) {
     if (rows >= kMaxIndex) return "per-element rows: too many rows";
     std::ostringstream k;
     k << "extern \"C\" __global__ __launch_bounds__(256) void " << entry_name(em.fk) << "(" << em.kernel_params_decl() << ") {\n    const uint rand_seed = seed_cell ? *seed_cell : seed_value;\n";
+    // (the small tables a row gathers from -- the coarse levels of a hash grid -- stay in memory: copied into LDS per
+    // workgroup, 2 / 8 / 15 / 28 thousand floats of them, the hash grid's encoding took 76 / 86 / 101 / 185 us against 74)
     k << "    const int dsc_row = (int)(blockIdx.x * 256u + threadIdx.x);\n";
     k << "    if (dsc_row >= " << S(rows) << ") return;\n";
     for (int o = 0; o < d.n_outputs; ++o) k << "    float o" << o << "[" << S(W) << "];\n";
