@@ -384,6 +384,191 @@ struct Emitter {
         return name;
     }
 
+    // Decomposition of an id given as an IndexForm whose terms each lie inside one axis of `shape`, several of them
+    // possibly inside the same axis (an id over [img, y, x, g, fy, fx] read as [img * y * x, g, fy * fx]): a coordinate
+    // is then the sum of its terms, none of which can carry into the next axis.  An axis that one term with the
+    // axis' own stride fills keeps the term's name.  Empty when a term straddles axes or an axis could overflow.
+    std::vector<string> emit_coords_grouped(std::ostream& o, const dsc_shape& shape, const IndexForm& form, const string& pfx) {
+        if (!form.valid || form.base != 0) return {};
+        int64_t st[DSC_MAX_DIM];
+        strides_of(shape, st);
+        std::vector<std::vector<std::pair<int64_t, string>>> parts(shape.rank);
+        std::vector<int64_t> reach(shape.rank, 0);
+        for (size_t t = 0; t < form.names.size(); ++t) {
+            if (form.coefs[t] == 0 || form.extents[t] <= 1) continue;
+            if (form.coefs[t] < 0) return {};
+            int axis = -1;
+            for (int i = 0; i < shape.rank; ++i)
+                if (shape.dims[i] > 1 && st[i] <= form.coefs[t]) { axis = i; break; }  // the outermost axis whose stride the term reaches
+            if (axis < 0 || form.coefs[t] % st[axis] != 0) return {};
+            const int64_t mult = form.coefs[t] / st[axis];
+            parts[axis].push_back({mult, form.names[t]});
+            reach[axis] += mult * (form.extents[t] - 1);
+        }
+        std::vector<string> names(shape.rank);
+        for (int i = 0; i < shape.rank; ++i) {
+            if (reach[i] >= shape.dims[i]) return {};
+            if (parts[i].empty()) { names[i] = "0"; continue; }
+            if (parts[i].size() == 1 && parts[i][0].first == 1) { names[i] = parts[i][0].second; continue; }
+            names[i] = pfx + "g" + to_string(i);
+            o << "    const int " << names[i] << " = ";
+            for (size_t j = 0; j < parts[i].size(); ++j) o << (j ? " + " : "") << "(" << S(parts[i][j].first) << ")*" << parts[i][j].second;
+            o << ";\n";
+        }
+        return names;
+    }
+
+    // ---- four elements along any coordinate -----------------------------------------------------------
+    // The elements of source `s` that view `v` selects at coord, with coordinate `q` taking coord[q] .. coord[q] + 3
+    // (a multiple of four inside an extent that is one), as a float4.  Where the quad's elements are not neighbours
+    // in the source -- four groups of a depthwise convolution, far apart in a product's own layout -- the index
+    // arithmetic of every level is still done once per quad, and the buffers at the end are read with one 16-byte load
+    // where the quad does walk memory there (the four channels of a pixel), with four words otherwise.  "" when a
+    // level cannot be evaluated that way (the caller then evaluates single elements).
+    string load_view_q(const Source& s, const dsc_view& v, const std::vector<string>& coord, int q) {
+        if (q < 0 || q >= v.out_shape.rank || v.out_shape.dims[q] % 4 != 0 || !is_identifier(coord[q])) return "";
+        int64_t base = 0, coef[DSC_MAX_DIM];
+        if (!affine_form(v, &base, coef)) return "";
+        if (s.buffer >= 0) {
+            const string b = "b" + to_string(s.buffer), idx = index_expr(v, coord);
+            if (coef[q] == 0) return "dsc_splat4(" + b + "[" + idx + "])";
+            bool aligned = coef[q] == 1 && base % 4 == 0;
+            for (int j = 0; j < v.out_shape.rank; ++j)
+                if (j != q && v.out_shape.dims[j] > 1 && coef[j] % 4 != 0) aligned = false;
+            if (aligned) return "*(const float4*)(" + b + " + " + idx + ")";
+            return "dsc_load4_strided(" + b + " + " + idx + ", " + S(coef[q]) + ")";
+        }
+        if (coef[q] == 0) {
+            const string one = load_view(s, v, coord);
+            return "dsc_splat4(" + one + ")";
+        }
+        IndexForm form = index_form(v, coord);
+        if (!form.valid) return "";
+        int qt = -1;
+        for (size_t t = 0; t < form.names.size(); ++t)
+            if (form.names[t] == coord[q]) qt = (int)t;
+        if (qt < 0) return "";
+        const string fn = instantiate_q(s.virt, form, qt);
+        if (fn.empty()) return "";
+        string args;
+        for (auto& n : form.names) args += n + ", ";
+        return fn + "(" + args + params_pass() + ")";
+    }
+
+    // The float4 of virtual producer `virt` for ids of the given form whose term `qt` takes its coordinate .. + 3.
+    string instantiate_q(int virt, const IndexForm& form, int qt) {
+        if (!form.valid || form.extents[qt] % 4 != 0) return "";
+        string sig = "Q" + to_string(virt) + "|" + to_string(qt) + "|" + S(form.base);
+        for (size_t t = 0; t < form.names.size(); ++t) sig += "," + S(form.coefs[t]) + "x" + S(form.extents[t]);
+        auto it = instances.find(sig);
+        if (it != instances.end()) return it->second;
+        const Virtual& vi = fk.virtuals[virt];
+        const dsc_kernel_desc& pd = vi.pe.raw();
+        const string name = "virt" + to_string(virt) + "_" + to_string(instances.size()) + "_q";
+        instances[sig] = name;  // (the graph of virtuals is acyclic)
+        IndexForm local = form;
+        string decl;
+        for (size_t t = 0; t < form.names.size(); ++t) {
+            local.names[t] = "a" + to_string(t);
+            decl += "int a" + to_string(t) + ", ";
+        }
+        const string qname = local.names[qt];
+        std::ostringstream body;
+        auto fail = [&]() { return instances[sig] = ""; };
+        // the axis of `shape` that the quad's term is the coordinate of
+        auto axis_of_quad = [&](const std::vector<string>& oc) {
+            for (size_t i = 0; i < oc.size(); ++i)
+                if (oc[i] == qname) return (int)i;
+            return -1;
+        };
+        const char* add4 = "    acc = make_float4(acc.x + w.x, acc.y + w.y, acc.z + w.z, acc.w + w.w);\n";
+        if (pd.kind == DSC_KERNEL_PER_ELEMENT) {
+            // a pure copy hands the quad on through its view; anything else is not evaluated this way
+            if (!(pd.n_inputs == 1 && pd.n_outputs == 1 && pd.n_ops >= 1 && pd.n_ops <= 2 && pd.ops[0].kind == DSC_PE_LOAD &&
+                  (pd.n_ops == 1 || (pd.ops[1].kind == DSC_PE_UNARY && pd.ops[1].op == DSC_UN_MOV && pd.ops[1].args[0] == 0)) &&
+                  vi.out_op == pd.n_ops - 1))
+                return fail();
+            const dsc_view& v = pd.inputs[0];
+            std::vector<string> oc = emit_coords_separable(body, v.out_shape, local, "vo");
+            if (oc.empty()) oc = emit_coords_grouped(body, v.out_shape, local, "vo");
+            const int qa = oc.empty() ? -1 : axis_of_quad(oc);
+            if (qa < 0) return fail();
+            const string x = load_view_q(vi.inputs[0], v, oc, qa);
+            if (x.empty()) return fail();
+            body << "    return " << x << ";\n";
+        } else if (pd.kind == DSC_KERNEL_UNPAD) {
+            const dsc_view& v = pd.inputs[0];
+            std::vector<string> oc = emit_coords_separable(body, pd.shape, local, "vo");
+            if (oc.empty()) oc = emit_coords_grouped(body, pd.shape, local, "vo");
+            const int qa = oc.empty() ? -1 : axis_of_quad(oc);
+            if (qa < 0 || qa == pd.axis) return fail();
+            auto ic = oc;
+            ic[pd.axis] = "kk";
+            const string x = load_view_q(vi.inputs[0], v, ic, qa);
+            if (x.empty()) return fail();
+            body << "    const int in_c = " << oc[pd.axis] << " + " << pd.pad << ";\n";
+            body << "    const int k_min = in_c - ((" << oc[pd.axis] << " == 0) ? " << pd.pad << " : 0);\n";
+            body << "    const int k_max = in_c + ((" << oc[pd.axis] << " == " << S(pd.shape.dims[pd.axis] - 1) << ") ? " << pd.pad << " : 0);\n";
+            body << "    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);\n    for (int kk = k_min; kk <= k_max; ++kk) {\n";
+            body << "        const float4 w = " << x << ";\n    " << add4 << "    }\n    return acc;\n";
+        } else if (pd.kind == DSC_KERNEL_WINDOWS_TO_IMAGE) {
+            const dsc_view& v = pd.inputs[0];
+            const int r = v.out_shape.rank, bd = pd.shape.rank - 3;
+            const int64_t out_h = v.out_shape.dims[r - 6], out_w = v.out_shape.dims[r - 5];
+            const int64_t fh = v.out_shape.dims[r - 3], fw = v.out_shape.dims[r - 2], group_nc = v.out_shape.dims[r - 1];
+            const int64_t sw = pd.stride_w, sh = pd.stride_h;
+            std::vector<string> oc = emit_coords_separable(body, pd.shape, local, "vo");
+            if (oc.empty()) oc = emit_coords_grouped(body, pd.shape, local, "vo");
+            const int qa = oc.empty() ? -1 : axis_of_quad(oc);
+            // the quad runs over channels: four of one group, or four groups of one channel each
+            if (qa != bd + 2 || !(group_nc % 4 == 0 || group_nc == 1)) return fail();
+            std::vector<string> ic(r);
+            for (int i = 0; i < bd; ++i) ic[i] = oc[i];
+            ic[bd] = "oyc"; ic[bd + 1] = "oxc"; ic[bd + 2] = "group_index"; ic[bd + 3] = "fyc"; ic[bd + 4] = "fxc"; ic[bd + 5] = "group_c";
+            const string x = load_view_q(vi.inputs[0], v, ic, group_nc == 1 ? bd + 2 : bd + 5);
+            if (x.empty()) return fail();
+            body << "    const int in_y = " << oc[bd] << ", in_x = " << oc[bd + 1] << ", in_c = " << oc[bd + 2] << ";\n";
+            body << "    const int group_index = in_c / " << S(group_nc) << ", group_c = in_c % " << S(group_nc) << ";\n";
+            body << "    const int fbx = in_x % " << S(sw) << ", fby = in_y % " << S(sh) << ";\n";
+            body << "    const int oxb = in_x / " << S(sw) << ", oyb = in_y / " << S(sh) << ";\n";
+            body << "    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);\n";
+            body << "#pragma unroll\n    for (int iy = 0; iy < " << S((fh + sh - 1) / sh) << "; ++iy)\n";
+            body << "#pragma unroll\n    for (int ix = 0; ix < " << S((fw + sw - 1) / sw) << "; ++ix) {\n";
+            body << "        const int fx = fbx + " << S(sw) << " * ix, fy = fby + " << S(sh) << " * iy;\n";
+            body << "        const int ox = oxb - ix, oy = oyb - iy;\n";
+            body << "        const bool ok = fx < " << S(fw) << " && fy < " << S(fh) << " && ox >= 0 && ox < " << S(out_w) << " && oy >= 0 && oy < " << S(out_h) << ";\n";
+            body << "        const int fxc = min(fx, " << S(fw - 1) << "), fyc = min(fy, " << S(fh - 1) << "), oxc = clampi(ox, 0, " << S(out_w - 1)
+                 << "), oyc = clampi(oy, 0, " << S(out_h - 1) << ");\n";
+            body << "        const float4 w = " << x << ";\n";
+            body << "        acc = make_float4(acc.x + (ok ? w.x : 0.f), acc.y + (ok ? w.y : 0.f), acc.z + (ok ? w.z : 0.f), acc.w + (ok ? w.w : 0.f));\n    }\n";
+            body << "    return acc;\n";
+        } else if (pd.kind == DSC_KERNEL_MATMUL) {
+            const MatMulDims g = matmul_dims(pd);
+            dsc_shape os{};
+            os.rank = 3;
+            const bool by_rows = pd.output_mode == DSC_MATMUL_ROWS;
+            os.dims[0] = by_rows ? g.m : g.batch; os.dims[1] = by_rows ? g.batch : g.m; os.dims[2] = g.n;
+            std::vector<string> oc = emit_coords_separable(body, os, local, "vo");
+            if (oc.empty()) oc = emit_coords_grouped(body, os, local, "vo");
+            const int qa = oc.empty() ? -1 : axis_of_quad(oc);
+            if (qa < 0) return fail();
+            const string cb = oc[by_rows ? 1 : 0], cm = oc[by_rows ? 0 : 1], cn = oc[2];
+            const int q_is = qa == 2 ? 2 : (qa == (by_rows ? 1 : 0) ? 0 : 1);  // 0: batch, 1: row, 2: column
+            // (coordinates that are literal zeros -- an extent of one -- are passed as they are: their axes carry no term)
+            const string xa = q_is == 2 ? "dsc_splat4(" + load_view(vi.inputs[0], pd.inputs[0], {cb, cm, "ck"}) + ")" : load_view_q(vi.inputs[0], pd.inputs[0], {cb, cm, "ck"}, q_is == 0 ? 0 : 1);
+            const string xb = q_is == 1 ? "dsc_splat4(" + load_view(vi.inputs[1], pd.inputs[1], {cb, "ck", cn}) + ")" : load_view_q(vi.inputs[1], pd.inputs[1], {cb, "ck", cn}, q_is == 0 ? 0 : 2);
+            if (xa.empty() || xb.empty()) return fail();
+            body << "    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);\n#pragma unroll\n    for (int ck = 0; ck < " << S(g.k) << "; ++ck) {\n";
+            body << "        const float4 x = " << xa << ";\n        const float4 y = " << xb << ";\n";
+            body << "        acc = make_float4(fmaf(x.x, y.x, acc.x), fmaf(x.y, y.y, acc.y), fmaf(x.z, y.z, acc.z), fmaf(x.w, y.w, acc.w));\n    }\n";
+            body << "    return acc;\n";
+        } else {
+            return fail();
+        }
+        funcs << "DSC_INLINE float4 " << name << "(" << decl << params_decl() << ") {\n" << body.str() << "}\n\n";
+        return name;
+    }
+
     // ---- four consecutive elements at once ------------------------------------------------------------
     // A consumer that wants elements id .. id + 3 of a source, id a multiple of four and the four of them inside one
     // run of the innermost axis of every view on the way, gets them from ONE evaluation: the index arithmetic of each
@@ -1250,6 +1435,36 @@ string gen_unpad(Emitter& em, Generated* out) {
     // evaluation and lane: from LDS)
     const auto tables = fk.inputs[0].virt >= 0 ? small_tables(fk, 1024) : std::vector<std::pair<int, int64_t>>();
     if (!tables.empty()) stage_small_tables(k, tables);
+    // Four elements of the innermost axis per thread where the chain behind the input can be evaluated for a quad (the
+    // four channels of a pixel share every index but the channel's, and the chain ends in 16-byte loads where the
+    // channels walk memory): a kernel of this kind is bound by the load instructions it issues.
+    {
+        const int L = d.shape.rank - 1;
+        string x4;
+        if (fk.inputs[0].virt >= 0 && L >= 1 && d.axis != L && d.shape.dims[L] % 4 == 0 && n % 4 == 0) {
+            std::vector<string> pc;
+            for (int i = 0; i < d.shape.rank; ++i) pc.push_back("c" + to_string(i));
+            pc[d.axis] = "kk";
+            x4 = em.load_view_q(fk.inputs[0], v, pc, L);
+        }
+        if (!x4.empty()) {
+            k << "    const uint gid = (blockIdx.x * 256u + threadIdx.x) * 4u;\n    if (gid >= " << S(n) << "u) return;\n";
+            auto c = em.emit_coords(k, d.shape, "gid", "c");
+            const string oc = c[d.axis];
+            k << "    const int in_c = " << oc << " + " << d.pad << ";\n";
+            k << "    const int k_min = in_c - ((" << oc << " == 0) ? " << d.pad << " : 0);\n";
+            k << "    const int k_max = in_c + ((" << oc << " == " << S(d.shape.dims[d.axis] - 1) << ") ? " << d.pad << " : 0);\n";
+            k << "    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);\n    for (int kk = k_min; kk <= k_max; ++kk) {\n";
+            k << "        const float4 w = " << x4 << ";\n";
+            k << "        sum = make_float4(sum.x + w.x, sum.y + w.y, sum.z + w.z, sum.w + w.w);\n    }\n";
+            k << "    " << ResultStore(em).four("sum", "gid") << "\n" << (tables.empty() ? "" : "    }\n") << "}\n";
+            out->grid = blocks_for(n / 4, 256);
+            out->block = 256;
+            out->source = k.str();
+            out->note = string(fk.has_epilogue ? "unpad x4 +epilogue" : "unpad x4") + (tables.empty() ? "" : ", small tables in LDS");
+            return "";
+        }
+    }
     k << "    const uint gid = blockIdx.x * 256u + threadIdx.x;\n    if (gid >= " << S(n) << "u) return;\n";
     auto c = em.emit_coords(k, d.shape, "gid", "c");
     const string oc = c[d.axis];
