@@ -2184,7 +2184,8 @@ struct Planner {
                     // loads per element the consumer stores: what one evaluation costs, times the evaluations behind each of
                     // the consumer's own reads, times those reads (a WindowsToImage over overlapping windows evaluates each
                     // element once per window: measured on the gradient of a 2x2 stride-1 max pooling, 30 loads per stored
-                    // element took as long as the four launches they replaced)
+                    // element took as long as the four launches they replaced, and with the chain evaluated four channels at a
+                    // time still 184 us against 35 + 20 for the two launches)
                     const double fan_in = cd.kind == DSC_KERNEL_PER_ELEMENT ? 1.0 : on_demand_reads(cd);
                     const double per_read = draft_unit_cost(p) * on_demand_reads(pd) * node_multiplicity(q, node);
                     if (per_read > 24.0 || per_read * fan_in > 16.0) continue;
