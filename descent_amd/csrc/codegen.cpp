@@ -448,7 +448,24 @@ struct Emitter {
         for (size_t t = 0; t < form.names.size(); ++t)
             if (form.names[t] == coord[q]) qt = (int)t;
         if (qt < 0) return "";
-        const string fn = instantiate_q(s.virt, form, qt);
+        string fn;
+        {
+            // four consecutive ids of a per-element or Reduce producer: the form for consecutive quads knows every op
+            const int vk = fk.virtuals[s.virt].pe.raw().kind;
+            if ((vk == DSC_KERNEL_PER_ELEMENT || vk == DSC_KERNEL_REDUCE) && form.coefs[qt] == 1) {
+                IndexForm last = form;  // the quad's term last, as that form wants it
+                std::swap(last.names[qt], last.names.back());
+                std::swap(last.coefs[qt], last.coefs.back());
+                std::swap(last.extents[qt], last.extents.back());
+                const string f4 = instantiate4(s.virt, last);
+                if (!f4.empty()) {
+                    string args4;
+                    for (auto& n : last.names) args4 += n + ", ";
+                    return f4 + "(" + args4 + params_pass() + ")";
+                }
+            }
+        }
+        fn = instantiate_q(s.virt, form, qt);
         if (fn.empty()) return "";
         string args;
         for (auto& n : form.names) args += n + ", ";
@@ -620,6 +637,9 @@ struct Emitter {
         if (it != instances.end()) return it->second;
         const Virtual& vi = fk.virtuals[virt];
         const dsc_kernel_desc& pd = vi.pe.raw();
+        // (gathered sums evaluated on demand have one quad form, along any coordinate: here the last term's)
+        if (pd.kind == DSC_KERNEL_UNPAD || pd.kind == DSC_KERNEL_WINDOWS_TO_IMAGE || pd.kind == DSC_KERNEL_MATMUL)
+            return instances[sig] = instantiate_q(virt, form, (int)form.names.size() - 1);
         if (pd.kind != DSC_KERNEL_PER_ELEMENT && pd.kind != DSC_KERNEL_REDUCE) return instances[sig] = "";
         const string name = "virt" + to_string(virt) + "_" + to_string(instances.size()) + "_x4";
         instances[sig] = name;  // (a producer never reads itself: the graph of virtuals is acyclic)

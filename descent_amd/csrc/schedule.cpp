@@ -2139,6 +2139,9 @@ struct Planner {
             const MatMulDims g = matmul_dims(d);
             return g.chunks == 1 && g.k <= 2;
         };
+        // tuning hook: DSC_CONV_TAKES_SUMS=0 keeps a WindowsToImage in front of a convolution backward kernel a launch
+        const char* cts = std::getenv("DSC_CONV_TAKES_SUMS");
+        const bool conv_takes_sums = !(cts && cts[0] == '0');
         auto carries_on_demand_sum = [](const FusedKernel& f) {
             for (auto& v : f.virtuals) {
                 const int k = v.pe.raw().kind;
@@ -2178,7 +2181,16 @@ struct Planner {
                     const Draft& q = drafts[cons[0]];
                     const dsc_kernel_desc& cd = q.fk.main.raw();
                     const bool plain = q.fk.parts.empty() && q.fk.row_stages.empty() && q.fk.row_width == 0 && !q.fk.has_epilogue;
-                    if (!plain || (cd.kind != DSC_KERNEL_PER_ELEMENT && cd.kind != DSC_KERNEL_UNPAD && cd.kind != DSC_KERNEL_WINDOWS_TO_IMAGE)) continue;
+                    // (the convolution backward kernels evaluate dC where they fill their tile: a WindowsToImage over
+                    // overlapping windows -- the gradient of a stride-1 pooling -- in front of them is evaluated there too.
+                    // Measured on the ConvBlurNet at batch 1000: the kernel with both gradients 34.3 -> 45.2 us for a
+                    // launch of 18.7 us less, the filter gradient alone 20.9 -> 42.3 us for one of 34.5 us less)
+                    const bool conv_dc = conv_takes_sums && cd.kind == DSC_KERNEL_MATMUL && q.fk.dgrad.on && (q.fk.dgrad.wgrad || q.fk.dgrad.wgrad_only) &&
+                                         pd.kind == DSC_KERNEL_WINDOWS_TO_IMAGE && !q.fk.dgrad.pm.on;
+                    if (!plain || (cd.kind != DSC_KERNEL_PER_ELEMENT && cd.kind != DSC_KERNEL_UNPAD && cd.kind != DSC_KERNEL_WINDOWS_TO_IMAGE && !conv_dc)) continue;
+                    if (conv_dc) {
+                        if (draft_unit_cost(p) * on_demand_reads(pd) * node_multiplicity(q, node) > 24.0) continue;
+                    } else {
                     // a per-element consumer that reads each element several times over (a broadcast) leaves it in memory
                     if (cd.kind == DSC_KERNEL_PER_ELEMENT && 2 * element_count(cd.shape) > 3 * element_count(pd.shape)) continue;
                     // loads per element the consumer stores: what one evaluation costs, times the evaluations behind each of
@@ -2189,6 +2201,7 @@ struct Planner {
                     const double fan_in = cd.kind == DSC_KERNEL_PER_ELEMENT ? 1.0 : on_demand_reads(cd);
                     const double per_read = draft_unit_cost(p) * on_demand_reads(pd) * node_multiplicity(q, node);
                     if (per_read > 24.0 || per_read * fan_in > 16.0) continue;
+                    }
                 }
                 if (is_pe && carries_on_demand_sum(p.fk))
                     for (int ci : cons)

@@ -49,6 +49,38 @@ def test_convnet_batch_1000_fused_unfused_and_oracle(hip_backend_session):
             assert rel_l2(fused[key], want[key]) <= TOL, f"{key} vs oracle: {rel_l2(fused[key], want[key])}"
 
 
+def test_conv_blur_net_batch_1000_vs_oracle_and_without_the_gathered_sums(hip_backend_session, monkeypatch):
+    """The ConvBlurNet (examples/fashion_mnist/main.rs:187-199) at the batch the step rate is quoted on: there the
+    convolution backward kernels take the gradient of the stride-1 max pools where they fill dC, and each blur's backward
+    chain is one launch.  Two Adam steps against the oracle, and against the same step with those fusions off."""
+    from descent_amd import Environment, workloads
+    from oracle.cpu_backend import CpuBackend
+
+    def run(env):
+        w = workloads.convnet(env, batch=1000, seed=5, blur_pool=True)
+        for i in range(2):
+            env.run(w.graph, 70 + i)
+        return w
+
+    gw = run(Environment(hip_backend_session, fused=True))
+    listing = next(iter(gw.graph.__dict__["_schedules"].values())).describe()
+    assert "WindowsToImage [" not in listing and listing.count("<4 fused producers>") == 2 and listing.count("unpad x4") == 2, listing
+    got = gw.snapshot()
+    want = run(Environment(CpuBackend())).snapshot()
+    monkeypatch.setenv("DSC_CONV_TAKES_SUMS", "0")
+    monkeypatch.setenv("DSC_FUSE_GATHER_SUMS", "0")
+    aw = run(Environment(hip_backend_session, fused=True))
+    apart_listing = next(iter(aw.graph.__dict__["_schedules"].values())).describe()
+    assert apart_listing.count("WindowsToImage [") == 4 and apart_listing.count("Unpad [") == 4, apart_listing
+    apart = aw.snapshot()
+    for key in want:
+        if key == "accuracy":
+            assert np.array_equal(got[key], want[key]) and np.array_equal(apart[key], want[key])
+        else:
+            assert rel_l2(got[key], want[key]) <= TOL, f"{key} vs oracle: {rel_l2(got[key], want[key])}"
+            assert rel_l2(got[key], apart[key]) <= TOL, f"{key} vs the launches apart: {rel_l2(got[key], apart[key])}"
+
+
 @pytest.mark.parametrize("variant", ["relu-pe", "siren"])
 def test_coordinate_mlp_512_fused_unfused(hip_backend_session, variant):
     from descent_amd import workloads
