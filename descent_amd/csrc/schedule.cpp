@@ -2044,8 +2044,30 @@ struct Planner {
             const dsc_kernel_desc& pd = p.fk.main.raw();
             if (pd.kind != DSC_KERNEL_PER_ELEMENT) continue;
             // the cluster and whatever was already inlined into it (an earlier cluster of this kind)
-            auto is_plain = [](const dsc_kernel_desc& d) {
-                if (d.kind != DSC_KERNEL_PER_ELEMENT || d.n_ops > 40) return false;
+            // A reader evaluates only what the outputs it takes depend on (the compiler drops the rest), so the bound
+            // on the work a reader repeats is on the ops behind one output: the cluster that turns the two coordinates of a
+            // point into a cell and a fraction per level of a hash grid has 85 ops and 32 outputs of five ops each --
+            // stored, it was 67 MB written per step and read back by the encoding and by every ScatterAdd.
+            auto ops_behind = [](const dsc_kernel_desc& d, int out_op) {
+                std::vector<char> seen(d.n_ops, 0);
+                std::vector<int> todo{out_op};
+                int count = 0;
+                while (!todo.empty()) {
+                    const int o = todo.back();
+                    todo.pop_back();
+                    if (o < 0 || o >= d.n_ops || seen[o]) continue;
+                    seen[o] = 1;
+                    ++count;
+                    const dsc_pe_op& op = d.ops[o];
+                    const int n_args = op.kind == DSC_PE_UNARY || op.kind == DSC_PE_GATHER ? 1 : op.kind == DSC_PE_BINARY ? 2 : op.kind == DSC_PE_SELECT ? 4 : 0;
+                    for (int a = 0; a < n_args; ++a) todo.push_back(op.args[a]);
+                }
+                return count;
+            };
+            auto is_plain = [&](const dsc_kernel_desc& d, int only_output /* -1: every output */) {
+                if (d.kind != DSC_KERNEL_PER_ELEMENT || d.n_ops > 256) return false;
+                for (int o = 0; o < d.n_outputs; ++o)
+                    if ((only_output < 0 || d.outputs[o] == only_output) && ops_behind(d, d.outputs[o]) > 40) return false;
                 for (int o = 0; o < d.n_ops; ++o) {
                     const dsc_pe_op& op = d.ops[o];
                     if (op.kind == DSC_PE_GATHER || op.kind == DSC_PE_RAND) return false;
@@ -2054,8 +2076,8 @@ struct Planner {
                 }
                 return true;
             };
-            bool plain = is_plain(pd) && p.fk.virtuals.size() <= 8;
-            for (auto& v : p.fk.virtuals) plain = plain && is_plain(v.pe.raw());
+            bool plain = is_plain(pd, -1) && p.fk.virtuals.size() <= 8;
+            for (auto& v : p.fk.virtuals) plain = plain && is_plain(v.pe.raw(), v.out_op);
             if (!plain) continue;
             size_t in_bytes = 0;
             bool ok = true;
@@ -2073,7 +2095,18 @@ struct Planner {
                 const int qk = q.fk.main.raw().kind;
                 if (ci <= i || !q.fk.parts.empty() || !q.fk.row_stages.empty() || q.fk.dgrad.on || q.fk.cfwd.on || q.fk.pool.on) ok = false;
                 if (qk != DSC_KERNEL_PER_ELEMENT && qk != DSC_KERNEL_REDUCE && qk != DSC_KERNEL_SCATTER_ADD) ok = false;
-                if ((int)q.fk.virtuals.size() + (int)p.fk.virtuals.size() + (int)p.outs.size() > 24) ok = false;
+                {
+                    // (a reader takes a producer per output it reads, not per output there is)
+                    int taken = 0;
+                    for (auto& out : p.outs) {
+                        bool reads = false;
+                        for_each_source(q.fk, [&](Source& src) {
+                            if (src.buffer >= 0 && q.params[src.buffer] == out.node && !q.fk.buffer_is_output[src.buffer]) reads = true;
+                        });
+                        taken += reads;
+                    }
+                    if ((int)q.fk.virtuals.size() + (int)p.fk.virtuals.size() + taken > 24) ok = false;
+                }
                 for (auto& o : q.outs)
                     for (auto& out : p.outs)
                         if (o.copy_from == out.node) ok = false;  // updated in place by the reader
