@@ -384,3 +384,16 @@ def test_the_backward_of_a_strided_depthwise_convolution_is_one_launch_of_gather
     monkeypatch.setenv("DSC_FUSE_GATHER_SUMS", "0")
     apart = hip_backend.check_schedule(workloads.convnet(_env(), batch=16, seed=1, blur_pool=True).graph, fused=True)
     assert apart.count("Unpad [") == 4 and apart.count("MatMul (k=1)") == 2 and int(apart.split()[0]) > int(fused.split()[0])
+
+
+def test_a_row_fused_launch_takes_the_light_producer_in_front_of_it(monkeypatch):
+    """The linear classifier's logits are the sum of a product's ten k-chunks with the bias on it (a per-element
+    cluster over a short Reduce), read element for element by the stages of the softmax cross-entropy
+    (src/loss.rs:4-34): the row-fused launch evaluates it, 5 -> 4 launches."""
+    w = workloads.linear_classifier(_env(), batch=1000, seed=1)
+    fused = hip_backend.check_schedule(w.graph, fused=True)
+    assert int(fused.split()[0]) == 4, fused
+    assert re.search(r"RowFused \[1000, 10\] \(\d+ clusters\) <2 fused producers>", fused), fused
+    monkeypatch.setenv("DSC_ROWS_TAKE_PRODUCERS", "0")
+    apart = hip_backend.check_schedule(workloads.linear_classifier(_env(), batch=1000, seed=1).graph, fused=True)
+    assert int(apart.split()[0]) == 5 and "PerElement (3 ops) [10000] <1 fused producers>" in apart, apart
